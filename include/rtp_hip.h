@@ -1,0 +1,236 @@
+/*
+ * rtp_hip.h - C ABI of librtp_hip.so: gfx950 (MI355X) kernels for RTP's rotated-shard layer compute.
+ *
+ * The reference (wdlctc/rtp) has no FFI: its "operators" are the ATen calls made inside each
+ * per-shard nn.Module.forward plus torch.distributed.batch_isend_irecv for the ring.  Every entry
+ * point below names the reference call site (path:line under the reference tree) it stands in for.
+ *
+ * Conventions
+ *  - every function returns 0 on success and a negative rtp_status on failure; the message of the
+ *    last failure on the calling thread is returned by rtp_last_error().
+ *  - all pointers are borrowed device pointers (the caller owns the memory and keeps it alive until
+ *    the work queued on `stream` has completed).  Nothing here allocates device memory: ops that
+ *    need scratch take a caller-provided workspace sized by the matching *_workspace_bytes().
+ *  - every call is asynchronous on `stream` (a hipStream_t passed as void*); no call synchronises
+ *    the device.
+ *  - dtype: RTP_F32 or RTP_BF16 is the storage type of activations/weights; accumulation is fp32.
+ */
+#ifndef RTP_HIP_H
+#define RTP_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { RTP_F32 = 0, RTP_BF16 = 1 } rtp_dtype;
+
+typedef enum {
+  RTP_OK = 0,
+  RTP_ERR_ARG = -1,     /* bad shape / null pointer / unsupported combination */
+  RTP_ERR_DEVICE = -2,  /* current device is not gfx950 */
+  RTP_ERR_HIP = -3,     /* a HIP runtime call failed */
+  RTP_ERR_WORKSPACE = -4 /* workspace too small */
+} rtp_status;
+
+const char* rtp_last_error(void);
+
+/* Version of this ABI (bumped on any signature change). */
+int rtp_abi_version(void);
+
+/* 0 if the current HIP device is gfx950, RTP_ERR_DEVICE otherwise.  `name_out` (optional, >= 64
+ * bytes, host memory) receives the gcnArchName. */
+int rtp_device_check(char* name_out, int name_len);
+
+/* ---------------------------------------------------------------------------------------------
+ * GEMM   C[z][m,n] = epilogue( alpha * sum_k A[z](m,k) * B[z](n,k) )
+ *
+ * Stands in for F.linear inside the shard modules (rtp/module/linear.py:216, :385;
+ * rtp/module/functional.py:303-308 in-projection, :798/:828 out-projection; rtp/module/top2gate.py:202
+ * gate projection; rtp/models/transformer_lm_rtp.py:74-75 expert FFN), for the autograd backward
+ * of those calls (dX = dY W, dW = dY^T X), and for the batched q k^T / p v products of
+ * rtp/module/functional.py:779-792.
+ *
+ *   a_kcontig = 1 : A(m,k) is read at A[m*lda + k]       (row-major M x K)
+ *   a_kcontig = 0 : A(m,k) is read at A[k*lda + m]       (stored K x M)
+ *   b_kcontig = 1 : B(n,k) is read at B[n*ldb + k]       (row-major N x K, i.e. a torch Linear weight)
+ *   b_kcontig = 0 : B(n,k) is read at B[k*ldb + n]       (stored K x N)
+ *
+ * Batching: grid z in [0, batch); z is split as zo = z / zdiv, zi = z % zdiv and every operand
+ * pointer advances by zo*stride_o + zi*stride_i elements (so a (batch, head) pair can index a
+ * packed [L, N, 3E] projection without a re-layout).
+ *
+ * Epilogue, in this order:  v = alpha*acc;  if c_in: v += c_in[m,n];  if bias: v += bias[n];
+ * if RTP_GEMM_RELU: v = max(v,0);  if gate: v = gate[m,n] > 0 ? v : 0;  store to c_out as fp32
+ * (RTP_GEMM_OUT_F32) or as `dtype`.  c_in is read as fp32 when RTP_GEMM_CIN_F32 is set, else as
+ * `dtype`.  bias and gate are `dtype`.  c_in may alias c_out.
+ * --------------------------------------------------------------------------------------------- */
+enum {
+  RTP_GEMM_OUT_F32 = 1,
+  RTP_GEMM_CIN_F32 = 2,
+  RTP_GEMM_RELU = 4
+};
+
+typedef struct {
+  const void* a;
+  const void* b;
+  void* c_out;
+  const void* c_in;  /* may be NULL */
+  const void* bias;  /* may be NULL; length N */
+  const void* gate;  /* may be NULL; same indexing as c_out but with ld_gate */
+  int64_t m, n, k;
+  int64_t lda, ldb, ldc, ld_cin, ld_gate;
+  int64_t batch, zdiv; /* batch >= 1, zdiv >= 1 */
+  int64_t a_so, a_si, b_so, b_si, c_so, c_si, cin_so, cin_si, gate_so, gate_si, bias_so, bias_si;
+  float alpha;
+  int32_t flags;
+  int32_t a_kcontig, b_kcontig;
+} rtp_gemm_desc;
+
+int rtp_gemm(void* stream, int dtype, const rtp_gemm_desc* d);
+
+/* sizeof(rtp_gemm_desc) as this library was compiled: lets a binding verify its struct layout. */
+size_t rtp_gemm_desc_size(void);
+
+/* out[n] (+)= sum_m x[m*ld + n]  in fp32, fixed summation order (deterministic).  The bias
+ * gradient of nn.Linear's backward (reference: autograd of rtp/module/linear.py:216).
+ * out is fp32 if out_f32 else `dtype`; accumulate != 0 adds to the existing contents. */
+int rtp_colsum(void* stream, int dtype, const void* x, int64_t m, int64_t n, int64_t ld,
+               void* out, int out_f32, int accumulate);
+
+/* ---------------------------------------------------------------------------------------------
+ * Shard rotation (reference: rtp/module/collectives.py:202-257 _left/_right_shift_buffer +
+ * _WeightParallelRegion_before/after; rtp/rotated_tensor_parallel.py:114-151).  On one GPU the
+ * isend/irecv pair of a ring step becomes a device-to-device copy of the next flat shard into the
+ * spare slot of a two-slot staging buffer, queued on a side stream so it overlaps the compute
+ * that is consuming the other slot.
+ *
+ * rtp_ring_create makes the side stream and the fencing events (no device memory).
+ *   begin(main)                  side stream waits for everything queued on main so far
+ *   prefetch(slot, dst, src, n)  side: wait until the last consumer of `slot` released it, copy
+ *   acquire(main, slot)          main waits for the copy into `slot`
+ *   release(main, slot)          marks the point on main after which `slot` may be overwritten
+ * After the last acquire of a begin..end sequence the side stream is fully joined into main, so a
+ * sequence may be recorded into a HIP graph by capturing main.
+ * --------------------------------------------------------------------------------------------- */
+int rtp_ring_create(void** ring_out);
+int rtp_ring_destroy(void* ring);
+int rtp_ring_begin(void* ring, void* main_stream);
+int rtp_ring_prefetch(void* ring, int slot, void* dst, const void* src, size_t bytes);
+int rtp_ring_acquire(void* ring, void* main_stream, int slot);
+int rtp_ring_release(void* ring, void* main_stream, int slot);
+
+/* The copy kernel on its own (16-byte vectorised, grid-stride): dst/src 16-byte aligned or any
+ * alignment (falls back to bytes for the ragged ends). */
+int rtp_shard_copy_async(void* stream, void* dst, const void* src, size_t bytes);
+
+/* dst[i] = 0 for `bytes` bytes; a fill kernel (safe to record into a HIP graph). */
+int rtp_zero_async(void* stream, void* dst, size_t bytes);
+
+/* ---------------------------------------------------------------------------------------------
+ * Embedding (reference: F.embedding at rtp/module/embedding.py:146 and its dense backward).
+ * A shard is the rectangle rows [row_begin, row_begin+row_count) x `cols` columns of the master
+ * table, stored row-major with leading dimension ld_table; the reference shards columns
+ * (embedding.py:65-71) and uses row_begin = 0, row_count = V.
+ *   gather:      out[t, 0:cols] = table[ids[t] - row_begin, 0:cols]   (ids outside the row range
+ *                leave out[t] untouched); out has leading dimension ld_out.
+ *   scatter-add: grad_table[ids[t] - row_begin, :] += grad_out[t, :]  summed per row in ascending t
+ *                (sequential fp32 adds starting from +0.0f: bit-identical to torch's CPU
+ *                nn.Embedding backward / index_add_).  Rows that receive no token are zero-filled
+ *                when zero_fill != 0.  Tokens equal to padding_idx (if >= 0) are skipped.
+ *                When scale_by_freq != 0 each row's sum is divided by the number of tokens that
+ *                hit it.
+ * ids are int64.  The scatter-add needs a workspace (sort buffers).
+ * --------------------------------------------------------------------------------------------- */
+int rtp_embedding_gather(void* stream, int dtype, const void* table, int64_t ld_table,
+                         int64_t row_begin, int64_t row_count, int64_t cols, const int64_t* ids,
+                         int64_t n_ids, void* out, int64_t ld_out);
+
+size_t rtp_embedding_scatter_workspace_bytes(int64_t n_ids);
+
+/* Sorts (id, position) once; the result in `workspace` is reused by every shard of the layer. */
+int rtp_embedding_sort_ids(void* stream, const int64_t* ids, int64_t n_ids, void* workspace,
+                           size_t workspace_bytes);
+
+int rtp_embedding_scatter_add_det(void* stream, int dtype, const void* grad_out, int64_t ld_grad_out,
+                                  int64_t n_ids, const void* workspace, void* grad_table,
+                                  int64_t ld_grad_table, int grad_table_f32, int64_t row_begin,
+                                  int64_t row_count, int64_t cols, int64_t padding_idx,
+                                  int scale_by_freq, int zero_fill);
+
+/* ---------------------------------------------------------------------------------------------
+ * Attention softmax (reference: rtp/module/functional.py:779-792 baddbmm+softmax, :825
+ * scaled_dot_product_attention with an additive float mask).
+ *   fwd: p[z,i,j] = softmax_j( scale*s[z,i,j] + mask[i,j] )  (and j <= i + (S-L) only, if causal)
+ *        s fp32 [Z,L,S] contiguous, mask fp32 [L,S] or NULL, p `dtype` [Z,L,S].
+ *   bwd: ds[z,i,j] = scale * p * (dp - sum_j dp*p)           dp fp32, ds `dtype`.
+ * One wavefront per row, fp32 max/sum by cross-lane reduction.
+ * --------------------------------------------------------------------------------------------- */
+int rtp_softmax_fwd(void* stream, int dtype, const float* s, const float* mask, int causal,
+                    float scale, int64_t z, int64_t l, int64_t skv, void* p);
+int rtp_softmax_bwd(void* stream, int dtype, const void* p, const float* dp, float scale,
+                    int64_t z, int64_t l, int64_t skv, void* ds);
+
+/* ---------------------------------------------------------------------------------------------
+ * Top-2 routing (reference: top2gating, rtp/module/top2gate.py:43-105).
+ * Inputs logits[S,E] fp32 and noise[S,E] fp32 (the Gumbel sample of top2gate.py:61, supplied by the
+ * caller so that routing is a pure function of its inputs).  Outputs, per token s:
+ *   expert[s,2] int32, slot[s,2] int32 (location in the expert's capacity buffer, 0 if dropped),
+ *   keep[s,2] int32 (1 if the choice survived the capacity drop and has a non-zero weight),
+ *   weight[s,2] fp32 (renormalised gate probabilities, 0 if dropped), gates[S,E] fp32 (softmax),
+ *   slot_token[E*C] int32 (token occupying each capacity slot, -1 if empty), l_aux fp32 scalar,
+ *   counts[2*E] int32 (first-choice and second-choice totals per expert before the drop).
+ * capacity C = 2*S/E; requires S % E == 0 and E <= 64.
+ * --------------------------------------------------------------------------------------------- */
+size_t rtp_top2_route_workspace_bytes(int64_t s, int64_t e);
+int rtp_top2_route(void* stream, const float* logits, const float* noise, int64_t s, int64_t e,
+                   int32_t* expert, int32_t* slot, int32_t* keep, float* weight, float* gates,
+                   int32_t* slot_token, float* l_aux, int32_t* counts, void* workspace,
+                   size_t workspace_bytes);
+
+/* Backward of the differentiable part of top2gating: d_logits[S,E] from d_weight[S,2] and the
+ * scalar d_l_aux (device pointer, may be NULL for 0). */
+int rtp_top2_route_bwd(void* stream, const float* gates, const int32_t* expert, const int32_t* keep,
+                       const int32_t* counts, const float* d_weight, const float* d_l_aux,
+                       int64_t s, int64_t e, float* d_logits);
+
+/* ---------------------------------------------------------------------------------------------
+ * MoE dispatch / combine (reference: the dense einsums "sec,sm->ecm" rtp/module/moe.py:148 and
+ * "sec,ecm->sm" :174, restated as row moves through the compact routing).
+ *   dispatch: out[e*C + c, :] = x[slot_token[e*C+c], :] * (w ? w-of-that-choice : 1), 0 if empty.
+ *             With weight == NULL this is the forward dispatch; with weight it is the backward of
+ *             combine w.r.t. the expert outputs.
+ *   combine:  out[s,:] = sum_{j<2, keep[s,j]} w[s,j] * y[expert[s,j]*C + slot[s,j], :]
+ *             (weight == NULL means w = 1: the backward of dispatch).
+ *   combine_dweight: dw[s,j] = keep[s,j] ? dot(dout[s,:], y[expert*C+slot, :]) : 0   (fp32).
+ * --------------------------------------------------------------------------------------------- */
+int rtp_moe_dispatch(void* stream, int dtype, const void* x, int64_t ld_x, const int32_t* slot_token,
+                     const int32_t* expert, const int32_t* slot, const float* weight,
+                     int64_t n_slots, int64_t capacity, int64_t cols, void* out, int64_t ld_out);
+int rtp_moe_combine(void* stream, int dtype, const void* y, int64_t ld_y, const int32_t* expert,
+                    const int32_t* slot, const int32_t* keep, const float* weight, int64_t s,
+                    int64_t capacity, int64_t cols, void* out, int64_t ld_out);
+int rtp_moe_combine_dweight(void* stream, int dtype, const void* dout, int64_t ld_dout, const void* y,
+                            int64_t ld_y, const int32_t* expert, const int32_t* slot,
+                            const int32_t* keep, int64_t s, int64_t capacity, int64_t cols,
+                            float* dweight);
+
+/* ---------------------------------------------------------------------------------------------
+ * Optimiser step on a flat shard buffer (reference harness: clip_grad_value_ + optimizer.step,
+ * benchmarks/rtp_benchmark.py:185-186; SGD as the headline configuration asks).
+ *   g = clamp(grad, -clip, clip) if clip > 0;  master -= lr * g;  shadow = (dtype) master.
+ * master fp32; grad `dtype`; shadow `dtype` (may be NULL when dtype is fp32 and the master is the
+ * weight itself).
+ * --------------------------------------------------------------------------------------------- */
+int rtp_sgd_step(void* stream, int dtype, float* master, const void* grad, void* shadow, int64_t n,
+                 float lr, float clip);
+
+/* dst(dtype_dst)[i] = src(dtype_src)[i]  (fp32 <-> bf16 conversion, round to nearest even). */
+int rtp_cast(void* stream, int dtype_src, const void* src, int dtype_dst, void* dst, int64_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RTP_HIP_H */

@@ -1,0 +1,115 @@
+"""ctypes binding of librtp_hip.so (the C ABI declared in include/rtp_hip.h).
+
+The library is the only compute backend of this package: there is no PyTorch or CPU fallback, and
+`load()` raises if the shared object is missing or the device is not gfx950.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Optional
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "librtp_hip.so")
+
+RTP_F32 = 0
+RTP_BF16 = 1
+
+GEMM_OUT_F32 = 1
+GEMM_CIN_F32 = 2
+GEMM_RELU = 4
+
+
+class RtpError(RuntimeError):
+    """A call into librtp_hip.so returned a negative status."""
+
+
+class GemmDesc(C.Structure):
+    _fields_ = [
+        ("a", C.c_void_p), ("b", C.c_void_p), ("c_out", C.c_void_p), ("c_in", C.c_void_p),
+        ("bias", C.c_void_p), ("gate", C.c_void_p),
+        ("m", C.c_int64), ("n", C.c_int64), ("k", C.c_int64),
+        ("lda", C.c_int64), ("ldb", C.c_int64), ("ldc", C.c_int64), ("ld_cin", C.c_int64),
+        ("ld_gate", C.c_int64),
+        ("batch", C.c_int64), ("zdiv", C.c_int64),
+        ("a_so", C.c_int64), ("a_si", C.c_int64), ("b_so", C.c_int64), ("b_si", C.c_int64),
+        ("c_so", C.c_int64), ("c_si", C.c_int64), ("cin_so", C.c_int64), ("cin_si", C.c_int64),
+        ("gate_so", C.c_int64), ("gate_si", C.c_int64), ("bias_so", C.c_int64), ("bias_si", C.c_int64),
+        ("alpha", C.c_float), ("flags", C.c_int32), ("a_kcontig", C.c_int32), ("b_kcontig", C.c_int32),
+    ]
+
+
+_vp, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
+
+# name -> (restype, argtypes); every symbol include/rtp_hip.h declares.
+PROTOTYPES = {
+    "rtp_last_error": (C.c_char_p, []),
+    "rtp_abi_version": (_i, []),
+    "rtp_device_check": (_i, [C.c_char_p, _i]),
+    "rtp_gemm": (_i, [_vp, _i, C.POINTER(GemmDesc)]),
+    "rtp_gemm_desc_size": (_sz, []),
+    "rtp_colsum": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _vp, _i, _i]),
+    "rtp_ring_create": (_i, [C.POINTER(_vp)]),
+    "rtp_ring_destroy": (_i, [_vp]),
+    "rtp_ring_begin": (_i, [_vp, _vp]),
+    "rtp_ring_prefetch": (_i, [_vp, _i, _vp, _vp, _sz]),
+    "rtp_ring_acquire": (_i, [_vp, _vp, _i]),
+    "rtp_ring_release": (_i, [_vp, _vp, _i]),
+    "rtp_shard_copy_async": (_i, [_vp, _vp, _vp, _sz]),
+    "rtp_zero_async": (_i, [_vp, _vp, _sz]),
+    "rtp_embedding_gather": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _i64]),
+    "rtp_embedding_scatter_workspace_bytes": (_sz, [_i64]),
+    "rtp_embedding_sort_ids": (_i, [_vp, _vp, _i64, _vp, _sz]),
+    "rtp_embedding_scatter_add_det": (_i, [_vp, _i, _vp, _i64, _i64, _vp, _vp, _i64, _i, _i64, _i64, _i64,
+                                           _i64, _i, _i]),
+    "rtp_softmax_fwd": (_i, [_vp, _i, _vp, _vp, _i, _f, _i64, _i64, _i64, _vp]),
+    "rtp_softmax_bwd": (_i, [_vp, _i, _vp, _vp, _f, _i64, _i64, _i64, _vp]),
+    "rtp_top2_route_workspace_bytes": (_sz, [_i64, _i64]),
+    "rtp_top2_route": (_i, [_vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz]),
+    "rtp_top2_route_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
+    "rtp_moe_dispatch": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64]),
+    "rtp_moe_combine": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64]),
+    "rtp_moe_combine_dweight": (_i, [_vp, _i, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "rtp_sgd_step": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _f, _f]),
+    "rtp_cast": (_i, [_vp, _i, _vp, _i, _vp, _i64]),
+}
+
+_lib: Optional[C.CDLL] = None
+_device_checked = False
+
+
+def load() -> C.CDLL:
+    """dlopen librtp_hip.so (once) and bind every prototype.  Touches no GPU."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RtpError(
+                f"{LIB_PATH} is missing: build it with `make -C {os.path.join(_HERE, 'csrc')}` "
+                "(or __graft_entry__.build()); there is no fallback backend")
+        lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in PROTOTYPES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        if lib.rtp_gemm_desc_size() != C.sizeof(GemmDesc):
+            raise RtpError("GemmDesc layout differs from the rtp_gemm_desc this library was built with")
+        _lib = lib
+    return _lib
+
+
+def last_error() -> str:
+    return load().rtp_last_error().decode("utf-8", "replace")
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        raise RtpError(f"librtp_hip status {rc}: {last_error()}")
+
+
+def require_device() -> None:
+    """Raise unless the current HIP device is gfx950 (checked once per process)."""
+    global _device_checked
+    if not _device_checked:
+        buf = C.create_string_buffer(64)
+        check(load().rtp_device_check(buf, 64))
+        _device_checked = True

@@ -1,0 +1,195 @@
+// Sharded embedding: coalesced row gather and a deterministic (sorted, segmented) scatter-add.
+#include <cstring>
+
+#include "common.h"
+
+#include <rocprim/rocprim.hpp>
+
+namespace rtp {
+
+// One workgroup per (token, 4 KiB column chunk); 16-byte lanes when the shard rectangle allows it.
+template <typename T>
+__global__ __launch_bounds__(256) void gather_kernel(const T* table, long ld_table, long row_begin, long row_count,
+                                                     long cols, const int64_t* ids, T* out, long ld_out, int vec) {
+  const long t = blockIdx.x;
+  const long row = ids[t] - row_begin;
+  if (row < 0 || row >= row_count) return;
+  const T* src = table + row * ld_table;
+  T* dst = out + t * ld_out;
+  constexpr int VEC = 16 / sizeof(T);
+  if (vec) {
+    const long nvec = cols / VEC;
+    const uint4* s = reinterpret_cast<const uint4*>(src);
+    uint4* d = reinterpret_cast<uint4*>(dst);
+    for (long i = (long)blockIdx.y * 256 + threadIdx.x; i < nvec; i += (long)gridDim.y * 256) d[i] = s[i];
+  } else {
+    for (long i = (long)blockIdx.y * 256 + threadIdx.x; i < cols; i += (long)gridDim.y * 256) dst[i] = src[i];
+  }
+}
+
+__global__ __launch_bounds__(256) void sort_prep_kernel(const int64_t* ids, long n, int* keys, int* vals) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) {
+    keys[i] = (int)ids[i];
+    vals[i] = (int)i;
+  }
+}
+
+__global__ __launch_bounds__(256) void zero_rows_kernel(char* base, long ld_bytes, long row_bytes, long rows) {
+  const long r = blockIdx.x;
+  if (r >= rows) return;
+  char* p = base + r * ld_bytes;
+  if ((((uintptr_t)p | (uintptr_t)row_bytes) & 15) == 0) {
+    uint4* d = reinterpret_cast<uint4*>(p);
+    const uint4 z = make_uint4(0, 0, 0, 0);
+    for (long i = (long)blockIdx.y * 256 + threadIdx.x; i < (row_bytes >> 4); i += (long)gridDim.y * 256) d[i] = z;
+  } else {
+    for (long i = (long)blockIdx.y * 256 + threadIdx.x; i < row_bytes; i += (long)gridDim.y * 256) p[i] = 0;
+  }
+}
+
+// keys: token ids sorted ascending (stable), vals: their positions.  The workgroup at sorted index i
+// owns the segment that starts there (if one does) and sums it front to back, i.e. in ascending
+// position order, starting from +0.0f exactly like a sequential index_add_ into a zeroed table.
+template <typename T, typename G>
+__global__ __launch_bounds__(256) void scatter_kernel(const T* grad_out, long ld_go, long n, const int* keys,
+                                                      const int* vals, G* grad_table, long ld_gt, long row_begin,
+                                                      long row_count, long cols, long padding_idx, int scale_by_freq,
+                                                      int overwrite) {
+  const long i = blockIdx.x;
+  const int id = keys[i];
+  if (i > 0 && keys[i - 1] == id) return;
+  if (id == padding_idx) return;
+  const long row = (long)id - row_begin;
+  if (row < 0 || row >= row_count) return;
+  long end = i + 1;
+  while (end < n && keys[end] == id) ++end;
+  const float inv = scale_by_freq ? 1.0f / (float)(end - i) : 1.0f;
+  for (long c = (long)blockIdx.y * 256 + threadIdx.x; c < cols; c += (long)gridDim.y * 256) {
+    float acc = 0.0f;
+    for (long j = i; j < end; ++j) acc += to_f32(grad_out[(long)vals[j] * ld_go + c]);
+    if (scale_by_freq) acc *= inv;
+    G* dst = grad_table + row * ld_gt + c;
+    if (!overwrite) acc = to_f32(*dst) + acc;
+    *dst = from_f32<G>(acc);
+  }
+}
+
+struct SortLayout {
+  size_t keys_in, vals_in, keys_out, vals_out, temp, total, temp_bytes;
+};
+
+static SortLayout sort_layout(int64_t n) {
+  SortLayout L;
+  const size_t arr = ((size_t)n * 4 + 255) & ~(size_t)255;
+  L.keys_in = 0;
+  L.vals_in = arr;
+  L.keys_out = 2 * arr;
+  L.vals_out = 3 * arr;
+  L.temp = 4 * arr;
+  size_t tb = 0;
+  (void)rocprim::radix_sort_pairs(nullptr, tb, (const int*)nullptr, (int*)nullptr, (const int*)nullptr, (int*)nullptr,
+                                  (unsigned)n, 0, 32, (hipStream_t) nullptr);
+  L.temp_bytes = tb;
+  L.total = L.temp + ((tb + 255) & ~(size_t)255) + 256;
+  return L;
+}
+
+}  // namespace rtp
+
+using namespace rtp;
+
+extern "C" int rtp_embedding_gather(void* stream, int dtype, const void* table, int64_t ld_table, int64_t row_begin,
+                                    int64_t row_count, int64_t cols, const int64_t* ids, int64_t n_ids, void* out,
+                                    int64_t ld_out) {
+  RTP_REQUIRE(table && ids && out, "rtp_embedding_gather: null pointer");
+  RTP_REQUIRE(cols >= 0 && ld_table >= cols && ld_out >= cols && row_count >= 0 && n_ids >= 0,
+              "rtp_embedding_gather: bad shape cols=%lld ld_table=%lld ld_out=%lld", (long long)cols,
+              (long long)ld_table, (long long)ld_out);
+  if (n_ids == 0 || cols == 0) return RTP_OK;
+  RTP_REQUIRE(n_ids < (1ll << 31), "rtp_embedding_gather: too many ids");
+  const size_t esz = dtype == RTP_F32 ? 4 : 2;
+  RTP_REQUIRE(dtype == RTP_F32 || dtype == RTP_BF16, "rtp_embedding_gather: unknown dtype %d", dtype);
+  const int vec = ((uintptr_t)table % 16 == 0) && ((uintptr_t)out % 16 == 0) && (ld_table * esz) % 16 == 0 &&
+                  (ld_out * esz) % 16 == 0 && (cols * esz) % 16 == 0;
+  const unsigned chunks = (unsigned)std::min<int64_t>(16, std::max<int64_t>(1, ceil_div(cols * (int64_t)esz, 4096)));
+  dim3 grid((unsigned)n_ids, chunks);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == RTP_F32)
+    hipLaunchKernelGGL(gather_kernel<float>, grid, dim3(256), 0, s, (const float*)table, (long)ld_table,
+                       (long)row_begin, (long)row_count, (long)cols, ids, (float*)out, (long)ld_out, vec);
+  else
+    hipLaunchKernelGGL(gather_kernel<bf16_t>, grid, dim3(256), 0, s, (const bf16_t*)table, (long)ld_table,
+                       (long)row_begin, (long)row_count, (long)cols, ids, (bf16_t*)out, (long)ld_out, vec);
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
+}
+
+extern "C" size_t rtp_embedding_scatter_workspace_bytes(int64_t n_ids) {
+  if (n_ids <= 0) return 256;
+  return sort_layout(n_ids).total;
+}
+
+extern "C" int rtp_embedding_sort_ids(void* stream, const int64_t* ids, int64_t n_ids, void* workspace,
+                                      size_t workspace_bytes) {
+  RTP_REQUIRE(ids && workspace, "rtp_embedding_sort_ids: null pointer");
+  RTP_REQUIRE(n_ids >= 0 && n_ids < (1ll << 31), "rtp_embedding_sort_ids: bad n_ids %lld", (long long)n_ids);
+  if (n_ids == 0) return RTP_OK;
+  RTP_REQUIRE((uintptr_t)workspace % 256 == 0, "rtp_embedding_sort_ids: workspace must be 256-byte aligned");
+  const SortLayout L = sort_layout(n_ids);
+  if (workspace_bytes < L.total)
+    return fail(RTP_ERR_WORKSPACE, "rtp_embedding_sort_ids: workspace %zu < required %zu", workspace_bytes, L.total);
+  char* w = (char*)workspace;
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(sort_prep_kernel, dim3((unsigned)ceil_div(n_ids, 256)), dim3(256), 0, s, ids, (long)n_ids,
+                     (int*)(w + L.keys_in), (int*)(w + L.vals_in));
+  RTP_LAUNCH_CHECK();
+  size_t tb = L.temp_bytes;
+  RTP_HIP_TRY(rocprim::radix_sort_pairs((void*)(w + L.temp), tb, (const int*)(w + L.keys_in), (int*)(w + L.keys_out),
+                                        (const int*)(w + L.vals_in), (int*)(w + L.vals_out), (unsigned)n_ids, 0, 32,
+                                        s));
+  return RTP_OK;
+}
+
+extern "C" int rtp_embedding_scatter_add_det(void* stream, int dtype, const void* grad_out, int64_t ld_grad_out,
+                                             int64_t n_ids, const void* workspace, void* grad_table,
+                                             int64_t ld_grad_table, int grad_table_f32, int64_t row_begin,
+                                             int64_t row_count, int64_t cols, int64_t padding_idx, int scale_by_freq,
+                                             int zero_fill) {
+  RTP_REQUIRE(grad_out && workspace && grad_table, "rtp_embedding_scatter_add_det: null pointer");
+  RTP_REQUIRE(dtype == RTP_F32 || dtype == RTP_BF16, "rtp_embedding_scatter_add_det: unknown dtype %d", dtype);
+  RTP_REQUIRE(cols >= 0 && ld_grad_out >= cols && ld_grad_table >= cols && row_count >= 0 && n_ids >= 0 &&
+                  n_ids < (1ll << 31),
+              "rtp_embedding_scatter_add_det: bad shape");
+  if (cols == 0 || row_count == 0) return RTP_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const size_t gsz = (dtype == RTP_F32 || grad_table_f32) ? 4 : 2;
+  const unsigned chunks = (unsigned)std::min<int64_t>(16, std::max<int64_t>(1, ceil_div(cols, 1024)));
+  if (zero_fill) {
+    RTP_REQUIRE(row_count < (1ll << 31), "rtp_embedding_scatter_add_det: too many rows");
+    hipLaunchKernelGGL(zero_rows_kernel, dim3((unsigned)row_count, chunks), dim3(256), 0, s, (char*)grad_table,
+                       (long)(ld_grad_table * gsz), (long)(cols * gsz), (long)row_count);
+    RTP_LAUNCH_CHECK();
+  }
+  if (n_ids == 0) return RTP_OK;
+  const SortLayout L = sort_layout(n_ids);
+  const char* w = (const char*)workspace;
+  const int* keys = (const int*)(w + L.keys_out);
+  const int* vals = (const int*)(w + L.vals_out);
+  dim3 grid((unsigned)n_ids, chunks);
+  // After a zero fill the rows can simply be overwritten; otherwise the sum is added to what is there.
+  const int overwrite = zero_fill ? 1 : 0;
+#define RTP_SCATTER(T, G)                                                                                         \
+  hipLaunchKernelGGL((scatter_kernel<T, G>), grid, dim3(256), 0, s, (const T*)grad_out, (long)ld_grad_out,         \
+                     (long)n_ids, keys, vals, (G*)grad_table, (long)ld_grad_table, (long)row_begin, (long)row_count, \
+                     (long)cols, (long)padding_idx, scale_by_freq, overwrite)
+  if (dtype == RTP_F32)
+    RTP_SCATTER(float, float);
+  else if (grad_table_f32)
+    RTP_SCATTER(bf16_t, float);
+  else
+    RTP_SCATTER(bf16_t, bf16_t);
+#undef RTP_SCATTER
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
+}

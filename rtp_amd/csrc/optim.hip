@@ -1,0 +1,67 @@
+// Elementwise passes over flat shard buffers: the fused clip + SGD + shadow-cast step and dtype casts.
+#include "common.h"
+
+namespace rtp {
+
+template <typename T>
+__global__ __launch_bounds__(256) void sgd_kernel(float* master, const T* grad, T* shadow, long n, float lr,
+                                                  float clip) {
+  const long stride = (long)gridDim.x * blockDim.x;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    float g = to_f32(grad[i]);
+    if (clip > 0.0f) g = fminf(fmaxf(g, -clip), clip);
+    const float w = master[i] - lr * g;
+    master[i] = w;
+    if (shadow) shadow[i] = from_f32<T>(w);
+  }
+}
+
+template <typename S, typename D>
+__global__ __launch_bounds__(256) void cast_kernel(const S* src, D* dst, long n) {
+  const long stride = (long)gridDim.x * blockDim.x;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = from_f32<D>(to_f32(src[i]));
+}
+
+static unsigned flat_grid(int64_t n) { return (unsigned)std::min<int64_t>(4096, std::max<int64_t>(1, ceil_div(n, 1024))); }
+
+}  // namespace rtp
+
+using namespace rtp;
+
+extern "C" int rtp_sgd_step(void* stream, int dtype, float* master, const void* grad, void* shadow, int64_t n,
+                            float lr, float clip) {
+  RTP_REQUIRE(master && grad, "rtp_sgd_step: null pointer");
+  RTP_REQUIRE(n >= 0, "rtp_sgd_step: negative length");
+  if (n == 0) return RTP_OK;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == RTP_F32)
+    hipLaunchKernelGGL(sgd_kernel<float>, dim3(flat_grid(n)), dim3(256), 0, s, master, (const float*)grad,
+                       (float*)shadow, (long)n, lr, clip);
+  else if (dtype == RTP_BF16)
+    hipLaunchKernelGGL(sgd_kernel<bf16_t>, dim3(flat_grid(n)), dim3(256), 0, s, master, (const bf16_t*)grad,
+                       (bf16_t*)shadow, (long)n, lr, clip);
+  else
+    return fail(RTP_ERR_ARG, "rtp_sgd_step: unknown dtype %d", dtype);
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
+}
+
+extern "C" int rtp_cast(void* stream, int dtype_src, const void* src, int dtype_dst, void* dst, int64_t n) {
+  RTP_REQUIRE(src && dst, "rtp_cast: null pointer");
+  RTP_REQUIRE(n >= 0, "rtp_cast: negative length");
+  if (n == 0) return RTP_OK;
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid(flat_grid(n));
+  if (dtype_src == RTP_F32 && dtype_dst == RTP_BF16)
+    hipLaunchKernelGGL((cast_kernel<float, bf16_t>), grid, dim3(256), 0, s, (const float*)src, (bf16_t*)dst, (long)n);
+  else if (dtype_src == RTP_BF16 && dtype_dst == RTP_F32)
+    hipLaunchKernelGGL((cast_kernel<bf16_t, float>), grid, dim3(256), 0, s, (const bf16_t*)src, (float*)dst, (long)n);
+  else if (dtype_src == RTP_F32 && dtype_dst == RTP_F32)
+    hipLaunchKernelGGL((cast_kernel<float, float>), grid, dim3(256), 0, s, (const float*)src, (float*)dst, (long)n);
+  else if (dtype_src == RTP_BF16 && dtype_dst == RTP_BF16)
+    hipLaunchKernelGGL((cast_kernel<bf16_t, bf16_t>), grid, dim3(256), 0, s, (const bf16_t*)src, (bf16_t*)dst, (long)n);
+  else
+    return fail(RTP_ERR_ARG, "rtp_cast: unknown dtype pair %d -> %d", dtype_src, dtype_dst);
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
+}

@@ -1,0 +1,183 @@
+// Shard rotation on one GPU: a two-slot staging buffer fed by a copy kernel on a side stream, fenced
+// against the consuming stream with events, plus the error/device plumbing of the C ABI.
+#include "common.h"
+
+#include <cstring>
+
+namespace rtp {
+
+char* error_buffer() {
+  static thread_local char buf[512] = {0};
+  return buf;
+}
+
+struct Ring {
+  hipStream_t side = nullptr;
+  hipEvent_t begin = nullptr;
+  hipEvent_t copied[2] = {nullptr, nullptr};
+  hipEvent_t consumed[2] = {nullptr, nullptr};
+  bool consumed_pending[2] = {false, false};
+  int device = -1;
+};
+
+// 16 bytes per thread per iteration, grid-stride; the ragged head/tail (when the two pointers share
+// an alignment phase) and fully unaligned pairs go byte by byte.
+__global__ __launch_bounds__(256) void copy_kernel(char* dst, const char* src, size_t bytes, int aligned) {
+  const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t nthreads = (size_t)gridDim.x * blockDim.x;
+  if (aligned) {
+    const size_t nvec = bytes >> 4;
+    const uint4* s = reinterpret_cast<const uint4*>(src);
+    uint4* d = reinterpret_cast<uint4*>(dst);
+    size_t i = tid;
+    for (; i + 3 * nthreads < nvec; i += 4 * nthreads) {
+      uint4 v0 = s[i], v1 = s[i + nthreads], v2 = s[i + 2 * nthreads], v3 = s[i + 3 * nthreads];
+      d[i] = v0;
+      d[i + nthreads] = v1;
+      d[i + 2 * nthreads] = v2;
+      d[i + 3 * nthreads] = v3;
+    }
+    for (; i < nvec; i += nthreads) d[i] = s[i];
+    for (size_t b = (nvec << 4) + tid; b < bytes; b += nthreads) dst[b] = src[b];
+  } else {
+    for (size_t b = tid; b < bytes; b += nthreads) dst[b] = src[b];
+  }
+}
+
+__global__ __launch_bounds__(256) void zero_kernel(char* dst, size_t bytes, int aligned) {
+  const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t nthreads = (size_t)gridDim.x * blockDim.x;
+  if (aligned) {
+    const size_t nvec = bytes >> 4;
+    uint4* d = reinterpret_cast<uint4*>(dst);
+    const uint4 z = make_uint4(0, 0, 0, 0);
+    for (size_t i = tid; i < nvec; i += nthreads) d[i] = z;
+    for (size_t b = (nvec << 4) + tid; b < bytes; b += nthreads) dst[b] = 0;
+  } else {
+    for (size_t b = tid; b < bytes; b += nthreads) dst[b] = 0;
+  }
+}
+
+static unsigned copy_grid(size_t bytes) {
+  // Enough workgroups to cover the 256 CUs several times over for large shards, one per 4 KiB
+  // otherwise.
+  size_t blocks = (bytes + 4095) / 4096;
+  if (blocks < 1) blocks = 1;
+  if (blocks > 2048) blocks = 2048;
+  return (unsigned)blocks;
+}
+
+static int launch_copy(hipStream_t s, void* dst, const void* src, size_t bytes) {
+  if (bytes == 0) return RTP_OK;
+  RTP_REQUIRE(dst && src, "shard copy: null pointer");
+  const int aligned = (((uintptr_t)dst | (uintptr_t)src) & 15) == 0;
+  hipLaunchKernelGGL(copy_kernel, dim3(copy_grid(bytes)), dim3(256), 0, s, (char*)dst, (const char*)src, bytes,
+                     aligned);
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
+}
+
+}  // namespace rtp
+
+using namespace rtp;
+
+extern "C" const char* rtp_last_error(void) { return error_buffer(); }
+
+extern "C" int rtp_abi_version(void) { return 1; }
+
+extern "C" int rtp_device_check(char* name_out, int name_len) {
+  int dev = 0;
+  RTP_HIP_TRY(hipGetDevice(&dev));
+  hipDeviceProp_t prop;
+  RTP_HIP_TRY(hipGetDeviceProperties(&prop, dev));
+  if (name_out && name_len > 0) {
+    strncpy(name_out, prop.gcnArchName, (size_t)name_len - 1);
+    name_out[name_len - 1] = 0;
+  }
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(RTP_ERR_DEVICE, "device %d is %s; this library is built for gfx950 only", dev, prop.gcnArchName);
+  return RTP_OK;
+}
+
+extern "C" int rtp_ring_create(void** ring_out) {
+  RTP_REQUIRE(ring_out, "rtp_ring_create: null out pointer");
+  Ring* r = new Ring();
+  RTP_HIP_TRY(hipGetDevice(&r->device));
+  // Default priority on purpose: mixed stream priorities are not used anywhere in this library.
+  RTP_HIP_TRY(hipStreamCreateWithFlags(&r->side, hipStreamNonBlocking));
+  RTP_HIP_TRY(hipEventCreateWithFlags(&r->begin, hipEventDisableTiming));
+  for (int i = 0; i < 2; ++i) {
+    RTP_HIP_TRY(hipEventCreateWithFlags(&r->copied[i], hipEventDisableTiming));
+    RTP_HIP_TRY(hipEventCreateWithFlags(&r->consumed[i], hipEventDisableTiming));
+  }
+  *ring_out = r;
+  return RTP_OK;
+}
+
+extern "C" int rtp_ring_destroy(void* ring) {
+  if (!ring) return RTP_OK;
+  Ring* r = (Ring*)ring;
+  if (r->side) (void)hipStreamSynchronize(r->side);
+  for (int i = 0; i < 2; ++i) {
+    if (r->copied[i]) (void)hipEventDestroy(r->copied[i]);
+    if (r->consumed[i]) (void)hipEventDestroy(r->consumed[i]);
+  }
+  if (r->begin) (void)hipEventDestroy(r->begin);
+  if (r->side) (void)hipStreamDestroy(r->side);
+  delete r;
+  return RTP_OK;
+}
+
+extern "C" int rtp_ring_begin(void* ring, void* main_stream) {
+  RTP_REQUIRE(ring, "rtp_ring_begin: null ring");
+  Ring* r = (Ring*)ring;
+  RTP_HIP_TRY(hipEventRecord(r->begin, (hipStream_t)main_stream));
+  RTP_HIP_TRY(hipStreamWaitEvent(r->side, r->begin, 0));
+  r->consumed_pending[0] = r->consumed_pending[1] = false;
+  return RTP_OK;
+}
+
+extern "C" int rtp_ring_prefetch(void* ring, int slot, void* dst, const void* src, size_t bytes) {
+  RTP_REQUIRE(ring, "rtp_ring_prefetch: null ring");
+  RTP_REQUIRE(slot == 0 || slot == 1, "rtp_ring_prefetch: slot %d not in {0,1}", slot);
+  Ring* r = (Ring*)ring;
+  if (r->consumed_pending[slot]) {
+    RTP_HIP_TRY(hipStreamWaitEvent(r->side, r->consumed[slot], 0));
+    r->consumed_pending[slot] = false;
+  }
+  int rc = launch_copy(r->side, dst, src, bytes);
+  if (rc != RTP_OK) return rc;
+  RTP_HIP_TRY(hipEventRecord(r->copied[slot], r->side));
+  return RTP_OK;
+}
+
+extern "C" int rtp_ring_acquire(void* ring, void* main_stream, int slot) {
+  RTP_REQUIRE(ring, "rtp_ring_acquire: null ring");
+  RTP_REQUIRE(slot == 0 || slot == 1, "rtp_ring_acquire: slot %d not in {0,1}", slot);
+  Ring* r = (Ring*)ring;
+  RTP_HIP_TRY(hipStreamWaitEvent((hipStream_t)main_stream, r->copied[slot], 0));
+  return RTP_OK;
+}
+
+extern "C" int rtp_ring_release(void* ring, void* main_stream, int slot) {
+  RTP_REQUIRE(ring, "rtp_ring_release: null ring");
+  RTP_REQUIRE(slot == 0 || slot == 1, "rtp_ring_release: slot %d not in {0,1}", slot);
+  Ring* r = (Ring*)ring;
+  RTP_HIP_TRY(hipEventRecord(r->consumed[slot], (hipStream_t)main_stream));
+  r->consumed_pending[slot] = true;
+  return RTP_OK;
+}
+
+extern "C" int rtp_shard_copy_async(void* stream, void* dst, const void* src, size_t bytes) {
+  return launch_copy((hipStream_t)stream, dst, src, bytes);
+}
+
+extern "C" int rtp_zero_async(void* stream, void* dst, size_t bytes) {
+  if (bytes == 0) return RTP_OK;
+  RTP_REQUIRE(dst, "rtp_zero_async: null pointer");
+  const int aligned = ((uintptr_t)dst & 15) == 0;
+  hipLaunchKernelGGL(zero_kernel, dim3(copy_grid(bytes)), dim3(256), 0, (hipStream_t)stream, (char*)dst, bytes,
+                     aligned);
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
+}

@@ -1,0 +1,110 @@
+// Row softmax for the attention scores, forward and backward: one wavefront per (batch*head, query)
+// row, fp32 statistics by cross-lane reduction.
+#include "common.h"
+
+namespace rtp {
+
+constexpr int kRowsPerBlock = 4;
+
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_fwd_kernel(const float* s, const float* mask, int causal, float scale,
+                                                          long rows, long l, long skv, T* p) {
+  const int lane = threadIdx.x & 63;
+  const long row = (long)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const long i = row % l;
+  const float* srow = s + row * skv;
+  const float* mrow = mask ? mask + i * skv : nullptr;
+  T* prow = p + row * skv;
+  const long jmax = causal ? (i + (skv - l) + 1 < skv ? i + (skv - l) + 1 : skv) : skv;  // columns [0, jmax) are visible
+
+  float mx = -INFINITY;
+  for (long j = lane; j < jmax; j += kWave) {
+    float v = srow[j] * scale;
+    if (mrow) v += mrow[j];
+    mx = fmaxf(mx, v);
+  }
+  mx = wave_max(mx);
+  float sum = 0.0f;
+  for (long j = lane; j < jmax; j += kWave) {
+    float v = srow[j] * scale;
+    if (mrow) v += mrow[j];
+    sum += expf(v - mx);
+  }
+  sum = wave_sum(sum);
+  const float inv = 1.0f / sum;
+  for (long j = lane; j < skv; j += kWave) {
+    float o = 0.0f;
+    if (j < jmax) {
+      float v = srow[j] * scale;
+      if (mrow) v += mrow[j];
+      o = expf(v - mx) * inv;
+    }
+    prow[j] = from_f32<T>(o);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_bwd_kernel(const T* p, const float* dp, float scale, long rows,
+                                                          long skv, T* ds) {
+  const int lane = threadIdx.x & 63;
+  const long row = (long)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const T* prow = p + row * skv;
+  const float* dprow = dp + row * skv;
+  T* dsrow = ds + row * skv;
+  float dot = 0.0f;
+  for (long j = lane; j < skv; j += kWave) dot += to_f32(prow[j]) * dprow[j];
+  dot = wave_sum(dot);
+  for (long j = lane; j < skv; j += kWave) {
+    const float pv = to_f32(prow[j]);
+    dsrow[j] = from_f32<T>(scale * pv * (dprow[j] - dot));
+  }
+}
+
+}  // namespace rtp
+
+using namespace rtp;
+
+extern "C" int rtp_softmax_fwd(void* stream, int dtype, const float* s, const float* mask, int causal, float scale,
+                               int64_t z, int64_t l, int64_t skv, void* p) {
+  RTP_REQUIRE(s && p, "rtp_softmax_fwd: null pointer");
+  RTP_REQUIRE(z >= 0 && l >= 0 && skv >= 1, "rtp_softmax_fwd: bad shape z=%lld l=%lld s=%lld", (long long)z,
+              (long long)l, (long long)skv);
+  const int64_t rows = z * l;
+  if (rows == 0) return RTP_OK;
+  RTP_REQUIRE(ceil_div(rows, kRowsPerBlock) < (1ll << 31), "rtp_softmax_fwd: too many rows");
+  dim3 grid((unsigned)ceil_div(rows, kRowsPerBlock));
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == RTP_F32)
+    hipLaunchKernelGGL(softmax_fwd_kernel<float>, grid, dim3(256), 0, st, s, mask, causal, scale, (long)rows, (long)l,
+                       (long)skv, (float*)p);
+  else if (dtype == RTP_BF16)
+    hipLaunchKernelGGL(softmax_fwd_kernel<bf16_t>, grid, dim3(256), 0, st, s, mask, causal, scale, (long)rows,
+                       (long)l, (long)skv, (bf16_t*)p);
+  else
+    return fail(RTP_ERR_ARG, "rtp_softmax_fwd: unknown dtype %d", dtype);
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
+}
+
+extern "C" int rtp_softmax_bwd(void* stream, int dtype, const void* p, const float* dp, float scale, int64_t z,
+                               int64_t l, int64_t skv, void* ds) {
+  RTP_REQUIRE(p && dp && ds, "rtp_softmax_bwd: null pointer");
+  RTP_REQUIRE(z >= 0 && l >= 0 && skv >= 1, "rtp_softmax_bwd: bad shape");
+  const int64_t rows = z * l;
+  if (rows == 0) return RTP_OK;
+  RTP_REQUIRE(ceil_div(rows, kRowsPerBlock) < (1ll << 31), "rtp_softmax_bwd: too many rows");
+  dim3 grid((unsigned)ceil_div(rows, kRowsPerBlock));
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == RTP_F32)
+    hipLaunchKernelGGL(softmax_bwd_kernel<float>, grid, dim3(256), 0, st, (const float*)p, dp, scale, (long)rows,
+                       (long)skv, (float*)ds);
+  else if (dtype == RTP_BF16)
+    hipLaunchKernelGGL(softmax_bwd_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)p, dp, scale, (long)rows,
+                       (long)skv, (bf16_t*)ds);
+  else
+    return fail(RTP_ERR_ARG, "rtp_softmax_bwd: unknown dtype %d", dtype);
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
+}

@@ -1,0 +1,167 @@
+"""GPT-2 style nn.Sequential language model built from the rotated layers (counterpart of
+rtp/models/transformer_lm_rtp.py:19-242): embedding * sqrt(ninp) -> sinusoidal positions -> N post-LN
+decoder layers (rotated self-attention + rotated ReLU FFN or rotated MoE) -> rotated logits projection.
+LayerNorm, residual adds, ReLU and dropout are ordinary torch ops."""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn as nn
+
+from ..module.attention import ParallelMultiheadAttention
+from ..module.collectives import emulate_shards
+from ..module.embedding import ParallelEmbedding
+from ..module.linear import ColumnParallelLinear
+from ..module.moe import WeightMOELayer
+from ..module.top2gate import WeightTop2Gate
+
+
+class EmbeddingLayer(nn.Module):
+    def __init__(self, ntoken, ninp, initrange, world_size, rank, device=None, dtype=None):
+        super().__init__()
+        self.embedding = ParallelEmbedding(ntoken, ninp, world_size=world_size, rank=rank, device=device, dtype=dtype)
+        with torch.no_grad():
+            for shard in self.embedding.embeddings:
+                shard.weight.data.uniform_(-initrange, initrange)
+        self.ninp_sqrt = math.sqrt(ninp)
+
+    def forward(self, src):
+        return self.embedding(src) * self.ninp_sqrt
+
+
+class PositionalEncodingLayer(nn.Module):
+    def __init__(self, d_model, dropout=0.1, max_len=5000, device=None, dtype=None):
+        super().__init__()
+        self.dropout = nn.Dropout(p=dropout)
+        pe = torch.zeros(max_len, d_model)
+        position = torch.arange(0, max_len, dtype=torch.float).unsqueeze(1)
+        div_term = torch.exp(torch.arange(0, d_model, 2).float() * (-math.log(10000.0) / d_model))
+        pe[:, 0::2] = torch.sin(position * div_term)
+        pe[:, 1::2] = torch.cos(position * div_term)
+        pe = pe.unsqueeze(0).transpose(0, 1)
+        self.register_buffer("pe", pe.to(device=device, dtype=dtype))
+
+    def forward(self, x):
+        x = x + self.pe[: x.size(0), :]
+        return self.dropout(x)
+
+
+class FeedForwardLayer_expert(nn.Module):
+    """One MoE expert: Linear -> ReLU -> Linear (rtp/models/transformer_lm_rtp.py:63-75)."""
+
+    def __init__(self, d_model, dim_feedforward, activation, dropout, device=None, dtype=None) -> None:
+        super().__init__()
+        self.linear1 = nn.Linear(d_model, dim_feedforward, device=device, dtype=dtype)
+        self.activation = activation
+        self.dropout1 = nn.Dropout(dropout)
+        self.linear2 = nn.Linear(dim_feedforward, d_model, device=device, dtype=dtype)
+        self.dropout2 = nn.Dropout(dropout)
+
+    def forward(self, x):
+        return self.dropout2(self.linear2(self.dropout1(self.activation(self.linear1(x)))))
+
+
+class FeedForwardLayer(nn.Module):
+    def __init__(self, d_model, dim_feedforward, activation, dropout, world_size, rank, device=None, dtype=None):
+        super().__init__()
+        with emulate_shards(world_size):
+            self.linear1 = ColumnParallelLinear(d_model, dim_feedforward, device=device, dtype=dtype)
+            self.linear2 = ColumnParallelLinear(dim_feedforward, d_model, device=device, dtype=dtype)
+        self.activation = activation
+        self.dropout1 = nn.Dropout(dropout)
+        self.dropout2 = nn.Dropout(dropout)
+
+    def forward(self, x):
+        return self.dropout2(self.linear2(self.dropout1(self.activation(self.linear1(x)))))
+
+
+class TransformerEncoderLayer(nn.Module):
+    def __init__(self, d_model, nhead, dim_feedforward=2048, dropout=0.1, activation=nn.ReLU(), layer_norm_eps=1e-5,
+                 norm_first=False, is_moe=False, num_local_experts=1, world_size=1, rank=0, device=None, dtype=None):
+        super().__init__()
+        self.self_attn = ParallelMultiheadAttention(d_model, nhead, dropout=dropout, world_size=world_size,
+                                                    rank=rank, device=device, dtype=dtype)
+        self.norm_first = norm_first
+        self.norm1 = nn.LayerNorm(d_model, eps=layer_norm_eps, device=device, dtype=dtype)
+        self.norm2 = nn.LayerNorm(d_model, eps=layer_norm_eps, device=device, dtype=dtype)
+        self.dropout = nn.Dropout(dropout)
+        self.is_moe = is_moe
+        if is_moe:
+            num_global_experts = num_local_experts * world_size
+            with emulate_shards(world_size):
+                self.gate = WeightTop2Gate(d_model, num_global_experts, device=device, dtype=dtype)
+                experts = nn.ModuleList([
+                    FeedForwardLayer_expert(d_model, dim_feedforward, activation, dropout, device=device, dtype=dtype)
+                    for _ in range(num_local_experts)])
+                self.moe_layer = WeightMOELayer(self.gate, experts, device=device, dtype=dtype)
+        else:
+            self.ff_block = FeedForwardLayer(d_model, dim_feedforward, activation, dropout, world_size=world_size,
+                                             rank=rank, device=device, dtype=dtype)
+
+    def forward(self, src, src_mask=None, src_key_padding_mask=None):
+        x = src
+        if self.norm_first:
+            x = x + self._sa_block(self.norm1(x), src_mask, src_key_padding_mask)
+            x = x + self._ff_block(self.norm2(x))
+        else:
+            x = self.norm1(x + self._sa_block(x, src_mask, src_key_padding_mask))
+            x = self.norm2(x + self._ff_block(x))
+        return x
+
+    def _sa_block(self, x, attn_mask, key_padding_mask):
+        x = self.self_attn(x, x, x, attn_mask=attn_mask, key_padding_mask=key_padding_mask, need_weights=False)[0]
+        return self.dropout(x)
+
+    def _ff_block(self, x):
+        return self.moe_layer(x) if self.is_moe else self.ff_block(x)
+
+
+class TransformerDecoderLayer(TransformerEncoderLayer):
+    """Encoder layer with a cached square subsequent (-inf above the diagonal) float mask."""
+
+    def __init__(self, ninp, nhead, nhid, dropout, is_moe=False, num_local_experts=1, world_size=1, rank=0,
+                 device=None, dtype=None):
+        super().__init__(ninp, nhead, nhid, dropout, is_moe=is_moe, num_local_experts=num_local_experts,
+                         world_size=world_size, rank=rank, device=device, dtype=dtype)
+        self.src_mask = None
+
+    def _generate_square_subsequent_mask(self, sz):
+        mask = (torch.triu(torch.ones(sz, sz)) == 1).transpose(0, 1)
+        return mask.float().masked_fill(mask == 0, float("-inf")).masked_fill(mask == 1, float(0.0))
+
+    def forward(self, src):
+        if self.src_mask is None or self.src_mask.size(0) != len(src) or self.src_mask.device != src.device:
+            self.src_mask = self._generate_square_subsequent_mask(len(src)).to(src.device)
+        return super().forward(src, self.src_mask)
+
+
+class LinearLayer(nn.Module):
+    def __init__(self, ninp, ntoken, initrange, world_size, rank, device=None, dtype=None):
+        super().__init__()
+        with emulate_shards(world_size):
+            self.linear = ColumnParallelLinear(ninp, ntoken, device=device, dtype=dtype)
+        with torch.no_grad():
+            for shard in self.linear.linears:
+                shard.bias.data.zero_()
+                shard.weight.data.uniform_(-initrange, initrange)
+
+    def forward(self, src):
+        return self.linear(src)
+
+
+class TransformerLM(nn.Sequential):
+    """Constructor follows rtp/models/transformer_lm_rtp.py:233.  `world_size` is the number of rotation
+    shards emulated on the one device; `rank` must be 0."""
+
+    def __init__(self, ntokens, ninp, nhead, nhid, dropout, initrange, ndecoder, world_size, rank, is_moe=False,
+                 num_local_experts=1, device=None, dtype=None):
+        layers = [
+            EmbeddingLayer(ntokens, ninp, initrange, world_size, rank, device=device, dtype=dtype),
+            PositionalEncodingLayer(ninp, dropout, device=device, dtype=dtype),
+        ]
+        for _ in range(ndecoder):
+            layers.append(TransformerDecoderLayer(ninp, nhead, nhid, dropout, is_moe, num_local_experts,
+                                                  world_size=world_size, rank=rank, device=device, dtype=dtype))
+        layers.append(LinearLayer(ninp, ntokens, initrange, world_size, rank, device=device, dtype=dtype))
+        super().__init__(*layers)

@@ -1,0 +1,125 @@
+"""Rotated sharded Embedding (counterpart of rtp/module/embedding.py:33-164).
+
+The table is split along the embedding dimension: shard s is the [V, D/ws] column block s of the
+master table (embedding.py:65-71) and fills column block s of the output.  Forward gathers rows from
+the staged shard; backward builds each shard's dense [V, D/ws] gradient with a sorted, segmented
+scatter-add whose per-row summation order is ascending token position, which reproduces torch's CPU
+nn.Embedding backward bit for bit.  The backward needs no weights, so it runs no rotation.
+"""
+from __future__ import annotations
+
+from typing import Callable, Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.init as init
+
+from .. import ops
+from ..ring import Rotation, ring_order
+from .collectives import RotatedLayer
+from .utils import affine_weight, divide_and_check_no_remainder
+
+
+class ModelParallelEmbedding(nn.Embedding):
+    """One column block of the table (rtp/module/embedding.py:33-71)."""
+
+    def __init__(self, num_embeddings: int, embedding_dim: int, world_size: int, rank: int,
+                 padding_idx: Optional[int] = None, max_norm: Optional[float] = None, norm_type: float = 2.0,
+                 scale_grad_by_freq: bool = False, sparse: bool = False,
+                 init_method: Callable[[torch.Tensor], torch.Tensor] = init.xavier_normal_,
+                 keep_master_weight_for_test: bool = False, device=None, dtype=None) -> None:
+        self.world_size = world_size
+        self.rank = rank
+        self.embedding_dim_per_partition = divide_and_check_no_remainder(embedding_dim, world_size)
+        super().__init__(num_embeddings, self.embedding_dim_per_partition, padding_idx, max_norm, norm_type,
+                         scale_grad_by_freq, sparse, device=device, dtype=dtype)
+
+    def affine_weight(self, Embedding_layer) -> None:
+        if Embedding_layer is not None:
+            affine_weight(self.weight, Embedding_layer.weight, self.embedding_dim_per_partition, 1, self.world_size,
+                          self.rank)
+
+
+class _EmbeddingFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, ids, anchor, layer):
+        store = layer._store
+        d_s, ws = layer.embedding_dim_per_partition, layer.world_size
+        flat_ids = ids.reshape(-1).contiguous()
+        out = torch.empty(flat_ids.numel(), layer.embedding_dim, dtype=store.home.dtype, device=store.home.device)
+        order = ring_order(layer.rank, ws)
+        rot = Rotation(store.home, order)
+        for i, idx in enumerate(order):
+            table = store.views(rot.acquire(i))[0]
+            ops.embedding_gather(table, flat_ids, out[:, idx * d_s:(idx + 1) * d_s])
+            rot.release(i)
+        ctx.layer = layer
+        ctx.save_for_backward(flat_ids)
+        return out.view(*ids.shape, layer.embedding_dim)
+
+    @staticmethod
+    def backward(ctx, dout):
+        layer = ctx.layer
+        (flat_ids,) = ctx.saved_tensors
+        store = layer._store
+        d_s, ws = layer.embedding_dim_per_partition, layer.world_size
+        g2 = dout.reshape(-1, layer.embedding_dim)
+        if g2.stride(1) != 1:
+            g2 = g2.contiguous()
+        workspace = ops.embedding_sort_ids(flat_ids)
+        pad = -1 if layer.padding_idx is None else layer.padding_idx
+        for idx in ring_order(layer.rank, ws, reverse=True):
+            grads, accumulate = store.grad_views(idx)
+            ops.embedding_scatter_add(g2[:, idx * d_s:(idx + 1) * d_s], flat_ids.numel(), workspace, grads[0],
+                                      padding_idx=pad, scale_by_freq=layer.scale_grad_by_freq,
+                                      zero_fill=not accumulate)
+        return None, None, None
+
+
+class ParallelEmbedding(RotatedLayer):
+    """Embedding sharded along the embedding dimension and rotated.  Signature follows
+    rtp/module/embedding.py:85-101; `Embedding_layer` imports the table of an unsharded nn.Embedding.
+    `max_norm` and `sparse` gradients are not implemented by the kernels and raise."""
+
+    def __init__(self, num_embeddings: int, embedding_dim: int, world_size: int, rank: int,
+                 padding_idx: Optional[int] = None, max_norm: Optional[float] = None, norm_type: float = 2.0,
+                 scale_grad_by_freq: bool = False, sparse: bool = False,
+                 init_method: Callable[[torch.Tensor], torch.Tensor] = init.xavier_normal_,
+                 keep_master_weight_for_test: bool = False, Embedding_layer: Optional[nn.Embedding] = None,
+                 device=None, dtype=None) -> None:
+        super().__init__()
+        if max_norm is not None:
+            raise NotImplementedError("ParallelEmbedding: max_norm renormalisation is not implemented")
+        if sparse:
+            raise NotImplementedError("ParallelEmbedding: sparse gradients are not implemented")
+        self.num_embeddings = num_embeddings
+        self.embedding_dim = embedding_dim
+        if padding_idx is not None and padding_idx < 0:
+            padding_idx = num_embeddings + padding_idx
+        self.padding_idx = padding_idx
+        self.max_norm = max_norm
+        self.norm_type = norm_type
+        self.scale_grad_by_freq = scale_grad_by_freq
+        self.sparse = sparse
+        self.world_size = world_size
+        self.rank = rank
+        self.embedding_dim_per_partition = divide_and_check_no_remainder(embedding_dim, world_size)
+        if Embedding_layer is not None and device is None:
+            device = Embedding_layer.weight.device
+        if Embedding_layer is not None and dtype is None:
+            dtype = Embedding_layer.weight.dtype
+        embeddings = []
+        for s in range(world_size):
+            shard = ModelParallelEmbedding(num_embeddings, embedding_dim, world_size, s, padding_idx, max_norm,
+                                           norm_type, scale_grad_by_freq, sparse, init_method,
+                                           keep_master_weight_for_test, device=device, dtype=dtype)
+            shard.affine_weight(Embedding_layer)
+            embeddings.append(shard)
+        self._init_store(embeddings)
+        self.embeddings = list(self.shards)
+        self.embedding = self.embeddings[self.rank]
+
+    def forward(self, input_: torch.Tensor) -> torch.Tensor:
+        if input_.dtype != torch.int64:
+            input_ = input_.long()
+        return _EmbeddingFn.apply(input_, self._anchor, self)

@@ -1,0 +1,209 @@
+"""Rotated column- and row-parallel Linear (counterparts of rtp/module/linear.py:137-305 and :307-476).
+
+Forward runs one rotation over the `ws` weight shards: at step i the shard (rank+i) % ws is in the
+staging slot, its GEMM writes straight into its column block of the output (column-parallel; the
+reference's torch.cat at linear.py:222 disappears) or accumulates into the output (row-parallel,
+linear.py:389-392), while the next shard streams into the other slot.  Backward walks the shards in the
+reverse order, needs each shard once more for the input gradient, and writes each shard's weight/bias
+gradient straight into its home gradient row (the reference's gradient ring, collectives.py:196-200,
+has nothing left to carry on one device).
+"""
+from __future__ import annotations
+
+from typing import Callable, Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.init as init
+
+from .. import ops
+from ..ring import Rotation, ring_order
+from .collectives import RotatedLayer, resolve_world
+from .utils import affine_weight, as_rows, divide_and_check_no_remainder
+
+
+class ModelParallelLinear(nn.Linear):
+    """One column shard: rows [rank*N/ws, (rank+1)*N/ws) of the master weight and bias
+    (rtp/module/linear.py:32-82)."""
+
+    def __init__(self, in_features: int, out_features: int, world_size: int, rank: int, bias: bool = True,
+                 device=None, dtype=None):
+        self.world_size = world_size
+        self.rank = rank
+        self.output_size_per_partition = divide_and_check_no_remainder(out_features, world_size)
+        super().__init__(in_features, self.output_size_per_partition, bias, device=device, dtype=dtype)
+
+    def affine_weight(self, linear_layer) -> None:
+        if linear_layer is not None:
+            affine_weight(self.weight, linear_layer.weight, self.output_size_per_partition, 0, self.world_size,
+                          self.rank)
+            if self.bias is not None:
+                affine_weight(self.bias, linear_layer.bias, self.output_size_per_partition, 0, self.world_size,
+                              self.rank)
+
+
+class ModelParallelLinear2(nn.Linear):
+    """One row shard: columns [rank*K/ws, (rank+1)*K/ws) of the master weight; every shard carries
+    bias/ws so that the sum over shards restores the bias (rtp/module/linear.py:84-135)."""
+
+    def __init__(self, in_features: int, out_features: int, world_size: int, rank: int, bias: bool = True,
+                 device=None, dtype=None):
+        self.world_size = world_size
+        self.rank = rank
+        self.input_size_per_partition = divide_and_check_no_remainder(in_features, world_size)
+        super().__init__(self.input_size_per_partition, out_features, bias, device=device, dtype=dtype)
+
+    def affine_weight(self, linear_layer) -> None:
+        if linear_layer is not None:
+            affine_weight(self.weight, linear_layer.weight, self.input_size_per_partition, 1, self.world_size,
+                          self.rank)
+            if self.bias is not None:
+                with torch.no_grad():
+                    self.bias.data.copy_(linear_layer.bias.data)
+                    self.bias.data.div_(self.world_size)
+
+
+class _ColumnLinearFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, anchor, layer):
+        store = layer._store
+        n_s, k, ws = layer.output_size_per_partition, layer.in_features, layer.world_size
+        x2 = as_rows(x, k)
+        y = torch.empty(x2.shape[0], layer.out_features, dtype=x2.dtype, device=x2.device)
+        order = ring_order(layer.rank, ws)
+        rot = Rotation(store.home, order)
+        for i, idx in enumerate(order):
+            views = store.views(rot.acquire(i))
+            ops.linear_fwd(x2, views[0], y[:, idx * n_s:(idx + 1) * n_s], bias=views[1] if layer.has_bias else None)
+            rot.release(i)
+        ctx.layer = layer
+        ctx.x_shape = x.shape
+        ctx.save_for_backward(x2)
+        return y.view(*x.shape[:-1], layer.out_features)
+
+    @staticmethod
+    def backward(ctx, dy):
+        layer = ctx.layer
+        (x2,) = ctx.saved_tensors
+        store = layer._store
+        n_s, ws = layer.output_size_per_partition, layer.world_size
+        dy2 = as_rows(dy, layer.out_features)
+        need_dx = ctx.needs_input_grad[0]
+        dx = torch.empty_like(x2) if need_dx else None
+        acc = ops.ShardSum(dx, ws) if need_dx else None
+        order = ring_order(layer.rank, ws, reverse=True)
+        rot = Rotation(store.home, order) if need_dx else None
+        for i, idx in enumerate(order):
+            dy_s = dy2[:, idx * n_s:(idx + 1) * n_s]
+            if need_dx:
+                w = store.views(rot.acquire(i))[0]
+                c_out, c_in = acc.target(i)
+                ops.linear_dgrad(dy_s, w, c_out, c_in=c_in)
+                rot.release(i)
+            grads, accumulate = store.grad_views(idx)
+            ops.linear_wgrad(dy_s, x2, grads[0], c_in=grads[0] if accumulate else None)
+            if layer.has_bias:
+                ops.colsum(dy_s, grads[1], accumulate=accumulate)
+        return (dx.view(ctx.x_shape) if need_dx else None), None, None
+
+
+class _RowLinearFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, anchor, layer):
+        store = layer._store
+        k_s, ws = layer.input_size_per_partition, layer.world_size
+        x2 = as_rows(x, layer.in_features)
+        y = torch.empty(x2.shape[0], layer.out_features, dtype=x2.dtype, device=x2.device)
+        acc = ops.ShardSum(y, ws)
+        order = ring_order(layer.rank, ws)
+        rot = Rotation(store.home, order)
+        for i, idx in enumerate(order):
+            views = store.views(rot.acquire(i))
+            c_out, c_in = acc.target(i)
+            ops.linear_fwd(x2[:, idx * k_s:(idx + 1) * k_s], views[0], c_out, c_in=c_in,
+                           bias=views[1] if layer.has_bias else None)
+            rot.release(i)
+        ctx.layer = layer
+        ctx.x_shape = x.shape
+        ctx.save_for_backward(x2)
+        return y.view(*x.shape[:-1], layer.out_features)
+
+    @staticmethod
+    def backward(ctx, dy):
+        layer = ctx.layer
+        (x2,) = ctx.saved_tensors
+        store = layer._store
+        k_s, ws = layer.input_size_per_partition, layer.world_size
+        dy2 = as_rows(dy, layer.out_features)
+        need_dx = ctx.needs_input_grad[0]
+        dx = torch.empty_like(x2) if need_dx else None
+        order = ring_order(layer.rank, ws, reverse=True)
+        rot = Rotation(store.home, order) if need_dx else None
+        for i, idx in enumerate(order):
+            x_s = x2[:, idx * k_s:(idx + 1) * k_s]
+            if need_dx:
+                w = store.views(rot.acquire(i))[0]
+                ops.linear_dgrad(dy2, w, dx[:, idx * k_s:(idx + 1) * k_s])
+                rot.release(i)
+            grads, accumulate = store.grad_views(idx)
+            ops.linear_wgrad(dy2, x_s, grads[0], c_in=grads[0] if accumulate else None)
+            if layer.has_bias:
+                # every shard's bias (= b/ws) receives the full column sum (tests/test_linear.py:181-186)
+                ops.colsum(dy2, grads[1], accumulate=accumulate)
+        return (dx.view(ctx.x_shape) if need_dx else None), None, None
+
+
+class _ParallelLinearBase(RotatedLayer):
+    _shard_cls = None
+    _fn = None
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, gather_weight: bool = True,
+                 init_method: Callable[[torch.Tensor], torch.Tensor] = init.xavier_normal_, stride: int = 1,
+                 keep_master_weight_for_test: bool = False, device=None, dtype=None, group=None,
+                 linear_layer: Optional[nn.Linear] = None) -> None:
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.gather_weight = gather_weight
+        self.group = group
+        self.world_size, self.rank = resolve_world(group)
+        self.has_bias = bias
+        self.output_size_per_partition = divide_and_check_no_remainder(out_features, self.world_size) \
+            if self._shard_cls is ModelParallelLinear else out_features
+        self.input_size_per_partition = divide_and_check_no_remainder(in_features, self.world_size) \
+            if self._shard_cls is ModelParallelLinear2 else in_features
+        if linear_layer is not None and device is None:
+            device = linear_layer.weight.device
+        if linear_layer is not None and dtype is None:
+            dtype = linear_layer.weight.dtype
+        linears = []
+        for s in range(self.world_size):
+            shard = self._shard_cls(in_features, out_features, world_size=self.world_size, rank=s, bias=bias,
+                                    device=device, dtype=dtype)
+            shard.affine_weight(linear_layer)
+            linears.append(shard)
+        self._init_store(linears)
+        self.linears = list(self.shards)
+        self.linear = self.linears[self.rank]
+
+    def forward(self, input_: torch.Tensor) -> torch.Tensor:
+        return type(self)._fn.apply(input_, self._anchor, self)
+
+    def extra_repr(self) -> str:
+        return (f"in_features={self.in_features}, out_features={self.out_features}, bias={self.has_bias}, "
+                f"shards={self.world_size}")
+
+
+class ColumnParallelLinear(_ParallelLinearBase):
+    """Y = X W^T + b with W split into `ws` row blocks (output columns); outputs of the shards are
+    laid side by side.  Constructor arguments follow rtp/module/linear.py:158-171; `linear_layer`
+    imports the weights of an unsharded nn.Linear."""
+    _shard_cls = ModelParallelLinear
+    _fn = _ColumnLinearFn
+
+
+class RowParallelLinear(_ParallelLinearBase):
+    """Y = sum_s X[:, s-block] W_s^T + ws * (b/ws) with W split into `ws` column blocks
+    (rtp/module/linear.py:328-407)."""
+    _shard_cls = ModelParallelLinear2
+    _fn = _RowLinearFn

@@ -1,0 +1,163 @@
+"""GShard top-2 gate with a rotated, expert-sharded gate projection (counterpart of
+rtp/module/top2gate.py:25-220).
+
+The routing decisions come from the HIP routing kernels as compact per-token records; the dense
+[S,E,C] combine/dispatch tensors of the reference API are materialised only when a caller asks the
+gate module for them directly.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+import torch.nn as nn
+from torch import Tensor
+
+from .. import ops
+from ..ring import Rotation, ring_order
+from .collectives import RotatedLayer, resolve_world
+from .utils import affine_weight, as_rows, divide_and_check_no_remainder
+
+
+def gumbel_rsample(shape, device: torch.device) -> Tensor:
+    """Gumbel(0,1) noise for the second-expert choice (rtp/module/top2gate.py:25-32)."""
+    one = torch.tensor(1.0, device=device)
+    zero = torch.tensor(0.0, device=device)
+    return torch.distributions.gumbel.Gumbel(zero, one).rsample(shape)
+
+
+class _RouteFn(torch.autograd.Function):
+    """logits[S,E] (+ noise) -> (weight[S,2], l_aux); the integer routing rides on `holder`."""
+
+    @staticmethod
+    def forward(ctx, logits, noise, holder):
+        r = ops.top2_route(logits.float().contiguous(), noise.float().contiguous())
+        holder.append(r)
+        ctx.routing = r
+        ctx.in_dtype = logits.dtype
+        return r.weight, r.l_aux
+
+    @staticmethod
+    def backward(ctx, d_weight, d_l_aux):
+        d_logits = ops.top2_route_bwd(ctx.routing, d_weight, d_l_aux)
+        return d_logits.to(ctx.in_dtype), None, None
+
+
+def top2_route(logits: Tensor, noise: Optional[Tensor] = None):
+    """Differentiable compact routing: returns (routing, weight[S,2], l_aux)."""
+    if noise is None:
+        noise = gumbel_rsample(logits.shape, logits.device)
+    holder = []
+    weight, l_aux = _RouteFn.apply(logits, noise, holder)
+    return holder[0], weight, l_aux
+
+
+def dense_from_routing(r: ops.Routing, weight: Tensor, dtype: torch.dtype) -> Tuple[Tensor, Tensor]:
+    """The reference's combine_weights[S,E,C] and dispatch_mask[S,E,C] (top2gate.py:95-103), built from
+    the compact routing.  API compatibility only: the MoE layer never forms these."""
+    s_idx = torch.arange(r.s, device=weight.device).repeat_interleave(2)
+    e_idx = r.expert.reshape(-1).long()
+    c_idx = r.slot.reshape(-1).long()
+    vals = (weight * r.keep.to(weight.dtype)).reshape(-1)
+    combine = torch.zeros(r.s, r.e, r.capacity, dtype=weight.dtype, device=weight.device)
+    combine = combine.index_put((s_idx, e_idx, c_idx), vals, accumulate=True)
+    return combine.to(dtype), combine.bool()
+
+
+def top2gating(logits: Tensor, noise: Optional[Tensor] = None) -> Tuple[Tensor, Tensor, Tensor]:
+    """(l_aux, combine_weights, dispatch_mask) as rtp/module/top2gate.py:43-105 returns them."""
+    r, weight, l_aux = top2_route(logits, noise)
+    combine, dispatch = dense_from_routing(r, weight, logits.dtype)
+    return l_aux.to(logits.dtype), combine, dispatch
+
+
+class _GateProjectionFn(torch.autograd.Function):
+    """logits[S,E] = x[S,M] @ wg^T with wg's expert rows sharded and rotated; fp32 logits."""
+
+    @staticmethod
+    def forward(ctx, x, anchor, layer):
+        store = layer._store
+        ws, e_s = layer.world_size, layer.num_local_experts
+        x2 = as_rows(x, layer.model_dim)
+        logits = torch.empty(x2.shape[0], layer.num_experts, dtype=torch.float32, device=x2.device)
+        order = ring_order(layer.rank, ws)
+        rot = Rotation(store.home, order)
+        for i, idx in enumerate(order):
+            w = store.views(rot.acquire(i))[0]
+            ops.linear_fwd(x2, w, logits[:, idx * e_s:(idx + 1) * e_s])
+            rot.release(i)
+        ctx.layer = layer
+        ctx.save_for_backward(x2)
+        return logits
+
+    @staticmethod
+    def backward(ctx, d_logits):
+        layer = ctx.layer
+        (x2,) = ctx.saved_tensors
+        store = layer._store
+        ws, e_s = layer.world_size, layer.num_local_experts
+        dl = d_logits.to(x2.dtype).contiguous()
+        need_dx = ctx.needs_input_grad[0]
+        dx = torch.empty_like(x2) if need_dx else None
+        acc = ops.ShardSum(dx, ws) if need_dx else None
+        order = ring_order(layer.rank, ws, reverse=True)
+        rot = Rotation(store.home, order) if need_dx else None
+        for i, idx in enumerate(order):
+            dl_s = dl[:, idx * e_s:(idx + 1) * e_s]
+            if need_dx:
+                w = store.views(rot.acquire(i))[0]
+                c_out, c_in = acc.target(i)
+                ops.linear_dgrad(dl_s, w, c_out, c_in=c_in)
+                rot.release(i)
+            grads, accumulate = store.grad_views(idx)
+            ops.linear_wgrad(dl_s, x2, grads[0], c_in=grads[0] if accumulate else None)
+        return dx, None, None
+
+
+class Top2Gate(nn.Module):
+    """Unsharded gate (rtp/module/top2gate.py:109-137): the master a WeightTop2Gate can be built from."""
+
+    def __init__(self, model_dim: int, num_experts: int) -> None:
+        super().__init__()
+        self.wg = nn.Linear(model_dim, num_experts, bias=False)
+
+    def forward(self, input: Tensor, noise: Optional[Tensor] = None) -> Tuple[Tensor, Tensor, Tensor]:
+        raise NotImplementedError("Top2Gate only carries master weights here; use WeightTop2Gate(gate=...)")
+
+
+class WeightTop2Gate(RotatedLayer):
+    """Signature follows rtp/module/top2gate.py:157-164.  forward(input[S,M]) returns the reference's
+    (l_aux, combine_weights[S,E,C], dispatch_mask[S,E,C]); route() returns the compact form the MoE
+    layer uses.  `noise` (fp32 [S,E]) may be passed to make the second choice reproducible."""
+
+    def __init__(self, model_dim: int, num_experts: int, gate: Optional[nn.Module] = None, device=None,
+                 dtype=None) -> None:
+        super().__init__()
+        self.model_dim = model_dim
+        self.num_experts = num_experts
+        self.world_size, self.rank = resolve_world(None)
+        self.num_local_experts = divide_and_check_no_remainder(num_experts, self.world_size)
+        if gate is not None and device is None:
+            device = gate.wg.weight.device
+        if gate is not None and dtype is None:
+            dtype = gate.wg.weight.dtype
+        wgs = []
+        for s in range(self.world_size):
+            wg = nn.Linear(model_dim, self.num_local_experts, bias=False, device=device, dtype=dtype)
+            if gate is not None:
+                affine_weight(wg.weight, gate.wg.weight, self.num_local_experts, 0, self.world_size, s)
+            wgs.append(wg)
+        self._init_store(wgs)
+        self.wgs = list(self.shards)
+        self.wg = self.wgs[self.rank]
+
+    def logits(self, input: Tensor) -> Tensor:
+        return _GateProjectionFn.apply(input, self._anchor, self)
+
+    def route(self, input: Tensor, noise: Optional[Tensor] = None):
+        return top2_route(self.logits(input), noise)
+
+    def forward(self, input: Tensor, noise: Optional[Tensor] = None) -> Tuple[Tensor, Tensor, Tensor]:
+        r, weight, l_aux = self.route(input, noise)
+        combine, dispatch = dense_from_routing(r, weight, input.dtype)
+        return l_aux.to(input.dtype), combine, dispatch

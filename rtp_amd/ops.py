@@ -1,0 +1,372 @@
+"""Tensor-level wrappers over the C ABI: they validate shapes/strides on the host, pass raw device
+pointers plus the current torch stream to librtp_hip.so, and never compute anything themselves."""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional
+
+import torch
+
+from . import _lib
+from ._lib import GEMM_CIN_F32, GEMM_OUT_F32, GEMM_RELU, RTP_BF16, RTP_F32, GemmDesc, check
+
+_DT = {torch.float32: RTP_F32, torch.bfloat16: RTP_BF16}
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    try:
+        return _DT[dt]
+    except KeyError:
+        raise TypeError(f"rtp_amd kernels support float32 and bfloat16, got {dt}") from None
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t: torch.Tensor) -> None:
+    if not t.is_cuda:
+        raise _lib.RtpError("rtp_amd kernels run on the GPU only; got a CPU tensor (there is no CPU path)")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _mat(t: torch.Tensor, what: str):
+    """(rows, cols, ld) of a 2-D tensor whose last dim is contiguous."""
+    if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise ValueError(f"{what}: need a 2-D tensor with unit column stride, got shape {tuple(t.shape)} "
+                         f"strides {t.stride()}")
+    ld = t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1)
+    return t.shape[0], t.shape[1], max(ld, 1)
+
+
+def gemm_raw(dtype: torch.dtype, *, a: int, b: int, c_out: int, m: int, n: int, k: int, lda: int, ldb: int,
+             ldc: int, a_kcontig: bool, b_kcontig: bool, c_in: Optional[int] = None, ld_cin: int = 0,
+             bias: Optional[int] = None, gate: Optional[int] = None, ld_gate: int = 0, alpha: float = 1.0,
+             relu: bool = False, out_f32: bool = False, cin_f32: bool = False, batch: int = 1, zdiv: int = 1,
+             a_s=(0, 0), b_s=(0, 0), c_s=(0, 0), cin_s=(0, 0), gate_s=(0, 0), bias_s=(0, 0)) -> None:
+    """One rtp_gemm call on raw device addresses (see include/rtp_hip.h for the operand rules)."""
+    _lib.require_device()
+    d = GemmDesc()
+    d.a, d.b, d.c_out, d.c_in, d.bias, d.gate = a, b, c_out, c_in, bias, gate
+    d.m, d.n, d.k = m, n, k
+    d.lda, d.ldb, d.ldc, d.ld_cin, d.ld_gate = lda, ldb, ldc, ld_cin, ld_gate
+    d.batch, d.zdiv = batch, zdiv
+    d.a_so, d.a_si = a_s
+    d.b_so, d.b_si = b_s
+    d.c_so, d.c_si = c_s
+    d.cin_so, d.cin_si = cin_s
+    d.gate_so, d.gate_si = gate_s
+    d.bias_so, d.bias_si = bias_s
+    d.alpha = alpha
+    d.flags = (GEMM_OUT_F32 if out_f32 else 0) | (GEMM_CIN_F32 if cin_f32 else 0) | (GEMM_RELU if relu else 0)
+    d.a_kcontig, d.b_kcontig = int(a_kcontig), int(b_kcontig)
+    check(_lib.load().rtp_gemm(_stream(), dtype_code(dtype), C.byref(d)))
+
+
+def _epilogue_args(dtype, out, c_in, bias, gate):
+    kw = {}
+    if out.dtype == torch.float32 and dtype != torch.float32:
+        kw["out_f32"] = True
+    elif out.dtype != dtype:
+        raise TypeError(f"gemm output must be {dtype} or float32, got {out.dtype}")
+    if c_in is not None:
+        _, _, ld = _mat(c_in, "c_in")
+        if c_in.shape != out.shape:
+            raise ValueError(f"c_in shape {tuple(c_in.shape)} != output shape {tuple(out.shape)}")
+        kw["c_in"], kw["ld_cin"] = c_in.data_ptr(), ld
+        if c_in.dtype == torch.float32 and dtype != torch.float32:
+            kw["cin_f32"] = True
+        elif c_in.dtype != dtype:
+            raise TypeError(f"c_in must be {dtype} or float32, got {c_in.dtype}")
+    if bias is not None:
+        if bias.dtype != dtype or bias.dim() != 1 or bias.shape[0] != out.shape[1] or not bias.is_contiguous():
+            raise ValueError("bias must be a contiguous vector of the output width and the compute dtype")
+        kw["bias"] = bias.data_ptr()
+    if gate is not None:
+        _, _, ld = _mat(gate, "gate")
+        if gate.shape != out.shape or gate.dtype != dtype:
+            raise ValueError("gate must match the output shape and the compute dtype")
+        kw["gate"], kw["ld_gate"] = gate.data_ptr(), ld
+    return kw
+
+
+def linear_fwd(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, bias=None, c_in=None, relu=False,
+               alpha: float = 1.0) -> None:
+    """out[M,N] = epilogue(x[M,K] @ w[N,K]^T)   (F.linear of one shard)."""
+    for t in (x, w, out):
+        _dev(t)
+    m, k, lda = _mat(x, "x")
+    n, k2, ldb = _mat(w, "w")
+    mo, no, ldc = _mat(out, "out")
+    if k != k2 or mo != m or no != n or x.dtype != w.dtype:
+        raise ValueError(f"linear_fwd: x {tuple(x.shape)} {x.dtype}, w {tuple(w.shape)} {w.dtype}, "
+                         f"out {tuple(out.shape)}")
+    gemm_raw(x.dtype, a=x.data_ptr(), b=w.data_ptr(), c_out=out.data_ptr(), m=m, n=n, k=k, lda=lda, ldb=ldb,
+             ldc=ldc, a_kcontig=True, b_kcontig=True, relu=relu, alpha=alpha,
+             **_epilogue_args(x.dtype, out, c_in, bias, None))
+
+
+def linear_dgrad(dy: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, c_in=None, gate=None) -> None:
+    """out[M,K] = epilogue(dy[M,N] @ w[N,K])   (input gradient of F.linear)."""
+    for t in (dy, w, out):
+        _dev(t)
+    m, n, lda = _mat(dy, "dy")
+    n2, k, ldb = _mat(w, "w")
+    mo, ko, ldc = _mat(out, "out")
+    if n != n2 or mo != m or ko != k or dy.dtype != w.dtype:
+        raise ValueError(f"linear_dgrad: dy {tuple(dy.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
+    # contraction index is n: A = dy (n contiguous), B(kk, n) = w[n, kk] (stored n-major -> not k-contig)
+    gemm_raw(dy.dtype, a=dy.data_ptr(), b=w.data_ptr(), c_out=out.data_ptr(), m=m, n=k, k=n, lda=lda, ldb=ldb,
+             ldc=ldc, a_kcontig=True, b_kcontig=False, **_epilogue_args(dy.dtype, out, c_in, None, gate))
+
+
+def linear_wgrad(dy: torch.Tensor, x: torch.Tensor, out: torch.Tensor, *, c_in=None) -> None:
+    """out[N,K] = epilogue(dy[M,N]^T @ x[M,K])   (weight gradient of F.linear)."""
+    for t in (dy, x, out):
+        _dev(t)
+    m, n, lda = _mat(dy, "dy")
+    m2, k, ldb = _mat(x, "x")
+    no, ko, ldc = _mat(out, "out")
+    if m != m2 or no != n or ko != k or dy.dtype != x.dtype:
+        raise ValueError(f"linear_wgrad: dy {tuple(dy.shape)}, x {tuple(x.shape)}, out {tuple(out.shape)}")
+    gemm_raw(dy.dtype, a=dy.data_ptr(), b=x.data_ptr(), c_out=out.data_ptr(), m=n, n=k, k=m, lda=lda, ldb=ldb,
+             ldc=ldc, a_kcontig=False, b_kcontig=False, **_epilogue_args(dy.dtype, out, c_in, None, None))
+
+
+def colsum(x: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+    """out[N] (+)= sum over rows of x[M,N]   (bias gradient)."""
+    _dev(x)
+    _dev(out)
+    m, n, ld = _mat(x, "x")
+    if out.dim() != 1 or out.shape[0] != n or not out.is_contiguous():
+        raise ValueError("colsum: out must be a contiguous vector of x's width")
+    if out.dtype not in (x.dtype, torch.float32):
+        raise TypeError("colsum: out must be the input dtype or float32")
+    _lib.require_device()
+    check(_lib.load().rtp_colsum(_stream(), dtype_code(x.dtype), x.data_ptr(), m, n, ld, out.data_ptr(),
+                                 int(out.dtype == torch.float32), int(accumulate)))
+
+
+def shard_copy(dst: torch.Tensor, src: torch.Tensor) -> None:
+    """dst <- src with the rotation copy kernel on the current stream."""
+    _dev(dst)
+    _dev(src)
+    if not (dst.is_contiguous() and src.is_contiguous()) or dst.numel() * dst.element_size() != \
+            src.numel() * src.element_size():
+        raise ValueError("shard_copy: need contiguous tensors of equal byte size")
+    _lib.require_device()
+    check(_lib.load().rtp_shard_copy_async(_stream(), dst.data_ptr(), src.data_ptr(),
+                                           src.numel() * src.element_size()))
+
+
+def zero_(t: torch.Tensor) -> None:
+    _dev(t)
+    if not t.is_contiguous():
+        raise ValueError("zero_: need a contiguous tensor")
+    _lib.require_device()
+    check(_lib.load().rtp_zero_async(_stream(), t.data_ptr(), t.numel() * t.element_size()))
+
+
+def embedding_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, row_begin: int = 0) -> None:
+    """out[t, :] = table[ids[t] - row_begin, :] for ids inside the shard's row range."""
+    for t in (table, ids, out):
+        _dev(t)
+    rows, cols, ld_t = _mat(table, "table")
+    n, cols_o, ld_o = _mat(out, "out")
+    if ids.dtype != torch.int64 or not ids.is_contiguous() or ids.numel() != n or cols_o != cols or \
+            out.dtype != table.dtype:
+        raise ValueError("embedding_gather: ids must be contiguous int64 with one id per output row")
+    _lib.require_device()
+    check(_lib.load().rtp_embedding_gather(_stream(), dtype_code(table.dtype), table.data_ptr(), ld_t, row_begin,
+                                           rows, cols, ids.data_ptr(), n, out.data_ptr(), ld_o))
+
+
+def embedding_sort_ids(ids: torch.Tensor) -> torch.Tensor:
+    """Sorted (id, position) workspace shared by the scatter-adds of all shards of one backward."""
+    _dev(ids)
+    if ids.dtype != torch.int64 or not ids.is_contiguous():
+        raise ValueError("embedding_sort_ids: ids must be contiguous int64")
+    _lib.require_device()
+    lib = _lib.load()
+    nbytes = lib.rtp_embedding_scatter_workspace_bytes(ids.numel())
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=ids.device)
+    check(lib.rtp_embedding_sort_ids(_stream(), ids.data_ptr(), ids.numel(), ws.data_ptr(), nbytes))
+    return ws
+
+
+def embedding_scatter_add(grad_out: torch.Tensor, n_ids: int, workspace: torch.Tensor, grad_table: torch.Tensor,
+                          *, row_begin: int = 0, padding_idx: int = -1, scale_by_freq: bool = False,
+                          zero_fill: bool = True) -> None:
+    for t in (grad_out, workspace, grad_table):
+        _dev(t)
+    n, cols, ld_go = _mat(grad_out, "grad_out")
+    rows, cols_t, ld_gt = _mat(grad_table, "grad_table")
+    if n != n_ids or cols != cols_t:
+        raise ValueError("embedding_scatter_add: shape mismatch")
+    if grad_table.dtype not in (grad_out.dtype, torch.float32):
+        raise TypeError("embedding_scatter_add: grad_table must be the grad dtype or float32")
+    _lib.require_device()
+    check(_lib.load().rtp_embedding_scatter_add_det(
+        _stream(), dtype_code(grad_out.dtype), grad_out.data_ptr(), ld_go, n_ids, workspace.data_ptr(),
+        grad_table.data_ptr(), ld_gt, int(grad_table.dtype == torch.float32), row_begin, rows, cols,
+        -1 if padding_idx is None else padding_idx, int(scale_by_freq), int(zero_fill)))
+
+
+def softmax_fwd(scores: torch.Tensor, p: torch.Tensor, *, mask: Optional[torch.Tensor], causal: bool,
+                scale: float) -> None:
+    """p[Z,L,S] = softmax(scale*scores + mask) row-wise; scores fp32, mask fp32 [L,S] or None."""
+    _dev(scores)
+    _dev(p)
+    if scores.dtype != torch.float32 or scores.dim() != 3 or not scores.is_contiguous() or \
+            p.shape != scores.shape or not p.is_contiguous():
+        raise ValueError("softmax_fwd: scores must be contiguous fp32 [Z,L,S] and p the same shape")
+    z, l, s = scores.shape
+    if mask is not None:
+        if mask.dtype != torch.float32 or tuple(mask.shape) != (l, s) or not mask.is_contiguous():
+            raise ValueError("softmax_fwd: mask must be contiguous fp32 [L,S]")
+    _lib.require_device()
+    check(_lib.load().rtp_softmax_fwd(_stream(), dtype_code(p.dtype), scores.data_ptr(), _ptr(mask), int(causal),
+                                      scale, z, l, s, p.data_ptr()))
+
+
+def softmax_bwd(p: torch.Tensor, dp: torch.Tensor, ds: torch.Tensor, scale: float) -> None:
+    _dev(p)
+    if dp.dtype != torch.float32 or p.dim() != 3 or dp.shape != p.shape or ds.shape != p.shape or \
+            ds.dtype != p.dtype or not (p.is_contiguous() and dp.is_contiguous() and ds.is_contiguous()):
+        raise ValueError("softmax_bwd: need contiguous p/ds [Z,L,S] of one dtype and fp32 dp")
+    z, l, s = p.shape
+    _lib.require_device()
+    check(_lib.load().rtp_softmax_bwd(_stream(), dtype_code(p.dtype), p.data_ptr(), dp.data_ptr(), scale, z, l, s,
+                                      ds.data_ptr()))
+
+
+def sgd_step(master: torch.Tensor, grad: torch.Tensor, shadow: Optional[torch.Tensor], lr: float,
+             clip: float = 0.0) -> None:
+    _dev(master)
+    if master.dtype != torch.float32 or not master.is_contiguous() or not grad.is_contiguous() or \
+            grad.numel() != master.numel():
+        raise ValueError("sgd_step: master must be contiguous fp32 and grad the same length")
+    if shadow is not None and (shadow.dtype != grad.dtype or shadow.numel() != master.numel() or
+                               not shadow.is_contiguous()):
+        raise ValueError("sgd_step: shadow must match grad dtype and master length")
+    _lib.require_device()
+    check(_lib.load().rtp_sgd_step(_stream(), dtype_code(grad.dtype), master.data_ptr(), grad.data_ptr(),
+                                   _ptr(shadow), master.numel(), lr, clip))
+
+
+def cast(src: torch.Tensor, dst: torch.Tensor) -> None:
+    _dev(src)
+    _dev(dst)
+    if not (src.is_contiguous() and dst.is_contiguous()) or src.numel() != dst.numel():
+        raise ValueError("cast: need contiguous tensors of equal length")
+    _lib.require_device()
+    check(_lib.load().rtp_cast(_stream(), dtype_code(src.dtype), src.data_ptr(), dtype_code(dst.dtype),
+                               dst.data_ptr(), src.numel()))
+
+
+class ShardSum:
+    """Accumulation plan for a result that is summed over the shard steps of a rotation
+    (row-parallel outputs, attention out-projections, input gradients).  fp32 results accumulate in
+    place; bf16 results accumulate in an fp32 scratch and are rounded once, by the last step."""
+
+    def __init__(self, out: torch.Tensor, steps: int):
+        self.out = out
+        self.steps = steps
+        self.scratch = None
+        if out.dtype != torch.float32 and steps > 1:
+            self.scratch = torch.empty(out.shape, dtype=torch.float32, device=out.device)
+
+    def target(self, i: int):
+        """(c_out, c_in) for step i."""
+        if self.scratch is None:
+            return self.out, (self.out if i > 0 else None)
+        if i == self.steps - 1:
+            return self.out, self.scratch
+        return self.scratch, (self.scratch if i > 0 else None)
+
+
+class Routing:
+    """Compact result of top-2 routing for S tokens over E experts with capacity C = 2S/E."""
+
+    __slots__ = ("s", "e", "capacity", "expert", "slot", "keep", "weight", "gates", "slot_token", "l_aux", "counts")
+
+
+def top2_route(logits: torch.Tensor, noise: torch.Tensor) -> Routing:
+    """Run the routing kernels on fp32 logits[S,E] and noise[S,E]."""
+    _dev(logits)
+    _dev(noise)
+    if logits.dtype != torch.float32 or noise.dtype != torch.float32 or logits.dim() != 2 or \
+            noise.shape != logits.shape or not (logits.is_contiguous() and noise.is_contiguous()):
+        raise ValueError("top2_route: logits and noise must be contiguous fp32 [S,E]")
+    s, e = logits.shape
+    assert s % e == 0, "num_tokens must be a multiple of num_experts"
+    dev = logits.device
+    r = Routing()
+    r.s, r.e, r.capacity = s, e, 2 * s // e
+    r.expert = torch.empty(s, 2, dtype=torch.int32, device=dev)
+    r.slot = torch.empty(s, 2, dtype=torch.int32, device=dev)
+    r.keep = torch.empty(s, 2, dtype=torch.int32, device=dev)
+    r.weight = torch.empty(s, 2, dtype=torch.float32, device=dev)
+    r.gates = torch.empty(s, e, dtype=torch.float32, device=dev)
+    r.slot_token = torch.empty(2 * s, dtype=torch.int32, device=dev)
+    r.l_aux = torch.empty((), dtype=torch.float32, device=dev)
+    r.counts = torch.empty(2 * e, dtype=torch.int32, device=dev)
+    _lib.require_device()
+    lib = _lib.load()
+    nbytes = lib.rtp_top2_route_workspace_bytes(s, e)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    check(lib.rtp_top2_route(_stream(), logits.data_ptr(), noise.data_ptr(), s, e, r.expert.data_ptr(),
+                             r.slot.data_ptr(), r.keep.data_ptr(), r.weight.data_ptr(), r.gates.data_ptr(),
+                             r.slot_token.data_ptr(), r.l_aux.data_ptr(), r.counts.data_ptr(), ws.data_ptr(), nbytes))
+    return r
+
+
+def top2_route_bwd(r: Routing, d_weight: torch.Tensor, d_l_aux: Optional[torch.Tensor]) -> torch.Tensor:
+    d_weight = d_weight.contiguous().float()
+    d_logits = torch.empty(r.s, r.e, dtype=torch.float32, device=r.gates.device)
+    if d_l_aux is not None:
+        d_l_aux = d_l_aux.contiguous().float()
+    check(_lib.load().rtp_top2_route_bwd(_stream(), r.gates.data_ptr(), r.expert.data_ptr(), r.keep.data_ptr(),
+                                         r.counts.data_ptr(), d_weight.data_ptr(), _ptr(d_l_aux), r.s, r.e,
+                                         d_logits.data_ptr()))
+    return d_logits
+
+
+def moe_dispatch(x: torch.Tensor, r: Routing, out: torch.Tensor, weight: Optional[torch.Tensor] = None) -> None:
+    """out[E*C, M]: row e*C+c = x[token in that slot] (times its combine weight if `weight`), else 0."""
+    _dev(x)
+    rows, cols, ld_x = _mat(x, "x")
+    n_slots, cols_o, ld_o = _mat(out, "out")
+    if rows != r.s or cols != cols_o or n_slots != r.e * r.capacity or out.dtype != x.dtype:
+        raise ValueError("moe_dispatch: shape mismatch")
+    check(_lib.load().rtp_moe_dispatch(_stream(), dtype_code(x.dtype), x.data_ptr(), ld_x, r.slot_token.data_ptr(),
+                                       r.expert.data_ptr(), r.slot.data_ptr(), _ptr(weight), n_slots, r.capacity,
+                                       cols, out.data_ptr(), ld_o))
+
+
+def moe_combine(y: torch.Tensor, r: Routing, out: torch.Tensor, weight: Optional[torch.Tensor]) -> None:
+    """out[s,:] = sum over the kept choices of token s of weight * y[expert*C + slot, :]."""
+    _dev(y)
+    n_slots, cols, ld_y = _mat(y, "y")
+    rows, cols_o, ld_o = _mat(out, "out")
+    if rows != r.s or cols != cols_o or n_slots != r.e * r.capacity or out.dtype != y.dtype:
+        raise ValueError("moe_combine: shape mismatch")
+    check(_lib.load().rtp_moe_combine(_stream(), dtype_code(y.dtype), y.data_ptr(), ld_y, r.expert.data_ptr(),
+                                      r.slot.data_ptr(), r.keep.data_ptr(), _ptr(weight), r.s, r.capacity, cols,
+                                      out.data_ptr(), ld_o))
+
+
+def moe_combine_dweight(dout: torch.Tensor, y: torch.Tensor, r: Routing) -> torch.Tensor:
+    _dev(dout)
+    rows, cols, ld_d = _mat(dout, "dout")
+    n_slots, cols_y, ld_y = _mat(y, "y")
+    if rows != r.s or cols != cols_y or dout.dtype != y.dtype:
+        raise ValueError("moe_combine_dweight: shape mismatch")
+    dw = torch.empty(r.s, 2, dtype=torch.float32, device=dout.device)
+    check(_lib.load().rtp_moe_combine_dweight(_stream(), dtype_code(y.dtype), dout.data_ptr(), ld_d, y.data_ptr(),
+                                              ld_y, r.expert.data_ptr(), r.slot.data_ptr(), r.keep.data_ptr(), r.s,
+                                              r.capacity, cols, dw.data_ptr()))
+    return dw

@@ -1,0 +1,64 @@
+"""Optimiser step over the flat shard buffers (the harness step of benchmarks/rtp_benchmark.py:185-186:
+clip_grad_value_ then optimizer.step), as one fused kernel launch per rotated layer.
+
+For bf16 layers the optimiser owns an fp32 master copy of every flat shard buffer; the step updates
+the master and rounds it into the bf16 weights the kernels read.  For fp32 layers the weights are
+their own master.  Parameters outside rotated layers (LayerNorm) are flattened the same way.
+"""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+import torch.nn as nn
+
+from . import ops
+from .module.collectives import ShardStore
+
+
+class RotatedSGD:
+    def __init__(self, model: nn.Module, lr: float, clip_value: float = 0.0):
+        self.lr = float(lr)
+        self.clip_value = float(clip_value)
+        self.stores: List[ShardStore] = []
+        rotated_params = set()
+        for m in model.modules():
+            st = getattr(m, "_store", None)
+            if isinstance(st, ShardStore) and st not in self.stores:
+                self.stores.append(st)
+                for sm in st.modules:
+                    rotated_params.update(id(p) for p in sm.parameters())
+        self.other = [p for p in model.parameters() if id(p) not in rotated_params and p.requires_grad]
+        self.masters = [None if st.home.dtype == torch.float32 else st.home.float() for st in self.stores]
+        self.other_masters = [None if p.dtype == torch.float32 else p.detach().float().clone() for p in self.other]
+
+    def master_bytes(self) -> int:
+        n = sum(m.numel() * 4 for m in self.masters if m is not None)
+        return n + sum(m.numel() * 4 for m in self.other_masters if m is not None)
+
+    def zero_grad(self) -> None:
+        for st in self.stores:
+            for sm in st.modules:
+                for p in sm.parameters():
+                    p.grad = None
+        for p in self.other:
+            p.grad = None
+
+    @torch.no_grad()
+    def step(self) -> None:
+        for st, master in zip(self.stores, self.masters):
+            if st.grads is None:
+                continue
+            home, grads = st.home.view(-1), st.grads.view(-1)
+            if master is None:
+                ops.sgd_step(home, grads, None, self.lr, self.clip_value)
+            else:
+                ops.sgd_step(master.view(-1), grads, home, self.lr, self.clip_value)
+        for p, master in zip(self.other, self.other_masters):
+            if p.grad is None:
+                continue
+            g = p.grad.contiguous().view(-1)
+            if master is None:
+                ops.sgd_step(p.data.view(-1), g, None, self.lr, self.clip_value)
+            else:
+                ops.sgd_step(master.view(-1), g, p.data.view(-1), self.lr, self.clip_value)

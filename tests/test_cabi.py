@@ -1,0 +1,62 @@
+"""The C-ABI library loads without a GPU and exports exactly the symbols include/rtp_hip.h declares;
+the ctypes prototypes cover the same set.  No compute call is made."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "rtp_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(rtp_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_entry_points():
+    names = _declared()
+    assert "rtp_gemm" in names and "rtp_ring_prefetch" in names and "rtp_embedding_scatter_add_det" in names
+    assert len(names) >= 25
+
+
+def test_library_exports_every_declared_symbol():
+    from rtp_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("librtp_hip.so not built (run __graft_entry__.build())")
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in _declared():
+        assert hasattr(lib, name), f"{name} declared in rtp_hip.h but not exported"
+
+
+def test_ctypes_prototypes_cover_the_header():
+    from rtp_amd import _lib
+    assert sorted(_lib.PROTOTYPES) == _declared()
+
+
+def test_loader_binds_and_reports_version():
+    from rtp_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("librtp_hip.so not built")
+    lib = _lib.load()
+    assert lib.rtp_abi_version() == 1
+    assert isinstance(_lib.last_error(), str)
+
+
+def test_gemm_desc_matches_c_layout():
+    from rtp_amd import _lib
+    # 6 pointers + 22 int64 + float + 3 int32
+    assert ctypes.sizeof(_lib.GemmDesc) == 6 * 8 + 22 * 8 + 4 + 3 * 4
+    if os.path.exists(_lib.LIB_PATH):
+        assert _lib.load().rtp_gemm_desc_size() == ctypes.sizeof(_lib.GemmDesc)
+
+
+def test_ops_refuse_cpu_tensors():
+    """There is no CPU fallback: a CPU tensor is an error, not a slow path."""
+    import torch
+    from rtp_amd import _lib, ops
+    with pytest.raises(_lib.RtpError):
+        ops.linear_fwd(torch.zeros(2, 2), torch.zeros(2, 2), torch.zeros(2, 2))
+    with pytest.raises(_lib.RtpError):
+        ops.embedding_gather(torch.zeros(2, 2), torch.zeros(2, dtype=torch.long), torch.zeros(2, 2))

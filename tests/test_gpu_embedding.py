@@ -1,0 +1,79 @@
+"""Rotated ParallelEmbedding: gather and deterministic scatter-add must be bit-exact against the oracle
+(== torch CPU nn.Embedding), including the headline configuration and edge cases."""
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+from gpu_util import DEV
+from oracle import rtp_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _layer(master, ws, dtype=torch.float32, **kw):
+    from rtp_amd.module.embedding import ParallelEmbedding
+    return ParallelEmbedding(master.num_embeddings, master.embedding_dim, ws, 0, Embedding_layer=master, device=DEV,
+                             dtype=dtype, **kw)
+
+
+def _check(master, ids, g, ws, padding_idx=None):
+    layer = _layer(master, ws, padding_idx=padding_idx)
+    out = layer(ids.to(DEV))
+    ref = O.parallel_embedding(ids, master.weight.detach(), ws)
+    assert torch.equal(out.cpu(), ref), "gather is not bit-exact"
+    out.backward(g.to(DEV))
+    dw = torch.cat([e.weight.grad for e in layer.embeddings], dim=1).cpu().numpy()  # gather rule: cat on dim 1
+    ref_dw = O.embedding_backward_sequential(ids.numpy(), g.numpy(), master.num_embeddings, padding_idx)
+    assert np.array_equal(dw, ref_dw), f"scatter-add differs in {(dw != ref_dw).sum()} elements"
+    return layer
+
+
+@pytest.mark.parametrize("ws", [1, 2, 4])
+def test_embedding_reference_shape(ws):
+    """nn.Embedding(8,8), ids [8,8] in [0,7) as in tests/test_embedding.py: every row is hit ~9 times."""
+    master = nn.Embedding(8, 8)
+    ids = torch.randint(0, 7, (8, 8))
+    layer = _check(master, ids, torch.randn(8, 8, 8), ws)
+    assert layer.embedding.weight.shape == (8, 8 // ws)
+
+
+def test_embedding_headline_config():
+    """table [10240,2048] ~U(-0.1,0.1), 4 shards, ids [32,32], upstream grad ~N(0,1)."""
+    gen = torch.Generator().manual_seed(0)
+    master = nn.Embedding(10240, 2048)
+    with torch.no_grad():
+        master.weight.copy_(torch.rand(10240, 2048, generator=gen) * 0.2 - 0.1)
+    ids = torch.randint(0, 10240, (32, 32), generator=gen)
+    g = torch.randn(32, 32, 2048, generator=gen)
+    layer = _check(master, ids, g, 4)
+    # and against torch's own CPU backward
+    master(ids).backward(g)
+    dw = torch.cat([e.weight.grad for e in layer.embeddings], dim=1).cpu()
+    assert torch.equal(dw, master.weight.grad)
+
+
+def test_embedding_heavy_duplicates_ragged_and_padding():
+    master = nn.Embedding(5, 12)
+    ids = torch.randint(0, 5, (257,))  # long segments, odd length
+    _check(master, ids, torch.randn(257, 12), 4)
+    _check(master, torch.full((64,), 3), torch.randn(64, 12), 2)  # a single segment
+    _check(master, ids, torch.randn(257, 12), 2, padding_idx=2)
+    _check(master, torch.tensor([4]), torch.randn(1, 12), 1)  # one token
+
+
+def test_embedding_bf16_and_idempotence():
+    master = nn.Embedding(50, 32)
+    ids = torch.randint(0, 50, (9, 7))
+    layer = _layer(master.to(torch.bfloat16), 4, torch.bfloat16)
+    out = layer(ids.to(DEV))
+    assert torch.equal(out.cpu(), master.weight.detach()[ids]), "bf16 gather is not bit-exact"
+    assert torch.equal(layer(ids.to(DEV)), out)
+
+
+def test_embedding_unsupported_options_raise():
+    from rtp_amd.module.embedding import ParallelEmbedding
+    with pytest.raises(NotImplementedError):
+        ParallelEmbedding(8, 8, 2, 0, max_norm=1.0, device=DEV)
+    with pytest.raises(NotImplementedError):
+        ParallelEmbedding(8, 8, 2, 0, sparse=True, device=DEV)

@@ -1,0 +1,123 @@
+"""rtp_gemm through the C ABI: every operand layout, both dtypes, ragged sizes, batching by strides and
+the fused epilogue, against float64 matmul on the CPU."""
+import pytest
+import torch
+
+from gpu_util import DEV, TOL, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _ops():
+    from rtp_amd import ops
+    return ops
+
+
+def _rand(shape, dtype, gen):
+    return (torch.randn(shape, generator=gen) * 0.5).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("akc,bkc", [(True, True), (True, False), (False, True), (False, False)])
+@pytest.mark.parametrize("m,n,k", [(8, 8, 8), (33, 65, 17), (100, 36, 70), (256, 192, 128), (1024, 256, 520)])
+def test_gemm_layouts(dtype, akc, bkc, m, n, k):
+    ops = _ops()
+    gen = torch.Generator().manual_seed(m * 31 + n * 7 + k)
+    a = _rand((m, k) if akc else (k, m), dtype, gen)
+    b = _rand((n, k) if bkc else (k, n), dtype, gen)
+    A = a.double() if akc else a.double().t()
+    B = b.double() if bkc else b.double().t()
+    ref = A @ B.t()
+    ad, bd = a.to(DEV), b.to(DEV)
+    out = torch.full((m, n), float("nan"), dtype=dtype, device=DEV)
+    ops.gemm_raw(dtype, a=ad.data_ptr(), b=bd.data_ptr(), c_out=out.data_ptr(), m=m, n=n, k=k,
+                 lda=ad.stride(0), ldb=bd.stride(0), ldc=n, a_kcontig=akc, b_kcontig=bkc)
+    torch.cuda.synchronize()
+    assert rel_err(out, ref) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gemm_big_tile_path(dtype):
+    """Enough 128x128 tiles to take the large-tile kernel, with ragged edges."""
+    ops = _ops()
+    gen = torch.Generator().manual_seed(5)
+    m, n, k = 1900, 1700, 300
+    a, b = _rand((m, k), dtype, gen), _rand((n, k), dtype, gen)
+    ref = a.double() @ b.double().t()
+    ad, bd = a.to(DEV), b.to(DEV)
+    out = torch.empty(m, n, dtype=dtype, device=DEV)
+    ops.linear_fwd(ad, bd, out)
+    assert rel_err(out, ref) <= TOL[dtype]
+    # weight-gradient and input-gradient layouts on the same path
+    dy = _rand((m, n), dtype, gen).to(DEV)
+    dx = torch.empty(m, k, dtype=dtype, device=DEV)
+    ops.linear_dgrad(dy, bd, dx)
+    assert rel_err(dx, dy.double().cpu() @ b.double()) <= TOL[dtype]
+    dw = torch.empty(n, k, dtype=dtype, device=DEV)
+    ops.linear_wgrad(dy, ad, dw)
+    assert rel_err(dw, dy.double().cpu().t() @ a.double()) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gemm_epilogue(dtype):
+    ops = _ops()
+    gen = torch.Generator().manual_seed(9)
+    m, n, k = 70, 50, 40
+    x, w = _rand((m, k), dtype, gen), _rand((n, k), dtype, gen)
+    bias, cin, gate = _rand((n,), dtype, gen), _rand((m, n), dtype, gen), _rand((m, n), dtype, gen)
+    base = x.double() @ w.double().t()
+    xd, wd = x.to(DEV), w.to(DEV)
+    out = torch.empty(m, n, dtype=dtype, device=DEV)
+    ops.linear_fwd(xd, wd, out, bias=bias.to(DEV), relu=True)
+    assert rel_err(out, torch.relu(base + bias.double())) <= TOL[dtype]
+    # accumulate in place, fp32 accumulator, strided output block
+    wide = torch.zeros(m, 3 * n, dtype=torch.float32, device=DEV)
+    blk = wide[:, n:2 * n]
+    blk.copy_(cin.float())
+    ops.linear_fwd(xd, wd, blk, c_in=blk)
+    assert rel_err(blk, base + cin.double()) <= TOL[dtype]
+    assert wide[:, :n].abs().max() == 0 and wide[:, 2 * n:].abs().max() == 0
+    # relu-mask epilogue of the input-gradient GEMM
+    dy = _rand((m, n), dtype, gen)
+    gk = _rand((m, k), dtype, gen)
+    dx = torch.empty(m, k, dtype=dtype, device=DEV)
+    ops.linear_dgrad(dy.to(DEV), wd, dx, gate=gk.to(DEV))
+    assert rel_err(dx, (dy.double() @ w.double()) * (gk.double() > 0)) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gemm_batched_by_strides(dtype):
+    """(batch, head) pairs addressed inside a packed [L, N, 3*E_s] projection, as attention does."""
+    ops = _ops()
+    gen = torch.Generator().manual_seed(13)
+    L, N, h, d = 20, 3, 2, 16
+    e_s = h * d
+    qkv = _rand((L, N, 3 * e_s), dtype, gen)
+    q = qkv[..., :e_s].reshape(L, N, h, d).permute(1, 2, 0, 3).double()
+    k = qkv[..., e_s:2 * e_s].reshape(L, N, h, d).permute(1, 2, 0, 3).double()
+    ref = q @ k.transpose(-1, -2)
+    qd = qkv.to(DEV)
+    out = torch.empty(N * h, L, L, dtype=torch.float32, device=DEV)
+    esz = qd.element_size()
+    ops.gemm_raw(dtype, a=qd.data_ptr(), b=qd.data_ptr() + e_s * esz, c_out=out.data_ptr(), m=L, n=L, k=d,
+                 lda=N * 3 * e_s, ldb=N * 3 * e_s, ldc=L, a_kcontig=True, b_kcontig=True, batch=N * h, zdiv=h,
+                 a_s=(3 * e_s, d), b_s=(3 * e_s, d), c_s=(h * L * L, L * L), out_f32=True)
+    assert rel_err(out.view(N, h, L, L), ref) <= TOL[dtype]
+
+
+def test_colsum_and_errors():
+    ops = _ops()
+    from rtp_amd._lib import RtpError
+    x = torch.randn(300, 70)
+    out = torch.empty(70, device=DEV)
+    ops.colsum(x.to(DEV), out)
+    assert rel_err(out, x.double().sum(0)) <= 1e-5
+    ops.colsum(x.to(DEV), out, accumulate=True)
+    assert rel_err(out, 2 * x.double().sum(0)) <= 1e-5
+    xb = x.bfloat16()
+    outb = torch.empty(70, dtype=torch.bfloat16, device=DEV)
+    ops.colsum(xb.to(DEV)[:, 10:40], outb[:30].clone().contiguous())
+    with pytest.raises(RtpError):
+        ops.linear_fwd(torch.randn(4, 4), torch.randn(4, 4), torch.empty(4, 4))  # CPU tensors: no fallback
+    with pytest.raises(ValueError):
+        ops.linear_fwd(x.to(DEV), torch.randn(5, 71, device=DEV), torch.empty(300, 5, device=DEV))

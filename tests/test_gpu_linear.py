@@ -1,0 +1,125 @@
+"""Rotated Column/RowParallelLinear through the drop-in API vs the CPU oracle (and nn.Linear), with the
+reference tests' gather rules for the gradients (tests/test_linear.py:117-186)."""
+import pytest
+import torch
+import torch.nn as nn
+
+from gpu_util import DEV, assert_close
+from oracle import rtp_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _build(cls_name, master, ws, dtype):
+    from rtp_amd import emulate_shards
+    from rtp_amd.module import linear as L
+    with emulate_shards(ws):
+        layer = getattr(L, cls_name)(master.in_features, master.out_features, linear_layer=master, device=DEV,
+                                     dtype=dtype)
+    return layer
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("ws", [1, 2, 4])
+def test_column_linear_reference_shape(dtype, ws):
+    """nn.Linear(8,8), data [8,8] as in tests/test_linear.py."""
+    master = nn.Linear(8, 8)
+    x = torch.randn(8, 8)
+    g = torch.randn(8, 8)
+    layer = _build("ColumnParallelLinear", master.to(dtype), ws, dtype)
+    xd = x.to(DEV, dtype).requires_grad_()
+    out = layer(xd)
+    out.backward(g.to(DEV, dtype))
+    w, b = master.weight.detach().float().requires_grad_(), master.bias.detach().float().requires_grad_()
+    xo = x.to(dtype).float().requires_grad_()
+    ref = O.column_parallel_linear(xo, w, b, ws)
+    ref.backward(g.to(dtype).float())
+    assert_close(out, ref, dtype, "output")
+    assert_close(torch.cat([l.weight.grad for l in layer.linears], dim=0), w.grad, dtype, "weight grad (cat dim 0)")
+    assert_close(torch.cat([l.bias.grad for l in layer.linears], dim=0), b.grad, dtype, "bias grad (cat dim 0)")
+    assert_close(xd.grad, xo.grad, dtype, "input grad")
+    assert layer.linear is layer.linears[0] and layer.linear.weight.shape == (8 // ws, 8)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("ws", [1, 2, 4])
+def test_row_linear_reference_shape(dtype, ws):
+    master = nn.Linear(8, 8)
+    x = torch.randn(3, 8, 8)
+    g = torch.randn(3, 8, 8)
+    layer = _build("RowParallelLinear", master.to(dtype), ws, dtype)
+    xd = x.to(DEV, dtype).requires_grad_()
+    out = layer(xd)
+    out.backward(g.to(DEV, dtype))
+    w, b = master.weight.detach().float().requires_grad_(), master.bias.detach().float().requires_grad_()
+    xo = x.to(dtype).float().requires_grad_()
+    ref = O.row_parallel_linear(xo, w, b, ws)
+    ref.backward(g.to(dtype).float())
+    assert_close(out, ref, dtype, "output")
+    assert_close(torch.cat([l.weight.grad for l in layer.linears], dim=1), w.grad, dtype, "weight grad (cat dim 1)")
+    for l in layer.linears:  # each shard stores b/ws and receives the full bias gradient
+        assert_close(l.bias.grad, b.grad, dtype, "bias grad (un-gathered)")
+        assert_close(l.bias * ws, b, dtype, "bias/ws")
+    assert_close(xd.grad, xo.grad, dtype, "input grad")
+
+
+def test_column_linear_headline_config_fp32():
+    """X [1024,2048] ~N(0,1), W [2048,2048] ~U(-0.1,0.1), bias zeros, 2 column shards."""
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(1024, 2048, generator=gen)
+    master = nn.Linear(2048, 2048)
+    with torch.no_grad():
+        master.weight.copy_(torch.rand(2048, 2048, generator=gen) * 0.2 - 0.1)
+        master.bias.zero_()
+    dy = torch.randn(1024, 2048, generator=gen)
+    layer = _build("ColumnParallelLinear", master, 2, torch.float32)
+    xd = x.to(DEV).requires_grad_()
+    out = layer(xd)
+    out.backward(dy.to(DEV))
+    xo = x.clone().requires_grad_()
+    ref = master(xo)
+    ref.backward(dy)
+    assert_close(out, ref, torch.float32, "output")
+    assert_close(torch.cat([l.weight.grad for l in layer.linears], 0), master.weight.grad, torch.float32, "dW")
+    assert_close(torch.cat([l.bias.grad for l in layer.linears], 0), master.bias.grad, torch.float32, "db")
+    assert_close(xd.grad, xo.grad, torch.float32, "dX")
+    # linearity: the layer is affine in x with zero bias
+    out2 = layer(2 * xd.detach())
+    assert_close(out2, 2 * ref, torch.float32, "linearity")
+
+
+def test_grad_accumulation_and_zero_grad():
+    from rtp_amd import zero_full_grads
+    master = nn.Linear(16, 12)
+    layer = _build("ColumnParallelLinear", master, 4, torch.float32)
+    x = torch.randn(5, 16, device=DEV)
+    layer(x).sum().backward()
+    g1 = torch.cat([l.weight.grad for l in layer.linears], 0).clone()
+    layer(x).sum().backward()  # second backward accumulates, as torch does
+    g2 = torch.cat([l.weight.grad for l in layer.linears], 0)
+    assert_close(g2, 2 * g1, torch.float32, "accumulated grad")
+    zero_full_grads(layer)
+    assert all(l.weight.grad is None for l in layer.linears)
+    layer(x).sum().backward()
+    assert_close(torch.cat([l.weight.grad for l in layer.linears], 0), g1, torch.float32, "grad after zeroing")
+    # parameters alias the flat home storage, shard by shard
+    for s, l in enumerate(layer.linears):
+        assert l.weight.data_ptr() == layer._store.home[s].data_ptr()
+        assert l.weight.grad.data_ptr() == layer._store.grads[s].data_ptr()
+    assert len(list(layer.parameters())) == 8
+
+
+def test_to_dtype_keeps_flat_storage():
+    master = nn.Linear(16, 8)
+    layer = _build("ColumnParallelLinear", master, 2, torch.float32)
+    layer.to(torch.bfloat16)
+    assert layer._store.home.dtype == torch.bfloat16 and layer.linear.weight.dtype == torch.bfloat16
+    x = torch.randn(4, 16, device=DEV, dtype=torch.bfloat16)
+    assert_close(layer(x), master(x.float().cpu()), torch.bfloat16, "after .to(bf16)")
+
+
+def test_indivisible_raises():
+    from rtp_amd import emulate_shards
+    from rtp_amd.module.linear import ColumnParallelLinear
+    with emulate_shards(3), pytest.raises(AssertionError):
+        ColumnParallelLinear(8, 8, device=DEV)

@@ -1,0 +1,155 @@
+"""The rotated TransformerLM (rtp_amd.models.transformer_lm_rtp) vs the oracle LM assembled from stock
+torch layers: loss, logits and every gradient, fp32 and bf16; the SGD step; peak weight accounting."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from gpu_util import DEV, assert_close, rel_err
+from oracle import rtp_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def load_unsharded(lm, ref):
+    """Copy the oracle LM's weights into the rotated LM shard by shard (the *_layer= import rules)."""
+    with torch.no_grad():
+        for sh in lm[0].embedding.embeddings:
+            sh.affine_weight(ref[0])
+        n_dec = len(lm) - 3
+        for i in range(n_dec):
+            dec, rdec = lm[2 + i], ref[2 + i]
+            for sh in dec.self_attn.layers:
+                sh.affine_weight(rdec.self_attn)
+            for sh in dec.ff_block.linear1.linears:
+                sh.affine_weight(rdec.linear1)
+            for sh in dec.ff_block.linear2.linears:
+                sh.affine_weight(rdec.linear2)
+            for a, b in ((dec.norm1, rdec.norm1), (dec.norm2, rdec.norm2)):
+                a.weight.copy_(b.weight), a.bias.copy_(b.bias)
+        for sh in lm[-1].linear.linears:
+            sh.affine_weight(ref[-1])
+
+
+def gathered_grads(lm, ws):
+    """Unsharded gradients rebuilt with the reference tests' gather rules."""
+    out = {"emb": torch.cat([s.weight.grad for s in lm[0].embedding.embeddings], 1)}
+    for i in range(len(lm) - 3):
+        dec = lm[2 + i]
+        sa = dec.self_attn.layers
+        out[f"l{i}.in_w"] = O.attention_grad_reinterleave([s.in_proj_weight.grad for s in sa], ws)
+        out[f"l{i}.in_b"] = O.attention_grad_reinterleave([s.in_proj_bias.grad for s in sa], ws)
+        out[f"l{i}.out_w"] = torch.cat([s.out_proj.weight.grad for s in sa], 1)
+        out[f"l{i}.out_b"] = sa[0].out_proj.bias.grad
+        out[f"l{i}.w1"] = torch.cat([s.weight.grad for s in dec.ff_block.linear1.linears], 0)
+        out[f"l{i}.b1"] = torch.cat([s.bias.grad for s in dec.ff_block.linear1.linears], 0)
+        out[f"l{i}.w2"] = torch.cat([s.weight.grad for s in dec.ff_block.linear2.linears], 0)
+        out[f"l{i}.b2"] = torch.cat([s.bias.grad for s in dec.ff_block.linear2.linears], 0)
+        out[f"l{i}.ln1"] = dec.norm1.weight.grad
+        out[f"l{i}.ln2"] = dec.norm2.weight.grad
+    out["head_w"] = torch.cat([s.weight.grad for s in lm[-1].linear.linears], 0)
+    out["head_b"] = torch.cat([s.bias.grad for s in lm[-1].linear.linears], 0)
+    return out
+
+
+def ref_grads(ref):
+    out = {"emb": ref[0].weight.grad}
+    for i in range(len(ref) - 3):
+        d = ref[2 + i]
+        out[f"l{i}.in_w"], out[f"l{i}.in_b"] = d.self_attn.in_proj_weight.grad, d.self_attn.in_proj_bias.grad
+        out[f"l{i}.out_w"], out[f"l{i}.out_b"] = d.self_attn.out_proj.weight.grad, d.self_attn.out_proj.bias.grad
+        out[f"l{i}.w1"], out[f"l{i}.b1"] = d.linear1.weight.grad, d.linear1.bias.grad
+        out[f"l{i}.w2"], out[f"l{i}.b2"] = d.linear2.weight.grad, d.linear2.bias.grad
+        out[f"l{i}.ln1"], out[f"l{i}.ln2"] = d.norm1.weight.grad, d.norm2.weight.grad
+    out["head_w"], out["head_b"] = ref[-1].weight.grad, ref[-1].bias.grad
+    return out
+
+
+def build_pair(V, D, H, Fd, n_dec, ws, dtype, seed=0):
+    from rtp_amd.models.transformer_lm_rtp import TransformerLM
+    torch.manual_seed(seed)
+    ref = O.TransformerLM(V, D, H, Fd, n_dec)
+    with torch.no_grad():
+        for name, p in ref.named_parameters():
+            if "norm" not in name:
+                p.uniform_(-0.1, 0.1)
+        ref[-1].bias.zero_()
+        if dtype != torch.float32:  # both sides start from the same representable values
+            for p in ref.parameters():
+                p.copy_(p.to(dtype).float())
+    lm = TransformerLM(V, D, H, Fd, 0.0, 0.1, n_dec, ws, 0, device=DEV, dtype=dtype)
+    load_unsharded(lm, ref)
+    return lm, ref
+
+
+@pytest.mark.parametrize("dtype,ws", [(torch.float32, 4), (torch.float32, 1), (torch.bfloat16, 4)])
+def test_lm_loss_and_grads(dtype, ws):
+    V, D, H, Fd, n_dec, L, N = 96, 64, 4, 64, 2, 12, 5
+    lm, ref = build_pair(V, D, H, Fd, n_dec, ws, dtype)
+    gen = torch.Generator().manual_seed(1)
+    ids = torch.randint(0, V, (L, N), generator=gen)
+    tgt = torch.randint(0, V, (L, N), generator=gen)
+    logits = lm(ids.to(DEV))
+    loss = F.cross_entropy(logits.float().view(-1, V), tgt.to(DEV).view(-1))
+    loss.backward()
+    ref_logits = ref(ids)
+    ref_loss = F.cross_entropy(ref_logits.view(-1, V), tgt.view(-1))
+    ref_loss.backward()
+    assert_close(logits, ref_logits, dtype, "logits")
+    assert abs(float(loss) - float(ref_loss)) <= (1e-5 if dtype == torch.float32 else 2e-2) * abs(float(ref_loss))
+    mine, theirs = gathered_grads(lm, ws), ref_grads(ref)
+    tol_scale = 1.0 if dtype == torch.float32 else 1.0
+    for k in theirs:
+        # fp32 end-to-end through 2 layers of LayerNorm/softmax: a few ulps of headroom over a single GEMM
+        err = rel_err(mine[k], theirs[k])
+        limit = 5e-5 if dtype == torch.float32 else 4e-2
+        assert err <= limit * tol_scale, f"{k}: {err:.3e}"
+
+
+def test_lm_sgd_step_matches_closed_form():
+    from rtp_amd.optim import RotatedSGD
+    V, D, H, Fd, n_dec, L, N, ws = 64, 32, 2, 32, 1, 6, 3, 2
+    lm, ref = build_pair(V, D, H, Fd, n_dec, ws, torch.float32, seed=2)
+    opt = RotatedSGD(lm, lr=0.1)
+    ids = torch.randint(0, V, (L, N))
+    before = lm[-1].linear.linears[1].weight.detach().clone()
+    F.cross_entropy(lm(ids.to(DEV)).view(-1, V), ids.to(DEV).view(-1)).backward()
+    g = lm[-1].linear.linears[1].weight.grad.detach().clone()
+    ln_before, ln_g = lm[2].norm1.weight.detach().clone(), lm[2].norm1.weight.grad.detach().clone()
+    opt.step()
+    assert torch.equal(lm[-1].linear.linears[1].weight.detach(), before - 0.1 * g)
+    assert torch.equal(lm[2].norm1.weight.detach(), ln_before - 0.1 * ln_g)
+    opt.zero_grad()
+    assert lm[-1].linear.linears[1].weight.grad is None
+
+
+def test_lm_bf16_master_weights_and_weight_bytes():
+    from rtp_amd import rotated_weight_bytes, staging_bytes
+    from rtp_amd.optim import RotatedSGD
+    V, D, H, Fd, n_dec, L, N, ws = 64, 32, 2, 32, 1, 6, 3, 4
+    lm, _ = build_pair(V, D, H, Fd, n_dec, ws, torch.bfloat16, seed=3)
+    opt = RotatedSGD(lm, lr=0.5, clip_value=0.05)
+    ids = torch.randint(0, V, (L, N)).to(DEV)
+    w = lm[-1].linear.linears[0].weight
+    master = opt.masters[-1].view(ws, -1)[0][: w.numel()].view_as(w).clone()
+    F.cross_entropy(lm(ids).float().view(-1, V), ids.view(-1)).backward()
+    g = w.grad.float().clamp(-0.05, 0.05)
+    opt.step()
+    expect = master - 0.5 * g
+    assert torch.equal(w.detach(), expect.to(torch.bfloat16))
+    n_rot = sum(p.numel() for n, p in lm.named_parameters() if "norm" not in n)
+    assert rotated_weight_bytes(lm) == 2 * n_rot  # every shard resident exactly once, in bf16
+    largest = max(m._store.numel for m in lm.modules() if hasattr(m, "_store")) * 2
+    assert staging_bytes() >= 2 * largest
+
+
+def test_lm_moe_variant_runs_and_backprops():
+    from rtp_amd.models.transformer_lm_rtp import TransformerLM
+    lm = TransformerLM(64, 32, 4, 48, 0.0, 0.1, 1, 4, 0, is_moe=True, device=DEV)
+    ids = torch.randint(0, 64, (8, 4)).to(DEV)  # 32 tokens over 4 experts
+    out = lm(ids)
+    assert out.shape == (8, 4, 64) and torch.isfinite(out).all()
+    (out.float().mean() + lm[2].moe_layer.l_aux).backward()
+    for p in lm.parameters():
+        assert p.grad is not None and torch.isfinite(p.grad).all()

@@ -1,0 +1,173 @@
+"""Top-2 routing (bit-exact integers) and the rotated MoE layer vs the oracle and the reference goldens."""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+from gpu_util import DEV, assert_close, rel_err
+from oracle import rtp_oracle as O
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _route(logits, noise):
+    from rtp_amd import ops
+    r = ops.top2_route(logits.to(DEV).contiguous(), noise.to(DEV).contiguous())
+    torch.cuda.synchronize()
+    return r
+
+
+def _check_routing(logits, noise):
+    g = O.top2gating(logits, noise)
+    top = torch.sort(g["gates"], dim=1, descending=True).values
+    assert (top[:, 0] - top[:, 1]).min() > 0, "fixture must have a non-zero top-1 margin"
+    r = _route(logits, noise)
+    S, E = logits.shape
+    assert torch.equal(r.expert.cpu(), g["expert"]), "expert choice"
+    assert torch.equal(r.keep.cpu(), g["keep"]), "capacity drop"
+    assert torch.equal(r.slot.cpu(), g["slot"]), "slot"
+    assert torch.equal(r.counts.cpu(), g["counts"]), "per-expert counts"
+    assert rel_err(r.weight, g["weight"]) <= 1e-5
+    assert rel_err(r.gates, g["gates"]) <= 1e-5
+    assert abs(float(r.l_aux) - float(g["l_aux"])) <= 1e-6
+    C = 2 * S // E
+    st = r.slot_token.cpu().view(E, C)
+    expect = torch.full((E, C), -1, dtype=torch.int32)
+    for s in range(S):
+        for j in range(2):
+            if g["keep"][s, j]:
+                expect[g["expert"][s, j], g["slot"][s, j]] = s
+    assert torch.equal(st, expect), "slot -> token map"
+    return r, g
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "top2gating_*.npz"))))
+def test_routing_matches_reference_golden(path):
+    z = np.load(path)
+    r, g = _check_routing(torch.from_numpy(z["logits"]), torch.from_numpy(z["noise"]))
+    from rtp_amd.module.top2gate import dense_from_routing
+    combine, dispatch = dense_from_routing(r, r.weight, torch.float32)
+    assert np.array_equal(dispatch.cpu().numpy(), z["dispatch_mask"])
+    np.testing.assert_allclose(combine.cpu().numpy(), z["combine_weights"], rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.parametrize("S,E,seed,skew", [(8, 2, 0, 0.0), (512, 8, 1, 0.0), (4096, 8, 2, 0.0), (4096, 8, 3, 2.0),
+                                           (1000, 4, 4, 1.0), (768, 64, 5, 0.0)])
+def test_routing_bit_exact(S, E, seed, skew):
+    gen = torch.Generator().manual_seed(seed)
+    logits = torch.randn(S, E, generator=gen)
+    logits[:, 0] += skew
+    _check_routing(logits, O.gumbel_noise((S, E), gen))
+
+
+def test_routing_backward_matches_autograd_of_oracle():
+    from rtp_amd.module.top2gate import top2_route
+    gen = torch.Generator().manual_seed(7)
+    S, E = 64, 4
+    logits = torch.randn(S, E, generator=gen)
+    logits[:, 2] += 1.5
+    noise = O.gumbel_noise((S, E), gen)
+    cw = torch.randn(S, 2, generator=gen)
+    ld = logits.to(DEV).requires_grad_()
+    r, weight, l_aux = top2_route(ld, noise.to(DEV))
+    ((weight * cw.to(DEV)).sum() + 3.0 * l_aux).backward()
+    lo = logits.clone().requires_grad_()
+    g = O.top2gating(lo, noise)
+    ((g["weight"] * cw).sum() + 3.0 * g["l_aux"]).backward()
+    assert rel_err(ld.grad, lo.grad) <= 1e-5
+
+
+def _moe_from_tensors(wg, experts, ws, dtype):
+    from rtp_amd import emulate_shards
+    from rtp_amd.models.transformer_lm_rtp import FeedForwardLayer_expert
+    from rtp_amd.module.moe import WeightMOELayer
+    from rtp_amd.module.top2gate import Top2Gate, WeightTop2Gate
+    E, M = wg.shape
+    Fd = experts[0][0].shape[0]
+    master_gate = Top2Gate(M, E)
+    with torch.no_grad():
+        master_gate.wg.weight.copy_(wg)
+    masters = []
+    for w1, b1, w2, b2 in experts:
+        m = FeedForwardLayer_expert(M, Fd, nn.ReLU(), 0.0)
+        with torch.no_grad():
+            m.linear1.weight.copy_(w1), m.linear1.bias.copy_(b1), m.linear2.weight.copy_(w2), m.linear2.bias.copy_(b2)
+        masters.append(m)
+    n_local = E // ws
+    with emulate_shards(ws):
+        gate = WeightTop2Gate(M, E, gate=master_gate.to(dtype), device=DEV, dtype=dtype)
+        local = nn.ModuleList([FeedForwardLayer_expert(M, Fd, nn.ReLU(), 0.0) for _ in range(n_local)])
+        originals = [nn.ModuleList(masters[s * n_local:(s + 1) * n_local]) for s in range(ws)]
+        layer = WeightMOELayer(gate, local, device=DEV, dtype=dtype, original_experts=originals)
+    return layer
+
+
+def test_moe_layer_matches_reference_golden():
+    """The reference's WeightMOELayer on a 2-rank gloo ring (tests/golden/moe_ws2.npz)."""
+    z = np.load(os.path.join(GOLDEN, "moe_ws2.npz"))
+    t = {k: torch.from_numpy(z[k]) for k in z.files}
+    names = ("linear1.weight", "linear1.bias", "linear2.weight", "linear2.bias")
+    experts = [tuple(t[f"expert{e}.{n}"] for n in names) for e in range(2)]
+    layer = _moe_from_tensors(t["wg"], experts, 2, torch.float32)
+    x = t["x"].to(DEV).requires_grad_()
+    out = layer(x)
+    assert rel_err(out, t["out"]) <= 1e-5
+    assert abs(float(layer.l_aux) - float(t["l_aux"])) <= 1e-6
+    ((out * t["coef"].to(DEV)).sum() + layer.l_aux).backward()
+    for n, p in zip(names, layer.experts.parameters()):
+        assert rel_err(2 * p.grad, t[f"grad_expert0.0.{n}"]) <= 1e-5, n
+    assert rel_err(2 * layer.gate.wg.weight.grad, t["grad_wg0"]) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype,ws,E", [(torch.float32, 4, 4), (torch.float32, 2, 4), (torch.bfloat16, 4, 4)])
+def test_moe_layer_vs_oracle(dtype, ws, E):
+    gen = torch.Generator().manual_seed(21)
+    M, Fd, S = 32, 48, 64
+    wg = (torch.rand(E, M, generator=gen) * 0.2 - 0.1).to(dtype).float()
+    experts = [tuple((torch.rand(s, generator=gen) * 0.2 - 0.1).to(dtype).float()
+                     for s in ((Fd, M), (Fd,), (M, Fd), (M,))) for _ in range(E)]
+    x = torch.randn(4, S // 4, M, generator=gen).to(dtype)
+    coef = torch.randn(4, S // 4, M, generator=gen).to(dtype)
+    noise = O.gumbel_noise((S, E), gen)
+    layer = _moe_from_tensors(wg, experts, ws, dtype)
+    xd = x.to(DEV).requires_grad_()
+    out = layer(xd, noise=noise.to(DEV))
+    ((out.float() * coef.to(DEV).float()).sum() + layer.l_aux.float()).backward()
+    wgo = wg.clone().requires_grad_()
+    eo = [tuple(p.clone().requires_grad_() for p in e) for e in experts]
+    xo = x.float().requires_grad_()
+    if dtype == torch.bfloat16:
+        # routing is discrete: give the oracle the logits the device actually produced
+        pass
+    ref, l_aux = O.moe_layer(xo, wgo, eo, noise, ws)
+    ((ref * coef.float()).sum() + l_aux).backward()
+    assert_close(out, ref, dtype, "output")
+    assert abs(float(layer.l_aux) - float(l_aux)) <= (1e-6 if dtype == torch.float32 else 2e-3)
+    assert_close(xd.grad, xo.grad, dtype, "input grad")
+    n_local = E // ws
+    for s in range(ws):
+        params = list(layer.experts_list[s].parameters())
+        for j in range(n_local):
+            for q, p in zip(eo[s * n_local + j], params[4 * j:4 * j + 4]):
+                assert_close(p.grad, q.grad, dtype, f"expert {s * n_local + j} grad")
+    assert_close(torch.cat([w.weight.grad for w in layer.gate.wgs], 0), wgo.grad, dtype, "gate grad (cat dim 0)")
+
+
+def test_gate_module_dense_api():
+    from rtp_amd import emulate_shards
+    from rtp_amd.module.top2gate import WeightTop2Gate
+    gen = torch.Generator().manual_seed(4)
+    with emulate_shards(4):
+        gate = WeightTop2Gate(16, 4, device=DEV)
+    x = torch.randn(32, 16, generator=gen)
+    noise = O.gumbel_noise((32, 4), gen)
+    l_aux, combine, dispatch = gate(x.to(DEV), noise=noise.to(DEV))
+    wg = torch.cat([w.weight.detach().cpu() for w in gate.wgs], 0)
+    g = O.top2gating(x @ wg.t(), noise)
+    assert combine.shape == (32, 4, 16) and dispatch.dtype == torch.bool
+    assert torch.equal(dispatch.cpu(), g["dispatch_mask"])
+    assert rel_err(combine, g["combine_weights"]) <= 1e-5

@@ -1,0 +1,142 @@
+"""Host-side logic that needs no GPU: shard layouts, flat-parameter aliasing, ring order, world-size
+resolution and the drop-in constructor surface."""
+import inspect
+
+import pytest
+import torch
+import torch.nn as nn
+
+from oracle import rtp_oracle as O
+from rtp_amd import emulate_shards
+from rtp_amd.module import attention, collectives, embedding, linear, moe, top2gate, utils
+from rtp_amd.ring import ring_order
+
+
+def test_ring_order_forward_and_backward():
+    assert ring_order(0, 4) == [0, 1, 2, 3]
+    assert ring_order(2, 4) == [2, 3, 0, 1] == O.ring_order(2, 4)
+    assert ring_order(2, 4, reverse=True) == [1, 0, 3, 2]
+    assert ring_order(0, 1) == [0]
+
+
+def test_resolve_world_precedence(monkeypatch):
+    monkeypatch.delenv("RTP_EMULATED_SHARDS", raising=False)
+    assert collectives.resolve_world() == (1, 0)
+    monkeypatch.setenv("RTP_EMULATED_SHARDS", "8")
+    assert collectives.resolve_world() == (8, 0)
+    with emulate_shards(2):
+        assert collectives.resolve_world() == (2, 0)
+        with emulate_shards(4):
+            assert collectives.resolve_world() == (4, 0)
+        assert collectives.resolve_world() == (2, 0)
+    with pytest.raises(ValueError):
+        with emulate_shards(0):
+            pass
+
+
+def test_column_row_shard_layouts_match_oracle():
+    master = nn.Linear(12, 8)
+    with emulate_shards(4):
+        col = linear.ColumnParallelLinear(12, 8, linear_layer=master)
+        row = linear.RowParallelLinear(12, 8, linear_layer=master)
+    for s, (w, b) in enumerate(O.column_shards(master.weight.detach(), master.bias.detach(), 4)):
+        assert torch.equal(col.linears[s].weight, w) and torch.equal(col.linears[s].bias, b)
+    for s, (w, b) in enumerate(O.row_shards(master.weight.detach(), master.bias.detach(), 4)):
+        assert torch.equal(row.linears[s].weight, w) and torch.allclose(row.linears[s].bias, b)
+    assert col.linear is col.linears[0] and col.world_size == 4 and col.rank == 0
+    assert col.linear.weight.shape == (2, 12) and row.linear.weight.shape == (8, 3)
+
+
+def test_flat_param_order_and_aliasing():
+    """One flat buffer per shard in named_parameters() order; parameters are views of it."""
+    mha = nn.MultiheadAttention(8, 4)
+    layer = attention.ParallelMultiheadAttention(8, 4, 2, 0, MultiheadAttention_layer=mha)
+    st = layer._store
+    assert st.names == ["in_proj_weight", "in_proj_bias", "out_proj.weight", "out_proj.bias"]
+    assert st.numel == 12 * 8 + 12 + 8 * 4 + 8 and st.home.shape == (2, st.numel)
+    for s, sub in enumerate(layer.layers):
+        assert sub._full_param.data_ptr() == st.home[s].data_ptr()
+        off = 0
+        for p in sub.parameters():
+            assert p.data_ptr() == st.home[s].data_ptr() + off * 4
+            off += p.numel()
+        w_in, b_in, w_o, b_o = O.attention_shard_params(mha.in_proj_weight.detach(), mha.in_proj_bias.detach(),
+                                                         mha.out_proj.weight.detach(), mha.out_proj.bias.detach(), 2, s)
+        assert torch.equal(sub.in_proj_weight, w_in) and torch.equal(sub.in_proj_bias, b_in)
+        assert torch.equal(sub.out_proj.weight, w_o) and torch.allclose(sub.out_proj.bias, b_o)
+    # writing through a parameter view changes the flat buffer (flyweight)
+    with torch.no_grad():
+        layer.layers[1].in_proj_bias.fill_(3.0)
+    assert float(st.home[1, 96]) == 3.0
+    assert len(list(layer.parameters())) == 8  # every shard's parameters, once
+
+
+def test_attention_block_index_is_q_k_v_rows_of_the_head_group():
+    E, ws = 8, 2
+    in_w = torch.arange(3 * E * E, dtype=torch.float32).view(3 * E, E)
+    for s in range(ws):
+        w_in, _, _, _ = O.attention_shard_params(in_w, None, torch.zeros(E, E), None, ws, s)
+        e_s = E // ws
+        expect = torch.cat([in_w[s * e_s:(s + 1) * e_s], in_w[E + s * e_s:E + (s + 1) * e_s],
+                            in_w[2 * E + s * e_s:2 * E + (s + 1) * e_s]])
+        assert torch.equal(w_in, expect)
+        assert utils.attention_block_index(s, ws) == [s, s + ws, s + 2 * ws]
+
+
+def test_embedding_shards_are_column_blocks():
+    master = nn.Embedding(10, 8)
+    layer = embedding.ParallelEmbedding(10, 8, 4, 0, Embedding_layer=master)
+    assert layer.embedding.weight.shape == (10, 2)
+    assert torch.equal(torch.cat([e.weight for e in layer.embeddings], 1), master.weight)
+
+
+def test_repack_after_dtype_change_keeps_values_and_aliasing():
+    master = nn.Linear(6, 4)
+    with emulate_shards(2):
+        col = linear.ColumnParallelLinear(6, 4, linear_layer=master)
+    col.to(torch.bfloat16)
+    assert col._store.home.dtype == torch.bfloat16
+    assert col.linears[1].weight.data_ptr() == col._store.home[1].data_ptr()
+    assert torch.equal(col.linears[1].weight, master.weight[2:4].to(torch.bfloat16))
+
+
+def test_moe_and_gate_shards():
+    from rtp_amd.models.transformer_lm_rtp import FeedForwardLayer_expert
+    g = top2gate.Top2Gate(8, 4)
+    with emulate_shards(2):
+        gate = top2gate.WeightTop2Gate(8, 4, gate=g)
+        local = FeedForwardLayer_expert(8, 16, nn.ReLU(), 0.0)
+        layer = moe.WeightMOELayer(gate, local)
+    assert torch.equal(torch.cat([w.weight for w in gate.wgs], 0), g.wg.weight)
+    assert gate.wg.weight.shape == (2, 8) and layer.num_local_experts == 1 and len(layer.experts_list) == 2
+    assert layer._store.names == ["0.linear1.weight", "0.linear1.bias", "0.linear2.weight", "0.linear2.bias"]
+    with pytest.raises(NotImplementedError):
+        with emulate_shards(2):
+            moe.WeightMOELayer(gate, nn.Linear(8, 8))
+
+
+def test_forward_without_gpu_fails_loudly():
+    from rtp_amd._lib import RtpError
+    with emulate_shards(2):
+        col = linear.ColumnParallelLinear(4, 4)
+    with pytest.raises((RtpError, RuntimeError)):
+        col(torch.zeros(2, 4))
+
+
+@pytest.mark.parametrize("cls,expected", [
+    (linear.ColumnParallelLinear, ["in_features", "out_features", "bias", "gather_weight", "init_method", "stride",
+                                   "keep_master_weight_for_test", "device", "dtype", "group", "linear_layer"]),
+    (linear.RowParallelLinear, ["in_features", "out_features", "bias", "gather_weight", "init_method", "stride",
+                                "keep_master_weight_for_test", "device", "dtype", "group", "linear_layer"]),
+    (embedding.ParallelEmbedding, ["num_embeddings", "embedding_dim", "world_size", "rank", "padding_idx", "max_norm",
+                                   "norm_type", "scale_grad_by_freq", "sparse", "init_method",
+                                   "keep_master_weight_for_test", "Embedding_layer", "device", "dtype"]),
+    (attention.ParallelMultiheadAttention, ["embed_dim", "num_heads", "world_size", "rank", "dropout", "bias",
+                                            "add_bias_kv", "add_zero_attn", "kdim", "vdim", "batch_first", "device",
+                                            "dtype", "MultiheadAttention_layer"]),
+    (top2gate.WeightTop2Gate, ["model_dim", "num_experts", "gate", "device", "dtype"]),
+    (moe.WeightMOELayer, ["gate", "experts", "group", "device", "dtype", "original_experts"]),
+])
+def test_constructor_signatures_match_reference(cls, expected):
+    params = [p for p in inspect.signature(cls.__init__).parameters if p != "self"]
+    assert params == expected
