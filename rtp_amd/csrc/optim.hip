@@ -10,7 +10,13 @@ __global__ __launch_bounds__(256) void sgd_kernel(float* master, const T* grad, 
   for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
     float g = to_f32(grad[i]);
     if (clip > 0.0f) g = fminf(fmaxf(g, -clip), clip);
-    const float w = master[i] - lr * g;
+    // two roundings (product, then difference): the plain closed form w - lr*g, not a fused multiply-add
+    float w;
+    {
+#pragma clang fp contract(off)
+      const float step = lr * g;
+      w = master[i] - step;
+    }
     master[i] = w;
     if (shadow) shadow[i] = from_f32<T>(w);
   }

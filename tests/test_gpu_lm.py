@@ -75,7 +75,15 @@ def build_pair(V, D, H, Fd, n_dec, ws, dtype, seed=0):
             if "norm" not in name:
                 p.uniform_(-0.1, 0.1)
         ref[-1].bias.zero_()
-        if dtype != torch.float32:  # both sides start from the same representable values
+        if dtype != torch.float32:
+            # bf16 vs fp32 differ by ~2^-9 per activation; a ReLU input that close to zero flips its mask and
+            # moves a whole weight-gradient column by O(1/sqrt(tokens)).  Keep the pre-activations away from
+            # the kink (half the units well inside the active side, half well inside the inactive side) so the
+            # comparison measures rounding, not the discontinuity; the fp32 cases exercise ReLU at random signs.
+            for i in range(n_dec):
+                b = ref[2 + i].linear1.bias
+                b.copy_(torch.where(torch.arange(b.numel()) % 2 == 0, 1.5, -1.5))
+            # both sides start from the same representable values
             for p in ref.parameters():
                 p.copy_(p.to(dtype).float())
     lm = TransformerLM(V, D, H, Fd, 0.0, 0.1, n_dec, ws, 0, device=DEV, dtype=dtype)
@@ -99,12 +107,13 @@ def test_lm_loss_and_grads(dtype, ws):
     assert_close(logits, ref_logits, dtype, "logits")
     assert abs(float(loss) - float(ref_loss)) <= (1e-5 if dtype == torch.float32 else 2e-2) * abs(float(ref_loss))
     mine, theirs = gathered_grads(lm, ws), ref_grads(ref)
-    tol_scale = 1.0 if dtype == torch.float32 else 1.0
-    for k in theirs:
-        # fp32 end-to-end through 2 layers of LayerNorm/softmax: a few ulps of headroom over a single GEMM
-        err = rel_err(mine[k], theirs[k])
-        limit = 5e-5 if dtype == torch.float32 else 4e-2
-        assert err <= limit * tol_scale, f"{k}: {err:.3e}"
+    errs = {k: rel_err(mine[k], theirs[k]) for k in theirs}
+    print({k: f"{v:.1e}" for k, v in errs.items()})
+    # fp32 end-to-end through 2 layers of LayerNorm/softmax: a few ulps of headroom over a single GEMM (1e-5);
+    # bf16: the north-star 2e-2
+    limit = 5e-5 if dtype == torch.float32 else 2e-2
+    for k, err in errs.items():
+        assert err <= limit, f"{k}: {err:.3e}"
 
 
 def test_lm_sgd_step_matches_closed_form():
@@ -127,7 +136,7 @@ def test_lm_sgd_step_matches_closed_form():
 def test_lm_bf16_master_weights_and_weight_bytes():
     from rtp_amd import rotated_weight_bytes, staging_bytes
     from rtp_amd.optim import RotatedSGD
-    V, D, H, Fd, n_dec, L, N, ws = 64, 32, 2, 32, 1, 6, 3, 4
+    V, D, H, Fd, n_dec, L, N, ws = 64, 32, 4, 32, 1, 6, 3, 4
     lm, _ = build_pair(V, D, H, Fd, n_dec, ws, torch.bfloat16, seed=3)
     opt = RotatedSGD(lm, lr=0.5, clip_value=0.05)
     ids = torch.randint(0, V, (L, N)).to(DEV)
