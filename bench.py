@@ -1,0 +1,199 @@
+#!/usr/bin/env python
+"""Headline benchmark: fwd + bwd + SGD step of the 10-layer RTP transformer LM (README configuration of
+the reference: vocab 10240, ninp 2048, nhid 2048, 32 heads, 10 decoder layers, seq 32, batch 32) on ONE
+MI355X, bf16 weights with fp32 master, 8 rotation shards emulated on the device, synthetic token ids.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+Prints one JSON line.  `value` is tokens/s over K timed steps with inputs resident in HBM.  `roofline`
+is the dominant kernel of the step (by summed duration), timed per launch with HIP events on the stream
+it runs on, during extra profiled steps that follow the timed region (so the events do not perturb
+`value`).  `cpu_baseline` is the CPU oracle (stock torch layers, fp32) timed on this box's host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+CFG = dict(vocab=10240, ninp=2048, nhid=2048, nhead=32, layers=10, seq=32, batch=32, shards=8)
+PEAK = {"bf16_mfma_tflops": 2500.0, "fp32_mfma_tflops": 157.3, "hbm_gbs": 8000.0}
+
+
+def step_flops(c):
+    """Algorithmic flops of one fwd+bwd step: 3 x (2*T*matmul params + attention core)."""
+    t = c["seq"] * c["batch"]
+    per_layer = 4 * c["ninp"] * c["ninp"] + 2 * c["ninp"] * c["nhid"]
+    matmul = c["layers"] * per_layer + c["ninp"] * c["vocab"]
+    attn = c["layers"] * 4 * c["batch"] * c["nhead"] * c["seq"] * c["seq"] * (c["ninp"] // c["nhead"])
+    return 3.0 * (2.0 * t * matmul + attn)
+
+
+def build(c, device, dtype):
+    import torch
+    from rtp_amd.models.transformer_lm_rtp import TransformerLM
+    from rtp_amd.module.collectives import ShardStore
+
+    torch.manual_seed(0)
+    lm = TransformerLM(c["vocab"], c["ninp"], c["nhead"], c["nhid"], 0.0, 0.1, c["layers"], c["shards"], 0,
+                       device=device, dtype=dtype)
+    with torch.no_grad():  # every rotated weight ~U(-0.1, 0.1), logits bias 0, LayerNorm gamma 1 / beta 0
+        for m in lm.modules():
+            st = getattr(m, "_store", None)
+            if isinstance(st, ShardStore):
+                st.home.uniform_(-0.1, 0.1)
+        for sh in lm[-1].linear.linears:
+            sh.bias.zero_()
+    return lm
+
+
+def cpu_baseline(c, steps=2):
+    """The oracle LM (stock nn.Embedding / nn.MultiheadAttention / nn.Linear / nn.LayerNorm, fp32) on the host
+    cores: same shapes, same step (zero grads, fwd, CE, bwd, clip, SGD)."""
+    import torch
+    import torch.nn.functional as F
+    from oracle import rtp_oracle as O
+
+    torch.manual_seed(0)
+    ref = O.TransformerLM(c["vocab"], c["ninp"], c["nhead"], c["nhid"], c["layers"])
+    with torch.no_grad():
+        for n, p in ref.named_parameters():
+            if "norm" not in n:
+                p.uniform_(-0.1, 0.1)
+    ids = torch.randint(0, c["vocab"], (c["seq"], c["batch"]))
+    tgt = torch.randint(0, c["vocab"], (c["seq"], c["batch"]))
+
+    def one():
+        for p in ref.parameters():
+            p.grad = None
+        loss = F.cross_entropy(ref(ids).view(-1, c["vocab"]), tgt.view(-1))
+        loss.backward()
+        with torch.no_grad():
+            for p in ref.parameters():
+                p.add_(p.grad.clamp_(-0.05, 0.05), alpha=-1e-3)
+
+    one()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        one()
+    dt = (time.perf_counter() - t0) / steps
+    return {"value": c["seq"] * c["batch"] / dt, "unit": "tokens/s", "cores": torch.get_num_threads(),
+            "kind": "port", "sample": f"{steps} full steps of the same configuration in fp32 after 1 warm-up "
+            f"({dt * 1e3:.0f} ms/step, os.cpu_count()={os.cpu_count()})"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--graph", action="store_true", help="replay the step from a captured HIP graph")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU's throughput: this build runs every rotation shard on a single MI355X and "
+              f"has no multi-GPU path (--gpus {args.gpus} is not supported)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import torch.nn.functional as F
+    from rtp_amd import _lib, rotated_weight_bytes, staging_bytes
+    from rtp_amd.optim import RotatedSGD
+
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    c = CFG
+    lm = build(c, dev, torch.bfloat16)
+    opt = RotatedSGD(lm, lr=1e-3, clip_value=0.05)
+    gen = torch.Generator().manual_seed(0)
+    ids = torch.randint(0, c["vocab"], (c["seq"], c["batch"]), generator=gen).to(dev)
+    tgt = torch.randint(0, c["vocab"], (c["seq"], c["batch"]), generator=gen).to(dev)
+    tokens = c["seq"] * c["batch"]
+    loss_box = [None]
+
+    def step():
+        opt.zero_grad()
+        logits = lm(ids)
+        loss = F.cross_entropy(logits.float().view(-1, c["vocab"]), tgt.view(-1))
+        loss.backward()
+        opt.step()
+        loss_box[0] = loss
+
+    for _ in range(max(args.warmup, 1)):
+        step()
+    torch.cuda.synchronize()
+    first_loss = float(loss_box[0])
+
+    run = step
+    if args.graph:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            step()
+        run = g.replay
+        run()
+        torch.cuda.synchronize()
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    last_loss = float(loss_box[0])
+
+    # Per-kernel timing with HIP events around every launch, on two extra eager steps.
+    _lib.profile_enable(True)
+    prof_steps = 2
+    for _ in range(prof_steps):
+        step()
+    stats = _lib.profile_collect()
+    _lib.profile_enable(False)
+    gemms = {k: v for k, v in stats.items() if k.startswith("gemm_")}
+    dom_name, dom = max(gemms.items(), key=lambda kv: kv[1]["total_ms"])
+    avg_ms = dom["total_ms"] / dom["launches"]
+    achieved = dom["flops"] / dom["launches"] / (avg_ms * 1e-3) / 1e12
+    all_gemm_ms = sum(v["total_ms"] for v in gemms.values()) / prof_steps
+    all_gemm_tflops = sum(v["flops"] for v in gemms.values()) / prof_steps / (all_gemm_ms * 1e-3) / 1e12
+    copy = stats.get("shard_copy")
+    kernels = {k: {"launches_per_step": v["launches"] // prof_steps, "ms_per_step": round(v["total_ms"] / prof_steps, 4),
+                   "tflops": round(v["flops"] / max(v["total_ms"], 1e-9) / 1e9, 2),
+                   "gbs": round(v["bytes"] / max(v["total_ms"], 1e-9) / 1e6, 1)} for k, v in sorted(stats.items())}
+
+    flops = step_flops(c)
+    out = {
+        "metric": "fwd+bwd tokens/s, 10-layer RTP LM, 1 MI355X; % MFMA peak; peak weight bytes",
+        "value": tokens / dt, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "10-layer RTP transformer LM fwd+bwd+SGD step: vocab 10240, ninp 2048, nhid 2048, "
+                               "32 heads, seq 32, batch 32, bf16 weights + fp32 master, 8 rotation shards emulated on "
+                               "one GPU, uniform random token ids, weights U(-0.1,0.1), dropout 0, lr 1e-3, clip 0.05",
+                   "tokens_per_step": tokens, "rotation_shards": c["shards"], "hip_graph": bool(args.graph)},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK["bf16_mfma_tflops"], "unit": "TFLOP/s",
+                     "frac": achieved / PEAK["bf16_mfma_tflops"], "traffic": None, "kernel": dom_name,
+                     "avg_launch_us": avg_ms * 1e3, "launches_per_step": dom["launches"] // prof_steps,
+                     "flops_per_launch": dom["flops"] / dom["launches"]},
+        "step_mfma_frac": flops / dt / (PEAK["bf16_mfma_tflops"] * 1e12),
+        "step_algorithmic_tflop": flops / 1e12,
+        "all_gemm_kernels": {"ms_per_step": all_gemm_ms, "tflops": all_gemm_tflops},
+        "shard_copy": None if copy is None else {"ms_per_step": copy["total_ms"] / prof_steps,
+                                                 "gbs": copy["bytes"] / copy["total_ms"] / 1e6,
+                                                 "frac_of_hbm_peak": copy["bytes"] / copy["total_ms"] / 1e6 / PEAK["hbm_gbs"]},
+        "kernels": kernels,
+        "peak_weight_bytes": {"rotated_weights_1x": rotated_weight_bytes(lm), "staging_two_slots": staging_bytes(dev),
+                              "fp32_master_separate": opt.master_bytes(),
+                              "ratio_weights_plus_staging_to_model": (rotated_weight_bytes(lm) + staging_bytes(dev)) /
+                              rotated_weight_bytes(lm)},
+        "loss_first_last": [first_loss, last_loss],
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(c)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -230,6 +230,26 @@ int rtp_sgd_step(void* stream, int dtype, float* master, const void* grad, void*
 /* dst(dtype_dst)[i] = src(dtype_src)[i]  (fp32 <-> bf16 conversion, round to nearest even). */
 int rtp_cast(void* stream, int dtype_src, const void* src, int dtype_dst, void* dst, int64_t n);
 
+/* ---------------------------------------------------------------------------------------------
+ * Measurement (no counterpart in the reference, which only prints words/s:
+ * benchmarks/rtp_benchmark.py:192-208).  With profiling enabled every kernel launch made by this
+ * library is bracketed by two HIP timing events on the stream it is launched on and booked under
+ * its kernel-variant name with the algorithmic flops and bytes of that launch.  rtp_profile_collect
+ * synchronises the device, sums the event durations per name into `out` (at most `max_out`
+ * entries, *n_out receives the count) and clears the records.  Must be off while a stream is being
+ * captured into a HIP graph.
+ * --------------------------------------------------------------------------------------------- */
+typedef struct {
+  char name[64];
+  int64_t launches;
+  double total_ms;
+  double flops; /* algorithmic, summed over launches */
+  double bytes; /* algorithmic, summed over launches */
+} rtp_kernel_stat;
+
+int rtp_profile_enable(int on);
+int rtp_profile_collect(rtp_kernel_stat* out, int max_out, int* n_out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -39,6 +39,11 @@ class GemmDesc(C.Structure):
     ]
 
 
+class KernelStat(C.Structure):
+    _fields_ = [("name", C.c_char * 64), ("launches", C.c_int64), ("total_ms", C.c_double),
+                ("flops", C.c_double), ("bytes", C.c_double)]
+
+
 _vp, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 
 # name -> (restype, argtypes); every symbol include/rtp_hip.h declares.
@@ -72,6 +77,8 @@ PROTOTYPES = {
     "rtp_moe_combine_dweight": (_i, [_vp, _i, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "rtp_sgd_step": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _f, _f]),
     "rtp_cast": (_i, [_vp, _i, _vp, _i, _vp, _i64]),
+    "rtp_profile_enable": (_i, [_i]),
+    "rtp_profile_collect": (_i, [C.POINTER(KernelStat), _i, C.POINTER(_i)]),
 }
 
 _lib: Optional[C.CDLL] = None
@@ -113,3 +120,16 @@ def require_device() -> None:
         buf = C.create_string_buffer(64)
         check(load().rtp_device_check(buf, 64))
         _device_checked = True
+
+
+def profile_enable(on: bool) -> None:
+    check(load().rtp_profile_enable(int(on)))
+
+
+def profile_collect():
+    """{kernel variant: {launches, total_ms, flops, bytes}} since profiling was enabled; clears the records."""
+    buf = (KernelStat * 64)()
+    n = C.c_int(0)
+    check(load().rtp_profile_collect(buf, 64, C.byref(n)))
+    return {buf[i].name.decode(): {"launches": buf[i].launches, "total_ms": buf[i].total_ms, "flops": buf[i].flops,
+                                   "bytes": buf[i].bytes} for i in range(n.value)}

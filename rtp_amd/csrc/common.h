@@ -68,4 +68,20 @@ __device__ __forceinline__ float wave_max(float v) {
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Optional per-launch timing (off by default; see rtp_profile_enable).  When enabled, the launch made
+// inside the scope is bracketed by two timing events on its own stream and booked under `name` with its
+// algorithmic flops / bytes.
+struct ProfileScope {
+  ProfileScope(hipStream_t stream, const char* name, double flops, double bytes);
+  ~ProfileScope();
+  ProfileScope(const ProfileScope&) = delete;
+  ProfileScope& operator=(const ProfileScope&) = delete;
+
+ private:
+  hipStream_t stream_;
+  hipEvent_t start_ = nullptr;
+  const char* name_;
+  double flops_, bytes_;
+};
+
 }  // namespace rtp

@@ -115,6 +115,7 @@ extern "C" int rtp_embedding_gather(void* stream, int dtype, const void* table, 
   const unsigned chunks = (unsigned)std::min<int64_t>(16, std::max<int64_t>(1, ceil_div(cols * (int64_t)esz, 4096)));
   dim3 grid((unsigned)n_ids, chunks);
   hipStream_t s = (hipStream_t)stream;
+  ProfileScope prof(s, "embedding_gather", 0.0, 2.0 * (double)n_ids * cols * esz + 8.0 * n_ids);
   if (dtype == RTP_F32)
     hipLaunchKernelGGL(gather_kernel<float>, grid, dim3(256), 0, s, (const float*)table, (long)ld_table,
                        (long)row_begin, (long)row_count, (long)cols, ids, (float*)out, (long)ld_out, vec);
@@ -167,6 +168,7 @@ extern "C" int rtp_embedding_scatter_add_det(void* stream, int dtype, const void
   const unsigned chunks = (unsigned)std::min<int64_t>(16, std::max<int64_t>(1, ceil_div(cols, 1024)));
   if (zero_fill) {
     RTP_REQUIRE(row_count < (1ll << 31), "rtp_embedding_scatter_add_det: too many rows");
+    ProfileScope prof(s, "embedding_grad_zero_fill", 0.0, (double)row_count * cols * gsz);
     hipLaunchKernelGGL(zero_rows_kernel, dim3((unsigned)row_count, chunks), dim3(256), 0, s, (char*)grad_table,
                        (long)(ld_grad_table * gsz), (long)(cols * gsz), (long)row_count);
     RTP_LAUNCH_CHECK();
@@ -183,6 +185,9 @@ extern "C" int rtp_embedding_scatter_add_det(void* stream, int dtype, const void
   hipLaunchKernelGGL((scatter_kernel<T, G>), grid, dim3(256), 0, s, (const T*)grad_out, (long)ld_grad_out,         \
                      (long)n_ids, keys, vals, (G*)grad_table, (long)ld_grad_table, (long)row_begin, (long)row_count, \
                      (long)cols, (long)padding_idx, scale_by_freq, overwrite)
+  // algorithmic bytes: read every upstream row once, write (or read-modify-write) every touched row once
+  ProfileScope prof(s, "embedding_scatter_add", (double)n_ids * cols,
+                    (double)n_ids * cols * ((dtype == RTP_F32 ? 4.0 : 2.0) + (zero_fill ? 1.0 : 2.0) * gsz) + 8.0 * n_ids);
   if (dtype == RTP_F32)
     RTP_SCATTER(float, float);
   else if (grad_table_f32)

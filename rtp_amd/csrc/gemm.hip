@@ -298,6 +298,19 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   RTP_REQUIRE(nb < (1ll << 31) && d->batch < 65536, "gemm grid too large (%lld tiles, batch %lld)",
               (long long)nb, (long long)d->batch);
   dim3 grid((unsigned)nb, (unsigned)d->batch, 1);
+  // variant name = the kernel template instance, e.g. gemm_bf16_64x64_kc_kc
+  static const char* const names[2][2][2][2] = {
+      {{{"gemm_f32_64x64_rc_rc", "gemm_f32_64x64_rc_kc"}, {"gemm_f32_64x64_kc_rc", "gemm_f32_64x64_kc_kc"}},
+       {{"gemm_f32_128x128_rc_rc", "gemm_f32_128x128_rc_kc"}, {"gemm_f32_128x128_kc_rc", "gemm_f32_128x128_kc_kc"}}},
+      {{{"gemm_bf16_64x64_rc_rc", "gemm_bf16_64x64_rc_kc"}, {"gemm_bf16_64x64_kc_rc", "gemm_bf16_64x64_kc_kc"}},
+       {{"gemm_bf16_128x128_rc_rc", "gemm_bf16_128x128_rc_kc"},
+        {"gemm_bf16_128x128_kc_rc", "gemm_bf16_128x128_kc_kc"}}}};
+  const double mnk = (double)d->m * (double)d->n * (double)d->batch;
+  const double out_sz = (d->flags & RTP_GEMM_OUT_F32) ? 4.0 : (double)sizeof(T);
+  const double cin_sz = d->c_in ? ((d->flags & RTP_GEMM_CIN_F32) ? 4.0 : (double)sizeof(T)) : 0.0;
+  const double bytes = ((double)d->m * d->k + (double)d->n * d->k) * d->batch * sizeof(T) + mnk * (out_sz + cin_sz);
+  ProfileScope prof(s, names[sizeof(T) == 2][big][d->a_kcontig != 0][d->b_kcontig != 0], 2.0 * mnk * (double)d->k,
+                    bytes);
   if (big) return launch_layout<T, 128, 128>(s, a, d->a_kcontig, d->b_kcontig, grid);
   return launch_layout<T, 64, 64>(s, a, d->a_kcontig, d->b_kcontig, grid);
 }
@@ -367,6 +380,7 @@ extern "C" int rtp_colsum(void* stream, int dtype, const void* x, int64_t m, int
   if (n == 0) return RTP_OK;
   hipStream_t s = (hipStream_t)stream;
   dim3 grid((unsigned)ceil_div(n, 64));
+  ProfileScope prof(s, "colsum", (double)m * n, (double)m * n * (dtype == RTP_F32 ? 4 : 2));
   if (dtype == RTP_F32)
     hipLaunchKernelGGL(colsum_kernel<float>, grid, dim3(kThreads), 0, s, (const float*)x, (long)m, (long)n,
                        (long)ld, out, 1, accumulate);

@@ -285,6 +285,8 @@ extern "C" int rtp_top2_route(void* stream, const float* logits, const float* no
   float* blockgate = (float*)(w + L.blockgate);
   const int C = (int)(2 * s / e);
   hipStream_t st = (hipStream_t)stream;
+  // three launches booked as one routing pass: reads logits+noise, writes gates and the compact records
+  ProfileScope prof(st, "top2_route", 0.0, (double)s * e * 12.0 + (double)s * 40.0);
   hipLaunchKernelGGL(route_choose_kernel, dim3((unsigned)L.nblocks), dim3(kTok), 0, st, logits, noise, (long)s,
                      (int)e, expert, rank, gates, slot_token, blockcnt, blockgate);
   RTP_LAUNCH_CHECK();
@@ -318,6 +320,7 @@ extern "C" int rtp_moe_dispatch(void* stream, int dtype, const void* x, int64_t 
               "rtp_moe_dispatch: bad shape");
   if (n_slots == 0 || cols == 0) return RTP_OK;
   dim3 grid((unsigned)n_slots, col_chunks(cols));
+  ProfileScope prof((hipStream_t)stream, "moe_dispatch", 0.0, 2.0 * (double)n_slots * cols * (dtype == RTP_F32 ? 4 : 2));
 #define A_(T) (const T*)x, (long)ld_x, slot_token, expert, slot, weight, (long)capacity, (long)cols, (T*)out, (long)ld_out
   if (dtype == RTP_F32)
     hipLaunchKernelGGL(dispatch_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, A_(float));
@@ -338,6 +341,7 @@ extern "C" int rtp_moe_combine(void* stream, int dtype, const void* y, int64_t l
               "rtp_moe_combine: bad shape");
   if (s == 0 || cols == 0) return RTP_OK;
   dim3 grid((unsigned)s, col_chunks(cols));
+  ProfileScope prof((hipStream_t)stream, "moe_combine", 4.0 * (double)s * cols, 3.0 * (double)s * cols * (dtype == RTP_F32 ? 4 : 2));
 #define A_(T) (const T*)y, (long)ld_y, expert, slot, keep, weight, (long)capacity, (long)cols, (T*)out, (long)ld_out
   if (dtype == RTP_F32)
     hipLaunchKernelGGL(combine_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, A_(float));

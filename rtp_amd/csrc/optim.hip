@@ -40,6 +40,7 @@ extern "C" int rtp_sgd_step(void* stream, int dtype, float* master, const void* 
   RTP_REQUIRE(n >= 0, "rtp_sgd_step: negative length");
   if (n == 0) return RTP_OK;
   hipStream_t s = (hipStream_t)stream;
+  ProfileScope prof(s, "sgd_step", 2.0 * (double)n, (double)n * (8.0 + (dtype == RTP_F32 ? 4 : 2) * (shadow ? 2.0 : 1.0)));
   if (dtype == RTP_F32)
     hipLaunchKernelGGL(sgd_kernel<float>, dim3(flat_grid(n)), dim3(256), 0, s, master, (const float*)grad,
                        (float*)shadow, (long)n, lr, clip);

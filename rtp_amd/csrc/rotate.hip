@@ -3,12 +3,47 @@
 #include "common.h"
 
 #include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
 
 namespace rtp {
 
 char* error_buffer() {
   static thread_local char buf[512] = {0};
   return buf;
+}
+
+struct ProfileRecord {
+  hipEvent_t start, stop;
+  const char* name;
+  double flops, bytes;
+};
+static std::mutex g_profile_mutex;
+static bool g_profile_on = false;
+static std::vector<ProfileRecord> g_profile_records;
+
+ProfileScope::ProfileScope(hipStream_t stream, const char* name, double flops, double bytes)
+    : stream_(stream), name_(name), flops_(flops), bytes_(bytes) {
+  if (!g_profile_on) return;
+  if (hipEventCreate(&start_) != hipSuccess) {
+    start_ = nullptr;
+    return;
+  }
+  (void)hipEventRecord(start_, stream_);
+}
+
+ProfileScope::~ProfileScope() {
+  if (!start_) return;
+  hipEvent_t stop = nullptr;
+  if (hipEventCreate(&stop) != hipSuccess) {
+    (void)hipEventDestroy(start_);
+    return;
+  }
+  (void)hipEventRecord(stop, stream_);
+  std::lock_guard<std::mutex> lock(g_profile_mutex);
+  g_profile_records.push_back({start_, stop, name_, flops_, bytes_});
 }
 
 struct Ring {
@@ -71,6 +106,7 @@ static int launch_copy(hipStream_t s, void* dst, const void* src, size_t bytes) 
   if (bytes == 0) return RTP_OK;
   RTP_REQUIRE(dst && src, "shard copy: null pointer");
   const int aligned = (((uintptr_t)dst | (uintptr_t)src) & 15) == 0;
+  ProfileScope prof(s, "shard_copy", 0.0, 2.0 * (double)bytes);
   hipLaunchKernelGGL(copy_kernel, dim3(copy_grid(bytes)), dim3(256), 0, s, (char*)dst, (const char*)src, bytes,
                      aligned);
   RTP_LAUNCH_CHECK();
@@ -179,5 +215,41 @@ extern "C" int rtp_zero_async(void* stream, void* dst, size_t bytes) {
   hipLaunchKernelGGL(zero_kernel, dim3(copy_grid(bytes)), dim3(256), 0, (hipStream_t)stream, (char*)dst, bytes,
                      aligned);
   RTP_LAUNCH_CHECK();
+  return RTP_OK;
+}
+
+extern "C" int rtp_profile_enable(int on) {
+  std::lock_guard<std::mutex> lock(g_profile_mutex);
+  g_profile_on = on != 0;
+  return RTP_OK;
+}
+
+extern "C" int rtp_profile_collect(rtp_kernel_stat* out, int max_out, int* n_out) {
+  RTP_REQUIRE(out && n_out && max_out > 0, "rtp_profile_collect: bad arguments");
+  RTP_HIP_TRY(hipDeviceSynchronize());
+  std::lock_guard<std::mutex> lock(g_profile_mutex);
+  std::map<std::string, rtp_kernel_stat> agg;
+  for (const ProfileRecord& r : g_profile_records) {
+    float ms = 0.0f;
+    if (hipEventElapsedTime(&ms, r.start, r.stop) != hipSuccess) ms = 0.0f;
+    (void)hipEventDestroy(r.start);
+    (void)hipEventDestroy(r.stop);
+    rtp_kernel_stat& st = agg[r.name];
+    if (st.launches == 0) {
+      memset(&st, 0, sizeof(st));
+      strncpy(st.name, r.name, sizeof(st.name) - 1);
+    }
+    st.launches += 1;
+    st.total_ms += ms;
+    st.flops += r.flops;
+    st.bytes += r.bytes;
+  }
+  g_profile_records.clear();
+  int n = 0;
+  for (auto& kv : agg) {
+    if (n >= max_out) break;
+    out[n++] = kv.second;
+  }
+  *n_out = n;
   return RTP_OK;
 }

@@ -76,6 +76,7 @@ extern "C" int rtp_softmax_fwd(void* stream, int dtype, const float* s, const fl
   RTP_REQUIRE(ceil_div(rows, kRowsPerBlock) < (1ll << 31), "rtp_softmax_fwd: too many rows");
   dim3 grid((unsigned)ceil_div(rows, kRowsPerBlock));
   hipStream_t st = (hipStream_t)stream;
+  ProfileScope prof(st, "softmax_fwd", 0.0, (double)rows * skv * (4.0 + (dtype == RTP_F32 ? 4 : 2)));
   if (dtype == RTP_F32)
     hipLaunchKernelGGL(softmax_fwd_kernel<float>, grid, dim3(256), 0, st, s, mask, causal, scale, (long)rows, (long)l,
                        (long)skv, (float*)p);
@@ -97,6 +98,7 @@ extern "C" int rtp_softmax_bwd(void* stream, int dtype, const void* p, const flo
   RTP_REQUIRE(ceil_div(rows, kRowsPerBlock) < (1ll << 31), "rtp_softmax_bwd: too many rows");
   dim3 grid((unsigned)ceil_div(rows, kRowsPerBlock));
   hipStream_t st = (hipStream_t)stream;
+  ProfileScope prof(st, "softmax_bwd", 0.0, (double)rows * skv * (4.0 + 2.0 * (dtype == RTP_F32 ? 4 : 2)));
   if (dtype == RTP_F32)
     hipLaunchKernelGGL(softmax_bwd_kernel<float>, grid, dim3(256), 0, st, (const float*)p, dp, scale, (long)rows,
                        (long)skv, (float*)ds);
