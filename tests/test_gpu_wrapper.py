@@ -1,0 +1,64 @@
+"""RotatedTensorParallel: wrap a stock torch model in place and compare it with an untouched copy
+(the structure of the reference's test.py:126-195 and test_net.py:135-177)."""
+import copy
+
+import pytest
+import torch
+import torch.nn as nn
+
+from gpu_util import DEV, assert_close
+from oracle import rtp_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+class Net(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.emb = nn.Embedding(40, 16)
+        self.attn = nn.MultiheadAttention(16, 4)
+        self.fc1 = nn.Linear(16, 24)   # out_features % ws == 0 -> column shards
+        self.fc2 = nn.Linear(24, 6)    # 6 % 4 != 0 but 24 % 4 == 0 -> row shards
+        self.norm = nn.LayerNorm(16)
+
+    def forward(self, ids):
+        x = self.emb(ids)
+        x = self.norm(x + self.attn(x, x, x, need_weights=False)[0])
+        return self.fc2(torch.relu(self.fc1(x)))
+
+
+def test_wrapper_matches_unwrapped_model():
+    from rtp_amd import emulate_shards
+    from rtp_amd.rotated_tensor_parallel import FlyweightWarpper, RotatedTensorParallel
+    ws = 4
+    ref = Net()
+    with emulate_shards(ws):
+        model = RotatedTensorParallel(copy.deepcopy(ref)).to(DEV)
+    kinds = [type(w.rotated).__name__ for w in model.FlyweightModule_list]
+    assert kinds == ["ParallelEmbedding", "ParallelMultiheadAttention", "ColumnParallelLinear", "RowParallelLinear"]
+    assert isinstance(model.module.fc2, FlyweightWarpper) and model.module.fc2.row_partition
+    assert isinstance(model.module.norm, nn.LayerNorm)
+    ids = torch.randint(0, 40, (7, 3))
+    g = torch.randn(7, 3, 6)
+    out = model(ids.to(DEV))
+    out.backward(g.to(DEV))
+    ref_out = ref(ids)
+    ref_out.backward(g)
+    assert_close(out, ref_out, torch.float32, "output")
+    m = model.module
+    # rank-r shard gradient == the matching slice of the unsharded gradient (test.py:182-193)
+    assert_close(torch.cat([s.weight.grad for s in m.fc1.module_list], 0), ref.fc1.weight.grad, torch.float32, "fc1")
+    assert_close(torch.cat([s.weight.grad for s in m.fc2.module_list], 1), ref.fc2.weight.grad, torch.float32, "fc2")
+    assert_close(m.fc2.module.bias.grad, ref.fc2.bias.grad, torch.float32, "fc2 bias")
+    assert_close(torch.cat([s.weight.grad for s in m.emb.module_list], 1), ref.emb.weight.grad, torch.float32, "emb")
+    assert_close(O.attention_grad_reinterleave([s.in_proj_weight.grad for s in m.attn.module_list], ws),
+                 ref.attn.in_proj_weight.grad, torch.float32, "attn in_proj")
+    assert_close(m.norm.weight.grad, ref.norm.weight.grad, torch.float32, "layernorm")
+    assert m.fc1.flat_param.data_ptr() == m.fc1.module.weight.data_ptr()
+
+
+def test_wrapper_indivisible_linear_raises():
+    from rtp_amd import emulate_shards
+    from rtp_amd.rotated_tensor_parallel import RotatedTensorParallel
+    with emulate_shards(4), pytest.raises(ValueError):
+        RotatedTensorParallel(nn.Sequential(nn.Linear(6, 7)))
