@@ -62,6 +62,17 @@ int rtp_device_check(char* name_out, int name_len);
  * pointer advances by zo*stride_o + zi*stride_i elements (so a (batch, head) pair can index a
  * packed [L, N, 3E] projection without a re-layout).
  *
+ * Several rotation shards in one launch (what the reference does as a Python loop of ws small
+ * matmuls, rtp/module/linear.py:211-220, :379-392):
+ *   groups: `groups` independent problems of identical shape; group g advances every operand by
+ *           g*stride_g elements (shard g's weight/bias in the flat shard buffer, its output column
+ *           block, ...).  Replaces the per-shard F.linear + torch.cat of a column-parallel layer.
+ *   ksegs:  the contraction is the concatenation of `ksegs` segments of length k; segment s reads A
+ *           at a + s*a_sk and B at b + s*b_sk.  Replaces the `output + output_parallel` running sum
+ *           over shards of row-parallel layers and the autograd sum of input gradients; the sum is
+ *           kept in the fp32 MFMA accumulators.  If bias_sk != 0 the epilogue adds one bias per
+ *           segment (bias + s*bias_sk), as every row-parallel shard carries bias/ws.
+ *
  * Epilogue, in this order:  v = alpha*acc;  if c_in: v += c_in[m,n];  if bias: v += bias[n];
  * if RTP_GEMM_RELU: v = max(v,0);  if gate: v = gate[m,n] > 0 ? v : 0;  store to c_out as fp32
  * (RTP_GEMM_OUT_F32) or as `dtype`.  c_in is read as fp32 when RTP_GEMM_CIN_F32 is set, else as
@@ -84,6 +95,9 @@ typedef struct {
   int64_t lda, ldb, ldc, ld_cin, ld_gate;
   int64_t batch, zdiv; /* batch >= 1, zdiv >= 1 */
   int64_t a_so, a_si, b_so, b_si, c_so, c_si, cin_so, cin_si, gate_so, gate_si, bias_so, bias_si;
+  int64_t groups, ksegs; /* >= 1 */
+  int64_t a_sg, b_sg, c_sg, cin_sg, gate_sg, bias_sg; /* per-group element strides */
+  int64_t a_sk, b_sk, bias_sk;                        /* per-K-segment element strides */
   float alpha;
   int32_t flags;
   int32_t a_kcontig, b_kcontig;
@@ -94,11 +108,16 @@ int rtp_gemm(void* stream, int dtype, const rtp_gemm_desc* d);
 /* sizeof(rtp_gemm_desc) as this library was compiled: lets a binding verify its struct layout. */
 size_t rtp_gemm_desc_size(void);
 
-/* out[n] (+)= sum_m x[m*ld + n]  in fp32, fixed summation order (deterministic).  The bias
- * gradient of nn.Linear's backward (reference: autograd of rtp/module/linear.py:216).
- * out is fp32 if out_f32 else `dtype`; accumulate != 0 adds to the existing contents. */
-int rtp_colsum(void* stream, int dtype, const void* x, int64_t m, int64_t n, int64_t ld,
-               void* out, int out_f32, int accumulate);
+/* Column sums in fp32 with a fixed summation order (deterministic): the bias gradient of nn.Linear's
+ * backward (reference: autograd of rtp/module/linear.py:216).  Column c of x[m, n] (leading
+ * dimension ld) is written to out[(c / seg) * seg_stride + c % seg], so the bias gradients of all
+ * shards of a layer (seg columns each, seg_stride apart in the flat gradient buffer) come from one
+ * call; seg <= 0 means one contiguous segment.  out is fp32 if out_f32 else `dtype`; accumulate != 0
+ * adds to the existing contents.  workspace: rtp_colsum_workspace_bytes(m, n) bytes, 256-aligned. */
+size_t rtp_colsum_workspace_bytes(int64_t m, int64_t n);
+int rtp_colsum(void* stream, int dtype, const void* x, int64_t m, int64_t n, int64_t ld, void* out,
+               int out_f32, int accumulate, int64_t seg, int64_t seg_stride, void* workspace,
+               size_t workspace_bytes);
 
 /* ---------------------------------------------------------------------------------------------
  * Shard rotation (reference: rtp/module/collectives.py:202-257 _left/_right_shift_buffer +
@@ -108,17 +127,23 @@ int rtp_colsum(void* stream, int dtype, const void* x, int64_t m, int64_t n, int
  * that is consuming the other slot.
  *
  * rtp_ring_create makes the side stream and the fencing events (no device memory).
- *   begin(main)                  side stream waits for everything queued on main so far
- *   prefetch(slot, dst, src, n)  side: wait until the last consumer of `slot` released it, copy
- *   acquire(main, slot)          main waits for the copy into `slot`
+ *   prefetch(main, slot, dst, src, n)  side stream: wait until the last consumer of `slot` released
+ *                                it, copy.  May be called several times per slot before acquire.
+ *                                A copy depends only on its slot, so the shards of the NEXT layer
+ *                                stream in while the current layer still computes.
+ *   acquire(main, slot)          main waits for the copies into `slot`
  *   release(main, slot)          marks the point on main after which `slot` may be overwritten
- * After the last acquire of a begin..end sequence the side stream is fully joined into main, so a
- * sequence may be recorded into a HIP graph by capturing main.
+ *   fence(main)                  the shards' home storage is modified by work queued on main up to
+ *                                here (optimizer step, weight load): the next prefetch waits for it.
+ *                                The first prefetch after create behaves as if fenced.
+ * Every copy is followed by an acquire on main, so the side stream is always joined back: a
+ * sequence may be recorded into a HIP graph by capturing main (the side stream is forked from main
+ * automatically when main is capturing).  After a capture ends, call fence before eager use.
  * --------------------------------------------------------------------------------------------- */
 int rtp_ring_create(void** ring_out);
 int rtp_ring_destroy(void* ring);
-int rtp_ring_begin(void* ring, void* main_stream);
-int rtp_ring_prefetch(void* ring, int slot, void* dst, const void* src, size_t bytes);
+int rtp_ring_fence(void* ring, void* main_stream);
+int rtp_ring_prefetch(void* ring, void* main_stream, int slot, void* dst, const void* src, size_t bytes);
 int rtp_ring_acquire(void* ring, void* main_stream, int slot);
 int rtp_ring_release(void* ring, void* main_stream, int slot);
 
@@ -135,7 +160,8 @@ int rtp_zero_async(void* stream, void* dst, size_t bytes);
  * table, stored row-major with leading dimension ld_table; the reference shards columns
  * (embedding.py:65-71) and uses row_begin = 0, row_count = V.
  *   gather:      out[t, 0:cols] = table[ids[t] - row_begin, 0:cols]   (ids outside the row range
- *                leave out[t] untouched); out has leading dimension ld_out.
+ *                leave out[t] untouched); out has leading dimension ld_out.  `groups` shards are
+ *                gathered by one launch: shard g reads table + g*table_sg, writes out + g*out_sg.
  *   scatter-add: grad_table[ids[t] - row_begin, :] += grad_out[t, :]  summed per row in ascending t
  *                (sequential fp32 adds starting from +0.0f: bit-identical to torch's CPU
  *                nn.Embedding backward / index_add_).  Rows that receive no token are zero-filled
@@ -146,7 +172,8 @@ int rtp_zero_async(void* stream, void* dst, size_t bytes);
  * --------------------------------------------------------------------------------------------- */
 int rtp_embedding_gather(void* stream, int dtype, const void* table, int64_t ld_table,
                          int64_t row_begin, int64_t row_count, int64_t cols, const int64_t* ids,
-                         int64_t n_ids, void* out, int64_t ld_out);
+                         int64_t n_ids, void* out, int64_t ld_out, int64_t groups, int64_t table_sg,
+                         int64_t out_sg);
 
 size_t rtp_embedding_scatter_workspace_bytes(int64_t n_ids);
 

@@ -35,6 +35,10 @@ class GemmDesc(C.Structure):
         ("a_so", C.c_int64), ("a_si", C.c_int64), ("b_so", C.c_int64), ("b_si", C.c_int64),
         ("c_so", C.c_int64), ("c_si", C.c_int64), ("cin_so", C.c_int64), ("cin_si", C.c_int64),
         ("gate_so", C.c_int64), ("gate_si", C.c_int64), ("bias_so", C.c_int64), ("bias_si", C.c_int64),
+        ("groups", C.c_int64), ("ksegs", C.c_int64),
+        ("a_sg", C.c_int64), ("b_sg", C.c_int64), ("c_sg", C.c_int64), ("cin_sg", C.c_int64),
+        ("gate_sg", C.c_int64), ("bias_sg", C.c_int64), ("a_sk", C.c_int64), ("b_sk", C.c_int64),
+        ("bias_sk", C.c_int64),
         ("alpha", C.c_float), ("flags", C.c_int32), ("a_kcontig", C.c_int32), ("b_kcontig", C.c_int32),
     ]
 
@@ -53,16 +57,17 @@ PROTOTYPES = {
     "rtp_device_check": (_i, [C.c_char_p, _i]),
     "rtp_gemm": (_i, [_vp, _i, C.POINTER(GemmDesc)]),
     "rtp_gemm_desc_size": (_sz, []),
-    "rtp_colsum": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _vp, _i, _i]),
+    "rtp_colsum_workspace_bytes": (_sz, [_i64, _i64]),
+    "rtp_colsum": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _vp, _i, _i, _i64, _i64, _vp, _sz]),
     "rtp_ring_create": (_i, [C.POINTER(_vp)]),
     "rtp_ring_destroy": (_i, [_vp]),
-    "rtp_ring_begin": (_i, [_vp, _vp]),
-    "rtp_ring_prefetch": (_i, [_vp, _i, _vp, _vp, _sz]),
+    "rtp_ring_fence": (_i, [_vp, _vp]),
+    "rtp_ring_prefetch": (_i, [_vp, _vp, _i, _vp, _vp, _sz]),
     "rtp_ring_acquire": (_i, [_vp, _vp, _i]),
     "rtp_ring_release": (_i, [_vp, _vp, _i]),
     "rtp_shard_copy_async": (_i, [_vp, _vp, _vp, _sz]),
     "rtp_zero_async": (_i, [_vp, _vp, _sz]),
-    "rtp_embedding_gather": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _i64]),
+    "rtp_embedding_gather": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i64]),
     "rtp_embedding_scatter_workspace_bytes": (_sz, [_i64]),
     "rtp_embedding_sort_ids": (_i, [_vp, _vp, _i64, _vp, _sz]),
     "rtp_embedding_scatter_add_det": (_i, [_vp, _i, _vp, _i64, _i64, _vp, _vp, _i64, _i, _i64, _i64, _i64,

@@ -10,12 +10,13 @@ namespace rtp {
 // One workgroup per (token, 4 KiB column chunk); 16-byte lanes when the shard rectangle allows it.
 template <typename T>
 __global__ __launch_bounds__(256) void gather_kernel(const T* table, long ld_table, long row_begin, long row_count,
-                                                     long cols, const int64_t* ids, T* out, long ld_out, int vec) {
+                                                     long cols, const int64_t* ids, T* out, long ld_out, int vec,
+                                                     long table_sg, long out_sg) {
   const long t = blockIdx.x;
   const long row = ids[t] - row_begin;
   if (row < 0 || row >= row_count) return;
-  const T* src = table + row * ld_table;
-  T* dst = out + t * ld_out;
+  const T* src = table + blockIdx.z * table_sg + row * ld_table;
+  T* dst = out + blockIdx.z * out_sg + t * ld_out;
   constexpr int VEC = 16 / sizeof(T);
   if (vec) {
     const long nvec = cols / VEC;
@@ -101,27 +102,31 @@ using namespace rtp;
 
 extern "C" int rtp_embedding_gather(void* stream, int dtype, const void* table, int64_t ld_table, int64_t row_begin,
                                     int64_t row_count, int64_t cols, const int64_t* ids, int64_t n_ids, void* out,
-                                    int64_t ld_out) {
+                                    int64_t ld_out, int64_t groups, int64_t table_sg, int64_t out_sg) {
   RTP_REQUIRE(table && ids && out, "rtp_embedding_gather: null pointer");
   RTP_REQUIRE(cols >= 0 && ld_table >= cols && ld_out >= cols && row_count >= 0 && n_ids >= 0,
               "rtp_embedding_gather: bad shape cols=%lld ld_table=%lld ld_out=%lld", (long long)cols,
               (long long)ld_table, (long long)ld_out);
   if (n_ids == 0 || cols == 0) return RTP_OK;
   RTP_REQUIRE(n_ids < (1ll << 31), "rtp_embedding_gather: too many ids");
+  RTP_REQUIRE(groups >= 1 && groups < 65536, "rtp_embedding_gather: groups=%lld out of range", (long long)groups);
   const size_t esz = dtype == RTP_F32 ? 4 : 2;
   RTP_REQUIRE(dtype == RTP_F32 || dtype == RTP_BF16, "rtp_embedding_gather: unknown dtype %d", dtype);
   const int vec = ((uintptr_t)table % 16 == 0) && ((uintptr_t)out % 16 == 0) && (ld_table * esz) % 16 == 0 &&
-                  (ld_out * esz) % 16 == 0 && (cols * esz) % 16 == 0;
+                  (ld_out * esz) % 16 == 0 && (cols * esz) % 16 == 0 && (table_sg * esz) % 16 == 0 &&
+                  (out_sg * esz) % 16 == 0;
   const unsigned chunks = (unsigned)std::min<int64_t>(16, std::max<int64_t>(1, ceil_div(cols * (int64_t)esz, 4096)));
-  dim3 grid((unsigned)n_ids, chunks);
+  dim3 grid((unsigned)n_ids, chunks, (unsigned)groups);
   hipStream_t s = (hipStream_t)stream;
-  ProfileScope prof(s, "embedding_gather", 0.0, 2.0 * (double)n_ids * cols * esz + 8.0 * n_ids);
+  ProfileScope prof(s, "embedding_gather", 0.0, (2.0 * (double)n_ids * cols * esz + 8.0 * n_ids) * groups);
   if (dtype == RTP_F32)
     hipLaunchKernelGGL(gather_kernel<float>, grid, dim3(256), 0, s, (const float*)table, (long)ld_table,
-                       (long)row_begin, (long)row_count, (long)cols, ids, (float*)out, (long)ld_out, vec);
+                       (long)row_begin, (long)row_count, (long)cols, ids, (float*)out, (long)ld_out, vec,
+                       (long)table_sg, (long)out_sg);
   else
     hipLaunchKernelGGL(gather_kernel<bf16_t>, grid, dim3(256), 0, s, (const bf16_t*)table, (long)ld_table,
-                       (long)row_begin, (long)row_count, (long)cols, ids, (bf16_t*)out, (long)ld_out, vec);
+                       (long)row_begin, (long)row_count, (long)cols, ids, (bf16_t*)out, (long)ld_out, vec,
+                       (long)table_sg, (long)out_sg);
   RTP_LAUNCH_CHECK();
   return RTP_OK;
 }

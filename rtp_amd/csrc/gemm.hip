@@ -1,12 +1,18 @@
 // LDS-staged MFMA GEMM for gfx950 (fp32 via v_mfma_f32_32x32x2_f32, bf16 via v_mfma_f32_32x32x16_bf16)
 // with the four operand layouts the rotated layers need (forward X W^T, input gradient dY W, weight
-// gradient dY^T X, batched q k^T / p v) and a fused epilogue (accumulate, bias, ReLU, ReLU-mask).
+// gradient dY^T X, batched q k^T / p v), a fused epilogue (accumulate, bias, ReLU, ReLU-mask), and two
+// ways of covering several rotation shards in ONE launch:
+//   groups     : independent problems that differ only by a constant pointer stride per operand
+//                (shard s of a column-parallel layer: W_s, b_s and the output column block s);
+//   K segments : one output whose contraction runs over several shards in turn
+//                (row-parallel outputs, input gradients of column-parallel layers: sum_s dY_s W_s),
+//                accumulated in the MFMA accumulators, so the cross-shard sum never leaves registers.
 //
 // Work decomposition: 256 threads = 4 wavefronts in a 2x2 arrangement over a BM x BN output tile;
 // each wavefront owns (BM/2)x(BN/2) as 32x32 MFMA blocks with fp32 accumulators in VGPRs.  The K loop
-// moves 64-byte-per-row slabs (32 bf16 / 16 fp32 values of k) global -> registers -> LDS, double
-// buffered in LDS so one barrier per slab suffices; the global loads of slab t+1 are in flight while
-// the MFMAs of slab t run.
+// moves 128-byte-per-row slabs (64 bf16 / 32 fp32 values of k) global -> registers -> LDS.  LDS is
+// double buffered (one barrier per slab) and the global loads run DEPTH slabs ahead of the MFMAs in a
+// ring of register buffers, which is what hides HBM/L2 latency when only one workgroup fits a CU.
 #include "common.h"
 
 namespace rtp {
@@ -21,10 +27,12 @@ struct GemmArgs {
   const char* c_in;
   const char* bias;
   const char* gate;
-  int m, n, k;
+  int m, n, k, ksegs;
   long lda, ldb, ldc, ld_cin, ld_gate;
-  int zdiv;
+  int batch, zdiv;
   long a_so, a_si, b_so, b_si, c_so, c_si, cin_so, cin_si, gate_so, gate_si, bias_so, bias_si;
+  long a_sg, b_sg, c_sg, cin_sg, gate_sg, bias_sg;
+  long a_sk, b_sk, bias_sk;
   float alpha;
   int flags;
   int vec_a, vec_b;
@@ -32,23 +40,31 @@ struct GemmArgs {
 };
 
 constexpr int kThreads = 256;
-constexpr int kRowPitchKC = 80;  // bytes per tile row when k is contiguous: 64 data + 16 pad
+constexpr int kSlabBytes = 128;               // bytes of k per tile row and slab
+constexpr int kRowPitchKC = kSlabBytes + 16;  // LDS row pitch when k is contiguous (16 B pad)
 
 // Moves one R x BK operand slab global -> registers -> LDS.
-//   KC  (k contiguous in memory): LDS holds [row][k], row pitch 80 bytes.
+//   KC  (k contiguous in memory): LDS holds [row][k], row pitch 144 bytes.
 //   !KC (rows contiguous in memory): LDS holds [k][row], k pitch R*sizeof(T)+16 bytes.
 template <typename T, int R, bool KC>
-struct SlabLoader {
+struct Slab {
   static constexpr int VEC = 16 / sizeof(T);
-  static constexpr int BK = 4 * VEC;
-  static constexpr int NV = R * 4 / kThreads;
-  static constexpr int RV = R / VEC;  // vectors per k line when rows are contiguous
+  static constexpr int BK = kSlabBytes / sizeof(T);
+  static constexpr int KV = BK / VEC;           // 16-byte vectors per row (= 8)
+  static constexpr int NV = R * KV / kThreads;  // vectors per thread
+  static constexpr int RV = R / VEC;            // vectors per k line when rows are contiguous
   static constexpr int PITCH = KC ? kRowPitchKC : (R * (int)sizeof(T) + 16);
   static constexpr int BYTES = KC ? R * kRowPitchKC : BK * PITCH;
   uint4 reg[NV];
 
-  __device__ __forceinline__ void load(const T* base, long ld, int row0, int rows, int k0, int kdim,
-                                       bool vec_ok, int tid) {
+  // FAST: every 16-byte vector of the slab is either wholly inside the operand or wholly outside it
+  // (guaranteed by the host: aligned pointers and strides, extents that are multiples of VEC), so a
+  // vector is loaded unconditionally from a clamped address and, if it lies beyond the contraction
+  // length, replaced by zeros with a select.  No branches, so all loads of a slab issue back to back.
+  // Rows beyond the operand are clamped too: they only feed accumulators the epilogue never stores.
+  // !FAST: element-wise guarded loads for ragged or unaligned operands.
+  template <bool FAST>
+  __device__ __forceinline__ void load(const T* base, long ld, int row0, int rows, int k0, int kdim, int tid) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int v = tid + i * kThreads;
@@ -57,22 +73,30 @@ struct SlabLoader {
         T e[VEC];
       } u;
       if (KC) {
-        const int row = row0 + (v >> 2);
-        const int k = k0 + (v & 3) * VEC;
-        const T* src = base + (long)row * ld + k;
-        if (vec_ok && row < rows && k + VEC <= kdim) {
-          u.q = *reinterpret_cast<const uint4*>(src);
+        const int row = row0 + v / KV;
+        const int k = k0 + (v % KV) * VEC;
+        if (FAST) {
+          const int rc = row < rows ? row : rows - 1;
+          const bool live = k < kdim;
+          const int kc = live ? k : 0;
+          u.q = *reinterpret_cast<const uint4*>(base + (long)rc * ld + kc);
+          if (!live) u.q = make_uint4(0, 0, 0, 0);
         } else {
+          const T* src = base + (long)row * ld + k;
 #pragma unroll
           for (int e = 0; e < VEC; ++e) u.e[e] = (row < rows && k + e < kdim) ? src[e] : (T)0.0f;
         }
       } else {
         const int k = k0 + v / RV;
         const int row = row0 + (v % RV) * VEC;
-        const T* src = base + (long)k * ld + row;
-        if (vec_ok && k < kdim && row + VEC <= rows) {
-          u.q = *reinterpret_cast<const uint4*>(src);
+        if (FAST) {
+          const bool live = k < kdim;
+          const int kc = live ? k : 0;
+          const int rc = row < rows ? row : 0;
+          u.q = *reinterpret_cast<const uint4*>(base + (long)kc * ld + rc);
+          if (!live) u.q = make_uint4(0, 0, 0, 0);
         } else {
+          const T* src = base + (long)k * ld + row;
 #pragma unroll
           for (int e = 0; e < VEC; ++e) u.e[e] = (k < kdim && row + e < rows) ? src[e] : (T)0.0f;
         }
@@ -85,7 +109,7 @@ struct SlabLoader {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int v = tid + i * kThreads;
-      char* dst = KC ? lds + (v >> 2) * kRowPitchKC + (v & 3) * 16 : lds + (v / RV) * PITCH + (v % RV) * 16;
+      char* dst = KC ? lds + (v / KV) * kRowPitchKC + (v % KV) * 16 : lds + (v / RV) * PITCH + (v % RV) * 16;
       *reinterpret_cast<uint4*>(dst) = reg[i];
     }
   }
@@ -107,7 +131,7 @@ struct Frag<float> {
 template <typename T, int R, bool KC>
 __device__ __forceinline__ Frag<T> read_frag(const char* lds, int row, int ks, int g) {
   constexpr int VEC = 16 / sizeof(T);
-  constexpr int PITCH = SlabLoader<T, R, KC>::PITCH;
+  constexpr int PITCH = Slab<T, R, KC>::PITCH;
   union {
     uint4 q;
     T e[VEC];
@@ -132,13 +156,42 @@ __device__ __forceinline__ void mma(const Frag<float>& a, const Frag<float>& b, 
   for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.f[e], b.f[e], c, 0, 0, 0);
 }
 
-template <typename T, int BM, int BN, bool AKC, bool BKC>
+template <typename T, int BM, int BN, bool AKC, bool BKC, int DEPTH, bool FAST>
+struct GemmTile {
+  using LA = Slab<T, BM, AKC>;
+  using LB = Slab<T, BN, BKC>;
+  static constexpr int BK = LA::BK;
+  static constexpr int WM = BM / 2, WN = BN / 2, MT = WM / 32, NT = WN / 32;
+  static constexpr int STAGE = LA::BYTES + LB::BYTES;
+  static constexpr int KSTEPS = 4;  // slab k extent / (2*VEC)
+
+  const GemmArgs& p;
+  const T* A;
+  const T* B;
+  int m0, n0, tid, nk_seg;
+  LA la[DEPTH];
+  LB lb[DEPTH];
+
+  __device__ __forceinline__ GemmTile(const GemmArgs& args) : p(args) {}
+
+  template <int R>
+  __device__ __forceinline__ void fetch(int slab) {
+    const int seg = slab / nk_seg;
+    const int k0 = (slab - seg * nk_seg) * BK;
+    la[R].template load<FAST>(A + seg * p.a_sk, p.lda, m0, p.m, k0, p.k, tid);
+    lb[R].template load<FAST>(B + seg * p.b_sk, p.ldb, n0, p.n, k0, p.k, tid);
+  }
+  template <int R>
+  __device__ __forceinline__ void stash(char* stage) {
+    la[R].store(stage, tid);
+    lb[R].store(stage + LA::BYTES, tid);
+  }
+};
+
+template <typename T, int BM, int BN, bool AKC, bool BKC, int DEPTH, bool FAST>
 __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs p) {
-  using LA = SlabLoader<T, BM, AKC>;
-  using LB = SlabLoader<T, BN, BKC>;
-  constexpr int BK = LA::BK;
-  constexpr int WM = BM / 2, WN = BN / 2, MT = WM / 32, NT = WN / 32;
-  constexpr int STAGE = LA::BYTES + LB::BYTES;
+  using G = GemmTile<T, BM, BN, AKC, BKC, DEPTH, FAST>;
+  constexpr int MT = G::MT, NT = G::NT, WM = G::WM, WN = G::WN, STAGE = G::STAGE;
   __shared__ __attribute__((aligned(16))) char lds[2 * STAGE];
 
   const int tid = threadIdx.x;
@@ -151,12 +204,18 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs p) {
   int bid = blockIdx.x;
   const int nb = p.tiles_m * p.tiles_n;
   if ((nb & 7) == 0) bid = (bid & 7) * (nb >> 3) + (bid >> 3);
-  const int m0 = (bid / p.tiles_n) * BM;
-  const int n0 = (bid % p.tiles_n) * BN;
 
-  const long zo = blockIdx.y / p.zdiv, zi = blockIdx.y % p.zdiv;
-  const T* A = reinterpret_cast<const T*>(p.a) + zo * p.a_so + zi * p.a_si;
-  const T* B = reinterpret_cast<const T*>(p.b) + zo * p.b_so + zi * p.b_si;
+  const int grp = blockIdx.y / p.batch, zb = blockIdx.y % p.batch;
+  const long zo = zb / p.zdiv, zi = zb % p.zdiv;
+
+  G t(p);
+  t.tid = tid;
+  t.m0 = (bid / p.tiles_n) * BM;
+  t.n0 = (bid % p.tiles_n) * BN;
+  t.A = reinterpret_cast<const T*>(p.a) + grp * p.a_sg + zo * p.a_so + zi * p.a_si;
+  t.B = reinterpret_cast<const T*>(p.b) + grp * p.b_sg + zo * p.b_so + zi * p.b_si;
+  t.nk_seg = (p.k + G::BK - 1) / G::BK;
+  const int nk = t.nk_seg * p.ksegs;
 
   f32x16 acc[MT][NT];
 #pragma unroll
@@ -166,27 +225,21 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  LA la;
-  LB lb;
-  const int nk = (p.k + BK - 1) / BK;
-  if (nk > 0) {
-    la.load(A, p.lda, m0, p.m, 0, p.k, p.vec_a, tid);
-    lb.load(B, p.ldb, n0, p.n, 0, p.k, p.vec_b, tid);
-    la.store(lds, tid);
-    lb.store(lds + LA::BYTES, tid);
-  }
+  // Prologue: slabs 0..DEPTH-1 into the register ring, slab 0 on into LDS stage 0.
+  if (nk > 0) t.template fetch<0>(0);
+  if (DEPTH > 1 && nk > 1) t.template fetch<1 % DEPTH>(1);
+  if (DEPTH > 2 && nk > 2) t.template fetch<2 % DEPTH>(2);
+  if (nk > 0) t.template stash<0>(lds);
   __syncthreads();
 
-  for (int kt = 0; kt < nk; ++kt) {
+  // Steady state for slab kt (register slot kt % DEPTH was just emptied into LDS): refill that slot
+  // with slab kt+DEPTH, run the MFMAs of slab kt from LDS stage kt&1, move slab kt+1 from its register
+  // slot to the other LDS stage, barrier.
+  auto compute = [&](int kt) {
     const char* sa = lds + (kt & 1) * STAGE;
-    const char* sb = sa + LA::BYTES;
-    const bool more = kt + 1 < nk;
-    if (more) {
-      la.load(A, p.lda, m0, p.m, (kt + 1) * BK, p.k, p.vec_a, tid);
-      lb.load(B, p.ldb, n0, p.n, (kt + 1) * BK, p.k, p.vec_b, tid);
-    }
+    const char* sb = sa + G::LA::BYTES;
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
+    for (int ks = 0; ks < G::KSTEPS; ++ks) {
       Frag<T> fa[MT], fb[NT];
 #pragma unroll
       for (int i = 0; i < MT; ++i) fa[i] = read_frag<T, BM, AKC>(sa, wm * WM + i * 32 + li, ks, g);
@@ -197,12 +250,27 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs p) {
 #pragma unroll
         for (int j = 0; j < NT; ++j) mma(fa[i], fb[j], acc[i][j]);
     }
-    if (more) {
-      char* da = lds + ((kt + 1) & 1) * STAGE;
-      la.store(da, tid);
-      lb.store(da + LA::BYTES, tid);
-    }
+  };
+
+  for (int kt = 0; kt < nk; kt += DEPTH) {
+    if (kt + DEPTH < nk) t.template fetch<0>(kt + DEPTH);
+    compute(kt);
+    if (kt + 1 < nk) t.template stash<1 % DEPTH>(lds + ((kt + 1) & 1) * STAGE);
     __syncthreads();
+    if (DEPTH > 1) {
+      if (kt + 1 >= nk) break;
+      if (kt + 1 + DEPTH < nk) t.template fetch<1 % DEPTH>(kt + 1 + DEPTH);
+      compute(kt + 1);
+      if (kt + 2 < nk) t.template stash<2 % DEPTH>(lds + ((kt + 2) & 1) * STAGE);
+      __syncthreads();
+    }
+    if (DEPTH > 2) {
+      if (kt + 2 >= nk) break;
+      if (kt + 2 + DEPTH < nk) t.template fetch<2 % DEPTH>(kt + 2 + DEPTH);
+      compute(kt + 2);
+      if (kt + 3 < nk) t.template stash<0>(lds + ((kt + 3) & 1) * STAGE);
+      __syncthreads();
+    }
   }
 
   // Epilogue.  Accumulator register r of lane (li, g) is output row 8*(r/4) + 4*g + r%4, column li
@@ -210,22 +278,29 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs p) {
   const bool out_f32 = p.flags & RTP_GEMM_OUT_F32;
   const bool cin_f32 = p.flags & RTP_GEMM_CIN_F32;
   const bool relu = p.flags & RTP_GEMM_RELU;
-  char* cbase = p.c_out + (zo * p.c_so + zi * p.c_si) * (out_f32 ? 4 : (long)sizeof(T));
+  char* cbase = p.c_out + (grp * p.c_sg + zo * p.c_so + zi * p.c_si) * (out_f32 ? 4 : (long)sizeof(T));
   const char* cin =
-      p.c_in ? p.c_in + (zo * p.cin_so + zi * p.cin_si) * (cin_f32 ? 4 : (long)sizeof(T)) : nullptr;
-  const T* bias = p.bias ? reinterpret_cast<const T*>(p.bias) + zo * p.bias_so + zi * p.bias_si : nullptr;
-  const T* gate = p.gate ? reinterpret_cast<const T*>(p.gate) + zo * p.gate_so + zi * p.gate_si : nullptr;
+      p.c_in ? p.c_in + (grp * p.cin_sg + zo * p.cin_so + zi * p.cin_si) * (cin_f32 ? 4 : (long)sizeof(T)) : nullptr;
+  const T* bias =
+      p.bias ? reinterpret_cast<const T*>(p.bias) + grp * p.bias_sg + zo * p.bias_so + zi * p.bias_si : nullptr;
+  const T* gate =
+      p.gate ? reinterpret_cast<const T*>(p.gate) + grp * p.gate_sg + zo * p.gate_so + zi * p.gate_si : nullptr;
 
 #pragma unroll
   for (int i = 0; i < MT; ++i) {
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
-      const int col = n0 + wn * WN + j * 32 + li;
+      const int col = t.n0 + wn * WN + j * 32 + li;
       if (col >= p.n) continue;
-      const float bv = bias ? to_f32(bias[col]) : 0.0f;
+      float bv = 0.0f;
+      if (bias) {
+        // a bias per K segment (row-parallel shards each carry bias/ws): summed in segment order
+        const int nb_seg = p.bias_sk ? p.ksegs : 1;
+        for (int sgm = 0; sgm < nb_seg; ++sgm) bv += to_f32(bias[sgm * p.bias_sk + col]);
+      }
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int row = m0 + wm * WM + i * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+        const int row = t.m0 + wm * WM + i * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
         if (row >= p.m) continue;
         float v = p.alpha * acc[i][j][r];
         if (cin) {
@@ -245,21 +320,30 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs p) {
   }
 }
 
-template <typename T, int BM, int BN>
+template <typename T, int BM, int BN, int DEPTH, bool FAST>
 static int launch_layout(hipStream_t s, const GemmArgs& a, bool akc, bool bkc, dim3 grid) {
   if (akc && bkc)
-    hipLaunchKernelGGL((gemm_kernel<T, BM, BN, true, true>), grid, dim3(kThreads), 0, s, a);
+    hipLaunchKernelGGL((gemm_kernel<T, BM, BN, true, true, DEPTH, FAST>), grid, dim3(kThreads), 0, s, a);
   else if (akc && !bkc)
-    hipLaunchKernelGGL((gemm_kernel<T, BM, BN, true, false>), grid, dim3(kThreads), 0, s, a);
+    hipLaunchKernelGGL((gemm_kernel<T, BM, BN, true, false, DEPTH, FAST>), grid, dim3(kThreads), 0, s, a);
   else if (!akc && bkc)
-    hipLaunchKernelGGL((gemm_kernel<T, BM, BN, false, true>), grid, dim3(kThreads), 0, s, a);
+    hipLaunchKernelGGL((gemm_kernel<T, BM, BN, false, true, DEPTH, FAST>), grid, dim3(kThreads), 0, s, a);
   else
-    hipLaunchKernelGGL((gemm_kernel<T, BM, BN, false, false>), grid, dim3(kThreads), 0, s, a);
+    hipLaunchKernelGGL((gemm_kernel<T, BM, BN, false, false, DEPTH, FAST>), grid, dim3(kThreads), 0, s, a);
   RTP_LAUNCH_CHECK();
   return RTP_OK;
 }
 
 static bool mult(int64_t v, int64_t q) { return v % q == 0; }
+
+// Tile shapes, largest first.  A shape is taken when it yields enough workgroups to occupy the 256 CUs;
+// otherwise the next smaller one is tried (the 10-layer LM's per-layer problems are 1024 x 2048: 128
+// tiles of 128x128 but 256 of 128x64).
+struct TileShape {
+  int bm, bn;
+  const char* tag;
+};
+static const TileShape kShapes[3] = {{128, 128, "128x128"}, {128, 64, "128x64"}, {64, 64, "64x64"}};
 
 template <typename T>
 static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
@@ -274,77 +358,118 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   a.m = (int)d->m;
   a.n = (int)d->n;
   a.k = (int)d->k;
+  a.ksegs = (int)d->ksegs;
   a.lda = d->lda;
   a.ldb = d->ldb;
   a.ldc = d->ldc;
   a.ld_cin = d->ld_cin;
   a.ld_gate = d->ld_gate;
+  a.batch = (int)d->batch;
   a.zdiv = (int)d->zdiv;
   a.a_so = d->a_so, a.a_si = d->a_si, a.b_so = d->b_so, a.b_si = d->b_si;
   a.c_so = d->c_so, a.c_si = d->c_si, a.cin_so = d->cin_so, a.cin_si = d->cin_si;
   a.gate_so = d->gate_so, a.gate_si = d->gate_si, a.bias_so = d->bias_so, a.bias_si = d->bias_si;
+  a.a_sg = d->a_sg, a.b_sg = d->b_sg, a.c_sg = d->c_sg, a.cin_sg = d->cin_sg;
+  a.gate_sg = d->gate_sg, a.bias_sg = d->bias_sg;
+  a.a_sk = d->a_sk, a.b_sk = d->b_sk, a.bias_sk = d->bias_sk;
   a.alpha = d->alpha;
   a.flags = d->flags;
-  a.vec_a = mult((int64_t)(uintptr_t)d->a, 16) && mult(d->lda, VEC) && mult(d->a_so, VEC) && mult(d->a_si, VEC);
-  a.vec_b = mult((int64_t)(uintptr_t)d->b, 16) && mult(d->ldb, VEC) && mult(d->b_so, VEC) && mult(d->b_si, VEC);
+  a.vec_a = mult((int64_t)(uintptr_t)d->a, 16) && mult(d->lda, VEC) && mult(d->a_so, VEC) && mult(d->a_si, VEC) &&
+            mult(d->a_sg, VEC) && mult(d->a_sk, VEC);
+  a.vec_b = mult((int64_t)(uintptr_t)d->b, 16) && mult(d->ldb, VEC) && mult(d->b_so, VEC) && mult(d->b_si, VEC) &&
+            mult(d->b_sg, VEC) && mult(d->b_sk, VEC);
 
-  // Large tiles when they already fill the 256 CUs, small tiles otherwise.
-  const int64_t big_tiles = ceil_div(d->m, 128) * ceil_div(d->n, 128) * d->batch;
-  const bool big = big_tiles >= 192;
-  const int bm = big ? 128 : 64;
-  a.tiles_m = (int)ceil_div(d->m, bm);
-  a.tiles_n = (int)ceil_div(d->n, bm);
+  // Branch-free loads need whole 16-byte vectors: aligned operands and extents that are multiples of VEC
+  // along each operand's contiguous axis.  Anything else goes to the guarded small-tile kernel.
+  const bool akc = d->a_kcontig, bkc = d->b_kcontig;
+  const bool fast = a.vec_a && a.vec_b && ((akc || bkc) ? mult(d->k, VEC) : true) && (akc || mult(d->m, VEC)) &&
+                    (bkc || mult(d->n, VEC)) && d->k > 0;
+  const int64_t nz = d->batch * d->groups;
+  int shape = 2;
+  for (int i = 0; fast && i < 3; ++i) {
+    const int64_t tiles = ceil_div(d->m, kShapes[i].bm) * ceil_div(d->n, kShapes[i].bn) * nz;
+    if (tiles >= 200) {
+      shape = i;
+      break;
+    }
+  }
+  const TileShape& ts = kShapes[shape];
+  a.tiles_m = (int)ceil_div(d->m, ts.bm);
+  a.tiles_n = (int)ceil_div(d->n, ts.bn);
   const int64_t nb = (int64_t)a.tiles_m * a.tiles_n;
-  RTP_REQUIRE(nb < (1ll << 31) && d->batch < 65536, "gemm grid too large (%lld tiles, batch %lld)",
-              (long long)nb, (long long)d->batch);
-  dim3 grid((unsigned)nb, (unsigned)d->batch, 1);
-  // variant name = the kernel template instance, e.g. gemm_bf16_64x64_kc_kc
-  static const char* const names[2][2][2][2] = {
-      {{{"gemm_f32_64x64_rc_rc", "gemm_f32_64x64_rc_kc"}, {"gemm_f32_64x64_kc_rc", "gemm_f32_64x64_kc_kc"}},
-       {{"gemm_f32_128x128_rc_rc", "gemm_f32_128x128_rc_kc"}, {"gemm_f32_128x128_kc_rc", "gemm_f32_128x128_kc_kc"}}},
-      {{{"gemm_bf16_64x64_rc_rc", "gemm_bf16_64x64_rc_kc"}, {"gemm_bf16_64x64_kc_rc", "gemm_bf16_64x64_kc_kc"}},
-       {{"gemm_bf16_128x128_rc_rc", "gemm_bf16_128x128_rc_kc"},
-        {"gemm_bf16_128x128_kc_rc", "gemm_bf16_128x128_kc_kc"}}}};
-  const double mnk = (double)d->m * (double)d->n * (double)d->batch;
+  RTP_REQUIRE(nb < (1ll << 31) && nz < 65536, "gemm grid too large (%lld tiles, %lld batch*groups)", (long long)nb,
+              (long long)nz);
+  dim3 grid((unsigned)nb, (unsigned)nz, 1);
+
+  // variant name = the kernel template instance, e.g. gemm_bf16_128x64_kc_kc
+  static const char* const layout_tag[2][2] = {{"rc_rc", "rc_kc"}, {"kc_rc", "kc_kc"}};
+  static thread_local char names[2][4][2][2][40];
+  char* name = names[sizeof(T) == 2][fast ? shape : 3][akc][bkc];
+  if (!name[0])
+    snprintf(name, 40, "gemm_%s_%s_%s", sizeof(T) == 2 ? "bf16" : "f32", fast ? ts.tag : "64x64_guarded",
+             layout_tag[akc][bkc]);
+  const double mn = (double)d->m * (double)d->n * (double)nz;
+  const double kk = (double)d->k * (double)d->ksegs;
   const double out_sz = (d->flags & RTP_GEMM_OUT_F32) ? 4.0 : (double)sizeof(T);
   const double cin_sz = d->c_in ? ((d->flags & RTP_GEMM_CIN_F32) ? 4.0 : (double)sizeof(T)) : 0.0;
-  const double bytes = ((double)d->m * d->k + (double)d->n * d->k) * d->batch * sizeof(T) + mnk * (out_sz + cin_sz);
-  ProfileScope prof(s, names[sizeof(T) == 2][big][d->a_kcontig != 0][d->b_kcontig != 0], 2.0 * mnk * (double)d->k,
-                    bytes);
-  if (big) return launch_layout<T, 128, 128>(s, a, d->a_kcontig, d->b_kcontig, grid);
-  return launch_layout<T, 64, 64>(s, a, d->a_kcontig, d->b_kcontig, grid);
+  const double bytes = ((double)d->m + (double)d->n) * kk * nz * sizeof(T) + mn * (out_sz + cin_sz);
+  ProfileScope prof(s, name, 2.0 * mn * kk, bytes);
+  if (!fast) return launch_layout<T, 64, 64, 1, false>(s, a, akc, bkc, grid);
+  switch (shape) {
+    case 0:
+      return launch_layout<T, 128, 128, 2, true>(s, a, akc, bkc, grid);
+    case 1:
+      return launch_layout<T, 128, 64, 3, true>(s, a, akc, bkc, grid);
+    default:
+      return launch_layout<T, 64, 64, 3, true>(s, a, akc, bkc, grid);
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
-// Column sum (bias gradient): 64 columns per workgroup, 4 row phases, fixed-order reduction.
+// Column sums (bias gradients) in two deterministic passes: 64 columns x a block of rows per
+// workgroup into fp32 partials, then a fixed-order sum of the partials.
+constexpr int kColsumRows = 64;
+
 template <typename T>
-__global__ __launch_bounds__(kThreads) void colsum_kernel(const T* x, long m, long n, long ld, void* out,
-                                                          int out_f32, int accumulate) {
-  __shared__ float part[4][64];
+__global__ __launch_bounds__(kThreads) void colsum_partial_kernel(const T* x, long m, long n, long ld, float* part) {
+  __shared__ float red[4][64];
   const int c = threadIdx.x & 63, ph = threadIdx.x >> 6;
   const long col = (long)blockIdx.x * 64 + c;
+  const long r0 = (long)blockIdx.y * kColsumRows;
+  const long r1 = r0 + kColsumRows < m ? r0 + kColsumRows : m;
   float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
   if (col < n) {
-    long r = ph;
-    for (; r + 12 < m; r += 16) {
+    long r = r0 + ph;
+    for (; r + 12 < r1; r += 16) {
       s0 += to_f32(x[r * ld + col]);
       s1 += to_f32(x[(r + 4) * ld + col]);
       s2 += to_f32(x[(r + 8) * ld + col]);
       s3 += to_f32(x[(r + 12) * ld + col]);
     }
-    for (; r < m; r += 4) s0 += to_f32(x[r * ld + col]);
+    for (; r < r1; r += 4) s0 += to_f32(x[r * ld + col]);
   }
-  part[ph][c] = (s0 + s1) + (s2 + s3);
+  red[ph][c] = (s0 + s1) + (s2 + s3);
   __syncthreads();
-  if (ph == 0 && col < n) {
-    float v = (part[0][c] + part[1][c]) + (part[2][c] + part[3][c]);
-    if (out_f32) {
-      float* o = reinterpret_cast<float*>(out);
-      o[col] = accumulate ? o[col] + v : v;
-    } else {
-      T* o = reinterpret_cast<T*>(out);
-      o[col] = from_f32<T>(accumulate ? to_f32(o[col]) + v : v);
-    }
+  if (ph == 0 && col < n) part[(long)blockIdx.y * n + col] = (red[0][c] + red[1][c]) + (red[2][c] + red[3][c]);
+}
+
+// out index of column c: (c / seg) * seg_stride + c % seg  (bias slices of consecutive shards sit
+// seg_stride elements apart in the flat gradient buffer).
+template <typename T>
+__global__ __launch_bounds__(kThreads) void colsum_final_kernel(const float* part, long nparts, long n, void* out,
+                                                                long seg, long seg_stride, int out_f32,
+                                                                int accumulate) {
+  const long col = (long)blockIdx.x * kThreads + threadIdx.x;
+  if (col >= n) return;
+  float v = 0.0f;
+  for (long p = 0; p < nparts; ++p) v += part[p * n + col];
+  const long o = (col / seg) * seg_stride + col % seg;
+  if (out_f32) {
+    float* dst = reinterpret_cast<float*>(out);
+    dst[o] = accumulate ? dst[o] + v : v;
+  } else {
+    T* dst = reinterpret_cast<T*>(out);
+    dst[o] = from_f32<T>(accumulate ? to_f32(dst[o]) + v : v);
   }
 }
 
@@ -357,8 +482,10 @@ extern "C" int rtp_gemm(void* stream, int dtype, const rtp_gemm_desc* d) {
   RTP_REQUIRE(d->m >= 0 && d->n >= 0 && d->k >= 0, "rtp_gemm: negative extent m=%lld n=%lld k=%lld",
               (long long)d->m, (long long)d->n, (long long)d->k);
   RTP_REQUIRE(d->m < (1ll << 31) && d->n < (1ll << 31) && d->k < (1ll << 31), "rtp_gemm: extent exceeds int32");
-  RTP_REQUIRE(d->batch >= 1 && d->zdiv >= 1, "rtp_gemm: batch=%lld zdiv=%lld must be >= 1",
-              (long long)d->batch, (long long)d->zdiv);
+  RTP_REQUIRE(d->batch >= 1 && d->zdiv >= 1 && d->groups >= 1 && d->ksegs >= 1,
+              "rtp_gemm: batch=%lld zdiv=%lld groups=%lld ksegs=%lld must be >= 1", (long long)d->batch,
+              (long long)d->zdiv, (long long)d->groups, (long long)d->ksegs);
+  RTP_REQUIRE(d->k * d->ksegs < (1ll << 31), "rtp_gemm: total contraction length exceeds int32");
   RTP_REQUIRE(d->lda >= 1 && d->ldb >= 1 && d->ldc >= 1, "rtp_gemm: leading dimensions must be >= 1");
   RTP_REQUIRE(!d->c_in || d->ld_cin >= 1, "rtp_gemm: ld_cin must be >= 1 when c_in is given");
   RTP_REQUIRE(!d->gate || d->ld_gate >= 1, "rtp_gemm: ld_gate must be >= 1 when gate is given");
@@ -371,24 +498,47 @@ extern "C" int rtp_gemm(void* stream, int dtype, const rtp_gemm_desc* d) {
 
 extern "C" size_t rtp_gemm_desc_size(void) { return sizeof(rtp_gemm_desc); }
 
-extern "C" int rtp_colsum(void* stream, int dtype, const void* x, int64_t m, int64_t n, int64_t ld, void* out,
-                          int out_f32, int accumulate) {
+extern "C" size_t rtp_colsum_workspace_bytes(int64_t m, int64_t n) {
   using namespace rtp;
-  RTP_REQUIRE(x && out, "rtp_colsum: null pointer");
+  if (m <= 0 || n <= 0) return 256;
+  return (size_t)(ceil_div(m, kColsumRows) * n * 4 + 256);
+}
+
+extern "C" int rtp_colsum(void* stream, int dtype, const void* x, int64_t m, int64_t n, int64_t ld, void* out,
+                          int out_f32, int accumulate, int64_t seg, int64_t seg_stride, void* workspace,
+                          size_t workspace_bytes) {
+  using namespace rtp;
+  RTP_REQUIRE(x && out && workspace, "rtp_colsum: null pointer");
   RTP_REQUIRE(m >= 0 && n >= 0 && ld >= n, "rtp_colsum: bad shape m=%lld n=%lld ld=%lld", (long long)m,
               (long long)n, (long long)ld);
+  RTP_REQUIRE(dtype == RTP_F32 || dtype == RTP_BF16, "rtp_colsum: unknown dtype %d", dtype);
   if (n == 0) return RTP_OK;
+  if (seg <= 0) {
+    seg = n;
+    seg_stride = n;
+  }
+  RTP_REQUIRE(seg_stride >= seg, "rtp_colsum: seg_stride %lld < seg %lld", (long long)seg_stride, (long long)seg);
+  const int64_t nparts = std::max<int64_t>(1, ceil_div(m, kColsumRows));
+  RTP_REQUIRE(nparts < 65536, "rtp_colsum: too many rows");
+  if (workspace_bytes < (size_t)(nparts * n * 4))
+    return fail(RTP_ERR_WORKSPACE, "rtp_colsum: workspace %zu < required %lld", workspace_bytes,
+                (long long)(nparts * n * 4));
   hipStream_t s = (hipStream_t)stream;
-  dim3 grid((unsigned)ceil_div(n, 64));
+  float* part = (float*)workspace;
   ProfileScope prof(s, "colsum", (double)m * n, (double)m * n * (dtype == RTP_F32 ? 4 : 2));
-  if (dtype == RTP_F32)
-    hipLaunchKernelGGL(colsum_kernel<float>, grid, dim3(kThreads), 0, s, (const float*)x, (long)m, (long)n,
-                       (long)ld, out, 1, accumulate);
-  else if (dtype == RTP_BF16)
-    hipLaunchKernelGGL(colsum_kernel<bf16_t>, grid, dim3(kThreads), 0, s, (const bf16_t*)x, (long)m, (long)n,
-                       (long)ld, out, out_f32, accumulate);
-  else
-    return fail(RTP_ERR_ARG, "rtp_colsum: unknown dtype %d", dtype);
+  dim3 grid((unsigned)ceil_div(n, 64), (unsigned)nparts);
+  dim3 grid2((unsigned)ceil_div(n, kThreads));
+  if (dtype == RTP_F32) {
+    hipLaunchKernelGGL(colsum_partial_kernel<float>, grid, dim3(kThreads), 0, s, (const float*)x, (long)m, (long)n,
+                       (long)ld, part);
+    hipLaunchKernelGGL(colsum_final_kernel<float>, grid2, dim3(kThreads), 0, s, part, (long)nparts, (long)n, out,
+                       (long)seg, (long)seg_stride, 1, accumulate);
+  } else {
+    hipLaunchKernelGGL(colsum_partial_kernel<bf16_t>, grid, dim3(kThreads), 0, s, (const bf16_t*)x, (long)m, (long)n,
+                       (long)ld, part);
+    hipLaunchKernelGGL(colsum_final_kernel<bf16_t>, grid2, dim3(kThreads), 0, s, part, (long)nparts, (long)n, out,
+                       (long)seg, (long)seg_stride, out_f32, accumulate);
+  }
   RTP_LAUNCH_CHECK();
   return RTP_OK;
 }

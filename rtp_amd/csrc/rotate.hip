@@ -48,12 +48,20 @@ ProfileScope::~ProfileScope() {
 
 struct Ring {
   hipStream_t side = nullptr;
-  hipEvent_t begin = nullptr;
+  hipEvent_t join = nullptr;  // a point on the consuming stream the side stream must not run ahead of
   hipEvent_t copied[2] = {nullptr, nullptr};
   hipEvent_t consumed[2] = {nullptr, nullptr};
   bool consumed_pending[2] = {false, false};
+  bool join_recorded = false;  // `join` holds a fence that the next prefetch still has to wait for
+  bool need_join = true;       // nothing orders the side stream after the consuming stream yet
   int device = -1;
 };
+
+static bool is_capturing(hipStream_t s) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &st) != hipSuccess) return false;
+  return st == hipStreamCaptureStatusActive;
+}
 
 // 16 bytes per thread per iteration, grid-stride; the ragged head/tail (when the two pointers share
 // an alignment phase) and fully unaligned pairs go byte by byte.
@@ -141,7 +149,7 @@ extern "C" int rtp_ring_create(void** ring_out) {
   RTP_HIP_TRY(hipGetDevice(&r->device));
   // Default priority on purpose: mixed stream priorities are not used anywhere in this library.
   RTP_HIP_TRY(hipStreamCreateWithFlags(&r->side, hipStreamNonBlocking));
-  RTP_HIP_TRY(hipEventCreateWithFlags(&r->begin, hipEventDisableTiming));
+  RTP_HIP_TRY(hipEventCreateWithFlags(&r->join, hipEventDisableTiming));
   for (int i = 0; i < 2; ++i) {
     RTP_HIP_TRY(hipEventCreateWithFlags(&r->copied[i], hipEventDisableTiming));
     RTP_HIP_TRY(hipEventCreateWithFlags(&r->consumed[i], hipEventDisableTiming));
@@ -158,25 +166,41 @@ extern "C" int rtp_ring_destroy(void* ring) {
     if (r->copied[i]) (void)hipEventDestroy(r->copied[i]);
     if (r->consumed[i]) (void)hipEventDestroy(r->consumed[i]);
   }
-  if (r->begin) (void)hipEventDestroy(r->begin);
+  if (r->join) (void)hipEventDestroy(r->join);
   if (r->side) (void)hipStreamDestroy(r->side);
   delete r;
   return RTP_OK;
 }
 
-extern "C" int rtp_ring_begin(void* ring, void* main_stream) {
-  RTP_REQUIRE(ring, "rtp_ring_begin: null ring");
+extern "C" int rtp_ring_fence(void* ring, void* main_stream) {
+  RTP_REQUIRE(ring, "rtp_ring_fence: null ring");
   Ring* r = (Ring*)ring;
-  RTP_HIP_TRY(hipEventRecord(r->begin, (hipStream_t)main_stream));
-  RTP_HIP_TRY(hipStreamWaitEvent(r->side, r->begin, 0));
+  RTP_HIP_TRY(hipEventRecord(r->join, (hipStream_t)main_stream));
+  r->join_recorded = true;
+  r->need_join = true;
+  // everything that consumed a slot so far is queued before the fence
   r->consumed_pending[0] = r->consumed_pending[1] = false;
   return RTP_OK;
 }
 
-extern "C" int rtp_ring_prefetch(void* ring, int slot, void* dst, const void* src, size_t bytes) {
+extern "C" int rtp_ring_prefetch(void* ring, void* main_stream, int slot, void* dst, const void* src,
+                                 size_t bytes) {
   RTP_REQUIRE(ring, "rtp_ring_prefetch: null ring");
   RTP_REQUIRE(slot == 0 || slot == 1, "rtp_ring_prefetch: slot %d not in {0,1}", slot);
   Ring* r = (Ring*)ring;
+  hipStream_t main = (hipStream_t)main_stream;
+  // While `main` is being captured into a graph the side stream has to be forked from it, or the copy
+  // would run now instead of being recorded.
+  if (is_capturing(main) && !is_capturing(r->side)) r->need_join = true, r->join_recorded = false;
+  if (r->need_join) {
+    if (!r->join_recorded) {
+      RTP_HIP_TRY(hipEventRecord(r->join, main));
+      r->consumed_pending[0] = r->consumed_pending[1] = false;
+    }
+    RTP_HIP_TRY(hipStreamWaitEvent(r->side, r->join, 0));
+    r->need_join = false;
+    r->join_recorded = false;
+  }
   if (r->consumed_pending[slot]) {
     RTP_HIP_TRY(hipStreamWaitEvent(r->side, r->consumed[slot], 0));
     r->consumed_pending[slot] = false;

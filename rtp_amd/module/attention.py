@@ -21,6 +21,7 @@ from torch.nn.parameter import Parameter
 
 from .. import ops
 from ..ring import Rotation, ring_order
+from . import shard_ops as S
 from .collectives import RotatedLayer
 from .utils import (affine_weight, affine_weight_attention, as_rows, attention_block_index,
                     divide_and_check_no_remainder)
@@ -87,123 +88,129 @@ class SubParallelMultiheadAttention(nn.Module):
                 self.out_proj.bias.data.div_(self.world_size)
 
 
-def _bmm(dtype, *, a, a_off, lda, a_kc, a_s, b, b_off, ldb, b_kc, b_s, c, c_off, ldc, c_s, m, n, k, batch, zdiv,
-         out_f32=False):
+def _bmm(dtype, *, a, a_off, lda, a_kc, a_s, a_sg, b, b_off, ldb, b_kc, b_s, b_sg, c, c_off, ldc, c_s, c_sg, m, n, k,
+         batch, zdiv, groups, out_f32=False):
     esz = a.element_size()
     csz = 4 if out_f32 else esz
     ops.gemm_raw(dtype, a=a.data_ptr() + a_off * esz, b=b.data_ptr() + b_off * esz, c_out=c.data_ptr() + c_off * csz,
                  m=m, n=n, k=k, lda=lda, ldb=ldb, ldc=ldc, a_kcontig=a_kc, b_kcontig=b_kc, batch=batch, zdiv=zdiv,
-                 a_s=a_s, b_s=b_s, c_s=c_s, out_f32=out_f32)
+                 a_s=a_s, b_s=b_s, c_s=c_s, out_f32=out_f32, groups=groups, a_sg=a_sg, b_sg=b_sg, c_sg=c_sg)
 
 
 class _AttentionFn(torch.autograd.Function):
+    """Buffers hold all head groups side by side: qkv [L*N, ws*3E_s] (group g at column block g, inside it
+    Q | K | V of that group), p [ws*N*h_s, L, L], o [L*N, E] (= the unsharded head order).  A (group,
+    batch, head) triple is addressed by strides inside the batched GEMM, so nothing is re-laid out."""
+
     @staticmethod
     def forward(ctx, x, anchor, layer, mask, causal, want_weights):
         store = layer._store
         L, N, E = x.shape
         ws, h_s, d, e_s = layer.world_size, layer.num_heads_per_partition, layer.head_dim, layer.embed_dim_per_partition
-        dt = x.dtype
+        dt, dev = x.dtype, x.device
         x2 = as_rows(x, E)
         rows, Z = L * N, N * h_s
         scale = 1.0 / math.sqrt(d)
-        out = torch.empty(rows, E, dtype=dt, device=x.device)
-        acc = ops.ShardSum(out, ws)
+        off = store.offsets
+        b_in_off, w_o_off, b_o_off = (off[1], off[2], off[3]) if layer.has_bias else (None, off[1], None)
+        qkv = torch.empty(rows, ws * 3 * e_s, dtype=dt, device=dev)
+        p = torch.empty(ws * Z, L, L, dtype=dt, device=dev)
+        o = torch.empty(rows, E, dtype=dt, device=dev)
+        out = torch.empty(rows, E, dtype=dt, device=dev)
+        ldq = N * ws * 3 * e_s
         order = ring_order(layer.rank, ws)
         rot = Rotation(store.home, order)
-        saved = {}
+        acc = ops.ShardSum(out, sum(len(w) for w in rot.windows))
+        i = 0
+        for j in range(rot.steps):
+            for flat, first, cnt in rot.acquire(j):
+                S.col_fwd(x2, flat, 0, 3 * e_s, E, b_in_off, qkv, first * 3 * e_s)
+                scores = torch.empty(cnt * Z, L, L, dtype=torch.float32, device=dev)
+                q0 = first * 3 * e_s
+                _bmm(dt, a=qkv, a_off=q0, lda=ldq, a_kc=True, a_s=(ws * 3 * e_s, d), a_sg=3 * e_s, b=qkv,
+                     b_off=q0 + e_s, ldb=ldq, b_kc=True, b_s=(ws * 3 * e_s, d), b_sg=3 * e_s, c=scores, c_off=0, ldc=L,
+                     c_s=(h_s * L * L, L * L), c_sg=Z * L * L, m=L, n=L, k=d, batch=Z, zdiv=h_s, groups=cnt,
+                     out_f32=True)
+                p_run = p[first * Z:(first + cnt) * Z]
+                ops.softmax_fwd(scores, p_run, mask=mask, causal=causal, scale=scale)
+                del scores
+                _bmm(dt, a=p, a_off=first * Z * L * L, lda=L, a_kc=True, a_s=(h_s * L * L, L * L), a_sg=Z * L * L,
+                     b=qkv, b_off=q0 + 2 * e_s, ldb=ldq, b_kc=False, b_s=(ws * 3 * e_s, d), b_sg=3 * e_s, c=o,
+                     c_off=first * e_s, ldc=N * E, c_s=(E, d), c_sg=e_s, m=L, n=d, k=L, batch=Z, zdiv=h_s, groups=cnt)
+                c_out, c_in = acc.target(i)
+                S.row_fwd(o, flat, w_o_off, E, e_s, b_o_off, c_out, first * e_s, c_in=c_in)
+                i += 1
+            rot.release(j)
         weights = None
-        for i, idx in enumerate(order):
-            views = store.views(rot.acquire(i))
-            w_in = views[0]
-            b_in, w_o, b_o = (views[1], views[2], views[3]) if layer.has_bias else (None, views[1], None)
-            qkv = torch.empty(rows, 3 * e_s, dtype=dt, device=x.device)
-            ops.linear_fwd(x2, w_in, qkv, bias=b_in)
-            scores = torch.empty(Z, L, L, dtype=torch.float32, device=x.device)
-            ld = N * 3 * e_s
-            _bmm(dt, a=qkv, a_off=0, lda=ld, a_kc=True, a_s=(3 * e_s, d), b=qkv, b_off=e_s, ldb=ld, b_kc=True,
-                 b_s=(3 * e_s, d), c=scores, c_off=0, ldc=L, c_s=(h_s * L * L, L * L), m=L, n=L, k=d, batch=Z,
-                 zdiv=h_s, out_f32=True)
-            p = torch.empty(Z, L, L, dtype=dt, device=x.device)
-            ops.softmax_fwd(scores, p, mask=mask, causal=causal, scale=scale)
-            del scores
-            o = torch.empty(rows, e_s, dtype=dt, device=x.device)
-            _bmm(dt, a=p, a_off=0, lda=L, a_kc=True, a_s=(h_s * L * L, L * L), b=qkv, b_off=2 * e_s, ldb=ld,
-                 b_kc=False, b_s=(3 * e_s, d), c=o, c_off=0, ldc=N * e_s, c_s=(e_s, d), m=L, n=d, k=L, batch=Z,
-                 zdiv=h_s)
-            c_out, c_in = acc.target(i)
-            ops.linear_fwd(o, w_o, c_out, c_in=c_in, bias=b_o)
-            rot.release(i)
-            saved[idx] = (qkv, p, o)
-            if want_weights and i == ws - 1:
-                weights = p.view(N, h_s, L, L)
+        if want_weights:
+            last = order[-1]
+            weights = p[last * Z:(last + 1) * Z].view(N, h_s, L, L)
         ctx.layer = layer
         ctx.dims = (L, N, E)
-        ctx.saved = saved
-        ctx.save_for_backward(x2)
+        ctx.save_for_backward(x2, qkv, p, o)
         ctx.mark_non_differentiable(*([weights] if weights is not None else []))
-        y = out.view(L, N, E)
-        return (y, weights) if weights is not None else (y, None)
+        return out.view(L, N, E), weights
 
     @staticmethod
     def backward(ctx, dout, _dweights=None):
         layer = ctx.layer
-        (x2,) = ctx.saved_tensors
+        x2, qkv, p, o = ctx.saved_tensors
         store = layer._store
         L, N, E = ctx.dims
         ws, h_s, d, e_s = layer.world_size, layer.num_heads_per_partition, layer.head_dim, layer.embed_dim_per_partition
-        dt = x2.dtype
+        dt, dev = x2.dtype, x2.device
         rows, Z = L * N, N * h_s
         scale = 1.0 / math.sqrt(d)
+        off = store.offsets
+        b_in_off, w_o_off, b_o_off = (off[1], off[2], off[3]) if layer.has_bias else (None, off[1], None)
         dout2 = as_rows(dout, E)
         need_dx = ctx.needs_input_grad[0]
         dx = torch.empty_like(x2) if need_dx else None
-        acc = ops.ShardSum(dx, ws) if need_dx else None
+        do = torch.empty(rows, E, dtype=dt, device=dev)
+        dqkv = torch.empty(rows, ws * 3 * e_s, dtype=dt, device=dev)
+        ldq = N * ws * 3 * e_s
         order = ring_order(layer.rank, ws, reverse=True)
         rot = Rotation(store.home, order)
-        ld = N * 3 * e_s
-        for i, idx in enumerate(order):
-            views = store.views(rot.acquire(i))
-            w_in = views[0]
-            w_o = views[2] if layer.has_bias else views[1]
-            qkv, p, o = ctx.saved.pop(idx)
-            grads, accumulate = store.grad_views(idx)
+        acc = ops.ShardSum(dx, sum(len(w) for w in rot.windows)) if need_dx else None
+        i = 0
+        for j in range(rot.steps):
+            for flat, first, cnt in rot.acquire(j):
+                q0 = first * 3 * e_s
+                # out-projection: dO_g = dOut W_o,g
+                S.row_dgrad(dout2, flat, w_o_off, E, e_s, do, first * e_s)
+                # attention core, all (group, batch, head) triples of the run in one launch each
+                dp = torch.empty(cnt * Z, L, L, dtype=torch.float32, device=dev)
+                _bmm(dt, a=do, a_off=first * e_s, lda=N * E, a_kc=True, a_s=(E, d), a_sg=e_s, b=qkv, b_off=q0 + 2 * e_s,
+                     ldb=ldq, b_kc=True, b_s=(ws * 3 * e_s, d), b_sg=3 * e_s, c=dp, c_off=0, ldc=L,
+                     c_s=(h_s * L * L, L * L), c_sg=Z * L * L, m=L, n=L, k=d, batch=Z, zdiv=h_s, groups=cnt, out_f32=True)
+                p_off = first * Z * L * L
+                # dV = P^T dO
+                _bmm(dt, a=p, a_off=p_off, lda=L, a_kc=False, a_s=(h_s * L * L, L * L), a_sg=Z * L * L, b=do,
+                     b_off=first * e_s, ldb=N * E, b_kc=False, b_s=(E, d), b_sg=e_s, c=dqkv, c_off=q0 + 2 * e_s, ldc=ldq,
+                     c_s=(ws * 3 * e_s, d), c_sg=3 * e_s, m=L, n=d, k=L, batch=Z, zdiv=h_s, groups=cnt)
+                ds = torch.empty(cnt * Z, L, L, dtype=dt, device=dev)
+                ops.softmax_bwd(p[first * Z:(first + cnt) * Z], dp, ds, scale)
+                del dp
+                # dQ = dS K
+                _bmm(dt, a=ds, a_off=0, lda=L, a_kc=True, a_s=(h_s * L * L, L * L), a_sg=Z * L * L, b=qkv,
+                     b_off=q0 + e_s, ldb=ldq, b_kc=False, b_s=(ws * 3 * e_s, d), b_sg=3 * e_s, c=dqkv, c_off=q0, ldc=ldq,
+                     c_s=(ws * 3 * e_s, d), c_sg=3 * e_s, m=L, n=d, k=L, batch=Z, zdiv=h_s, groups=cnt)
+                # dK = dS^T Q
+                _bmm(dt, a=ds, a_off=0, lda=L, a_kc=False, a_s=(h_s * L * L, L * L), a_sg=Z * L * L, b=qkv, b_off=q0,
+                     ldb=ldq, b_kc=False, b_s=(ws * 3 * e_s, d), b_sg=3 * e_s, c=dqkv, c_off=q0 + e_s, ldc=ldq,
+                     c_s=(ws * 3 * e_s, d), c_sg=3 * e_s, m=L, n=d, k=L, batch=Z, zdiv=h_s, groups=cnt)
+                # in-projection input gradient: dX += sum_g dQKV_g W_in,g
+                if need_dx:
+                    c_out, c_in = acc.target(i)
+                    S.col_dgrad(dqkv, flat, 0, 3 * e_s, E, c_out, q0, c_in=c_in)
+                i += 1
+            rot.release(j)
+        for first, cnt, accumulate in store.grad_runs(order):
+            S.row_wgrad(dout2, o, store.grads, first, w_o_off, E, e_s, first * e_s, cnt, accumulate)
+            S.col_wgrad(dqkv, x2, store.grads, first, 0, 3 * e_s, E, first * 3 * e_s, cnt, accumulate)
             if layer.has_bias:
-                g_w_in, g_b_in, g_w_o, g_b_o = grads
-            else:
-                (g_w_in, g_w_o), g_b_in, g_b_o = grads, None, None
-            # out-projection
-            do = torch.empty(rows, e_s, dtype=dt, device=x2.device)
-            ops.linear_dgrad(dout2, w_o, do)
-            ops.linear_wgrad(dout2, o, g_w_o, c_in=g_w_o if accumulate else None)
-            if g_b_o is not None:
-                ops.colsum(dout2, g_b_o, accumulate=accumulate)
-            # attention core
-            dqkv = torch.empty(rows, 3 * e_s, dtype=dt, device=x2.device)
-            dp = torch.empty(Z, L, L, dtype=torch.float32, device=x2.device)
-            _bmm(dt, a=do, a_off=0, lda=N * e_s, a_kc=True, a_s=(e_s, d), b=qkv, b_off=2 * e_s, ldb=ld, b_kc=True,
-                 b_s=(3 * e_s, d), c=dp, c_off=0, ldc=L, c_s=(h_s * L * L, L * L), m=L, n=L, k=d, batch=Z, zdiv=h_s,
-                 out_f32=True)
-            # dV = P^T dO
-            _bmm(dt, a=p, a_off=0, lda=L, a_kc=False, a_s=(h_s * L * L, L * L), b=do, b_off=0, ldb=N * e_s,
-                 b_kc=False, b_s=(e_s, d), c=dqkv, c_off=2 * e_s, ldc=ld, c_s=(3 * e_s, d), m=L, n=d, k=L, batch=Z,
-                 zdiv=h_s)
-            ds = torch.empty(Z, L, L, dtype=dt, device=x2.device)
-            ops.softmax_bwd(p, dp, ds, scale)
-            del dp
-            # dQ = dS K
-            _bmm(dt, a=ds, a_off=0, lda=L, a_kc=True, a_s=(h_s * L * L, L * L), b=qkv, b_off=e_s, ldb=ld, b_kc=False,
-                 b_s=(3 * e_s, d), c=dqkv, c_off=0, ldc=ld, c_s=(3 * e_s, d), m=L, n=d, k=L, batch=Z, zdiv=h_s)
-            # dK = dS^T Q
-            _bmm(dt, a=ds, a_off=0, lda=L, a_kc=False, a_s=(h_s * L * L, L * L), b=qkv, b_off=0, ldb=ld, b_kc=False,
-                 b_s=(3 * e_s, d), c=dqkv, c_off=e_s, ldc=ld, c_s=(3 * e_s, d), m=L, n=d, k=L, batch=Z, zdiv=h_s)
-            # in-projection
-            if need_dx:
-                c_out, c_in = acc.target(i)
-                ops.linear_dgrad(dqkv, w_in, c_out, c_in=c_in)
-            rot.release(i)
-            ops.linear_wgrad(dqkv, x2, g_w_in, c_in=g_w_in if accumulate else None)
-            if g_b_in is not None:
-                ops.colsum(dqkv, g_b_in, accumulate=accumulate)
+                S.row_bgrad(dout2, store.grads, first, b_o_off, E, cnt, accumulate)
+                S.col_bgrad(dqkv, store.grads, first, b_in_off, 3 * e_s, first * 3 * e_s, cnt, accumulate)
         return (dx.view(L, N, E) if need_dx else None), None, None, None, None, None
 
 

@@ -75,6 +75,7 @@ class ShardStore:
                 raise ValueError("all shards of a layer must have identical parameter shapes")
         self.home: Optional[torch.Tensor] = None
         self.grads: Optional[torch.Tensor] = None
+        self._overwrite = set()
         self.pack()
 
     # -- storage ---------------------------------------------------------------------------------
@@ -96,6 +97,10 @@ class ShardStore:
                     home[s, off:off + n].copy_(p.data.reshape(-1))
         self.home = home
         self.grads = None
+        self._overwrite.clear()
+        if home.is_cuda:
+            from .. import ring
+            ring.fence(home.device)
         for s in range(self.world_size):
             self.modules[s]._full_param = home[s]
             self.modules[s]._full_grad = None
@@ -119,6 +124,11 @@ class ShardStore:
             for m in self.modules:
                 for p in m.parameters():
                     p.grad = None
+        if s in self._overwrite:
+            # zeroed by mark_overwrite(): the views are still attached, their contents are to be replaced
+            self._overwrite.discard(s)
+            if all(p.grad is not None for p in self.params(s)):
+                return self.views(self.grads[s]), False
         params = self.params(s)
         views = self.views(self.grads[s])
         fresh = any(p.grad is None for p in params)
@@ -133,6 +143,25 @@ class ShardStore:
                 v.copy_(p.grad)
                 p.grad = v
         return views, True
+
+    def mark_overwrite(self) -> None:
+        """Cheap zero_grad for a training loop: keep the .grad views attached and let the next backward
+        overwrite every shard's gradient instead of accumulating into it."""
+        if self.grads is not None:
+            self._overwrite = set(range(self.world_size))
+
+    def grad_runs(self, order: Sequence[int]):
+        """Attach gradient storage to every shard in `order` and return maximal runs (first, count,
+        accumulate) of consecutive shards that share the same accumulate flag, so that a grouped kernel can
+        write a whole run of gradient rows in one launch."""
+        flags = {s: self.grad_views(s)[1] for s in order}
+        ids = sorted(flags)
+        runs, start = [], ids[0]
+        for a, b in zip(ids, ids[1:] + [None]):
+            if b is None or b != a + 1 or flags[b] != flags[a]:
+                runs.append((start, a - start + 1, flags[a]))
+                start = b
+        return runs
 
     def weight_bytes(self) -> int:
         return self.world_size * self.numel * self.home.element_size()

@@ -47,12 +47,13 @@ class _EmbeddingFn(torch.autograd.Function):
         d_s, ws = layer.embedding_dim_per_partition, layer.world_size
         flat_ids = ids.reshape(-1).contiguous()
         out = torch.empty(flat_ids.numel(), layer.embedding_dim, dtype=store.home.dtype, device=store.home.device)
-        order = ring_order(layer.rank, ws)
-        rot = Rotation(store.home, order)
-        for i, idx in enumerate(order):
-            table = store.views(rot.acquire(i))[0]
-            ops.embedding_gather(table, flat_ids, out[:, idx * d_s:(idx + 1) * d_s])
-            rot.release(i)
+        rot = Rotation(store.home, ring_order(layer.rank, ws))
+        for j in range(rot.steps):
+            for flat, first, cnt in rot.acquire(j):
+                table = flat[0].view(layer.num_embeddings, d_s)
+                ops.embedding_gather(table, flat_ids, out[:, first * d_s:(first + 1) * d_s], groups=cnt,
+                                     table_sg=store.numel, out_sg=d_s)
+            rot.release(j)
         ctx.layer = layer
         ctx.save_for_backward(flat_ids)
         return out.view(*ids.shape, layer.embedding_dim)

@@ -18,6 +18,7 @@ import torch.nn.init as init
 
 from .. import ops
 from ..ring import Rotation, ring_order
+from . import shard_ops as S
 from .collectives import RotatedLayer, resolve_world
 from .utils import affine_weight, as_rows, divide_and_check_no_remainder
 
@@ -70,12 +71,12 @@ class _ColumnLinearFn(torch.autograd.Function):
         n_s, k, ws = layer.output_size_per_partition, layer.in_features, layer.world_size
         x2 = as_rows(x, k)
         y = torch.empty(x2.shape[0], layer.out_features, dtype=x2.dtype, device=x2.device)
-        order = ring_order(layer.rank, ws)
-        rot = Rotation(store.home, order)
-        for i, idx in enumerate(order):
-            views = store.views(rot.acquire(i))
-            ops.linear_fwd(x2, views[0], y[:, idx * n_s:(idx + 1) * n_s], bias=views[1] if layer.has_bias else None)
-            rot.release(i)
+        b_off = n_s * k if layer.has_bias else None
+        rot = Rotation(store.home, ring_order(layer.rank, ws))
+        for j in range(rot.steps):
+            for flat, first, cnt in rot.acquire(j):
+                S.col_fwd(x2, flat, 0, n_s, k, b_off, y, first * n_s)
+            rot.release(j)
         ctx.layer = layer
         ctx.x_shape = x.shape
         ctx.save_for_backward(x2)
@@ -86,24 +87,26 @@ class _ColumnLinearFn(torch.autograd.Function):
         layer = ctx.layer
         (x2,) = ctx.saved_tensors
         store = layer._store
-        n_s, ws = layer.output_size_per_partition, layer.world_size
+        n_s, k, ws = layer.output_size_per_partition, layer.in_features, layer.world_size
         dy2 = as_rows(dy, layer.out_features)
         need_dx = ctx.needs_input_grad[0]
-        dx = torch.empty_like(x2) if need_dx else None
-        acc = ops.ShardSum(dx, ws) if need_dx else None
         order = ring_order(layer.rank, ws, reverse=True)
-        rot = Rotation(store.home, order) if need_dx else None
-        for i, idx in enumerate(order):
-            dy_s = dy2[:, idx * n_s:(idx + 1) * n_s]
-            if need_dx:
-                w = store.views(rot.acquire(i))[0]
-                c_out, c_in = acc.target(i)
-                ops.linear_dgrad(dy_s, w, c_out, c_in=c_in)
-                rot.release(i)
-            grads, accumulate = store.grad_views(idx)
-            ops.linear_wgrad(dy_s, x2, grads[0], c_in=grads[0] if accumulate else None)
+        dx = None
+        if need_dx:
+            dx = torch.empty_like(x2)
+            rot = Rotation(store.home, order)
+            acc = ops.ShardSum(dx, sum(len(w) for w in rot.windows))
+            i = 0
+            for j in range(rot.steps):
+                for flat, first, cnt in rot.acquire(j):
+                    c_out, c_in = acc.target(i)
+                    S.col_dgrad(dy2, flat, 0, n_s, k, c_out, first * n_s, c_in=c_in)
+                    i += 1
+                rot.release(j)
+        for first, cnt, accumulate in store.grad_runs(order):
+            S.col_wgrad(dy2, x2, store.grads, first, 0, n_s, k, first * n_s, cnt, accumulate)
             if layer.has_bias:
-                ops.colsum(dy_s, grads[1], accumulate=accumulate)
+                S.col_bgrad(dy2, store.grads, first, n_s * k, n_s, first * n_s, cnt, accumulate)
         return (dx.view(ctx.x_shape) if need_dx else None), None, None
 
 
@@ -111,45 +114,45 @@ class _RowLinearFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, anchor, layer):
         store = layer._store
-        k_s, ws = layer.input_size_per_partition, layer.world_size
+        k_s, n, ws = layer.input_size_per_partition, layer.out_features, layer.world_size
         x2 = as_rows(x, layer.in_features)
-        y = torch.empty(x2.shape[0], layer.out_features, dtype=x2.dtype, device=x2.device)
-        acc = ops.ShardSum(y, ws)
-        order = ring_order(layer.rank, ws)
-        rot = Rotation(store.home, order)
-        for i, idx in enumerate(order):
-            views = store.views(rot.acquire(i))
-            c_out, c_in = acc.target(i)
-            ops.linear_fwd(x2[:, idx * k_s:(idx + 1) * k_s], views[0], c_out, c_in=c_in,
-                           bias=views[1] if layer.has_bias else None)
-            rot.release(i)
+        y = torch.empty(x2.shape[0], n, dtype=x2.dtype, device=x2.device)
+        b_off = n * k_s if layer.has_bias else None
+        rot = Rotation(store.home, ring_order(layer.rank, ws))
+        acc = ops.ShardSum(y, sum(len(w) for w in rot.windows))
+        i = 0
+        for j in range(rot.steps):
+            for flat, first, cnt in rot.acquire(j):
+                c_out, c_in = acc.target(i)
+                S.row_fwd(x2, flat, 0, n, k_s, b_off, c_out, first * k_s, c_in=c_in)
+                i += 1
+            rot.release(j)
         ctx.layer = layer
         ctx.x_shape = x.shape
         ctx.save_for_backward(x2)
-        return y.view(*x.shape[:-1], layer.out_features)
+        return y.view(*x.shape[:-1], n)
 
     @staticmethod
     def backward(ctx, dy):
         layer = ctx.layer
         (x2,) = ctx.saved_tensors
         store = layer._store
-        k_s, ws = layer.input_size_per_partition, layer.world_size
-        dy2 = as_rows(dy, layer.out_features)
+        k_s, n, ws = layer.input_size_per_partition, layer.out_features, layer.world_size
+        dy2 = as_rows(dy, n)
         need_dx = ctx.needs_input_grad[0]
-        dx = torch.empty_like(x2) if need_dx else None
         order = ring_order(layer.rank, ws, reverse=True)
-        rot = Rotation(store.home, order) if need_dx else None
-        for i, idx in enumerate(order):
-            x_s = x2[:, idx * k_s:(idx + 1) * k_s]
-            if need_dx:
-                w = store.views(rot.acquire(i))[0]
-                ops.linear_dgrad(dy2, w, dx[:, idx * k_s:(idx + 1) * k_s])
-                rot.release(i)
-            grads, accumulate = store.grad_views(idx)
-            ops.linear_wgrad(dy2, x_s, grads[0], c_in=grads[0] if accumulate else None)
+        dx = None
+        if need_dx:
+            dx = torch.empty_like(x2)
+            rot = Rotation(store.home, order)
+            for j in range(rot.steps):
+                for flat, first, cnt in rot.acquire(j):
+                    S.row_dgrad(dy2, flat, 0, n, k_s, dx, first * k_s)
+                rot.release(j)
+        for first, cnt, accumulate in store.grad_runs(order):
+            S.row_wgrad(dy2, x2, store.grads, first, 0, n, k_s, first * k_s, cnt, accumulate)
             if layer.has_bias:
-                # every shard's bias (= b/ws) receives the full column sum (tests/test_linear.py:181-186)
-                ops.colsum(dy2, grads[1], accumulate=accumulate)
+                S.row_bgrad(dy2, store.grads, first, n * k_s, n, cnt, accumulate)
         return (dx.view(ctx.x_shape) if need_dx else None), None, None
 
 

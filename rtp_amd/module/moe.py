@@ -58,62 +58,93 @@ class _CombineFn(torch.autograd.Function):
 
 
 class _ExpertsFn(torch.autograd.Function):
-    """y[e*C:(e+1)*C] = linear2(relu(linear1(x[e*C:(e+1)*C]))) with expert shards rotated."""
+    """y[e*C:(e+1)*C] = linear2(relu(linear1(x[e*C:(e+1)*C]))) for every expert e, expert shards rotated.
+    The experts of a staged run are one group each of a grouped GEMM: group g reads its own capacity slab."""
+
+    @staticmethod
+    def _geom(layer, x):
+        store = layer._store
+        n_local = layer.num_local_experts
+        c_rows = x.shape[0] // (layer.world_size * n_local)
+        m_dim = x.shape[1]
+        f_dim = store.shapes[0][0]
+        return store, n_local, c_rows, m_dim, f_dim
 
     @staticmethod
     def forward(ctx, x, anchor, layer):
-        store = layer._store
-        ws, n_local = layer.world_size, layer.num_local_experts
-        rows_per_expert = x.shape[0] // (ws * n_local)
+        store, n_local, c_rows, m_dim, f_dim = _ExpertsFn._geom(layer, x)
+        es = x.element_size()
+        h = torch.empty(x.shape[0], f_dim, dtype=x.dtype, device=x.device)
         y = torch.empty_like(x)
-        hidden = []
-        order = ring_order(layer.rank, ws)
-        rot = Rotation(store.home, order)
-        for i, idx in enumerate(order):
-            views = store.views(rot.acquire(i))
-            for j in range(n_local):
-                w1, b1, w2, b2 = views[4 * j:4 * j + 4]
-                r0 = (idx * n_local + j) * rows_per_expert
-                chunk = x[r0:r0 + rows_per_expert]
-                h = torch.empty(rows_per_expert, w1.shape[0], dtype=x.dtype, device=x.device)
-                ops.linear_fwd(chunk, w1, h, bias=b1, relu=True)
-                ops.linear_fwd(h, w2, y[r0:r0 + rows_per_expert], bias=b2)
-                hidden.append((idx, j, h))
-            rot.release(i)
+        rot = Rotation(store.home, ring_order(layer.rank, layer.world_size))
+        for j in range(rot.steps):
+            for flat, first, cnt in rot.acquire(j):
+                for le in range(n_local):
+                    w1, b1, w2, b2 = store.offsets[4 * le:4 * le + 4]
+                    r0 = (first * n_local + le) * c_rows
+                    common = dict(groups=cnt, b_sg=store.numel, bias_sg=store.numel, a_kcontig=True, b_kcontig=True)
+                    ops.gemm_raw(x.dtype, a=x.data_ptr() + r0 * m_dim * es, b=flat.data_ptr() + w1 * es,
+                                 bias=flat.data_ptr() + b1 * es, c_out=h.data_ptr() + r0 * f_dim * es, m=c_rows,
+                                 n=f_dim, k=m_dim, lda=m_dim, ldb=m_dim, ldc=f_dim, relu=True,
+                                 a_sg=n_local * c_rows * m_dim, c_sg=n_local * c_rows * f_dim, **common)
+                    ops.gemm_raw(x.dtype, a=h.data_ptr() + r0 * f_dim * es, b=flat.data_ptr() + w2 * es,
+                                 bias=flat.data_ptr() + b2 * es, c_out=y.data_ptr() + r0 * m_dim * es, m=c_rows,
+                                 n=m_dim, k=f_dim, lda=f_dim, ldb=f_dim, ldc=m_dim,
+                                 a_sg=n_local * c_rows * f_dim, c_sg=n_local * c_rows * m_dim, **common)
+            rot.release(j)
         ctx.layer = layer
-        ctx.hidden = {(idx, j): h for idx, j, h in hidden}
-        ctx.save_for_backward(x)
+        ctx.save_for_backward(x, h)
         return y
 
     @staticmethod
     def backward(ctx, dy):
         layer = ctx.layer
-        (x,) = ctx.saved_tensors
-        store = layer._store
-        ws, n_local = layer.world_size, layer.num_local_experts
-        rows_per_expert = x.shape[0] // (ws * n_local)
-        dy = dy if dy.stride(1) == 1 else dy.contiguous()
+        x, h = ctx.saved_tensors
+        store, n_local, c_rows, m_dim, f_dim = _ExpertsFn._geom(layer, x)
+        es = x.element_size()
+        dy = dy.contiguous()
+        dh = torch.empty_like(h)
         dx = torch.empty_like(x)
-        order = ring_order(layer.rank, ws, reverse=True)
+        order = ring_order(layer.rank, layer.world_size, reverse=True)
         rot = Rotation(store.home, order)
-        for i, idx in enumerate(order):
-            views = store.views(rot.acquire(i))
-            grads, accumulate = store.grad_views(idx)
-            for j in range(n_local):
-                w1, b1, w2, b2 = views[4 * j:4 * j + 4]
-                g_w1, g_b1, g_w2, g_b2 = grads[4 * j:4 * j + 4]
-                r0 = (idx * n_local + j) * rows_per_expert
-                h = ctx.hidden.pop((idx, j))
-                dy_e = dy[r0:r0 + rows_per_expert]
-                dh = torch.empty_like(h)
-                ops.linear_dgrad(dy_e, w2, dh, gate=h)
-                ops.linear_dgrad(dh, w1, dx[r0:r0 + rows_per_expert])
-                c = (lambda g: g if accumulate else None)
-                ops.linear_wgrad(dy_e, h, g_w2, c_in=c(g_w2))
-                ops.colsum(dy_e, g_b2, accumulate=accumulate)
-                ops.linear_wgrad(dh, x[r0:r0 + rows_per_expert], g_w1, c_in=c(g_w1))
-                ops.colsum(dh, g_b1, accumulate=accumulate)
-            rot.release(i)
+        for j in range(rot.steps):
+            for flat, first, cnt in rot.acquire(j):
+                for le in range(n_local):
+                    w1, _, w2, _ = store.offsets[4 * le:4 * le + 4]
+                    r0 = (first * n_local + le) * c_rows
+                    common = dict(groups=cnt, b_sg=store.numel, a_kcontig=True, b_kcontig=False)
+                    # dH = (dY W2) masked by H > 0 ; dX = dH W1
+                    ops.gemm_raw(x.dtype, a=dy.data_ptr() + r0 * m_dim * es, b=flat.data_ptr() + w2 * es,
+                                 c_out=dh.data_ptr() + r0 * f_dim * es, gate=h.data_ptr() + r0 * f_dim * es,
+                                 ld_gate=f_dim, gate_sg=n_local * c_rows * f_dim, m=c_rows, n=f_dim, k=m_dim, lda=m_dim,
+                                 ldb=f_dim, ldc=f_dim, a_sg=n_local * c_rows * m_dim, c_sg=n_local * c_rows * f_dim,
+                                 **common)
+                    ops.gemm_raw(x.dtype, a=dh.data_ptr() + r0 * f_dim * es, b=flat.data_ptr() + w1 * es,
+                                 c_out=dx.data_ptr() + r0 * m_dim * es, m=c_rows, n=m_dim, k=f_dim, lda=f_dim,
+                                 ldb=m_dim, ldc=m_dim, a_sg=n_local * c_rows * f_dim, c_sg=n_local * c_rows * m_dim,
+                                 **common)
+            rot.release(j)
+        runs = store.grad_runs(order)  # attaches (and on first use allocates) the gradient storage
+        g = store.grads
+        for first, cnt, accumulate in runs:
+            for le in range(n_local):
+                w1, b1, w2, b2 = store.offsets[4 * le:4 * le + 4]
+                r0 = (first * n_local + le) * c_rows
+                base = g.data_ptr() + first * store.numel * es
+                common = dict(groups=cnt, c_sg=store.numel, cin_sg=store.numel, a_kcontig=False, b_kcontig=False)
+                # dW2 = dY^T H ; dW1 = dH^T X  (contraction over the expert's capacity rows)
+                c2 = base + w2 * es
+                ops.gemm_raw(x.dtype, a=dy.data_ptr() + r0 * m_dim * es, b=h.data_ptr() + r0 * f_dim * es, c_out=c2,
+                             c_in=c2 if accumulate else None, ld_cin=f_dim, m=m_dim, n=f_dim, k=c_rows, lda=m_dim,
+                             ldb=f_dim, ldc=f_dim, a_sg=n_local * c_rows * m_dim, b_sg=n_local * c_rows * f_dim, **common)
+                c1 = base + w1 * es
+                ops.gemm_raw(x.dtype, a=dh.data_ptr() + r0 * f_dim * es, b=x.data_ptr() + r0 * m_dim * es, c_out=c1,
+                             c_in=c1 if accumulate else None, ld_cin=m_dim, m=f_dim, n=m_dim, k=c_rows, lda=f_dim,
+                             ldb=m_dim, ldc=m_dim, a_sg=n_local * c_rows * f_dim, b_sg=n_local * c_rows * m_dim, **common)
+                for s in range(first, first + cnt):  # bias gradients: column sums over each expert's own rows
+                    r = (s * n_local + le) * c_rows
+                    ops.colsum(dy[r:r + c_rows], g[s, b2:b2 + m_dim], accumulate=accumulate)
+                    ops.colsum(dh[r:r + c_rows], g[s, b1:b1 + f_dim], accumulate=accumulate)
         return dx, None, None
 
 

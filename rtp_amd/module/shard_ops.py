@@ -1,0 +1,112 @@
+"""Grouped launches over a run of consecutive shards staged as `flat` = [count, numel].
+
+A weight matrix of the layer is described by (offset inside a flat shard, rows, cols); shard g of the run
+is found `numel` elements after shard g-1, which is the group / K-segment stride handed to rtp_gemm.
+Column-style matrices (output features sharded) use one group per shard; row-style matrices (input
+features sharded) contract over the shards as K segments, so their cross-shard sum stays in the MFMA
+accumulators.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .. import ops
+
+
+def _rows(t: torch.Tensor):
+    m, n, ld = ops._mat(t, "operand")
+    return m, n, ld
+
+
+def col_fwd(x2, flat, w_off, n_s, k, bias_off, out, col0, *, relu=False):
+    """out[:, col0 + g*n_s : col0 + (g+1)*n_s] = x2 @ W_g^T (+ b_g), g over the run."""
+    cnt, numel = flat.shape
+    es = flat.element_size()
+    m, _, lda = _rows(x2)
+    _, _, ldc = _rows(out)
+    out_f32 = out.dtype == torch.float32 and flat.dtype != torch.float32
+    osz = 4 if out_f32 else es
+    ops.gemm_raw(flat.dtype, a=x2.data_ptr(), b=flat.data_ptr() + w_off * es, c_out=out.data_ptr() + col0 * osz,
+                 bias=None if bias_off is None else flat.data_ptr() + bias_off * es, m=m, n=n_s, k=k, lda=lda, ldb=k,
+                 ldc=ldc, a_kcontig=True, b_kcontig=True, relu=relu, out_f32=out_f32, groups=cnt, b_sg=numel,
+                 bias_sg=numel, c_sg=n_s)
+
+
+def col_dgrad(dy2, flat, w_off, n_s, k, out, col0, c_in: Optional[torch.Tensor] = None, gate=None):
+    """out[M, k] = (c_in +) sum_g dy2[:, col0 + g*n_s : ...] @ W_g   (contraction segmented over shards)."""
+    cnt, numel = flat.shape
+    es = flat.element_size()
+    m, _, lda = _rows(dy2)
+    _, _, ldc = _rows(out)
+    kw = ops._epilogue_args(flat.dtype, out, c_in, None, gate)
+    ops.gemm_raw(flat.dtype, a=dy2.data_ptr() + col0 * es, b=flat.data_ptr() + w_off * es, c_out=out.data_ptr(), m=m,
+                 n=k, k=n_s, lda=lda, ldb=k, ldc=ldc, a_kcontig=True, b_kcontig=False, ksegs=cnt, a_sk=n_s,
+                 b_sk=numel, **kw)
+
+
+def col_wgrad(dy2, x2, grads, first, w_off, n_s, k, col0, cnt, accumulate):
+    """grads[first+g, w_off : w_off + n_s*k] (+)= dy2[:, col0 + g*n_s : ...]^T @ x2, g < cnt."""
+    numel = grads.shape[1]
+    es = grads.element_size()
+    m, _, lda = _rows(dy2)
+    _, _, ldb = _rows(x2)
+    c = grads.data_ptr() + (first * numel + w_off) * es
+    ops.gemm_raw(grads.dtype, a=dy2.data_ptr() + col0 * es, b=x2.data_ptr(), c_out=c, m=n_s, n=k, k=m, lda=lda,
+                 ldb=ldb, ldc=k, a_kcontig=False, b_kcontig=False, groups=cnt, a_sg=n_s, c_sg=numel,
+                 c_in=c if accumulate else None, ld_cin=k, cin_sg=numel)
+
+
+def col_bgrad(dy2, grads, first, b_off, n_s, col0, cnt, accumulate):
+    """grads[first+g, b_off : b_off+n_s] (+)= column sums of dy2[:, col0 + g*n_s : ...]."""
+    numel = grads.shape[1]
+    block = dy2[:, col0:col0 + cnt * n_s]
+    ops.colsum(block, grads[first, b_off:b_off + n_s], accumulate=accumulate, seg=n_s, seg_stride=numel)
+
+
+def row_fwd(x2, flat, w_off, n, k_s, bias_off, out, col0, c_in: Optional[torch.Tensor] = None):
+    """out[M, n] = (c_in +) sum_g x2[:, col0 + g*k_s : ...] @ W_g^T + sum_g b_g."""
+    cnt, numel = flat.shape
+    es = flat.element_size()
+    m, _, lda = _rows(x2)
+    _, _, ldc = _rows(out)
+    kw = ops._epilogue_args(flat.dtype, out, c_in, None, None)
+    ops.gemm_raw(flat.dtype, a=x2.data_ptr() + col0 * es, b=flat.data_ptr() + w_off * es, c_out=out.data_ptr(), m=m,
+                 n=n, k=k_s, lda=lda, ldb=k_s, ldc=ldc, a_kcontig=True, b_kcontig=True,
+                 bias=None if bias_off is None else flat.data_ptr() + bias_off * es, bias_sk=numel, ksegs=cnt,
+                 a_sk=k_s, b_sk=numel, **kw)
+
+
+def row_dgrad(dy2, flat, w_off, n, k_s, out, col0):
+    """out[:, col0 + g*k_s : ...] = dy2 @ W_g, g over the run."""
+    cnt, numel = flat.shape
+    es = flat.element_size()
+    m, _, lda = _rows(dy2)
+    _, _, ldc = _rows(out)
+    ops.gemm_raw(flat.dtype, a=dy2.data_ptr(), b=flat.data_ptr() + w_off * es, c_out=out.data_ptr() + col0 * es, m=m,
+                 n=k_s, k=n, lda=lda, ldb=k_s, ldc=ldc, a_kcontig=True, b_kcontig=False, groups=cnt, b_sg=numel,
+                 c_sg=k_s)
+
+
+def row_wgrad(dy2, x2, grads, first, w_off, n, k_s, col0, cnt, accumulate):
+    """grads[first+g, w_off : w_off + n*k_s] (+)= dy2^T @ x2[:, col0 + g*k_s : ...]."""
+    numel = grads.shape[1]
+    es = grads.element_size()
+    m, _, lda = _rows(dy2)
+    _, _, ldb = _rows(x2)
+    c = grads.data_ptr() + (first * numel + w_off) * es
+    ops.gemm_raw(grads.dtype, a=dy2.data_ptr(), b=x2.data_ptr() + col0 * es, c_out=c, m=n, n=k_s, k=m, lda=lda,
+                 ldb=ldb, ldc=k_s, a_kcontig=False, b_kcontig=False, groups=cnt, b_sg=k_s, c_sg=numel,
+                 c_in=c if accumulate else None, ld_cin=k_s, cin_sg=numel)
+
+
+def row_bgrad(dy2, grads, first, b_off, n, cnt, accumulate):
+    """Every row-style shard stores bias/ws and receives the full column sum (tests/test_linear.py:181-186)."""
+    tmp = torch.empty(n, dtype=grads.dtype, device=grads.device)
+    ops.colsum(dy2, tmp)
+    dst = grads[first:first + cnt, b_off:b_off + n]
+    if accumulate:
+        dst.add_(tmp)
+    else:
+        dst.copy_(tmp.expand(cnt, n))

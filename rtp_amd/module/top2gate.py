@@ -15,6 +15,7 @@ from torch import Tensor
 
 from .. import ops
 from ..ring import Rotation, ring_order
+from . import shard_ops as S
 from .collectives import RotatedLayer, resolve_world
 from .utils import affine_weight, as_rows, divide_and_check_no_remainder
 
@@ -80,12 +81,11 @@ class _GateProjectionFn(torch.autograd.Function):
         ws, e_s = layer.world_size, layer.num_local_experts
         x2 = as_rows(x, layer.model_dim)
         logits = torch.empty(x2.shape[0], layer.num_experts, dtype=torch.float32, device=x2.device)
-        order = ring_order(layer.rank, ws)
-        rot = Rotation(store.home, order)
-        for i, idx in enumerate(order):
-            w = store.views(rot.acquire(i))[0]
-            ops.linear_fwd(x2, w, logits[:, idx * e_s:(idx + 1) * e_s])
-            rot.release(i)
+        rot = Rotation(store.home, ring_order(layer.rank, ws))
+        for j in range(rot.steps):
+            for flat, first, cnt in rot.acquire(j):
+                S.col_fwd(x2, flat, 0, e_s, layer.model_dim, None, logits, first * e_s)
+            rot.release(j)
         ctx.layer = layer
         ctx.save_for_backward(x2)
         return logits
@@ -98,19 +98,21 @@ class _GateProjectionFn(torch.autograd.Function):
         ws, e_s = layer.world_size, layer.num_local_experts
         dl = d_logits.to(x2.dtype).contiguous()
         need_dx = ctx.needs_input_grad[0]
-        dx = torch.empty_like(x2) if need_dx else None
-        acc = ops.ShardSum(dx, ws) if need_dx else None
         order = ring_order(layer.rank, ws, reverse=True)
-        rot = Rotation(store.home, order) if need_dx else None
-        for i, idx in enumerate(order):
-            dl_s = dl[:, idx * e_s:(idx + 1) * e_s]
-            if need_dx:
-                w = store.views(rot.acquire(i))[0]
-                c_out, c_in = acc.target(i)
-                ops.linear_dgrad(dl_s, w, c_out, c_in=c_in)
-                rot.release(i)
-            grads, accumulate = store.grad_views(idx)
-            ops.linear_wgrad(dl_s, x2, grads[0], c_in=grads[0] if accumulate else None)
+        dx = None
+        if need_dx:
+            dx = torch.empty_like(x2)
+            rot = Rotation(store.home, order)
+            acc = ops.ShardSum(dx, sum(len(w) for w in rot.windows))
+            i = 0
+            for j in range(rot.steps):
+                for flat, first, cnt in rot.acquire(j):
+                    c_out, c_in = acc.target(i)
+                    S.col_dgrad(dl, flat, 0, e_s, layer.model_dim, c_out, first * e_s, c_in=c_in)
+                    i += 1
+                rot.release(j)
+        for first, cnt, accumulate in store.grad_runs(order):
+            S.col_wgrad(dl, x2, store.grads, first, 0, e_s, layer.model_dim, first * e_s, cnt, accumulate)
         return dx, None, None
 
 

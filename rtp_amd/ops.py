@@ -46,7 +46,9 @@ def gemm_raw(dtype: torch.dtype, *, a: int, b: int, c_out: int, m: int, n: int, 
              ldc: int, a_kcontig: bool, b_kcontig: bool, c_in: Optional[int] = None, ld_cin: int = 0,
              bias: Optional[int] = None, gate: Optional[int] = None, ld_gate: int = 0, alpha: float = 1.0,
              relu: bool = False, out_f32: bool = False, cin_f32: bool = False, batch: int = 1, zdiv: int = 1,
-             a_s=(0, 0), b_s=(0, 0), c_s=(0, 0), cin_s=(0, 0), gate_s=(0, 0), bias_s=(0, 0)) -> None:
+             a_s=(0, 0), b_s=(0, 0), c_s=(0, 0), cin_s=(0, 0), gate_s=(0, 0), bias_s=(0, 0), groups: int = 1,
+             a_sg: int = 0, b_sg: int = 0, c_sg: int = 0, cin_sg: int = 0, gate_sg: int = 0, bias_sg: int = 0,
+             ksegs: int = 1, a_sk: int = 0, b_sk: int = 0, bias_sk: int = 0) -> None:
     """One rtp_gemm call on raw device addresses (see include/rtp_hip.h for the operand rules)."""
     _lib.require_device()
     d = GemmDesc()
@@ -60,6 +62,9 @@ def gemm_raw(dtype: torch.dtype, *, a: int, b: int, c_out: int, m: int, n: int, 
     d.cin_so, d.cin_si = cin_s
     d.gate_so, d.gate_si = gate_s
     d.bias_so, d.bias_si = bias_s
+    d.groups, d.ksegs = groups, ksegs
+    d.a_sg, d.b_sg, d.c_sg, d.cin_sg, d.gate_sg, d.bias_sg = a_sg, b_sg, c_sg, cin_sg, gate_sg, bias_sg
+    d.a_sk, d.b_sk, d.bias_sk = a_sk, b_sk, bias_sk
     d.alpha = alpha
     d.flags = (GEMM_OUT_F32 if out_f32 else 0) | (GEMM_CIN_F32 if cin_f32 else 0) | (GEMM_RELU if relu else 0)
     d.a_kcontig, d.b_kcontig = int(a_kcontig), int(b_kcontig)
@@ -136,18 +141,25 @@ def linear_wgrad(dy: torch.Tensor, x: torch.Tensor, out: torch.Tensor, *, c_in=N
              ldc=ldc, a_kcontig=False, b_kcontig=False, **_epilogue_args(dy.dtype, out, c_in, None, None))
 
 
-def colsum(x: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
-    """out[N] (+)= sum over rows of x[M,N]   (bias gradient)."""
+def colsum(x: torch.Tensor, out: torch.Tensor, accumulate: bool = False, seg: int = 0, seg_stride: int = 0) -> None:
+    """Column sums of x[M,N] (bias gradients).  With seg == 0: out[N] (+)= sums.  With seg > 0 column c goes
+    to out.view(-1)[(c // seg) * seg_stride + c % seg]: `out` is then the first segment's destination inside
+    a larger buffer that holds one segment per shard, seg_stride elements apart."""
     _dev(x)
     _dev(out)
     m, n, ld = _mat(x, "x")
-    if out.dim() != 1 or out.shape[0] != n or not out.is_contiguous():
+    if seg == 0 and (out.dim() != 1 or out.shape[0] != n or not out.is_contiguous()):
         raise ValueError("colsum: out must be a contiguous vector of x's width")
+    if seg and (n % seg != 0 or seg_stride < seg):
+        raise ValueError("colsum: width must be a multiple of seg and seg_stride >= seg")
     if out.dtype not in (x.dtype, torch.float32):
         raise TypeError("colsum: out must be the input dtype or float32")
     _lib.require_device()
-    check(_lib.load().rtp_colsum(_stream(), dtype_code(x.dtype), x.data_ptr(), m, n, ld, out.data_ptr(),
-                                 int(out.dtype == torch.float32), int(accumulate)))
+    lib = _lib.load()
+    nbytes = lib.rtp_colsum_workspace_bytes(m, n)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    check(lib.rtp_colsum(_stream(), dtype_code(x.dtype), x.data_ptr(), m, n, ld, out.data_ptr(),
+                         int(out.dtype == torch.float32), int(accumulate), seg, seg_stride, ws.data_ptr(), nbytes))
 
 
 def shard_copy(dst: torch.Tensor, src: torch.Tensor) -> None:
@@ -170,8 +182,10 @@ def zero_(t: torch.Tensor) -> None:
     check(_lib.load().rtp_zero_async(_stream(), t.data_ptr(), t.numel() * t.element_size()))
 
 
-def embedding_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, row_begin: int = 0) -> None:
-    """out[t, :] = table[ids[t] - row_begin, :] for ids inside the shard's row range."""
+def embedding_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, row_begin: int = 0, groups: int = 1,
+                     table_sg: int = 0, out_sg: int = 0) -> None:
+    """out[t, :] = table[ids[t] - row_begin, :] for ids inside the shard's row range.  With groups > 1,
+    `table` / `out` are shard 0's table and output block; shard g sits table_sg / out_sg elements further."""
     for t in (table, ids, out):
         _dev(t)
     rows, cols, ld_t = _mat(table, "table")
@@ -181,7 +195,8 @@ def embedding_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, 
         raise ValueError("embedding_gather: ids must be contiguous int64 with one id per output row")
     _lib.require_device()
     check(_lib.load().rtp_embedding_gather(_stream(), dtype_code(table.dtype), table.data_ptr(), ld_t, row_begin,
-                                           rows, cols, ids.data_ptr(), n, out.data_ptr(), ld_o))
+                                           rows, cols, ids.data_ptr(), n, out.data_ptr(), ld_o, groups, table_sg,
+                                           out_sg))
 
 
 def embedding_sort_ids(ids: torch.Tensor) -> torch.Tensor:

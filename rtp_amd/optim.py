@@ -12,7 +12,7 @@ from typing import List, Optional
 import torch
 import torch.nn as nn
 
-from . import ops
+from . import ops, ring
 from .module.collectives import ShardStore
 
 
@@ -37,10 +37,10 @@ class RotatedSGD:
         return n + sum(m.numel() * 4 for m in self.other_masters if m is not None)
 
     def zero_grad(self) -> None:
+        """Rotated layers keep their gradient views attached and overwrite them in the next backward (no
+        per-parameter work); other parameters get .grad = None as torch does."""
         for st in self.stores:
-            for sm in st.modules:
-                for p in sm.parameters():
-                    p.grad = None
+            st.mark_overwrite()
         for p in self.other:
             p.grad = None
 
@@ -62,3 +62,5 @@ class RotatedSGD:
                 ops.sgd_step(p.data.view(-1), g, None, self.lr, self.clip_value)
             else:
                 ops.sgd_step(master.view(-1), g, p.data.view(-1), self.lr, self.clip_value)
+        if self.stores:
+            ring.fence(self.stores[0].home.device)  # staging copies of the next step must see the new weights

@@ -1,15 +1,17 @@
 """Single-GPU shard rotation: the ring of rtp/module/collectives.py:202-317 collapsed onto one device.
 
-Every shard of a layer lives exactly once in the layer's home storage.  A rotation visits the shards
-in ring order; while step i computes on the shard sitting in one slot of a two-slot staging buffer, the
-copy kernel streams the shard of step i+1 into the other slot on a side stream (what a neighbour's
-isend/irecv does in the multi-GPU reference).  The staging buffer is shared by all layers of a device,
-so the resident weight bytes are 1x the model plus two slots of the largest shard.
+Every shard of a layer lives exactly once in the layer's home storage.  A rotation visits the shards in
+ring order, `window` shards at a time: while the kernels of one window read its shards from one slot of a
+two-slot staging buffer, the copy kernel streams the next window -- of this layer, or the first window
+of the next layer -- into the other slot on a side stream (what a neighbour's isend/irecv does in the
+multi-GPU reference).  window = 1 is the reference's step-by-step schedule; a larger window lets one
+grouped kernel launch cover several ring steps.  The staging buffer is shared by all layers of a device,
+so the resident weight bytes are 1x the model plus two slots of the largest window.
 """
 from __future__ import annotations
 
 import ctypes as C
-from typing import Dict, List, Optional, Sequence
+from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
@@ -18,6 +20,19 @@ from ._lib import check
 
 _SLOT_ALIGN = 256
 _ELEMENT_SIZE = {torch.float32: 4, torch.bfloat16: 2}
+_window: Optional[int] = None
+
+
+def set_rotation_window(window: Optional[int]) -> None:
+    """Ring steps staged and computed together (None = all shards of a layer, 1 = one shard per step)."""
+    global _window
+    if window is not None and window < 1:
+        raise ValueError("rotation window must be >= 1")
+    _window = window
+
+
+def rotation_window() -> Optional[int]:
+    return _window
 
 
 class DeviceRing:
@@ -32,7 +47,7 @@ class DeviceRing:
         self._handle = handle
         self.slot_bytes = 0
         self.staging: Optional[torch.Tensor] = None
-        self.peak_slot_bytes = 0
+        self.next_slot = 0
 
     def reserve(self, nbytes: int) -> None:
         if nbytes <= self.slot_bytes:
@@ -41,14 +56,16 @@ class DeviceRing:
         torch.cuda.synchronize(self.device)
         self.slot_bytes = (nbytes + _SLOT_ALIGN - 1) // _SLOT_ALIGN * _SLOT_ALIGN
         self.staging = torch.empty(2 * self.slot_bytes, dtype=torch.uint8, device=self.device)
-        self.peak_slot_bytes = max(self.peak_slot_bytes, self.slot_bytes)
+        self.fence()
 
-    def slot_ptr(self, slot: int) -> int:
-        return self.staging.data_ptr() + slot * self.slot_bytes
+    def take_slot(self) -> int:
+        slot = self.next_slot
+        self.next_slot ^= 1
+        return slot
 
-    def slot_view(self, slot: int, numel: int, dtype: torch.dtype) -> torch.Tensor:
-        nbytes = numel * _ELEMENT_SIZE[dtype]
-        return self.staging[slot * self.slot_bytes: slot * self.slot_bytes + nbytes].view(dtype)
+    def fence(self) -> None:
+        """Home storage was written by work queued on the current stream: the next staging copy waits."""
+        check(_lib.load().rtp_ring_fence(self._handle, torch.cuda.current_stream(self.device).cuda_stream))
 
     def __del__(self):
         try:
@@ -69,6 +86,16 @@ def device_ring(device: torch.device) -> DeviceRing:
     return ring
 
 
+def fence(device: Optional[torch.device] = None) -> None:
+    """Call after modifying rotated weights in place with your own kernels (optimizer step, weight load)
+    and after ending a HIP-graph capture: orders the next staging copy after that work."""
+    if device is None:
+        device = torch.device("cuda", torch.cuda.current_device())
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    if idx in _rings:
+        _rings[idx].fence()
+
+
 def staging_bytes(device: Optional[torch.device] = None) -> int:
     """Bytes held by the two staging slots on `device` (0 before the first rotation)."""
     if device is None:
@@ -78,42 +105,70 @@ def staging_bytes(device: Optional[torch.device] = None) -> int:
     return 0 if ring is None else 2 * ring.slot_bytes
 
 
-class Rotation:
-    """One pass over the shards of a layer, in the given order.
+Run = Tuple[torch.Tensor, int, int]  # (staged [count, numel] view, first shard index, count)
 
-        rot = Rotation(home, order)          # home: [ws, numel] tensor, order: shard indices
-        for i in range(len(order)):
-            flat = rot.acquire(i)            # staged copy of shard order[i]; prefetches order[i+1]
-            ... launch kernels that read `flat` on the current stream ...
-            rot.release(i)
+
+class Rotation:
+    """One pass over the shards of a layer in ring order, `window` ring steps at a time.
+
+        rot = Rotation(home, order)            # home: [ws, numel], order: shard index per ring step
+        for j in range(rot.steps):
+            for staged, first, count in rot.acquire(j):   # staged[i] is a copy of home[first + i]
+                ... launch kernels that read `staged` on the current stream ...
+            rot.release(j)
+
+    A window's shards are staged in ascending index order as runs of consecutive shards, so a grouped
+    kernel can address them with one stride.
     """
 
-    def __init__(self, home: torch.Tensor, order: Sequence[int]):
+    def __init__(self, home: torch.Tensor, order: Sequence[int], window: Optional[int] = None):
         if home.dim() != 2 or not home.is_contiguous():
             raise ValueError("Rotation: home must be a contiguous [shards, numel] tensor")
         self.home = home
-        self.order = list(order)
         self.numel = home.shape[1]
         self.nbytes = self.numel * home.element_size()
+        order = list(order)
+        w = window if window is not None else _window
+        w = len(order) if w is None else max(1, min(int(w), len(order)))
+        self.windows: List[List[Tuple[int, int]]] = []
+        for i in range(0, len(order), w):
+            ids = sorted(order[i:i + w])
+            runs, start = [], ids[0]
+            for a, b in zip(ids, ids[1:] + [None]):
+                if b is None or b != a + 1:
+                    runs.append((start, a - start + 1))
+                    start = b
+            self.windows.append(runs)
+        self.steps = len(self.windows)
         self.ring = device_ring(home.device)
-        self.ring.reserve(self.nbytes)
+        self.ring.reserve(w * self.nbytes)
         self.lib = _lib.load()
         self.stream = torch.cuda.current_stream(home.device).cuda_stream
-        check(self.lib.rtp_ring_begin(self.ring._handle, self.stream))
+        self.slots = [None] * self.steps
         self._prefetch(0)
 
-    def _prefetch(self, i: int) -> None:
-        src = self.home.data_ptr() + self.order[i] * self.nbytes
-        check(self.lib.rtp_ring_prefetch(self.ring._handle, i & 1, self.ring.slot_ptr(i & 1), src, self.nbytes))
+    def _prefetch(self, j: int) -> None:
+        slot = self.slots[j] = self.ring.take_slot()
+        dst = self.ring.staging.data_ptr() + slot * self.ring.slot_bytes
+        for first, count in self.windows[j]:
+            check(self.lib.rtp_ring_prefetch(self.ring._handle, self.stream, slot, dst,
+                                             self.home.data_ptr() + first * self.nbytes, count * self.nbytes))
+            dst += count * self.nbytes
 
-    def acquire(self, i: int) -> torch.Tensor:
-        if i + 1 < len(self.order):
-            self._prefetch(i + 1)
-        check(self.lib.rtp_ring_acquire(self.ring._handle, self.stream, i & 1))
-        return self.ring.slot_view(i & 1, self.numel, self.home.dtype)
+    def acquire(self, j: int) -> List[Run]:
+        if j + 1 < self.steps:
+            self._prefetch(j + 1)
+        slot = self.slots[j]
+        check(self.lib.rtp_ring_acquire(self.ring._handle, self.stream, slot))
+        out, off = [], slot * self.ring.slot_bytes
+        for first, count in self.windows[j]:
+            nb = count * self.nbytes
+            out.append((self.ring.staging[off:off + nb].view(self.home.dtype).view(count, self.numel), first, count))
+            off += nb
+        return out
 
-    def release(self, i: int) -> None:
-        check(self.lib.rtp_ring_release(self.ring._handle, self.stream, i & 1))
+    def release(self, j: int) -> None:
+        check(self.lib.rtp_ring_release(self.ring._handle, self.stream, self.slots[j]))
 
 
 def ring_order(rank: int, world_size: int, reverse: bool = False) -> List[int]:

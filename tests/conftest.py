@@ -18,3 +18,14 @@ def _seed():
 
     torch.manual_seed(0)
     yield
+
+
+@pytest.fixture(params=[None, 1, 3], ids=["window=all", "window=1", "window=3"])
+def rotation_window(request):
+    """Runs a GPU test under three rotation schedules: all shards of a layer staged together (one grouped
+    launch per layer), one shard per ring step (the reference's schedule), and a window that does not
+    divide the shard count (ragged last window)."""
+    from rtp_amd.ring import set_rotation_window
+    set_rotation_window(request.param)
+    yield request.param
+    set_rotation_window(None)

@@ -8,7 +8,7 @@ import torch.nn as nn
 from gpu_util import DEV
 from oracle import rtp_oracle as O
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("rotation_window")]
 
 
 def _layer(master, ws, dtype=torch.float32, **kw):

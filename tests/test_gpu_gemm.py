@@ -121,3 +121,52 @@ def test_colsum_and_errors():
         ops.linear_fwd(torch.randn(4, 4), torch.randn(4, 4), torch.empty(4, 4))  # CPU tensors: no fallback
     with pytest.raises(ValueError):
         ops.linear_fwd(x.to(DEV), torch.randn(5, 71, device=DEV), torch.empty(300, 5, device=DEV))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gemm_groups_and_k_segments(dtype):
+    """Several shards in one launch: groups (column-parallel forward) and K segments (sum over shards)."""
+    ops = _ops()
+    gen = torch.Generator().manual_seed(17)
+    ws, m, k, n_s = 4, 150, 96, 40
+    numel = n_s * k + n_s  # flat shard: [weight, bias]
+    home = _rand((ws, numel), dtype, gen)
+    x = _rand((m, k), dtype, gen)
+    hd, xd = home.to(DEV), x.to(DEV)
+    y = torch.full((m, ws * n_s), float("nan"), dtype=dtype, device=DEV)
+    ops.gemm_raw(dtype, a=xd.data_ptr(), b=hd.data_ptr(), c_out=y.data_ptr(), bias=hd.data_ptr() + n_s * k * hd.element_size(),
+                 m=m, n=n_s, k=k, lda=k, ldb=k, ldc=ws * n_s, a_kcontig=True, b_kcontig=True, groups=ws,
+                 b_sg=numel, bias_sg=numel, c_sg=n_s)
+    w = home[:, :n_s * k].reshape(ws * n_s, k).double()
+    b = home[:, n_s * k:].reshape(-1).double()
+    assert rel_err(y, x.double() @ w.t() + b) <= TOL[dtype]
+    # input gradient of the same layer: dX = sum_s dY[:, s-block] @ W_s, contraction segmented over shards
+    dy = _rand((m, ws * n_s), dtype, gen)
+    dyd = dy.to(DEV)
+    dx = torch.empty(m, k, dtype=dtype, device=DEV)
+    ops.gemm_raw(dtype, a=dyd.data_ptr(), b=hd.data_ptr(), c_out=dx.data_ptr(), m=m, n=k, k=n_s, lda=ws * n_s, ldb=k,
+                 ldc=k, a_kcontig=True, b_kcontig=False, ksegs=ws, a_sk=n_s, b_sk=numel)
+    assert rel_err(dx, dy.double() @ w) <= TOL[dtype]
+    # weight gradients of all shards: group g writes dW_g = dY[:, g-block]^T @ X into its flat gradient row
+    grads = torch.zeros(ws, numel, dtype=dtype, device=DEV)
+    ops.gemm_raw(dtype, a=dyd.data_ptr(), b=xd.data_ptr(), c_out=grads.data_ptr(), m=n_s, n=k, k=m, lda=ws * n_s, ldb=k,
+                 ldc=k, a_kcontig=False, b_kcontig=False, groups=ws, a_sg=n_s, c_sg=numel)
+    ops.colsum(dyd, grads[0, n_s * k:], seg=n_s, seg_stride=numel)
+    assert rel_err(grads[:, :n_s * k].reshape(ws * n_s, k), dy.double().t() @ x.double()) <= TOL[dtype]
+    assert rel_err(grads[:, n_s * k:].reshape(-1), dy.double().sum(0)) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,n,k", [(1024, 2048, 2048), (2048, 2048, 1024), (512, 640, 300)])
+def test_gemm_mid_tile_path(dtype, m, n, k):
+    """Shapes that select the 128x64 tile (and its three-slab register ring)."""
+    ops = _ops()
+    gen = torch.Generator().manual_seed(m + n)
+    a, b = _rand((m, k), dtype, gen), _rand((n, k), dtype, gen)
+    out = torch.empty(m, n, dtype=dtype, device=DEV)
+    ops.linear_fwd(a.to(DEV), b.to(DEV), out)
+    assert rel_err(out, a.double() @ b.double().t()) <= TOL[dtype]
+    dy = _rand((m, n), dtype, gen).to(DEV)
+    dw = torch.empty(n, k, dtype=dtype, device=DEV)
+    ops.linear_wgrad(dy, a.to(DEV), dw)
+    assert rel_err(dw, dy.double().cpu().t() @ a.double()) <= TOL[dtype]

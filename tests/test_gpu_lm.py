@@ -9,7 +9,7 @@ import torch.nn.functional as F
 from gpu_util import DEV, assert_close, rel_err
 from oracle import rtp_oracle as O
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("rotation_window")]
 
 
 def load_unsharded(lm, ref):
@@ -129,8 +129,14 @@ def test_lm_sgd_step_matches_closed_form():
     opt.step()
     assert torch.equal(lm[-1].linear.linears[1].weight.detach(), before - 0.1 * g)
     assert torch.equal(lm[2].norm1.weight.detach(), ln_before - 0.1 * ln_g)
+    # zero_grad keeps the gradient views attached and makes the next backward overwrite them
     opt.zero_grad()
-    assert lm[-1].linear.linears[1].weight.grad is None
+    assert lm[2].norm1.weight.grad is None
+    F.cross_entropy(lm(ids.to(DEV)).view(-1, V), ids.to(DEV).view(-1)).backward()
+    g2 = lm[-1].linear.linears[1].weight.grad.detach().clone()
+    opt.zero_grad()
+    F.cross_entropy(lm(ids.to(DEV)).view(-1, V), ids.to(DEV).view(-1)).backward()
+    assert torch.equal(lm[-1].linear.linears[1].weight.grad, g2)  # overwritten, not accumulated
 
 
 def test_lm_bf16_master_weights_and_weight_bytes():

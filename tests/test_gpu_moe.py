@@ -10,7 +10,7 @@ import torch.nn as nn
 from gpu_util import DEV, assert_close, rel_err
 from oracle import rtp_oracle as O
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("rotation_window")]
 GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
 
 

@@ -8,7 +8,8 @@ from gpu_util import DEV
 pytestmark = pytest.mark.gpu
 
 
-def test_rotation_delivers_each_shard_in_ring_order():
+@pytest.mark.parametrize("window", [1, 3, None])
+def test_rotation_delivers_each_shard_in_ring_order(window):
     from rtp_amd.ring import Rotation, ring_order
     ws, numel = 8, 100_003
     home = torch.randn(ws, numel, device=DEV)
@@ -16,36 +17,62 @@ def test_rotation_delivers_each_shard_in_ring_order():
     for rank in (0, 3):
         order = ring_order(rank, ws)
         assert sorted(order) == list(range(ws)) and order[0] == rank
-        rot = Rotation(home, order)
-        for i, idx in enumerate(order):
-            flat = rot.acquire(i)
-            seen.append((idx, flat.clone()))
-            rot.release(i)
+        rot = Rotation(home, order, window=window)
+        visited = []
+        for j in range(rot.steps):
+            for flat, first, cnt in rot.acquire(j):
+                assert flat.shape == (cnt, numel)
+                seen.append((first, cnt, flat.clone()))
+                visited += list(range(first, first + cnt))
+            rot.release(j)
+        assert sorted(visited) == list(range(ws))
+        w = window or ws
+        for j, win in enumerate(rot.windows):  # window j holds ring steps j*w .. j*w+w-1
+            assert sorted(s for f, c in win for s in range(f, f + c)) == sorted(order[j * w:(j + 1) * w])
     torch.cuda.synchronize()
-    for idx, flat in seen:
-        assert torch.equal(flat, home[idx])
+    for first, cnt, flat in seen:
+        assert torch.equal(flat, home[first:first + cnt])
     assert ring_order(2, 4, reverse=True) == [1, 0, 3, 2]
 
 
-def test_rotation_fencing_under_slot_reuse():
-    """A slow consumer (large reduction) reads slot s while the prefetch of step i+2 wants the same slot:
-    the checksum of what each step consumed must be the checksum of its own shard."""
+@pytest.mark.parametrize("window", [1, 2])
+def test_rotation_fencing_under_slot_reuse(window):
+    """A slow consumer (large matmul) reads a slot while later prefetches want it again, across several
+    back-to-back rotations that share the two slots: what each step consumed must be its own shards."""
     from rtp_amd.ring import Rotation, ring_order
     ws, numel = 6, 4_000_000
-    home = torch.arange(ws, device=DEV, dtype=torch.float32).view(ws, 1).repeat(1, numel).contiguous()
+    home = torch.arange(1, ws + 1, device=DEV, dtype=torch.float32).view(ws, 1).repeat(1, numel).contiguous()
     sums = []
     for _ in range(5):
-        order = ring_order(0, ws)
-        rot = Rotation(home, order)
-        for i, idx in enumerate(order):
-            flat = rot.acquire(i)
-            a = flat.view(2000, 2000)
-            sums.append((idx, (a @ a[:, :64]).sum() / max(idx, 1) ** 2))  # heavy kernel reading the slot
-            rot.release(i)
+        rot = Rotation(home, ring_order(0, ws), window=window)
+        for j in range(rot.steps):
+            for flat, first, cnt in rot.acquire(j):
+                for i in range(cnt):
+                    a = flat[i].view(2000, 2000)
+                    sums.append((first + i, (a @ a[:, :64]).sum()))  # heavy kernel reading the slot
+            rot.release(j)
     torch.cuda.synchronize()
     for idx, s in sums:
-        expect = 0.0 if idx == 0 else 2000 * 2000 * 64.0
-        assert abs(float(s) - expect) <= 1e-3 * max(expect, 1.0), (idx, float(s), expect)
+        expect = 2000 * 2000 * 64.0 * (idx + 1) ** 2
+        assert abs(float(s) - expect) <= 1e-3 * expect, (idx, float(s), expect)
+
+
+def test_fence_orders_staging_after_weight_update():
+    """Weights rewritten by a kernel on the compute stream, then fence(): the next rotation stages the new
+    values, not the old ones."""
+    from rtp_amd import ring
+    from rtp_amd.ring import Rotation, ring_order
+    home = torch.zeros(4, 1_000_000, device=DEV)
+    for step in range(1, 4):
+        big = torch.randn(3000, 3000, device=DEV)
+        (big @ big).sum()  # keep the compute stream busy ahead of the update
+        home.fill_(float(step))
+        ring.fence()
+        rot = Rotation(home, ring_order(0, 4))
+        (flat, first, cnt), = rot.acquire(0)
+        got = flat.sum().item()
+        rot.release(0)
+        assert got == step * 4 * 1_000_000.0
 
 
 def test_copy_and_zero_kernels_ragged():

@@ -9,7 +9,7 @@ import torch.nn as nn
 from gpu_util import DEV, assert_close
 from oracle import rtp_oracle as O
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("rotation_window")]
 
 
 class Net(nn.Module):
