@@ -15,6 +15,8 @@
 // ring of register buffers, which is what hides HBM/L2 latency when only one workgroup fits a CU.
 #include "common.h"
 
+#include <type_traits>
+
 namespace rtp {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -59,9 +61,10 @@ struct Slab {
 
   // FAST: every 16-byte vector of the slab is either wholly inside the operand or wholly outside it
   // (guaranteed by the host: aligned pointers and strides, extents that are multiples of VEC), so a
-  // vector is loaded unconditionally from a clamped address and, if it lies beyond the contraction
-  // length, replaced by zeros with a select.  No branches, so all loads of a slab issue back to back.
-  // Rows beyond the operand are clamped too: they only feed accumulators the epilogue never stores.
+  // vector is loaded unconditionally from a clamped address; vectors beyond the contraction length are
+  // replaced by zeros later, when the registers are moved to LDS (store with ktail), so nothing here
+  // consumes a load result and all loads of a slab stay in flight.  Rows beyond the operand are clamped
+  // too: they only feed accumulators the epilogue never stores.
   // !FAST: element-wise guarded loads for ragged or unaligned operands.
   template <bool FAST>
   __device__ __forceinline__ void load(const T* base, long ld, int row0, int rows, int k0, int kdim, int tid) {
@@ -77,10 +80,8 @@ struct Slab {
         const int k = k0 + (v % KV) * VEC;
         if (FAST) {
           const int rc = row < rows ? row : rows - 1;
-          const bool live = k < kdim;
-          const int kc = live ? k : 0;
+          const int kc = k < kdim ? k : 0;
           u.q = *reinterpret_cast<const uint4*>(base + (long)rc * ld + kc);
-          if (!live) u.q = make_uint4(0, 0, 0, 0);
         } else {
           const T* src = base + (long)row * ld + k;
 #pragma unroll
@@ -90,11 +91,9 @@ struct Slab {
         const int k = k0 + v / RV;
         const int row = row0 + (v % RV) * VEC;
         if (FAST) {
-          const bool live = k < kdim;
-          const int kc = live ? k : 0;
+          const int kc = k < kdim ? k : 0;
           const int rc = row < rows ? row : 0;
           u.q = *reinterpret_cast<const uint4*>(base + (long)kc * ld + rc);
-          if (!live) u.q = make_uint4(0, 0, 0, 0);
         } else {
           const T* src = base + (long)k * ld + row;
 #pragma unroll
@@ -105,12 +104,22 @@ struct Slab {
     }
   }
 
-  __device__ __forceinline__ void store(char* lds, int tid) const {
+  // ktail: the slab that starts at k0 reaches beyond kdim, zero the vectors that lie outside.
+  __device__ __forceinline__ void store(char* lds, int tid, bool ktail, int k0, int kdim) const {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int v = tid + i * kThreads;
       char* dst = KC ? lds + (v / KV) * kRowPitchKC + (v % KV) * 16 : lds + (v / RV) * PITCH + (v % RV) * 16;
-      *reinterpret_cast<uint4*>(dst) = reg[i];
+      uint4 q = reg[i];
+      if (ktail) {
+        const int k = KC ? k0 + (v % KV) * VEC : k0 + v / RV;
+        const bool live = k < kdim;
+        q.x = live ? q.x : 0u;
+        q.y = live ? q.y : 0u;
+        q.z = live ? q.z : 0u;
+        q.w = live ? q.w : 0u;
+      }
+      *reinterpret_cast<uint4*>(dst) = q;
     }
   }
 };
@@ -156,6 +165,56 @@ __device__ __forceinline__ void mma(const Frag<float>& a, const Frag<float>& b, 
   for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.f[e], b.f[e], c, 0, 0, 0);
 }
 
+// Fused epilogue shared by the GEMM kernels.  Accumulator register r of lane (li, g) is output row
+// 8*(r/4) + 4*g + r%4, column li of its 32x32 block.
+template <typename T, int MT, int NT, int WM, int WN>
+__device__ __forceinline__ void store_tile(const GemmArgs& p, f32x16 (&acc)[MT][NT], int m0, int n0, int wm, int wn,
+                                           int li, int g, int grp, long zo, long zi) {
+  const bool out_f32 = p.flags & RTP_GEMM_OUT_F32;
+  const bool cin_f32 = p.flags & RTP_GEMM_CIN_F32;
+  const bool relu = p.flags & RTP_GEMM_RELU;
+  char* cbase = p.c_out + (grp * p.c_sg + zo * p.c_so + zi * p.c_si) * (out_f32 ? 4 : (long)sizeof(T));
+  const char* cin =
+      p.c_in ? p.c_in + (grp * p.cin_sg + zo * p.cin_so + zi * p.cin_si) * (cin_f32 ? 4 : (long)sizeof(T)) : nullptr;
+  const T* bias =
+      p.bias ? reinterpret_cast<const T*>(p.bias) + grp * p.bias_sg + zo * p.bias_so + zi * p.bias_si : nullptr;
+  const T* gate =
+      p.gate ? reinterpret_cast<const T*>(p.gate) + grp * p.gate_sg + zo * p.gate_so + zi * p.gate_si : nullptr;
+
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const int col = n0 + wn * WN + j * 32 + li;
+      if (col >= p.n) continue;
+      float bv = 0.0f;
+      if (bias) {
+        // a bias per K segment (row-parallel shards each carry bias/ws): summed in segment order
+        const int nb_seg = p.bias_sk ? p.ksegs : 1;
+        for (int sgm = 0; sgm < nb_seg; ++sgm) bv += to_f32(bias[sgm * p.bias_sk + col]);
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = m0 + wm * WM + i * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+        if (row >= p.m) continue;
+        float v = p.alpha * acc[i][j][r];
+        if (cin) {
+          const long off = (long)row * p.ld_cin + col;
+          v += cin_f32 ? reinterpret_cast<const float*>(cin)[off] : to_f32(reinterpret_cast<const T*>(cin)[off]);
+        }
+        v += bv;
+        if (relu) v = fmaxf(v, 0.0f);
+        if (gate) v = to_f32(gate[(long)row * p.ld_gate + col]) > 0.0f ? v : 0.0f;
+        const long off = (long)row * p.ldc + col;
+        if (out_f32)
+          reinterpret_cast<float*>(cbase)[off] = v;
+        else
+          reinterpret_cast<T*>(cbase)[off] = from_f32<T>(v);
+      }
+    }
+  }
+}
+
 template <typename T, int BM, int BN, bool AKC, bool BKC, int DEPTH, bool FAST>
 struct GemmTile {
   using LA = Slab<T, BM, AKC>;
@@ -181,10 +240,14 @@ struct GemmTile {
     la[R].template load<FAST>(A + seg * p.a_sk, p.lda, m0, p.m, k0, p.k, tid);
     lb[R].template load<FAST>(B + seg * p.b_sk, p.ldb, n0, p.n, k0, p.k, tid);
   }
+  // `slab` is the slab held by register slot R; only the last slab of a K segment can be partial.
   template <int R>
-  __device__ __forceinline__ void stash(char* stage) {
-    la[R].store(stage, tid);
-    lb[R].store(stage + LA::BYTES, tid);
+  __device__ __forceinline__ void stash(char* stage, int slab) {
+    const int seg = slab / nk_seg;
+    const int k0 = (slab - seg * nk_seg) * BK;
+    const bool ktail = FAST && k0 + BK > p.k;
+    la[R].store(stage, tid, ktail, k0, p.k);
+    lb[R].store(stage + LA::BYTES, tid, ktail, k0, p.k);
   }
 };
 
@@ -229,12 +292,9 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs p) {
   if (nk > 0) t.template fetch<0>(0);
   if (DEPTH > 1 && nk > 1) t.template fetch<1 % DEPTH>(1);
   if (DEPTH > 2 && nk > 2) t.template fetch<2 % DEPTH>(2);
-  if (nk > 0) t.template stash<0>(lds);
+  if (nk > 0) t.template stash<0>(lds, 0);
   __syncthreads();
 
-  // Steady state for slab kt (register slot kt % DEPTH was just emptied into LDS): refill that slot
-  // with slab kt+DEPTH, run the MFMAs of slab kt from LDS stage kt&1, move slab kt+1 from its register
-  // slot to the other LDS stage, barrier.
   auto compute = [&](int kt) {
     const char* sa = lds + (kt & 1) * STAGE;
     const char* sb = sa + G::LA::BYTES;
@@ -252,72 +312,297 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs p) {
     }
   };
 
-  for (int kt = 0; kt < nk; kt += DEPTH) {
+  // Steady state for slab kt (register slot kt % DEPTH was just emptied into LDS): refill that slot
+  // with slab kt+DEPTH, run the MFMAs of slab kt from LDS stage kt&1, move slab kt+1 from its register
+  // slot to the other LDS stage, barrier.  While 2*DEPTH slabs remain none of this needs a guard, so the
+  // loop body is branch-free and the loads of DEPTH slabs stay in flight across the barriers.
+  int kt = 0;
+  for (; kt + 2 * DEPTH <= nk; kt += DEPTH) {
+    t.template fetch<0>(kt + DEPTH);
+    compute(kt);
+    t.template stash<1 % DEPTH>(lds + ((kt + 1) & 1) * STAGE, kt + 1);
+    __syncthreads();
+    if (DEPTH > 1) {
+      t.template fetch<1 % DEPTH>(kt + 1 + DEPTH);
+      compute(kt + 1);
+      t.template stash<2 % DEPTH>(lds + ((kt + 2) & 1) * STAGE, kt + 2);
+      __syncthreads();
+    }
+    if (DEPTH > 2) {
+      t.template fetch<2 % DEPTH>(kt + 2 + DEPTH);
+      compute(kt + 2);
+      t.template stash<0>(lds + ((kt + 3) & 1) * STAGE, kt + 3);
+      __syncthreads();
+    }
+  }
+  // Drain: the same phases with guards (kt is a multiple of DEPTH, so the slot assignment continues).
+  for (; kt < nk; kt += DEPTH) {
     if (kt + DEPTH < nk) t.template fetch<0>(kt + DEPTH);
     compute(kt);
-    if (kt + 1 < nk) t.template stash<1 % DEPTH>(lds + ((kt + 1) & 1) * STAGE);
+    if (kt + 1 < nk) t.template stash<1 % DEPTH>(lds + ((kt + 1) & 1) * STAGE, kt + 1);
     __syncthreads();
     if (DEPTH > 1) {
       if (kt + 1 >= nk) break;
       if (kt + 1 + DEPTH < nk) t.template fetch<1 % DEPTH>(kt + 1 + DEPTH);
       compute(kt + 1);
-      if (kt + 2 < nk) t.template stash<2 % DEPTH>(lds + ((kt + 2) & 1) * STAGE);
+      if (kt + 2 < nk) t.template stash<2 % DEPTH>(lds + ((kt + 2) & 1) * STAGE, kt + 2);
       __syncthreads();
     }
     if (DEPTH > 2) {
       if (kt + 2 >= nk) break;
       if (kt + 2 + DEPTH < nk) t.template fetch<2 % DEPTH>(kt + 2 + DEPTH);
       compute(kt + 2);
-      if (kt + 3 < nk) t.template stash<0>(lds + ((kt + 3) & 1) * STAGE);
+      if (kt + 3 < nk) t.template stash<0>(lds + ((kt + 3) & 1) * STAGE, kt + 3);
       __syncthreads();
     }
   }
 
-  // Epilogue.  Accumulator register r of lane (li, g) is output row 8*(r/4) + 4*g + r%4, column li
-  // of its 32x32 block.
-  const bool out_f32 = p.flags & RTP_GEMM_OUT_F32;
-  const bool cin_f32 = p.flags & RTP_GEMM_CIN_F32;
-  const bool relu = p.flags & RTP_GEMM_RELU;
-  char* cbase = p.c_out + (grp * p.c_sg + zo * p.c_so + zi * p.c_si) * (out_f32 ? 4 : (long)sizeof(T));
-  const char* cin =
-      p.c_in ? p.c_in + (grp * p.cin_sg + zo * p.cin_so + zi * p.cin_si) * (cin_f32 ? 4 : (long)sizeof(T)) : nullptr;
-  const T* bias =
-      p.bias ? reinterpret_cast<const T*>(p.bias) + grp * p.bias_sg + zo * p.bias_so + zi * p.bias_si : nullptr;
-  const T* gate =
-      p.gate ? reinterpret_cast<const T*>(p.gate) + grp * p.gate_sg + zo * p.gate_so + zi * p.gate_si : nullptr;
+  store_tile<T, MT, NT, WM, WN>(p, acc, t.m0, t.n0, wm, wn, li, g, grp, zo, zi);
+}
 
+// ---------------------------------------------------------------------------------------------
+// Direct-to-LDS pipeline (the fast path).  Slabs go global -> LDS with global_load_lds_dwordx4: no
+// staging registers, NSTAGE LDS stages, and the loads of NSTAGE-1 slabs stay in flight while the MFMAs of
+// the current slab run.  The compiler does not order these asynchronous LDS writes against later LDS
+// reads, so the kernel does it by hand: before the workgroup barrier that ends phase kt every wave waits
+// until its own loads of slab kt+1 have landed (s_waitcnt vmcnt(N), loads retire in order) and until its
+// LDS reads of slab kt are done (lgkmcnt(0)); the stage refilled in phase kt+1 is the one read in phase kt.
+//
+// A wave-level load writes 64 lanes x 16 B = 1 KiB of consecutive LDS, so rows cannot be padded.  For a
+// k-contiguous operand (LDS [row][128 B]) bank conflicts are avoided by an XOR swizzle instead: the
+// 16-byte chunk c of row r is kept at chunk position c ^ (r & 7); the lane that fills position cp of row
+// r fetches chunk cp ^ (r & 7) from global memory.  A row-contiguous operand is kept as [k][rows].
+// Vectors beyond the contraction length are fetched from a 16-byte block of zeros; rows beyond the
+// operand are clamped (they only feed accumulators that are never stored).
+__device__ __attribute__((aligned(16))) unsigned int g_zero16[4] = {0u, 0u, 0u, 0u};
+
+// s_waitcnt with vmcnt = VM, lgkmcnt = 0, expcnt untouched (gfx9 encoding).
+#define RTP_WAIT_VM_LGKM0(VM) __builtin_amdgcn_s_waitcnt(((VM)&0xF) | (((VM) >> 4) << 14) | (0x7 << 4))
+
+typedef __attribute__((address_space(1))) const void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+template <typename T, int R, bool KC>
+struct DmaOperand {
+  static constexpr int VEC = 16 / sizeof(T);
+  static constexpr int NI = R / 32;               // load instructions per wave and slab
+  static constexpr int BYTES = R * kSlabBytes;    // one stage of this operand
+  static constexpr int LINE = R * (int)sizeof(T); // bytes of one k line when rows are contiguous
+  const T* ptr[NI];
+  int koff[NI];
+
+  __device__ __forceinline__ void init(const T* base, long ld, int row0, int rows, int wave, int lane) {
 #pragma unroll
-  for (int i = 0; i < MT; ++i) {
-#pragma unroll
-    for (int j = 0; j < NT; ++j) {
-      const int col = t.n0 + wn * WN + j * 32 + li;
-      if (col >= p.n) continue;
-      float bv = 0.0f;
-      if (bias) {
-        // a bias per K segment (row-parallel shards each carry bias/ws): summed in segment order
-        const int nb_seg = p.bias_sk ? p.ksegs : 1;
-        for (int sgm = 0; sgm < nb_seg; ++sgm) bv += to_f32(bias[sgm * p.bias_sk + col]);
-      }
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = t.m0 + wm * WM + i * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
-        if (row >= p.m) continue;
-        float v = p.alpha * acc[i][j][r];
-        if (cin) {
-          const long off = (long)row * p.ld_cin + col;
-          v += cin_f32 ? reinterpret_cast<const float*>(cin)[off] : to_f32(reinterpret_cast<const T*>(cin)[off]);
-        }
-        v += bv;
-        if (relu) v = fmaxf(v, 0.0f);
-        if (gate) v = to_f32(gate[(long)row * p.ld_gate + col]) > 0.0f ? v : 0.0f;
-        const long off = (long)row * p.ldc + col;
-        if (out_f32)
-          reinterpret_cast<float*>(cbase)[off] = v;
-        else
-          reinterpret_cast<T*>(cbase)[off] = from_f32<T>(v);
+    for (int i = 0; i < NI; ++i) {
+      const int j = wave * NI + i;  // which KiB of the stage
+      if (KC) {
+        const int row = j * 8 + (lane >> 3);
+        const int c = (lane & 7) ^ (row & 7);
+        const int rr = row0 + row < rows ? row0 + row : rows - 1;
+        ptr[i] = base + (long)rr * ld + c * VEC;
+        koff[i] = c * VEC;
+      } else {
+        const int byte = lane * 16;
+        const int kl = j * (1024 / LINE) + byte / LINE;
+        int rr = row0 + (byte % LINE) / (int)sizeof(T);
+        if (rr + VEC > rows) rr = 0;
+        ptr[i] = base + (long)kl * ld + rr;
+        koff[i] = kl;
       }
     }
   }
+
+  // off: element offset of the slab (K segment stride + k0, or k0 lines), k0: first k of the slab.
+  __device__ __forceinline__ void issue(char* stage, long off, int k0, int kdim, int wave) const {
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const T* src = ptr[i] + off;
+      if (k0 + koff[i] >= kdim) src = reinterpret_cast<const T*>(g_zero16);
+      // Issued as inline assembly on purpose: the compiler's own bookkeeping for this instruction makes
+      // LDS reads wait for ALL outstanding loads once per pipeline round; the kernel's explicit
+      // s_waitcnt + barrier protocol (see above) is the ordering that counts.
+      const unsigned lds_addr = (unsigned)(uintptr_t)(lptr_t)(stage + (wave * NI + i) * 1024);
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                   :
+                   : "s"(lds_addr), "v"(src)
+                   : "memory", "m0");
+    }
+  }
+};
+
+template <typename T, int R, bool KC>
+__device__ __forceinline__ Frag<T> read_frag_dma(const char* st, int row, int ks, int g) {
+  constexpr int VEC = 16 / sizeof(T);
+  constexpr int LINE = R * (int)sizeof(T);
+  union {
+    uint4 q;
+    T e[VEC];
+    Frag<T> f;
+  } u;
+  if (KC) {
+    u.q = *reinterpret_cast<const uint4*>(st + row * kSlabBytes + (((2 * ks + g) ^ (row & 7)) << 4));
+  } else {
+    const char* p = st + (2 * ks + g) * VEC * LINE + row * (int)sizeof(T);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) u.e[e] = *reinterpret_cast<const T*>(p + e * LINE);
+  }
+  return u.f;
+}
+
+template <typename T, int BM, int BN, bool AKC, bool BKC, int NSTAGE>
+__global__ __launch_bounds__(kThreads) void gemm_dma_kernel(GemmArgs p) {
+  using DA = DmaOperand<T, BM, AKC>;
+  using DB = DmaOperand<T, BN, BKC>;
+  constexpr int BK = kSlabBytes / sizeof(T);
+  constexpr int WM = BM / 2, WN = BN / 2, MT = WM / 32, NT = WN / 32;
+  constexpr int STAGE = DA::BYTES + DB::BYTES;
+  constexpr int D = NSTAGE - 1;            // slabs in flight
+  constexpr int NI = DA::NI + DB::NI;      // loads per wave and slab
+  static_assert((D - 1) * NI < 64, "vmcnt is a 6-bit counter");
+  // One __shared__ array per stage, always addressed with a compile-time stage index: distinct arrays
+  // let the compiler see that LDS reads of one stage do not alias the asynchronous writes into another,
+  // so it does not make every LDS read wait for all outstanding loads.
+  static_assert(NSTAGE >= 2 && NSTAGE <= 5, "2..5 LDS stages");
+  __shared__ __attribute__((aligned(1024))) char st0[STAGE];
+  __shared__ __attribute__((aligned(1024))) char st1[STAGE];
+  __shared__ __attribute__((aligned(1024))) char st2[NSTAGE > 2 ? STAGE : 16];
+  __shared__ __attribute__((aligned(1024))) char st3[NSTAGE > 3 ? STAGE : 16];
+  __shared__ __attribute__((aligned(1024))) char st4[NSTAGE > 4 ? STAGE : 16];
+  auto stage = [&](auto S) -> char* {
+    constexpr int s_ = decltype(S)::value % NSTAGE;
+    if constexpr (s_ == 0) return st0;
+    else if constexpr (s_ == 1) return st1;
+    else if constexpr (s_ == 2) return st2;
+    else if constexpr (s_ == 3) return st3;
+    else return st4;
+  };
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int li = lane & 31, g = lane >> 5;
+
+  int bid = blockIdx.x;
+  const int nb = p.tiles_m * p.tiles_n;
+  if ((nb & 7) == 0) bid = (bid & 7) * (nb >> 3) + (bid >> 3);
+  const int m0 = (bid / p.tiles_n) * BM;
+  const int n0 = (bid % p.tiles_n) * BN;
+  const int grp = blockIdx.y / p.batch, zb = blockIdx.y % p.batch;
+  const long zo = zb / p.zdiv, zi = zb % p.zdiv;
+  const T* A = reinterpret_cast<const T*>(p.a) + grp * p.a_sg + zo * p.a_so + zi * p.a_si;
+  const T* B = reinterpret_cast<const T*>(p.b) + grp * p.b_sg + zo * p.b_so + zi * p.b_si;
+
+  DA da;
+  DB db;
+  da.init(A, p.lda, m0, p.m, wave, lane);
+  db.init(B, p.ldb, n0, p.n, wave, lane);
+  const int nk_seg = (p.k + BK - 1) / BK;
+  const int nk = nk_seg * p.ksegs;
+
+  // issue(S, slab): start the loads of `slab` into stage S (S == slab % NSTAGE).
+  auto issue = [&](auto S, int slab) {
+    const int seg = slab / nk_seg;
+    const int k0 = (slab - seg * nk_seg) * BK;
+    char* st = stage(S);
+    da.issue(st, seg * p.a_sk + (AKC ? (long)k0 : (long)k0 * p.lda), k0, p.k, wave);
+    db.issue(st + DA::BYTES, seg * p.b_sk + (BKC ? (long)k0 : (long)k0 * p.ldb), k0, p.k, wave);
+  };
+
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  auto compute = [&](auto S) {
+    const char* sa = stage(S);
+    const char* sb = sa + DA::BYTES;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      Frag<T> fa[MT], fb[NT];
+#pragma unroll
+      for (int i = 0; i < MT; ++i) fa[i] = read_frag_dma<T, BM, AKC>(sa, wm * WM + i * 32 + li, ks, g);
+#pragma unroll
+      for (int j = 0; j < NT; ++j) fb[j] = read_frag_dma<T, BN, BKC>(sb, wn * WN + j * 32 + li, ks, g);
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) mma(fa[i], fb[j], acc[i][j]);
+    }
+  };
+
+  // Phase for slab k held in stage S: refill the stage read in the previous phase with slab k+D, run the
+  // MFMAs of slab k, wait for slab k+1 (the oldest of the D slabs in flight) and for this wave's LDS reads.
+  auto steady_phase = [&](auto S, int k) {
+    issue(std::integral_constant<int, (decltype(S)::value + D) % NSTAGE>{}, k + D);
+    compute(S);
+    RTP_WAIT_VM_LGKM0((D - 1) * NI);
+    __builtin_amdgcn_s_barrier();
+  };
+  auto drain_phase = [&](auto S, int k) {
+    if (k >= nk) return;
+    if (k + D < nk) {
+      issue(std::integral_constant<int, (decltype(S)::value + D) % NSTAGE>{}, k + D);
+      compute(S);
+      RTP_WAIT_VM_LGKM0((D - 1) * NI);
+    } else {
+      compute(S);
+      RTP_WAIT_VM_LGKM0(0);
+    }
+    __builtin_amdgcn_s_barrier();
+  };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  using I3 = std::integral_constant<int, 3>;
+  using I4 = std::integral_constant<int, 4>;
+
+  // Prologue: slabs 0..D-1 in flight, slab 0 landed.
+  if (0 < nk) issue(I0{}, 0);
+  if (D > 1 && 1 < nk) issue(I1{}, 1);
+  if (D > 2 && 2 < nk) issue(I2{}, 2);
+  if (D > 3 && 3 < nk) issue(I3{}, 3);
+  if (nk >= D) {
+    RTP_WAIT_VM_LGKM0((D - 1) * NI);
+  } else {
+    RTP_WAIT_VM_LGKM0(0);
+  }
+  __builtin_amdgcn_s_barrier();
+
+  int kt = 0;
+  for (; kt + NSTAGE - 1 + D < nk; kt += NSTAGE) {  // every phase of the round may issue
+    steady_phase(I0{}, kt);
+    steady_phase(I1{}, kt + 1);
+    if (NSTAGE > 2) steady_phase(I2{}, kt + 2);
+    if (NSTAGE > 3) steady_phase(I3{}, kt + 3);
+    if (NSTAGE > 4) steady_phase(I4{}, kt + 4);
+  }
+  for (; kt < nk; kt += NSTAGE) {
+    drain_phase(I0{}, kt);
+    drain_phase(I1{}, kt + 1);
+    if (NSTAGE > 2) drain_phase(I2{}, kt + 2);
+    if (NSTAGE > 3) drain_phase(I3{}, kt + 3);
+    if (NSTAGE > 4) drain_phase(I4{}, kt + 4);
+  }
+
+  store_tile<T, MT, NT, WM, WN>(p, acc, m0, n0, wm, wn, li, g, grp, zo, zi);
+}
+
+template <typename T, int BM, int BN, int NSTAGE>
+static int launch_dma(hipStream_t s, const GemmArgs& a, bool akc, bool bkc, dim3 grid) {
+  if (akc && bkc)
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, true, NSTAGE>), grid, dim3(kThreads), 0, s, a);
+  else if (akc && !bkc)
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, false, NSTAGE>), grid, dim3(kThreads), 0, s, a);
+  else if (!akc && bkc)
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, true, NSTAGE>), grid, dim3(kThreads), 0, s, a);
+  else
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, false, NSTAGE>), grid, dim3(kThreads), 0, s, a);
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
 }
 
 template <typename T, int BM, int BN, int DEPTH, bool FAST>
@@ -417,11 +702,11 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   if (!fast) return launch_layout<T, 64, 64, 1, false>(s, a, akc, bkc, grid);
   switch (shape) {
     case 0:
-      return launch_layout<T, 128, 128, 2, true>(s, a, akc, bkc, grid);
+      return launch_dma<T, 128, 128, 4>(s, a, akc, bkc, grid);
     case 1:
-      return launch_layout<T, 128, 64, 3, true>(s, a, akc, bkc, grid);
+      return launch_dma<T, 128, 64, 5>(s, a, akc, bkc, grid);
     default:
-      return launch_layout<T, 64, 64, 3, true>(s, a, akc, bkc, grid);
+      return launch_dma<T, 64, 64, 4>(s, a, akc, bkc, grid);
   }
 }
 
