@@ -430,19 +430,34 @@ struct DmaOperand {
   }
 };
 
+typedef short short4_t __attribute__((ext_vector_type(4)));
+
+// rowbase: first tile row of the 32-row MFMA block; the lane's own row is rowbase + lane % 32.
 template <typename T, int R, bool KC>
-__device__ __forceinline__ Frag<T> read_frag_dma(const char* st, int row, int ks, int g) {
+__device__ __forceinline__ Frag<T> read_frag_dma(const char* st, int rowbase, int lane, int ks) {
   constexpr int VEC = 16 / sizeof(T);
   constexpr int LINE = R * (int)sizeof(T);
+  const int li = lane & 31, g = lane >> 5;
   union {
     uint4 q;
     T e[VEC];
+    short4_t h[2];
     Frag<T> f;
   } u;
   if (KC) {
+    const int row = rowbase + li;
     u.q = *reinterpret_cast<const uint4*>(st + row * kSlabBytes + (((2 * ks + g) ^ (row & 7)) << 4));
+  } else if (sizeof(T) == 2) {
+    // LDS holds [k][rows] (rows contiguous) but the MFMA wants 8 consecutive k per lane.  gfx950's
+    // transposing LDS read does the 16-bit transpose inside each group of 16 lanes: lane s of a group
+    // supplies the address of 4 consecutive rows at k line (s / 4); the group then receives, in lane j,
+    // the 4 consecutive k of row (4 * (s % 4) ... ) + j.  Two such reads give the 8 k of the lane's row.
+    const int s16 = lane & 15, blk = (lane >> 4) & 1;
+    const char* p = st + ((2 * ks + g) * 8 + (s16 >> 2)) * LINE + (rowbase + 16 * blk + 4 * (s16 & 3)) * 2;
+    u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(p));
+    u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(p + 4 * LINE));
   } else {
-    const char* p = st + (2 * ks + g) * VEC * LINE + row * (int)sizeof(T);
+    const char* p = st + (2 * ks + g) * VEC * LINE + (rowbase + li) * (int)sizeof(T);
 #pragma unroll
     for (int e = 0; e < VEC; ++e) u.e[e] = *reinterpret_cast<const T*>(p + e * LINE);
   }
@@ -517,20 +532,29 @@ __global__ __launch_bounds__(kThreads) void gemm_dma_kernel(GemmArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
+  // The fragments of k-step ks+1 are read from LDS while the MFMAs of k-step ks run (two register sets).
   auto compute = [&](auto S) {
     const char* sa = stage(S);
     const char* sb = sa + DA::BYTES;
+    Frag<T> fa[2][MT], fb[2][NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) fa[0][i] = read_frag_dma<T, BM, AKC>(sa, wm * WM + i * 32, lane, 0);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) fb[0][j] = read_frag_dma<T, BN, BKC>(sb, wn * WN + j * 32, lane, 0);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      Frag<T> fa[MT], fb[NT];
+      if (ks + 1 < 4) {
 #pragma unroll
-      for (int i = 0; i < MT; ++i) fa[i] = read_frag_dma<T, BM, AKC>(sa, wm * WM + i * 32 + li, ks, g);
+        for (int i = 0; i < MT; ++i)
+          fa[(ks + 1) & 1][i] = read_frag_dma<T, BM, AKC>(sa, wm * WM + i * 32, lane, ks + 1);
 #pragma unroll
-      for (int j = 0; j < NT; ++j) fb[j] = read_frag_dma<T, BN, BKC>(sb, wn * WN + j * 32 + li, ks, g);
+        for (int j = 0; j < NT; ++j)
+          fb[(ks + 1) & 1][j] = read_frag_dma<T, BN, BKC>(sb, wn * WN + j * 32, lane, ks + 1);
+      }
 #pragma unroll
       for (int i = 0; i < MT; ++i)
 #pragma unroll
-        for (int j = 0; j < NT; ++j) mma(fa[i], fb[j], acc[i][j]);
+        for (int j = 0; j < NT; ++j) mma(fa[ks & 1][i], fb[ks & 1][j], acc[i][j]);
     }
   };
 
