@@ -92,7 +92,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--graph", action="store_true", help="replay the step from a captured HIP graph")
+    ap.add_argument("--no-graph", dest="graph", action="store_false",
+                    help="launch every kernel eagerly instead of replaying the step from a captured HIP graph")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU's throughput: this build runs every rotation shard on a single MI355X and "
@@ -101,7 +102,7 @@ def main():
 
     import torch
     import torch.nn.functional as F
-    from rtp_amd import _lib, rotated_weight_bytes, staging_bytes
+    from rtp_amd import _lib, ring, rotated_weight_bytes, staging_bytes
     from rtp_amd.optim import RotatedSGD
 
     dev = torch.device("cuda", 0)
@@ -121,18 +122,27 @@ def main():
         loss = F.cross_entropy(logits.float().view(-1, c["vocab"]), tgt.view(-1))
         loss.backward()
         opt.step()
-        loss_box[0] = loss
+        loss_box[0] = loss.detach()  # detached: a live autograd graph would pin last step's AccumulateGrad nodes
 
-    for _ in range(max(args.warmup, 1)):
-        step()
+    # Warm-up on a side stream (the documented recipe for whole-step graph capture: autograd's gradient
+    # accumulators remember the stream they were created on, and it must not be the default stream).
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(max(args.warmup, 1)):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
+    ring.fence(dev)
     first_loss = float(loss_box[0])
 
     run = step
     if args.graph:
+        # The whole step (both streams of the rotation included) recorded once into a HIP graph and replayed.
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
             step()
+        ring.fence(dev)  # the ring's last fence was recorded inside the capture; re-arm it for eager use
         run = g.replay
         run()
         torch.cuda.synchronize()

@@ -629,6 +629,64 @@ static int launch_dma(hipStream_t s, const GemmArgs& a, bool akc, bool bkc, dim3
   return RTP_OK;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Tiny batched problems (one attention head at sequence length <= 64: 32 x 32 x 64 per (batch, head)):
+// one wavefront per 32 x 32 output block, operands read straight from global memory into MFMA
+// fragments (no LDS, no barriers).  Thousands of independent wavefronts hide the load latency.
+template <typename T, bool AKC, bool BKC>
+__global__ __launch_bounds__(kThreads) void gemm_tiny_kernel(GemmArgs p, long nblocks) {
+  constexpr int VEC = 16 / sizeof(T);
+  const int lane = threadIdx.x & 63;
+  const long blk = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (blk >= nblocks) return;
+  const int li = lane & 31, g = lane >> 5;
+  const int tiles = p.tiles_m * p.tiles_n;
+  const long z = blk / tiles;
+  const int tile = (int)(blk % tiles);
+  const int m0 = (tile / p.tiles_n) * 32, n0 = (tile % p.tiles_n) * 32;
+  const int grp = (int)(z / p.batch), zb = (int)(z % p.batch);
+  const long zo = zb / p.zdiv, zi = zb % p.zdiv;
+  const T* A = reinterpret_cast<const T*>(p.a) + grp * p.a_sg + zo * p.a_so + zi * p.a_si;
+  const T* B = reinterpret_cast<const T*>(p.b) + grp * p.b_sg + zo * p.b_so + zi * p.b_si;
+
+  f32x16 acc[1][1];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[0][0][r] = 0.0f;
+
+  // fragment of `rows`-row operand X for this lane's row and the VEC k values starting at k
+  auto frag = [&](const T* X, long ld, bool kc, bool vec_ok, int row, int rows, int k) {
+    union {
+      uint4 q;
+      T e[VEC];
+      Frag<T> f;
+    } u;
+    if (kc) {
+      const T* src = X + (long)row * ld + k;
+      if (vec_ok && row < rows && k + VEC <= p.k) {
+        u.q = *reinterpret_cast<const uint4*>(src);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) u.e[e] = (row < rows && k + e < p.k) ? src[e] : (T)0.0f;
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) u.e[e] = (row < rows && k + e < p.k) ? X[(long)(k + e) * ld + row] : (T)0.0f;
+    }
+    return u.f;
+  };
+
+  for (int seg = 0; seg < p.ksegs; ++seg) {
+    const T* As = A + seg * p.a_sk;
+    const T* Bs = B + seg * p.b_sk;
+    for (int k0 = 0; k0 < p.k; k0 += 2 * VEC) {
+      const Frag<T> fa = frag(As, p.lda, AKC, p.vec_a, m0 + li, p.m, k0 + g * VEC);
+      const Frag<T> fb = frag(Bs, p.ldb, BKC, p.vec_b, n0 + li, p.n, k0 + g * VEC);
+      mma(fa, fb, acc[0][0]);
+    }
+  }
+  store_tile<T, 1, 1, 32, 32>(p, acc, m0, n0, 0, 0, li, g, grp, zo, zi);
+}
+
 template <typename T, int BM, int BN, int DEPTH, bool FAST>
 static int launch_layout(hipStream_t s, const GemmArgs& a, bool akc, bool bkc, dim3 grid) {
   if (akc && bkc)
@@ -694,8 +752,35 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   const bool fast = a.vec_a && a.vec_b && ((akc || bkc) ? mult(d->k, VEC) : true) && (akc || mult(d->m, VEC)) &&
                     (bkc || mult(d->n, VEC)) && d->k > 0;
   const int64_t nz = d->batch * d->groups;
+  if (d->m <= 64 && d->n <= 64 && d->k * d->ksegs <= 256) {
+    // one wavefront per 32 x 32 block
+    a.tiles_m = (int)ceil_div(d->m, 32);
+    a.tiles_n = (int)ceil_div(d->n, 32);
+    const int64_t nblocks = (int64_t)a.tiles_m * a.tiles_n * nz;
+    RTP_REQUIRE(ceil_div(nblocks, 4) < (1ll << 31), "gemm grid too large");
+    static const char* const tiny_names[2][2][2] = {
+        {{"gemm_f32_tiny_rc_rc", "gemm_f32_tiny_rc_kc"}, {"gemm_f32_tiny_kc_rc", "gemm_f32_tiny_kc_kc"}},
+        {{"gemm_bf16_tiny_rc_rc", "gemm_bf16_tiny_rc_kc"}, {"gemm_bf16_tiny_kc_rc", "gemm_bf16_tiny_kc_kc"}}};
+    const double mn_ = (double)d->m * (double)d->n * (double)nz, kk_ = (double)d->k * (double)d->ksegs;
+    ProfileScope prof(s, tiny_names[sizeof(T) == 2][akc][bkc], 2.0 * mn_ * kk_,
+                      ((double)d->m + (double)d->n) * kk_ * nz * sizeof(T) + mn_ * sizeof(T));
+    dim3 tgrid((unsigned)ceil_div(nblocks, 4));
+    if (akc && bkc)
+      hipLaunchKernelGGL((gemm_tiny_kernel<T, true, true>), tgrid, dim3(kThreads), 0, s, a, (long)nblocks);
+    else if (akc && !bkc)
+      hipLaunchKernelGGL((gemm_tiny_kernel<T, true, false>), tgrid, dim3(kThreads), 0, s, a, (long)nblocks);
+    else if (!akc && bkc)
+      hipLaunchKernelGGL((gemm_tiny_kernel<T, false, true>), tgrid, dim3(kThreads), 0, s, a, (long)nblocks);
+    else
+      hipLaunchKernelGGL((gemm_tiny_kernel<T, false, false>), tgrid, dim3(kThreads), 0, s, a, (long)nblocks);
+    RTP_LAUNCH_CHECK();
+    return RTP_OK;
+  }
   int shape = 2;
   for (int i = 0; fast && i < 3; ++i) {
+    // never a tile that is mostly padding: a 32 x 32 problem (one attention head at seq 32) stays at 64 x 64
+    if (kShapes[i].bm > 64 && kShapes[i].bm > ceil_div(d->m, 64) * 64) continue;
+    if (kShapes[i].bn > 64 && kShapes[i].bn > ceil_div(d->n, 64) * 64) continue;
     const int64_t tiles = ceil_div(d->m, kShapes[i].bm) * ceil_div(d->n, kShapes[i].bn) * nz;
     if (tiles >= 200) {
       shape = i;

@@ -22,6 +22,44 @@ __global__ __launch_bounds__(256) void sgd_kernel(float* master, const T* grad, 
   }
 }
 
+// Four parameters per lane and iteration: 16-byte master accesses, 8- or 16-byte gradient / shadow accesses.
+template <typename T>
+__global__ __launch_bounds__(256) void sgd_vec4_kernel(float4* master, const T* grad, T* shadow, long n4, float lr,
+                                                       float clip) {
+  const long stride = (long)gridDim.x * blockDim.x;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+    union {
+      T e[4];
+      uint2 u2;
+      uint4 u4;
+    } g, sh;
+    if (sizeof(T) == 2)
+      g.u2 = reinterpret_cast<const uint2*>(grad)[i];
+    else
+      g.u4 = reinterpret_cast<const uint4*>(grad)[i];
+    float4 w = master[i];
+    float* wf = reinterpret_cast<float*>(&w);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float gv = to_f32(g.e[e]);
+      if (clip > 0.0f) gv = fminf(fmaxf(gv, -clip), clip);
+      {
+#pragma clang fp contract(off)
+        const float step = lr * gv;
+        wf[e] = wf[e] - step;
+      }
+      sh.e[e] = from_f32<T>(wf[e]);
+    }
+    master[i] = w;
+    if (shadow) {
+      if (sizeof(T) == 2)
+        reinterpret_cast<uint2*>(shadow)[i] = sh.u2;
+      else
+        reinterpret_cast<uint4*>(shadow)[i] = sh.u4;
+    }
+  }
+}
+
 template <typename S, typename D>
 __global__ __launch_bounds__(256) void cast_kernel(const S* src, D* dst, long n) {
   const long stride = (long)gridDim.x * blockDim.x;
@@ -40,8 +78,18 @@ extern "C" int rtp_sgd_step(void* stream, int dtype, float* master, const void* 
   RTP_REQUIRE(n >= 0, "rtp_sgd_step: negative length");
   if (n == 0) return RTP_OK;
   hipStream_t s = (hipStream_t)stream;
+  const size_t tsz = dtype == RTP_F32 ? 4 : 2;
+  const bool vec4 = n % 4 == 0 && (uintptr_t)master % 16 == 0 && (uintptr_t)grad % (4 * tsz) == 0 &&
+                    (!shadow || (uintptr_t)shadow % (4 * tsz) == 0);
   ProfileScope prof(s, "sgd_step", 2.0 * (double)n, (double)n * (8.0 + (dtype == RTP_F32 ? 4 : 2) * (shadow ? 2.0 : 1.0)));
-  if (dtype == RTP_F32)
+  if (dtype != RTP_F32 && dtype != RTP_BF16) return fail(RTP_ERR_ARG, "rtp_sgd_step: unknown dtype %d", dtype);
+  if (vec4 && dtype == RTP_F32)
+    hipLaunchKernelGGL(sgd_vec4_kernel<float>, dim3(flat_grid(n / 4)), dim3(256), 0, s, (float4*)master,
+                       (const float*)grad, (float*)shadow, (long)(n / 4), lr, clip);
+  else if (vec4)
+    hipLaunchKernelGGL(sgd_vec4_kernel<bf16_t>, dim3(flat_grid(n / 4)), dim3(256), 0, s, (float4*)master,
+                       (const bf16_t*)grad, (bf16_t*)shadow, (long)(n / 4), lr, clip);
+  else if (dtype == RTP_F32)
     hipLaunchKernelGGL(sgd_kernel<float>, dim3(flat_grid(n)), dim3(256), 0, s, master, (const float*)grad,
                        (float*)shadow, (long)n, lr, clip);
   else if (dtype == RTP_BF16)
