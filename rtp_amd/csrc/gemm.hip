@@ -15,6 +15,7 @@
 // ring of register buffers, which is what hides HBM/L2 latency when only one workgroup fits a CU.
 #include "common.h"
 
+#include <cstdlib>
 #include <type_traits>
 
 namespace rtp {
@@ -39,6 +40,7 @@ struct GemmArgs {
   int flags;
   int vec_a, vec_b;
   int tiles_m, tiles_n;
+  int xg, xm, xn;  // split of the (batch*groups, tiles_m, tiles_n) space over the 8 XCDs; xg == 0: none
 };
 
 constexpr int kThreads = 256;
@@ -362,11 +364,12 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs p) {
 
 // ---------------------------------------------------------------------------------------------
 // Direct-to-LDS pipeline (the fast path).  Slabs go global -> LDS with global_load_lds_dwordx4: no
-// staging registers, NSTAGE LDS stages, and the loads of NSTAGE-1 slabs stay in flight while the MFMAs of
-// the current slab run.  The compiler does not order these asynchronous LDS writes against later LDS
-// reads, so the kernel does it by hand: before the workgroup barrier that ends phase kt every wave waits
-// until its own loads of slab kt+1 have landed (s_waitcnt vmcnt(N), loads retire in order) and until its
-// LDS reads of slab kt are done (lgkmcnt(0)); the stage refilled in phase kt+1 is the one read in phase kt.
+// staging registers, NSTAGE LDS stages, up to NSTAGE-1 slabs in flight while the MFMAs of the current slab
+// run.  The compiler does not order these asynchronous LDS writes against later LDS reads, so the kernel
+// does it by hand: in the middle of the phase of slab k every wave waits until its own loads of slab k+1
+// have landed (s_waitcnt vmcnt(N), loads retire in order) and then meets the workgroup barrier; after the
+// barrier slab k+1 may be read, and the stage of slab k-1 (whose fragments every wave consumed in its
+// previous phase) is refilled.
 //
 // A wave-level load writes 64 lanes x 16 B = 1 KiB of consecutive LDS, so rows cannot be padded.  For a
 // k-contiguous operand (LDS [row][128 B]) bank conflicts are avoided by an XOR swizzle instead: the
@@ -374,18 +377,37 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs p) {
 // r fetches chunk cp ^ (r & 7) from global memory.  A row-contiguous operand is kept as [k][rows].
 // Vectors beyond the contraction length are fetched from a 16-byte block of zeros; rows beyond the
 // operand are clamped (they only feed accumulators that are never stored).
+//
+// The workgroup has NW >= 4 waves: waves 0..3 run the MFMAs, and ALL NW waves share the loads, so the address
+// arithmetic and the issue slots of the loads are spread over more wavefronts.
 __device__ __attribute__((aligned(16))) unsigned int g_zero16[4] = {0u, 0u, 0u, 0u};
 
 // s_waitcnt with vmcnt = VM, lgkmcnt = 0, expcnt untouched (gfx9 encoding).
 #define RTP_WAIT_VM_LGKM0(VM) __builtin_amdgcn_s_waitcnt(((VM)&0xF) | (((VM) >> 4) << 14) | (0x7 << 4))
+// s_waitcnt with vmcnt = VM only (expcnt and lgkmcnt untouched).
+#define RTP_WAIT_VM(VM) __builtin_amdgcn_s_waitcnt(((VM)&0xF) | (((VM) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
 
 typedef __attribute__((address_space(1))) const void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 
-template <typename T, int R, bool KC>
+// LDS has 64 four-byte banks (256 bytes per clock).  Swizzles keep the lanes that are served in one clock on
+// different banks:
+//  * k-contiguous operand, [row][128 B]: 16 consecutive rows read the same 16-byte chunk c; row r keeps it at
+//    chunk position c ^ ((r >> 1) & 7), which together with the row's parity (rows alternate between the two
+//    128-byte halves of the bank space) gives 16 different 16-byte bank slots.
+//  * row-contiguous 16-bit operand, [k][rows]: a transposing read touches 4 consecutive k lines x 64 bytes; the
+//    chunk index inside k line kl is XORed with rc_swizzle(kl) so that the 4 lines fall on different slots.
+template <typename T, int R>
+__device__ __forceinline__ constexpr int rc_swizzle(int kl) {
+  if (sizeof(T) != 2) return 0;
+  return R >= 128 ? (kl & 3) << 2 : ((kl >> 1) & 1) << 2;
+}
+
+template <typename T, int R, bool KC, int NW>
 struct DmaOperand {
   static constexpr int VEC = 16 / sizeof(T);
-  static constexpr int NI = R / 32;               // load instructions per wave and slab
+  static_assert((R / 8) % NW == 0, "every wave issues the same number of loads");
+  static constexpr int NI = R / 8 / NW;           // load instructions per wave and slab
   static constexpr int BYTES = R * kSlabBytes;    // one stage of this operand
   static constexpr int LINE = R * (int)sizeof(T); // bytes of one k line when rows are contiguous
   const T* ptr[NI];
@@ -397,14 +419,15 @@ struct DmaOperand {
       const int j = wave * NI + i;  // which KiB of the stage
       if (KC) {
         const int row = j * 8 + (lane >> 3);
-        const int c = (lane & 7) ^ (row & 7);
+        const int c = (lane & 7) ^ ((row >> 1) & 7);
         const int rr = row0 + row < rows ? row0 + row : rows - 1;
         ptr[i] = base + (long)rr * ld + c * VEC;
         koff[i] = c * VEC;
       } else {
         const int byte = lane * 16;
         const int kl = j * (1024 / LINE) + byte / LINE;
-        int rr = row0 + (byte % LINE) / (int)sizeof(T);
+        const int chunk = ((byte % LINE) >> 4) ^ rc_swizzle<T, R>(kl);  // which 16 bytes of the k line land here
+        int rr = row0 + chunk * VEC;
         if (rr + VEC > rows) rr = 0;
         ptr[i] = base + (long)kl * ld + rr;
         koff[i] = kl;
@@ -412,21 +435,29 @@ struct DmaOperand {
     }
   }
 
-  // off: element offset of the slab (K segment stride + k0, or k0 lines), k0: first k of the slab.
-  __device__ __forceinline__ void issue(char* stage, long off, int k0, int kdim, int wave) const {
+  // off: element offset of the slab (K segment offset + k0, or k0 lines), k0: first k of the slab.  `tail` is
+  // uniform: only the last slab of a K segment can reach beyond the contraction length, and only then are the
+  // per-vector checks made.
+  __device__ __forceinline__ void issue(char* stage, long off, int k0, int kdim, int wave, bool tail) const {
+    if (tail) {
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      const T* src = ptr[i] + off;
-      if (k0 + koff[i] >= kdim) src = reinterpret_cast<const T*>(g_zero16);
-      // Issued as inline assembly on purpose: the compiler's own bookkeeping for this instruction makes
-      // LDS reads wait for ALL outstanding loads once per pipeline round; the kernel's explicit
-      // s_waitcnt + barrier protocol (see above) is the ordering that counts.
-      const unsigned lds_addr = (unsigned)(uintptr_t)(lptr_t)(stage + (wave * NI + i) * 1024);
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                   :
-                   : "s"(lds_addr), "v"(src)
-                   : "memory", "m0");
+      for (int i = 0; i < NI; ++i) {
+        const T* src = ptr[i] + off;
+        if (k0 + koff[i] >= kdim) src = reinterpret_cast<const T*>(g_zero16);
+        dma(stage + (wave * NI + i) * 1024, src);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NI; ++i) dma(stage + (wave * NI + i) * 1024, ptr[i] + off);
     }
+  }
+
+  // Issued as inline assembly on purpose: the compiler's own bookkeeping for this instruction makes LDS
+  // reads wait for ALL outstanding loads once per pipeline round; the kernel's explicit s_waitcnt + barrier
+  // protocol is the ordering that counts.
+  static __device__ __forceinline__ void dma(char* dst, const T* src) {
+    const unsigned lds_addr = (unsigned)(uintptr_t)(lptr_t)dst;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(src) : "memory");
   }
 };
 
@@ -446,16 +477,20 @@ __device__ __forceinline__ Frag<T> read_frag_dma(const char* st, int rowbase, in
   } u;
   if (KC) {
     const int row = rowbase + li;
-    u.q = *reinterpret_cast<const uint4*>(st + row * kSlabBytes + (((2 * ks + g) ^ (row & 7)) << 4));
+    u.q = *reinterpret_cast<const uint4*>(st + row * kSlabBytes + (((2 * ks + g) ^ ((row >> 1) & 7)) << 4));
   } else if (sizeof(T) == 2) {
     // LDS holds [k][rows] (rows contiguous) but the MFMA wants 8 consecutive k per lane.  gfx950's
     // transposing LDS read does the 16-bit transpose inside each group of 16 lanes: lane s of a group
     // supplies the address of 4 consecutive rows at k line (s / 4); the group then receives, in lane j,
     // the 4 consecutive k of row (4 * (s % 4) ... ) + j.  Two such reads give the 8 k of the lane's row.
     const int s16 = lane & 15, blk = (lane >> 4) & 1;
-    const char* p = st + ((2 * ks + g) * 8 + (s16 >> 2)) * LINE + (rowbase + 16 * blk + 4 * (s16 & 3)) * 2;
-    u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(p));
-    u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(p + 4 * LINE));
+    const int kl = (2 * ks + g) * 8 + (s16 >> 2);         // k line of the first read; the second is kl + 4
+    const int rb = (rowbase + 16 * blk + 4 * (s16 & 3)) * 2;  // byte of the lane's 4 rows inside the k line
+    const int c0 = (rb >> 4) ^ rc_swizzle<T, R>(kl), c1 = (rb >> 4) ^ rc_swizzle<T, R>(kl + 4);
+    const char* p0 = st + kl * LINE + (c0 << 4) + (rb & 15);
+    const char* p1 = st + (kl + 4) * LINE + (c1 << 4) + (rb & 15);
+    u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(p0));
+    u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(p1));
   } else {
     const char* p = st + (2 * ks + g) * VEC * LINE + (rowbase + li) * (int)sizeof(T);
 #pragma unroll
@@ -464,20 +499,19 @@ __device__ __forceinline__ Frag<T> read_frag_dma(const char* st, int rowbase, in
   return u.f;
 }
 
-template <typename T, int BM, int BN, bool AKC, bool BKC, int NSTAGE>
-__global__ __launch_bounds__(kThreads) void gemm_dma_kernel(GemmArgs p) {
-  using DA = DmaOperand<T, BM, AKC>;
-  using DB = DmaOperand<T, BN, BKC>;
+template <typename T, int BM, int BN, bool AKC, bool BKC, int NSTAGE, int NW>
+__global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(GemmArgs p) {
+  using DA = DmaOperand<T, BM, AKC, NW>;
+  using DB = DmaOperand<T, BN, BKC, NW>;
   constexpr int BK = kSlabBytes / sizeof(T);
   constexpr int WM = BM / 2, WN = BN / 2, MT = WM / 32, NT = WN / 32;
   constexpr int STAGE = DA::BYTES + DB::BYTES;
-  constexpr int D = NSTAGE - 1;            // slabs in flight
   constexpr int NI = DA::NI + DB::NI;      // loads per wave and slab
-  static_assert((D - 1) * NI < 64, "vmcnt is a 6-bit counter");
+  static_assert((NSTAGE - 2) * NI < 64, "vmcnt is a 6-bit counter");
   // One __shared__ array per stage, always addressed with a compile-time stage index: distinct arrays
   // let the compiler see that LDS reads of one stage do not alias the asynchronous writes into another,
   // so it does not make every LDS read wait for all outstanding loads.
-  static_assert(NSTAGE >= 2 && NSTAGE <= 5, "2..5 LDS stages");
+  static_assert(NSTAGE >= 3 && NSTAGE <= 5, "3..5 LDS stages");
   __shared__ __attribute__((aligned(1024))) char st0[STAGE];
   __shared__ __attribute__((aligned(1024))) char st1[STAGE];
   __shared__ __attribute__((aligned(1024))) char st2[NSTAGE > 2 ? STAGE : 16];
@@ -495,15 +529,29 @@ __global__ __launch_bounds__(kThreads) void gemm_dma_kernel(GemmArgs p) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
+  const bool computes = wave < 4;  // waves 4.. only load
+  const int wm = (wave >> 1) & 1, wn = wave & 1;
   const int li = lane & 31, g = lane >> 5;
 
-  int bid = blockIdx.x;
-  const int nb = p.tiles_m * p.tiles_n;
-  if ((nb & 7) == 0) bid = (bid & 7) * (nb >> 3) + (bid >> 3);
-  const int m0 = (bid / p.tiles_n) * BM;
-  const int n0 = (bid % p.tiles_n) * BN;
-  const int grp = blockIdx.y / p.batch, zb = blockIdx.y % p.batch;
+  // Workgroups are handed to the 8 XCDs round-robin in launch order, and every XCD has its own L2.  The
+  // host splits the (batch*groups, tiles_m, tiles_n) space into 8 bricks (xg * xm * xn == 8) chosen so that
+  // the operand rows one XCD touches are as few as possible; workgroup `id` works on brick id % 8.
+  int tile_m, tile_n, z;
+  if (p.xg) {
+    const int id = blockIdx.x + blockIdx.y * gridDim.x;
+    const int xcd = id & 7, slot = id >> 3;
+    const int nbk = p.tiles_n / p.xn, mbk = p.tiles_m / p.xm, zbk = (int)gridDim.y / p.xg;
+    tile_n = (xcd % p.xn) * nbk + slot % nbk;
+    tile_m = ((xcd / p.xn) % p.xm) * mbk + (slot / nbk) % mbk;
+    z = (xcd / (p.xn * p.xm)) * zbk + slot / (nbk * mbk);
+  } else {
+    tile_m = blockIdx.x / p.tiles_n;
+    tile_n = blockIdx.x % p.tiles_n;
+    z = blockIdx.y;
+  }
+  const int m0 = tile_m * BM;
+  const int n0 = tile_n * BN;
+  const int grp = z / p.batch, zb = z % p.batch;
   const long zo = zb / p.zdiv, zi = zb % p.zdiv;
   const T* A = reinterpret_cast<const T*>(p.a) + grp * p.a_sg + zo * p.a_so + zi * p.a_si;
   const T* B = reinterpret_cast<const T*>(p.b) + grp * p.b_sg + zo * p.b_so + zi * p.b_si;
@@ -515,13 +563,25 @@ __global__ __launch_bounds__(kThreads) void gemm_dma_kernel(GemmArgs p) {
   const int nk_seg = (p.k + BK - 1) / BK;
   const int nk = nk_seg * p.ksegs;
 
-  // issue(S, slab): start the loads of `slab` into stage S (S == slab % NSTAGE).
-  auto issue = [&](auto S, int slab) {
-    const int seg = slab / nk_seg;
-    const int k0 = (slab - seg * nk_seg) * BK;
+  // Slabs are issued strictly in order; the cursor of the next slab to issue lives in scalar registers
+  // and is advanced by additions only.
+  const long step_a = AKC ? (long)BK : (long)BK * p.lda, step_b = BKC ? (long)BK : (long)BK * p.ldb;
+  const long wrap_a = p.a_sk - nk_seg * step_a, wrap_b = p.b_sk - nk_seg * step_b;
+  int ik0 = 0;
+  long off_a = 0, off_b = 0;
+  auto issue = [&](auto S) {
     char* st = stage(S);
-    da.issue(st, seg * p.a_sk + (AKC ? (long)k0 : (long)k0 * p.lda), k0, p.k, wave);
-    db.issue(st + DA::BYTES, seg * p.b_sk + (BKC ? (long)k0 : (long)k0 * p.ldb), k0, p.k, wave);
+    const bool tail = ik0 + BK > p.k;
+    da.issue(st, off_a, ik0, p.k, wave, tail);
+    db.issue(st + DA::BYTES, off_b, ik0, p.k, wave, tail);
+    ik0 += BK;
+    off_a += step_a;
+    off_b += step_b;
+    if (ik0 >= p.k) {
+      ik0 = 0;
+      off_a += wrap_a;
+      off_b += wrap_b;
+    }
   };
 
   f32x16 acc[MT][NT];
@@ -532,51 +592,60 @@ __global__ __launch_bounds__(kThreads) void gemm_dma_kernel(GemmArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  // The fragments of k-step ks+1 are read from LDS while the MFMAs of k-step ks run (two register sets).
-  auto compute = [&](auto S) {
+  // Fragment registers of one slab in two halves (k-steps 0,1 and 2,3).  While the MFMAs of one half run,
+  // the other half is being read from LDS -- the first half of the NEXT slab during the second half of
+  // this one -- so an LDS read always has a half slab of MFMAs to hide behind.
+  Frag<T> fa[4][MT], fb[4][NT];
+  auto read_half = [&](auto S, auto H) {
+    if (!computes) return;
     const char* sa = stage(S);
     const char* sb = sa + DA::BYTES;
-    Frag<T> fa[2][MT], fb[2][NT];
+    constexpr int h = decltype(H)::value;
 #pragma unroll
-    for (int i = 0; i < MT; ++i) fa[0][i] = read_frag_dma<T, BM, AKC>(sa, wm * WM + i * 32, lane, 0);
+    for (int ks = 2 * h; ks < 2 * h + 2; ++ks) {
 #pragma unroll
-    for (int j = 0; j < NT; ++j) fb[0][j] = read_frag_dma<T, BN, BKC>(sb, wn * WN + j * 32, lane, 0);
+      for (int i = 0; i < MT; ++i) fa[ks][i] = read_frag_dma<T, BM, AKC>(sa, wm * WM + i * 32, lane, ks);
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      if (ks + 1 < 4) {
+      for (int j = 0; j < NT; ++j) fb[ks][j] = read_frag_dma<T, BN, BKC>(sb, wn * WN + j * 32, lane, ks);
+    }
+  };
+  auto mma_half = [&](auto H) {
+    if (!computes) return;
+    constexpr int h = decltype(H)::value;
 #pragma unroll
-        for (int i = 0; i < MT; ++i)
-          fa[(ks + 1) & 1][i] = read_frag_dma<T, BM, AKC>(sa, wm * WM + i * 32, lane, ks + 1);
-#pragma unroll
-        for (int j = 0; j < NT; ++j)
-          fb[(ks + 1) & 1][j] = read_frag_dma<T, BN, BKC>(sb, wn * WN + j * 32, lane, ks + 1);
-      }
+    for (int ks = 2 * h; ks < 2 * h + 2; ++ks)
 #pragma unroll
       for (int i = 0; i < MT; ++i)
 #pragma unroll
-        for (int j = 0; j < NT; ++j) mma(fa[ks & 1][i], fb[ks & 1][j], acc[i][j]);
-    }
+        for (int j = 0; j < NT; ++j) mma(fa[ks][i], fb[ks][j], acc[i][j]);
   };
+  using H0 = std::integral_constant<int, 0>;
+  using H1 = std::integral_constant<int, 1>;
 
-  // Phase for slab k held in stage S: refill the stage read in the previous phase with slab k+D, run the
-  // MFMAs of slab k, wait for slab k+1 (the oldest of the D slabs in flight) and for this wave's LDS reads.
-  auto steady_phase = [&](auto S, int k) {
-    issue(std::integral_constant<int, (decltype(S)::value + D) % NSTAGE>{}, k + D);
-    compute(S);
-    RTP_WAIT_VM_LGKM0((D - 1) * NI);
-    __builtin_amdgcn_s_barrier();
-  };
-  auto drain_phase = [&](auto S, int k) {
-    if (k >= nk) return;
-    if (k + D < nk) {
-      issue(std::integral_constant<int, (decltype(S)::value + D) % NSTAGE>{}, k + D);
-      compute(S);
-      RTP_WAIT_VM_LGKM0((D - 1) * NI);
-    } else {
-      compute(S);
-      RTP_WAIT_VM_LGKM0(0);
+  // Phase of slab k (held in stage S = k % NSTAGE).  On entry slab k is visible to every wave and the first
+  // half of its fragments is in registers.  Slabs up to k + NSTAGE - 2 have been issued.
+  //   read second half of slab k | MFMAs of the first half
+  //   wait for this wave's loads of slab k+1, barrier: slab k+1 is visible and every wave has finished
+  //     reading slab k-1, whose stage is refilled with slab k + NSTAGE - 1
+  //   read first half of slab k+1 | MFMAs of the second half of slab k
+  // STEADY: every condition below is known to hold, so the phase is branch-free.
+  auto phase = [&](auto S, int k, auto STEADY) {
+    constexpr int s_ = decltype(S)::value;
+    constexpr bool steady = decltype(STEADY)::value;
+    if (!steady && k >= nk) return;
+    read_half(S, H1{});
+    mma_half(H0{});
+    if (steady || k + 1 < nk) {
+      if (steady || k + NSTAGE - 2 < nk) {
+        RTP_WAIT_VM((NSTAGE - 3) * NI);
+      } else {
+        RTP_WAIT_VM(0);
+      }
+      __builtin_amdgcn_s_barrier();
+      if (steady || k + NSTAGE - 1 < nk) issue(std::integral_constant<int, (s_ + NSTAGE - 1) % NSTAGE>{});
+      read_half(std::integral_constant<int, (s_ + 1) % NSTAGE>{}, H0{});
     }
-    __builtin_amdgcn_s_barrier();
+    mma_half(H1{});
   };
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
@@ -584,47 +653,49 @@ __global__ __launch_bounds__(kThreads) void gemm_dma_kernel(GemmArgs p) {
   using I3 = std::integral_constant<int, 3>;
   using I4 = std::integral_constant<int, 4>;
 
-  // Prologue: slabs 0..D-1 in flight, slab 0 landed.
-  if (0 < nk) issue(I0{}, 0);
-  if (D > 1 && 1 < nk) issue(I1{}, 1);
-  if (D > 2 && 2 < nk) issue(I2{}, 2);
-  if (D > 3 && 3 < nk) issue(I3{}, 3);
-  if (nk >= D) {
-    RTP_WAIT_VM_LGKM0((D - 1) * NI);
+  // Prologue: slabs 0..NSTAGE-2 issued, slab 0 landed and its first half in registers.
+  if (0 < nk) issue(I0{});
+  if (1 < nk) issue(I1{});
+  if (NSTAGE > 3 && 2 < nk) issue(I2{});
+  if (NSTAGE > 4 && 3 < nk) issue(I3{});
+  if (nk >= NSTAGE - 1) {
+    RTP_WAIT_VM((NSTAGE - 2) * NI);
   } else {
-    RTP_WAIT_VM_LGKM0(0);
+    RTP_WAIT_VM(0);
   }
   __builtin_amdgcn_s_barrier();
+  if (0 < nk) read_half(I0{}, H0{});
 
   int kt = 0;
-  for (; kt + NSTAGE - 1 + D < nk; kt += NSTAGE) {  // every phase of the round may issue
-    steady_phase(I0{}, kt);
-    steady_phase(I1{}, kt + 1);
-    if (NSTAGE > 2) steady_phase(I2{}, kt + 2);
-    if (NSTAGE > 3) steady_phase(I3{}, kt + 3);
-    if (NSTAGE > 4) steady_phase(I4{}, kt + 4);
+  for (; kt + 2 * NSTAGE - 2 < nk; kt += NSTAGE) {  // the last phase of the round (slab kt+NSTAGE-1) still issues
+    phase(I0{}, kt, std::true_type{});
+    phase(I1{}, kt + 1, std::true_type{});
+    phase(I2{}, kt + 2, std::true_type{});
+    if (NSTAGE > 3) phase(I3{}, kt + 3, std::true_type{});
+    if (NSTAGE > 4) phase(I4{}, kt + 4, std::true_type{});
   }
   for (; kt < nk; kt += NSTAGE) {
-    drain_phase(I0{}, kt);
-    drain_phase(I1{}, kt + 1);
-    if (NSTAGE > 2) drain_phase(I2{}, kt + 2);
-    if (NSTAGE > 3) drain_phase(I3{}, kt + 3);
-    if (NSTAGE > 4) drain_phase(I4{}, kt + 4);
+    phase(I0{}, kt, std::false_type{});
+    phase(I1{}, kt + 1, std::false_type{});
+    phase(I2{}, kt + 2, std::false_type{});
+    if (NSTAGE > 3) phase(I3{}, kt + 3, std::false_type{});
+    if (NSTAGE > 4) phase(I4{}, kt + 4, std::false_type{});
   }
 
-  store_tile<T, MT, NT, WM, WN>(p, acc, m0, n0, wm, wn, li, g, grp, zo, zi);
+  if (computes) store_tile<T, MT, NT, WM, WN>(p, acc, m0, n0, wm, wn, li, g, grp, zo, zi);
 }
 
-template <typename T, int BM, int BN, int NSTAGE>
+template <typename T, int BM, int BN, int NSTAGE, int NW>
 static int launch_dma(hipStream_t s, const GemmArgs& a, bool akc, bool bkc, dim3 grid) {
+  const dim3 block(NW * 64);
   if (akc && bkc)
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, true, NSTAGE>), grid, dim3(kThreads), 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, true, NSTAGE, NW>), grid, block, 0, s, a);
   else if (akc && !bkc)
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, false, NSTAGE>), grid, dim3(kThreads), 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, false, NSTAGE, NW>), grid, block, 0, s, a);
   else if (!akc && bkc)
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, true, NSTAGE>), grid, dim3(kThreads), 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, true, NSTAGE, NW>), grid, block, 0, s, a);
   else
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, false, NSTAGE>), grid, dim3(kThreads), 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, false, NSTAGE, NW>), grid, block, 0, s, a);
   RTP_LAUNCH_CHECK();
   return RTP_OK;
 }
@@ -710,7 +781,8 @@ struct TileShape {
   int bm, bn;
   const char* tag;
 };
-static const TileShape kShapes[3] = {{128, 128, "128x128"}, {128, 64, "128x64"}, {64, 64, "64x64"}};
+static const TileShape kShapes[4] = {{256, 128, "256x128"}, {128, 128, "128x128"}, {128, 64, "128x64"}, {64, 64, "64x64"}};
+constexpr int kNumShapes = 4;
 
 template <typename T>
 static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
@@ -776,13 +848,17 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
     RTP_LAUNCH_CHECK();
     return RTP_OK;
   }
-  int shape = 2;
-  for (int i = 0; fast && i < 3; ++i) {
+  static const int min_tiles = [] {
+    const char* e = getenv("RTP_GEMM_MIN_TILES");
+    return e ? atoi(e) : 200;
+  }();
+  int shape = kNumShapes - 1;
+  for (int i = 0; fast && i < kNumShapes; ++i) {
     // never a tile that is mostly padding: a 32 x 32 problem (one attention head at seq 32) stays at 64 x 64
     if (kShapes[i].bm > 64 && kShapes[i].bm > ceil_div(d->m, 64) * 64) continue;
     if (kShapes[i].bn > 64 && kShapes[i].bn > ceil_div(d->n, 64) * 64) continue;
     const int64_t tiles = ceil_div(d->m, kShapes[i].bm) * ceil_div(d->n, kShapes[i].bn) * nz;
-    if (tiles >= 200) {
+    if (tiles >= min_tiles) {
       shape = i;
       break;
     }
@@ -794,11 +870,34 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   RTP_REQUIRE(nb < (1ll << 31) && nz < 65536, "gemm grid too large (%lld tiles, %lld batch*groups)", (long long)nb,
               (long long)nz);
   dim3 grid((unsigned)nb, (unsigned)nz, 1);
+  // XCD bricks: among the splits xg*xm*xn == 8 that divide the launch evenly, take the one with the fewest
+  // operand bytes per XCD (A rows x K of the brick's row tiles, B likewise; an operand that differs per
+  // batch/group entry counts once per entry of the brick).
+  a.xg = a.xm = a.xn = 0;
+  if (fast) {
+    const bool a_per_z = d->batch > 1 || (d->groups > 1 && d->a_sg != 0);
+    const bool b_per_z = d->batch > 1 || (d->groups > 1 && d->b_sg != 0);
+    double best = 0.0;
+    for (int xg = 1; xg <= 8; xg *= 2)
+      for (int xm = 1; xg * xm <= 8; xm *= 2) {
+        const int xn = 8 / (xg * xm);
+        if (nz % xg || a.tiles_m % xm || a.tiles_n % xn) continue;
+        const double zb = (double)(nz / xg);
+        const double cost = (double)(a.tiles_m / xm) * ts.bm * (a_per_z ? zb : 1.0) +
+                            (double)(a.tiles_n / xn) * ts.bn * (b_per_z ? zb : 1.0);
+        if (a.xg == 0 || cost < best) {
+          best = cost;
+          a.xg = xg;
+          a.xm = xm;
+          a.xn = xn;
+        }
+      }
+  }
 
   // variant name = the kernel template instance, e.g. gemm_bf16_128x64_kc_kc
   static const char* const layout_tag[2][2] = {{"rc_rc", "rc_kc"}, {"kc_rc", "kc_kc"}};
-  static thread_local char names[2][4][2][2][40];
-  char* name = names[sizeof(T) == 2][fast ? shape : 3][akc][bkc];
+  static thread_local char names[2][kNumShapes + 1][2][2][40];
+  char* name = names[sizeof(T) == 2][fast ? shape : kNumShapes][akc][bkc];
   if (!name[0])
     snprintf(name, 40, "gemm_%s_%s_%s", sizeof(T) == 2 ? "bf16" : "f32", fast ? ts.tag : "64x64_guarded",
              layout_tag[akc][bkc]);
@@ -811,11 +910,13 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   if (!fast) return launch_layout<T, 64, 64, 1, false>(s, a, akc, bkc, grid);
   switch (shape) {
     case 0:
-      return launch_dma<T, 128, 128, 4>(s, a, akc, bkc, grid);
+      return launch_dma<T, 256, 128, 3, 4>(s, a, akc, bkc, grid);
     case 1:
-      return launch_dma<T, 128, 64, 5>(s, a, akc, bkc, grid);
+      return launch_dma<T, 128, 128, 4, 8>(s, a, akc, bkc, grid);
+    case 2:
+      return launch_dma<T, 128, 64, 5, 8>(s, a, akc, bkc, grid);
     default:
-      return launch_dma<T, 64, 64, 4>(s, a, akc, bkc, grid);
+      return launch_dma<T, 64, 64, 4, 8>(s, a, akc, bkc, grid);
   }
 }
 
