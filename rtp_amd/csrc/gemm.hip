@@ -40,6 +40,7 @@ struct GemmArgs {
   int flags;
   int vec_a, vec_b;
   int tiles_m, tiles_n;
+  int vec_c;       // every epilogue operand allows 16-byte accesses of 8 columns
   int xg, xm, xn;  // split of the (batch*groups, tiles_m, tiles_n) space over the 8 XCDs; xg == 0: none
 };
 
@@ -362,6 +363,127 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs p) {
   store_tile<T, MT, NT, WM, WN>(p, acc, t.m0, t.n0, wm, wn, li, g, grp, zo, zi);
 }
 
+// Epilogue of the direct-to-LDS kernel.  `ct` is the BM x BN tile of raw accumulators in LDS (row pitch BN+4
+// floats).  Thread `tid` of NTHR finishes chunks of 8 consecutive columns: alpha * acc (+ c_in) (+ bias) -> ReLU ->
+// gate mask -> store, the same order of operations as store_tile.  With p.vec_c (16-byte aligned operands and
+// n % 8 == 0, checked by the host) every global access of a chunk is a 16-byte vector.
+template <typename T>
+__device__ __forceinline__ void load8(const T* src, float (&v)[8]) {
+  if (sizeof(T) == 2) {
+    union {
+      uint4 q;
+      T e[8];
+    } u;
+    u.q = *reinterpret_cast<const uint4*>(src);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = to_f32(u.e[e]);
+  } else {
+    const float4 lo = reinterpret_cast<const float4*>(src)[0], hi = reinterpret_cast<const float4*>(src)[1];
+    v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w, v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
+  }
+}
+template <typename T>
+__device__ __forceinline__ void store8(T* dst, const float (&v)[8]) {
+  if (sizeof(T) == 2) {
+    union {
+      uint4 q;
+      T e[8];
+    } u;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) u.e[e] = from_f32<T>(v[e]);
+    *reinterpret_cast<uint4*>(dst) = u.q;
+  } else {
+    reinterpret_cast<float4*>(dst)[0] = make_float4(v[0], v[1], v[2], v[3]);
+    reinterpret_cast<float4*>(dst)[1] = make_float4(v[4], v[5], v[6], v[7]);
+  }
+}
+
+template <typename T, int BM, int BN, int NTHR>
+__device__ __forceinline__ void finish_tile(const GemmArgs& p, const float* ct, int m0, int n0, int tid, int grp,
+                                            long zo, long zi) {
+  constexpr int CP = BN + 4, CPR = BN / 8, CHUNKS = BM * CPR;
+  const bool out_f32 = p.flags & RTP_GEMM_OUT_F32;
+  const bool cin_f32 = p.flags & RTP_GEMM_CIN_F32;
+  const bool relu = p.flags & RTP_GEMM_RELU;
+  char* cbase = p.c_out + (grp * p.c_sg + zo * p.c_so + zi * p.c_si) * (out_f32 ? 4 : (long)sizeof(T));
+  const char* cin =
+      p.c_in ? p.c_in + (grp * p.cin_sg + zo * p.cin_so + zi * p.cin_si) * (cin_f32 ? 4 : (long)sizeof(T)) : nullptr;
+  const T* bias =
+      p.bias ? reinterpret_cast<const T*>(p.bias) + grp * p.bias_sg + zo * p.bias_so + zi * p.bias_si : nullptr;
+  const T* gate =
+      p.gate ? reinterpret_cast<const T*>(p.gate) + grp * p.gate_sg + zo * p.gate_so + zi * p.gate_si : nullptr;
+  const int nb_seg = p.bias_sk ? p.ksegs : 1;  // a bias per K segment is summed in segment order
+
+  for (int c = tid; c < CHUNKS; c += NTHR) {
+    const int lr = c / CPR, lc = (c % CPR) * 8;
+    const int row = m0 + lr, col = n0 + lc;
+    if (row >= p.m || col >= p.n) continue;
+    float v[8], t[8];
+    {
+      const float4 lo = *reinterpret_cast<const float4*>(ct + lr * CP + lc);
+      const float4 hi = *reinterpret_cast<const float4*>(ct + lr * CP + lc + 4);
+      v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w, v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] *= p.alpha;
+    if (p.vec_c) {
+      if (cin) {
+        const long off = (long)row * p.ld_cin + col;
+        if (cin_f32)
+          load8(reinterpret_cast<const float*>(cin) + off, t);
+        else
+          load8(reinterpret_cast<const T*>(cin) + off, t);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] += t[e];
+      }
+      if (bias) {
+        float bv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int sgm = 0; sgm < nb_seg; ++sgm) {
+          load8(bias + sgm * p.bias_sk + col, t);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) bv[e] += t[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] += bv[e];
+      }
+      if (relu) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = fmaxf(v[e], 0.0f);
+      }
+      if (gate) {
+        load8(gate + (long)row * p.ld_gate + col, t);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = t[e] > 0.0f ? v[e] : 0.0f;
+      }
+      const long off = (long)row * p.ldc + col;
+      if (out_f32)
+        store8(reinterpret_cast<float*>(cbase) + off, v);
+      else
+        store8(reinterpret_cast<T*>(cbase) + off, v);
+    } else {
+      for (int e = 0; e < 8 && col + e < p.n; ++e) {
+        float x = v[e];
+        if (cin) {
+          const long off = (long)row * p.ld_cin + col + e;
+          x += cin_f32 ? reinterpret_cast<const float*>(cin)[off] : to_f32(reinterpret_cast<const T*>(cin)[off]);
+        }
+        if (bias) {
+          float bv = 0.0f;
+          for (int sgm = 0; sgm < nb_seg; ++sgm) bv += to_f32(bias[sgm * p.bias_sk + col + e]);
+          x += bv;
+        }
+        if (relu) x = fmaxf(x, 0.0f);
+        if (gate) x = to_f32(gate[(long)row * p.ld_gate + col + e]) > 0.0f ? x : 0.0f;
+        const long off = (long)row * p.ldc + col + e;
+        if (out_f32)
+          reinterpret_cast<float*>(cbase)[off] = x;
+        else
+          reinterpret_cast<T*>(cbase)[off] = from_f32<T>(x);
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Direct-to-LDS pipeline (the fast path).  Slabs go global -> LDS with global_load_lds_dwordx4: no
 // staging registers, NSTAGE LDS stages, up to NSTAGE-1 slabs in flight while the MFMAs of the current slab
@@ -378,8 +500,9 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs p) {
 // Vectors beyond the contraction length are fetched from a 16-byte block of zeros; rows beyond the
 // operand are clamped (they only feed accumulators that are never stored).
 //
-// The workgroup has NW >= 4 waves: waves 0..3 run the MFMAs, and ALL NW waves share the loads, so the address
-// arithmetic and the issue slots of the loads are spread over more wavefronts.
+// The workgroup has 8 waves with separate roles: waves 0..3 run the MFMAs of a 2x2 grid of wave tiles and
+// issue no global loads; waves 4..7 only issue the loads and count them down.  Scalar bookkeeping for the
+// loads therefore does not take issue slots from the MFMA waves.
 __device__ __attribute__((aligned(16))) unsigned int g_zero16[4] = {0u, 0u, 0u, 0u};
 
 // s_waitcnt with vmcnt = VM, lgkmcnt = 0, expcnt untouched (gfx9 encoding).
@@ -403,20 +526,21 @@ __device__ __forceinline__ constexpr int rc_swizzle(int kl) {
   return R >= 128 ? (kl & 3) << 2 : ((kl >> 1) & 1) << 2;
 }
 
-template <typename T, int R, bool KC, int NW>
+template <typename T, int R, bool KC, int NL>
 struct DmaOperand {
   static constexpr int VEC = 16 / sizeof(T);
-  static_assert((R / 8) % NW == 0, "every wave issues the same number of loads");
-  static constexpr int NI = R / 8 / NW;           // load instructions per wave and slab
+  static_assert((R / 8) % NL == 0, "every loader wave issues the same number of loads");
+  static constexpr int NI = R / 8 / NL;           // load instructions per loader wave and slab
   static constexpr int BYTES = R * kSlabBytes;    // one stage of this operand
   static constexpr int LINE = R * (int)sizeof(T); // bytes of one k line when rows are contiguous
-  const T* ptr[NI];
-  int koff[NI];
+  const T* ptr[NI];  // source of the NEXT slab's vector, advanced in place
+  int koff[NI];      // k of the vector inside its slab
 
-  __device__ __forceinline__ void init(const T* base, long ld, int row0, int rows, int wave, int lane) {
+  // lw: index of the loader wave (0..NL-1).
+  __device__ __forceinline__ void init(const T* base, long ld, int row0, int rows, int lw, int lane) {
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-      const int j = wave * NI + i;  // which KiB of the stage
+      const int j = lw * NI + i;  // which KiB of the stage
       if (KC) {
         const int row = j * 8 + (lane >> 3);
         const int c = (lane & 7) ^ ((row >> 1) & 7);
@@ -435,29 +559,23 @@ struct DmaOperand {
     }
   }
 
-  // off: element offset of the slab (K segment offset + k0, or k0 lines), k0: first k of the slab.  `tail` is
-  // uniform: only the last slab of a K segment can reach beyond the contraction length, and only then are the
-  // per-vector checks made.
-  __device__ __forceinline__ void issue(char* stage, long off, int k0, int kdim, int wave, bool tail) const {
-    if (tail) {
+  // Start the loads of the next slab into the stage at LDS byte address `lds_stage` (this operand's part) and
+  // move the pointers on by `advance` elements.  LAST: the slab is the last of its K segment (first k = k0),
+  // the only one that can reach beyond the contraction length kdim; vectors beyond it come from a block of zeros.
+  template <bool LAST>
+  __device__ __forceinline__ void issue(unsigned lds_stage, int lw, long advance, int k0, int kdim) {
 #pragma unroll
-      for (int i = 0; i < NI; ++i) {
-        const T* src = ptr[i] + off;
-        if (k0 + koff[i] >= kdim) src = reinterpret_cast<const T*>(g_zero16);
-        dma(stage + (wave * NI + i) * 1024, src);
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < NI; ++i) dma(stage + (wave * NI + i) * 1024, ptr[i] + off);
+    for (int i = 0; i < NI; ++i) {
+      const T* src = ptr[i];
+      if (LAST && k0 + koff[i] >= kdim) src = reinterpret_cast<const T*>(g_zero16);
+      // Inline assembly on purpose: the compiler must not track this instruction (it would make LDS reads wait
+      // for all outstanding loads); the kernel's explicit s_waitcnt + barrier protocol is the ordering that counts.
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                   :
+                   : "s"(lds_stage + (unsigned)((lw * NI + i) * 1024)), "v"(src)
+                   : "memory");
+      ptr[i] += advance;
     }
-  }
-
-  // Issued as inline assembly on purpose: the compiler's own bookkeeping for this instruction makes LDS
-  // reads wait for ALL outstanding loads once per pipeline round; the kernel's explicit s_waitcnt + barrier
-  // protocol is the ordering that counts.
-  static __device__ __forceinline__ void dma(char* dst, const T* src) {
-    const unsigned lds_addr = (unsigned)(uintptr_t)(lptr_t)dst;
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(src) : "memory");
   }
 };
 
@@ -499,37 +617,24 @@ __device__ __forceinline__ Frag<T> read_frag_dma(const char* st, int rowbase, in
   return u.f;
 }
 
-template <typename T, int BM, int BN, bool AKC, bool BKC, int NSTAGE, int NW>
-__global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(GemmArgs p) {
-  using DA = DmaOperand<T, BM, AKC, NW>;
-  using DB = DmaOperand<T, BN, BKC, NW>;
+template <typename T, int BM, int BN, bool AKC, bool BKC, int NSTAGE>
+__global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
+  constexpr int NL = 4;  // loader waves (waves 4..7); waves 0..3 compute
+  using DA = DmaOperand<T, BM, AKC, NL>;
+  using DB = DmaOperand<T, BN, BKC, NL>;
   constexpr int BK = kSlabBytes / sizeof(T);
   constexpr int WM = BM / 2, WN = BN / 2, MT = WM / 32, NT = WN / 32;
   constexpr int STAGE = DA::BYTES + DB::BYTES;
-  constexpr int NI = DA::NI + DB::NI;      // loads per wave and slab
+  constexpr int NI = DA::NI + DB::NI;  // loads per loader wave and slab
   static_assert((NSTAGE - 2) * NI < 64, "vmcnt is a 6-bit counter");
-  // One __shared__ array per stage, always addressed with a compile-time stage index: distinct arrays
-  // let the compiler see that LDS reads of one stage do not alias the asynchronous writes into another,
-  // so it does not make every LDS read wait for all outstanding loads.
   static_assert(NSTAGE >= 3 && NSTAGE <= 5, "3..5 LDS stages");
-  __shared__ __attribute__((aligned(1024))) char st0[STAGE];
-  __shared__ __attribute__((aligned(1024))) char st1[STAGE];
-  __shared__ __attribute__((aligned(1024))) char st2[NSTAGE > 2 ? STAGE : 16];
-  __shared__ __attribute__((aligned(1024))) char st3[NSTAGE > 3 ? STAGE : 16];
-  __shared__ __attribute__((aligned(1024))) char st4[NSTAGE > 4 ? STAGE : 16];
-  auto stage = [&](auto S) -> char* {
-    constexpr int s_ = decltype(S)::value % NSTAGE;
-    if constexpr (s_ == 0) return st0;
-    else if constexpr (s_ == 1) return st1;
-    else if constexpr (s_ == 2) return st2;
-    else if constexpr (s_ == 3) return st3;
-    else return st4;
-  };
+  static_assert(BM * (BN + 4) * 4 <= NSTAGE * STAGE, "the epilogue stages the fp32 tile in the slab memory");
+  // Stage addresses are compile-time offsets into one array, so LDS reads carry immediate offsets.
+  __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const bool computes = wave < 4;  // waves 4.. only load
   const int wm = (wave >> 1) & 1, wn = wave & 1;
   const int li = lane & 31, g = lane >> 5;
 
@@ -553,36 +658,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(GemmArgs p) {
   const int n0 = tile_n * BN;
   const int grp = z / p.batch, zb = z % p.batch;
   const long zo = zb / p.zdiv, zi = zb % p.zdiv;
-  const T* A = reinterpret_cast<const T*>(p.a) + grp * p.a_sg + zo * p.a_so + zi * p.a_si;
-  const T* B = reinterpret_cast<const T*>(p.b) + grp * p.b_sg + zo * p.b_so + zi * p.b_si;
-
-  DA da;
-  DB db;
-  da.init(A, p.lda, m0, p.m, wave, lane);
-  db.init(B, p.ldb, n0, p.n, wave, lane);
   const int nk_seg = (p.k + BK - 1) / BK;
   const int nk = nk_seg * p.ksegs;
-
-  // Slabs are issued strictly in order; the cursor of the next slab to issue lives in scalar registers
-  // and is advanced by additions only.
-  const long step_a = AKC ? (long)BK : (long)BK * p.lda, step_b = BKC ? (long)BK : (long)BK * p.ldb;
-  const long wrap_a = p.a_sk - nk_seg * step_a, wrap_b = p.b_sk - nk_seg * step_b;
-  int ik0 = 0;
-  long off_a = 0, off_b = 0;
-  auto issue = [&](auto S) {
-    char* st = stage(S);
-    const bool tail = ik0 + BK > p.k;
-    da.issue(st, off_a, ik0, p.k, wave, tail);
-    db.issue(st + DA::BYTES, off_b, ik0, p.k, wave, tail);
-    ik0 += BK;
-    off_a += step_a;
-    off_b += step_b;
-    if (ik0 >= p.k) {
-      ik0 = 0;
-      off_a += wrap_a;
-      off_b += wrap_b;
-    }
-  };
 
   f32x16 acc[MT][NT];
 #pragma unroll
@@ -592,110 +669,163 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(GemmArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  // Fragment registers of one slab in two halves (k-steps 0,1 and 2,3).  While the MFMAs of one half run,
-  // the other half is being read from LDS -- the first half of the NEXT slab during the second half of
-  // this one -- so an LDS read always has a half slab of MFMAs to hide behind.
-  Frag<T> fa[4][MT], fb[4][NT];
-  auto read_half = [&](auto S, auto H) {
-    if (!computes) return;
-    const char* sa = stage(S);
-    const char* sb = sa + DA::BYTES;
-    constexpr int h = decltype(H)::value;
-#pragma unroll
-    for (int ks = 2 * h; ks < 2 * h + 2; ++ks) {
-#pragma unroll
-      for (int i = 0; i < MT; ++i) fa[ks][i] = read_frag_dma<T, BM, AKC>(sa, wm * WM + i * 32, lane, ks);
-#pragma unroll
-      for (int j = 0; j < NT; ++j) fb[ks][j] = read_frag_dma<T, BN, BKC>(sb, wn * WN + j * 32, lane, ks);
-    }
-  };
-  auto mma_half = [&](auto H) {
-    if (!computes) return;
-    constexpr int h = decltype(H)::value;
-#pragma unroll
-    for (int ks = 2 * h; ks < 2 * h + 2; ++ks)
-#pragma unroll
-      for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int j = 0; j < NT; ++j) mma(fa[ks][i], fb[ks][j], acc[i][j]);
-  };
-  using H0 = std::integral_constant<int, 0>;
-  using H1 = std::integral_constant<int, 1>;
-
-  // Phase of slab k (held in stage S = k % NSTAGE).  On entry slab k is visible to every wave and the first
-  // half of its fragments is in registers.  Slabs up to k + NSTAGE - 2 have been issued.
-  //   read second half of slab k | MFMAs of the first half
-  //   wait for this wave's loads of slab k+1, barrier: slab k+1 is visible and every wave has finished
-  //     reading slab k-1, whose stage is refilled with slab k + NSTAGE - 1
-  //   read first half of slab k+1 | MFMAs of the second half of slab k
-  // STEADY: every condition below is known to hold, so the phase is branch-free.
-  auto phase = [&](auto S, int k, auto STEADY) {
-    constexpr int s_ = decltype(S)::value;
-    constexpr bool steady = decltype(STEADY)::value;
-    if (!steady && k >= nk) return;
-    read_half(S, H1{});
-    mma_half(H0{});
-    if (steady || k + 1 < nk) {
-      if (steady || k + NSTAGE - 2 < nk) {
-        RTP_WAIT_VM((NSTAGE - 3) * NI);
+  // Barrier protocol: both paths meet the same nk barriers.  Barrier k is passed when slab k is visible to
+  // every wave: a loader reaches it only after its own loads of slab k have landed.  A compute wave reaches
+  // barrier k+1 after the MFMAs that consumed the last fragments of slab k-1, so once barrier k+1 is passed
+  // the loaders may refill the stage of slab k-1 (with slab k-1+NSTAGE).
+  if (wave >= 4) {
+    // ---- loader waves: issue slabs strictly in order, NSTAGE-1 ahead of the slab being consumed ----
+    const int lw = wave - 4;
+    const T* A = reinterpret_cast<const T*>(p.a) + grp * p.a_sg + zo * p.a_so + zi * p.a_si;
+    const T* B = reinterpret_cast<const T*>(p.b) + grp * p.b_sg + zo * p.b_so + zi * p.b_si;
+    DA da;
+    DB db;
+    da.init(A, p.lda, m0, p.m, lw, lane);
+    db.init(B, p.ldb, n0, p.n, lw, lane);
+    const long step_a = AKC ? (long)BK : (long)BK * p.lda, step_b = BKC ? (long)BK : (long)BK * p.ldb;
+    // after the last slab of a segment the pointers move to the start of the next segment
+    const long last_a = step_a + p.a_sk - nk_seg * step_a, last_b = step_b + p.b_sk - nk_seg * step_b;
+    const int k0_last = (nk_seg - 1) * BK;
+    const unsigned lds0 = (unsigned)(uintptr_t)(lptr_t)lds;
+    unsigned fill = lds0;  // LDS address of the stage the next slab goes to
+    int left = nk_seg;     // slabs left in the current K segment, the next one included
+    auto issue = [&]() {
+      if (left != 1) {
+        da.template issue<false>(fill, lw, step_a, 0, 0);
+        db.template issue<false>(fill + DA::BYTES, lw, step_b, 0, 0);
+        --left;
       } else {
-        RTP_WAIT_VM(0);
+        da.template issue<true>(fill, lw, last_a, k0_last, p.k);
+        db.template issue<true>(fill + DA::BYTES, lw, last_b, k0_last, p.k);
+        left = nk_seg;
       }
-      __builtin_amdgcn_s_barrier();
-      if (steady || k + NSTAGE - 1 < nk) issue(std::integral_constant<int, (s_ + NSTAGE - 1) % NSTAGE>{});
-      read_half(std::integral_constant<int, (s_ + 1) % NSTAGE>{}, H0{});
+      fill += STAGE;
+      if (fill == lds0 + NSTAGE * STAGE) fill = lds0;
+    };
+    const int ahead = nk < NSTAGE - 1 ? nk : NSTAGE - 1;
+    for (int s_ = 0; s_ < ahead; ++s_) issue();
+    if (nk >= NSTAGE - 1) {
+      RTP_WAIT_VM((NSTAGE - 2) * NI);
+    } else {
+      RTP_WAIT_VM(0);
     }
-    mma_half(H1{});
-  };
-  using I0 = std::integral_constant<int, 0>;
-  using I1 = std::integral_constant<int, 1>;
-  using I2 = std::integral_constant<int, 2>;
-  using I3 = std::integral_constant<int, 3>;
-  using I4 = std::integral_constant<int, 4>;
-
-  // Prologue: slabs 0..NSTAGE-2 issued, slab 0 landed and its first half in registers.
-  if (0 < nk) issue(I0{});
-  if (1 < nk) issue(I1{});
-  if (NSTAGE > 3 && 2 < nk) issue(I2{});
-  if (NSTAGE > 4 && 3 < nk) issue(I3{});
-  if (nk >= NSTAGE - 1) {
-    RTP_WAIT_VM((NSTAGE - 2) * NI);
+    __builtin_amdgcn_s_barrier();  // barrier 0
+    int k = 0;
+    for (; k + NSTAGE - 1 < nk; ++k) {  // slab k+NSTAGE-1 exists: steady state
+      RTP_WAIT_VM((NSTAGE - 3) * NI);   // slabs k+2 .. k+NSTAGE-2 may still be in flight
+      __builtin_amdgcn_s_barrier();     // barrier k+1
+      issue();                          // slab k+NSTAGE-1 into the stage of slab k-1
+    }
+    for (; k + 1 < nk; ++k) {
+      RTP_WAIT_VM(0);
+      __builtin_amdgcn_s_barrier();
+    }
   } else {
-    RTP_WAIT_VM(0);
+    // ---- compute waves ----
+    // The 4 k-steps of a slab are taken in NG groups of G k-steps, with two sets of fragment registers:
+    // while the MFMAs of one group run, the next group is read from LDS into the other set -- the first
+    // group of the NEXT slab during the last group of this one -- so an LDS read always has a group of
+    // MFMAs to hide behind.  Big tiles take G = 1 to fit the register file.
+    constexpr int G = (MT * NT >= 8) ? 1 : 2, NG = 4 / G;
+    Frag<T> fa[2][G][MT], fb[2][G][NT];
+    auto read_group = [&](auto S, auto Q) {
+      const char* sa = lds + (decltype(S)::value % NSTAGE) * STAGE;
+      const char* sb = sa + DA::BYTES;
+      constexpr int q = decltype(Q)::value;
+#pragma unroll
+      for (int e = 0; e < G; ++e) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i) fa[q & 1][e][i] = read_frag_dma<T, BM, AKC>(sa, wm * WM + i * 32, lane, q * G + e);
+#pragma unroll
+        for (int j = 0; j < NT; ++j) fb[q & 1][e][j] = read_frag_dma<T, BN, BKC>(sb, wn * WN + j * 32, lane, q * G + e);
+      }
+    };
+    auto mma_group = [&](auto Q) {
+      constexpr int q = decltype(Q)::value;
+#pragma unroll
+      for (int e = 0; e < G; ++e)
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+          for (int j = 0; j < NT; ++j) mma(fa[q & 1][e][i], fb[q & 1][e][j], acc[i][j]);
+    };
+    using Q0 = std::integral_constant<int, 0>;
+    using Q1 = std::integral_constant<int, 1>;
+    using Q2 = std::integral_constant<int, 2>;
+    using Q3 = std::integral_constant<int, 3>;
+    // Phase of slab k (stage S = k % NSTAGE); on entry the first group of its fragments is in registers.
+    auto phase = [&](auto S, int k, auto STEADY) {
+      constexpr bool steady = decltype(STEADY)::value;
+      if (!steady && k >= nk) return;
+      read_group(S, Q1{});
+      mma_group(Q0{});
+      if (NG == 4) {
+        read_group(S, Q2{});
+        mma_group(Q1{});
+        read_group(S, Q3{});
+        mma_group(Q2{});
+      }
+      if (steady || k + 1 < nk) {
+        __builtin_amdgcn_s_barrier();  // barrier k+1: slab k+1 is visible
+        read_group(std::integral_constant<int, (decltype(S)::value + 1) % NSTAGE>{}, Q0{});
+      }
+      mma_group(std::integral_constant<int, NG - 1>{});
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+    using I4 = std::integral_constant<int, 4>;
+    __builtin_amdgcn_s_barrier();  // barrier 0
+    read_group(I0{}, Q0{});
+    int kt = 0;
+    for (; kt + NSTAGE < nk; kt += NSTAGE) {
+      phase(I0{}, kt, std::true_type{});
+      phase(I1{}, kt + 1, std::true_type{});
+      phase(I2{}, kt + 2, std::true_type{});
+      if (NSTAGE > 3) phase(I3{}, kt + 3, std::true_type{});
+      if (NSTAGE > 4) phase(I4{}, kt + 4, std::true_type{});
+    }
+    for (; kt < nk; kt += NSTAGE) {
+      phase(I0{}, kt, std::false_type{});
+      phase(I1{}, kt + 1, std::false_type{});
+      phase(I2{}, kt + 2, std::false_type{});
+      if (NSTAGE > 3) phase(I3{}, kt + 3, std::false_type{});
+      if (NSTAGE > 4) phase(I4{}, kt + 4, std::false_type{});
+    }
   }
-  __builtin_amdgcn_s_barrier();
-  if (0 < nk) read_half(I0{}, H0{});
+  const bool computes = wave < 4;
 
-  int kt = 0;
-  for (; kt + 2 * NSTAGE - 2 < nk; kt += NSTAGE) {  // the last phase of the round (slab kt+NSTAGE-1) still issues
-    phase(I0{}, kt, std::true_type{});
-    phase(I1{}, kt + 1, std::true_type{});
-    phase(I2{}, kt + 2, std::true_type{});
-    if (NSTAGE > 3) phase(I3{}, kt + 3, std::true_type{});
-    if (NSTAGE > 4) phase(I4{}, kt + 4, std::true_type{});
+  // Epilogue through LDS: the accumulators (fp32) are laid out as the BM x BN tile, then every thread of the
+  // workgroup, loader waves included, finishes 8 consecutive columns of one row and writes them with 16-byte
+  // stores.
+  __builtin_amdgcn_s_barrier();  // every wave has read its last fragments
+  constexpr int CP = BN + 4;     // row pitch in floats
+  float* ct = reinterpret_cast<float*>(lds);
+  if (computes) {
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          ct[(wm * WM + i * 32 + 8 * (r >> 2) + 4 * g + (r & 3)) * CP + wn * WN + j * 32 + li] = acc[i][j][r];
   }
-  for (; kt < nk; kt += NSTAGE) {
-    phase(I0{}, kt, std::false_type{});
-    phase(I1{}, kt + 1, std::false_type{});
-    phase(I2{}, kt + 2, std::false_type{});
-    if (NSTAGE > 3) phase(I3{}, kt + 3, std::false_type{});
-    if (NSTAGE > 4) phase(I4{}, kt + 4, std::false_type{});
-  }
-
-  if (computes) store_tile<T, MT, NT, WM, WN>(p, acc, m0, n0, wm, wn, li, g, grp, zo, zi);
+  __syncthreads();
+  finish_tile<T, BM, BN, 512>(p, ct, m0, n0, tid, grp, zo, zi);
 }
 
-template <typename T, int BM, int BN, int NSTAGE, int NW>
+template <typename T, int BM, int BN, int NSTAGE>
 static int launch_dma(hipStream_t s, const GemmArgs& a, bool akc, bool bkc, dim3 grid) {
-  const dim3 block(NW * 64);
+  const dim3 block(512);
   if (akc && bkc)
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, true, NSTAGE, NW>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, true, NSTAGE>), grid, block, 0, s, a);
   else if (akc && !bkc)
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, false, NSTAGE, NW>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, false, NSTAGE>), grid, block, 0, s, a);
   else if (!akc && bkc)
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, true, NSTAGE, NW>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, true, NSTAGE>), grid, block, 0, s, a);
   else
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, false, NSTAGE, NW>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, false, NSTAGE>), grid, block, 0, s, a);
   RTP_LAUNCH_CHECK();
   return RTP_OK;
 }
@@ -818,6 +948,16 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   a.vec_b = mult((int64_t)(uintptr_t)d->b, 16) && mult(d->ldb, VEC) && mult(d->b_so, VEC) && mult(d->b_si, VEC) &&
             mult(d->b_sg, VEC) && mult(d->b_sk, VEC);
 
+  {
+    auto ok = [](const void* ptr, int64_t ld, int64_t so, int64_t si, int64_t sg) {
+      return mult((int64_t)(uintptr_t)ptr, 16) && mult(ld, 8) && mult(so, 8) && mult(si, 8) && mult(sg, 8);
+    };
+    a.vec_c = mult(d->n, 8) && ok(d->c_out, d->ldc, d->c_so, d->c_si, d->c_sg) &&
+              (!d->c_in || ok(d->c_in, d->ld_cin, d->cin_so, d->cin_si, d->cin_sg)) &&
+              (!d->gate || ok(d->gate, d->ld_gate, d->gate_so, d->gate_si, d->gate_sg)) &&
+              (!d->bias || (ok(d->bias, 8, d->bias_so, d->bias_si, d->bias_sg) && mult(d->bias_sk, 8)));
+  }
+
   // Branch-free loads need whole 16-byte vectors: aligned operands and extents that are multiples of VEC
   // along each operand's contiguous axis.  Anything else goes to the guarded small-tile kernel.
   const bool akc = d->a_kcontig, bkc = d->b_kcontig;
@@ -910,13 +1050,13 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   if (!fast) return launch_layout<T, 64, 64, 1, false>(s, a, akc, bkc, grid);
   switch (shape) {
     case 0:
-      return launch_dma<T, 256, 128, 3, 4>(s, a, akc, bkc, grid);
+      return launch_dma<T, 256, 128, 3>(s, a, akc, bkc, grid);
     case 1:
-      return launch_dma<T, 128, 128, 4, 8>(s, a, akc, bkc, grid);
+      return launch_dma<T, 128, 128, 4>(s, a, akc, bkc, grid);
     case 2:
-      return launch_dma<T, 128, 64, 5, 8>(s, a, akc, bkc, grid);
+      return launch_dma<T, 128, 64, 5>(s, a, akc, bkc, grid);
     default:
-      return launch_dma<T, 64, 64, 4, 8>(s, a, akc, bkc, grid);
+      return launch_dma<T, 64, 64, 4>(s, a, akc, bkc, grid);
   }
 }
 
