@@ -1088,6 +1088,70 @@ __global__ __launch_bounds__(kThreads) void colsum_partial_kernel(const T* x, lo
   if (ph == 0 && col < n) part[(long)blockIdx.y * n + col] = (red[0][c] + red[1][c]) + (red[2][c] + red[3][c]);
 }
 
+// Single-pass variant for a few thousand rows: one workgroup of 512 threads owns 32 columns; each thread walks
+// its rows with 16-byte loads (VEC columns, 4 loads in flight), and the per-thread sums are combined through LDS
+// in a fixed order (row groups in 4 quarters, then the quarters).
+constexpr int kOnepassThreads = 512, kOnepassCols = 32;
+template <typename T>
+__global__ __launch_bounds__(kOnepassThreads) void colsum_onepass_kernel(const T* x, long m, long n, long ld, void* out,
+                                                                         long seg, long seg_stride, int out_f32,
+                                                                         int accumulate) {
+  constexpr int VEC = 16 / sizeof(T), LPR = kOnepassCols / VEC, RG = kOnepassThreads / LPR;
+  __shared__ float red[RG][kOnepassCols + 1];
+  __shared__ float quarter[4][kOnepassCols];
+  const int cl = (threadIdx.x % LPR) * VEC, rg = threadIdx.x / LPR;
+  const long col = (long)blockIdx.x * kOnepassCols + cl;
+  float acc[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) acc[e] = 0.0f;
+  if (col < n) {  // n is a multiple of VEC, so the vector is wholly inside
+    union V {
+      uint4 q;
+      T e[VEC];
+    };
+    const T* src = x + col;
+    long r = rg;
+    for (; r + 3 * RG < m; r += 4 * RG) {
+      V u0, u1, u2, u3;
+      u0.q = *reinterpret_cast<const uint4*>(src + r * ld);
+      u1.q = *reinterpret_cast<const uint4*>(src + (r + RG) * ld);
+      u2.q = *reinterpret_cast<const uint4*>(src + (r + 2 * RG) * ld);
+      u3.q = *reinterpret_cast<const uint4*>(src + (r + 3 * RG) * ld);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc[e] += (to_f32(u0.e[e]) + to_f32(u1.e[e])) + (to_f32(u2.e[e]) + to_f32(u3.e[e]));
+    }
+    for (; r < m; r += RG) {
+      V u;
+      u.q = *reinterpret_cast<const uint4*>(src + r * ld);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc[e] += to_f32(u.e[e]);
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) red[rg][cl + e] = acc[e];
+  __syncthreads();
+  if (threadIdx.x < 4 * kOnepassCols) {
+    const int c = threadIdx.x % kOnepassCols, qd = threadIdx.x / kOnepassCols;
+    float v = 0.0f;
+    for (int r = qd * (RG / 4); r < (qd + 1) * (RG / 4); ++r) v += red[r][c];
+    quarter[qd][c] = v;
+  }
+  __syncthreads();
+  const long c = (long)blockIdx.x * kOnepassCols + threadIdx.x;
+  if (threadIdx.x < kOnepassCols && c < n) {
+    const int t = threadIdx.x;
+    const float v = (quarter[0][t] + quarter[1][t]) + (quarter[2][t] + quarter[3][t]);
+    const long o = (c / seg) * seg_stride + c % seg;
+    if (out_f32) {
+      float* dst = reinterpret_cast<float*>(out);
+      dst[o] = accumulate ? dst[o] + v : v;
+    } else {
+      T* dst = reinterpret_cast<T*>(out);
+      dst[o] = from_f32<T>(accumulate ? to_f32(dst[o]) + v : v);
+    }
+  }
+}
+
 // out index of column c: (c / seg) * seg_stride + c % seg  (bias slices of consecutive shards sit
 // seg_stride elements apart in the flat gradient buffer).
 template <typename T>
@@ -1161,6 +1225,18 @@ extern "C" int rtp_colsum(void* stream, int dtype, const void* x, int64_t m, int
   hipStream_t s = (hipStream_t)stream;
   float* part = (float*)workspace;
   ProfileScope prof(s, "colsum", (double)m * n, (double)m * n * (dtype == RTP_F32 ? 4 : 2));
+  const int vec = dtype == RTP_F32 ? 4 : 8;
+  if (m <= 4096 && (uintptr_t)x % 16 == 0 && ld % vec == 0 && n % vec == 0) {
+    dim3 g1((unsigned)ceil_div(n, kOnepassCols));
+    if (dtype == RTP_F32)
+      hipLaunchKernelGGL(colsum_onepass_kernel<float>, g1, dim3(kOnepassThreads), 0, s, (const float*)x, (long)m, (long)n,
+                         (long)ld, out, (long)seg, (long)seg_stride, 1, accumulate);
+    else
+      hipLaunchKernelGGL(colsum_onepass_kernel<bf16_t>, g1, dim3(kOnepassThreads), 0, s, (const bf16_t*)x, (long)m, (long)n,
+                         (long)ld, out, (long)seg, (long)seg_stride, out_f32, accumulate);
+    RTP_LAUNCH_CHECK();
+    return RTP_OK;
+  }
   dim3 grid((unsigned)ceil_div(n, 64), (unsigned)nparts);
   dim3 grid2((unsigned)ceil_div(n, kThreads));
   if (dtype == RTP_F32) {

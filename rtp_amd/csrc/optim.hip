@@ -22,22 +22,30 @@ __global__ __launch_bounds__(256) void sgd_kernel(float* master, const T* grad, 
   }
 }
 
-// Four parameters per lane and iteration: 16-byte master accesses, 8- or 16-byte gradient / shadow accesses.
+// Four parameters per lane and access: 16-byte master accesses, 8- or 16-byte gradient / shadow accesses; two
+// such groups are loaded before either is used, so each lane keeps four loads in flight.
 template <typename T>
-__global__ __launch_bounds__(256) void sgd_vec4_kernel(float4* master, const T* grad, T* shadow, long n4, float lr,
-                                                       float clip) {
-  const long stride = (long)gridDim.x * blockDim.x;
-  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
-    union {
-      T e[4];
-      uint2 u2;
-      uint4 u4;
-    } g, sh;
+struct Sgd4 {
+  union Pack {
+    T e[4];
+    uint2 u2;
+    uint4 u4;
+  };
+  static __device__ __forceinline__ Pack load(const T* p, long i) {
+    Pack v;
     if (sizeof(T) == 2)
-      g.u2 = reinterpret_cast<const uint2*>(grad)[i];
+      v.u2 = reinterpret_cast<const uint2*>(p)[i];
     else
-      g.u4 = reinterpret_cast<const uint4*>(grad)[i];
-    float4 w = master[i];
+      v.u4 = reinterpret_cast<const uint4*>(p)[i];
+    return v;
+  }
+  static __device__ __forceinline__ void store(T* p, long i, const Pack& v) {
+    if (sizeof(T) == 2)
+      reinterpret_cast<uint2*>(p)[i] = v.u2;
+    else
+      reinterpret_cast<uint4*>(p)[i] = v.u4;
+  }
+  static __device__ __forceinline__ void update(float4& w, const Pack& g, Pack& sh, float lr, float clip) {
     float* wf = reinterpret_cast<float*>(&w);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
@@ -50,13 +58,35 @@ __global__ __launch_bounds__(256) void sgd_vec4_kernel(float4* master, const T* 
       }
       sh.e[e] = from_f32<T>(wf[e]);
     }
-    master[i] = w;
+  }
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void sgd_vec4_kernel(float4* master, const T* grad, T* shadow, long n4, float lr,
+                                                       float clip) {
+  using P = typename Sgd4<T>::Pack;
+  const long stride = (long)gridDim.x * blockDim.x;
+  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  for (; i + stride < n4; i += 2 * stride) {
+    const P g0 = Sgd4<T>::load(grad, i), g1 = Sgd4<T>::load(grad, i + stride);
+    float4 w0 = master[i], w1 = master[i + stride];
+    P s0, s1;
+    Sgd4<T>::update(w0, g0, s0, lr, clip);
+    Sgd4<T>::update(w1, g1, s1, lr, clip);
+    master[i] = w0;
+    master[i + stride] = w1;
     if (shadow) {
-      if (sizeof(T) == 2)
-        reinterpret_cast<uint2*>(shadow)[i] = sh.u2;
-      else
-        reinterpret_cast<uint4*>(shadow)[i] = sh.u4;
+      Sgd4<T>::store(shadow, i, s0);
+      Sgd4<T>::store(shadow, i + stride, s1);
     }
+  }
+  for (; i < n4; i += stride) {
+    const P g0 = Sgd4<T>::load(grad, i);
+    float4 w0 = master[i];
+    P s0;
+    Sgd4<T>::update(w0, g0, s0, lr, clip);
+    master[i] = w0;
+    if (shadow) Sgd4<T>::store(shadow, i, s0);
   }
 }
 
