@@ -22,6 +22,13 @@ if ROOT not in sys.path:
 
 CFG = dict(vocab=10240, ninp=2048, nhid=2048, nhead=32, layers=10, seq=32, batch=32, shards=8)
 PEAK = {"bf16_mfma_tflops": 2500.0, "fp32_mfma_tflops": 157.3, "hbm_gbs": 8000.0}
+# Memory-side traffic per launch of the GEMM variants of this workload, KiB, averaged over the launches of a step:
+# FETCH_SIZE * 1.9934 + WRITE_SIZE * 1.0000 from two rocprofv3 --pmc runs of this script; the factors are what the same
+# counters read for the library's plain copy kernel on a copy of known size (profiles/lm_step_pmc_fetch_write.txt).
+MEASURED_TRAFFIC_KIB = {
+    "gemm_bf16_128x64_kc_rc": 56049.3, "gemm_bf16_128x64_kc_kc": 36954.5, "gemm_bf16_128x128_rc_rc": 32894.2,
+    "gemm_bf16_256x128_rc_rc": 88941.3, "gemm_bf16_128x128_kc_kc": 106399.3,
+}
 
 
 def step_flops(c):
@@ -184,7 +191,10 @@ def main():
                                "one GPU, uniform random token ids, weights U(-0.1,0.1), dropout 0, lr 1e-3, clip 0.05",
                    "tokens_per_step": tokens, "rotation_shards": c["shards"], "hip_graph": bool(args.graph)},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK["bf16_mfma_tflops"], "unit": "TFLOP/s",
-                     "frac": achieved / PEAK["bf16_mfma_tflops"], "traffic": None, "kernel": dom_name,
+                     "frac": achieved / PEAK["bf16_mfma_tflops"],
+                     "traffic": (MEASURED_TRAFFIC_KIB[dom_name] * 1024.0 if dom_name in MEASURED_TRAFFIC_KIB else None),
+                     "traffic_unit": "bytes per launch (counter runs, see profiles/)",
+                     "algorithmic_bytes_per_launch": dom["bytes"] / dom["launches"], "kernel": dom_name,
                      "avg_launch_us": avg_ms * 1e3, "launches_per_step": dom["launches"] // prof_steps,
                      "flops_per_launch": dom["flops"] / dom["launches"]},
         "step_mfma_frac": flops / dt / (PEAK["bf16_mfma_tflops"] * 1e12),
