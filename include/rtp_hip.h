@@ -201,6 +201,29 @@ int rtp_softmax_bwd(void* stream, int dtype, const void* p, const float* dp, flo
                     int64_t z, int64_t l, int64_t skv, void* ds);
 
 /* ---------------------------------------------------------------------------------------------
+ * Fused attention core for short sequences (reference: the per-head-group core of
+ * multi_head_attention_forward, rtp/module/functional.py:779-800 and :815-830: q k^T -> (+mask) softmax ->
+ * p v, and its autograd backward).  bf16 only, L <= 32, head dimension D in {32, 64, 128}
+ * (rtp_attn_supported says whether a shape qualifies; otherwise compose rtp_gemm + rtp_softmax_*).
+ * One wavefront per (group, batch, head); scores and probabilities never leave registers except for the
+ * stored p.  Element (l, b, h, g, dd) of q/k/v/dq/dk/dv is at base + l*s_l + b*s_b + h*s_h + g*s_g + dd, of
+ * o/dout at base + l*o_l + b*o_b + h*o_h + g*o_g + dd (strides in elements, multiples of 8; bases 16-byte
+ * aligned).  p is [G][N][H][L][L] bf16, written by fwd and read by bwd.  mask: additive fp32 [L][L] or
+ * NULL; causal != 0 hides keys j > i.  scale multiplies the scores before the mask is added.
+ *   fwd: p = softmax(scale * q k^T + mask), o = p v
+ *   bwd: dv = p^T dout, dp = dout v^T, ds = scale * p o (dp - rowsum(dp o p)), dq = ds k, dk = ds^T q
+ * --------------------------------------------------------------------------------------------- */
+int rtp_attn_supported(int dtype, int64_t L, int64_t D);
+int rtp_attn_fwd(void* stream, int dtype, const void* q, const void* k, const void* v, int64_t s_l,
+                 int64_t s_b, int64_t s_h, int64_t s_g, void* o, int64_t o_l, int64_t o_b, int64_t o_h,
+                 int64_t o_g, void* p, const float* mask, int causal, float scale, int64_t L, int64_t N,
+                 int64_t H, int64_t D, int64_t G);
+int rtp_attn_bwd(void* stream, int dtype, const void* q, const void* k, const void* v, int64_t s_l,
+                 int64_t s_b, int64_t s_h, int64_t s_g, const void* dout, int64_t o_l, int64_t o_b,
+                 int64_t o_h, int64_t o_g, const void* p, void* dq, void* dk, void* dv, float scale,
+                 int64_t L, int64_t N, int64_t H, int64_t D, int64_t G);
+
+/* ---------------------------------------------------------------------------------------------
  * Top-2 routing (reference: top2gating, rtp/module/top2gate.py:43-105).
  * Inputs logits[S,E] fp32 and noise[S,E] fp32 (the Gumbel sample of top2gate.py:61, supplied by the
  * caller so that routing is a pure function of its inputs).  Outputs, per token s:

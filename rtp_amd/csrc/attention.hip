@@ -1,0 +1,341 @@
+// Fused attention core for short sequences (L <= 32), bf16: one wavefront owns one (group, batch, head)
+// problem and keeps scores, probabilities and their gradients in registers.
+//
+//   forward : S^T = K Q^T (MFMA) -> softmax over keys (fp32, in registers) -> P stored (bf16) -> O^T = V^T P^T (MFMA)
+//   backward: dP^T = V dO^T -> dS = scale * P o (dP - rowsum(dP o P)) -> dQ^T = K^T dS^T, dK^T = Q^T dS, dV^T = dO^T P
+//
+// The transposed products are chosen so that the softmax axis (keys) lies along the accumulator REGISTERS
+// of a lane: MFMA 32x32 accumulator register r of lane (li, g) is row 8*(r/4) + 4*g + r%4, column li.  With
+// rows = keys and columns = queries a lane holds 16 keys of one query, its partner lane (li, 1-g) the other 16,
+// so a row reduction is 15 in-lane operations and one cross-lane exchange.  The same registers, rounded to
+// bf16, are directly the B operand of the next product: an MFMA contracts over "k slots" (8 per lane and
+// instruction), and which key sits in which slot is free as long as A and B agree; the A operand (V^T, K^T)
+// is gathered from LDS in the matching order.
+#include "common.h"
+
+namespace rtp {
+
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+
+struct AttnArgs {
+  // element (l, b, h, g, dd) of q/k/v (and dq/dk/dv) at base + l*s_l + b*s_b + h*s_h + g*s_g + dd
+  const bf16_t *q, *k, *v;
+  bf16_t *dq, *dk, *dv;
+  long s_l, s_b, s_h, s_g;
+  // element (l, b, h, g, dd) of o / dout at base + l*o_l + b*o_b + h*o_h + g*o_g + dd
+  bf16_t* o;
+  const bf16_t* dout;
+  long o_l, o_b, o_h, o_g;
+  bf16_t* p;          // probabilities [G][N][H][L][L]
+  const float* mask;  // additive [L][L] or null
+  int causal;
+  float scale;
+  int L, N, H;
+  long nprob;  // G * N * H
+};
+
+constexpr int kSeqMax = 32;
+constexpr int kPPitch = kSeqMax + 8;  // row pitch of the P / dS tiles in LDS
+
+// 32 x D tile (rows beyond L zero) global -> LDS with 16-byte accesses, row pitch D + 8 elements.
+template <int D>
+__device__ __forceinline__ void load_tile(bf16_t* tile, const bf16_t* base, long s_l, int L, int lane) {
+  constexpr int CPR = D / 8;
+  for (int c = lane; c < kSeqMax * CPR; c += kWave) {
+    const int row = c / CPR, cc = c % CPR;
+    uint4 val = make_uint4(0u, 0u, 0u, 0u);
+    if (row < L) val = *reinterpret_cast<const uint4*>(base + row * s_l + cc * 8);
+    *reinterpret_cast<uint4*>(tile + row * (D + 8) + cc * 8) = val;
+  }
+}
+
+// Operand fragment with the contraction index contiguous in the tile: row li, elements 16*ks + 8*g ...
+__device__ __forceinline__ bf16x8 frag_rowmajor(const bf16_t* tile, int pitch, int li, int g, int ks) {
+  return *reinterpret_cast<const bf16x8*>(tile + li * pitch + 16 * ks + 8 * g);
+}
+// Contraction index = tile row, in ACCUMULATOR order: slot e of instruction m in lane group g is row
+// 8*(2m + e/4) + 4g + e%4 (the row that accumulator register 8m + e of that lane group holds).
+__device__ __forceinline__ bf16x8 gather_acc_order(const bf16_t* tile, int pitch, int col, int m, int g) {
+  bf16x8 f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) f[e] = tile[(8 * (2 * m + (e >> 2)) + 4 * g + (e & 3)) * pitch + col];
+  return f;
+}
+// Contraction index = tile row, in natural order: slot e of instruction m in lane group g is row 16m + 8g + e.
+__device__ __forceinline__ bf16x8 gather_natural(const bf16_t* tile, int pitch, int col, int m, int g) {
+  bf16x8 f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) f[e] = tile[(16 * m + 8 * g + e) * pitch + col];
+  return f;
+}
+
+// Accumulator (rows = feature dd, columns = sequence position li) -> dst[li][32*db + dd], 4 consecutive dd
+// (8 bytes) per store.
+__device__ __forceinline__ void store_transposed(bf16_t* dst_row, int db, int g, const f32x16& acc) {
+#pragma unroll
+  for (int a4 = 0; a4 < 4; ++a4) {
+    union {
+      uint2 u;
+      bf16_t e[4];
+    } pk;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) pk.e[e] = from_f32<bf16_t>(acc[4 * a4 + e]);
+    *reinterpret_cast<uint2*>(dst_row + 32 * db + 8 * a4 + 4 * g) = pk.u;
+  }
+}
+
+struct Problem {
+  long z, qkv_off, o_off;
+  bool live;
+};
+__device__ __forceinline__ Problem locate(const AttnArgs& a, int waves_per_block) {
+  Problem pr;
+  pr.z = (long)blockIdx.x * waves_per_block + (threadIdx.x >> 6);
+  pr.live = pr.z < a.nprob;
+  if (!pr.live) pr.z = a.nprob - 1;  // idle waves redo the last problem and store nothing
+  const long h = pr.z % a.H, b = (pr.z / a.H) % a.N, g = pr.z / ((long)a.H * a.N);
+  pr.qkv_off = b * a.s_b + h * a.s_h + g * a.s_g;
+  pr.o_off = b * a.o_b + h * a.o_h + g * a.o_g;
+  return pr;
+}
+
+template <int DB, int NWV>
+__global__ __launch_bounds__(NWV * 64) void attn_fwd_small_kernel(AttnArgs a) {
+  constexpr int D = 32 * DB, P = D + 8;
+  __shared__ __attribute__((aligned(16))) bf16_t tiles[NWV][3][kSeqMax * P];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, li = lane & 31, g = lane >> 5;
+  const Problem pr = locate(a, NWV);
+  bf16_t* Qs = tiles[wave][0];
+  bf16_t* Ks = tiles[wave][1];
+  bf16_t* Vs = tiles[wave][2];
+  load_tile<D>(Qs, a.q + pr.qkv_off, a.s_l, a.L, lane);
+  load_tile<D>(Ks, a.k + pr.qkv_off, a.s_l, a.L, lane);
+  load_tile<D>(Vs, a.v + pr.qkv_off, a.s_l, a.L, lane);
+  __syncthreads();
+
+  // S^T[key][query]
+  f32x16 s;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) s[r] = 0.0f;
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ++ks)
+    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rowmajor(Ks, P, li, g, ks), frag_rowmajor(Qs, P, li, g, ks), s, 0,
+                                                0, 0);
+
+  // softmax over the keys of query li
+  const bool qlive = li < a.L;
+  float val[16];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int key = 8 * (r >> 2) + 4 * g + (r & 3);
+    const bool visible = key < a.L && (!a.causal || key <= li);
+    float x = s[r] * a.scale;
+    if (a.mask && qlive && key < a.L) x += a.mask[li * a.L + key];
+    val[r] = visible ? x : -INFINITY;
+    mx = fmaxf(mx, val[r]);
+  }
+  mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+  float sum = 0.0f;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int key = 8 * (r >> 2) + 4 * g + (r & 3);
+    const bool visible = key < a.L && (!a.causal || key <= li);
+    val[r] = visible ? expf(val[r] - mx) : 0.0f;
+    sum += val[r];
+  }
+  sum += __shfl_xor(sum, 32, kWave);
+  const float inv = 1.0f / sum;
+  bf16x8 pb[2];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) pb[r >> 3][r & 7] = from_f32<bf16_t>(val[r] * inv);
+  if (pr.live && qlive) {
+    bf16_t* prow = a.p + (pr.z * a.L + li) * a.L;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int key = 8 * (r >> 2) + 4 * g + (r & 3);
+      if (key < a.L) prow[key] = pb[r >> 3][r & 7];
+    }
+  }
+
+  // O^T[dd][query] = sum_key V[key][dd] P[query][key]
+#pragma unroll
+  for (int db = 0; db < DB; ++db) {
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_acc_order(Vs, P, 32 * db + li, m, g), pb[m], acc, 0, 0, 0);
+    if (pr.live && qlive) store_transposed(a.o + pr.o_off + li * a.o_l, db, g, acc);
+  }
+}
+
+template <int DB, int NWV>
+__global__ __launch_bounds__(NWV * 64) void attn_bwd_small_kernel(AttnArgs a) {
+  constexpr int D = 32 * DB, P = D + 8;
+  __shared__ __attribute__((aligned(16))) bf16_t tiles[NWV][4][kSeqMax * P];
+  __shared__ __attribute__((aligned(16))) bf16_t ptiles[NWV][2][kSeqMax * kPPitch];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, li = lane & 31, g = lane >> 5;
+  const Problem pr = locate(a, NWV);
+  bf16_t* Qs = tiles[wave][0];
+  bf16_t* Ks = tiles[wave][1];
+  bf16_t* Vs = tiles[wave][2];
+  bf16_t* Gs = tiles[wave][3];  // dO
+  bf16_t* DSs = ptiles[wave][0];
+  bf16_t* Ps = ptiles[wave][1];
+  load_tile<D>(Qs, a.q + pr.qkv_off, a.s_l, a.L, lane);
+  load_tile<D>(Ks, a.k + pr.qkv_off, a.s_l, a.L, lane);
+  load_tile<D>(Vs, a.v + pr.qkv_off, a.s_l, a.L, lane);
+  load_tile<D>(Gs, a.dout + pr.o_off, a.o_l, a.L, lane);
+  __syncthreads();
+
+  // dP^T[key][query] = sum_dd V[key][dd] dO[query][dd]
+  f32x16 dp;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) dp[r] = 0.0f;
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ++ks)
+    dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rowmajor(Vs, P, li, g, ks), frag_rowmajor(Gs, P, li, g, ks), dp, 0,
+                                                 0, 0);
+  const bool qlive = li < a.L;
+  const bf16_t* prow = a.p + (pr.z * a.L + (qlive ? li : 0)) * a.L;
+  float pv[16];
+  float dot = 0.0f;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int key = 8 * (r >> 2) + 4 * g + (r & 3);
+    pv[r] = (qlive && key < a.L) ? to_f32(prow[key]) : 0.0f;
+    dot += pv[r] * dp[r];
+  }
+  dot += __shfl_xor(dot, 32, kWave);
+  bf16x8 dsb[2];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) dsb[r >> 3][r & 7] = from_f32<bf16_t>(a.scale * pv[r] * (dp[r] - dot));
+  // dS and P as [query][key] tiles for the products that contract over the queries
+#pragma unroll
+  for (int a4 = 0; a4 < 4; ++a4) {
+    union {
+      uint2 u;
+      bf16_t e[4];
+    } d4, p4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      d4.e[e] = dsb[(4 * a4 + e) >> 3][(4 * a4 + e) & 7];
+      p4.e[e] = from_f32<bf16_t>(pv[4 * a4 + e]);
+    }
+    *reinterpret_cast<uint2*>(DSs + li * kPPitch + 8 * a4 + 4 * g) = d4.u;
+    *reinterpret_cast<uint2*>(Ps + li * kPPitch + 8 * a4 + 4 * g) = p4.u;
+  }
+  __syncthreads();
+
+  const bool store = pr.live && qlive;  // li is the query for dQ and the key for dK / dV; both run to L
+#pragma unroll
+  for (int db = 0; db < DB; ++db) {
+    f32x16 acc;
+    // dQ^T[dd][query] = sum_key K[key][dd] dS[query][key]
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_acc_order(Ks, P, 32 * db + li, m, g), dsb[m], acc, 0, 0, 0);
+    if (store) store_transposed(a.dq + pr.qkv_off + li * a.s_l, db, g, acc);
+    // dK^T[dd][key] = sum_query Q[query][dd] dS[query][key]
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_natural(Qs, P, 32 * db + li, m, g),
+                                                    gather_natural(DSs, kPPitch, li, m, g), acc, 0, 0, 0);
+    if (store) store_transposed(a.dk + pr.qkv_off + li * a.s_l, db, g, acc);
+    // dV^T[dd][key] = sum_query dO[query][dd] P[query][key]
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_natural(Gs, P, 32 * db + li, m, g),
+                                                    gather_natural(Ps, kPPitch, li, m, g), acc, 0, 0, 0);
+    if (store) store_transposed(a.dv + pr.qkv_off + li * a.s_l, db, g, acc);
+  }
+}
+
+static bool aligned8(int64_t v) { return v % 8 == 0; }
+
+static int check_common(const char* who, int dtype, int64_t L, int64_t N, int64_t H, int64_t D, int64_t G, int64_t s_l,
+                        int64_t s_b, int64_t s_h, int64_t s_g, int64_t o_l, int64_t o_b, int64_t o_h, int64_t o_g) {
+  RTP_REQUIRE(dtype == RTP_BF16, "%s: only bf16 is implemented (dtype %d)", who, dtype);
+  RTP_REQUIRE(L >= 1 && L <= kSeqMax, "%s: sequence length %lld not in 1..%d", who, (long long)L, kSeqMax);
+  RTP_REQUIRE(D == 32 || D == 64 || D == 128, "%s: head dimension %lld not in {32, 64, 128}", who, (long long)D);
+  RTP_REQUIRE(N >= 1 && H >= 1 && G >= 1, "%s: batch, heads and groups must be >= 1", who);
+  RTP_REQUIRE(aligned8(s_l) && aligned8(s_b) && aligned8(s_h) && aligned8(s_g) && aligned8(o_l) && aligned8(o_b) &&
+                  aligned8(o_h) && aligned8(o_g),
+              "%s: strides must be multiples of 8 elements", who);
+  RTP_REQUIRE(ceil_div(G * N * H, 2) < (1ll << 31), "%s: too many problems", who);
+  return RTP_OK;
+}
+
+}  // namespace rtp
+
+using namespace rtp;
+
+extern "C" int rtp_attn_supported(int dtype, int64_t L, int64_t D) {
+  return dtype == RTP_BF16 && L >= 1 && L <= kSeqMax && (D == 32 || D == 64 || D == 128);
+}
+
+extern "C" int rtp_attn_fwd(void* stream, int dtype, const void* q, const void* k, const void* v, int64_t s_l,
+                            int64_t s_b, int64_t s_h, int64_t s_g, void* o, int64_t o_l, int64_t o_b, int64_t o_h,
+                            int64_t o_g, void* p, const float* mask, int causal, float scale, int64_t L, int64_t N,
+                            int64_t H, int64_t D, int64_t G) {
+  RTP_REQUIRE(q && k && v && o && p, "rtp_attn_fwd: null pointer");
+  if (int rc = check_common("rtp_attn_fwd", dtype, L, N, H, D, G, s_l, s_b, s_h, s_g, o_l, o_b, o_h, o_g)) return rc;
+  RTP_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o) % 16 == 0,
+              "rtp_attn_fwd: q, k, v, o must be 16-byte aligned");
+  AttnArgs a{};
+  a.q = (const bf16_t*)q, a.k = (const bf16_t*)k, a.v = (const bf16_t*)v;
+  a.s_l = s_l, a.s_b = s_b, a.s_h = s_h, a.s_g = s_g;
+  a.o = (bf16_t*)o, a.o_l = o_l, a.o_b = o_b, a.o_h = o_h, a.o_g = o_g;
+  a.p = (bf16_t*)p, a.mask = mask, a.causal = causal, a.scale = scale;
+  a.L = (int)L, a.N = (int)N, a.H = (int)H, a.nprob = G * N * H;
+  hipStream_t st = (hipStream_t)stream;
+  const double np = (double)a.nprob;
+  ProfileScope prof(st, "attn_fwd_small", 4.0 * np * L * L * D, np * (4.0 * L * D + (double)L * L) * 2.0);
+  const unsigned grid = (unsigned)ceil_div(a.nprob, 4);
+  if (D == 32)
+    hipLaunchKernelGGL((attn_fwd_small_kernel<1, 4>), dim3(grid), dim3(256), 0, st, a);
+  else if (D == 64)
+    hipLaunchKernelGGL((attn_fwd_small_kernel<2, 4>), dim3(grid), dim3(256), 0, st, a);
+  else
+    hipLaunchKernelGGL((attn_fwd_small_kernel<4, 4>), dim3(grid), dim3(256), 0, st, a);
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
+}
+
+extern "C" int rtp_attn_bwd(void* stream, int dtype, const void* q, const void* k, const void* v, int64_t s_l,
+                            int64_t s_b, int64_t s_h, int64_t s_g, const void* dout, int64_t o_l, int64_t o_b,
+                            int64_t o_h, int64_t o_g, const void* p, void* dq, void* dk, void* dv, float scale,
+                            int64_t L, int64_t N, int64_t H, int64_t D, int64_t G) {
+  RTP_REQUIRE(q && k && v && dout && p && dq && dk && dv, "rtp_attn_bwd: null pointer");
+  if (int rc = check_common("rtp_attn_bwd", dtype, L, N, H, D, G, s_l, s_b, s_h, s_g, o_l, o_b, o_h, o_g)) return rc;
+  RTP_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)dout | (uintptr_t)dq | (uintptr_t)dk |
+               (uintptr_t)dv) % 16 == 0,
+              "rtp_attn_bwd: q, k, v, dout, dq, dk, dv must be 16-byte aligned");
+  AttnArgs a{};
+  a.q = (const bf16_t*)q, a.k = (const bf16_t*)k, a.v = (const bf16_t*)v;
+  a.dq = (bf16_t*)dq, a.dk = (bf16_t*)dk, a.dv = (bf16_t*)dv;
+  a.s_l = s_l, a.s_b = s_b, a.s_h = s_h, a.s_g = s_g;
+  a.dout = (const bf16_t*)dout, a.o_l = o_l, a.o_b = o_b, a.o_h = o_h, a.o_g = o_g;
+  a.p = (bf16_t*)const_cast<void*>(p), a.scale = scale;
+  a.L = (int)L, a.N = (int)N, a.H = (int)H, a.nprob = G * N * H;
+  hipStream_t st = (hipStream_t)stream;
+  const double np = (double)a.nprob;
+  ProfileScope prof(st, "attn_bwd_small", 8.0 * np * L * L * D, np * (7.0 * L * D + (double)L * L) * 2.0);
+  if (D == 32)
+    hipLaunchKernelGGL((attn_bwd_small_kernel<1, 4>), dim3((unsigned)ceil_div(a.nprob, 4)), dim3(256), 0, st, a);
+  else if (D == 64)
+    hipLaunchKernelGGL((attn_bwd_small_kernel<2, 4>), dim3((unsigned)ceil_div(a.nprob, 4)), dim3(256), 0, st, a);
+  else
+    hipLaunchKernelGGL((attn_bwd_small_kernel<4, 2>), dim3((unsigned)ceil_div(a.nprob, 2)), dim3(128), 0, st, a);
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
+}

@@ -118,6 +118,7 @@ class _AttentionFn(torch.autograd.Function):
         o = torch.empty(rows, E, dtype=dt, device=dev)
         out = torch.empty(rows, E, dtype=dt, device=dev)
         ldq = N * ws * 3 * e_s
+        fused = ops.attn_supported(dt, L, d)
         order = ring_order(layer.rank, ws)
         rot = Rotation(store.home, order)
         acc = ops.ShardSum(out, sum(len(w) for w in rot.windows))
@@ -125,8 +126,17 @@ class _AttentionFn(torch.autograd.Function):
         for j in range(rot.steps):
             for flat, first, cnt in rot.acquire(j):
                 S.col_fwd(x2, flat, 0, 3 * e_s, E, b_in_off, qkv, first * 3 * e_s)
-                scores = torch.empty(cnt * Z, L, L, dtype=torch.float32, device=dev)
                 q0 = first * 3 * e_s
+                if fused:
+                    # scores, softmax and p v in one launch, one wavefront per (group, batch, head)
+                    ops.attn_fwd(qkv, q0, q0 + e_s, q0 + 2 * e_s, (ldq, ws * 3 * e_s, d, 3 * e_s), o, first * e_s,
+                                 (N * E, E, d, e_s), p[first * Z:(first + cnt) * Z], mask, causal, scale, L, N, h_s,
+                                 d, cnt)
+                    c_out, c_in = acc.target(i)
+                    S.row_fwd(o, flat, w_o_off, E, e_s, b_o_off, c_out, first * e_s, c_in=c_in)
+                    i += 1
+                    continue
+                scores = torch.empty(cnt * Z, L, L, dtype=torch.float32, device=dev)
                 _bmm(dt, a=qkv, a_off=q0, lda=ldq, a_kc=True, a_s=(ws * 3 * e_s, d), a_sg=3 * e_s, b=qkv,
                      b_off=q0 + e_s, ldb=ldq, b_kc=True, b_s=(ws * 3 * e_s, d), b_sg=3 * e_s, c=scores, c_off=0, ldc=L,
                      c_s=(h_s * L * L, L * L), c_sg=Z * L * L, m=L, n=L, k=d, batch=Z, zdiv=h_s, groups=cnt,
@@ -169,6 +179,7 @@ class _AttentionFn(torch.autograd.Function):
         do = torch.empty(rows, E, dtype=dt, device=dev)
         dqkv = torch.empty(rows, ws * 3 * e_s, dtype=dt, device=dev)
         ldq = N * ws * 3 * e_s
+        fused = ops.attn_supported(dt, L, d)
         order = ring_order(layer.rank, ws, reverse=True)
         rot = Rotation(store.home, order)
         acc = ops.ShardSum(dx, sum(len(w) for w in rot.windows)) if need_dx else None
@@ -178,6 +189,14 @@ class _AttentionFn(torch.autograd.Function):
                 q0 = first * 3 * e_s
                 # out-projection: dO_g = dOut W_o,g
                 S.row_dgrad(dout2, flat, w_o_off, E, e_s, do, first * e_s)
+                if fused:
+                    ops.attn_bwd(qkv, q0, q0 + e_s, q0 + 2 * e_s, (ldq, ws * 3 * e_s, d, 3 * e_s), do, first * e_s,
+                                 (N * E, E, d, e_s), p[first * Z:(first + cnt) * Z], dqkv, scale, L, N, h_s, d, cnt)
+                    if need_dx:
+                        c_out, c_in = acc.target(i)
+                        S.col_dgrad(dqkv, flat, 0, 3 * e_s, E, c_out, q0, c_in=c_in)
+                    i += 1
+                    continue
                 # attention core, all (group, batch, head) triples of the run in one launch each
                 dp = torch.empty(cnt * Z, L, L, dtype=torch.float32, device=dev)
                 _bmm(dt, a=do, a_off=first * e_s, lda=N * E, a_kc=True, a_s=(E, d), a_sg=e_s, b=qkv, b_off=q0 + 2 * e_s,

@@ -258,6 +258,48 @@ def softmax_bwd(p: torch.Tensor, dp: torch.Tensor, ds: torch.Tensor, scale: floa
                                       ds.data_ptr()))
 
 
+def attn_supported(dtype: torch.dtype, L: int, d: int) -> bool:
+    """Whether the fused short-sequence attention core handles this shape (bf16, L <= 32, d in {32, 64, 128})."""
+    if dtype != torch.bfloat16:
+        return False
+    return bool(_lib.load().rtp_attn_supported(dtype_code(dtype), L, d))
+
+
+def attn_fwd(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, qkv_strides, o: torch.Tensor, o_off: int,
+             o_strides, p: torch.Tensor, mask: Optional[torch.Tensor], causal: bool, scale: float, L: int, N: int,
+             H: int, d: int, G: int) -> None:
+    """Fused q k^T -> softmax -> p v for G*N*H (group, batch, head) problems addressed by element strides
+    (s_l, s_b, s_h, s_g) into the packed projection `qkv` (offsets in elements) and `o`; p [G*N*H, L, L]."""
+    _dev(qkv)
+    esz = qkv.element_size()
+    if p.dtype != qkv.dtype or o.dtype != qkv.dtype or not p.is_contiguous() or p.numel() != G * N * H * L * L:
+        raise ValueError("attn_fwd: p must be contiguous [G*N*H, L, L] of the operand dtype")
+    if mask is not None and (mask.dtype != torch.float32 or tuple(mask.shape) != (L, L) or not mask.is_contiguous()):
+        raise ValueError("attn_fwd: mask must be a contiguous fp32 [L, L] tensor")
+    _lib.require_device()
+    base = qkv.data_ptr()
+    check(_lib.load().rtp_attn_fwd(_stream(), dtype_code(qkv.dtype), base + q_off * esz, base + k_off * esz,
+                                   base + v_off * esz, *qkv_strides, o.data_ptr() + o_off * esz, *o_strides,
+                                   p.data_ptr(), mask.data_ptr() if mask is not None else None, int(causal), scale,
+                                   L, N, H, d, G))
+
+
+def attn_bwd(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, qkv_strides, dout: torch.Tensor, o_off: int,
+             o_strides, p: torch.Tensor, dqkv: torch.Tensor, scale: float, L: int, N: int, H: int, d: int,
+             G: int) -> None:
+    """Backward of attn_fwd: writes dq, dk, dv into `dqkv` (same layout and offsets as `qkv`)."""
+    _dev(qkv)
+    esz = qkv.element_size()
+    if dqkv.dtype != qkv.dtype or dqkv.shape != qkv.shape or dqkv.stride() != qkv.stride() or dout.dtype != qkv.dtype:
+        raise ValueError("attn_bwd: dqkv must match qkv, dout must share its dtype")
+    _lib.require_device()
+    base, dbase = qkv.data_ptr(), dqkv.data_ptr()
+    check(_lib.load().rtp_attn_bwd(_stream(), dtype_code(qkv.dtype), base + q_off * esz, base + k_off * esz,
+                                   base + v_off * esz, *qkv_strides, dout.data_ptr() + o_off * esz, *o_strides,
+                                   p.data_ptr(), dbase + q_off * esz, dbase + k_off * esz, dbase + v_off * esz, scale,
+                                   L, N, H, d, G))
+
+
 def sgd_step(master: torch.Tensor, grad: torch.Tensor, shadow: Optional[torch.Tensor], lr: float,
              clip: float = 0.0) -> None:
     _dev(master)

@@ -98,3 +98,69 @@ def test_attention_unsupported_raise():
         layer(x, x, x, key_padding_mask=torch.zeros(2, 4, dtype=torch.bool, device=DEV))
     with pytest.raises(NotImplementedError):
         ParallelMultiheadAttention(8, 2, 2, 0, kdim=4, device=DEV)
+
+
+@pytest.mark.parametrize("E,H,L,N,ws,masked,need_weights", [
+    (128, 4, 32, 3, 2, True, False),     # head_dim 32, full 32-token tile
+    (256, 4, 7, 5, 4, False, True),      # head_dim 64, ragged L, returned weights
+    (512, 4, 19, 2, 2, True, True),      # head_dim 128
+    (2048, 32, 32, 4, 8, True, False),   # the LM layer: 32 heads in 8 groups, seq 32
+])
+def test_attention_fused_short_sequence_bf16(E, H, L, N, ws, masked, need_weights):
+    """bf16 with L <= 32 takes the fused core (one wavefront per head); same oracle, same tolerance."""
+    from rtp_amd import ops
+    assert ops.attn_supported(torch.bfloat16, L, E // H)
+    _run(E, H, L, N, ws, torch.bfloat16, masked, need_weights, seed=4)
+
+
+@pytest.mark.parametrize("L,d,causal,use_mask", [(32, 64, True, False), (13, 32, False, True), (32, 128, False, False),
+                                                 (1, 64, True, False)])
+def test_attn_core_against_torch_fp32(L, d, causal, use_mask):
+    """rtp_attn_fwd / rtp_attn_bwd through the C ABI on a packed [L, N, G*3*H*d] projection, against plain
+    fp32 torch attention on the same bf16 inputs (tolerance 2e-2 of the largest reference entry)."""
+    from rtp_amd import ops
+    gen = torch.Generator().manual_seed(L * 131 + d)
+    N, H, G = 3, 2, 2
+    e_s = H * d
+    qkv = (torch.randn(L, N, G * 3 * e_s, generator=gen) * 0.5).to(torch.bfloat16)
+    dout = torch.randn(L, N, G * e_s, generator=gen).to(torch.bfloat16)
+    mask = (torch.randn(L, L, generator=gen) * 2.0) if use_mask else None
+    scale = 1.0 / d ** 0.5
+    # reference
+    x = qkv.float().view(L, N, G, 3, H, d).requires_grad_()
+    q, k, v = x[:, :, :, 0], x[:, :, :, 1], x[:, :, :, 2]                 # [L, N, G, H, d]
+    s = torch.einsum("lnghd,mnghd->nghlm", q, k) * scale
+    if mask is not None:
+        s = s + mask
+    if causal:
+        s = s + _causal(L)
+    p_ref = torch.softmax(s, dim=-1)
+    o_ref = torch.einsum("nghlm,mnghd->lnghd", p_ref, v).reshape(L, N, G * e_s)
+    o_ref.backward(dout.float())
+    # device
+    qd, dd = qkv.to(DEV), dout.to(DEV)
+    o = torch.empty(L, N, G * e_s, dtype=torch.bfloat16, device=DEV)
+    p = torch.empty(G * N * H, L, L, dtype=torch.bfloat16, device=DEV)
+    dqkv = torch.zeros_like(qd)
+    ld = G * 3 * e_s
+    qs, os_ = (N * ld, ld, d, 3 * e_s), (N * G * e_s, G * e_s, d, e_s)
+    ops.attn_fwd(qd, 0, e_s, 2 * e_s, qs, o, 0, os_, p, None if mask is None else mask.to(DEV), causal, scale,
+                 L, N, H, d, G)
+    ops.attn_bwd(qd, 0, e_s, 2 * e_s, qs, dd, 0, os_, p, dqkv, scale, L, N, H, d, G)
+    assert_close(o, o_ref, torch.bfloat16, "o")
+    assert_close(p.view(G, N, H, L, L), p_ref.permute(1, 0, 2, 3, 4), torch.bfloat16, "p")
+    assert_close(dqkv, x.grad.reshape(L, N, ld), torch.bfloat16, "dqkv")
+
+
+def test_attn_core_rejects_unsupported():
+    from rtp_amd import ops
+    from rtp_amd._lib import RtpError
+    assert not ops.attn_supported(torch.float32, 16, 64)
+    assert not ops.attn_supported(torch.bfloat16, 33, 64)
+    assert not ops.attn_supported(torch.bfloat16, 16, 48)
+    qkv = torch.zeros(33, 1, 3 * 64, dtype=torch.bfloat16, device=DEV)
+    o = torch.zeros(33, 1, 64, dtype=torch.bfloat16, device=DEV)
+    p = torch.zeros(1, 33, 33, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RtpError):
+        ops.attn_fwd(qkv, 0, 64, 128, (192, 192, 64, 192), o, 0, (64, 64, 64, 64), p, None, False, 0.125, 33, 1, 1,
+                     64, 1)
