@@ -224,6 +224,24 @@ int rtp_attn_bwd(void* stream, int dtype, const void* q, const void* k, const vo
                  int64_t L, int64_t N, int64_t H, int64_t D, int64_t G);
 
 /* ---------------------------------------------------------------------------------------------
+ * Residual add + LayerNorm of the post-LN decoder layer (reference: norm1(x + sa_block(x)) and
+ * norm2(x + ff_block(x)), rtp/models/transformer_lm_rtp.py:176-177, there two ATen calls each way).
+ *   fwd: z = x + r (rounded to `dtype`; r NULL: z = x, z_out unused), y = (z - mean) * rstd * gamma + beta,
+ *        mean / rstd fp32 [rows].  z_out is what bwd needs.
+ *   bwd: dz = rstd * (g - mean_c(g) - zhat * mean_c(g * zhat)), g = dy * gamma, zhat = (z - mean) * rstd;
+ *        dgamma = sum_rows dy * zhat, dbeta = sum_rows dy (dbeta may be NULL); fixed summation order.
+ * fp32 or bf16, rows contiguous, cols a multiple of 16 bytes and <= 2048 (rtp_layernorm_supported).
+ * --------------------------------------------------------------------------------------------- */
+int rtp_layernorm_supported(int dtype, int64_t cols);
+int rtp_add_layernorm_fwd(void* stream, int dtype, const void* x, const void* r, const void* gamma,
+                          const void* beta, float eps, int64_t rows, int64_t cols, void* z_out, void* y,
+                          float* mean, float* rstd);
+size_t rtp_layernorm_bwd_workspace_bytes(int64_t rows, int64_t cols);
+int rtp_layernorm_bwd(void* stream, int dtype, const void* dy, const void* z, const void* gamma,
+                      const float* mean, const float* rstd, int64_t rows, int64_t cols, void* dz,
+                      void* dgamma, void* dbeta, void* workspace, size_t workspace_bytes);
+
+/* ---------------------------------------------------------------------------------------------
  * Top-2 routing (reference: top2gating, rtp/module/top2gate.py:43-105).
  * Inputs logits[S,E] fp32 and noise[S,E] fp32 (the Gumbel sample of top2gate.py:61, supplied by the
  * caller so that routing is a pure function of its inputs).  Outputs, per token s:

@@ -1,7 +1,7 @@
 """GPT-2 style nn.Sequential language model built from the rotated layers (counterpart of
 rtp/models/transformer_lm_rtp.py:19-242): embedding * sqrt(ninp) -> sinusoidal positions -> N post-LN
 decoder layers (rotated self-attention + rotated ReLU FFN or rotated MoE) -> rotated logits projection.
-LayerNorm, residual adds, ReLU and dropout are ordinary torch ops."""
+Residual add + LayerNorm is one fused kernel each way (module/norm.py); ReLU and dropout are ordinary torch ops."""
 from __future__ import annotations
 
 import math
@@ -14,6 +14,7 @@ from ..module.collectives import emulate_shards
 from ..module.embedding import ParallelEmbedding
 from ..module.linear import ColumnParallelLinear
 from ..module.moe import WeightMOELayer
+from ..module.norm import add_layer_norm
 from ..module.top2gate import WeightTop2Gate
 
 
@@ -105,8 +106,8 @@ class TransformerEncoderLayer(nn.Module):
             x = x + self._sa_block(self.norm1(x), src_mask, src_key_padding_mask)
             x = x + self._ff_block(self.norm2(x))
         else:
-            x = self.norm1(x + self._sa_block(x, src_mask, src_key_padding_mask))
-            x = self.norm2(x + self._ff_block(x))
+            x = add_layer_norm(x, self._sa_block(x, src_mask, src_key_padding_mask), self.norm1)
+            x = add_layer_norm(x, self._ff_block(x), self.norm2)
         return x
 
     def _sa_block(self, x, attn_mask, key_padding_mask):

@@ -1,0 +1,44 @@
+"""Residual add fused with LayerNorm for the post-LN decoder layers (the reference computes
+norm1(x + sa_block(x)) / norm2(x + ff_block(x)) with two ATen calls each way,
+rtp/models/transformer_lm_rtp.py:176-177).  The LayerNorm parameters stay ordinary nn.LayerNorm parameters."""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from .. import ops
+
+
+class _AddLayerNormFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, r, weight, bias, eps):
+        x2, r2 = x.contiguous(), r.contiguous()
+        cols = x2.shape[-1]
+        rows = x2.numel() // cols
+        z = torch.empty_like(x2)
+        y = torch.empty_like(x2)
+        mean = torch.empty(rows, dtype=torch.float32, device=x2.device)
+        rstd = torch.empty(rows, dtype=torch.float32, device=x2.device)
+        ops.add_layernorm_fwd(x2, r2, weight, bias, eps, z, y, mean, rstd)
+        ctx.save_for_backward(z, weight, mean, rstd)
+        ctx.has_bias = bias is not None
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        z, weight, mean, rstd = ctx.saved_tensors
+        dz = torch.empty_like(z)
+        dgamma = torch.empty_like(weight)
+        dbeta = torch.empty_like(weight) if ctx.has_bias else None
+        ops.layernorm_bwd(dy.contiguous(), z, weight, mean, rstd, dz, dgamma, dbeta)
+        return dz, dz, dgamma, dbeta, None
+
+
+def add_layer_norm(x: torch.Tensor, r: torch.Tensor, norm: nn.LayerNorm) -> torch.Tensor:
+    """norm(x + r).  Fused on the device when the row length qualifies, else the two torch calls."""
+    fused = (x.is_cuda and x.shape == r.shape and x.dtype == r.dtype and norm.elementwise_affine
+             and len(norm.normalized_shape) == 1 and norm.normalized_shape[0] == x.shape[-1]
+             and norm.weight.dtype == x.dtype and ops.layernorm_supported(x.dtype, x.shape[-1]))
+    if not fused:
+        return norm(x + r)
+    return _AddLayerNormFn.apply(x, r, norm.weight, norm.bias, norm.eps)

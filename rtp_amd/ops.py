@@ -300,6 +300,51 @@ def attn_bwd(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, qkv_strides,
                                    L, N, H, d, G))
 
 
+def layernorm_supported(dtype: torch.dtype, cols: int) -> bool:
+    if dtype not in (torch.float32, torch.bfloat16):
+        return False
+    return bool(_lib.load().rtp_layernorm_supported(dtype_code(dtype), cols))
+
+
+def add_layernorm_fwd(x: torch.Tensor, r: Optional[torch.Tensor], gamma: torch.Tensor, beta: Optional[torch.Tensor],
+                      eps: float, z: Optional[torch.Tensor], y: torch.Tensor, mean: torch.Tensor,
+                      rstd: torch.Tensor) -> None:
+    """y = LayerNorm(x + r) over the last axis; z receives x + r; mean / rstd are fp32 [rows]."""
+    _dev(x)
+    cols = x.shape[-1]
+    rows = x.numel() // max(cols, 1)
+    tensors = [t for t in (x, r, z, y) if t is not None]
+    if any(t.dtype != x.dtype or t.shape != x.shape or not t.is_contiguous() for t in tensors):
+        raise ValueError("add_layernorm_fwd: x, r, z, y must be contiguous, of one shape and dtype")
+    if gamma.dtype != x.dtype or gamma.numel() != cols or (beta is not None and (beta.dtype != x.dtype or
+                                                                                  beta.numel() != cols)):
+        raise ValueError("add_layernorm_fwd: gamma / beta must be vectors of the row length in x's dtype")
+    if mean.dtype != torch.float32 or rstd.dtype != torch.float32 or mean.numel() != rows or rstd.numel() != rows:
+        raise ValueError("add_layernorm_fwd: mean / rstd must be fp32 [rows]")
+    _lib.require_device()
+    check(_lib.load().rtp_add_layernorm_fwd(
+        _stream(), dtype_code(x.dtype), x.data_ptr(), r.data_ptr() if r is not None else None, gamma.data_ptr(),
+        beta.data_ptr() if beta is not None else None, eps, rows, cols, z.data_ptr() if z is not None else None,
+        y.data_ptr(), mean.data_ptr(), rstd.data_ptr()))
+
+
+def layernorm_bwd(dy: torch.Tensor, z: torch.Tensor, gamma: torch.Tensor, mean: torch.Tensor, rstd: torch.Tensor,
+                  dz: torch.Tensor, dgamma: torch.Tensor, dbeta: Optional[torch.Tensor]) -> None:
+    _dev(dy)
+    cols = z.shape[-1]
+    rows = z.numel() // max(cols, 1)
+    if any(t.dtype != z.dtype or t.shape != z.shape or not t.is_contiguous() for t in (dy, dz)) or \
+            not z.is_contiguous():
+        raise ValueError("layernorm_bwd: dy, z, dz must be contiguous, of one shape and dtype")
+    _lib.require_device()
+    lib = _lib.load()
+    nbytes = lib.rtp_layernorm_bwd_workspace_bytes(rows, cols)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=z.device)
+    check(lib.rtp_layernorm_bwd(_stream(), dtype_code(z.dtype), dy.data_ptr(), z.data_ptr(), gamma.data_ptr(),
+                                mean.data_ptr(), rstd.data_ptr(), rows, cols, dz.data_ptr(), dgamma.data_ptr(),
+                                dbeta.data_ptr() if dbeta is not None else None, ws.data_ptr(), nbytes))
+
+
 def sgd_step(master: torch.Tensor, grad: torch.Tensor, shadow: Optional[torch.Tensor], lr: float,
              clip: float = 0.0) -> None:
     _dev(master)
