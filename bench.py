@@ -99,6 +99,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--sgd-overlap", dest="sgd_overlap", action="store_true",
+                    help="apply each rotated layer's SGD update right after that layer's backward, on a second stream "
+                         "(measured: no gain, the update and the backward compete for memory bandwidth)")
     ap.add_argument("--no-graph", dest="graph", action="store_false",
                     help="launch every kernel eagerly instead of replaying the step from a captured HIP graph")
     args = ap.parse_args()
@@ -116,7 +119,7 @@ def main():
     torch.cuda.set_device(dev)
     c = CFG
     lm = build(c, dev, torch.bfloat16)
-    opt = RotatedSGD(lm, lr=1e-3, clip_value=0.05)
+    opt = RotatedSGD(lm, lr=1e-3, clip_value=0.05, overlap_backward=args.sgd_overlap)
     gen = torch.Generator().manual_seed(0)
     ids = torch.randint(0, c["vocab"], (c["seq"], c["batch"]), generator=gen).to(dev)
     tgt = torch.randint(0, c["vocab"], (c["seq"], c["batch"]), generator=gen).to(dev)
@@ -189,7 +192,8 @@ def main():
         "config": {"workload": "10-layer RTP transformer LM fwd+bwd+SGD step: vocab 10240, ninp 2048, nhid 2048, "
                                "32 heads, seq 32, batch 32, bf16 weights + fp32 master, 8 rotation shards emulated on "
                                "one GPU, uniform random token ids, weights U(-0.1,0.1), dropout 0, lr 1e-3, clip 0.05",
-                   "tokens_per_step": tokens, "rotation_shards": c["shards"], "hip_graph": bool(args.graph)},
+                   "tokens_per_step": tokens, "rotation_shards": c["shards"], "hip_graph": bool(args.graph),
+                   "sgd_overlapped_with_backward": bool(args.sgd_overlap)},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK["bf16_mfma_tflops"], "unit": "TFLOP/s",
                      "frac": achieved / PEAK["bf16_mfma_tflops"],
                      "traffic": (MEASURED_TRAFFIC_KIB[dom_name] * 1024.0 if dom_name in MEASURED_TRAFFIC_KIB else None),

@@ -230,6 +230,7 @@ class _AttentionFn(torch.autograd.Function):
             if layer.has_bias:
                 S.row_bgrad(dout2, store.grads, first, b_o_off, E, cnt, accumulate)
                 S.col_bgrad(dqkv, store.grads, first, b_in_off, 3 * e_s, first * 3 * e_s, cnt, accumulate)
+        store.grads_ready()
         return (dx.view(L, N, E) if need_dx else None), None, None, None, None, None
 
 

@@ -76,6 +76,7 @@ class ShardStore:
         self.home: Optional[torch.Tensor] = None
         self.grads: Optional[torch.Tensor] = None
         self._overwrite = set()
+        self.on_grads_ready = None  # optional callable(store): the layer's backward has written every gradient row
         self.pack()
 
     # -- storage ---------------------------------------------------------------------------------
@@ -162,6 +163,12 @@ class ShardStore:
                 runs.append((start, a - start + 1, flags[a]))
                 start = b
         return runs
+
+    def grads_ready(self) -> None:
+        """Called by a layer at the end of its backward, after the last kernel that writes `grads` has been
+        launched on the current stream."""
+        if self.on_grads_ready is not None:
+            self.on_grads_ready(self)
 
     def weight_bytes(self) -> int:
         return self.world_size * self.numel * self.home.element_size()

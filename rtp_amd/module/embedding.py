@@ -74,6 +74,7 @@ class _EmbeddingFn(torch.autograd.Function):
             ops.embedding_scatter_add(g2[:, idx * d_s:(idx + 1) * d_s], flat_ids.numel(), workspace, grads[0],
                                       padding_idx=pad, scale_by_freq=layer.scale_grad_by_freq,
                                       zero_fill=not accumulate)
+        store.grads_ready()
         return None, None, None
 
 

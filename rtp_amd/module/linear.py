@@ -107,6 +107,7 @@ class _ColumnLinearFn(torch.autograd.Function):
             S.col_wgrad(dy2, x2, store.grads, first, 0, n_s, k, first * n_s, cnt, accumulate)
             if layer.has_bias:
                 S.col_bgrad(dy2, store.grads, first, n_s * k, n_s, first * n_s, cnt, accumulate)
+        store.grads_ready()
         return (dx.view(ctx.x_shape) if need_dx else None), None, None
 
 
@@ -153,6 +154,7 @@ class _RowLinearFn(torch.autograd.Function):
             S.row_wgrad(dy2, x2, store.grads, first, 0, n, k_s, first * k_s, cnt, accumulate)
             if layer.has_bias:
                 S.row_bgrad(dy2, store.grads, first, n * k_s, n, cnt, accumulate)
+        store.grads_ready()
         return (dx.view(ctx.x_shape) if need_dx else None), None, None
 
 

@@ -145,6 +145,7 @@ class _ExpertsFn(torch.autograd.Function):
                     r = (s * n_local + le) * c_rows
                     ops.colsum(dy[r:r + c_rows], g[s, b2:b2 + m_dim], accumulate=accumulate)
                     ops.colsum(dh[r:r + c_rows], g[s, b1:b1 + f_dim], accumulate=accumulate)
+        store.grads_ready()
         return dx, None, None
 
 

@@ -113,6 +113,7 @@ class _GateProjectionFn(torch.autograd.Function):
                 rot.release(j)
         for first, cnt, accumulate in store.grad_runs(order):
             S.col_wgrad(dl, x2, store.grads, first, 0, e_s, layer.model_dim, first * e_s, cnt, accumulate)
+        store.grads_ready()
         return dx, None, None
 
 

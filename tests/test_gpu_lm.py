@@ -168,3 +168,41 @@ def test_lm_moe_variant_runs_and_backprops():
     (out.float().mean() + lm[2].moe_layer.l_aux).backward()
     for p in lm.parameters():
         assert p.grad is not None and torch.isfinite(p.grad).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_lm_sgd_overlapped_with_backward_is_bit_identical(dtype):
+    """overlap_backward=True updates each rotated layer right after its backward on a second stream; after
+    step() every weight, master and gradient equals the sequential optimiser's, step after step."""
+    from rtp_amd.optim import RotatedSGD
+    V, D, H, Fd, n_dec, L, N, ws = 64, 32, 4, 64, 2, 6, 3, 4
+    lm_a, _ = build_pair(V, D, H, Fd, n_dec, ws, dtype, seed=5)
+    lm_b, _ = build_pair(V, D, H, Fd, n_dec, ws, dtype, seed=5)
+    opt_a = RotatedSGD(lm_a, lr=0.05, clip_value=0.05)
+    opt_b = RotatedSGD(lm_b, lr=0.05, clip_value=0.05, overlap_backward=True)
+    gen = torch.Generator().manual_seed(0)
+    for step in range(3):
+        ids = torch.randint(0, V, (L, N), generator=gen).to(DEV)
+        for lm, opt in ((lm_a, opt_a), (lm_b, opt_b)):
+            opt.zero_grad()
+            F.cross_entropy(lm(ids).float().view(-1, V), ids.view(-1)).backward()
+            opt.step()
+        torch.cuda.synchronize()
+        for (na, pa), (nb, pb) in zip(lm_a.named_parameters(), lm_b.named_parameters()):
+            assert na == nb and torch.equal(pa, pb), f"step {step}: {na} differs"
+            assert torch.equal(pa.grad, pb.grad), f"step {step}: grad of {na} differs"
+        for ma, mb in zip(opt_a.masters, opt_b.masters):
+            assert (ma is None and mb is None) or torch.equal(ma, mb)
+
+
+def test_lm_sgd_overlap_rejects_gradient_accumulation():
+    from rtp_amd.optim import RotatedSGD
+    V, D, H, Fd, n_dec, L, N, ws = 64, 32, 2, 32, 1, 6, 3, 2
+    lm, _ = build_pair(V, D, H, Fd, n_dec, ws, torch.float32, seed=6)
+    opt = RotatedSGD(lm, lr=0.1, overlap_backward=True)
+    ids = torch.randint(0, V, (L, N)).to(DEV)
+    F.cross_entropy(lm(ids).view(-1, V), ids.view(-1)).backward()
+    with pytest.raises(RuntimeError):
+        F.cross_entropy(lm(ids).view(-1, V), ids.view(-1)).backward()
+    opt.step()
+    torch.cuda.synchronize()
