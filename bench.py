@@ -102,6 +102,9 @@ def main():
     ap.add_argument("--sgd-overlap", dest="sgd_overlap", action="store_true",
                     help="apply each rotated layer's SGD update right after that layer's backward, on a second stream "
                          "(measured: no gain, the update and the backward compete for memory bandwidth)")
+    ap.add_argument("--no-wgrad-overlap", dest="wgrad_overlap", action="store_false",
+                    help="launch weight / bias gradient kernels on the compute stream instead of a second stream "
+                         "beside the input-gradient chain")
     ap.add_argument("--no-graph", dest="graph", action="store_false",
                     help="launch every kernel eagerly instead of replaying the step from a captured HIP graph")
     args = ap.parse_args()
@@ -116,6 +119,7 @@ def main():
     from rtp_amd.optim import RotatedSGD
 
     dev = torch.device("cuda", 0)
+    ring.set_wgrad_overlap(args.wgrad_overlap)
     torch.cuda.set_device(dev)
     c = CFG
     lm = build(c, dev, torch.bfloat16)
@@ -193,7 +197,8 @@ def main():
                                "32 heads, seq 32, batch 32, bf16 weights + fp32 master, 8 rotation shards emulated on "
                                "one GPU, uniform random token ids, weights U(-0.1,0.1), dropout 0, lr 1e-3, clip 0.05",
                    "tokens_per_step": tokens, "rotation_shards": c["shards"], "hip_graph": bool(args.graph),
-                   "sgd_overlapped_with_backward": bool(args.sgd_overlap)},
+                   "sgd_overlapped_with_backward": bool(args.sgd_overlap),
+                   "wgrad_on_second_stream": bool(args.wgrad_overlap)},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK["bf16_mfma_tflops"], "unit": "TFLOP/s",
                      "frac": achieved / PEAK["bf16_mfma_tflops"],
                      "traffic": (MEASURED_TRAFFIC_KIB[dom_name] * 1024.0 if dom_name in MEASURED_TRAFFIC_KIB else None),

@@ -17,7 +17,7 @@ import torch.nn as nn
 import torch.nn.init as init
 
 from .. import ops
-from ..ring import Rotation, ring_order
+from ..ring import Rotation, ring_order, wgrad_scope
 from . import shard_ops as S
 from .collectives import RotatedLayer, resolve_world
 from .utils import affine_weight, as_rows, divide_and_check_no_remainder
@@ -103,11 +103,13 @@ class _ColumnLinearFn(torch.autograd.Function):
                     S.col_dgrad(dy2, flat, 0, n_s, k, c_out, first * n_s, c_in=c_in)
                     i += 1
                 rot.release(j)
-        for first, cnt, accumulate in store.grad_runs(order):
-            S.col_wgrad(dy2, x2, store.grads, first, 0, n_s, k, first * n_s, cnt, accumulate)
-            if layer.has_bias:
-                S.col_bgrad(dy2, store.grads, first, n_s * k, n_s, first * n_s, cnt, accumulate)
-        store.grads_ready()
+        runs = store.grad_runs(order)
+        with wgrad_scope(dy2.device, (dy2, x2)):
+            for first, cnt, accumulate in runs:
+                S.col_wgrad(dy2, x2, store.grads, first, 0, n_s, k, first * n_s, cnt, accumulate)
+                if layer.has_bias:
+                    S.col_bgrad(dy2, store.grads, first, n_s * k, n_s, first * n_s, cnt, accumulate)
+            store.grads_ready()
         return (dx.view(ctx.x_shape) if need_dx else None), None, None
 
 
@@ -150,11 +152,13 @@ class _RowLinearFn(torch.autograd.Function):
                 for flat, first, cnt in rot.acquire(j):
                     S.row_dgrad(dy2, flat, 0, n, k_s, dx, first * k_s)
                 rot.release(j)
-        for first, cnt, accumulate in store.grad_runs(order):
-            S.row_wgrad(dy2, x2, store.grads, first, 0, n, k_s, first * k_s, cnt, accumulate)
-            if layer.has_bias:
-                S.row_bgrad(dy2, store.grads, first, n * k_s, n, cnt, accumulate)
-        store.grads_ready()
+        runs = store.grad_runs(order)
+        with wgrad_scope(dy2.device, (dy2, x2)):
+            for first, cnt, accumulate in runs:
+                S.row_wgrad(dy2, x2, store.grads, first, 0, n, k_s, first * k_s, cnt, accumulate)
+                if layer.has_bias:
+                    S.row_bgrad(dy2, store.grads, first, n * k_s, n, cnt, accumulate)
+            store.grads_ready()
         return (dx.view(ctx.x_shape) if need_dx else None), None, None
 
 

@@ -79,6 +79,8 @@ class RotatedSGD:
 
     @torch.no_grad()
     def step(self) -> None:
+        if self.stores:
+            ring.join_wgrad(self.stores[0].home.device)
         for st, master in zip(self.stores, self.masters):
             if st.grads is None or id(st) in self._early:
                 continue

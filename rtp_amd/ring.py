@@ -11,6 +11,7 @@ so the resident weight bytes are 1x the model plus two slots of the largest wind
 from __future__ import annotations
 
 import ctypes as C
+import os
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
@@ -33,6 +34,71 @@ def set_rotation_window(window: Optional[int]) -> None:
 
 def rotation_window() -> Optional[int]:
     return _window
+
+
+# ---- weight gradients on a second stream -----------------------------------------------------------
+# A layer's weight / bias gradients are needed only by the optimiser, while its input gradient is needed by
+# the next layer of the backward pass.  With the switch on, the gradient products of the parameters are
+# launched on a second stream (after everything already launched on the compute stream), so they fill the
+# launch gaps and tails of the input-gradient chain.  The compute stream rejoins at the end of the backward
+# pass (an autograd engine callback) and in join_wgrad().
+_wgrad_overlap = os.environ.get("RTP_WGRAD_OVERLAP", "0") == "1"
+_wgrad_streams: Dict[int, "torch.cuda.Stream"] = {}
+_wgrad_dirty: Dict[int, bool] = {}
+_wgrad_keepalive: Dict[int, list] = {}
+
+
+def set_wgrad_overlap(on: bool) -> None:
+    global _wgrad_overlap
+    _wgrad_overlap = bool(on)
+
+
+def wgrad_overlap() -> bool:
+    return _wgrad_overlap
+
+
+def join_wgrad(device: Optional[torch.device] = None) -> None:
+    """Make the current stream wait for the parameter-gradient work launched on the second stream."""
+    idx = torch.cuda.current_device() if device is None or device.index is None else device.index
+    if _wgrad_dirty.get(idx):
+        torch.cuda.current_stream(idx).wait_stream(_wgrad_streams[idx])
+        _wgrad_dirty[idx] = False
+        _wgrad_keepalive.get(idx, []).clear()
+
+
+class wgrad_scope:
+    """Context manager around a layer's parameter-gradient launches.  `tensors` are the operands those
+    launches read that autograd may free or reuse when the layer's backward returns."""
+
+    def __init__(self, device: torch.device, tensors: Sequence[torch.Tensor] = ()):
+        self.device, self.tensors, self.ctx = device, tensors, None
+
+    def __enter__(self):
+        if not _wgrad_overlap:
+            return self
+        idx = self.device.index if self.device.index is not None else torch.cuda.current_device()
+        aux = _wgrad_streams.get(idx)
+        if aux is None:
+            aux = _wgrad_streams[idx] = torch.cuda.Stream(device=idx)  # default priority
+        aux.wait_stream(torch.cuda.current_stream(idx))
+        # Hold the operands until the compute stream has rejoined: while a second reference exists autograd
+        # neither frees a gradient buffer nor accumulates into it in place under the second stream's reads.
+        _wgrad_keepalive.setdefault(idx, []).extend(t for t in self.tensors if t is not None)
+        if not _wgrad_dirty.get(idx):
+            _wgrad_dirty[idx] = True
+            if True:
+                try:  # rejoin when the running backward pass ends
+                    torch.autograd.Variable._execution_engine.queue_callback(lambda: join_wgrad(torch.device("cuda", idx)))
+                except RuntimeError:
+                    pass  # not inside a backward pass: the caller joins explicitly
+        self.ctx = torch.cuda.stream(aux)
+        self.ctx.__enter__()
+        return self
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+        return False
 
 
 class DeviceRing:

@@ -206,3 +206,24 @@ def test_lm_sgd_overlap_rejects_gradient_accumulation():
         F.cross_entropy(lm(ids).view(-1, V), ids.view(-1)).backward()
     opt.step()
     torch.cuda.synchronize()
+
+
+def test_lm_weight_gradients_on_second_stream_are_bit_identical():
+    """ring.set_wgrad_overlap(True) moves the parameter-gradient launches to a second stream that rejoins at
+    the end of the backward pass: same gradients, bit for bit, readable right after backward()."""
+    from rtp_amd import ring
+    V, D, H, Fd, n_dec, L, N, ws = 64, 32, 4, 64, 2, 6, 3, 4
+    lm_a, _ = build_pair(V, D, H, Fd, n_dec, ws, torch.bfloat16, seed=7)
+    lm_b, _ = build_pair(V, D, H, Fd, n_dec, ws, torch.bfloat16, seed=7)
+    ids = torch.randint(0, V, (L, N)).to(DEV)
+    F.cross_entropy(lm_a(ids).float().view(-1, V), ids.view(-1)).backward()
+    ring.set_wgrad_overlap(True)
+    try:
+        for _ in range(2):
+            for p in lm_b.parameters():
+                p.grad = None
+            F.cross_entropy(lm_b(ids).float().view(-1, V), ids.view(-1)).backward()
+    finally:
+        ring.set_wgrad_overlap(False)
+    for (na, pa), (nb, pb) in zip(lm_a.named_parameters(), lm_b.named_parameters()):
+        assert torch.equal(pa.grad, pb.grad), f"grad of {na} differs"
