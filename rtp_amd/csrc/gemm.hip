@@ -904,9 +904,8 @@ static int launch_layout(hipStream_t s, const GemmArgs& a, bool akc, bool bkc, d
 
 static bool mult(int64_t v, int64_t q) { return v % q == 0; }
 
-// Tile shapes, largest first.  A shape is taken when it yields enough workgroups to occupy the 256 CUs;
-// otherwise the next smaller one is tried (the 10-layer LM's per-layer problems are 1024 x 2048: 128
-// tiles of 128x128 but 256 of 128x64).
+// Tile shapes, largest first; launch_gemm picks one with a cost model (the 10-layer LM's per-layer problems
+// are 1024 x 2048 outputs: 128 tiles of 128x128 but exactly 256, one per CU, of 128x64).
 struct TileShape {
   int bm, bn;
   const char* tag;
@@ -988,19 +987,26 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
     RTP_LAUNCH_CHECK();
     return RTP_OK;
   }
-  static const int min_tiles = [] {
-    const char* e = getenv("RTP_GEMM_MIN_TILES");
-    return e ? atoi(e) : 200;
+  // Tile choice by a cost model: the launch runs in ceil(tiles / 256 CUs) rounds, a round costs the tile's
+  // measured time per K slab (ns, 4096^3 bf16 on MI355X: bigger tiles do ~30 % more outputs per ns, so what
+  // decides is mostly how evenly the tile count fills the CUs) plus a fixed prologue / epilogue.
+  static const int forced = [] {
+    const char* e = getenv("RTP_GEMM_TILE");  // debugging aid: index into kShapes
+    return e ? atoi(e) : -1;
   }();
+  static const double slab_ns[kNumShapes] = {1059.0, 540.0, 294.0, 172.0};
+  const double nslabs = (double)ceil_div(d->k * (int64_t)sizeof(T), kSlabBytes) * (double)d->ksegs;
   int shape = kNumShapes - 1;
+  double best = 0.0;
   for (int i = 0; fast && i < kNumShapes; ++i) {
     // never a tile that is mostly padding: a 32 x 32 problem (one attention head at seq 32) stays at 64 x 64
     if (kShapes[i].bm > 64 && kShapes[i].bm > ceil_div(d->m, 64) * 64) continue;
     if (kShapes[i].bn > 64 && kShapes[i].bn > ceil_div(d->n, 64) * 64) continue;
     const int64_t tiles = ceil_div(d->m, kShapes[i].bm) * ceil_div(d->n, kShapes[i].bn) * nz;
-    if (tiles >= min_tiles) {
+    const double cost = (double)ceil_div(tiles, 256) * (nslabs * slab_ns[i] + 3000.0);
+    if (best == 0.0 || cost < best || i == forced) {
+      best = i == forced ? -1.0 : cost;
       shape = i;
-      break;
     }
   }
   const TileShape& ts = kShapes[shape];
