@@ -1,7 +1,7 @@
 """GPT-2 style nn.Sequential language model built from the rotated layers (counterpart of
 rtp/models/transformer_lm_rtp.py:19-242): embedding * sqrt(ninp) -> sinusoidal positions -> N post-LN
 decoder layers (rotated self-attention + rotated ReLU FFN or rotated MoE) -> rotated logits projection.
-Residual add + LayerNorm is one fused kernel each way (module/norm.py); ReLU and dropout are ordinary torch ops."""
+Residual add + LayerNorm is one fused kernel each way (module/norm.py); the FFN's ReLU is folded into its two products (module/linear.py); dropout is an ordinary torch op."""
 from __future__ import annotations
 
 import math
@@ -12,7 +12,7 @@ import torch.nn as nn
 from ..module.attention import ParallelMultiheadAttention
 from ..module.collectives import emulate_shards
 from ..module.embedding import ParallelEmbedding
-from ..module.linear import ColumnParallelLinear
+from ..module.linear import ColumnParallelLinear, column_relu_mlp
 from ..module.moe import WeightMOELayer
 from ..module.norm import add_layer_norm
 from ..module.top2gate import WeightTop2Gate
@@ -74,6 +74,9 @@ class FeedForwardLayer(nn.Module):
         self.dropout2 = nn.Dropout(dropout)
 
     def forward(self, x):
+        if isinstance(self.activation, nn.ReLU) and not (self.training and self.dropout1.p > 0) and x.is_cuda:
+            # ReLU folded into the epilogues of the two rotated products
+            return self.dropout2(column_relu_mlp(x, self.linear1, self.linear2))
         return self.dropout2(self.linear2(self.dropout1(self.activation(self.linear1(x)))))
 
 

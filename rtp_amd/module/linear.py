@@ -113,6 +113,73 @@ class _ColumnLinearFn(torch.autograd.Function):
         return (dx.view(ctx.x_shape) if need_dx else None), None, None
 
 
+class _ColumnReluMlpFn(torch.autograd.Function):
+    """linear2(relu(linear1(x))) over two column-parallel layers with the ReLU folded into the matrix products:
+    forward in the epilogue of linear1's product, backward as a mask (h > 0) in the epilogue of linear2's
+    input-gradient product.  Same values as the three separate modules."""
+
+    @staticmethod
+    def forward(ctx, x, anchor1, anchor2, lin1, lin2):
+        k1, f, n2 = lin1.in_features, lin1.out_features, lin2.out_features
+        x2 = as_rows(x, k1)
+        rows, dt, dev = x2.shape[0], x2.dtype, x2.device
+        h = torch.empty(rows, f, dtype=dt, device=dev)
+        y = torch.empty(rows, n2, dtype=dt, device=dev)
+        for lin, src, dst, relu in ((lin1, x2, h, True), (lin2, h, y, False)):
+            n_s, k = lin.output_size_per_partition, lin.in_features
+            b_off = n_s * k if lin.has_bias else None
+            rot = Rotation(lin._store.home, ring_order(lin.rank, lin.world_size))
+            for j in range(rot.steps):
+                for flat, first, cnt in rot.acquire(j):
+                    S.col_fwd(src, flat, 0, n_s, k, b_off, dst, first * n_s, relu=relu)
+                rot.release(j)
+        ctx.layers = (lin1, lin2)
+        ctx.x_shape = x.shape
+        ctx.save_for_backward(x2, h)
+        return y.view(*x.shape[:-1], n2)
+
+    @staticmethod
+    def backward(ctx, dy):
+        lin1, lin2 = ctx.layers
+        x2, h = ctx.saved_tensors
+        dy2 = as_rows(dy, lin2.out_features)
+        need_dx = ctx.needs_input_grad[0]
+        dh = torch.empty_like(h)
+        dx = torch.empty_like(x2) if need_dx else None
+        # (layer, its output gradient, its input, its input gradient, mask applied to that input gradient)
+        for lin, g, inp, dinp, gate in ((lin2, dy2, h, dh, h), (lin1, dh, x2, dx, None)):
+            store = lin._store
+            n_s, k = lin.output_size_per_partition, lin.in_features
+            order = ring_order(lin.rank, lin.world_size, reverse=True)
+            if dinp is not None:
+                rot = Rotation(store.home, order)
+                steps = sum(len(w) for w in rot.windows)
+                acc = ops.ShardSum(dinp, steps)
+                i = 0
+                for j in range(rot.steps):
+                    for flat, first, cnt in rot.acquire(j):
+                        c_out, c_in = acc.target(i)
+                        S.col_dgrad(g, flat, 0, n_s, k, c_out, first * n_s, c_in=c_in,
+                                    gate=gate if i == steps - 1 else None)
+                        i += 1
+                    rot.release(j)
+            runs = store.grad_runs(order)
+            with wgrad_scope(g.device, (g, inp)):
+                for first, cnt, accumulate in runs:
+                    S.col_wgrad(g, inp, store.grads, first, 0, n_s, k, first * n_s, cnt, accumulate)
+                    if lin.has_bias:
+                        S.col_bgrad(g, store.grads, first, n_s * k, n_s, first * n_s, cnt, accumulate)
+                store.grads_ready()
+        return (dx.view(ctx.x_shape) if need_dx else None), None, None, None, None
+
+
+def column_relu_mlp(x: torch.Tensor, lin1: "ColumnParallelLinear", lin2: "ColumnParallelLinear") -> torch.Tensor:
+    """lin2(relu(lin1(x))) with the ReLU fused into the products of the two rotated layers."""
+    if lin1.out_features != lin2.in_features:
+        raise ValueError("column_relu_mlp: lin1.out_features must equal lin2.in_features")
+    return _ColumnReluMlpFn.apply(x, lin1._anchor, lin2._anchor, lin1, lin2)
+
+
 class _RowLinearFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, anchor, layer):

@@ -123,3 +123,34 @@ def test_indivisible_raises():
     from rtp_amd.module.linear import ColumnParallelLinear
     with emulate_shards(3), pytest.raises(AssertionError):
         ColumnParallelLinear(8, 8, device=DEV)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("ws", [1, 4])
+def test_column_relu_mlp_matches_separate_modules(dtype, ws):
+    """column_relu_mlp(x, lin1, lin2) == lin2(relu(lin1(x))) with nn.Linear masters, outputs and every gradient
+    (the ReLU lives in the epilogues of the rotated products)."""
+    from rtp_amd.module.linear import column_relu_mlp
+    gen = torch.Generator().manual_seed(11 + ws)
+    m1, m2 = nn.Linear(64, 96), nn.Linear(96, 32)
+    with torch.no_grad():
+        for p in list(m1.parameters()) + list(m2.parameters()):
+            p.copy_(torch.rand(p.shape, generator=gen) * 0.4 - 0.2)
+    x = torch.randn(5, 7, 64, generator=gen)
+    g = torch.randn(5, 7, 32, generator=gen)
+    l1 = _build("ColumnParallelLinear", m1.to(dtype), ws, dtype)
+    l2 = _build("ColumnParallelLinear", m2.to(dtype), ws, dtype)
+    xd = x.to(DEV, dtype).requires_grad_()
+    out = column_relu_mlp(xd, l1, l2)
+    out.backward(g.to(DEV, dtype))
+    r1, r2 = nn.Linear(64, 96), nn.Linear(96, 32)
+    r1.load_state_dict({k: v.float() for k, v in m1.state_dict().items()})
+    r2.load_state_dict({k: v.float() for k, v in m2.state_dict().items()})
+    xo = x.to(dtype).float().requires_grad_()
+    ref = r2(torch.relu(r1(xo)))
+    ref.backward(g.to(dtype).float())
+    assert_close(out, ref, dtype, "output")
+    assert_close(xd.grad, xo.grad, dtype, "input grad")
+    for layer, r in ((l1, r1), (l2, r2)):
+        assert_close(torch.cat([l.weight.grad for l in layer.linears], dim=0), r.weight.grad, dtype, "weight grad")
+        assert_close(torch.cat([l.bias.grad for l in layer.linears], dim=0), r.bias.grad, dtype, "bias grad")
