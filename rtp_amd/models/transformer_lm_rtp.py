@@ -9,6 +9,7 @@ import math
 import torch
 import torch.nn as nn
 
+from .. import ring
 from ..module.attention import ParallelMultiheadAttention
 from ..module.collectives import emulate_shards
 from ..module.embedding import ParallelEmbedding
@@ -102,6 +103,14 @@ class TransformerEncoderLayer(nn.Module):
         else:
             self.ff_block = FeedForwardLayer(d_model, dim_feedforward, activation, dropout, world_size=world_size,
                                              rank=rank, device=device, dtype=dtype)
+
+        # the block's rotated layers always run back to back: stage them together (one copy-stream wait per block)
+        members = [self.self_attn._store]
+        if is_moe:
+            members += [self.gate._store, self.moe_layer._store]
+        else:
+            members += [self.ff_block.linear1._store, self.ff_block.linear2._store]
+        ring.group_stores(members)
 
     def forward(self, src, src_mask=None, src_key_padding_mask=None):
         x = src

@@ -120,7 +120,7 @@ class _AttentionFn(torch.autograd.Function):
         ldq = N * ws * 3 * e_s
         fused = ops.attn_supported(dt, L, d)
         order = ring_order(layer.rank, ws)
-        rot = Rotation(store.home, order)
+        rot = Rotation(store.home, order, group=store.stage_group)
         acc = ops.ShardSum(out, sum(len(w) for w in rot.windows))
         i = 0
         for j in range(rot.steps):
@@ -181,7 +181,7 @@ class _AttentionFn(torch.autograd.Function):
         ldq = N * ws * 3 * e_s
         fused = ops.attn_supported(dt, L, d)
         order = ring_order(layer.rank, ws, reverse=True)
-        rot = Rotation(store.home, order)
+        rot = Rotation(store.home, order, group=store.stage_group)
         acc = ops.ShardSum(dx, sum(len(w) for w in rot.windows)) if need_dx else None
         i = 0
         for j in range(rot.steps):

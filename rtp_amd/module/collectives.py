@@ -76,6 +76,7 @@ class ShardStore:
         self.home: Optional[torch.Tensor] = None
         self.grads: Optional[torch.Tensor] = None
         self._overwrite = set()
+        self.stage_group = None  # set by ring.group_stores
         self.on_grads_ready = None  # optional callable(store): the layer's backward has written every gradient row
         self.pack()
 

@@ -47,7 +47,7 @@ class _EmbeddingFn(torch.autograd.Function):
         d_s, ws = layer.embedding_dim_per_partition, layer.world_size
         flat_ids = ids.reshape(-1).contiguous()
         out = torch.empty(flat_ids.numel(), layer.embedding_dim, dtype=store.home.dtype, device=store.home.device)
-        rot = Rotation(store.home, ring_order(layer.rank, ws))
+        rot = Rotation(store.home, ring_order(layer.rank, ws), group=store.stage_group)
         for j in range(rot.steps):
             for flat, first, cnt in rot.acquire(j):
                 table = flat[0].view(layer.num_embeddings, d_s)

@@ -72,7 +72,7 @@ class _ColumnLinearFn(torch.autograd.Function):
         x2 = as_rows(x, k)
         y = torch.empty(x2.shape[0], layer.out_features, dtype=x2.dtype, device=x2.device)
         b_off = n_s * k if layer.has_bias else None
-        rot = Rotation(store.home, ring_order(layer.rank, ws))
+        rot = Rotation(store.home, ring_order(layer.rank, ws), group=store.stage_group)
         for j in range(rot.steps):
             for flat, first, cnt in rot.acquire(j):
                 S.col_fwd(x2, flat, 0, n_s, k, b_off, y, first * n_s)
@@ -94,7 +94,7 @@ class _ColumnLinearFn(torch.autograd.Function):
         dx = None
         if need_dx:
             dx = torch.empty_like(x2)
-            rot = Rotation(store.home, order)
+            rot = Rotation(store.home, order, group=store.stage_group)
             acc = ops.ShardSum(dx, sum(len(w) for w in rot.windows))
             i = 0
             for j in range(rot.steps):
@@ -128,7 +128,7 @@ class _ColumnReluMlpFn(torch.autograd.Function):
         for lin, src, dst, relu in ((lin1, x2, h, True), (lin2, h, y, False)):
             n_s, k = lin.output_size_per_partition, lin.in_features
             b_off = n_s * k if lin.has_bias else None
-            rot = Rotation(lin._store.home, ring_order(lin.rank, lin.world_size))
+            rot = Rotation(lin._store.home, ring_order(lin.rank, lin.world_size), group=lin._store.stage_group)
             for j in range(rot.steps):
                 for flat, first, cnt in rot.acquire(j):
                     S.col_fwd(src, flat, 0, n_s, k, b_off, dst, first * n_s, relu=relu)
@@ -152,7 +152,7 @@ class _ColumnReluMlpFn(torch.autograd.Function):
             n_s, k = lin.output_size_per_partition, lin.in_features
             order = ring_order(lin.rank, lin.world_size, reverse=True)
             if dinp is not None:
-                rot = Rotation(store.home, order)
+                rot = Rotation(store.home, order, group=store.stage_group)
                 steps = sum(len(w) for w in rot.windows)
                 acc = ops.ShardSum(dinp, steps)
                 i = 0
@@ -188,7 +188,7 @@ class _RowLinearFn(torch.autograd.Function):
         x2 = as_rows(x, layer.in_features)
         y = torch.empty(x2.shape[0], n, dtype=x2.dtype, device=x2.device)
         b_off = n * k_s if layer.has_bias else None
-        rot = Rotation(store.home, ring_order(layer.rank, ws))
+        rot = Rotation(store.home, ring_order(layer.rank, ws), group=store.stage_group)
         acc = ops.ShardSum(y, sum(len(w) for w in rot.windows))
         i = 0
         for j in range(rot.steps):
@@ -214,7 +214,7 @@ class _RowLinearFn(torch.autograd.Function):
         dx = None
         if need_dx:
             dx = torch.empty_like(x2)
-            rot = Rotation(store.home, order)
+            rot = Rotation(store.home, order, group=store.stage_group)
             for j in range(rot.steps):
                 for flat, first, cnt in rot.acquire(j):
                     S.row_dgrad(dy2, flat, 0, n, k_s, dx, first * k_s)

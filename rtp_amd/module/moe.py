@@ -76,7 +76,7 @@ class _ExpertsFn(torch.autograd.Function):
         es = x.element_size()
         h = torch.empty(x.shape[0], f_dim, dtype=x.dtype, device=x.device)
         y = torch.empty_like(x)
-        rot = Rotation(store.home, ring_order(layer.rank, layer.world_size))
+        rot = Rotation(store.home, ring_order(layer.rank, layer.world_size), group=store.stage_group)
         for j in range(rot.steps):
             for flat, first, cnt in rot.acquire(j):
                 for le in range(n_local):
@@ -106,7 +106,7 @@ class _ExpertsFn(torch.autograd.Function):
         dh = torch.empty_like(h)
         dx = torch.empty_like(x)
         order = ring_order(layer.rank, layer.world_size, reverse=True)
-        rot = Rotation(store.home, order)
+        rot = Rotation(store.home, order, group=store.stage_group)
         for j in range(rot.steps):
             for flat, first, cnt in rot.acquire(j):
                 for le in range(n_local):

@@ -81,7 +81,7 @@ class _GateProjectionFn(torch.autograd.Function):
         ws, e_s = layer.world_size, layer.num_local_experts
         x2 = as_rows(x, layer.model_dim)
         logits = torch.empty(x2.shape[0], layer.num_experts, dtype=torch.float32, device=x2.device)
-        rot = Rotation(store.home, ring_order(layer.rank, ws))
+        rot = Rotation(store.home, ring_order(layer.rank, ws), group=store.stage_group)
         for j in range(rot.steps):
             for flat, first, cnt in rot.acquire(j):
                 S.col_fwd(x2, flat, 0, e_s, layer.model_dim, None, logits, first * e_s)
@@ -102,7 +102,7 @@ class _GateProjectionFn(torch.autograd.Function):
         dx = None
         if need_dx:
             dx = torch.empty_like(x2)
-            rot = Rotation(store.home, order)
+            rot = Rotation(store.home, order, group=store.stage_group)
             acc = ops.ShardSum(dx, sum(len(w) for w in rot.windows))
             i = 0
             for j in range(rot.steps):

@@ -114,6 +114,8 @@ class DeviceRing:
         self.slot_bytes = 0
         self.staging: Optional[torch.Tensor] = None
         self.next_slot = 0
+        self.epoch = 0
+        self.holder: List[Optional["StageGroup"]] = [None, None]
 
     def reserve(self, nbytes: int) -> None:
         if nbytes <= self.slot_bytes:
@@ -124,13 +126,26 @@ class DeviceRing:
         self.staging = torch.empty(2 * self.slot_bytes, dtype=torch.uint8, device=self.device)
         self.fence()
 
-    def take_slot(self) -> int:
-        slot = self.next_slot
-        self.next_slot ^= 1
-        return slot
+    def take_slot(self, stream: int = 0) -> int:
+        """Next staging slot, alternating, but never one that a stage group still reads (its remaining members
+        have not rotated yet); if both are held, the older group is dropped and will stage again."""
+        for cand in (self.next_slot, self.next_slot ^ 1):
+            g = self.holder[cand]
+            if g is None or g.slot != cand or not g.remaining:
+                self.holder[cand] = None
+                self.next_slot = cand ^ 1
+                return cand
+        cand = self.next_slot
+        g = self.holder[cand]
+        check(_lib.load().rtp_ring_release(self._handle, stream, cand))
+        g.slot = None
+        self.holder[cand] = None
+        self.next_slot = cand ^ 1
+        return cand
 
     def fence(self) -> None:
         """Home storage was written by work queued on the current stream: the next staging copy waits."""
+        self.epoch += 1  # staged copies made before this point are stale
         check(_lib.load().rtp_ring_fence(self._handle, torch.cuda.current_stream(self.device).cuda_stream))
 
     def __del__(self):
@@ -174,6 +189,65 @@ def staging_bytes(device: Optional[torch.device] = None) -> int:
 Run = Tuple[torch.Tensor, int, int]  # (staged [count, numel] view, first shard index, count)
 
 
+class StageGroup:
+    """Layers whose rotations always run back to back (the rotated layers of one decoder block).  When a whole
+    layer is staged per rotation (window = all), the first member to rotate stages every member into one slot
+    and the others find their shards there: one wait on the copy stream and one slot hand-back per block and
+    pass instead of one per layer -- each is a dependency between two hardware queues, which costs several
+    microseconds of idle compute stream even when the copy finished long ago."""
+
+    def __init__(self, stores: Sequence[object]):
+        self.stores = list(stores)  # objects with a `.home` [shards, numel] tensor
+        for st in self.stores:
+            st.stage_group = self
+        self.slot: Optional[int] = None
+        self.epoch = -1
+        self.offsets: List[int] = []
+        self.remaining: set = set()
+        self.acquired = False
+
+    def total_bytes(self) -> int:
+        return sum((st.home.numel() * st.home.element_size() + _SLOT_ALIGN - 1) // _SLOT_ALIGN * _SLOT_ALIGN
+                   for st in self.stores)
+
+    def usable(self, home: torch.Tensor) -> bool:
+        return all(st.home is not None and st.home.device == home.device for st in self.stores)
+
+    def member(self, home: torch.Tensor) -> int:
+        for i, st in enumerate(self.stores):
+            if st.home is home:
+                return i
+        return -1
+
+    def stage(self, ring: "DeviceRing", lib, stream: int) -> None:
+        """Copy every member's shards into one slot (on the ring's copy stream)."""
+        ring.reserve(self.total_bytes())
+        if self.slot is not None and self.epoch == ring.epoch and self.remaining:
+            lib.rtp_ring_release(ring._handle, stream, self.slot)  # an unfinished pass: hand its slot back first
+            self.slot = None
+        self.remaining = set()
+        self.slot = ring.take_slot(stream)
+        ring.holder[self.slot] = self
+        self.epoch = ring.epoch
+        self.offsets, off = [], 0
+        base = ring.staging.data_ptr() + self.slot * ring.slot_bytes
+        for st in self.stores:
+            nb = st.home.numel() * st.home.element_size()
+            check(lib.rtp_ring_prefetch(ring._handle, stream, self.slot, base + off, st.home.data_ptr(), nb))
+            self.offsets.append(off)
+            off += (nb + _SLOT_ALIGN - 1) // _SLOT_ALIGN * _SLOT_ALIGN
+        self.remaining = set(range(len(self.stores)))
+        self.acquired = False
+
+
+def group_stores(stores: Sequence[object]) -> StageGroup:
+    """Declare that the layers owning `stores` (ShardStore objects) always rotate one after another.
+    RTP_STAGE_GROUPS=0 in the environment turns the grouping off (every layer stages for itself)."""
+    if os.environ.get("RTP_STAGE_GROUPS", "1") == "0":
+        return None
+    return StageGroup(stores)
+
+
 class Rotation:
     """One pass over the shards of a layer in ring order, `window` ring steps at a time.
 
@@ -187,10 +261,12 @@ class Rotation:
     kernel can address them with one stride.
     """
 
-    def __init__(self, home: torch.Tensor, order: Sequence[int], window: Optional[int] = None):
+    def __init__(self, home: torch.Tensor, order: Sequence[int], window: Optional[int] = None,
+                 group: Optional[StageGroup] = None):
         if home.dim() != 2 or not home.is_contiguous():
             raise ValueError("Rotation: home must be a contiguous [shards, numel] tensor")
         self.home = home
+        self.group = None
         self.numel = home.shape[1]
         self.nbytes = self.numel * home.element_size()
         order = list(order)
@@ -207,14 +283,21 @@ class Rotation:
             self.windows.append(runs)
         self.steps = len(self.windows)
         self.ring = device_ring(home.device)
-        self.ring.reserve(w * self.nbytes)
         self.lib = _lib.load()
         self.stream = torch.cuda.current_stream(home.device).cuda_stream
         self.slots = [None] * self.steps
+        if group is not None and self.steps == 1 and w == home.shape[0] and group.usable(home):
+            self.member = group.member(home)
+            if self.member >= 0:
+                self.group = group
+                if group.slot is None or group.epoch != self.ring.epoch or self.member not in group.remaining:
+                    group.stage(self.ring, self.lib, self.stream)
+                return
+        self.ring.reserve(w * self.nbytes)
         self._prefetch(0)
 
     def _prefetch(self, j: int) -> None:
-        slot = self.slots[j] = self.ring.take_slot()
+        slot = self.slots[j] = self.ring.take_slot(self.stream)
         dst = self.ring.staging.data_ptr() + slot * self.ring.slot_bytes
         for first, count in self.windows[j]:
             check(self.lib.rtp_ring_prefetch(self.ring._handle, self.stream, slot, dst,
@@ -222,6 +305,15 @@ class Rotation:
             dst += count * self.nbytes
 
     def acquire(self, j: int) -> List[Run]:
+        if self.group is not None:
+            g = self.group
+            if not g.acquired:
+                check(self.lib.rtp_ring_acquire(self.ring._handle, self.stream, g.slot))
+                g.acquired = True
+            off = g.slot * self.ring.slot_bytes + g.offsets[self.member]
+            nb = self.home.shape[0] * self.nbytes
+            staged = self.ring.staging[off:off + nb].view(self.home.dtype).view(self.home.shape[0], self.numel)
+            return [(staged, 0, self.home.shape[0])]
         if j + 1 < self.steps:
             self._prefetch(j + 1)
         slot = self.slots[j]
@@ -234,6 +326,14 @@ class Rotation:
         return out
 
     def release(self, j: int) -> None:
+        if self.group is not None:
+            g = self.group
+            g.remaining.discard(self.member)
+            if not g.remaining and g.slot is not None:  # the last member of the block: hand the slot back
+                check(self.lib.rtp_ring_release(self.ring._handle, self.stream, g.slot))
+                self.ring.holder[g.slot] = None
+                g.slot = None
+            return
         check(self.lib.rtp_ring_release(self.ring._handle, self.stream, self.slots[j]))
 
 
