@@ -81,7 +81,8 @@ int rtp_device_check(char* name_out, int name_len);
 enum {
   RTP_GEMM_OUT_F32 = 1,
   RTP_GEMM_CIN_F32 = 2,
-  RTP_GEMM_RELU = 4
+  RTP_GEMM_RELU = 4,
+  RTP_GEMM_STREAM_OUT = 8 /* c_out is not read again soon (weight gradients): non-temporal stores */
 };
 
 typedef struct {

@@ -4,6 +4,6 @@ Python host code mirroring the reference's rtp.* API over hand-written HIP kerne
 C ABI of librtp_hip.so.  No kernel has a PyTorch or CPU fallback.
 """
 from .module.collectives import emulate_shards, rotated_weight_bytes, zero_full_grads  # noqa: F401
-from .ring import staging_bytes  # noqa: F401
+from .ring import rotation_window, set_rotation_window, staging_bytes  # noqa: F401
 
 __all__ = ["emulate_shards", "rotated_weight_bytes", "zero_full_grads", "staging_bytes"]

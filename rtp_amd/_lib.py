@@ -10,7 +10,8 @@ import os
 from typing import Optional
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "librtp_hip.so")
+# RTP_HIP_LIB in the environment names another build of the library (same ABI)
+LIB_PATH = os.environ.get("RTP_HIP_LIB") or os.path.join(_HERE, "lib", "librtp_hip.so")
 
 RTP_F32 = 0
 RTP_BF16 = 1
@@ -18,6 +19,7 @@ RTP_BF16 = 1
 GEMM_OUT_F32 = 1
 GEMM_CIN_F32 = 2
 GEMM_RELU = 4
+GEMM_STREAM_OUT = 8
 
 
 class RtpError(RuntimeError):

@@ -66,6 +66,37 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// Streaming accesses: data that is touched once per step (home shards read by the rotation copy, optimiser
+// state) is loaded and stored non-temporally so that it does not push the matrix-product operands out of the
+// L2 and the memory-side cache.
+typedef unsigned int nt_u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int nt_u32x2 __attribute__((ext_vector_type(2)));
+typedef float nt_f32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 nt_load(const uint4* p) {
+  const nt_u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const nt_u32x4*>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint2 nt_load(const uint2* p) {
+  const nt_u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const nt_u32x2*>(p));
+  return make_uint2(v.x, v.y);
+}
+__device__ __forceinline__ float4 nt_load(const float4* p) {
+  const nt_f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const nt_f32x4*>(p));
+  return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void nt_store(float4 a, float4* p) {
+  const nt_f32x4 v = {a.x, a.y, a.z, a.w};
+  __builtin_nontemporal_store(v, reinterpret_cast<nt_f32x4*>(p));
+}
+__device__ __forceinline__ void nt_store(uint2 a, uint2* p) {
+  const nt_u32x2 v = {a.x, a.y};
+  __builtin_nontemporal_store(v, reinterpret_cast<nt_u32x2*>(p));
+}
+__device__ __forceinline__ void nt_store(uint4 a, uint4* p) {
+  const nt_u32x4 v = {a.x, a.y, a.z, a.w};
+  __builtin_nontemporal_store(v, reinterpret_cast<nt_u32x4*>(p));
+}
+
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Optional per-launch timing (off by default; see rtp_profile_enable).  When enabled, the launch made

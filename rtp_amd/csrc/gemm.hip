@@ -383,7 +383,7 @@ __device__ __forceinline__ void load8(const T* src, float (&v)[8]) {
   }
 }
 template <typename T>
-__device__ __forceinline__ void store8(T* dst, const float (&v)[8]) {
+__device__ __forceinline__ void store8(T* dst, const float (&v)[8], bool stream) {
   if (sizeof(T) == 2) {
     union {
       uint4 q;
@@ -391,7 +391,13 @@ __device__ __forceinline__ void store8(T* dst, const float (&v)[8]) {
     } u;
 #pragma unroll
     for (int e = 0; e < 8; ++e) u.e[e] = from_f32<T>(v[e]);
-    *reinterpret_cast<uint4*>(dst) = u.q;
+    if (stream)
+      nt_store(u.q, reinterpret_cast<uint4*>(dst));
+    else
+      *reinterpret_cast<uint4*>(dst) = u.q;
+  } else if (stream) {
+    nt_store(make_float4(v[0], v[1], v[2], v[3]), reinterpret_cast<float4*>(dst));
+    nt_store(make_float4(v[4], v[5], v[6], v[7]), reinterpret_cast<float4*>(dst) + 1);
   } else {
     reinterpret_cast<float4*>(dst)[0] = make_float4(v[0], v[1], v[2], v[3]);
     reinterpret_cast<float4*>(dst)[1] = make_float4(v[4], v[5], v[6], v[7]);
@@ -402,6 +408,7 @@ template <typename T, int BM, int BN, int NTHR>
 __device__ __forceinline__ void finish_tile(const GemmArgs& p, const float* ct, int m0, int n0, int tid, int grp,
                                             long zo, long zi) {
   constexpr int CP = BN + 4, CPR = BN / 8, CHUNKS = BM * CPR;
+  const bool stream_out = p.flags & RTP_GEMM_STREAM_OUT;
   const bool out_f32 = p.flags & RTP_GEMM_OUT_F32;
   const bool cin_f32 = p.flags & RTP_GEMM_CIN_F32;
   const bool relu = p.flags & RTP_GEMM_RELU;
@@ -457,9 +464,9 @@ __device__ __forceinline__ void finish_tile(const GemmArgs& p, const float* ct, 
       }
       const long off = (long)row * p.ldc + col;
       if (out_f32)
-        store8(reinterpret_cast<float*>(cbase) + off, v);
+        store8(reinterpret_cast<float*>(cbase) + off, v, stream_out);
       else
-        store8(reinterpret_cast<T*>(cbase) + off, v);
+        store8(reinterpret_cast<T*>(cbase) + off, v, stream_out);
     } else {
       for (int e = 0; e < 8 && col + e < p.n; ++e) {
         float x = v[e];

@@ -34,16 +34,16 @@ struct Sgd4 {
   static __device__ __forceinline__ Pack load(const T* p, long i) {
     Pack v;
     if (sizeof(T) == 2)
-      v.u2 = reinterpret_cast<const uint2*>(p)[i];
+      v.u2 = nt_load(reinterpret_cast<const uint2*>(p) + i);
     else
-      v.u4 = reinterpret_cast<const uint4*>(p)[i];
+      v.u4 = nt_load(reinterpret_cast<const uint4*>(p) + i);
     return v;
   }
   static __device__ __forceinline__ void store(T* p, long i, const Pack& v) {
     if (sizeof(T) == 2)
-      reinterpret_cast<uint2*>(p)[i] = v.u2;
+      nt_store(v.u2, reinterpret_cast<uint2*>(p) + i);
     else
-      reinterpret_cast<uint4*>(p)[i] = v.u4;
+      nt_store(v.u4, reinterpret_cast<uint4*>(p) + i);
   }
   static __device__ __forceinline__ void update(float4& w, const Pack& g, Pack& sh, float lr, float clip) {
     float* wf = reinterpret_cast<float*>(&w);
@@ -69,12 +69,12 @@ __global__ __launch_bounds__(256) void sgd_vec4_kernel(float4* master, const T* 
   long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
   for (; i + stride < n4; i += 2 * stride) {
     const P g0 = Sgd4<T>::load(grad, i), g1 = Sgd4<T>::load(grad, i + stride);
-    float4 w0 = master[i], w1 = master[i + stride];
+    float4 w0 = nt_load(master + i), w1 = nt_load(master + i + stride);
     P s0, s1;
     Sgd4<T>::update(w0, g0, s0, lr, clip);
     Sgd4<T>::update(w1, g1, s1, lr, clip);
-    master[i] = w0;
-    master[i + stride] = w1;
+    nt_store(w0, master + i);
+    nt_store(w1, master + i + stride);
     if (shadow) {
       Sgd4<T>::store(shadow, i, s0);
       Sgd4<T>::store(shadow, i + stride, s1);

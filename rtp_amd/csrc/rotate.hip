@@ -74,7 +74,9 @@ __global__ __launch_bounds__(256) void copy_kernel(char* dst, const char* src, s
     uint4* d = reinterpret_cast<uint4*>(dst);
     size_t i = tid;
     for (; i + 3 * nthreads < nvec; i += 4 * nthreads) {
-      uint4 v0 = s[i], v1 = s[i + nthreads], v2 = s[i + 2 * nthreads], v3 = s[i + 3 * nthreads];
+      // the source is read once per pass; the destination is about to be read by the matrix products
+      uint4 v0 = nt_load(s + i), v1 = nt_load(s + i + nthreads), v2 = nt_load(s + i + 2 * nthreads),
+            v3 = nt_load(s + i + 3 * nthreads);
       d[i] = v0;
       d[i + nthreads] = v1;
       d[i + 2 * nthreads] = v2;

@@ -55,7 +55,7 @@ def col_wgrad(dy2, x2, grads, first, w_off, n_s, k, col0, cnt, accumulate):
     c = grads.data_ptr() + (first * numel + w_off) * es
     ops.gemm_raw(grads.dtype, a=dy2.data_ptr() + col0 * es, b=x2.data_ptr(), c_out=c, m=n_s, n=k, k=m, lda=lda,
                  ldb=ldb, ldc=k, a_kcontig=False, b_kcontig=False, groups=cnt, a_sg=n_s, c_sg=numel,
-                 c_in=c if accumulate else None, ld_cin=k, cin_sg=numel)
+                 c_in=c if accumulate else None, ld_cin=k, cin_sg=numel, stream_out=True)
 
 
 def col_bgrad(dy2, grads, first, b_off, n_s, col0, cnt, accumulate):
@@ -98,7 +98,7 @@ def row_wgrad(dy2, x2, grads, first, w_off, n, k_s, col0, cnt, accumulate):
     c = grads.data_ptr() + (first * numel + w_off) * es
     ops.gemm_raw(grads.dtype, a=dy2.data_ptr(), b=x2.data_ptr() + col0 * es, c_out=c, m=n, n=k_s, k=m, lda=lda,
                  ldb=ldb, ldc=k_s, a_kcontig=False, b_kcontig=False, groups=cnt, b_sg=k_s, c_sg=numel,
-                 c_in=c if accumulate else None, ld_cin=k_s, cin_sg=numel)
+                 c_in=c if accumulate else None, ld_cin=k_s, cin_sg=numel, stream_out=True)
 
 
 def row_bgrad(dy2, grads, first, b_off, n, cnt, accumulate):

@@ -8,7 +8,7 @@ from typing import Optional
 import torch
 
 from . import _lib
-from ._lib import GEMM_CIN_F32, GEMM_OUT_F32, GEMM_RELU, RTP_BF16, RTP_F32, GemmDesc, check
+from ._lib import GEMM_CIN_F32, GEMM_OUT_F32, GEMM_RELU, GEMM_STREAM_OUT, RTP_BF16, RTP_F32, GemmDesc, check
 
 _DT = {torch.float32: RTP_F32, torch.bfloat16: RTP_BF16}
 
@@ -48,7 +48,7 @@ def gemm_raw(dtype: torch.dtype, *, a: int, b: int, c_out: int, m: int, n: int, 
              relu: bool = False, out_f32: bool = False, cin_f32: bool = False, batch: int = 1, zdiv: int = 1,
              a_s=(0, 0), b_s=(0, 0), c_s=(0, 0), cin_s=(0, 0), gate_s=(0, 0), bias_s=(0, 0), groups: int = 1,
              a_sg: int = 0, b_sg: int = 0, c_sg: int = 0, cin_sg: int = 0, gate_sg: int = 0, bias_sg: int = 0,
-             ksegs: int = 1, a_sk: int = 0, b_sk: int = 0, bias_sk: int = 0) -> None:
+             ksegs: int = 1, a_sk: int = 0, b_sk: int = 0, bias_sk: int = 0, stream_out: bool = False) -> None:
     """One rtp_gemm call on raw device addresses (see include/rtp_hip.h for the operand rules)."""
     _lib.require_device()
     d = GemmDesc()
@@ -66,7 +66,8 @@ def gemm_raw(dtype: torch.dtype, *, a: int, b: int, c_out: int, m: int, n: int, 
     d.a_sg, d.b_sg, d.c_sg, d.cin_sg, d.gate_sg, d.bias_sg = a_sg, b_sg, c_sg, cin_sg, gate_sg, bias_sg
     d.a_sk, d.b_sk, d.bias_sk = a_sk, b_sk, bias_sk
     d.alpha = alpha
-    d.flags = (GEMM_OUT_F32 if out_f32 else 0) | (GEMM_CIN_F32 if cin_f32 else 0) | (GEMM_RELU if relu else 0)
+    d.flags = (GEMM_OUT_F32 if out_f32 else 0) | (GEMM_CIN_F32 if cin_f32 else 0) | (GEMM_RELU if relu else 0) | \
+        (GEMM_STREAM_OUT if stream_out else 0)
     d.a_kcontig, d.b_kcontig = int(a_kcontig), int(b_kcontig)
     check(_lib.load().rtp_gemm(_stream(), dtype_code(dtype), C.byref(d)))
 
