@@ -106,9 +106,13 @@ __global__ __launch_bounds__(256) void zero_kernel(char* dst, size_t bytes, int 
 static unsigned copy_grid(size_t bytes) {
   // Enough workgroups to cover the 256 CUs several times over for large shards, one per 4 KiB
   // otherwise.
+  static const size_t cap = [] {
+    const char* e = getenv("RTP_COPY_BLOCKS");
+    return e ? (size_t)atoi(e) : (size_t)2048;
+  }();
   size_t blocks = (bytes + 4095) / 4096;
   if (blocks < 1) blocks = 1;
-  if (blocks > 2048) blocks = 2048;
+  if (blocks > cap) blocks = cap;
   return (unsigned)blocks;
 }
 
