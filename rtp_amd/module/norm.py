@@ -21,16 +21,31 @@ class _AddLayerNormFn(torch.autograd.Function):
         rstd = torch.empty(rows, dtype=torch.float32, device=x2.device)
         ops.add_layernorm_fwd(x2, r2, weight, bias, eps, z, y, mean, rstd)
         ctx.save_for_backward(z, weight, mean, rstd)
-        ctx.has_bias = bias is not None
+        ctx.bias = bias
         return y
 
     @staticmethod
     def backward(ctx, dy):
         z, weight, mean, rstd = ctx.saved_tensors
         dz = torch.empty_like(z)
-        dgamma = torch.empty_like(weight)
-        dbeta = torch.empty_like(weight) if ctx.has_bias else None
+        bias = ctx.bias
+        # An optimiser may have given the parameters persistent gradient slices (RotatedSGD): right after its
+        # zero_grad() the kernel writes the gradients there and autograd gets nothing to accumulate.
+        ws, bs = getattr(weight, "_rtp_grad_sink", None), getattr(bias, "_rtp_grad_sink", None) if bias is not None else None
+        direct = ws is not None and ws.overwrite and (bias is None or (bs is not None and bs.overwrite))
+        if direct:
+            dgamma, dbeta = ws.view, (bs.view if bias is not None else None)
+        else:
+            dgamma = torch.empty_like(weight)
+            dbeta = torch.empty_like(weight) if bias is not None else None
         ops.layernorm_bwd(dy.contiguous(), z, weight, mean, rstd, dz, dgamma, dbeta)
+        if direct:
+            ws.overwrite = False
+            weight.grad = ws.view
+            if bias is not None:
+                bs.overwrite = False
+                bias.grad = bs.view
+            return dz, dz, None, None, None
         return dz, dz, dgamma, dbeta, None
 
 

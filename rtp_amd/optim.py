@@ -3,7 +3,8 @@ clip_grad_value_ then optimizer.step), as one fused kernel launch per rotated la
 
 For bf16 layers the optimiser owns an fp32 master copy of every flat shard buffer; the step updates
 the master and rounds it into the bf16 weights the kernels read.  For fp32 layers the weights are
-their own master.  Parameters outside rotated layers (LayerNorm) are flattened the same way.
+their own master.  Parameters outside rotated layers (LayerNorm) are flattened into one buffer (weights,
+gradients, master) and updated by one launch.
 
 `overlap_backward=True` applies a rotated layer's update as soon as that layer's backward has written its
 gradients, on a second stream, so the memory-bound update runs under the matrix products of the layers
@@ -23,6 +24,16 @@ from . import ops, ring
 from .module.collectives import ShardStore
 
 
+class GradSink:
+    """Persistent gradient slice of a parameter that is not part of a rotated layer."""
+
+    __slots__ = ("view", "overwrite")
+
+    def __init__(self, view: torch.Tensor):
+        self.view = view
+        self.overwrite = False  # True after zero_grad(): the next gradient replaces the slice's contents
+
+
 class RotatedSGD:
     def __init__(self, model: nn.Module, lr: float, clip_value: float = 0.0, overlap_backward: bool = False):
         self.lr = float(lr)
@@ -38,7 +49,7 @@ class RotatedSGD:
                     rotated_params.update(id(p) for p in sm.parameters())
         self.other = [p for p in model.parameters() if id(p) not in rotated_params and p.requires_grad]
         self.masters = [None if st.home.dtype == torch.float32 else st.home.float() for st in self.stores]
-        self.other_masters = [None if p.dtype == torch.float32 else p.detach().float().clone() for p in self.other]
+        self._flatten_other()
         self._early = set()  # stores already updated during the current backward
         self._aux = None
         if self.overlap_backward and self.stores:
@@ -46,17 +57,52 @@ class RotatedSGD:
             for st in self.stores:
                 st.on_grads_ready = self._update_early
 
+    def _flatten_other(self) -> None:
+        """Parameters outside rotated layers (LayerNorm) of one device and dtype are re-pointed into ONE flat
+        buffer, their gradients into another (views attached as .grad for good) and their fp32 master into a
+        third, so that the whole set is updated by one launch.  A parameter carries `_rtp_grad_sink`: a layer
+        that computes its gradient with its own kernel (module/norm.py) may write it straight into the view."""
+        self.flat = self.flat_grad = self.flat_master = None
+        self.sinks: List[GradSink] = []
+        if not self.other:
+            return
+        p0 = self.other[0]
+        if any(p.device != p0.device or p.dtype != p0.dtype or not p.is_cuda for p in self.other):
+            raise NotImplementedError("RotatedSGD: parameters outside rotated layers must share one CUDA device and dtype")
+        sizes = [(p.numel() + 7) // 8 * 8 for p in self.other]  # 16-byte aligned slices
+        total = sum(sizes)
+        self.flat = torch.zeros(total, dtype=p0.dtype, device=p0.device)
+        self.flat_grad = torch.zeros(total, dtype=p0.dtype, device=p0.device)
+        off = 0
+        with torch.no_grad():
+            for p, n in zip(self.other, sizes):
+                view = self.flat[off:off + p.numel()].view(p.shape)
+                view.copy_(p.data)
+                p.data = view
+                gview = self.flat_grad[off:off + p.numel()].view(p.shape)
+                sink = GradSink(gview)
+                p._rtp_grad_sink = sink
+                p.grad = gview
+                self.sinks.append(sink)
+                off += n
+        self.flat_master = None if p0.dtype == torch.float32 else self.flat.float()
+
     def master_bytes(self) -> int:
         n = sum(m.numel() * 4 for m in self.masters if m is not None)
-        return n + sum(m.numel() * 4 for m in self.other_masters if m is not None)
+        return n + (self.flat_master.numel() * 4 if self.flat_master is not None else 0)
 
     def zero_grad(self) -> None:
         """Rotated layers keep their gradient views attached and overwrite them in the next backward (no
         per-parameter work); other parameters get .grad = None as torch does."""
         for st in self.stores:
             st.mark_overwrite()
-        for p in self.other:
-            p.grad = None
+        if self.flat_grad is not None:
+            # one fill for all of them; the views stay attached, and a layer that writes its own gradient
+            # overwrites instead of accumulating
+            self.flat_grad.zero_()
+            for p, sink in zip(self.other, self.sinks):
+                sink.overwrite = True
+                p.grad = sink.view
 
     def _update_store(self, st: ShardStore, master: Optional[torch.Tensor]) -> None:
         home, grads = st.home.view(-1), st.grads.view(-1)
@@ -88,13 +134,17 @@ class RotatedSGD:
         if self._early:
             torch.cuda.current_stream(self.stores[0].home.device).wait_stream(self._aux)
             self._early.clear()
-        for p, master in zip(self.other, self.other_masters):
-            if p.grad is None:
-                continue
-            g = p.grad.contiguous().view(-1)
-            if master is None:
-                ops.sgd_step(p.data.view(-1), g, None, self.lr, self.clip_value)
+        if self.flat is not None:
+            for p, sink in zip(self.other, self.sinks):
+                if p.grad is None:
+                    sink.view.zero_()  # someone dropped the gradient: nothing to apply
+                    p.grad = sink.view
+                elif p.grad.data_ptr() != sink.view.data_ptr():
+                    sink.view.copy_(p.grad)  # someone attached a tensor of their own: fold it in
+                    p.grad = sink.view
+            if self.flat_master is None:
+                ops.sgd_step(self.flat, self.flat_grad, None, self.lr, self.clip_value)
             else:
-                ops.sgd_step(master.view(-1), g, p.data.view(-1), self.lr, self.clip_value)
+                ops.sgd_step(self.flat_master, self.flat_grad, self.flat, self.lr, self.clip_value)
         if self.stores:
             ring.fence(self.stores[0].home.device)  # staging copies of the next step must see the new weights
