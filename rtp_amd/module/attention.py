@@ -20,7 +20,7 @@ from torch.nn.modules.linear import NonDynamicallyQuantizableLinear
 from torch.nn.parameter import Parameter
 
 from .. import ops
-from ..ring import Rotation, ring_order, wgrad_scope
+from ..ring import Rotation, ring_order, run_wgrad
 from . import shard_ops as S
 from .collectives import RotatedLayer
 from .utils import (affine_weight, affine_weight_attention, as_rows, attention_block_index,
@@ -225,7 +225,8 @@ class _AttentionFn(torch.autograd.Function):
                 i += 1
             rot.release(j)
         runs = store.grad_runs(order)
-        with wgrad_scope(dev, (dout2, o, dqkv, x2)):
+
+        def param_grads():
             for first, cnt, accumulate in runs:
                 S.row_wgrad(dout2, o, store.grads, first, w_o_off, E, e_s, first * e_s, cnt, accumulate)
                 S.col_wgrad(dqkv, x2, store.grads, first, 0, 3 * e_s, E, first * 3 * e_s, cnt, accumulate)
@@ -233,6 +234,8 @@ class _AttentionFn(torch.autograd.Function):
                     S.row_bgrad(dout2, store.grads, first, b_o_off, E, cnt, accumulate)
                     S.col_bgrad(dqkv, store.grads, first, b_in_off, 3 * e_s, first * 3 * e_s, cnt, accumulate)
             store.grads_ready()
+
+        run_wgrad(dev, param_grads, (dout2, o, dqkv, x2))
         return (dx.view(L, N, E) if need_dx else None), None, None, None, None, None
 
 

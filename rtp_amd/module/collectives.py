@@ -78,6 +78,7 @@ class ShardStore:
         self._overwrite = set()
         self.stage_group = None  # set by ring.group_stores
         self.on_grads_ready = None  # optional callable(store): the layer's backward has written every gradient row
+        self.on_backward = None     # optional callable(store): the layer's backward has started (called at once)
         self.pack()
 
     # -- storage ---------------------------------------------------------------------------------
@@ -153,6 +154,11 @@ class ShardStore:
             self._overwrite = set(range(self.world_size))
 
     def grad_runs(self, order: Sequence[int]):
+        if self.on_backward is not None:
+            self.on_backward(self)
+        return self._grad_runs(order)
+
+    def _grad_runs(self, order: Sequence[int]):
         """Attach gradient storage to every shard in `order` and return maximal runs (first, count,
         accumulate) of consecutive shards that share the same accumulate flag, so that a grouped kernel can
         write a whole run of gradient rows in one launch."""

@@ -69,6 +69,8 @@ class _EmbeddingFn(torch.autograd.Function):
             g2 = g2.contiguous()
         workspace = ops.embedding_sort_ids(flat_ids)
         pad = -1 if layer.padding_idx is None else layer.padding_idx
+        if store.on_backward is not None:
+            store.on_backward(store)
         for idx in ring_order(layer.rank, ws, reverse=True):
             grads, accumulate = store.grad_views(idx)
             ops.embedding_scatter_add(g2[:, idx * d_s:(idx + 1) * d_s], flat_ids.numel(), workspace, grads[0],

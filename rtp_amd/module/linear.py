@@ -17,7 +17,7 @@ import torch.nn as nn
 import torch.nn.init as init
 
 from .. import ops
-from ..ring import Rotation, ring_order, wgrad_scope
+from ..ring import Rotation, ring_order, run_wgrad
 from . import shard_ops as S
 from .collectives import RotatedLayer, resolve_world
 from .utils import affine_weight, as_rows, divide_and_check_no_remainder
@@ -104,12 +104,15 @@ class _ColumnLinearFn(torch.autograd.Function):
                     i += 1
                 rot.release(j)
         runs = store.grad_runs(order)
-        with wgrad_scope(dy2.device, (dy2, x2)):
+
+        def param_grads():
             for first, cnt, accumulate in runs:
                 S.col_wgrad(dy2, x2, store.grads, first, 0, n_s, k, first * n_s, cnt, accumulate)
                 if layer.has_bias:
                     S.col_bgrad(dy2, store.grads, first, n_s * k, n_s, first * n_s, cnt, accumulate)
             store.grads_ready()
+
+        run_wgrad(dy2.device, param_grads, (dy2, x2))
         return (dx.view(ctx.x_shape) if need_dx else None), None, None
 
 
@@ -164,12 +167,15 @@ class _ColumnReluMlpFn(torch.autograd.Function):
                         i += 1
                     rot.release(j)
             runs = store.grad_runs(order)
-            with wgrad_scope(g.device, (g, inp)):
+
+            def param_grads(lin=lin, store=store, g=g, inp=inp, runs=runs, n_s=n_s, k=k):
                 for first, cnt, accumulate in runs:
                     S.col_wgrad(g, inp, store.grads, first, 0, n_s, k, first * n_s, cnt, accumulate)
                     if lin.has_bias:
                         S.col_bgrad(g, store.grads, first, n_s * k, n_s, first * n_s, cnt, accumulate)
                 store.grads_ready()
+
+            run_wgrad(g.device, param_grads, (g, inp))
         return (dx.view(ctx.x_shape) if need_dx else None), None, None, None, None
 
 
@@ -220,12 +226,15 @@ class _RowLinearFn(torch.autograd.Function):
                     S.row_dgrad(dy2, flat, 0, n, k_s, dx, first * k_s)
                 rot.release(j)
         runs = store.grad_runs(order)
-        with wgrad_scope(dy2.device, (dy2, x2)):
+
+        def param_grads():
             for first, cnt, accumulate in runs:
                 S.row_wgrad(dy2, x2, store.grads, first, 0, n, k_s, first * k_s, cnt, accumulate)
                 if layer.has_bias:
                     S.row_bgrad(dy2, store.grads, first, n * k_s, n, cnt, accumulate)
             store.grads_ready()
+
+        run_wgrad(dy2.device, param_grads, (dy2, x2))
         return (dx.view(ctx.x_shape) if need_dx else None), None, None
 
 

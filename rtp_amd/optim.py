@@ -55,6 +55,7 @@ class RotatedSGD:
         if self.overlap_backward and self.stores:
             self._aux = torch.cuda.Stream(device=self.stores[0].home.device)  # default priority
             for st in self.stores:
+                st.on_backward = self._announce
                 st.on_grads_ready = self._update_early
 
     def _flatten_other(self) -> None:
@@ -111,14 +112,17 @@ class RotatedSGD:
         else:
             ops.sgd_step(master.view(-1), grads, home, self.lr, self.clip_value)
 
-    @torch.no_grad()
-    def _update_early(self, st: ShardStore) -> None:
-        """Gradient-ready callback of a store: update it on the second stream, after everything launched so far
-        on the current stream (the layer's own products read the staged copy of the weights and are among it)."""
+    def _announce(self, st: ShardStore) -> None:
+        """Backward-started callback of a store (runs at once, in the layer's backward)."""
         if id(st) in self._early:
             raise RuntimeError("RotatedSGD(overlap_backward=True): a rotated layer produced gradients twice before "
                                "step(); use overlap_backward=False for gradient accumulation or shared layers")
         self._early.add(id(st))
+
+    @torch.no_grad()
+    def _update_early(self, st: ShardStore) -> None:
+        """Gradient-ready callback of a store: update it on the second stream, after everything launched so far
+        on the current stream (the layer's own products read the staged copy of the weights and are among it)."""
         self._aux.wait_stream(torch.cuda.current_stream(st.home.device))
         with torch.cuda.stream(self._aux):
             self._update_store(st, self.masters[self.stores.index(st)])

@@ -41,11 +41,14 @@ def rotation_window() -> Optional[int]:
 # the next layer of the backward pass.  With the switch on, the gradient products of the parameters are
 # launched on a second stream (after everything already launched on the compute stream), so they fill the
 # launch gaps and tails of the input-gradient chain.  The compute stream rejoins at the end of the backward
-# pass (an autograd engine callback) and in join_wgrad().
+# pass (an autograd engine callback) and in join_wgrad().  Tensors produced inside `fn` on the second stream
+# (workspaces) are allocated and freed there.
 _wgrad_overlap = os.environ.get("RTP_WGRAD_OVERLAP", "0") == "1"
 _wgrad_streams: Dict[int, "torch.cuda.Stream"] = {}
 _wgrad_dirty: Dict[int, bool] = {}
 _wgrad_keepalive: Dict[int, list] = {}
+_wgrad_pending: Dict[int, list] = {}
+_WGRAD_BATCH = int(os.environ.get("RTP_WGRAD_BATCH", "9"))  # layers per fork (three decoder blocks; measured optimum)
 
 
 def set_wgrad_overlap(on: bool) -> None:
@@ -58,47 +61,52 @@ def wgrad_overlap() -> bool:
 
 
 def join_wgrad(device: Optional[torch.device] = None) -> None:
-    """Make the current stream wait for the parameter-gradient work launched on the second stream."""
+    """Launch what is still deferred and make the current stream wait for the parameter-gradient work on the
+    second stream."""
     idx = torch.cuda.current_device() if device is None or device.index is None else device.index
+    _flush_wgrad(idx)
     if _wgrad_dirty.get(idx):
         torch.cuda.current_stream(idx).wait_stream(_wgrad_streams[idx])
         _wgrad_dirty[idx] = False
         _wgrad_keepalive.get(idx, []).clear()
 
 
-class wgrad_scope:
-    """Context manager around a layer's parameter-gradient launches.  `tensors` are the operands those
-    launches read that autograd may free or reuse when the layer's backward returns."""
+def _flush_wgrad(idx: int) -> None:
+    pending = _wgrad_pending.get(idx)
+    if not pending:
+        return
+    aux = _wgrad_streams.get(idx)
+    if aux is None:
+        aux = _wgrad_streams[idx] = torch.cuda.Stream(device=idx)  # default priority
+    aux.wait_stream(torch.cuda.current_stream(idx))
+    with torch.cuda.stream(aux):
+        for fn in pending:
+            fn()
+    pending.clear()
 
-    def __init__(self, device: torch.device, tensors: Sequence[torch.Tensor] = ()):
-        self.device, self.tensors, self.ctx = device, tensors, None
 
-    def __enter__(self):
-        if not _wgrad_overlap:
-            return self
-        idx = self.device.index if self.device.index is not None else torch.cuda.current_device()
-        aux = _wgrad_streams.get(idx)
-        if aux is None:
-            aux = _wgrad_streams[idx] = torch.cuda.Stream(device=idx)  # default priority
-        aux.wait_stream(torch.cuda.current_stream(idx))
-        # Hold the operands until the compute stream has rejoined: while a second reference exists autograd
-        # neither frees a gradient buffer nor accumulates into it in place under the second stream's reads.
-        _wgrad_keepalive.setdefault(idx, []).extend(t for t in self.tensors if t is not None)
-        if not _wgrad_dirty.get(idx):
-            _wgrad_dirty[idx] = True
-            if True:
-                try:  # rejoin when the running backward pass ends
-                    torch.autograd.Variable._execution_engine.queue_callback(lambda: join_wgrad(torch.device("cuda", idx)))
-                except RuntimeError:
-                    pass  # not inside a backward pass: the caller joins explicitly
-        self.ctx = torch.cuda.stream(aux)
-        self.ctx.__enter__()
-        return self
-
-    def __exit__(self, *exc):
-        if self.ctx is not None:
-            self.ctx.__exit__(*exc)
-        return False
+def run_wgrad(device: torch.device, fn, tensors: Sequence[torch.Tensor] = ()) -> None:
+    """Run `fn`, which launches a layer's parameter-gradient kernels.  Without the overlap switch: now, on the
+    current stream.  With it: deferred until `_WGRAD_BATCH` layers have queued up (or the backward pass ends) and
+    then on the second stream -- one fork of the compute stream per batch, since every fork and join between
+    two hardware queues idles the compute stream for several microseconds.  `tensors` are the operands `fn`
+    reads that autograd may free or reuse when the layer's backward returns."""
+    if not _wgrad_overlap:
+        fn()
+        return
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    # Hold the operands until the compute stream has rejoined: while a second reference exists autograd
+    # neither frees a gradient buffer nor accumulates into it in place under the second stream's reads.
+    _wgrad_keepalive.setdefault(idx, []).extend(t for t in tensors if t is not None)
+    _wgrad_pending.setdefault(idx, []).append(fn)
+    if not _wgrad_dirty.get(idx):
+        _wgrad_dirty[idx] = True
+        try:  # rejoin when the running backward pass ends
+            torch.autograd.Variable._execution_engine.queue_callback(lambda: join_wgrad(torch.device("cuda", idx)))
+        except RuntimeError:
+            pass  # not inside a backward pass: the caller joins explicitly
+    if len(_wgrad_pending[idx]) >= _WGRAD_BATCH:
+        _flush_wgrad(idx)
 
 
 class DeviceRing:
