@@ -168,7 +168,8 @@ int rtp_zero_async(void* stream, void* dst, size_t bytes);
  *                nn.Embedding backward / index_add_).  Rows that receive no token are zero-filled
  *                when zero_fill != 0.  Tokens equal to padding_idx (if >= 0) are skipped.
  *                When scale_by_freq != 0 each row's sum is divided by the number of tokens that
- *                hit it.
+ *                hit it.  `groups` shards in one launch: shard g reads grad_out + g*grad_out_sg and
+ *                writes grad_table + g*grad_table_sg (elements).
  * ids are int64.  The scatter-add needs a workspace (sort buffers).
  * --------------------------------------------------------------------------------------------- */
 int rtp_embedding_gather(void* stream, int dtype, const void* table, int64_t ld_table,
@@ -186,7 +187,8 @@ int rtp_embedding_scatter_add_det(void* stream, int dtype, const void* grad_out,
                                   int64_t n_ids, const void* workspace, void* grad_table,
                                   int64_t ld_grad_table, int grad_table_f32, int64_t row_begin,
                                   int64_t row_count, int64_t cols, int64_t padding_idx,
-                                  int scale_by_freq, int zero_fill);
+                                  int scale_by_freq, int zero_fill, int64_t groups, int64_t grad_out_sg,
+                                  int64_t grad_table_sg);
 
 /* ---------------------------------------------------------------------------------------------
  * Attention softmax (reference: rtp/module/functional.py:779-792 baddbmm+softmax, :825

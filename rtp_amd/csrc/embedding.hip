@@ -36,10 +36,11 @@ __global__ __launch_bounds__(256) void sort_prep_kernel(const int64_t* ids, long
   }
 }
 
-__global__ __launch_bounds__(256) void zero_rows_kernel(char* base, long ld_bytes, long row_bytes, long rows) {
+__global__ __launch_bounds__(256) void zero_rows_kernel(char* base, long ld_bytes, long row_bytes, long rows,
+                                                        long group_bytes) {
   const long r = blockIdx.x;
   if (r >= rows) return;
-  char* p = base + r * ld_bytes;
+  char* p = base + blockIdx.z * group_bytes + r * ld_bytes;
   if ((((uintptr_t)p | (uintptr_t)row_bytes) & 15) == 0) {
     uint4* d = reinterpret_cast<uint4*>(p);
     const uint4 z = make_uint4(0, 0, 0, 0);
@@ -56,7 +57,9 @@ template <typename T, typename G>
 __global__ __launch_bounds__(256) void scatter_kernel(const T* grad_out, long ld_go, long n, const int* keys,
                                                       const int* vals, G* grad_table, long ld_gt, long row_begin,
                                                       long row_count, long cols, long padding_idx, int scale_by_freq,
-                                                      int overwrite) {
+                                                      int overwrite, long go_sg, long gt_sg) {
+  grad_out += blockIdx.z * go_sg;  // group = shard: its column block of the upstream gradient, its own table
+  grad_table += blockIdx.z * gt_sg;
   const long i = blockIdx.x;
   const int id = keys[i];
   if (i > 0 && keys[i - 1] == id) return;
@@ -161,8 +164,11 @@ extern "C" int rtp_embedding_scatter_add_det(void* stream, int dtype, const void
                                              int64_t n_ids, const void* workspace, void* grad_table,
                                              int64_t ld_grad_table, int grad_table_f32, int64_t row_begin,
                                              int64_t row_count, int64_t cols, int64_t padding_idx, int scale_by_freq,
-                                             int zero_fill) {
+                                             int zero_fill, int64_t groups, int64_t grad_out_sg,
+                                             int64_t grad_table_sg) {
   RTP_REQUIRE(grad_out && workspace && grad_table, "rtp_embedding_scatter_add_det: null pointer");
+  RTP_REQUIRE(groups >= 1 && groups < 65536, "rtp_embedding_scatter_add_det: groups %lld not in 1..65535",
+              (long long)groups);
   RTP_REQUIRE(dtype == RTP_F32 || dtype == RTP_BF16, "rtp_embedding_scatter_add_det: unknown dtype %d", dtype);
   RTP_REQUIRE(cols >= 0 && ld_grad_out >= cols && ld_grad_table >= cols && row_count >= 0 && n_ids >= 0 &&
                   n_ids < (1ll << 31),
@@ -173,9 +179,10 @@ extern "C" int rtp_embedding_scatter_add_det(void* stream, int dtype, const void
   const unsigned chunks = (unsigned)std::min<int64_t>(16, std::max<int64_t>(1, ceil_div(cols, 1024)));
   if (zero_fill) {
     RTP_REQUIRE(row_count < (1ll << 31), "rtp_embedding_scatter_add_det: too many rows");
-    ProfileScope prof(s, "embedding_grad_zero_fill", 0.0, (double)row_count * cols * gsz);
-    hipLaunchKernelGGL(zero_rows_kernel, dim3((unsigned)row_count, chunks), dim3(256), 0, s, (char*)grad_table,
-                       (long)(ld_grad_table * gsz), (long)(cols * gsz), (long)row_count);
+    ProfileScope prof(s, "embedding_grad_zero_fill", 0.0, (double)groups * row_count * cols * gsz);
+    hipLaunchKernelGGL(zero_rows_kernel, dim3((unsigned)row_count, chunks, (unsigned)groups), dim3(256), 0, s,
+                       (char*)grad_table, (long)(ld_grad_table * gsz), (long)(cols * gsz), (long)row_count,
+                       (long)(grad_table_sg * gsz));
     RTP_LAUNCH_CHECK();
   }
   if (n_ids == 0) return RTP_OK;
@@ -183,16 +190,16 @@ extern "C" int rtp_embedding_scatter_add_det(void* stream, int dtype, const void
   const char* w = (const char*)workspace;
   const int* keys = (const int*)(w + L.keys_out);
   const int* vals = (const int*)(w + L.vals_out);
-  dim3 grid((unsigned)n_ids, chunks);
+  dim3 grid((unsigned)n_ids, chunks, (unsigned)groups);
   // After a zero fill the rows can simply be overwritten; otherwise the sum is added to what is there.
   const int overwrite = zero_fill ? 1 : 0;
 #define RTP_SCATTER(T, G)                                                                                         \
   hipLaunchKernelGGL((scatter_kernel<T, G>), grid, dim3(256), 0, s, (const T*)grad_out, (long)ld_grad_out,         \
                      (long)n_ids, keys, vals, (G*)grad_table, (long)ld_grad_table, (long)row_begin, (long)row_count, \
-                     (long)cols, (long)padding_idx, scale_by_freq, overwrite)
+                     (long)cols, (long)padding_idx, scale_by_freq, overwrite, (long)grad_out_sg, (long)grad_table_sg)
   // algorithmic bytes: read every upstream row once, write (or read-modify-write) every touched row once
-  ProfileScope prof(s, "embedding_scatter_add", (double)n_ids * cols,
-                    (double)n_ids * cols * ((dtype == RTP_F32 ? 4.0 : 2.0) + (zero_fill ? 1.0 : 2.0) * gsz) + 8.0 * n_ids);
+  ProfileScope prof(s, "embedding_scatter_add", (double)groups * n_ids * cols,
+                    (double)groups * n_ids * cols * ((dtype == RTP_F32 ? 4.0 : 2.0) + (zero_fill ? 1.0 : 2.0) * gsz) + 8.0 * n_ids);
   if (dtype == RTP_F32)
     RTP_SCATTER(float, float);
   else if (grad_table_f32)

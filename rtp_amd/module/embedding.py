@@ -71,11 +71,13 @@ class _EmbeddingFn(torch.autograd.Function):
         pad = -1 if layer.padding_idx is None else layer.padding_idx
         if store.on_backward is not None:
             store.on_backward(store)
-        for idx in ring_order(layer.rank, ws, reverse=True):
-            grads, accumulate = store.grad_views(idx)
-            ops.embedding_scatter_add(g2[:, idx * d_s:(idx + 1) * d_s], flat_ids.numel(), workspace, grads[0],
+        # runs of consecutive shards with the same overwrite / accumulate state go out as one grouped launch
+        for first, cnt, accumulate in store._grad_runs(ring_order(layer.rank, ws, reverse=True)):
+            table = store.grads[first, :store.numels[0]].view(store.shapes[0])
+            ops.embedding_scatter_add(g2[:, first * d_s:(first + 1) * d_s], flat_ids.numel(), workspace, table,
                                       padding_idx=pad, scale_by_freq=layer.scale_grad_by_freq,
-                                      zero_fill=not accumulate)
+                                      zero_fill=not accumulate, groups=cnt, grad_out_sg=d_s,
+                                      grad_table_sg=store.grads.shape[1])
         store.grads_ready()
         return None, None, None
 

@@ -215,7 +215,11 @@ def embedding_sort_ids(ids: torch.Tensor) -> torch.Tensor:
 
 def embedding_scatter_add(grad_out: torch.Tensor, n_ids: int, workspace: torch.Tensor, grad_table: torch.Tensor,
                           *, row_begin: int = 0, padding_idx: int = -1, scale_by_freq: bool = False,
-                          zero_fill: bool = True) -> None:
+                          zero_fill: bool = True, groups: int = 1, grad_out_sg: int = 0,
+                          grad_table_sg: int = 0) -> None:
+    """grad_table[id] (+)= sum of the grad_out rows whose token is id, in ascending position order.  With
+    groups > 1, group g reads grad_out + g*grad_out_sg and writes grad_table + g*grad_table_sg (elements):
+    all shards of an embedding in one launch."""
     for t in (grad_out, workspace, grad_table):
         _dev(t)
     n, cols, ld_go = _mat(grad_out, "grad_out")
@@ -228,7 +232,8 @@ def embedding_scatter_add(grad_out: torch.Tensor, n_ids: int, workspace: torch.T
     check(_lib.load().rtp_embedding_scatter_add_det(
         _stream(), dtype_code(grad_out.dtype), grad_out.data_ptr(), ld_go, n_ids, workspace.data_ptr(),
         grad_table.data_ptr(), ld_gt, int(grad_table.dtype == torch.float32), row_begin, rows, cols,
-        -1 if padding_idx is None else padding_idx, int(scale_by_freq), int(zero_fill)))
+        -1 if padding_idx is None else padding_idx, int(scale_by_freq), int(zero_fill), groups, grad_out_sg,
+        grad_table_sg))
 
 
 def softmax_fwd(scores: torch.Tensor, p: torch.Tensor, *, mask: Optional[torch.Tensor], causal: bool,
