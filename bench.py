@@ -93,12 +93,136 @@ def cpu_baseline(c, steps=2):
             f"({dt * 1e3:.0f} ms/step, os.cpu_count()={os.cpu_count()})"}
 
 
+def layer_workload(name, steps, warmup):
+    """The reference's other configurations (single rotated layers), fwd+bwd, timed with the same event
+    bracketing; one JSON line with the layer's own algorithmic work and the dominant kernel's roofline."""
+    import torch
+    import torch.nn as nn
+    from rtp_amd import _lib, emulate_shards
+
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    gen = torch.Generator().manual_seed(0)
+
+    def uni(*shape):
+        return torch.rand(*shape, generator=gen) * 0.2 - 0.1
+
+    if name == "linear":  # fp32 column-parallel Linear [1024,2048] x [2048,2048], 2 shards
+        from rtp_amd.module.linear import ColumnParallelLinear
+        master = nn.Linear(2048, 2048)
+        with torch.no_grad():
+            master.weight.copy_(uni(2048, 2048)), master.bias.zero_()
+        with emulate_shards(2):
+            layer = ColumnParallelLinear(2048, 2048, linear_layer=master, device=dev, dtype=torch.float32)
+        x = torch.randn(1024, 2048, generator=gen).to(dev).requires_grad_()
+        g = torch.randn(1024, 2048, generator=gen).to(dev)
+        fn = lambda: layer(x).backward(g)
+        work = {"flops": 3 * 2.0 * 1024 * 2048 * 2048, "bytes": None, "bound": "mfma", "peak": PEAK["fp32_mfma_tflops"],
+                "dtype": "f32", "desc": "column-parallel Linear fwd+bwd, X [1024,2048], W [2048,2048], 2 shards, fp32"}
+    elif name == "embedding":  # table [10240,2048] fp32, 4 shards, ids [32,32]
+        from rtp_amd.module.embedding import ParallelEmbedding
+        master = nn.Embedding(10240, 2048)
+        with torch.no_grad():
+            master.weight.copy_(uni(10240, 2048))
+        layer = ParallelEmbedding(10240, 2048, 4, 0, Embedding_layer=master, device=dev, dtype=torch.float32)
+        ids = torch.randint(0, 10240, (32, 32), generator=gen).to(dev)
+        g = torch.randn(32, 32, 2048, generator=gen).to(dev)
+        fn = lambda: layer(ids).backward(g)
+        # gather 16 MiB + scatter-add <= 24 MiB of algorithmic traffic (the 80 MiB dense zero fill is not counted)
+        work = {"flops": None, "bytes": (16 + 24) * 2.0 ** 20, "bound": "hbm", "peak": PEAK["hbm_gbs"], "dtype": "f32",
+                "desc": "vocab-sharded Embedding fwd+bwd, table [10240,2048] fp32 in 4 shards, ids [32,32]"}
+    elif name == "attention":  # d_model 2048, 32 heads in 8 groups, batch 8, seq 512, causal, bf16
+        from rtp_amd.module.attention import ParallelMultiheadAttention
+        mha = nn.MultiheadAttention(2048, 32, bias=True)
+        with torch.no_grad():
+            for p_ in mha.parameters():
+                p_.copy_(uni(*p_.shape))
+        layer = ParallelMultiheadAttention(2048, 32, 8, 0, MultiheadAttention_layer=mha.to(torch.bfloat16), device=dev,
+                                           dtype=torch.bfloat16)
+        x = torch.randn(512, 8, 2048, generator=gen).to(dev, torch.bfloat16).requires_grad_()
+        g = torch.randn(512, 8, 2048, generator=gen).to(dev, torch.bfloat16)
+        fn = lambda: layer(x, x, x, is_causal=True, need_weights=False)[0].backward(g)
+        proj = 2.0 * 4096 * 2048 * (6144 + 2048)
+        core = 4.0 * 8 * 32 * 512 * 512 * 64
+        work = {"flops": 3 * proj + 3.5 * core, "bytes": None, "bound": "mfma", "peak": PEAK["bf16_mfma_tflops"],
+                "dtype": "bf16", "desc": "head-sharded attention fwd+bwd, d_model 2048, 32 heads in 8 groups, batch 8, "
+                "seq 512, causal, bf16 (attention core counted in full, not halved for causality)"}
+    elif name == "moe":  # 8 experts, top-2, d_model 2048, d_ff 8192, 4096 tokens, bf16
+        from rtp_amd.models.transformer_lm_rtp import FeedForwardLayer_expert
+        from rtp_amd.module.moe import WeightMOELayer
+        from rtp_amd.module.top2gate import Top2Gate, WeightTop2Gate
+        mg = Top2Gate(2048, 8)
+        with torch.no_grad():
+            mg.wg.weight.copy_(uni(8, 2048))
+        masters = []
+        for _ in range(8):
+            m = FeedForwardLayer_expert(2048, 8192, nn.ReLU(), 0.0)
+            with torch.no_grad():
+                for p_ in m.parameters():
+                    p_.copy_(uni(*p_.shape))
+            masters.append(m.to(torch.bfloat16))
+        with emulate_shards(8):
+            gate = WeightTop2Gate(2048, 8, gate=mg.to(torch.bfloat16), device=dev, dtype=torch.bfloat16)
+            local = nn.ModuleList([FeedForwardLayer_expert(2048, 8192, nn.ReLU(), 0.0)])
+            layer = WeightMOELayer(gate, local, device=dev, dtype=torch.bfloat16,
+                                   original_experts=[nn.ModuleList([m]) for m in masters])
+        x = torch.randn(8, 512, 2048, generator=gen).to(dev, torch.bfloat16).requires_grad_()
+        g = torch.randn(8, 512, 2048, generator=gen).to(dev, torch.bfloat16)
+        u = torch.rand(4096, 8, generator=gen).clamp(min=torch.finfo(torch.float32).tiny, max=1 - torch.finfo(torch.float32).eps)
+        noise = (-torch.log(-torch.log(u))).to(dev)  # Gumbel(0,1) routing noise, drawn on the host
+        fn = lambda: (layer(x, noise=noise) * g).sum().backward()
+        work = {"flops": 3 * 8192 * 2.0 * 2 * 2048 * 8192, "bytes": None, "bound": "mfma", "peak": PEAK["bf16_mfma_tflops"],
+                "dtype": "bf16", "desc": "expert-sharded MoE layer fwd+bwd, 8 experts, top-2, d_model 2048, d_ff 8192, "
+                "4096 tokens, bf16 (flops for 8192 routed pairs, i.e. nothing dropped)"}
+    else:
+        raise SystemExit(f"unknown workload {name}")
+
+    for _ in range(max(warmup, 1)):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    _lib.profile_enable(True)
+    fn(), fn()
+    stats = _lib.profile_collect()
+    _lib.profile_enable(False)
+    kernels = {k: {"launches": v["launches"] // 2, "ms": round(v["total_ms"] / 2, 4),
+                   "tflops": round(v["flops"] / max(v["total_ms"], 1e-9) / 1e9, 2),
+                   "gbs": round(v["bytes"] / max(v["total_ms"], 1e-9) / 1e6, 1)} for k, v in sorted(stats.items())}
+    dom_name, dom = max(stats.items(), key=lambda kv: kv[1]["total_ms"])
+    avg_ms = dom["total_ms"] / dom["launches"]
+    if work["bound"] == "mfma":
+        achieved = dom["flops"] / dom["launches"] / (avg_ms * 1e-3) / 1e12
+        whole = work["flops"] / dt / 1e12
+        unit = "TFLOP/s"
+    else:
+        achieved = dom["bytes"] / dom["launches"] / (avg_ms * 1e-3) / 1e9
+        whole = work["bytes"] / dt / 1e9
+        unit = "GB/s"
+    out = {"metric": f"fwd+bwd time of one rotated layer ({name})", "value": dt * 1e3, "unit": "ms", "n_gpus": 1,
+           "steps": steps, "warmup": warmup, "ms_per_step": dt * 1e3, "higher_is_better": False, "scaling": "weak",
+           "vs_baseline": None, "dtype": work["dtype"], "data": "synthetic",
+           "config": {"workload": work["desc"], "launch_mode": "eager (CPU launch overhead included)"},
+           "roofline": {"bound": work["bound"], "achieved": achieved, "peak": work["peak"], "unit": unit,
+                        "frac": achieved / work["peak"], "traffic": None, "kernel": dom_name,
+                        "avg_launch_us": avg_ms * 1e3},
+           "whole_layer": {"achieved": whole, "unit": unit, "frac": whole / work["peak"]},
+           "kernels": kernels}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--workload", default="lm", choices=["lm", "linear", "embedding", "attention", "moe"],
+                    help="lm: the headline training step (default); the others time one rotated layer of the "
+                         "reference's remaining configurations, fwd+bwd")
     ap.add_argument("--sgd-overlap", dest="sgd_overlap", action="store_true",
                     help="apply each rotated layer's SGD update right after that layer's backward, on a second stream "
                          "(measured: no gain, the update and the backward compete for memory bandwidth)")
@@ -112,6 +236,10 @@ def main():
         print(f"bench.py measures one GPU's throughput: this build runs every rotation shard on a single MI355X and "
               f"has no multi-GPU path (--gpus {args.gpus} is not supported)", file=sys.stderr)
         sys.exit(2)
+
+    if args.workload != "lm":
+        layer_workload(args.workload, args.steps, args.warmup)
+        return
 
     import torch
     import torch.nn.functional as F

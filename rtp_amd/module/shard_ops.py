@@ -53,6 +53,13 @@ def col_wgrad(dy2, x2, grads, first, w_off, n_s, k, col0, cnt, accumulate):
     m, _, lda = _rows(dy2)
     _, _, ldb = _rows(x2)
     c = grads.data_ptr() + (first * numel + w_off) * es
+    if n_s == 1 and cnt > 1:
+        # one output row per shard (a gate with one expert per shard): the run is a single product whose
+        # output rows are the shards' gradient rows, `numel` apart -- vector loads instead of 1-row groups
+        ops.gemm_raw(grads.dtype, a=dy2.data_ptr() + col0 * es, b=x2.data_ptr(), c_out=c, m=cnt, n=k, k=m, lda=lda,
+                     ldb=ldb, ldc=numel, a_kcontig=False, b_kcontig=False,
+                     c_in=c if accumulate else None, ld_cin=numel, stream_out=True)
+        return
     ops.gemm_raw(grads.dtype, a=dy2.data_ptr() + col0 * es, b=x2.data_ptr(), c_out=c, m=n_s, n=k, k=m, lda=lda,
                  ldb=ldb, ldc=k, a_kcontig=False, b_kcontig=False, groups=cnt, a_sg=n_s, c_sg=numel,
                  c_in=c if accumulate else None, ld_cin=k, cin_sg=numel, stream_out=True)
