@@ -298,6 +298,18 @@ int rtp_moe_combine_dweight(void* stream, int dtype, const void* dout, int64_t l
 int rtp_sgd_step(void* stream, int dtype, float* master, const void* grad, void* shadow, int64_t n,
                  float lr, float clip);
 
+/* The same update for many buffers in one launch.  `chunks` is a table in DEVICE memory, one entry per
+ * workgroup: 16-byte aligned pointers into the buffers and a parameter count that is a multiple of 4 (the
+ * caller cuts its buffers into chunks of, say, 16384 parameters).  total_params only feeds the profiler. */
+typedef struct {
+  float* master;
+  const void* grad;
+  void* shadow; /* NULL: the master is the weight */
+  int64_t n;
+} rtp_sgd_chunk;
+int rtp_sgd_step_multi(void* stream, int dtype, const rtp_sgd_chunk* chunks, int64_t n_chunks, float lr,
+                       float clip, double total_params);
+
 /* dst(dtype_dst)[i] = src(dtype_src)[i]  (fp32 <-> bf16 conversion, round to nearest even). */
 int rtp_cast(void* stream, int dtype_src, const void* src, int dtype_dst, void* dst, int64_t n);
 

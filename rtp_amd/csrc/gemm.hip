@@ -634,7 +634,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   constexpr int STAGE = DA::BYTES + DB::BYTES;
   constexpr int NI = DA::NI + DB::NI;  // loads per loader wave and slab
   static_assert((NSTAGE - 2) * NI < 64, "vmcnt is a 6-bit counter");
-  static_assert(NSTAGE >= 3 && NSTAGE <= 5, "3..5 LDS stages");
+  static_assert(NSTAGE >= 3 && NSTAGE <= 6, "3..6 LDS stages");
   static_assert(BM * (BN + 4) * 4 <= NSTAGE * STAGE, "the epilogue stages the fp32 tile in the slab memory");
   // Stage addresses are compile-time offsets into one array, so LDS reads carry immediate offsets.
   __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE];
@@ -783,6 +783,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
     using I2 = std::integral_constant<int, 2>;
     using I3 = std::integral_constant<int, 3>;
     using I4 = std::integral_constant<int, 4>;
+    using I5 = std::integral_constant<int, 5>;
     __builtin_amdgcn_s_barrier();  // barrier 0
     read_group(I0{}, Q0{});
     int kt = 0;
@@ -792,6 +793,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
       phase(I2{}, kt + 2, std::true_type{});
       if (NSTAGE > 3) phase(I3{}, kt + 3, std::true_type{});
       if (NSTAGE > 4) phase(I4{}, kt + 4, std::true_type{});
+      if (NSTAGE > 5) phase(I5{}, kt + 5, std::true_type{});
     }
     for (; kt < nk; kt += NSTAGE) {
       phase(I0{}, kt, std::false_type{});
@@ -799,6 +801,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
       phase(I2{}, kt + 2, std::false_type{});
       if (NSTAGE > 3) phase(I3{}, kt + 3, std::false_type{});
       if (NSTAGE > 4) phase(I4{}, kt + 4, std::false_type{});
+      if (NSTAGE > 5) phase(I5{}, kt + 5, std::false_type{});
     }
   }
   const bool computes = wave < 4;

@@ -90,6 +90,47 @@ __global__ __launch_bounds__(256) void sgd_vec4_kernel(float4* master, const T* 
   }
 }
 
+// Many tensors in one launch: workgroup b updates chunk b of a device-resident table, four parameters per lane
+// and access, two accesses in flight.
+struct SgdChunk {
+  float* master;
+  const void* grad;
+  void* shadow;  // may be null
+  long n;        // parameters in the chunk, a multiple of 4; the three pointers are 16-byte aligned
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void sgd_multi_kernel(const SgdChunk* chunks, float lr, float clip) {
+  using P = typename Sgd4<T>::Pack;
+  const SgdChunk c = chunks[blockIdx.x];
+  float4* master = reinterpret_cast<float4*>(c.master);
+  const T* grad = reinterpret_cast<const T*>(c.grad);
+  T* shadow = reinterpret_cast<T*>(c.shadow);
+  const long n4 = c.n >> 2;
+  long i = threadIdx.x;
+  for (; i + 256 < n4; i += 512) {
+    const P g0 = Sgd4<T>::load(grad, i), g1 = Sgd4<T>::load(grad, i + 256);
+    float4 w0 = nt_load(master + i), w1 = nt_load(master + i + 256);
+    P s0, s1;
+    Sgd4<T>::update(w0, g0, s0, lr, clip);
+    Sgd4<T>::update(w1, g1, s1, lr, clip);
+    nt_store(w0, master + i);
+    nt_store(w1, master + i + 256);
+    if (shadow) {
+      Sgd4<T>::store(shadow, i, s0);
+      Sgd4<T>::store(shadow, i + 256, s1);
+    }
+  }
+  for (; i < n4; i += 256) {
+    const P g0 = Sgd4<T>::load(grad, i);
+    float4 w0 = nt_load(master + i);
+    P s0;
+    Sgd4<T>::update(w0, g0, s0, lr, clip);
+    nt_store(w0, master + i);
+    if (shadow) Sgd4<T>::store(shadow, i, s0);
+  }
+}
+
 template <typename S, typename D>
 __global__ __launch_bounds__(256) void cast_kernel(const S* src, D* dst, long n) {
   const long stride = (long)gridDim.x * blockDim.x;
@@ -127,6 +168,25 @@ extern "C" int rtp_sgd_step(void* stream, int dtype, float* master, const void* 
                        (bf16_t*)shadow, (long)n, lr, clip);
   else
     return fail(RTP_ERR_ARG, "rtp_sgd_step: unknown dtype %d", dtype);
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
+}
+
+extern "C" int rtp_sgd_step_multi(void* stream, int dtype, const rtp_sgd_chunk* chunks, int64_t n_chunks, float lr,
+                                  float clip, double total_params) {
+  static_assert(sizeof(rtp_sgd_chunk) == sizeof(SgdChunk), "rtp_sgd_chunk layout");
+  RTP_REQUIRE(chunks, "rtp_sgd_step_multi: null chunk table");
+  RTP_REQUIRE(n_chunks >= 0 && n_chunks < (1ll << 31), "rtp_sgd_step_multi: chunk count %lld out of range",
+              (long long)n_chunks);
+  RTP_REQUIRE(dtype == RTP_F32 || dtype == RTP_BF16, "rtp_sgd_step_multi: unknown dtype %d", dtype);
+  if (n_chunks == 0) return RTP_OK;
+  hipStream_t s = (hipStream_t)stream;
+  ProfileScope prof(s, "sgd_step", 2.0 * total_params, total_params * (dtype == RTP_F32 ? 12.0 : 12.0));
+  const SgdChunk* table = reinterpret_cast<const SgdChunk*>(chunks);
+  if (dtype == RTP_F32)
+    hipLaunchKernelGGL(sgd_multi_kernel<float>, dim3((unsigned)n_chunks), dim3(256), 0, s, table, lr, clip);
+  else
+    hipLaunchKernelGGL(sgd_multi_kernel<bf16_t>, dim3((unsigned)n_chunks), dim3(256), 0, s, table, lr, clip);
   RTP_LAUNCH_CHECK();
   return RTP_OK;
 }

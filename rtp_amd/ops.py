@@ -365,6 +365,35 @@ def sgd_step(master: torch.Tensor, grad: torch.Tensor, shadow: Optional[torch.Te
                                    _ptr(shadow), master.numel(), lr, clip))
 
 
+SGD_CHUNK = 16384  # parameters per workgroup of the multi-buffer update
+
+
+def sgd_chunk_table(items, device) -> Optional[torch.Tensor]:
+    """Device table for sgd_step_multi from (master, grad, shadow-or-None) triples of flat tensors, or None when
+    some buffer does not allow 16-byte accesses (then update the buffers one by one)."""
+    rows = []
+    for master, grad, shadow in items:
+        n = master.numel()
+        ptrs = [master.data_ptr(), grad.data_ptr()] + ([shadow.data_ptr()] if shadow is not None else [])
+        if n % 4 or any(p % 16 for p in ptrs) or grad.numel() != n or (shadow is not None and shadow.numel() != n):
+            return None
+        gs = grad.element_size()
+        for off in range(0, n, SGD_CHUNK):
+            cnt = min(SGD_CHUNK, n - off)
+            rows.append((master.data_ptr() + off * 4, grad.data_ptr() + off * gs,
+                         shadow.data_ptr() + off * gs if shadow is not None else 0, cnt))
+    if not rows:
+        return None
+    return torch.tensor(rows, dtype=torch.int64).to(device)
+
+
+def sgd_step_multi(table: torch.Tensor, dtype: torch.dtype, lr: float, clip: float, total_params: int) -> None:
+    _dev(table)
+    _lib.require_device()
+    check(_lib.load().rtp_sgd_step_multi(_stream(), dtype_code(dtype), table.data_ptr(), table.shape[0], lr, clip,
+                                         float(total_params)))
+
+
 def cast(src: torch.Tensor, dst: torch.Tensor) -> None:
     _dev(src)
     _dev(dst)

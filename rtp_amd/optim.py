@@ -51,6 +51,8 @@ class RotatedSGD:
         self.masters = [None if st.home.dtype == torch.float32 else st.home.float() for st in self.stores]
         self._flatten_other()
         self._early = set()  # stores already updated during the current backward
+        self._table = self._table_key = None
+        self._table_params, self._table_dtype = 0, None
         self._aux = None
         if self.overlap_backward and self.stores:
             self._aux = torch.cuda.Stream(device=self.stores[0].home.device)  # default priority
@@ -119,6 +121,15 @@ class RotatedSGD:
                                "step(); use overlap_backward=False for gradient accumulation or shared layers")
         self._early.add(id(st))
 
+    def _fold_other_grads(self) -> None:
+        for p, sink in zip(self.other, self.sinks):
+            if p.grad is None:
+                sink.view.zero_()  # someone dropped the gradient: nothing to apply
+                p.grad = sink.view
+            elif p.grad.data_ptr() != sink.view.data_ptr():
+                sink.view.copy_(p.grad)  # someone attached a tensor of their own: fold it in
+                p.grad = sink.view
+
     @torch.no_grad()
     def _update_early(self, st: ShardStore) -> None:
         """Gradient-ready callback of a store: update it on the second stream, after everything launched so far
@@ -127,10 +138,43 @@ class RotatedSGD:
         with torch.cuda.stream(self._aux):
             self._update_store(st, self.masters[self.stores.index(st)])
 
+    def _multi_table(self):
+        """Chunk table covering every buffer (rotated stores + the flat non-rotated parameters), rebuilt only when
+        a buffer moved; None when a buffer cannot be updated this way."""
+        items, dtype = [], None
+        for st, master in zip(self.stores, self.masters):
+            if st.grads is None:
+                return None
+            home, grads = st.home.view(-1), st.grads.view(-1)
+            items.append((home, grads, None) if master is None else (master.view(-1), grads, home))
+            dtype = home.dtype if dtype is None else dtype
+            if home.dtype != dtype:
+                return None
+        if self.flat is not None:
+            if dtype is not None and self.flat.dtype != dtype:
+                return None
+            dtype = self.flat.dtype
+            items.append((self.flat, self.flat_grad, None) if self.flat_master is None
+                         else (self.flat_master, self.flat_grad, self.flat))
+        key = tuple(t.data_ptr() for it in items for t in it if t is not None)
+        if key != self._table_key:
+            self._table_key = key
+            self._table = ops.sgd_chunk_table(items, items[0][0].device) if items else None
+            self._table_params = sum(it[0].numel() for it in items)
+            self._table_dtype = dtype
+        return self._table
+
     @torch.no_grad()
     def step(self) -> None:
         if self.stores:
             ring.join_wgrad(self.stores[0].home.device)
+        table = None if (self._early or self.overlap_backward) else self._multi_table()
+        if table is not None:
+            self._fold_other_grads()
+            ops.sgd_step_multi(table, self._table_dtype, self.lr, self.clip_value, self._table_params)
+            if self.stores:
+                ring.fence(self.stores[0].home.device)
+            return
         for st, master in zip(self.stores, self.masters):
             if st.grads is None or id(st) in self._early:
                 continue
@@ -139,13 +183,7 @@ class RotatedSGD:
             torch.cuda.current_stream(self.stores[0].home.device).wait_stream(self._aux)
             self._early.clear()
         if self.flat is not None:
-            for p, sink in zip(self.other, self.sinks):
-                if p.grad is None:
-                    sink.view.zero_()  # someone dropped the gradient: nothing to apply
-                    p.grad = sink.view
-                elif p.grad.data_ptr() != sink.view.data_ptr():
-                    sink.view.copy_(p.grad)  # someone attached a tensor of their own: fold it in
-                    p.grad = sink.view
+            self._fold_other_grads()
             if self.flat_master is None:
                 ops.sgd_step(self.flat, self.flat_grad, None, self.lr, self.clip_value)
             else:
