@@ -533,12 +533,20 @@ __device__ __forceinline__ constexpr int rc_swizzle(int kl) {
   return R >= 128 ? (kl & 3) << 2 : ((kl >> 1) & 1) << 2;
 }
 
-template <typename T, int R, bool KC, int NL>
+// Chunk swizzle of a k-contiguous operand whose slab rows are SB bytes (128: 8 chunks, 64: 4 chunks): 16
+// consecutive rows reading the same chunk must land on 16 different 16-byte slots of the 256-byte bank space.
+template <int SB>
+__device__ __forceinline__ constexpr int kc_swizzle(int row) {
+  return SB == 128 ? (row >> 1) & 7 : (row >> 2) & 3;
+}
+
+template <typename T, int R, bool KC, int NL, int SB>
 struct DmaOperand {
   static constexpr int VEC = 16 / sizeof(T);
-  static_assert((R / 8) % NL == 0, "every loader wave issues the same number of loads");
-  static constexpr int NI = R / 8 / NL;           // load instructions per loader wave and slab
-  static constexpr int BYTES = R * kSlabBytes;    // one stage of this operand
+  static_assert(SB == 128 || SB == 64, "slab rows of 128 or 64 bytes");
+  static_assert((R * SB / 1024) % NL == 0, "every loader wave issues the same number of loads");
+  static constexpr int NI = R * SB / 1024 / NL;   // load instructions (1 KiB each) per loader wave and slab
+  static constexpr int BYTES = R * SB;            // one stage of this operand
   static constexpr int LINE = R * (int)sizeof(T); // bytes of one k line when rows are contiguous
   const T* ptr[NI];  // source of the NEXT slab's vector, advanced in place
   int koff[NI];      // k of the vector inside its slab
@@ -549,8 +557,9 @@ struct DmaOperand {
     for (int i = 0; i < NI; ++i) {
       const int j = lw * NI + i;  // which KiB of the stage
       if (KC) {
-        const int row = j * 8 + (lane >> 3);
-        const int c = (lane & 7) ^ ((row >> 1) & 7);
+        constexpr int LPR = SB / 16;  // lanes (16-byte chunks) per row
+        const int row = j * (64 / LPR) + lane / LPR;
+        const int c = (lane % LPR) ^ kc_swizzle<SB>(row);
         const int rr = row0 + row < rows ? row0 + row : rows - 1;
         ptr[i] = base + (long)rr * ld + c * VEC;
         koff[i] = c * VEC;
@@ -589,7 +598,7 @@ struct DmaOperand {
 typedef short short4_t __attribute__((ext_vector_type(4)));
 
 // rowbase: first tile row of the 32-row MFMA block; the lane's own row is rowbase + lane % 32.
-template <typename T, int R, bool KC>
+template <typename T, int R, bool KC, int SB>
 __device__ __forceinline__ Frag<T> read_frag_dma(const char* st, int rowbase, int lane, int ks) {
   constexpr int VEC = 16 / sizeof(T);
   constexpr int LINE = R * (int)sizeof(T);
@@ -602,7 +611,7 @@ __device__ __forceinline__ Frag<T> read_frag_dma(const char* st, int rowbase, in
   } u;
   if (KC) {
     const int row = rowbase + li;
-    u.q = *reinterpret_cast<const uint4*>(st + row * kSlabBytes + (((2 * ks + g) ^ ((row >> 1) & 7)) << 4));
+    u.q = *reinterpret_cast<const uint4*>(st + row * SB + (((2 * ks + g) ^ kc_swizzle<SB>(row)) << 4));
   } else if (sizeof(T) == 2) {
     // LDS holds [k][rows] (rows contiguous) but the MFMA wants 8 consecutive k per lane.  gfx950's
     // transposing LDS read does the 16-bit transpose inside each group of 16 lanes: lane s of a group
@@ -624,17 +633,19 @@ __device__ __forceinline__ Frag<T> read_frag_dma(const char* st, int rowbase, in
   return u.f;
 }
 
-template <typename T, int BM, int BN, bool AKC, bool BKC, int NSTAGE>
+template <typename T, int BM, int BN, bool AKC, bool BKC, int NSTAGE, int SB>
 __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   constexpr int NL = 4;  // loader waves (waves 4..7); waves 0..3 compute
-  using DA = DmaOperand<T, BM, AKC, NL>;
-  using DB = DmaOperand<T, BN, BKC, NL>;
-  constexpr int BK = kSlabBytes / sizeof(T);
+  using DA = DmaOperand<T, BM, AKC, NL, SB>;
+  using DB = DmaOperand<T, BN, BKC, NL, SB>;
+  constexpr int BK = SB / sizeof(T);
+  constexpr int KS = SB / 32;  // MFMA k-steps per slab
   constexpr int WM = BM / 2, WN = BN / 2, MT = WM / 32, NT = WN / 32;
   constexpr int STAGE = DA::BYTES + DB::BYTES;
   constexpr int NI = DA::NI + DB::NI;  // loads per loader wave and slab
   static_assert((NSTAGE - 2) * NI < 64, "vmcnt is a 6-bit counter");
-  static_assert(NSTAGE >= 3 && NSTAGE <= 6, "3..6 LDS stages");
+  static_assert(NSTAGE >= 3, "at least 3 LDS stages");
+  static_assert(NSTAGE * STAGE <= 160 * 1024, "160 KiB of LDS per workgroup");
   static_assert(BM * (BN + 4) * 4 <= NSTAGE * STAGE, "the epilogue stages the fp32 tile in the slab memory");
   // Stage addresses are compile-time offsets into one array, so LDS reads carry immediate offsets.
   __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE];
@@ -729,11 +740,12 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
     }
   } else {
     // ---- compute waves ----
-    // The 4 k-steps of a slab are taken in NG groups of G k-steps, with two sets of fragment registers:
+    // The KS k-steps of a slab are taken in NG groups of G k-steps, with two sets of fragment registers:
     // while the MFMAs of one group run, the next group is read from LDS into the other set -- the first
     // group of the NEXT slab during the last group of this one -- so an LDS read always has a group of
     // MFMAs to hide behind.  Big tiles take G = 1 to fit the register file.
-    constexpr int G = (MT * NT >= 8) ? 1 : 2, NG = 4 / G;
+    constexpr int G = (KS == 4 && MT * NT < 8) ? 2 : 1, NG = KS / G;
+    static_assert(NG == 2 || NG == 4, "two or four fragment groups per slab");
     Frag<T> fa[2][G][MT], fb[2][G][NT];
     auto read_group = [&](auto S, auto Q) {
       const char* sa = lds + (decltype(S)::value % NSTAGE) * STAGE;
@@ -742,9 +754,11 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
 #pragma unroll
       for (int e = 0; e < G; ++e) {
 #pragma unroll
-        for (int i = 0; i < MT; ++i) fa[q & 1][e][i] = read_frag_dma<T, BM, AKC>(sa, wm * WM + i * 32, lane, q * G + e);
+        for (int i = 0; i < MT; ++i)
+          fa[q & 1][e][i] = read_frag_dma<T, BM, AKC, SB>(sa, wm * WM + i * 32, lane, q * G + e);
 #pragma unroll
-        for (int j = 0; j < NT; ++j) fb[q & 1][e][j] = read_frag_dma<T, BN, BKC>(sb, wn * WN + j * 32, lane, q * G + e);
+        for (int j = 0; j < NT; ++j)
+          fb[q & 1][e][j] = read_frag_dma<T, BN, BKC, SB>(sb, wn * WN + j * 32, lane, q * G + e);
       }
     };
     auto mma_group = [&](auto Q) {
@@ -778,31 +792,17 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
       }
       mma_group(std::integral_constant<int, NG - 1>{});
     };
-    using I0 = std::integral_constant<int, 0>;
-    using I1 = std::integral_constant<int, 1>;
-    using I2 = std::integral_constant<int, 2>;
-    using I3 = std::integral_constant<int, 3>;
-    using I4 = std::integral_constant<int, 4>;
-    using I5 = std::integral_constant<int, 5>;
+    // one round = NSTAGE phases with compile-time stage indices
+    auto round = [&](int kt, auto STEADY) {
+      [&]<int... S>(std::integer_sequence<int, S...>) {
+        (phase(std::integral_constant<int, S>{}, kt + S, STEADY), ...);
+      }(std::make_integer_sequence<int, NSTAGE>{});
+    };
     __builtin_amdgcn_s_barrier();  // barrier 0
-    read_group(I0{}, Q0{});
+    read_group(std::integral_constant<int, 0>{}, Q0{});
     int kt = 0;
-    for (; kt + NSTAGE < nk; kt += NSTAGE) {
-      phase(I0{}, kt, std::true_type{});
-      phase(I1{}, kt + 1, std::true_type{});
-      phase(I2{}, kt + 2, std::true_type{});
-      if (NSTAGE > 3) phase(I3{}, kt + 3, std::true_type{});
-      if (NSTAGE > 4) phase(I4{}, kt + 4, std::true_type{});
-      if (NSTAGE > 5) phase(I5{}, kt + 5, std::true_type{});
-    }
-    for (; kt < nk; kt += NSTAGE) {
-      phase(I0{}, kt, std::false_type{});
-      phase(I1{}, kt + 1, std::false_type{});
-      phase(I2{}, kt + 2, std::false_type{});
-      if (NSTAGE > 3) phase(I3{}, kt + 3, std::false_type{});
-      if (NSTAGE > 4) phase(I4{}, kt + 4, std::false_type{});
-      if (NSTAGE > 5) phase(I5{}, kt + 5, std::false_type{});
-    }
+    for (; kt + NSTAGE < nk; kt += NSTAGE) round(kt, std::true_type{});
+    for (; kt < nk; kt += NSTAGE) round(kt, std::false_type{});
   }
   const bool computes = wave < 4;
 
@@ -825,17 +825,17 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   finish_tile<T, BM, BN, 512>(p, ct, m0, n0, tid, grp, zo, zi);
 }
 
-template <typename T, int BM, int BN, int NSTAGE>
+template <typename T, int BM, int BN, int NSTAGE, int SB>
 static int launch_dma(hipStream_t s, const GemmArgs& a, bool akc, bool bkc, dim3 grid) {
   const dim3 block(512);
   if (akc && bkc)
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, true, NSTAGE>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, true, NSTAGE, SB>), grid, block, 0, s, a);
   else if (akc && !bkc)
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, false, NSTAGE>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, false, NSTAGE, SB>), grid, block, 0, s, a);
   else if (!akc && bkc)
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, true, NSTAGE>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, true, NSTAGE, SB>), grid, block, 0, s, a);
   else
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, false, NSTAGE>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, false, NSTAGE, SB>), grid, block, 0, s, a);
   RTP_LAUNCH_CHECK();
   return RTP_OK;
 }
@@ -1005,7 +1005,7 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
     return e ? atoi(e) : -1;
   }();
   static const double slab_ns[kNumShapes] = {1059.0, 540.0, 294.0, 172.0};
-  const double nslabs = (double)ceil_div(d->k * (int64_t)sizeof(T), kSlabBytes) * (double)d->ksegs;
+  static const int slab_bytes[kNumShapes] = {128, 128, 128, 128};
   int shape = kNumShapes - 1;
   double best = 0.0;
   for (int i = 0; fast && i < kNumShapes; ++i) {
@@ -1013,6 +1013,7 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
     if (kShapes[i].bm > 64 && kShapes[i].bm > ceil_div(d->m, 64) * 64) continue;
     if (kShapes[i].bn > 64 && kShapes[i].bn > ceil_div(d->n, 64) * 64) continue;
     const int64_t tiles = ceil_div(d->m, kShapes[i].bm) * ceil_div(d->n, kShapes[i].bn) * nz;
+    const double nslabs = (double)ceil_div(d->k * (int64_t)sizeof(T), slab_bytes[i]) * (double)d->ksegs;
     const double cost = (double)ceil_div(tiles, 256) * (nslabs * slab_ns[i] + 3000.0);
     if (best == 0.0 || cost < best || i == forced) {
       best = i == forced ? -1.0 : cost;
@@ -1066,13 +1067,13 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   if (!fast) return launch_layout<T, 64, 64, 1, false>(s, a, akc, bkc, grid);
   switch (shape) {
     case 0:
-      return launch_dma<T, 256, 128, 3>(s, a, akc, bkc, grid);
+      return launch_dma<T, 256, 128, 3, 128>(s, a, akc, bkc, grid);
     case 1:
-      return launch_dma<T, 128, 128, 4>(s, a, akc, bkc, grid);
+      return launch_dma<T, 128, 128, 4, 128>(s, a, akc, bkc, grid);
     case 2:
-      return launch_dma<T, 128, 64, 5>(s, a, akc, bkc, grid);
+      return launch_dma<T, 128, 64, 5, 128>(s, a, akc, bkc, grid);
     default:
-      return launch_dma<T, 64, 64, 4>(s, a, akc, bkc, grid);
+      return launch_dma<T, 64, 64, 4, 128>(s, a, akc, bkc, grid);
   }
 }
 
