@@ -87,3 +87,43 @@ def test_copy_and_zero_kernels_ragged():
         assert torch.equal(dst2[1:n + 1], src[:n]) and dst2[0] == 7 and dst2[n + 1] == 7
         ops.zero_(dst2[1:n + 1])
         assert dst2[1:n + 1].sum() == 0 and dst2[0] == 7 and dst2[n + 1] == 7
+
+
+def test_stage_group_partial_use_and_restage():
+    """Layers of a stage group may also be used alone, out of order, or after a weight update: a member that
+    finds no valid staged copy of itself stages the group again, and a finished pass hands the slot back."""
+    import torch.nn as nn
+    from rtp_amd import emulate_shards, ring
+    from rtp_amd.module.linear import ColumnParallelLinear
+    torch.manual_seed(0)
+    with emulate_shards(4):
+        a = ColumnParallelLinear(32, 64, device=DEV)
+        b = ColumnParallelLinear(64, 32, device=DEV)
+    ring.group_stores([a._store, b._store])
+    x = torch.randn(5, 32, device=DEV)
+
+    def ref(layer, inp):
+        w = torch.cat([l.weight for l in layer.linears], 0)
+        bias = torch.cat([l.bias for l in layer.linears], 0)
+        return inp @ w.t() + bias
+
+    saved = ring.rotation_window()
+    ring.set_rotation_window(None)
+    try:
+        with torch.no_grad():
+            ya = a(x)                      # stages the group, uses one member only
+            ya2 = a(x)                     # the same member again: stages again
+            yb = b(ya)                     # the other member of that staging
+            assert torch.allclose(ya, ref(a, x), atol=1e-5) and torch.equal(ya, ya2)
+            assert torch.allclose(yb, ref(b, ya), atol=1e-5)
+            for l in b.linears:            # weights change under the staged copy
+                l.weight.mul_(2.0)
+            ring.fence(x.device)
+            yb2 = b(ya)
+            assert torch.allclose(yb2, ref(b, ya), atol=1e-5)
+            yb3 = b(ya)                    # b, then a: reverse order of the declaration
+            ya3 = a(x)
+            assert torch.equal(yb3, yb2) and torch.equal(ya3, ya)
+    finally:
+        ring.set_rotation_window(saved)
+    torch.cuda.synchronize()
