@@ -15,7 +15,7 @@ from ..module.collectives import emulate_shards
 from ..module.embedding import ParallelEmbedding
 from ..module.linear import ColumnParallelLinear, column_relu_mlp
 from ..module.moe import WeightMOELayer
-from ..module.norm import add_layer_norm
+from ..module.norm import add_layer_norm, layer_norm_fusable
 from ..module.top2gate import WeightTop2Gate
 
 
@@ -74,10 +74,16 @@ class FeedForwardLayer(nn.Module):
         self.dropout1 = nn.Dropout(dropout)
         self.dropout2 = nn.Dropout(dropout)
 
-    def forward(self, x):
-        if isinstance(self.activation, nn.ReLU) and not (self.training and self.dropout1.p > 0) and x.is_cuda:
+    def fusable(self, x) -> bool:
+        return isinstance(self.activation, nn.ReLU) and not (self.training and self.dropout1.p > 0) and x.is_cuda
+
+    def forward(self, x, residual_grad=False):
+        if self.fusable(x):
             # ReLU folded into the epilogues of the two rotated products
-            return self.dropout2(column_relu_mlp(x, self.linear1, self.linear2))
+            y = column_relu_mlp(x, self.linear1, self.linear2, residual_grad=residual_grad)
+            return y if self.dropout2.p == 0.0 or not self.training else self.dropout2(y)
+        if residual_grad:
+            raise RuntimeError("FeedForwardLayer: residual_grad needs the fused ReLU path")
         return self.dropout2(self.linear2(self.dropout1(self.activation(self.linear1(x)))))
 
 
@@ -118,13 +124,22 @@ class TransformerEncoderLayer(nn.Module):
             x = x + self._sa_block(self.norm1(x), src_mask, src_key_padding_mask)
             x = x + self._ff_block(self.norm2(x))
         else:
-            x = add_layer_norm(x, self._sa_block(x, src_mask, src_key_padding_mask), self.norm1)
-            x = add_layer_norm(x, self._ff_block(x), self.norm2)
+            # With the fused add + LayerNorm, x's gradient is routed through the branch: its last input-gradient
+            # product adds the residual part in its epilogue instead of a separate elementwise add.
+            no_drop = self.dropout.p == 0.0 or not self.training  # nothing between a branch and its LayerNorm
+            via = layer_norm_fusable(x, self.norm1) and x.requires_grad and torch.is_grad_enabled() and no_drop
+            x = add_layer_norm(x, self._sa_block(x, src_mask, src_key_padding_mask, residual_grad=via), self.norm1,
+                               x_grad_via_branch=via)
+            via = (via and not self.is_moe and self.ff_block.fusable(x)
+                   and (self.ff_block.dropout2.p == 0.0 or not self.training))
+            x = add_layer_norm(x, self.ff_block(x, residual_grad=True) if via else self._ff_block(x), self.norm2,
+                               x_grad_via_branch=via)
         return x
 
-    def _sa_block(self, x, attn_mask, key_padding_mask):
-        x = self.self_attn(x, x, x, attn_mask=attn_mask, key_padding_mask=key_padding_mask, need_weights=False)[0]
-        return self.dropout(x)
+    def _sa_block(self, x, attn_mask, key_padding_mask, residual_grad=False):
+        x = self.self_attn(x, x, x, attn_mask=attn_mask, key_padding_mask=key_padding_mask, need_weights=False,
+                           residual_grad=residual_grad)[0]
+        return x if self.dropout.p == 0.0 or not self.training else self.dropout(x)
 
     def _ff_block(self, x):
         return self.moe_layer(x) if self.is_moe else self.ff_block(x)

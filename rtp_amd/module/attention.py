@@ -103,7 +103,7 @@ class _AttentionFn(torch.autograd.Function):
     batch, head) triple is addressed by strides inside the batched GEMM, so nothing is re-laid out."""
 
     @staticmethod
-    def forward(ctx, x, anchor, layer, mask, causal, want_weights):
+    def forward(ctx, x, anchor, layer, mask, causal, want_weights, residual_grad=False):
         store = layer._store
         L, N, E = x.shape
         ws, h_s, d, e_s = layer.world_size, layer.num_heads_per_partition, layer.head_dim, layer.embed_dim_per_partition
@@ -157,6 +157,7 @@ class _AttentionFn(torch.autograd.Function):
             weights = p[last * Z:(last + 1) * Z].view(N, h_s, L, L)
         ctx.layer = layer
         ctx.dims = (L, N, E)
+        ctx.residual_grad = residual_grad
         ctx.save_for_backward(x2, qkv, p, o)
         ctx.mark_non_differentiable(*([weights] if weights is not None else []))
         return out.view(L, N, E), weights
@@ -182,7 +183,10 @@ class _AttentionFn(torch.autograd.Function):
         fused = ops.attn_supported(dt, L, d)
         order = ring_order(layer.rank, ws, reverse=True)
         rot = Rotation(store.home, order, group=store.stage_group)
-        acc = ops.ShardSum(dx, sum(len(w) for w in rot.windows)) if need_dx else None
+        # residual_grad: the caller's y = norm(x + attention(x)) sends x's whole gradient through this function,
+        # which adds the output gradient to its own input gradient in the epilogue of the last product
+        init = dout2 if ctx.residual_grad else None
+        acc = ops.ShardSum(dx, sum(len(w) for w in rot.windows), init=init) if need_dx else None
         i = 0
         for j in range(rot.steps):
             for flat, first, cnt in rot.acquire(j):
@@ -236,7 +240,7 @@ class _AttentionFn(torch.autograd.Function):
             store.grads_ready()
 
         run_wgrad(dev, param_grads, (dout2, o, dqkv, x2))
-        return (dx.view(L, N, E) if need_dx else None), None, None, None, None, None
+        return (dx.view(L, N, E) if need_dx else None), None, None, None, None, None, None
 
 
 class ParallelMultiheadAttention(RotatedLayer):
@@ -270,7 +274,7 @@ class ParallelMultiheadAttention(RotatedLayer):
 
     def forward(self, query: Tensor, key: Tensor, value: Tensor, key_padding_mask: Optional[Tensor] = None,
                 need_weights: bool = True, attn_mask: Optional[Tensor] = None, average_attn_weights: bool = True,
-                is_causal: bool = False, test_tensor=None) -> Tuple[Tensor, Optional[Tensor]]:
+                is_causal: bool = False, test_tensor=None, residual_grad: bool = False) -> Tuple[Tensor, Optional[Tensor]]:
         if not (key is query and value is query):
             if not (key.data_ptr() == query.data_ptr() == value.data_ptr() and key.shape == query.shape == value.shape
                     and key.stride() == query.stride() == value.stride()):
@@ -293,7 +297,7 @@ class ParallelMultiheadAttention(RotatedLayer):
             mask = mask.to(device=x.device, dtype=torch.float32).contiguous()
         elif is_causal:
             causal = True
-        out, weights = _AttentionFn.apply(x, self._anchor, self, mask, causal, bool(need_weights))
+        out, weights = _AttentionFn.apply(x, self._anchor, self, mask, causal, bool(need_weights), bool(residual_grad))
         if need_weights and weights is not None and average_attn_weights:
             weights = weights.float().mean(dim=1).to(out.dtype)
         if self.batch_first:

@@ -122,7 +122,7 @@ class _ColumnReluMlpFn(torch.autograd.Function):
     input-gradient product.  Same values as the three separate modules."""
 
     @staticmethod
-    def forward(ctx, x, anchor1, anchor2, lin1, lin2):
+    def forward(ctx, x, anchor1, anchor2, lin1, lin2, residual_grad=False):
         k1, f, n2 = lin1.in_features, lin1.out_features, lin2.out_features
         x2 = as_rows(x, k1)
         rows, dt, dev = x2.shape[0], x2.dtype, x2.device
@@ -138,6 +138,7 @@ class _ColumnReluMlpFn(torch.autograd.Function):
                 rot.release(j)
         ctx.layers = (lin1, lin2)
         ctx.x_shape = x.shape
+        ctx.residual_grad = residual_grad
         ctx.save_for_backward(x2, h)
         return y.view(*x.shape[:-1], n2)
 
@@ -157,7 +158,9 @@ class _ColumnReluMlpFn(torch.autograd.Function):
             if dinp is not None:
                 rot = Rotation(store.home, order, group=store.stage_group)
                 steps = sum(len(w) for w in rot.windows)
-                acc = ops.ShardSum(dinp, steps)
+                # residual_grad: y = norm(x + mlp(x)) sends x's whole gradient through here (dy + mlp'(dy))
+                init = dy2 if (ctx.residual_grad and lin is lin1) else None
+                acc = ops.ShardSum(dinp, steps, init=init)
                 i = 0
                 for j in range(rot.steps):
                     for flat, first, cnt in rot.acquire(j):
@@ -176,14 +179,19 @@ class _ColumnReluMlpFn(torch.autograd.Function):
                 store.grads_ready()
 
             run_wgrad(g.device, param_grads, (g, inp))
-        return (dx.view(ctx.x_shape) if need_dx else None), None, None, None, None
+        return (dx.view(ctx.x_shape) if need_dx else None), None, None, None, None, None
 
 
-def column_relu_mlp(x: torch.Tensor, lin1: "ColumnParallelLinear", lin2: "ColumnParallelLinear") -> torch.Tensor:
-    """lin2(relu(lin1(x))) with the ReLU fused into the products of the two rotated layers."""
+def column_relu_mlp(x: torch.Tensor, lin1: "ColumnParallelLinear", lin2: "ColumnParallelLinear",
+                    residual_grad: bool = False) -> torch.Tensor:
+    """lin2(relu(lin1(x))) with the ReLU fused into the products of the two rotated layers.  residual_grad: the
+    backward returns dy + mlp'(dy), for a caller whose residual connection does not propagate x's gradient itself
+    (add_layer_norm(..., x_grad_via_branch=True))."""
     if lin1.out_features != lin2.in_features:
         raise ValueError("column_relu_mlp: lin1.out_features must equal lin2.in_features")
-    return _ColumnReluMlpFn.apply(x, lin1._anchor, lin2._anchor, lin1, lin2)
+    if residual_grad and lin2.out_features != lin1.in_features:
+        raise ValueError("column_relu_mlp: residual_grad needs an output of the input's width")
+    return _ColumnReluMlpFn.apply(x, lin1._anchor, lin2._anchor, lin1, lin2, bool(residual_grad))
 
 
 class _RowLinearFn(torch.autograd.Function):

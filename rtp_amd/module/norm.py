@@ -11,7 +11,7 @@ from .. import ops
 
 class _AddLayerNormFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, r, weight, bias, eps):
+    def forward(ctx, x, r, weight, bias, eps, x_grad_via_branch=False):
         x2, r2 = x.contiguous(), r.contiguous()
         cols = x2.shape[-1]
         rows = x2.numel() // cols
@@ -22,6 +22,7 @@ class _AddLayerNormFn(torch.autograd.Function):
         ops.add_layernorm_fwd(x2, r2, weight, bias, eps, z, y, mean, rstd)
         ctx.save_for_backward(z, weight, mean, rstd)
         ctx.bias = bias
+        ctx.x_grad_via_branch = x_grad_via_branch
         return y
 
     @staticmethod
@@ -45,15 +46,25 @@ class _AddLayerNormFn(torch.autograd.Function):
             if bias is not None:
                 bs.overwrite = False
                 bias.grad = bs.view
-            return dz, dz, None, None, None
-        return dz, dz, dgamma, dbeta, None
+            return (None if ctx.x_grad_via_branch else dz), dz, None, None, None, None
+        return (None if ctx.x_grad_via_branch else dz), dz, dgamma, dbeta, None, None
 
 
-def add_layer_norm(x: torch.Tensor, r: torch.Tensor, norm: nn.LayerNorm) -> torch.Tensor:
-    """norm(x + r).  Fused on the device when the row length qualifies, else the two torch calls."""
-    fused = (x.is_cuda and x.shape == r.shape and x.dtype == r.dtype and norm.elementwise_affine
-             and len(norm.normalized_shape) == 1 and norm.normalized_shape[0] == x.shape[-1]
-             and norm.weight.dtype == x.dtype and ops.layernorm_supported(x.dtype, x.shape[-1]))
+def layer_norm_fusable(x: torch.Tensor, norm: nn.LayerNorm) -> bool:
+    """Whether add_layer_norm(x, r, norm) takes the fused kernels for a branch output r shaped like x."""
+    return bool(x.is_cuda and norm.elementwise_affine and len(norm.normalized_shape) == 1
+                and norm.normalized_shape[0] == x.shape[-1] and norm.weight.dtype == x.dtype
+                and ops.layernorm_supported(x.dtype, x.shape[-1]))
+
+
+def add_layer_norm(x: torch.Tensor, r: torch.Tensor, norm: nn.LayerNorm, x_grad_via_branch: bool = False) -> torch.Tensor:
+    """norm(x + r).  Fused on the device when the row length qualifies, else the two torch calls.
+    x_grad_via_branch: r = f(x) was computed by a rotated layer called with residual_grad=True, whose backward
+    already returns the residual part of x's gradient (added in the epilogue of its last product), so this
+    function gives x no gradient of its own.  Only valid when layer_norm_fusable(x, norm)."""
+    fused = layer_norm_fusable(x, norm) and x.shape == r.shape and x.dtype == r.dtype
     if not fused:
+        if x_grad_via_branch:
+            raise RuntimeError("add_layer_norm: x_grad_via_branch needs the fused path (check layer_norm_fusable)")
         return norm(x + r)
-    return _AddLayerNormFn.apply(x, r, norm.weight, norm.bias, norm.eps)
+    return _AddLayerNormFn.apply(x, r, norm.weight, norm.bias, norm.eps, bool(x_grad_via_branch))

@@ -409,9 +409,11 @@ class ShardSum:
     (row-parallel outputs, attention out-projections, input gradients).  fp32 results accumulate in
     place; bf16 results accumulate in an fp32 scratch and are rounded once, by the last step."""
 
-    def __init__(self, out: torch.Tensor, steps: int):
+    def __init__(self, out: torch.Tensor, steps: int, init: Optional[torch.Tensor] = None):
+        """`init`, if given, is an addend of the sum (the first step reads it as its c_in)."""
         self.out = out
         self.steps = steps
+        self.init = init
         self.scratch = None
         if out.dtype != torch.float32 and steps > 1:
             self.scratch = torch.empty(out.shape, dtype=torch.float32, device=out.device)
@@ -419,10 +421,10 @@ class ShardSum:
     def target(self, i: int):
         """(c_out, c_in) for step i."""
         if self.scratch is None:
-            return self.out, (self.out if i > 0 else None)
+            return self.out, (self.out if i > 0 else self.init)
         if i == self.steps - 1:
             return self.out, self.scratch
-        return self.scratch, (self.scratch if i > 0 else None)
+        return self.scratch, (self.scratch if i > 0 else self.init)
 
 
 class Routing:
