@@ -244,6 +244,7 @@ def main():
     import torch
     import torch.nn.functional as F
     from rtp_amd import _lib, ring, rotated_weight_bytes, staging_bytes
+    from rtp_amd.module.loss import cross_entropy
     from rtp_amd.optim import RotatedSGD
 
     dev = torch.device("cuda", 0)
@@ -261,7 +262,7 @@ def main():
     def step():
         opt.zero_grad()
         logits = lm(ids)
-        loss = F.cross_entropy(logits.float().view(-1, c["vocab"]), tgt.view(-1))
+        loss = cross_entropy(logits.view(-1, c["vocab"]), tgt.view(-1))
         loss.backward()
         opt.step()
         loss_box[0] = loss.detach()  # detached: a live autograd graph would pin last step's AccumulateGrad nodes

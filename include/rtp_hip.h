@@ -245,6 +245,24 @@ int rtp_layernorm_bwd(void* stream, int dtype, const void* dy, const void* z, co
                       void* dgamma, void* dbeta, void* workspace, size_t workspace_bytes);
 
 /* ---------------------------------------------------------------------------------------------
+ * Softmax cross-entropy over the vocabulary axis of the LM's logits (reference harness:
+ * nn.CrossEntropyLoss()(outputs.view(-1, vocab_size), labels.view(-1)), test_transformer.py:195-197,
+ * there a log-softmax, a gather and their backward over an fp32 copy of the logits).
+ *   fwd: stats[r] = {m, s}, m = max_j logits[r, j], s = sum_j exp(logits[r, j] - m) (fp32 [rows, 2]);
+ *        loss[r] = (m - logits[r, target[r]]) + log s (fp32 [rows]).
+ *   bwd: dlogits[r, j] = (exp(logits[r, j] - m) / s - [j == target[r]]) * dloss[r * dloss_stride],
+ *        dloss fp32 (dloss_stride 0: one scalar for all rows, 1: one value per row).
+ * A row whose target lies outside [0, cols) has loss 0 and gradient 0 (an ignored row).
+ * fp32 or bf16 logits, statistics in fp32; cols and both leading dimensions multiples of 16 bytes.
+ * dlogits may alias logits.
+ * --------------------------------------------------------------------------------------------- */
+int rtp_softmax_xent_fwd(void* stream, int dtype, const void* logits, int64_t ld, int64_t rows, int64_t cols,
+                         const int64_t* target, float* loss, float* stats);
+int rtp_softmax_xent_bwd(void* stream, int dtype, const void* logits, int64_t ld, int64_t rows, int64_t cols,
+                         const int64_t* target, const float* stats, const float* dloss, int64_t dloss_stride,
+                         void* dlogits, int64_t ld_dlogits);
+
+/* ---------------------------------------------------------------------------------------------
  * Top-2 routing (reference: top2gating, rtp/module/top2gate.py:43-105).
  * Inputs logits[S,E] fp32 and noise[S,E] fp32 (the Gumbel sample of top2gate.py:61, supplied by the
  * caller so that routing is a pure function of its inputs).  Outputs, per token s:

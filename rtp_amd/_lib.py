@@ -85,6 +85,8 @@ PROTOTYPES = {
     "rtp_add_layernorm_fwd": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _f, _i64, _i64, _vp, _vp, _vp, _vp]),
     "rtp_layernorm_bwd_workspace_bytes": (_sz, [_i64, _i64]),
     "rtp_layernorm_bwd": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _sz]),
+    "rtp_softmax_xent_fwd": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _vp, _vp, _vp]),
+    "rtp_softmax_xent_bwd": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _i64]),
     "rtp_top2_route_workspace_bytes": (_sz, [_i64, _i64]),
     "rtp_top2_route": (_i, [_vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz]),
     "rtp_top2_route_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),

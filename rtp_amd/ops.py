@@ -3,7 +3,7 @@ pointers plus the current torch stream to librtp_hip.so, and never compute anyth
 from __future__ import annotations
 
 import ctypes as C
-from typing import Optional
+from typing import Optional, Tuple
 
 import torch
 
@@ -349,6 +349,60 @@ def layernorm_bwd(dy: torch.Tensor, z: torch.Tensor, gamma: torch.Tensor, mean: 
     check(lib.rtp_layernorm_bwd(_stream(), dtype_code(z.dtype), dy.data_ptr(), z.data_ptr(), gamma.data_ptr(),
                                 mean.data_ptr(), rstd.data_ptr(), rows, cols, dz.data_ptr(), dgamma.data_ptr(),
                                 dbeta.data_ptr() if dbeta is not None else None, ws.data_ptr(), nbytes))
+
+
+def softmax_xent_supported(logits: torch.Tensor) -> bool:
+    if logits.dtype not in (torch.float32, torch.bfloat16) or logits.dim() != 2 or not logits.is_cuda:
+        return False
+    vec = 16 // logits.element_size()
+    return bool(logits.stride(1) == 1 and logits.shape[1] >= vec and logits.shape[1] % vec == 0
+                and logits.stride(0) >= logits.shape[1] and logits.stride(0) % vec == 0
+                and logits.data_ptr() % 16 == 0)
+
+
+def _xent_check(who: str, logits: torch.Tensor, target: torch.Tensor) -> None:
+    _dev(logits)
+    if not softmax_xent_supported(logits):
+        raise ValueError(f"{who}: logits must be fp32/bf16 [rows, cols], unit column stride, cols and the row "
+                         "stride multiples of 16 bytes")
+    if target.dtype != torch.int64 or target.numel() != logits.shape[0] or not target.is_contiguous() or \
+            target.device != logits.device:
+        raise ValueError(f"{who}: target must be contiguous int64 [rows] on the logits' device")
+
+
+def softmax_xent_fwd(logits: torch.Tensor, target: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-row cross-entropy loss (fp32 [rows]) and softmax statistics {max, sum exp} (fp32 [rows, 2])."""
+    _xent_check("softmax_xent_fwd", logits, target)
+    rows, cols = logits.shape
+    loss = torch.empty(rows, dtype=torch.float32, device=logits.device)
+    stats = torch.empty((rows, 2), dtype=torch.float32, device=logits.device)
+    _lib.require_device()
+    check(_lib.load().rtp_softmax_xent_fwd(_stream(), dtype_code(logits.dtype), logits.data_ptr(), logits.stride(0),
+                                           rows, cols, target.data_ptr(), loss.data_ptr(), stats.data_ptr()))
+    return loss, stats
+
+
+def softmax_xent_bwd(logits: torch.Tensor, target: torch.Tensor, stats: torch.Tensor, dloss: torch.Tensor,
+                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """dlogits = (softmax(logits) - onehot(target)) * dloss[row]; dloss fp32 [rows], stride 0 or 1."""
+    _xent_check("softmax_xent_bwd", logits, target)
+    rows, cols = logits.shape
+    if dloss.dtype != torch.float32 or dloss.numel() != rows or dloss.dim() != 1:
+        raise ValueError("softmax_xent_bwd: dloss must be fp32 [rows]")
+    if stats.dtype != torch.float32 or stats.shape != (rows, 2) or not stats.is_contiguous():
+        raise ValueError("softmax_xent_bwd: stats must be the contiguous fp32 [rows, 2] of softmax_xent_fwd")
+    if rows > 1 and dloss.stride(0) not in (0, 1):
+        dloss = dloss.contiguous()
+    stride = dloss.stride(0) if rows > 1 else 0
+    if out is None:
+        out = torch.empty((rows, cols), dtype=logits.dtype, device=logits.device)
+    elif out.shape != logits.shape or out.dtype != logits.dtype or not softmax_xent_supported(out):
+        raise ValueError("softmax_xent_bwd: out must match logits")
+    _lib.require_device()
+    check(_lib.load().rtp_softmax_xent_bwd(_stream(), dtype_code(logits.dtype), logits.data_ptr(), logits.stride(0),
+                                           rows, cols, target.data_ptr(), stats.data_ptr(), dloss.data_ptr(), stride,
+                                           out.data_ptr(), out.stride(0)))
+    return out
 
 
 def sgd_step(master: torch.Tensor, grad: torch.Tensor, shadow: Optional[torch.Tensor], lr: float,

@@ -1,0 +1,81 @@
+"""Two-kernel softmax cross-entropy against torch's F.cross_entropy on the fp32 image of the same logits."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from gpu_util import DEV, assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(rows, cols, dtype, seed, pad=0):
+    gen = torch.Generator().manual_seed(seed)
+    store = (torch.randn(rows, cols + pad, generator=gen) * 3.0).to(dtype)
+    target = torch.randint(0, cols, (rows,), generator=gen)
+    return store, target
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,cols,pad", [(1024, 10240, 0), (7, 8, 0), (33, 1000, 24), (1, 4096, 0), (64, 50264, 8)])
+def test_cross_entropy_matches_torch(dtype, rows, cols, pad):
+    from rtp_amd.module.loss import cross_entropy
+    store, target = _case(rows, cols, dtype, rows + cols, pad)
+    ref_in = store[:, :cols].float().clone().requires_grad_()
+    ref = F.cross_entropy(ref_in, target)
+    ref.backward()
+    dev_store = store.to(DEV)
+    x = dev_store[:, :cols].detach().requires_grad_()
+    assert x.stride(0) == cols + pad
+    loss = cross_entropy(x, target.to(DEV))
+    loss.backward()
+    assert loss.dtype == torch.float32
+    assert abs(loss.item() - ref.item()) <= 1e-5 * abs(ref.item())
+    assert x.grad.dtype == dtype
+    assert_close(x.grad, ref_in.grad, dtype, "dlogits")
+
+
+@pytest.mark.parametrize("reduction", ["none", "sum", "mean"])
+def test_cross_entropy_reductions_ignore_index_and_upstream_gradient(reduction):
+    from rtp_amd.module.loss import CrossEntropyLoss
+    rows, cols = 96, 512
+    store, target = _case(rows, cols, torch.bfloat16, 5)
+    target[::5] = -100
+    ref_in = store.float().clone().requires_grad_()
+    ref = F.cross_entropy(ref_in, target, reduction=reduction, ignore_index=-100)
+    w = torch.linspace(0.5, 2.0, rows) if reduction == "none" else torch.tensor(1.7)
+    (ref * w).sum().backward()
+    x = store.to(DEV).requires_grad_()
+    out = CrossEntropyLoss(ignore_index=-100, reduction=reduction)(x, target.to(DEV))
+    (out * w.to(DEV)).sum().backward()
+    assert_close(out, ref, torch.float32, "loss")
+    assert_close(x.grad, ref_in.grad, torch.bfloat16, "dlogits")
+    assert torch.count_nonzero(x.grad[::5]).item() == 0   # ignored rows get no gradient
+
+
+def test_cross_entropy_extreme_logits_stay_finite():
+    from rtp_amd.module.loss import cross_entropy
+    x = torch.zeros(4, 64, dtype=torch.float32)
+    x[0, 3] = 3.0e4
+    x[1, :] = -3.0e4
+    x[2, 5] = -3.0e4
+    target = torch.tensor([3, 0, 5, 1])
+    ref_in = x.clone().requires_grad_()
+    ref = F.cross_entropy(ref_in, target, reduction="none")
+    ref.sum().backward()
+    xd = x.to(DEV).requires_grad_()
+    out = cross_entropy(xd, target.to(DEV), reduction="none")
+    out.sum().backward()
+    assert torch.isfinite(out).all() and torch.isfinite(xd.grad).all()
+    assert_close(out, ref, torch.float32, "loss")
+    assert_close(xd.grad, ref_in.grad, torch.float32, "dlogits")
+
+
+def test_cross_entropy_falls_back_for_unsupported_layouts():
+    from rtp_amd import ops
+    from rtp_amd.module.loss import cross_entropy
+    x = torch.randn(6, 37, device=DEV)
+    t = torch.randint(0, 37, (6,), device=DEV)
+    assert not ops.softmax_xent_supported(x)
+    assert torch.equal(cross_entropy(x, t), F.cross_entropy(x, t))
+    with pytest.raises(ValueError):
+        ops.softmax_xent_fwd(x, t)
