@@ -548,11 +548,20 @@ struct DmaOperand {
   static constexpr int NI = R * SB / 1024 / NL;   // load instructions (1 KiB each) per loader wave and slab
   static constexpr int BYTES = R * SB;            // one stage of this operand
   static constexpr int LINE = R * (int)sizeof(T); // bytes of one k line when rows are contiguous
-  const T* ptr[NI];  // source of the NEXT slab's vector, advanced in place
-  int koff[NI];      // k of the vector inside its slab
+  // The lane's vector sits at `ofs` bytes from the slab's base pointer, which is the same for every lane and lives
+  // in scalar registers: the loader's steady state then has no vector-ALU instruction at all.  (A vector add per
+  // load has to compete for issue slots with the MFMAs of the compute wave on the same SIMD, and loses: measured,
+  // per-lane 64-bit pointers make the loads of a slab take the MFMA time longer.)
+  unsigned ofs[NI];
+  int koff[NI];  // k of the vector inside its slab
 
-  // lw: index of the loader wave (0..NL-1).
-  __device__ __forceinline__ void init(const T* base, long ld, int row0, int rows, int lw, int lane) {
+  // Base pointer of the first slab: row row0 of a K-contiguous operand, element row0 of k line 0 otherwise.
+  __device__ __forceinline__ static const char* slab_base(const T* x, long ld, int row0) {
+    return reinterpret_cast<const char*>(KC ? x + (long)row0 * ld : x + row0);
+  }
+
+  // lw: index of the loader wave (0..NL-1).  The host guarantees that a tile's offsets fit 32 bits.
+  __device__ __forceinline__ void init(long ld, int row0, int rows, int lw, int lane) {
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
       const int j = lw * NI + i;  // which KiB of the stage
@@ -560,37 +569,42 @@ struct DmaOperand {
         constexpr int LPR = SB / 16;  // lanes (16-byte chunks) per row
         const int row = j * (64 / LPR) + lane / LPR;
         const int c = (lane % LPR) ^ kc_swizzle<SB>(row);
-        const int rr = row0 + row < rows ? row0 + row : rows - 1;
-        ptr[i] = base + (long)rr * ld + c * VEC;
+        const int rr = row0 + row < rows ? row : rows - 1 - row0;  // rows past the end re-read the last one
+        ofs[i] = (unsigned)((long)rr * ld * (long)sizeof(T)) + (unsigned)(c * 16);
         koff[i] = c * VEC;
       } else {
         const int byte = lane * 16;
         const int kl = j * (1024 / LINE) + byte / LINE;
-        const int chunk = ((byte % LINE) >> 4) ^ rc_swizzle<T, R>(kl);  // which 16 bytes of the k line land here
-        int rr = row0 + chunk * VEC;
-        if (rr + VEC > rows) rr = 0;
-        ptr[i] = base + (long)kl * ld + rr;
+        int chunk = ((byte % LINE) >> 4) ^ rc_swizzle<T, R>(kl);  // which 16 bytes of the k line land here
+        if (row0 + chunk * VEC + VEC > rows) chunk = 0;           // past the end: re-read the tile's first rows
+        ofs[i] = (unsigned)((long)kl * ld * (long)sizeof(T)) + (unsigned)(chunk * 16);
         koff[i] = kl;
       }
     }
   }
 
-  // Start the loads of the next slab into the stage at LDS byte address `lds_stage` (this operand's part) and
-  // move the pointers on by `advance` elements.  LAST: the slab is the last of its K segment (first k = k0),
-  // the only one that can reach beyond the contraction length kdim; vectors beyond it come from a block of zeros.
-  template <bool LAST>
-  __device__ __forceinline__ void issue(unsigned lds_stage, int lw, long advance, int k0, int kdim) {
+  // Start the loads of the slab at `base` into the stage at LDS byte address `lds_stage` (this operand's part).
+  // TAIL: the slab is the last of its K segment (first k = k0) and reaches beyond the contraction length kdim;
+  // vectors beyond it come from a block of zeros (per-lane addresses, the one case that needs them).
+  template <bool TAIL>
+  __device__ __forceinline__ void issue(unsigned lds_stage, int lw, const char* base, int k0, int kdim) const {
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-      const T* src = ptr[i];
-      if (LAST && k0 + koff[i] >= kdim) src = reinterpret_cast<const T*>(g_zero16);
       // Inline assembly on purpose: the compiler must not track this instruction (it would make LDS reads wait
       // for all outstanding loads); the kernel's explicit s_waitcnt + barrier protocol is the ordering that counts.
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                   :
-                   : "s"(lds_stage + (unsigned)((lw * NI + i) * 1024)), "v"(src)
-                   : "memory");
-      ptr[i] += advance;
+      if (TAIL) {
+        const char* src = base + ofs[i];
+        if (k0 + koff[i] >= kdim) src = reinterpret_cast<const char*>(g_zero16);
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                     :
+                     : "s"(lds_stage + (unsigned)((lw * NI + i) * 1024)), "v"(src)
+                     : "memory");
+      } else {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(lds_stage + (unsigned)((lw * NI + i) * 1024)), "v"(ofs[i]), "s"(base)
+                     : "memory");
+      }
     }
   }
 };
@@ -698,23 +712,34 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
     const T* B = reinterpret_cast<const T*>(p.b) + grp * p.b_sg + zo * p.b_so + zi * p.b_si;
     DA da;
     DB db;
-    da.init(A, p.lda, m0, p.m, lw, lane);
-    db.init(B, p.ldb, n0, p.n, lw, lane);
-    const long step_a = AKC ? (long)BK : (long)BK * p.lda, step_b = BKC ? (long)BK : (long)BK * p.ldb;
+    da.init(p.lda, m0, p.m, lw, lane);
+    db.init(p.ldb, n0, p.n, lw, lane);
+    const char* ca = DA::slab_base(A, p.lda, m0);  // base of the next slab, uniform: scalar registers
+    const char* cb = DB::slab_base(B, p.ldb, n0);
+    constexpr long SZ = (long)sizeof(T);
+    const long step_a = (AKC ? (long)BK : (long)BK * p.lda) * SZ, step_b = (BKC ? (long)BK : (long)BK * p.ldb) * SZ;
     // after the last slab of a segment the pointers move to the start of the next segment
-    const long last_a = step_a + p.a_sk - nk_seg * step_a, last_b = step_b + p.b_sk - nk_seg * step_b;
+    const long last_a = step_a + p.a_sk * SZ - nk_seg * step_a, last_b = step_b + p.b_sk * SZ - nk_seg * step_b;
     const int k0_last = (nk_seg - 1) * BK;
+    const bool tail = p.k % BK != 0;
     const unsigned lds0 = (unsigned)(uintptr_t)(lptr_t)lds;
     unsigned fill = lds0;  // LDS address of the stage the next slab goes to
     int left = nk_seg;     // slabs left in the current K segment, the next one included
     auto issue = [&]() {
+      if (left != 1 || !tail) {
+        da.template issue<false>(fill, lw, ca, 0, 0);
+        db.template issue<false>(fill + DA::BYTES, lw, cb, 0, 0);
+      } else {
+        da.template issue<true>(fill, lw, ca, k0_last, p.k);
+        db.template issue<true>(fill + DA::BYTES, lw, cb, k0_last, p.k);
+      }
       if (left != 1) {
-        da.template issue<false>(fill, lw, step_a, 0, 0);
-        db.template issue<false>(fill + DA::BYTES, lw, step_b, 0, 0);
+        ca += step_a;
+        cb += step_b;
         --left;
       } else {
-        da.template issue<true>(fill, lw, last_a, k0_last, p.k);
-        db.template issue<true>(fill + DA::BYTES, lw, last_b, k0_last, p.k);
+        ca += last_a;
+        cb += last_b;
         left = nk_seg;
       }
       fill += STAGE;
@@ -970,8 +995,10 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   // Branch-free loads need whole 16-byte vectors: aligned operands and extents that are multiples of VEC
   // along each operand's contiguous axis.  Anything else goes to the guarded small-tile kernel.
   const bool akc = d->a_kcontig, bkc = d->b_kcontig;
+  // ... and a tile's byte offsets from its first vector must fit 32 bits (256 rows or k lines of one leading dimension)
+  const int64_t ld_max = ((int64_t)1 << 24) / (int64_t)sizeof(T) - 64;
   const bool fast = a.vec_a && a.vec_b && ((akc || bkc) ? mult(d->k, VEC) : true) && (akc || mult(d->m, VEC)) &&
-                    (bkc || mult(d->n, VEC)) && d->k > 0;
+                    (bkc || mult(d->n, VEC)) && d->k > 0 && d->lda <= ld_max && d->ldb <= ld_max;
   const int64_t nz = d->batch * d->groups;
   if (d->m <= 64 && d->n <= 64 && d->k * d->ksegs <= 256) {
     // one wavefront per 32 x 32 block
@@ -1004,7 +1031,7 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
     const char* e = getenv("RTP_GEMM_TILE");  // debugging aid: index into kShapes
     return e ? atoi(e) : -1;
   }();
-  static const double slab_ns[kNumShapes] = {1059.0, 540.0, 294.0, 172.0};
+  static const double slab_ns[kNumShapes] = {966.0, 470.0, 283.0, 167.0};
   static const int slab_bytes[kNumShapes] = {128, 128, 128, 128};
   int shape = kNumShapes - 1;
   double best = 0.0;

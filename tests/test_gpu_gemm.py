@@ -19,7 +19,7 @@ def _rand(shape, dtype, gen):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("akc,bkc", [(True, True), (True, False), (False, True), (False, False)])
-@pytest.mark.parametrize("m,n,k", [(8, 8, 8), (33, 65, 17), (100, 36, 70), (256, 192, 128), (1024, 256, 520)])
+@pytest.mark.parametrize("m,n,k", [(8, 8, 8), (33, 65, 17), (100, 36, 70), (256, 192, 128), (1024, 256, 520), (1000, 200, 136)])
 def test_gemm_layouts(dtype, akc, bkc, m, n, k):
     ops = _ops()
     gen = torch.Generator().manual_seed(m * 31 + n * 7 + k)
@@ -170,3 +170,21 @@ def test_gemm_mid_tile_path(dtype, m, n, k):
     dw = torch.empty(n, k, dtype=dtype, device=DEV)
     ops.linear_wgrad(dy, a.to(DEV), dw)
     assert rel_err(dw, dy.double().cpu().t() @ a.double()) <= TOL[dtype]
+
+
+def test_gemm_huge_leading_dimension_takes_guarded_kernel():
+    """A tile's byte offsets must fit 32 bits in the wave-specialised kernel; a leading dimension beyond that
+    (here 16 MiB per row) is served by the guarded kernel with the same result."""
+    ops = _ops()
+    m, n, k, lda = 16, 64, 64, 1 << 23
+    gen = torch.Generator().manual_seed(3)
+    a = _rand((m, k), torch.bfloat16, gen)
+    b = _rand((n, k), torch.bfloat16, gen)
+    big = torch.zeros(m * lda, dtype=torch.bfloat16, device=DEV)
+    big.view(m, lda)[:, :k] = a.to(DEV)
+    bd = b.to(DEV)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.gemm_raw(torch.bfloat16, a=big.data_ptr(), b=bd.data_ptr(), c_out=out.data_ptr(), m=m, n=n, k=k,
+                 lda=lda, ldb=k, ldc=n, a_kcontig=True, b_kcontig=True)
+    torch.cuda.synchronize()
+    assert rel_err(out, a.double() @ b.double().t()) <= TOL[torch.bfloat16]
