@@ -647,7 +647,7 @@ __device__ __forceinline__ Frag<T> read_frag_dma(const char* st, int rowbase, in
   return u.f;
 }
 
-template <typename T, int BM, int BN, bool AKC, bool BKC, int NSTAGE, int SB>
+template <typename T, int BM, int BN, bool AKC, bool BKC, int NSTAGE, int SB, int PD>
 __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   constexpr int NL = 4;  // loader waves (waves 4..7); waves 0..3 compute
   using DA = DmaOperand<T, BM, AKC, NL, SB>;
@@ -765,57 +765,53 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
     }
   } else {
     // ---- compute waves ----
-    // The KS k-steps of a slab are taken in NG groups of G k-steps, with two sets of fragment registers:
-    // while the MFMAs of one group run, the next group is read from LDS into the other set -- the first
-    // group of the NEXT slab during the last group of this one -- so an LDS read always has a group of
-    // MFMAs to hide behind.  Big tiles take G = 1 to fit the register file.
-    constexpr int G = (KS == 4 && MT * NT < 8) ? 2 : 1, NG = KS / G;
-    static_assert(NG == 2 || NG == 4, "two or four fragment groups per slab");
-    Frag<T> fa[2][G][MT], fb[2][G][NT];
-    auto read_group = [&](auto S, auto Q) {
+    // Software pipeline over k-steps (KS per slab, numbered through the slabs): the fragments of k-step t + PD are
+    // read from LDS right before the MFMAs of k-step t are issued, into one of PD + 1 register sets.  A wave gets
+    // one 16-byte LDS read back every ~16 clocks after ~130-200 clocks of latency, so a read needs several k-steps
+    // of MFMAs (32 clocks each) to hide behind; PD is chosen per tile shape for that.  The barrier that makes slab
+    // k+1 visible sits right before its first fragment read, i.e. PD k-steps before its first MFMA.
+    constexpr int NSET = PD + 1;
+    static_assert(PD >= 1 && PD <= KS, "prefetch distance of 1..KS k-steps");
+    static_assert((NSTAGE * KS) % NSET == 0, "register set of a k-step must not depend on the round");
+    Frag<T> fa[NSET][MT], fb[NSET][NT];
+    auto read_step = [&](auto S, auto Q, auto SET) {
       const char* sa = lds + (decltype(S)::value % NSTAGE) * STAGE;
       const char* sb = sa + DA::BYTES;
-      constexpr int q = decltype(Q)::value;
+      constexpr int q = decltype(Q)::value, set = decltype(SET)::value;
 #pragma unroll
-      for (int e = 0; e < G; ++e) {
+      for (int i = 0; i < MT; ++i) fa[set][i] = read_frag_dma<T, BM, AKC, SB>(sa, wm * WM + i * 32, lane, q);
 #pragma unroll
-        for (int i = 0; i < MT; ++i)
-          fa[q & 1][e][i] = read_frag_dma<T, BM, AKC, SB>(sa, wm * WM + i * 32, lane, q * G + e);
-#pragma unroll
-        for (int j = 0; j < NT; ++j)
-          fb[q & 1][e][j] = read_frag_dma<T, BN, BKC, SB>(sb, wn * WN + j * 32, lane, q * G + e);
-      }
+      for (int j = 0; j < NT; ++j) fb[set][j] = read_frag_dma<T, BN, BKC, SB>(sb, wn * WN + j * 32, lane, q);
     };
-    auto mma_group = [&](auto Q) {
-      constexpr int q = decltype(Q)::value;
+    auto mma_step = [&](auto SET) {
+      constexpr int set = decltype(SET)::value;
 #pragma unroll
-      for (int e = 0; e < G; ++e)
+      for (int i = 0; i < MT; ++i)
 #pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-          for (int j = 0; j < NT; ++j) mma(fa[q & 1][e][i], fb[q & 1][e][j], acc[i][j]);
+        for (int j = 0; j < NT; ++j) mma(fa[set][i], fb[set][j], acc[i][j]);
     };
-    using Q0 = std::integral_constant<int, 0>;
-    using Q1 = std::integral_constant<int, 1>;
-    using Q2 = std::integral_constant<int, 2>;
-    using Q3 = std::integral_constant<int, 3>;
-    // Phase of slab k (stage S = k % NSTAGE); on entry the first group of its fragments is in registers.
-    auto phase = [&](auto S, int k, auto STEADY) {
+    // k-step Q of slab k (stage S).  The scheduling fences keep the order written here: left alone, the compiler
+    // sinks every LDS read to just before the MFMA that uses it (fewest live registers), which puts the LDS
+    // latency in front of each MFMA instead of behind earlier ones.
+    auto step = [&](auto S, auto Q, int k, auto STEADY) {
       constexpr bool steady = decltype(STEADY)::value;
-      if (!steady && k >= nk) return;
-      read_group(S, Q1{});
-      mma_group(Q0{});
-      if (NG == 4) {
-        read_group(S, Q2{});
-        mma_group(Q1{});
-        read_group(S, Q3{});
-        mma_group(Q2{});
+      constexpr int s = decltype(S)::value, q = decltype(Q)::value;
+      constexpr int t = s * KS + q;                            // k-step number inside the round
+      constexpr int tq = (q + PD) % KS, ds = (q + PD) / KS;    // the k-step to prefetch: tq of slab k + ds
+      if (steady || k + ds < nk) {
+        if (ds == 1 && tq == 0) __builtin_amdgcn_s_barrier();  // barrier k+1: slab k+1 is visible
+        read_step(std::integral_constant<int, (s + ds) % NSTAGE>{}, std::integral_constant<int, tq>{},
+                  std::integral_constant<int, (t + PD) % NSET>{});
       }
-      if (steady || k + 1 < nk) {
-        __builtin_amdgcn_s_barrier();  // barrier k+1: slab k+1 is visible
-        read_group(std::integral_constant<int, (decltype(S)::value + 1) % NSTAGE>{}, Q0{});
-      }
-      mma_group(std::integral_constant<int, NG - 1>{});
+      __builtin_amdgcn_sched_barrier(0);
+      mma_step(std::integral_constant<int, t % NSET>{});
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    auto phase = [&](auto S, int k, auto STEADY) {
+      if (!decltype(STEADY)::value && k >= nk) return;
+      [&]<int... Q>(std::integer_sequence<int, Q...>) {
+        (step(S, std::integral_constant<int, Q>{}, k, STEADY), ...);
+      }(std::make_integer_sequence<int, KS>{});
     };
     // one round = NSTAGE phases with compile-time stage indices
     auto round = [&](int kt, auto STEADY) {
@@ -824,7 +820,11 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
       }(std::make_integer_sequence<int, NSTAGE>{});
     };
     __builtin_amdgcn_s_barrier();  // barrier 0
-    read_group(std::integral_constant<int, 0>{}, Q0{});
+    [&]<int... Q>(std::integer_sequence<int, Q...>) {
+      (read_step(std::integral_constant<int, 0>{}, std::integral_constant<int, Q>{}, std::integral_constant<int, Q>{}),
+       ...);
+    }(std::make_integer_sequence<int, PD>{});
+    __builtin_amdgcn_sched_barrier(0);
     int kt = 0;
     for (; kt + NSTAGE < nk; kt += NSTAGE) round(kt, std::true_type{});
     for (; kt < nk; kt += NSTAGE) round(kt, std::false_type{});
@@ -850,17 +850,17 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   finish_tile<T, BM, BN, 512>(p, ct, m0, n0, tid, grp, zo, zi);
 }
 
-template <typename T, int BM, int BN, int NSTAGE, int SB>
+template <typename T, int BM, int BN, int NSTAGE, int SB, int PD>
 static int launch_dma(hipStream_t s, const GemmArgs& a, bool akc, bool bkc, dim3 grid) {
   const dim3 block(512);
   if (akc && bkc)
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, true, NSTAGE, SB>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, true, NSTAGE, SB, PD>), grid, block, 0, s, a);
   else if (akc && !bkc)
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, false, NSTAGE, SB>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, false, NSTAGE, SB, PD>), grid, block, 0, s, a);
   else if (!akc && bkc)
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, true, NSTAGE, SB>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, true, NSTAGE, SB, PD>), grid, block, 0, s, a);
   else
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, false, NSTAGE, SB>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, false, NSTAGE, SB, PD>), grid, block, 0, s, a);
   RTP_LAUNCH_CHECK();
   return RTP_OK;
 }
@@ -1094,13 +1094,13 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   if (!fast) return launch_layout<T, 64, 64, 1, false>(s, a, akc, bkc, grid);
   switch (shape) {
     case 0:
-      return launch_dma<T, 256, 128, 3, 128>(s, a, akc, bkc, grid);
+      return launch_dma<T, 256, 128, 3, 128, 1>(s, a, akc, bkc, grid);
     case 1:
-      return launch_dma<T, 128, 128, 4, 128>(s, a, akc, bkc, grid);
+      return launch_dma<T, 128, 128, 4, 128, 3>(s, a, akc, bkc, grid);
     case 2:
-      return launch_dma<T, 128, 64, 5, 128>(s, a, akc, bkc, grid);
+      return launch_dma<T, 128, 64, 5, 128, 4>(s, a, akc, bkc, grid);
     default:
-      return launch_dma<T, 64, 64, 4, 128>(s, a, akc, bkc, grid);
+      return launch_dma<T, 64, 64, 4, 128, 3>(s, a, akc, bkc, grid);
   }
 }
 
