@@ -77,12 +77,20 @@ int rtp_device_check(char* name_out, int name_len);
  * if RTP_GEMM_RELU: v = max(v,0);  if gate: v = gate[m,n] > 0 ? v : 0;  store to c_out as fp32
  * (RTP_GEMM_OUT_F32) or as `dtype`.  c_in is read as fp32 when RTP_GEMM_CIN_F32 is set, else as
  * `dtype`.  bias and gate are `dtype`.  c_in may alias c_out.
+ *
+ * Bias gradient from the same launch (a_rowsum != NULL): a_rowsum[group*rowsum_sg + m] = sum over the
+ * whole contraction of A(m, k), in fp32 with a fixed order, stored as `dtype` (added to the existing value
+ * with RTP_GEMM_ROWSUM_ACCUM).  In the weight-gradient product dW = dY^T X the operand A is dY^T, so this
+ * is nn.Linear's bias gradient (reference: autograd of rtp/module/linear.py:216) without a second pass
+ * over dY.  Only for descriptors rtp_gemm_rowsum_fused() accepts (A stored K x M, batch == 1, and the
+ * alignment the wave-specialised kernel needs); rtp_gemm rejects others, callers use rtp_colsum there.
  * --------------------------------------------------------------------------------------------- */
 enum {
   RTP_GEMM_OUT_F32 = 1,
   RTP_GEMM_CIN_F32 = 2,
   RTP_GEMM_RELU = 4,
-  RTP_GEMM_STREAM_OUT = 8 /* c_out is not read again soon (weight gradients): non-temporal stores */
+  RTP_GEMM_STREAM_OUT = 8, /* c_out is not read again soon (weight gradients): non-temporal stores */
+  RTP_GEMM_ROWSUM_ACCUM = 16 /* a_rowsum is added to, not overwritten */
 };
 
 typedef struct {
@@ -102,9 +110,14 @@ typedef struct {
   float alpha;
   int32_t flags;
   int32_t a_kcontig, b_kcontig;
+  void* a_rowsum;    /* may be NULL; length M per group */
+  int64_t rowsum_sg; /* per-group element stride of a_rowsum */
 } rtp_gemm_desc;
 
 int rtp_gemm(void* stream, int dtype, const rtp_gemm_desc* d);
+
+/* 1 if rtp_gemm would produce d->a_rowsum for this descriptor (the pointer itself may still be NULL), else 0. */
+int rtp_gemm_rowsum_fused(int dtype, const rtp_gemm_desc* d);
 
 /* sizeof(rtp_gemm_desc) as this library was compiled: lets a binding verify its struct layout. */
 size_t rtp_gemm_desc_size(void);

@@ -20,6 +20,7 @@ GEMM_OUT_F32 = 1
 GEMM_CIN_F32 = 2
 GEMM_RELU = 4
 GEMM_STREAM_OUT = 8
+GEMM_ROWSUM_ACCUM = 16
 
 
 class RtpError(RuntimeError):
@@ -42,6 +43,7 @@ class GemmDesc(C.Structure):
         ("gate_sg", C.c_int64), ("bias_sg", C.c_int64), ("a_sk", C.c_int64), ("b_sk", C.c_int64),
         ("bias_sk", C.c_int64),
         ("alpha", C.c_float), ("flags", C.c_int32), ("a_kcontig", C.c_int32), ("b_kcontig", C.c_int32),
+        ("a_rowsum", C.c_void_p), ("rowsum_sg", C.c_int64),
     ]
 
 
@@ -58,6 +60,8 @@ PROTOTYPES = {
     "rtp_abi_version": (_i, []),
     "rtp_device_check": (_i, [C.c_char_p, _i]),
     "rtp_gemm": (_i, [_vp, _i, C.POINTER(GemmDesc)]),
+    "rtp_gemm_rowsum_fused": (_i, [_i, C.POINTER(GemmDesc)]),
+    "rtp_gemm_rowsum_fused": (_i, [_i, C.POINTER(GemmDesc)]),
     "rtp_gemm_desc_size": (_sz, []),
     "rtp_colsum_workspace_bytes": (_sz, [_i64, _i64]),
     "rtp_colsum": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _vp, _i, _i, _i64, _i64, _vp, _sz]),

@@ -42,6 +42,8 @@ struct GemmArgs {
   int tiles_m, tiles_n;
   int vec_c;       // every epilogue operand allows 16-byte accesses of 8 columns
   int xg, xm, xn;  // split of the (batch*groups, tiles_m, tiles_n) space over the 8 XCDs; xg == 0: none
+  char* a_rowsum;  // bias gradient output (sum over k of A's rows), or null
+  long rowsum_sg;
 };
 
 constexpr int kThreads = 256;
@@ -166,6 +168,21 @@ __device__ __forceinline__ void mma(const Frag<float>& a, const Frag<float>& b, 
   // Lane group g holds k = 4g+e in element e, so MFMA number e contracts k in {e, 4+e}.
 #pragma unroll
   for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.f[e], b.f[e], c, 0, 0, 0);
+}
+
+// Sum of the fragment's k values in fp32 (the lane's share of a row sum of A).
+__device__ __forceinline__ float frag_sum(const Frag<bf16_t>& a, float s) {
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  const bf16x2 one = {(__bf16)1.0f, (__bf16)1.0f};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const bf16x2 pr = {a.v[2 * e], a.v[2 * e + 1]};
+    s = __builtin_amdgcn_fdot2_f32_bf16(pr, one, s, false);
+  }
+  return s;
+}
+__device__ __forceinline__ float frag_sum(const Frag<float>& a, float s) {
+  return s + ((a.f[0] + a.f[1]) + (a.f[2] + a.f[3]));
 }
 
 // Fused epilogue shared by the GEMM kernels.  Accumulator register r of lane (li, g) is output row
@@ -701,6 +718,10 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
+  float rsum[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) rsum[i] = 0.0f;
+
   // Barrier protocol: both paths meet the same nk barriers.  Barrier k is passed when slab k is visible to
   // every wave: a loader reaches it only after its own loads of slab k have landed.  A compute wave reaches
   // barrier k+1 after the MFMAs that consumed the last fragments of slab k-1, so once barrier k+1 is passed
@@ -774,6 +795,9 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
     static_assert(PD >= 1 && PD <= KS, "prefetch distance of 1..KS k-steps");
     static_assert((NSTAGE * KS) % NSET == 0, "register set of a k-step must not depend on the round");
     Frag<T> fa[NSET][MT], fb[NSET][NT];
+    // Row sums of A (a bias gradient) ride along in the waves of the tile row's first tile that own column
+    // block 0: each lane adds up the k values of its own row as the fragments pass by.
+    const bool rowsum = p.a_rowsum != nullptr && tile_n == 0 && wn == 0;
     auto read_step = [&](auto S, auto Q, auto SET) {
       const char* sa = lds + (decltype(S)::value % NSTAGE) * STAGE;
       const char* sb = sa + DA::BYTES;
@@ -789,6 +813,10 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
       for (int i = 0; i < MT; ++i)
 #pragma unroll
         for (int j = 0; j < NT; ++j) mma(fa[set][i], fb[set][j], acc[i][j]);
+      if (rowsum) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i) rsum[i] = frag_sum(fa[set][i], rsum[i]);
+      }
     };
     // k-step Q of slab k (stage S).  The scheduling fences keep the order written here: left alone, the compiler
     // sinks every LDS read to just before the MFMA that uses it (fewest live registers), which puts the LDS
@@ -799,12 +827,26 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
       constexpr int t = s * KS + q;                            // k-step number inside the round
       constexpr int tq = (q + PD) % KS, ds = (q + PD) / KS;    // the k-step to prefetch: tq of slab k + ds
       if (steady || k + ds < nk) {
-        if (ds == 1 && tq == 0) __builtin_amdgcn_s_barrier();  // barrier k+1: slab k+1 is visible
+        if (ds == 1 && tq == 0) {
+          __builtin_amdgcn_s_barrier();  // barrier k+1: slab k+1 is visible
+          __builtin_amdgcn_sched_barrier(0);
+        }
         read_step(std::integral_constant<int, (s + ds) % NSTAGE>{}, std::integral_constant<int, tq>{},
                   std::integral_constant<int, (t + PD) % NSET>{});
       }
-      __builtin_amdgcn_sched_barrier(0);
       mma_step(std::integral_constant<int, t % NSET>{});
+      // Issue order inside the step: one MFMA, then its share of the step's LDS reads, and so on.  A wave issues in
+      // order and an MFMA holds the issue port until the matrix pipe takes it, so only what sits between two
+      // MFMAs is issued in an MFMA's shadow; reads bunched up before the first MFMA would leave the pipe idle.
+      constexpr int RPF_A = AKC ? 1 : (sizeof(T) == 2 ? 2 : 4), RPF_B = BKC ? 1 : (sizeof(T) == 2 ? 2 : 4);
+      constexpr int NR = MT * RPF_A + NT * RPF_B, NM = MT * NT * (sizeof(T) == 2 ? 1 : 4);
+      constexpr int PER = (NR + NM - 1) / NM;
+      [&]<int... I>(std::integer_sequence<int, I...>) {
+        ((__builtin_amdgcn_sched_group_barrier(0x008, 1, 0),
+          (I * PER < NR ? __builtin_amdgcn_sched_group_barrier(0x100, (I + 1) * PER <= NR ? PER : NR - I * PER, 0)
+                        : (void)0)),
+         ...);
+      }(std::make_integer_sequence<int, NM>{});
       __builtin_amdgcn_sched_barrier(0);
     };
     auto phase = [&](auto S, int k, auto STEADY) {
@@ -830,6 +872,16 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
     for (; kt < nk; kt += NSTAGE) round(kt, std::false_type{});
   }
   const bool computes = wave < 4;
+  if (computes && p.a_rowsum != nullptr && tile_n == 0 && wn == 0) {
+    // lanes 0..31 and 32..63 hold the two k halves of the same 32 rows
+    T* dst = reinterpret_cast<T*>(p.a_rowsum) + grp * p.rowsum_sg;
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const float v = rsum[i] + __shfl_xor(rsum[i], 32, 64);
+      const int row = m0 + wm * WM + i * 32 + li;
+      if (g == 0 && row < p.m) dst[row] = from_f32<T>((p.flags & RTP_GEMM_ROWSUM_ACCUM) ? to_f32(dst[row]) + v : v);
+    }
+  }
 
   // Epilogue through LDS: the accumulators (fp32) are laid out as the BM x BN tile, then every thread of the
   // workgroup, loader waves included, finishes 8 consecutive columns of one row and writes them with 16-byte
@@ -948,6 +1000,31 @@ struct TileShape {
 static const TileShape kShapes[4] = {{256, 128, "256x128"}, {128, 128, "128x128"}, {128, 64, "128x64"}, {64, 64, "64x64"}};
 constexpr int kNumShapes = 4;
 
+// One wavefront per 32 x 32 block is the better kernel for one attention head at sequence length <= 64.
+static bool is_tiny(const rtp_gemm_desc* d) { return d->m <= 64 && d->n <= 64 && d->k * d->ksegs <= 256; }
+
+// Whether the wave-specialised kernel can run the problem.  Its branch-free loads need whole 16-byte vectors:
+// aligned operands and extents that are multiples of VEC along each operand's contiguous axis; and a tile's
+// byte offsets from its first vector must fit 32 bits (256 rows or k lines of one leading dimension).
+// Anything else goes to the guarded small-tile kernel.
+template <typename T>
+static bool takes_dma_kernel(const rtp_gemm_desc* d) {
+  constexpr int VEC = 16 / sizeof(T);
+  const bool vec_a = mult((int64_t)(uintptr_t)d->a, 16) && mult(d->lda, VEC) && mult(d->a_so, VEC) &&
+                     mult(d->a_si, VEC) && mult(d->a_sg, VEC) && mult(d->a_sk, VEC);
+  const bool vec_b = mult((int64_t)(uintptr_t)d->b, 16) && mult(d->ldb, VEC) && mult(d->b_so, VEC) &&
+                     mult(d->b_si, VEC) && mult(d->b_sg, VEC) && mult(d->b_sk, VEC);
+  const bool akc = d->a_kcontig, bkc = d->b_kcontig;
+  const int64_t ld_max = ((int64_t)1 << 24) / (int64_t)sizeof(T) - 64;
+  return vec_a && vec_b && ((akc || bkc) ? mult(d->k, VEC) : true) && (akc || mult(d->m, VEC)) &&
+         (bkc || mult(d->n, VEC)) && d->k > 0 && d->lda <= ld_max && d->ldb <= ld_max;
+}
+
+template <typename T>
+static bool rowsum_fused(const rtp_gemm_desc* d) {
+  return !d->a_kcontig && d->batch == 1 && !is_tiny(d) && takes_dma_kernel<T>(d);
+}
+
 template <typename T>
 static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   constexpr int VEC = 16 / sizeof(T);
@@ -992,15 +1069,14 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
               (!d->bias || (ok(d->bias, 8, d->bias_so, d->bias_si, d->bias_sg) && mult(d->bias_sk, 8)));
   }
 
-  // Branch-free loads need whole 16-byte vectors: aligned operands and extents that are multiples of VEC
-  // along each operand's contiguous axis.  Anything else goes to the guarded small-tile kernel.
   const bool akc = d->a_kcontig, bkc = d->b_kcontig;
-  // ... and a tile's byte offsets from its first vector must fit 32 bits (256 rows or k lines of one leading dimension)
-  const int64_t ld_max = ((int64_t)1 << 24) / (int64_t)sizeof(T) - 64;
-  const bool fast = a.vec_a && a.vec_b && ((akc || bkc) ? mult(d->k, VEC) : true) && (akc || mult(d->m, VEC)) &&
-                    (bkc || mult(d->n, VEC)) && d->k > 0 && d->lda <= ld_max && d->ldb <= ld_max;
+  const bool fast = takes_dma_kernel<T>(d);
   const int64_t nz = d->batch * d->groups;
-  if (d->m <= 64 && d->n <= 64 && d->k * d->ksegs <= 256) {
+  a.a_rowsum = (char*)d->a_rowsum;
+  a.rowsum_sg = d->rowsum_sg;
+  RTP_REQUIRE(!d->a_rowsum || rowsum_fused<T>(d),
+              "rtp_gemm: a_rowsum needs A stored K x M, batch == 1 and vector-aligned operands (rtp_gemm_rowsum_fused)");
+  if (is_tiny(d)) {
     // one wavefront per 32 x 32 block
     a.tiles_m = (int)ceil_div(d->m, 32);
     a.tiles_n = (int)ceil_div(d->n, 32);
@@ -1237,6 +1313,14 @@ extern "C" int rtp_gemm(void* stream, int dtype, const rtp_gemm_desc* d) {
   if (dtype == RTP_F32) return launch_gemm<float>(s, d);
   if (dtype == RTP_BF16) return launch_gemm<bf16_t>(s, d);
   return fail(RTP_ERR_ARG, "rtp_gemm: unknown dtype %d", dtype);
+}
+
+extern "C" int rtp_gemm_rowsum_fused(int dtype, const rtp_gemm_desc* d) {
+  using namespace rtp;
+  if (!d || !d->a || !d->b || d->m <= 0 || d->n <= 0 || d->k <= 0 || d->groups < 1 || d->ksegs < 1) return 0;
+  if (dtype == RTP_F32) return rowsum_fused<float>(d) ? 1 : 0;
+  if (dtype == RTP_BF16) return rowsum_fused<bf16_t>(d) ? 1 : 0;
+  return 0;
 }
 
 extern "C" size_t rtp_gemm_desc_size(void) { return sizeof(rtp_gemm_desc); }

@@ -232,11 +232,10 @@ class _AttentionFn(torch.autograd.Function):
 
         def param_grads():
             for first, cnt, accumulate in runs:
-                S.row_wgrad(dout2, o, store.grads, first, w_o_off, E, e_s, first * e_s, cnt, accumulate)
-                S.col_wgrad(dqkv, x2, store.grads, first, 0, 3 * e_s, E, first * 3 * e_s, cnt, accumulate)
-                if layer.has_bias:
-                    S.row_bgrad(dout2, store.grads, first, b_o_off, E, cnt, accumulate)
-                    S.col_bgrad(dqkv, store.grads, first, b_in_off, 3 * e_s, first * 3 * e_s, cnt, accumulate)
+                S.row_wgrad(dout2, o, store.grads, first, w_o_off, E, e_s, first * e_s, cnt, accumulate,
+                            b_off=b_o_off if layer.has_bias else None)
+                S.col_wgrad(dqkv, x2, store.grads, first, 0, 3 * e_s, E, first * 3 * e_s, cnt, accumulate,
+                            b_off=b_in_off if layer.has_bias else None)
             store.grads_ready()
 
         run_wgrad(dev, param_grads, (dout2, o, dqkv, x2))

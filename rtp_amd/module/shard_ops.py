@@ -46,8 +46,9 @@ def col_dgrad(dy2, flat, w_off, n_s, k, out, col0, c_in: Optional[torch.Tensor] 
                  b_sk=numel, **kw)
 
 
-def col_wgrad(dy2, x2, grads, first, w_off, n_s, k, col0, cnt, accumulate):
-    """grads[first+g, w_off : w_off + n_s*k] (+)= dy2[:, col0 + g*n_s : ...]^T @ x2, g < cnt."""
+def col_wgrad(dy2, x2, grads, first, w_off, n_s, k, col0, cnt, accumulate, b_off: Optional[int] = None):
+    """grads[first+g, w_off : w_off + n_s*k] (+)= dy2[:, col0 + g*n_s : ...]^T @ x2, g < cnt; with `b_off` also the
+    bias gradients grads[first+g, b_off : b_off + n_s] (+)= column sums of the same block of dy2."""
     numel = grads.shape[1]
     es = grads.element_size()
     m, _, lda = _rows(dy2)
@@ -59,10 +60,17 @@ def col_wgrad(dy2, x2, grads, first, w_off, n_s, k, col0, cnt, accumulate):
         ops.gemm_raw(grads.dtype, a=dy2.data_ptr() + col0 * es, b=x2.data_ptr(), c_out=c, m=cnt, n=k, k=m, lda=lda,
                      ldb=ldb, ldc=numel, a_kcontig=False, b_kcontig=False,
                      c_in=c if accumulate else None, ld_cin=numel, stream_out=True)
+        if b_off is not None:
+            col_bgrad(dy2, grads, first, b_off, n_s, col0, cnt, accumulate)
         return
-    ops.gemm_raw(grads.dtype, a=dy2.data_ptr() + col0 * es, b=x2.data_ptr(), c_out=c, m=n_s, n=k, k=m, lda=lda,
-                 ldb=ldb, ldc=k, a_kcontig=False, b_kcontig=False, groups=cnt, a_sg=n_s, c_sg=numel,
-                 c_in=c if accumulate else None, ld_cin=k, cin_sg=numel, stream_out=True)
+    # the bias gradient is the row sum of the product's first operand dy^T: the same launch adds it up
+    rs = None if b_off is None else grads.data_ptr() + (first * numel + b_off) * es
+    fused = ops.gemm_raw(grads.dtype, a=dy2.data_ptr() + col0 * es, b=x2.data_ptr(), c_out=c, m=n_s, n=k, k=m, lda=lda,
+                         ldb=ldb, ldc=k, a_kcontig=False, b_kcontig=False, groups=cnt, a_sg=n_s, c_sg=numel,
+                         c_in=c if accumulate else None, ld_cin=k, cin_sg=numel, stream_out=True,
+                         rowsum=rs, rowsum_sg=numel, rowsum_accum=accumulate)
+    if b_off is not None and not fused:
+        col_bgrad(dy2, grads, first, b_off, n_s, col0, cnt, accumulate)
 
 
 def col_bgrad(dy2, grads, first, b_off, n_s, col0, cnt, accumulate):
@@ -96,20 +104,26 @@ def row_dgrad(dy2, flat, w_off, n, k_s, out, col0):
                  c_sg=k_s)
 
 
-def row_wgrad(dy2, x2, grads, first, w_off, n, k_s, col0, cnt, accumulate):
-    """grads[first+g, w_off : w_off + n*k_s] (+)= dy2^T @ x2[:, col0 + g*k_s : ...]."""
+def row_wgrad(dy2, x2, grads, first, w_off, n, k_s, col0, cnt, accumulate, b_off: Optional[int] = None):
+    """grads[first+g, w_off : w_off + n*k_s] (+)= dy2^T @ x2[:, col0 + g*k_s : ...]; with `b_off` also the bias
+    gradients grads[first+g, b_off : b_off + n] (+)= column sums of dy2 (every shard of a row-style layer stores
+    bias/ws and receives the full sum, tests/test_linear.py:181-186)."""
     numel = grads.shape[1]
     es = grads.element_size()
     m, _, lda = _rows(dy2)
     _, _, ldb = _rows(x2)
     c = grads.data_ptr() + (first * numel + w_off) * es
-    ops.gemm_raw(grads.dtype, a=dy2.data_ptr(), b=x2.data_ptr() + col0 * es, c_out=c, m=n, n=k_s, k=m, lda=lda,
-                 ldb=ldb, ldc=k_s, a_kcontig=False, b_kcontig=False, groups=cnt, b_sg=k_s, c_sg=numel,
-                 c_in=c if accumulate else None, ld_cin=k_s, cin_sg=numel, stream_out=True)
+    rs = None if b_off is None else grads.data_ptr() + (first * numel + b_off) * es
+    fused = ops.gemm_raw(grads.dtype, a=dy2.data_ptr(), b=x2.data_ptr() + col0 * es, c_out=c, m=n, n=k_s, k=m, lda=lda,
+                         ldb=ldb, ldc=k_s, a_kcontig=False, b_kcontig=False, groups=cnt, b_sg=k_s, c_sg=numel,
+                         c_in=c if accumulate else None, ld_cin=k_s, cin_sg=numel, stream_out=True,
+                         rowsum=rs, rowsum_sg=numel, rowsum_accum=accumulate)
+    if b_off is not None and not fused:
+        row_bgrad(dy2, grads, first, b_off, n, cnt, accumulate)
 
 
 def row_bgrad(dy2, grads, first, b_off, n, cnt, accumulate):
-    """Every row-style shard stores bias/ws and receives the full column sum (tests/test_linear.py:181-186)."""
+    """grads[first+g, b_off : b_off + n] (+)= column sums of dy2 for every shard g of the run."""
     tmp = torch.empty(n, dtype=grads.dtype, device=grads.device)
     ops.colsum(dy2, tmp)
     dst = grads[first:first + cnt, b_off:b_off + n]

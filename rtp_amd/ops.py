@@ -8,7 +8,8 @@ from typing import Optional, Tuple
 import torch
 
 from . import _lib
-from ._lib import GEMM_CIN_F32, GEMM_OUT_F32, GEMM_RELU, GEMM_STREAM_OUT, RTP_BF16, RTP_F32, GemmDesc, check
+from ._lib import (GEMM_CIN_F32, GEMM_OUT_F32, GEMM_RELU, GEMM_ROWSUM_ACCUM, GEMM_STREAM_OUT, RTP_BF16, RTP_F32, GemmDesc,
+                   check)
 
 _DT = {torch.float32: RTP_F32, torch.bfloat16: RTP_BF16}
 
@@ -48,8 +49,13 @@ def gemm_raw(dtype: torch.dtype, *, a: int, b: int, c_out: int, m: int, n: int, 
              relu: bool = False, out_f32: bool = False, cin_f32: bool = False, batch: int = 1, zdiv: int = 1,
              a_s=(0, 0), b_s=(0, 0), c_s=(0, 0), cin_s=(0, 0), gate_s=(0, 0), bias_s=(0, 0), groups: int = 1,
              a_sg: int = 0, b_sg: int = 0, c_sg: int = 0, cin_sg: int = 0, gate_sg: int = 0, bias_sg: int = 0,
-             ksegs: int = 1, a_sk: int = 0, b_sk: int = 0, bias_sk: int = 0, stream_out: bool = False) -> None:
-    """One rtp_gemm call on raw device addresses (see include/rtp_hip.h for the operand rules)."""
+             ksegs: int = 1, a_sk: int = 0, b_sk: int = 0, bias_sk: int = 0, stream_out: bool = False,
+             rowsum: Optional[int] = None, rowsum_sg: int = 0, rowsum_accum: bool = False) -> bool:
+    """One rtp_gemm call on raw device addresses (see include/rtp_hip.h for the operand rules).
+
+    `rowsum` asks for the row sums of A (the bias gradient of a weight-gradient product) from the same launch.
+    Returns whether they were produced: False means the library cannot fuse them for these operands, the
+    product ran without them and the caller owes a separate column sum."""
     _lib.require_device()
     d = GemmDesc()
     d.a, d.b, d.c_out, d.c_in, d.bias, d.gate = a, b, c_out, c_in, bias, gate
@@ -67,9 +73,13 @@ def gemm_raw(dtype: torch.dtype, *, a: int, b: int, c_out: int, m: int, n: int, 
     d.a_sk, d.b_sk, d.bias_sk = a_sk, b_sk, bias_sk
     d.alpha = alpha
     d.flags = (GEMM_OUT_F32 if out_f32 else 0) | (GEMM_CIN_F32 if cin_f32 else 0) | (GEMM_RELU if relu else 0) | \
-        (GEMM_STREAM_OUT if stream_out else 0)
+        (GEMM_STREAM_OUT if stream_out else 0) | (GEMM_ROWSUM_ACCUM if rowsum_accum else 0)
     d.a_kcontig, d.b_kcontig = int(a_kcontig), int(b_kcontig)
-    check(_lib.load().rtp_gemm(_stream(), dtype_code(dtype), C.byref(d)))
+    lib = _lib.load()
+    fused = rowsum is not None and bool(lib.rtp_gemm_rowsum_fused(dtype_code(dtype), C.byref(d)))
+    d.a_rowsum, d.rowsum_sg = (rowsum, rowsum_sg) if fused else (None, 0)
+    check(lib.rtp_gemm(_stream(), dtype_code(dtype), C.byref(d)))
+    return fused
 
 
 def _epilogue_args(dtype, out, c_in, bias, gate):

@@ -188,3 +188,52 @@ def test_gemm_huge_leading_dimension_takes_guarded_kernel():
                  lda=lda, ldb=k, ldc=n, a_kcontig=True, b_kcontig=True)
     torch.cuda.synchronize()
     assert rel_err(out, a.double() @ b.double().t()) <= TOL[torch.bfloat16]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("accumulate", [False, True])
+@pytest.mark.parametrize("m,n,k,groups", [(256, 2048, 1024, 8), (72, 136, 200, 3), (768, 64, 520, 1), (8, 128, 72, 2)])
+def test_gemm_fused_row_sums_of_a(dtype, accumulate, m, n, k, groups):
+    """a_rowsum: the bias gradient of dW = dY^T X from the same launch, per group, against an fp64 column sum."""
+    ops = _ops()
+    gen = torch.Generator().manual_seed(m + n + k + groups)
+    dy = _rand((k, groups * m), dtype, gen)           # [tokens, out features of all groups]
+    x = _rand((k, n), dtype, gen)
+    numel = m * n + m + 8                             # flat gradient row: weight, bias, padding
+    grads = _rand((groups, numel), dtype, gen)
+    before = grads.clone()
+    dyd, xd, gd = dy.to(DEV), x.to(DEV), grads.to(DEV)
+    es = gd.element_size()
+    fused = ops.gemm_raw(dtype, a=dyd.data_ptr(), b=xd.data_ptr(), c_out=gd.data_ptr(), m=m, n=n, k=k,
+                         lda=groups * m, ldb=n, ldc=n, a_kcontig=False, b_kcontig=False, groups=groups, a_sg=m,
+                         c_sg=numel, c_in=gd.data_ptr() if accumulate else None, ld_cin=n, cin_sg=numel,
+                         rowsum=gd.data_ptr() + m * n * es, rowsum_sg=numel, rowsum_accum=accumulate)
+    torch.cuda.synchronize()
+    assert fused
+    got = gd.cpu()
+    for g in range(groups):
+        blk = dy[:, g * m:(g + 1) * m].double()
+        w_ref = blk.t() @ x.double()
+        b_ref = blk.sum(0)
+        if accumulate:
+            w_ref = w_ref + before[g, :m * n].double().view(m, n)
+            b_ref = b_ref + before[g, m * n:m * n + m].double()
+        assert rel_err(got[g, :m * n].view(m, n), w_ref) <= TOL[dtype]
+        assert rel_err(got[g, m * n:m * n + m], b_ref) <= TOL[dtype]
+        assert torch.equal(got[g, m * n + m:], before[g, m * n + m:])   # padding untouched
+
+
+def test_gemm_row_sums_fall_back_when_not_fusable():
+    """A K-contiguous A (or unaligned operands) cannot carry the row sums: gemm_raw says so and leaves them alone."""
+    ops = _ops()
+    gen = torch.Generator().manual_seed(9)
+    a = _rand((128, 256), torch.float32, gen).to(DEV)
+    b = _rand((64, 256), torch.float32, gen).to(DEV)
+    c = torch.empty(128, 64, device=DEV)
+    rs = torch.full((128,), 7.0, device=DEV)
+    fused = ops.gemm_raw(torch.float32, a=a.data_ptr(), b=b.data_ptr(), c_out=c.data_ptr(), m=128, n=64, k=256,
+                         lda=256, ldb=256, ldc=64, a_kcontig=True, b_kcontig=True, rowsum=rs.data_ptr())
+    torch.cuda.synchronize()
+    assert not fused
+    assert torch.equal(rs, torch.full((128,), 7.0, device=DEV))
+    assert rel_err(c, a.double() @ b.double().t()) <= TOL[torch.float32]
