@@ -23,6 +23,28 @@ namespace rtp {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
+// Division of a 32-bit unsigned number by a launch constant with a multiply-high and two shifts (Granlund and
+// Montgomery's round-up method, exact for every 32-bit dividend): integer division by a run-time value costs a
+// few dozen dependent instructions on this hardware, and the wave-specialised kernel would otherwise do ten of
+// them before it can issue its first load.
+struct FastDiv {
+  unsigned d, mul, s1, s2;
+};
+inline FastDiv make_fastdiv(unsigned d) {
+  FastDiv f;
+  f.d = d;
+  unsigned s = 0;
+  while ((1ull << s) < d) ++s;  // ceil(log2 d)
+  f.mul = (unsigned)((((1ull << s) - d) << 32) / d + 1);
+  f.s1 = s < 1 ? s : 1;
+  f.s2 = s < 1 ? 0 : s - 1;
+  return f;
+}
+__device__ __forceinline__ unsigned fast_div(unsigned n, const FastDiv& f) {
+  const unsigned t = __umulhi(n, f.mul);
+  return (t + ((n - t) >> f.s1)) >> f.s2;
+}
+
 struct GemmArgs {
   const char* a;
   const char* b;
@@ -44,6 +66,9 @@ struct GemmArgs {
   int xg, xm, xn;  // split of the (batch*groups, tiles_m, tiles_n) space over the 8 XCDs; xg == 0: none
   char* a_rowsum;  // bias gradient output (sum over k of A's rows), or null
   long rowsum_sg;
+  // wave-specialised kernel: tile mapping without run-time divisions
+  FastDiv d_batch, d_zdiv, d_tiles_n, d_nbk, d_mbk;  // nbk / mbk: tiles per XCD brick along n / m
+  int xn_shift, xm_shift, zbk;                       // log2 of xn and xm, batch*groups entries per brick
 };
 
 constexpr int kThreads = 256;
@@ -692,21 +717,22 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   // the operand rows one XCD touches are as few as possible; workgroup `id` works on brick id % 8.
   int tile_m, tile_n, z;
   if (p.xg) {
-    const int id = blockIdx.x + blockIdx.y * gridDim.x;
-    const int xcd = id & 7, slot = id >> 3;
-    const int nbk = p.tiles_n / p.xn, mbk = p.tiles_m / p.xm, zbk = (int)gridDim.y / p.xg;
-    tile_n = (xcd % p.xn) * nbk + slot % nbk;
-    tile_m = ((xcd / p.xn) % p.xm) * mbk + (slot / nbk) % mbk;
-    z = (xcd / (p.xn * p.xm)) * zbk + slot / (nbk * mbk);
+    const unsigned id = blockIdx.x + blockIdx.y * gridDim.x;
+    const unsigned xcd = id & 7, slot = id >> 3;
+    const unsigned sn = fast_div(slot, p.d_nbk);    // slot / nbk
+    const unsigned snm = fast_div(sn, p.d_mbk);     // slot / (nbk * mbk)
+    tile_n = (int)((xcd & ((1u << p.xn_shift) - 1)) * p.d_nbk.d + (slot - sn * p.d_nbk.d));
+    tile_m = (int)(((xcd >> p.xn_shift) & ((1u << p.xm_shift) - 1)) * p.d_mbk.d + (sn - snm * p.d_mbk.d));
+    z = (int)((xcd >> (p.xn_shift + p.xm_shift)) * p.zbk + snm);
   } else {
-    tile_m = blockIdx.x / p.tiles_n;
-    tile_n = blockIdx.x % p.tiles_n;
+    tile_m = (int)fast_div(blockIdx.x, p.d_tiles_n);
+    tile_n = (int)(blockIdx.x - tile_m * p.d_tiles_n.d);
     z = blockIdx.y;
   }
   const int m0 = tile_m * BM;
   const int n0 = tile_n * BN;
-  const int grp = z / p.batch, zb = z % p.batch;
-  const long zo = zb / p.zdiv, zi = zb % p.zdiv;
+  const int grp = (int)fast_div(z, p.d_batch), zb = z - grp * (int)p.d_batch.d;
+  const long zo = fast_div(zb, p.d_zdiv), zi = zb - (int)zo * (int)p.d_zdiv.d;
   const int nk_seg = (p.k + BK - 1) / BK;
   const int nk = nk_seg * p.ksegs;
 
@@ -1153,6 +1179,15 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
         }
       }
   }
+
+  a.d_batch = make_fastdiv((unsigned)d->batch);
+  a.d_zdiv = make_fastdiv((unsigned)d->zdiv);
+  a.d_tiles_n = make_fastdiv((unsigned)a.tiles_n);
+  a.d_nbk = make_fastdiv((unsigned)(a.xg ? a.tiles_n / a.xn : 1));
+  a.d_mbk = make_fastdiv((unsigned)(a.xg ? a.tiles_m / a.xm : 1));
+  a.xn_shift = a.xn == 8 ? 3 : a.xn == 4 ? 2 : a.xn == 2 ? 1 : 0;
+  a.xm_shift = a.xm == 8 ? 3 : a.xm == 4 ? 2 : a.xm == 2 ? 1 : 0;
+  a.zbk = a.xg ? (int)(nz / a.xg) : 0;
 
   // variant name = the kernel template instance, e.g. gemm_bf16_128x64_kc_kc
   static const char* const layout_tag[2][2] = {{"rc_rc", "rc_kc"}, {"kc_rc", "kc_kc"}};
