@@ -689,6 +689,18 @@ __device__ __forceinline__ Frag<T> read_frag_dma(const char* st, int rowbase, in
   return u.f;
 }
 
+// Reads one word of every 64-byte line of the kernel arguments (and of the launch dimensions behind them) in one
+// batch.  The scalar cache is cold at kernel start and the compiler fetches arguments where they are first used,
+// which would put one trip to memory in front of the tile mapping, one in front of the loaders' address set-up and
+// one in front of the epilogue; after this every later fetch hits the cache.
+__device__ __forceinline__ void touch_kernel_arguments() {
+  static_assert(sizeof(GemmArgs) <= 7 * 64, "seven lines cover the arguments");
+  typedef const __attribute__((address_space(4))) int* kernarg_t;
+  kernarg_t ka = (kernarg_t)__builtin_amdgcn_kernarg_segment_ptr();
+  const int w0 = ka[0], w1 = ka[16], w2 = ka[32], w3 = ka[48], w4 = ka[64], w5 = ka[80], w6 = ka[96];
+  asm volatile("" ::"s"(w0), "s"(w1), "s"(w2), "s"(w3), "s"(w4), "s"(w5), "s"(w6));
+}
+
 template <typename T, int BM, int BN, bool AKC, bool BKC, int NSTAGE, int SB, int PD>
 __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   constexpr int NL = 4;  // loader waves (waves 4..7); waves 0..3 compute
@@ -706,6 +718,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   // Stage addresses are compile-time offsets into one array, so LDS reads carry immediate offsets.
   __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE];
 
+  touch_kernel_arguments();
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -715,20 +728,20 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   // Workgroups are handed to the 8 XCDs round-robin in launch order, and every XCD has its own L2.  The
   // host splits the (batch*groups, tiles_m, tiles_n) space into 8 bricks (xg * xm * xn == 8) chosen so that
   // the operand rows one XCD touches are as few as possible; workgroup `id` works on brick id % 8.
-  int tile_m, tile_n, z;
-  if (p.xg) {
-    const unsigned id = blockIdx.x + blockIdx.y * gridDim.x;
-    const unsigned xcd = id & 7, slot = id >> 3;
-    const unsigned sn = fast_div(slot, p.d_nbk);    // slot / nbk
-    const unsigned snm = fast_div(sn, p.d_mbk);     // slot / (nbk * mbk)
-    tile_n = (int)((xcd & ((1u << p.xn_shift) - 1)) * p.d_nbk.d + (slot - sn * p.d_nbk.d));
-    tile_m = (int)(((xcd >> p.xn_shift) & ((1u << p.xm_shift) - 1)) * p.d_mbk.d + (sn - snm * p.d_mbk.d));
-    z = (int)((xcd >> (p.xn_shift + p.xm_shift)) * p.zbk + snm);
-  } else {
-    tile_m = (int)fast_div(blockIdx.x, p.d_tiles_n);
-    tile_n = (int)(blockIdx.x - tile_m * p.d_tiles_n.d);
-    z = blockIdx.y;
-  }
+  // Both mappings are computed and one is selected, without a branch: every kernel argument is then fetched by
+  // one batch of scalar loads at entry instead of three dependent rounds (each a trip to memory on a cold cache).
+  const unsigned id = blockIdx.x + blockIdx.y * gridDim.x;
+  const unsigned xcd = id & 7, slot = id >> 3;
+  const unsigned sn = fast_div(slot, p.d_nbk);  // slot / nbk
+  const unsigned snm = fast_div(sn, p.d_mbk);   // slot / (nbk * mbk)
+  const int tile_n_x = (int)((xcd & ((1u << p.xn_shift) - 1)) * p.d_nbk.d + (slot - sn * p.d_nbk.d));
+  const int tile_m_x = (int)(((xcd >> p.xn_shift) & ((1u << p.xm_shift) - 1)) * p.d_mbk.d + (sn - snm * p.d_mbk.d));
+  const int z_x = (int)((xcd >> (p.xn_shift + p.xm_shift)) * p.zbk + snm);
+  const int tile_m_p = (int)fast_div(blockIdx.x, p.d_tiles_n);
+  const int tile_n_p = (int)(blockIdx.x - tile_m_p * p.d_tiles_n.d);
+  const bool bricks = p.xg != 0;
+  const int tile_m = bricks ? tile_m_x : tile_m_p, tile_n = bricks ? tile_n_x : tile_n_p;
+  const int z = bricks ? z_x : (int)blockIdx.y;
   const int m0 = tile_m * BM;
   const int n0 = tile_n * BN;
   const int grp = (int)fast_div(z, p.d_batch), zb = z - grp * (int)p.d_batch.d;
