@@ -102,6 +102,7 @@ __device__ __forceinline__ Problem locate(const AttnArgs& a, int waves_per_block
 
 template <int DB, int NWV>
 __global__ __launch_bounds__(NWV * 64) void attn_fwd_small_kernel(AttnArgs a) {
+  touch_kernel_arguments<sizeof(AttnArgs)>();
   constexpr int D = 32 * DB, P = D + 8;
   __shared__ __attribute__((aligned(16))) bf16_t tiles[NWV][3][kSeqMax * P];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, li = lane & 31, g = lane >> 5;
@@ -174,6 +175,7 @@ __global__ __launch_bounds__(NWV * 64) void attn_fwd_small_kernel(AttnArgs a) {
 
 template <int DB, int NWV>
 __global__ __launch_bounds__(NWV * 64) void attn_bwd_small_kernel(AttnArgs a) {
+  touch_kernel_arguments<sizeof(AttnArgs)>();
   constexpr int D = 32 * DB, P = D + 8;
   __shared__ __attribute__((aligned(16))) bf16_t tiles[NWV][4][kSeqMax * P];
   __shared__ __attribute__((aligned(16))) bf16_t ptiles[NWV][2][kSeqMax * kPPitch];

@@ -689,18 +689,6 @@ __device__ __forceinline__ Frag<T> read_frag_dma(const char* st, int rowbase, in
   return u.f;
 }
 
-// Reads one word of every 64-byte line of the kernel arguments (and of the launch dimensions behind them) in one
-// batch.  The scalar cache is cold at kernel start and the compiler fetches arguments where they are first used,
-// which would put one trip to memory in front of the tile mapping, one in front of the loaders' address set-up and
-// one in front of the epilogue; after this every later fetch hits the cache.
-__device__ __forceinline__ void touch_kernel_arguments() {
-  static_assert(sizeof(GemmArgs) <= 7 * 64, "seven lines cover the arguments");
-  typedef const __attribute__((address_space(4))) int* kernarg_t;
-  kernarg_t ka = (kernarg_t)__builtin_amdgcn_kernarg_segment_ptr();
-  const int w0 = ka[0], w1 = ka[16], w2 = ka[32], w3 = ka[48], w4 = ka[64], w5 = ka[80], w6 = ka[96];
-  asm volatile("" ::"s"(w0), "s"(w1), "s"(w2), "s"(w3), "s"(w4), "s"(w5), "s"(w6));
-}
-
 template <typename T, int BM, int BN, bool AKC, bool BKC, int NSTAGE, int SB, int PD>
 __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   constexpr int NL = 4;  // loader waves (waves 4..7); waves 0..3 compute
@@ -718,7 +706,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   // Stage addresses are compile-time offsets into one array, so LDS reads carry immediate offsets.
   __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE];
 
-  touch_kernel_arguments();
+  touch_kernel_arguments<sizeof(GemmArgs)>();
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);

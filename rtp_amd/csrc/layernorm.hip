@@ -34,6 +34,7 @@ __global__ __launch_bounds__(kLnThreads) void add_layernorm_fwd_kernel(const T* 
                                                                        const T* beta, float eps, long rows, int cols,
                                                                        T* z_out, T* y, float* mean_out,
                                                                        float* rstd_out) {
+  touch_kernel_arguments<88>();
   constexpr int VEC = Vec16<T>::N;
   __shared__ float slots[2][4];
   const long row = blockIdx.x;
@@ -106,6 +107,7 @@ template <typename T, int NV>
 __global__ __launch_bounds__(kLnThreads) void layernorm_bwd_kernel(const T* dy, const T* z, const T* gamma,
                                                                    const float* mean, const float* rstd, long rows,
                                                                    int cols, T* dz, float* part) {
+  touch_kernel_arguments<72>();
   constexpr int VEC = Vec16<T>::N, RB = kLnBwdRows;
   __shared__ float slots[RB][2][4];
   const int nvec = cols / VEC;

@@ -67,6 +67,7 @@ template <typename T>
 __global__ __launch_bounds__(kXentThreads) void xent_bwd_kernel(const T* x, long ld, int cols, const long* target,
                                                                 const float2* stats, const float* dloss, long dloss_stride,
                                                                 T* dx, long ld_dx) {
+  touch_kernel_arguments<72>();
   constexpr int VEC = XVec<T>::N;
   const long row = blockIdx.x;
   const T* xr = x + row * ld;
