@@ -38,17 +38,33 @@ struct AttnArgs {
 constexpr int kSeqMax = 32;
 constexpr int kPPitch = kSeqMax + 8;  // row pitch of the P / dS tiles in LDS
 
-// 32 x D tile (rows beyond L zero) global -> LDS with 16-byte accesses, row pitch D + 8 elements.
-template <int D>
-__device__ __forceinline__ void load_tile(bf16_t* tile, const bf16_t* base, long s_l, int L, int lane) {
-  constexpr int CPR = D / 8;
-  for (int c = lane; c < kSeqMax * CPR; c += kWave) {
-    const int row = c / CPR, cc = c % CPR;
-    uint4 val = make_uint4(0u, 0u, 0u, 0u);
-    if (row < L) val = *reinterpret_cast<const uint4*>(base + row * s_l + cc * 8);
-    *reinterpret_cast<uint4*>(tile + row * (D + 8) + cc * 8) = val;
+// NT tiles of 32 x D (rows beyond L zero) global -> LDS with 16-byte accesses, row pitch D + 8 elements.  Every
+// load of every tile is issued before the first LDS write, and without branches (rows beyond L re-read row 0 and are
+// zeroed afterwards): a wave owns its problem alone, so a load that waits for the previous one to land puts a full
+// trip to memory on the kernel's critical path, and there would be a dozen of them.
+template <int D, int NT>
+struct TileRegs {
+  static constexpr int CPR = D / 8, NIT = kSeqMax * CPR / kWave;
+  uint4 val[NT][NIT];
+  __device__ __forceinline__ void fetch(const bf16_t* const (&base)[NT], const long (&s_l)[NT], int L, int lane) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) {
+        const int c = lane + it * kWave, row = c / CPR, cc = c % CPR;
+        val[t][it] = *reinterpret_cast<const uint4*>(base[t] + (row < L ? row : 0) * s_l[t] + cc * 8);
+      }
   }
-}
+  __device__ __forceinline__ void commit(bf16_t* const (&tile)[NT], int L, int lane) const {
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) {
+        const int c = lane + it * kWave, row = c / CPR, cc = c % CPR;
+        *reinterpret_cast<uint4*>(tile[t] + row * (D + 8) + cc * 8) = row < L ? val[t][it] : make_uint4(0u, 0u, 0u, 0u);
+      }
+  }
+};
 
 // Operand fragment with the contraction index contiguous in the tile: row li, elements 16*ks + 8*g ...
 __device__ __forceinline__ bf16x8 frag_rowmajor(const bf16_t* tile, int pitch, int li, int g, int ks) {
@@ -110,9 +126,41 @@ __global__ __launch_bounds__(NWV * 64) void attn_fwd_small_kernel(AttnArgs a) {
   bf16_t* Qs = tiles[wave][0];
   bf16_t* Ks = tiles[wave][1];
   bf16_t* Vs = tiles[wave][2];
-  load_tile<D>(Qs, a.q + pr.qkv_off, a.s_l, a.L, lane);
-  load_tile<D>(Ks, a.k + pr.qkv_off, a.s_l, a.L, lane);
-  load_tile<D>(Vs, a.v + pr.qkv_off, a.s_l, a.L, lane);
+  // Tiles first, then the additive mask values of this lane's 16 (query li, key) pairs; the mask is not looked at
+  // before the softmax, so its loads are in flight during the tile hand-over and the first product.
+  const bool qlive = li < a.L;
+  // keys come in runs of 4: with L % 4 == 0 whole runs are inside or outside the sequence (8-byte accesses to P)
+  const bool quads = a.L % 4 == 0 && reinterpret_cast<uintptr_t>(a.p) % 8 == 0;
+  TileRegs<D, 3> regs;
+  {
+    const bf16_t* const src[3] = {a.q + pr.qkv_off, a.k + pr.qkv_off, a.v + pr.qkv_off};
+    const long sl[3] = {a.s_l, a.s_l, a.s_l};
+    regs.fetch(src, sl, a.L, lane);
+  }
+  float mk[16];
+  const bool mask_quads = a.L % 4 == 0 && reinterpret_cast<uintptr_t>(a.mask) % 16 == 0;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) mk[r] = 0.0f;
+  if (a.mask) {
+    if (mask_quads) {
+#pragma unroll
+      for (int a4 = 0; a4 < 4; ++a4) {
+        const int key0 = 8 * a4 + 4 * g;
+        const float4 m4 = *reinterpret_cast<const float4*>(a.mask + ((qlive && key0 < a.L) ? li * a.L + key0 : 0));
+        mk[4 * a4 + 0] = m4.x, mk[4 * a4 + 1] = m4.y, mk[4 * a4 + 2] = m4.z, mk[4 * a4 + 3] = m4.w;
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = 8 * (r >> 2) + 4 * g + (r & 3);
+        mk[r] = a.mask[(qlive && key < a.L) ? li * a.L + key : 0];
+      }
+    }
+  }
+  {
+    bf16_t* const tl[3] = {Qs, Ks, Vs};
+    regs.commit(tl, a.L, lane);
+  }
   __syncthreads();
 
   // S^T[key][query]
@@ -125,15 +173,13 @@ __global__ __launch_bounds__(NWV * 64) void attn_fwd_small_kernel(AttnArgs a) {
                                                 0, 0);
 
   // softmax over the keys of query li
-  const bool qlive = li < a.L;
   float val[16];
   float mx = -INFINITY;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int key = 8 * (r >> 2) + 4 * g + (r & 3);
     const bool visible = key < a.L && (!a.causal || key <= li);
-    float x = s[r] * a.scale;
-    if (a.mask && qlive && key < a.L) x += a.mask[li * a.L + key];
+    const float x = s[r] * a.scale + ((qlive && key < a.L) ? mk[r] : 0.0f);  // outside: an unrelated mask entry
     val[r] = visible ? x : -INFINITY;
     mx = fmaxf(mx, val[r]);
   }
@@ -153,10 +199,23 @@ __global__ __launch_bounds__(NWV * 64) void attn_fwd_small_kernel(AttnArgs a) {
   for (int r = 0; r < 16; ++r) pb[r >> 3][r & 7] = from_f32<bf16_t>(val[r] * inv);
   if (pr.live && qlive) {
     bf16_t* prow = a.p + (pr.z * a.L + li) * a.L;
+    if (quads) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int key = 8 * (r >> 2) + 4 * g + (r & 3);
-      if (key < a.L) prow[key] = pb[r >> 3][r & 7];
+      for (int a4 = 0; a4 < 4; ++a4) {
+        union {
+          uint2 u;
+          bf16_t e[4];
+        } pk;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) pk.e[e] = pb[(4 * a4 + e) >> 3][(4 * a4 + e) & 7];
+        if (8 * a4 + 4 * g < a.L) *reinterpret_cast<uint2*>(prow + 8 * a4 + 4 * g) = pk.u;
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = 8 * (r >> 2) + 4 * g + (r & 3);
+        if (key < a.L) prow[key] = pb[r >> 3][r & 7];
+      }
     }
   }
 
@@ -187,10 +246,39 @@ __global__ __launch_bounds__(NWV * 64) void attn_bwd_small_kernel(AttnArgs a) {
   bf16_t* Gs = tiles[wave][3];  // dO
   bf16_t* DSs = ptiles[wave][0];
   bf16_t* Ps = ptiles[wave][1];
-  load_tile<D>(Qs, a.q + pr.qkv_off, a.s_l, a.L, lane);
-  load_tile<D>(Ks, a.k + pr.qkv_off, a.s_l, a.L, lane);
-  load_tile<D>(Vs, a.v + pr.qkv_off, a.s_l, a.L, lane);
-  load_tile<D>(Gs, a.dout + pr.o_off, a.o_l, a.L, lane);
+  // Tiles first, then this lane's 16 probabilities P[query li][key]: they are not needed before dP is there.
+  const bool qlive = li < a.L;
+  TileRegs<D, 4> regs;
+  {
+    const bf16_t* const src[4] = {a.q + pr.qkv_off, a.k + pr.qkv_off, a.v + pr.qkv_off, a.dout + pr.o_off};
+    const long sl[4] = {a.s_l, a.s_l, a.s_l, a.o_l};
+    regs.fetch(src, sl, a.L, lane);
+  }
+  const bf16_t* prow = a.p + (pr.z * a.L + (qlive ? li : 0)) * a.L;
+  // keys come in runs of 4: with L % 4 == 0 whole runs are inside or outside the sequence (8-byte accesses to P)
+  const bool quads = a.L % 4 == 0 && reinterpret_cast<uintptr_t>(a.p) % 8 == 0;
+  union {
+    uint2 u;
+    bf16_t e[4];
+  } p4[4];
+  bf16_t p1[16];
+  if (quads) {
+#pragma unroll
+    for (int a4 = 0; a4 < 4; ++a4) {
+      const int key0 = 8 * a4 + 4 * g;
+      p4[a4].u = *reinterpret_cast<const uint2*>(prow + ((qlive && key0 < a.L) ? key0 : 0));
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int key = 8 * (r >> 2) + 4 * g + (r & 3);
+      p1[r] = prow[(qlive && key < a.L) ? key : 0];
+    }
+  }
+  {
+    bf16_t* const tl[4] = {Qs, Ks, Vs, Gs};
+    regs.commit(tl, a.L, lane);
+  }
   __syncthreads();
 
   // dP^T[key][query] = sum_dd V[key][dd] dO[query][dd]
@@ -201,14 +289,13 @@ __global__ __launch_bounds__(NWV * 64) void attn_bwd_small_kernel(AttnArgs a) {
   for (int ks = 0; ks < D / 16; ++ks)
     dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rowmajor(Vs, P, li, g, ks), frag_rowmajor(Gs, P, li, g, ks), dp, 0,
                                                  0, 0);
-  const bool qlive = li < a.L;
-  const bf16_t* prow = a.p + (pr.z * a.L + (qlive ? li : 0)) * a.L;
   float pv[16];
   float dot = 0.0f;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int key = 8 * (r >> 2) + 4 * g + (r & 3);
-    pv[r] = (qlive && key < a.L) ? to_f32(prow[key]) : 0.0f;
+    const float pr_ = to_f32(quads ? p4[r >> 2].e[r & 3] : p1[r]);
+    pv[r] = (qlive && key < a.L) ? pr_ : 0.0f;
     dot += pv[r] * dp[r];
   }
   dot += __shfl_xor(dot, 32, kWave);
