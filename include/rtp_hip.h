@@ -266,7 +266,8 @@ int rtp_layernorm_bwd(void* stream, int dtype, const void* dy, const void* z, co
  *   bwd: dlogits[r, j] = (exp(logits[r, j] - m) / s - [j == target[r]]) * dloss[r * dloss_stride],
  *        dloss fp32 (dloss_stride 0: one scalar for all rows, 1: one value per row).
  * A row whose target lies outside [0, cols) has loss 0 and gradient 0 (an ignored row).
- * fp32 or bf16 logits, statistics in fp32; cols and both leading dimensions multiples of 16 bytes.
+ * fp32 or bf16 logits, statistics in fp32; cols and both leading dimensions multiples of 16 bytes, cols at
+ * most 8192 vectors of 16 bytes (65536 bf16 or 32768 fp32 classes: a row is held in registers).
  * dlogits may alias logits.
  * --------------------------------------------------------------------------------------------- */
 int rtp_softmax_xent_fwd(void* stream, int dtype, const void* logits, int64_t ld, int64_t rows, int64_t cols,

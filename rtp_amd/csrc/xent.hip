@@ -32,7 +32,10 @@ __device__ __forceinline__ float block_reduce(float v, float* slot, bool is_max)
   return is_max ? fmaxf(fmaxf(slot[0], slot[1]), fmaxf(slot[2], slot[3])) : (slot[0] + slot[1]) + (slot[2] + slot[3]);
 }
 
-template <typename T>
+// NV: 16-byte vectors per thread (the row has at most NV * 256 of them).  Every vector of the row is requested
+// before the first one is used and stays in registers for the second pass: a thread that loads in a loop waits out
+// one trip to memory per iteration, and the row would be read twice.
+template <typename T, int NV>
 __global__ __launch_bounds__(kXentThreads) void xent_fwd_kernel(const T* x, long ld, int cols, const long* target,
                                                                 float* loss, float2* stats) {
   constexpr int VEC = XVec<T>::N;
@@ -40,21 +43,27 @@ __global__ __launch_bounds__(kXentThreads) void xent_fwd_kernel(const T* x, long
   const long row = blockIdx.x;
   const T* xr = x + row * ld;
   const int nvec = cols / VEC;  // cols is a multiple of VEC
-  float mx = -INFINITY;
-  for (int c = threadIdx.x; c < nvec; c += kXentThreads) {
-    XVec<T> v;
-    v.q = reinterpret_cast<const uint4*>(xr)[c];
+  XVec<T> v[NV];
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) mx = fmaxf(mx, to_f32(v.e[e]));
+  for (int i = 0; i < NV; ++i) {
+    const int c = threadIdx.x + i * kXentThreads;
+    v[i].q = reinterpret_cast<const uint4*>(xr)[c < nvec ? c : 0];
   }
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < NV; ++i)
+    if (threadIdx.x + i * kXentThreads < nvec) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) mx = fmaxf(mx, to_f32(v[i].e[e]));
+    }
   mx = block_reduce(mx, slots[0], true);
   float sum = 0.0f;
-  for (int c = threadIdx.x; c < nvec; c += kXentThreads) {  // second pass: the row is L2 resident
-    XVec<T> v;
-    v.q = reinterpret_cast<const uint4*>(xr)[c];
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) sum += expf(to_f32(v.e[e]) - mx);
-  }
+  for (int i = 0; i < NV; ++i)
+    if (threadIdx.x + i * kXentThreads < nvec) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) sum += expf(to_f32(v[i].e[e]) - mx);
+    }
   sum = block_reduce(sum, slots[1], false);
   if (threadIdx.x == 0) {
     const long t = target[row];
@@ -63,7 +72,7 @@ __global__ __launch_bounds__(kXentThreads) void xent_fwd_kernel(const T* x, long
   }
 }
 
-template <typename T>
+template <typename T, int NV>
 __global__ __launch_bounds__(kXentThreads) void xent_bwd_kernel(const T* x, long ld, int cols, const long* target,
                                                                 const float2* stats, const float* dloss, long dloss_stride,
                                                                 T* dx, long ld_dx) {
@@ -72,23 +81,56 @@ __global__ __launch_bounds__(kXentThreads) void xent_bwd_kernel(const T* x, long
   const long row = blockIdx.x;
   const T* xr = x + row * ld;
   T* dr = dx + row * ld_dx;
+  const int nvec = cols / VEC;
+  XVec<T> v[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = threadIdx.x + i * kXentThreads;
+    v[i].q = reinterpret_cast<const uint4*>(xr)[c < nvec ? c : 0];
+  }
   const long t = target[row];
   const bool live = t >= 0 && t < cols;
   const float2 st = stats[row];
   const float mx = st.x, inv = 1.0f / st.y;
   const float s = live ? dloss[row * dloss_stride] : 0.0f;
-  const int nvec = cols / VEC;
-  for (int c = threadIdx.x; c < nvec; c += kXentThreads) {
-    XVec<T> v, o;
-    v.q = reinterpret_cast<const uint4*>(xr)[c];
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) {
-      float g = expf(to_f32(v.e[e]) - mx) * inv;
-      if ((long)c * VEC + e == t) g -= 1.0f;
-      o.e[e] = from_f32<T>(g * s);
+  for (int i = 0; i < NV; ++i) {
+    const int c = threadIdx.x + i * kXentThreads;
+    if (c < nvec) {
+      XVec<T> o;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        float g = expf(to_f32(v[i].e[e]) - mx) * inv;
+        if ((long)c * VEC + e == t) g -= 1.0f;
+        o.e[e] = from_f32<T>(g * s);
+      }
+      reinterpret_cast<uint4*>(dr)[c] = o.q;
     }
-    reinterpret_cast<uint4*>(dr)[c] = o.q;
   }
+}
+
+// The kernels are instantiated for 1, 2, 4, 8, 16 and 32 vectors per thread: rows of up to 65536 16-bit classes.
+constexpr int kXentMaxVectors = 32 * kXentThreads;
+
+template <typename T, typename... Args>
+static void launch_xent_fwd(int nv, dim3 grid, hipStream_t st, Args... args) {
+  const dim3 block(kXentThreads);
+  if (nv <= 1) hipLaunchKernelGGL((xent_fwd_kernel<T, 1>), grid, block, 0, st, args...);
+  else if (nv <= 2) hipLaunchKernelGGL((xent_fwd_kernel<T, 2>), grid, block, 0, st, args...);
+  else if (nv <= 4) hipLaunchKernelGGL((xent_fwd_kernel<T, 4>), grid, block, 0, st, args...);
+  else if (nv <= 8) hipLaunchKernelGGL((xent_fwd_kernel<T, 8>), grid, block, 0, st, args...);
+  else if (nv <= 16) hipLaunchKernelGGL((xent_fwd_kernel<T, 16>), grid, block, 0, st, args...);
+  else hipLaunchKernelGGL((xent_fwd_kernel<T, 32>), grid, block, 0, st, args...);
+}
+template <typename T, typename... Args>
+static void launch_xent_bwd(int nv, dim3 grid, hipStream_t st, Args... args) {
+  const dim3 block(kXentThreads);
+  if (nv <= 1) hipLaunchKernelGGL((xent_bwd_kernel<T, 1>), grid, block, 0, st, args...);
+  else if (nv <= 2) hipLaunchKernelGGL((xent_bwd_kernel<T, 2>), grid, block, 0, st, args...);
+  else if (nv <= 4) hipLaunchKernelGGL((xent_bwd_kernel<T, 4>), grid, block, 0, st, args...);
+  else if (nv <= 8) hipLaunchKernelGGL((xent_bwd_kernel<T, 8>), grid, block, 0, st, args...);
+  else if (nv <= 16) hipLaunchKernelGGL((xent_bwd_kernel<T, 16>), grid, block, 0, st, args...);
+  else hipLaunchKernelGGL((xent_bwd_kernel<T, 32>), grid, block, 0, st, args...);
 }
 
 }  // namespace rtp
@@ -98,10 +140,11 @@ using namespace rtp;
 static int xent_check(const char* who, int dtype, int64_t ld, int64_t rows, int64_t cols, const void* x) {
   RTP_REQUIRE(dtype == RTP_F32 || dtype == RTP_BF16, "%s: unknown dtype %d", who, dtype);
   const int vec = dtype == RTP_F32 ? 4 : 8;
-  RTP_REQUIRE(rows >= 0 && rows < (1ll << 31) && cols >= vec && cols < (1ll << 31) && cols % vec == 0 && ld >= cols &&
-                  ld % vec == 0 && (uintptr_t)x % 16 == 0,
-              "%s: need rows < 2^31, cols a multiple of %d, ld >= cols and a multiple of %d, 16-byte aligned logits", who,
-              vec, vec);
+  RTP_REQUIRE(rows >= 0 && rows < (1ll << 31) && cols >= vec && cols <= (int64_t)kXentMaxVectors * vec &&
+                  cols % vec == 0 && ld >= cols && ld % vec == 0 && (uintptr_t)x % 16 == 0,
+              "%s: need rows < 2^31, cols a multiple of %d and at most %d, ld >= cols and a multiple of %d, 16-byte "
+              "aligned logits",
+              who, vec, kXentMaxVectors * vec, vec);
   return RTP_OK;
 }
 
@@ -113,12 +156,13 @@ extern "C" int rtp_softmax_xent_fwd(void* stream, int dtype, const void* logits,
   if (rows == 0) return RTP_OK;
   hipStream_t st = (hipStream_t)stream;
   ProfileScope prof(st, "softmax_xent_fwd", 0.0, (double)rows * cols * (dtype == RTP_F32 ? 4.0 : 2.0));
+  const int nv = (int)ceil_div(cols / (dtype == RTP_F32 ? 4 : 8), kXentThreads);
   if (dtype == RTP_F32)
-    hipLaunchKernelGGL(xent_fwd_kernel<float>, dim3((unsigned)rows), dim3(kXentThreads), 0, st, (const float*)logits,
-                       (long)ld, (int)cols, (const long*)target, loss, (float2*)stats);
+    launch_xent_fwd<float>(nv, dim3((unsigned)rows), st, (const float*)logits, (long)ld, (int)cols, (const long*)target, loss,
+                           (float2*)stats);
   else
-    hipLaunchKernelGGL(xent_fwd_kernel<bf16_t>, dim3((unsigned)rows), dim3(kXentThreads), 0, st, (const bf16_t*)logits,
-                       (long)ld, (int)cols, (const long*)target, loss, (float2*)stats);
+    launch_xent_fwd<bf16_t>(nv, dim3((unsigned)rows), st, (const bf16_t*)logits, (long)ld, (int)cols, (const long*)target,
+                            loss, (float2*)stats);
   RTP_LAUNCH_CHECK();
   return RTP_OK;
 }
@@ -134,14 +178,13 @@ extern "C" int rtp_softmax_xent_bwd(void* stream, int dtype, const void* logits,
   if (rows == 0) return RTP_OK;
   hipStream_t st = (hipStream_t)stream;
   ProfileScope prof(st, "softmax_xent_bwd", 0.0, 2.0 * (double)rows * cols * (dtype == RTP_F32 ? 4.0 : 2.0));
+  const int nv = (int)ceil_div(cols / (dtype == RTP_F32 ? 4 : 8), kXentThreads);
   if (dtype == RTP_F32)
-    hipLaunchKernelGGL(xent_bwd_kernel<float>, dim3((unsigned)rows), dim3(kXentThreads), 0, st, (const float*)logits,
-                       (long)ld, (int)cols, (const long*)target, (const float2*)stats, dloss, (long)dloss_stride,
-                       (float*)dlogits, (long)ld_dlogits);
+    launch_xent_bwd<float>(nv, dim3((unsigned)rows), st, (const float*)logits, (long)ld, (int)cols, (const long*)target,
+                           (const float2*)stats, dloss, (long)dloss_stride, (float*)dlogits, (long)ld_dlogits);
   else
-    hipLaunchKernelGGL(xent_bwd_kernel<bf16_t>, dim3((unsigned)rows), dim3(kXentThreads), 0, st, (const bf16_t*)logits,
-                       (long)ld, (int)cols, (const long*)target, (const float2*)stats, dloss, (long)dloss_stride,
-                       (bf16_t*)dlogits, (long)ld_dlogits);
+    launch_xent_bwd<bf16_t>(nv, dim3((unsigned)rows), st, (const bf16_t*)logits, (long)ld, (int)cols, (const long*)target,
+                            (const float2*)stats, dloss, (long)dloss_stride, (bf16_t*)dlogits, (long)ld_dlogits);
   RTP_LAUNCH_CHECK();
   return RTP_OK;
 }

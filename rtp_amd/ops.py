@@ -365,7 +365,8 @@ def softmax_xent_supported(logits: torch.Tensor) -> bool:
     if logits.dtype not in (torch.float32, torch.bfloat16) or logits.dim() != 2 or not logits.is_cuda:
         return False
     vec = 16 // logits.element_size()
-    return bool(logits.stride(1) == 1 and logits.shape[1] >= vec and logits.shape[1] % vec == 0
+    # a row is held in registers: at most 32 vectors of 16 bytes per thread of a 256-thread workgroup
+    return bool(logits.stride(1) == 1 and vec <= logits.shape[1] <= 32 * 256 * vec and logits.shape[1] % vec == 0
                 and logits.stride(0) >= logits.shape[1] and logits.stride(0) % vec == 0
                 and logits.data_ptr() % 16 == 0)
 
