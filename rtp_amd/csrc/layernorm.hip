@@ -112,30 +112,40 @@ __global__ __launch_bounds__(kLnThreads) void layernorm_bwd_kernel(const T* dy, 
   __shared__ float slots[RB][2][4];
   const int nvec = cols / VEC;
   const long row0 = (long)blockIdx.x * RB;
-  // every load of the block is issued before the first reduction
+  // Every load of the block is issued before the first reduction, and without branches (rows and vectors outside
+  // re-read the block's first ones and are zeroed afterwards): a conditional load is a branch, and the compiler
+  // waits for the loads of one row before it issues the next row's.
   Vec16<T> ra[RB][NV], rb[RB][NV], gm[NV];
   float mu[RB], rs[RB];
 #pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = threadIdx.x + i * kLnThreads;
+    gm[i].q = reinterpret_cast<const uint4*>(gamma)[c < nvec ? c : 0];  // vectors outside meet zeroed dy / z only
+  }
+#pragma unroll
   for (int rr = 0; rr < RB; ++rr) {
     const bool live = row0 + rr < rows;
-    mu[rr] = live ? mean[row0 + rr] : 0.0f;
-    rs[rr] = live ? rstd[row0 + rr] : 0.0f;
+    const long r = live ? row0 + rr : row0;
+    mu[rr] = mean[r];
+    rs[rr] = rstd[r];
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int c = threadIdx.x + i * kLnThreads;
-      ra[rr][i].q = make_uint4(0u, 0u, 0u, 0u);
-      rb[rr][i].q = make_uint4(0u, 0u, 0u, 0u);
-      if (live && c < nvec) {
-        ra[rr][i].q = reinterpret_cast<const uint4*>(dy + (row0 + rr) * cols)[c];
-        rb[rr][i].q = reinterpret_cast<const uint4*>(z + (row0 + rr) * cols)[c];
-      }
+      const int cc = c < nvec ? c : 0;
+      ra[rr][i].q = reinterpret_cast<const uint4*>(dy + r * cols)[cc];
+      rb[rr][i].q = reinterpret_cast<const uint4*>(z + r * cols)[cc];
     }
   }
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int c = threadIdx.x + i * kLnThreads;
-    gm[i].q = make_uint4(0u, 0u, 0u, 0u);
-    if (c < nvec) gm[i].q = reinterpret_cast<const uint4*>(gamma)[c];
+  for (int rr = 0; rr < RB; ++rr) {
+    const bool live = row0 + rr < rows;
+    if (!live) mu[rr] = rs[rr] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+      if (!live || threadIdx.x + i * kLnThreads >= nvec) {
+        ra[rr][i].q = make_uint4(0u, 0u, 0u, 0u);
+        rb[rr][i].q = make_uint4(0u, 0u, 0u, 0u);
+      }
   }
   float dg[NV][VEC], db[NV][VEC];
 #pragma unroll
@@ -201,8 +211,8 @@ __global__ __launch_bounds__(kLnThreads) void layernorm_bwd_kernel(const T* dy, 
   }
 }
 
-// 32 columns of the [2][cols] sums per workgroup: 8 groups of threads each add an eighth of the blocks (in
-// order, four loads in flight), then the eighths are added in order.
+// 32 columns of the [2][cols] sums per workgroup: 8 groups of threads each add an eighth of the blocks (a fixed
+// order, sixteen loads in flight), then the eighths are added in order.
 template <typename T>
 __global__ __launch_bounds__(256) void layernorm_bwd_final_kernel(const float* part, long nblocks, int cols, T* dgamma,
                                                                   T* dbeta) {
@@ -211,18 +221,22 @@ __global__ __launch_bounds__(256) void layernorm_bwd_final_kernel(const float* p
   const int c = blockIdx.x * 32 + cl;  // column of the [2 * cols] row
   const long per = (nblocks + 7) / 8;
   const long b0 = grp * per, b1 = b0 + per < nblocks ? b0 + per : nblocks;
-  float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+  float acc[16];
+#pragma unroll
+  for (int j = 0; j < 16; ++j) acc[j] = 0.0f;
   if (c < 2 * cols) {
     long b = b0;
-    for (; b + 3 < b1; b += 4) {
-      s0 += part[b * 2 * cols + c];
-      s1 += part[(b + 1) * 2 * cols + c];
-      s2 += part[(b + 2) * 2 * cols + c];
-      s3 += part[(b + 3) * 2 * cols + c];
+    for (; b + 15 < b1; b += 16) {
+#pragma unroll
+      for (int j = 0; j < 16; ++j) acc[j] += part[(b + j) * 2 * cols + c];
     }
-    for (; b < b1; ++b) s0 += part[b * 2 * cols + c];
+    for (; b < b1; ++b) acc[0] += part[b * 2 * cols + c];
   }
-  eighth[grp][cl] = (s0 + s1) + (s2 + s3);
+#pragma unroll
+  for (int w = 8; w >= 1; w >>= 1)
+#pragma unroll
+    for (int j = 0; j < w; ++j) acc[j] += acc[j + w];
+  eighth[grp][cl] = acc[0];
   __syncthreads();
   if (grp == 0 && c < 2 * cols) {
     float s = 0.0f;
