@@ -12,6 +12,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void gather_kernel(const T* table, long ld_table, long row_begin, long row_count,
                                                      long cols, const int64_t* ids, T* out, long ld_out, int vec,
                                                      long table_sg, long out_sg) {
+  touch_kernel_arguments<104>();
   const long t = blockIdx.x;
   const long row = ids[t] - row_begin;
   if (row < 0 || row >= row_count) return;
@@ -58,6 +59,7 @@ __global__ __launch_bounds__(256) void scatter_kernel(const T* grad_out, long ld
                                                       const int* vals, G* grad_table, long ld_gt, long row_begin,
                                                       long row_count, long cols, long padding_idx, int scale_by_freq,
                                                       int overwrite, long go_sg, long gt_sg) {
+  touch_kernel_arguments<120>();
   grad_out += blockIdx.z * go_sg;  // group = shard: its column block of the upstream gradient, its own table
   grad_table += blockIdx.z * gt_sg;
   const long i = blockIdx.x;
@@ -180,9 +182,17 @@ extern "C" int rtp_embedding_scatter_add_det(void* stream, int dtype, const void
   if (zero_fill) {
     RTP_REQUIRE(row_count < (1ll << 31), "rtp_embedding_scatter_add_det: too many rows");
     ProfileScope prof(s, "embedding_grad_zero_fill", 0.0, (double)groups * row_count * cols * gsz);
-    hipLaunchKernelGGL(zero_rows_kernel, dim3((unsigned)row_count, chunks, (unsigned)groups), dim3(256), 0, s,
-                       (char*)grad_table, (long)(ld_grad_table * gsz), (long)(cols * gsz), (long)row_count,
-                       (long)(grad_table_sg * gsz));
+    if (ld_grad_table == cols) {
+      // a group's table is one contiguous block: fill it as such (a workgroup per 512-byte row slice is mostly idle)
+      const int64_t bytes = row_count * cols * gsz;
+      const unsigned wgs = (unsigned)std::min<int64_t>(2048, std::max<int64_t>(1, ceil_div(bytes, 16384)));
+      hipLaunchKernelGGL(zero_rows_kernel, dim3(1, wgs, (unsigned)groups), dim3(256), 0, s, (char*)grad_table,
+                         (long)bytes, (long)bytes, 1l, (long)(grad_table_sg * gsz));
+    } else {
+      hipLaunchKernelGGL(zero_rows_kernel, dim3((unsigned)row_count, chunks, (unsigned)groups), dim3(256), 0, s,
+                         (char*)grad_table, (long)(ld_grad_table * gsz), (long)(cols * gsz), (long)row_count,
+                         (long)(grad_table_sg * gsz));
+    }
     RTP_LAUNCH_CHECK();
   }
   if (n_ids == 0) return RTP_OK;
