@@ -12,7 +12,6 @@ template <typename T>
 __global__ __launch_bounds__(256) void gather_kernel(const T* table, long ld_table, long row_begin, long row_count,
                                                      long cols, const int64_t* ids, T* out, long ld_out, int vec,
                                                      long table_sg, long out_sg) {
-  touch_kernel_arguments<104>();
   const long t = blockIdx.x;
   const long row = ids[t] - row_begin;
   if (row < 0 || row >= row_count) return;
@@ -59,7 +58,6 @@ __global__ __launch_bounds__(256) void scatter_kernel(const T* grad_out, long ld
                                                       const int* vals, G* grad_table, long ld_gt, long row_begin,
                                                       long row_count, long cols, long padding_idx, int scale_by_freq,
                                                       int overwrite, long go_sg, long gt_sg) {
-  touch_kernel_arguments<120>();
   grad_out += blockIdx.z * go_sg;  // group = shard: its column block of the upstream gradient, its own table
   grad_table += blockIdx.z * gt_sg;
   const long i = blockIdx.x;
