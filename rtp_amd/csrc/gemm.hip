@@ -590,6 +590,7 @@ struct DmaOperand {
   static constexpr int NI = R * SB / 1024 / NL;   // load instructions (1 KiB each) per loader wave and slab
   static constexpr int BYTES = R * SB;            // one stage of this operand
   static constexpr int LINE = R * (int)sizeof(T); // bytes of one k line when rows are contiguous
+  static_assert(KC || 1024 % LINE == 0 || LINE % 1024 == 0, "a 1 KiB load covers whole k lines or a whole fraction of one");
   // The lane's vector sits at `ofs` bytes from the slab's base pointer, which is the same for every lane and lives
   // in scalar registers: the loader's steady state then has no vector-ALU instruction at all.  (A vector add per
   // load has to compete for issue slots with the MFMAs of the compute wave on the same SIMD, and loses: measured,
@@ -932,7 +933,20 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
 template <typename T, int BM, int BN, int NSTAGE, int SB, int PD>
 static int launch_dma(hipStream_t s, const GemmArgs& a, bool akc, bool bkc, dim3 grid) {
   const dim3 block(512);
-  if (akc && bkc)
+  // A row-contiguous operand is staged as k lines of R elements, and a 1 KiB load must cover whole lines (or a
+  // whole fraction of one): tile extents that are not powers of two only exist for K-contiguous operands.
+  constexpr bool A_RC_OK = (BM & (BM - 1)) == 0, B_RC_OK = (BN & (BN - 1)) == 0;
+  if constexpr (!A_RC_OK || !B_RC_OK) {
+    RTP_REQUIRE((akc || A_RC_OK) && (bkc || B_RC_OK), "gemm: tile %d x %d needs K-contiguous operands", BM, BN);
+    if constexpr (!B_RC_OK && A_RC_OK) {
+      if (akc)
+        hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, true, NSTAGE, SB, PD>), grid, block, 0, s, a);
+      else
+        hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, true, NSTAGE, SB, PD>), grid, block, 0, s, a);
+    }
+    RTP_LAUNCH_CHECK();
+    return RTP_OK;
+  } else if (akc && bkc)
     hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, true, NSTAGE, SB, PD>), grid, block, 0, s, a);
   else if (akc && !bkc)
     hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, false, NSTAGE, SB, PD>), grid, block, 0, s, a);
@@ -1024,8 +1038,9 @@ struct TileShape {
   int bm, bn;
   const char* tag;
 };
-static const TileShape kShapes[4] = {{256, 128, "256x128"}, {128, 128, "128x128"}, {128, 64, "128x64"}, {64, 64, "64x64"}};
-constexpr int kNumShapes = 4;
+static const TileShape kShapes[5] = {{256, 128, "256x128"}, {128, 128, "128x128"}, {128, 64, "128x64"}, {64, 64, "64x64"},
+                                     {128, 192, "128x192"}};
+constexpr int kNumShapes = 5;
 
 // One wavefront per 32 x 32 block is the better kernel for one attention head at sequence length <= 64.
 static bool is_tiny(const rtp_gemm_desc* d) { return d->m <= 64 && d->n <= 64 && d->k * d->ksegs <= 256; }
@@ -1134,12 +1149,13 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
     const char* e = getenv("RTP_GEMM_TILE");  // debugging aid: index into kShapes
     return e ? atoi(e) : -1;
   }();
-  static const double slab_ns[kNumShapes] = {966.0, 470.0, 283.0, 167.0};
-  static const int slab_bytes[kNumShapes] = {128, 128, 128, 128};
-  int shape = kNumShapes - 1;
+  static const double slab_ns[kNumShapes] = {966.0, 470.0, 283.0, 167.0, 720.0};
+  static const int slab_bytes[kNumShapes] = {128, 128, 128, 128, 128};
+  int shape = 3;  // 64 x 64 unless the model finds something cheaper
   double best = 0.0;
   for (int i = 0; fast && i < kNumShapes; ++i) {
     // never a tile that is mostly padding: a 32 x 32 problem (one attention head at seq 32) stays at 64 x 64
+    if ((!akc && (kShapes[i].bm & (kShapes[i].bm - 1))) || (!bkc && (kShapes[i].bn & (kShapes[i].bn - 1)))) continue;
     if (kShapes[i].bm > 64 && kShapes[i].bm > ceil_div(d->m, 64) * 64) continue;
     if (kShapes[i].bn > 64 && kShapes[i].bn > ceil_div(d->n, 64) * 64) continue;
     const int64_t tiles = ceil_div(d->m, kShapes[i].bm) * ceil_div(d->n, kShapes[i].bn) * nz;
@@ -1211,6 +1227,8 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
       return launch_dma<T, 128, 128, 4, 128, 3>(s, a, akc, bkc, grid);
     case 2:
       return launch_dma<T, 128, 64, 5, 128, 4>(s, a, akc, bkc, grid);
+    case 4:
+      return launch_dma<T, 128, 192, 3, 128, 2>(s, a, akc, bkc, grid);
     default:
       return launch_dma<T, 64, 64, 4, 128, 3>(s, a, akc, bkc, grid);
   }

@@ -237,3 +237,24 @@ def test_gemm_row_sums_fall_back_when_not_fusable():
     assert not fused
     assert torch.equal(rs, torch.full((128,), 7.0, device=DEV))
     assert rel_err(c, a.double() @ b.double().t()) <= TOL[torch.float32]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("akc", [True, False])
+@pytest.mark.parametrize("m,n,k", [(1024, 6144, 256), (1000, 6000, 136)])
+def test_gemm_wide_tile_shapes(dtype, akc, m, n, k):
+    """Problems whose tile count fills the 256 CUs exactly with 128 x 192 tiles (the packed q/k/v projection of the
+    LM: 1024 x 6144), ragged in every extent in the second case; B must be K-contiguous for that shape."""
+    ops = _ops()
+    gen = torch.Generator().manual_seed(m + n + k)
+    a = _rand((m, k) if akc else (k, m), dtype, gen)
+    b = _rand((n, k), dtype, gen)
+    bias = _rand((n,), dtype, gen)
+    A = a.double() if akc else a.double().t()
+    ref = A @ b.double().t() + bias.double()
+    ad, bd, biasd = a.to(DEV), b.to(DEV), bias.to(DEV)
+    out = torch.full((m, n), float("nan"), dtype=dtype, device=DEV)
+    ops.gemm_raw(dtype, a=ad.data_ptr(), b=bd.data_ptr(), c_out=out.data_ptr(), m=m, n=n, k=k, lda=ad.stride(0),
+                 ldb=k, ldc=n, a_kcontig=akc, b_kcontig=True, bias=biasd.data_ptr())
+    torch.cuda.synchronize()
+    assert rel_err(out, ref) <= TOL[dtype]
