@@ -132,19 +132,26 @@ class _ExpertsFn(torch.autograd.Function):
                 r0 = (first * n_local + le) * c_rows
                 base = g.data_ptr() + first * store.numel * es
                 common = dict(groups=cnt, c_sg=store.numel, cin_sg=store.numel, a_kcontig=False, b_kcontig=False)
-                # dW2 = dY^T H ; dW1 = dH^T X  (contraction over the expert's capacity rows)
+                # dW2 = dY^T H ; dW1 = dH^T X  (contraction over the expert's capacity rows); the bias gradients are
+                # the row sums of the first operands and come out of the same launches where the library can fuse them
                 c2 = base + w2 * es
-                ops.gemm_raw(x.dtype, a=dy.data_ptr() + r0 * m_dim * es, b=h.data_ptr() + r0 * f_dim * es, c_out=c2,
-                             c_in=c2 if accumulate else None, ld_cin=f_dim, m=m_dim, n=f_dim, k=c_rows, lda=m_dim,
-                             ldb=f_dim, ldc=f_dim, a_sg=n_local * c_rows * m_dim, b_sg=n_local * c_rows * f_dim, **common)
+                fused2 = ops.gemm_raw(
+                    x.dtype, a=dy.data_ptr() + r0 * m_dim * es, b=h.data_ptr() + r0 * f_dim * es, c_out=c2,
+                    c_in=c2 if accumulate else None, ld_cin=f_dim, m=m_dim, n=f_dim, k=c_rows, lda=m_dim, ldb=f_dim,
+                    ldc=f_dim, a_sg=n_local * c_rows * m_dim, b_sg=n_local * c_rows * f_dim, rowsum=base + b2 * es,
+                    rowsum_sg=store.numel, rowsum_accum=accumulate, **common)
                 c1 = base + w1 * es
-                ops.gemm_raw(x.dtype, a=dh.data_ptr() + r0 * f_dim * es, b=x.data_ptr() + r0 * m_dim * es, c_out=c1,
-                             c_in=c1 if accumulate else None, ld_cin=m_dim, m=f_dim, n=m_dim, k=c_rows, lda=f_dim,
-                             ldb=m_dim, ldc=m_dim, a_sg=n_local * c_rows * f_dim, b_sg=n_local * c_rows * m_dim, **common)
-                for s in range(first, first + cnt):  # bias gradients: column sums over each expert's own rows
+                fused1 = ops.gemm_raw(
+                    x.dtype, a=dh.data_ptr() + r0 * f_dim * es, b=x.data_ptr() + r0 * m_dim * es, c_out=c1,
+                    c_in=c1 if accumulate else None, ld_cin=m_dim, m=f_dim, n=m_dim, k=c_rows, lda=f_dim, ldb=m_dim,
+                    ldc=m_dim, a_sg=n_local * c_rows * f_dim, b_sg=n_local * c_rows * m_dim, rowsum=base + b1 * es,
+                    rowsum_sg=store.numel, rowsum_accum=accumulate, **common)
+                for s in range(first, first + cnt):  # otherwise: column sums over each expert's own rows
                     r = (s * n_local + le) * c_rows
-                    ops.colsum(dy[r:r + c_rows], g[s, b2:b2 + m_dim], accumulate=accumulate)
-                    ops.colsum(dh[r:r + c_rows], g[s, b1:b1 + f_dim], accumulate=accumulate)
+                    if not fused2:
+                        ops.colsum(dy[r:r + c_rows], g[s, b2:b2 + m_dim], accumulate=accumulate)
+                    if not fused1:
+                        ops.colsum(dh[r:r + c_rows], g[s, b1:b1 + f_dim], accumulate=accumulate)
         store.grads_ready()
         return dx, None, None
 
