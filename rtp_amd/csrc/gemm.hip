@@ -67,8 +67,11 @@ struct GemmArgs {
   char* a_rowsum;  // bias gradient output (sum over k of A's rows), or null
   long rowsum_sg;
   // wave-specialised kernel: tile mapping without run-time divisions
-  FastDiv d_batch, d_zdiv, d_tiles_n, d_nbk, d_mbk;  // nbk / mbk: tiles per XCD brick along n / m
-  int xn_shift, xm_shift, zbk;                       // log2 of xn and xm, batch*groups entries per brick
+  // A brick is mbk x nbk tiles; its tiles are handed out panel by panel, a panel being all mbk tile rows of `panel`
+  // consecutive tile columns with the row running fastest -- see the kernel.
+  FastDiv d_batch, d_zdiv, d_tiles_n, d_brick, d_panel, d_mbk;  // divisors mbk*nbk, mbk*panel, mbk
+  int nbk, panel;
+  int xn_shift, xm_shift, zbk;  // log2 of xn and xm, batch*groups entries per brick
 };
 
 constexpr int kThreads = 256;
@@ -721,11 +724,15 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   // one batch of scalar loads at entry instead of three dependent rounds (each a trip to memory on a cold cache).
   const unsigned id = blockIdx.x + blockIdx.y * gridDim.x;
   const unsigned xcd = id & 7, slot = id >> 3;
-  const unsigned sn = fast_div(slot, p.d_nbk);  // slot / nbk
-  const unsigned snm = fast_div(sn, p.d_mbk);   // slot / (nbk * mbk)
-  const int tile_n_x = (int)((xcd & ((1u << p.xn_shift) - 1)) * p.d_nbk.d + (slot - sn * p.d_nbk.d));
-  const int tile_m_x = (int)(((xcd >> p.xn_shift) & ((1u << p.xm_shift) - 1)) * p.d_mbk.d + (sn - snm * p.d_mbk.d));
-  const int z_x = (int)((xcd >> (p.xn_shift + p.xm_shift)) * p.zbk + snm);
+  // The ~32 workgroups an XCD runs at a time should cover a compact block of the brick, not a row of it: they
+  // share the XCD's L2, and a 4 x 8 block of tiles reads 12 tile-operands where a 1 x 32 row reads 33.
+  const unsigned zl = fast_div(slot, p.d_brick);  // entry of the batch*groups axis inside the brick
+  const unsigned t = slot - zl * p.d_brick.d;      // tile inside the mbk x nbk brick
+  const unsigned pn = fast_div(t, p.d_panel), r = t - pn * p.d_panel.d;
+  const unsigned cn = fast_div(r, p.d_mbk), cm = r - cn * p.d_mbk.d;
+  const int tile_n_x = (int)((xcd & ((1u << p.xn_shift) - 1)) * p.nbk + pn * p.panel + cn);
+  const int tile_m_x = (int)(((xcd >> p.xn_shift) & ((1u << p.xm_shift) - 1)) * p.d_mbk.d + cm);
+  const int z_x = (int)((xcd >> (p.xn_shift + p.xm_shift)) * p.zbk + zl);
   const int tile_m_p = (int)fast_div(blockIdx.x, p.d_tiles_n);
   const int tile_n_p = (int)(blockIdx.x - tile_m_p * p.d_tiles_n.d);
   const bool bricks = p.xg != 0;
@@ -1200,8 +1207,17 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   a.d_batch = make_fastdiv((unsigned)d->batch);
   a.d_zdiv = make_fastdiv((unsigned)d->zdiv);
   a.d_tiles_n = make_fastdiv((unsigned)a.tiles_n);
-  a.d_nbk = make_fastdiv((unsigned)(a.xg ? a.tiles_n / a.xn : 1));
-  a.d_mbk = make_fastdiv((unsigned)(a.xg ? a.tiles_m / a.xm : 1));
+  {
+    const int nbk = a.xg ? a.tiles_n / a.xn : 1, mbk = a.xg ? a.tiles_m / a.xm : 1;
+    // panel width: the largest power of two that divides nbk and keeps a panel (mbk rows) within ~32 tiles
+    int panel = 1;
+    while (panel * 2 * mbk <= 32 && nbk % (panel * 2) == 0) panel *= 2;
+    a.nbk = nbk;
+    a.panel = panel;
+    a.d_brick = make_fastdiv((unsigned)(nbk * mbk));
+    a.d_panel = make_fastdiv((unsigned)(mbk * panel));
+    a.d_mbk = make_fastdiv((unsigned)mbk);
+  }
   a.xn_shift = a.xn == 8 ? 3 : a.xn == 4 ? 2 : a.xn == 2 ? 1 : 0;
   a.xm_shift = a.xm == 8 ? 3 : a.xm == 4 ? 2 : a.xm == 2 ? 1 : 0;
   a.zbk = a.xg ? (int)(nz / a.xg) : 0;
