@@ -240,6 +240,28 @@ int rtp_attn_bwd(void* stream, int dtype, const void* q, const void* k, const vo
                  int64_t L, int64_t N, int64_t H, int64_t D, int64_t G);
 
 /* ---------------------------------------------------------------------------------------------
+ * Fused attention core for any sequence length (reference: the same per-head-group core,
+ * rtp/module/functional.py:779-800 and :815-830, there bmm -> softmax -> bmm with the [L, L] probabilities
+ * in memory).  bf16 only, D in {32, 64, 128}; addressing, mask, causal and scale as for rtp_attn_fwd.  One
+ * wavefront per (group, batch, head, 32-query block) walks the keys in blocks of 32 with a running softmax;
+ * the probabilities are never stored.  lse and delta are fp32 [G][N][H][L].
+ *   fwd: o = softmax(scale * q k^T + mask) v,  lse = log sum_j exp(scale * q k_j + mask_j)
+ *   bwd: p recomputed from lse; delta = rowsum(dout o o) (written here, scratch for the caller);
+ *        dv = p^T dout, ds = scale * p o (dout v^T - delta), dq = ds k, dk = ds^T q
+ * A query whose keys are all masked with -inf gets o = 0 and lse = 0 (torch gives NaN there).
+ * --------------------------------------------------------------------------------------------- */
+int rtp_attn_flash_supported(int dtype, int64_t L, int64_t D);
+int rtp_attn_flash_fwd(void* stream, int dtype, const void* q, const void* k, const void* v, int64_t s_l,
+                       int64_t s_b, int64_t s_h, int64_t s_g, void* o, int64_t o_l, int64_t o_b, int64_t o_h,
+                       int64_t o_g, float* lse, const float* mask, int causal, float scale, int64_t L,
+                       int64_t N, int64_t H, int64_t D, int64_t G);
+int rtp_attn_flash_bwd(void* stream, int dtype, const void* q, const void* k, const void* v, int64_t s_l,
+                       int64_t s_b, int64_t s_h, int64_t s_g, const void* o, const void* dout, int64_t o_l,
+                       int64_t o_b, int64_t o_h, int64_t o_g, const float* lse, float* delta, void* dq,
+                       void* dk, void* dv, const float* mask, int causal, float scale, int64_t L, int64_t N,
+                       int64_t H, int64_t D, int64_t G);
+
+/* ---------------------------------------------------------------------------------------------
  * Residual add + LayerNorm of the post-LN decoder layer (reference: norm1(x + sa_block(x)) and
  * norm2(x + ff_block(x)), rtp/models/transformer_lm_rtp.py:176-177, there two ATen calls each way).
  *   fwd: z = x + r (rounded to `dtype`; r NULL: z = x, z_out unused), y = (z - mean) * rstd * gamma + beta,

@@ -349,12 +349,400 @@ __global__ __launch_bounds__(NWV * 64) void attn_bwd_small_kernel(AttnArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Any sequence length: the same one-wavefront-per-tile pieces in a loop over 32-key (or 32-query) blocks with a
+// running softmax, so the [L, L] probabilities never go to memory.  Forward keeps log-sum-exp per query; backward
+// recomputes the probabilities from it, once in a pass that owns a query block (dQ, and the row dot products
+// delta = sum_d dO*O) and once in a pass that owns a key block (dK, dV): no atomics, fixed summation order.
+// A wave works on its own LDS tiles and never meets another wave, so block counts may differ per wave (causal).
+struct FlashArgs {
+  const bf16_t *q, *k, *v;
+  bf16_t *dq, *dk, *dv;
+  long s_l, s_b, s_h, s_g;  // element strides of q / k / v (and dq / dk / dv): sequence, batch, head, group
+  bf16_t* o;                // forward output; backward reads it for delta
+  const bf16_t* dout;
+  long o_l, o_b, o_h, o_g;  // element strides of o / dout
+  float* lse;               // [G*N*H][L] log-sum-exp of the scaled, masked scores
+  float* delta;             // [G*N*H][L] row dot products dO . O (written by the dQ pass, read by the dK/dV pass)
+  const float* mask;        // additive [L][L] or null
+  int causal;
+  float scale;
+  int L, N, H, nblk;  // nblk = ceil(L / 32)
+  long nprob;         // G * N * H
+};
+
+// Orders a wave's LDS writes before its own later LDS reads of other lanes' data (no instruction is needed for
+// that, the LDS serves a wave's accesses in order; this keeps the compiler from reordering them).
+__device__ __forceinline__ void wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+struct FlashItem {
+  long z, qkv_off, o_off;
+  int blk;
+  bool live;
+};
+__device__ __forceinline__ FlashItem flash_locate(const FlashArgs& a, int waves_per_block) {
+  FlashItem it;
+  long w = (long)blockIdx.x * waves_per_block + (threadIdx.x >> 6);
+  const long total = a.nprob * a.nblk;
+  it.live = w < total;
+  if (!it.live) w = total - 1;  // idle waves redo the last item and store nothing
+  it.z = w / a.nblk;
+  it.blk = (int)(w - it.z * a.nblk);
+  const long h = it.z % a.H, b = (it.z / a.H) % a.N, g = it.z / ((long)a.H * a.N);
+  it.qkv_off = b * a.s_b + h * a.s_h + g * a.s_g;
+  it.o_off = b * a.o_b + h * a.o_h + g * a.o_g;
+  return it;
+}
+
+// The 16 additive mask values of lane (li, g) for queries q0 + li and keys k0 + 8*(r/4) + 4*g + r%4; entries outside
+// the sequence read element 0 (their scores are discarded anyway).
+__device__ __forceinline__ void flash_mask(const FlashArgs& a, int query, int k0, int g, float (&mk)[16]) {
+#pragma unroll
+  for (int r = 0; r < 16; ++r) mk[r] = 0.0f;
+  if (!a.mask) return;
+  if (a.L % 4 == 0 && reinterpret_cast<uintptr_t>(a.mask) % 16 == 0) {
+#pragma unroll
+    for (int a4 = 0; a4 < 4; ++a4) {
+      const int key0 = k0 + 8 * a4 + 4 * g;
+      const float4 m4 =
+          *reinterpret_cast<const float4*>(a.mask + ((query < a.L && key0 < a.L) ? (long)query * a.L + key0 : 0));
+      mk[4 * a4 + 0] = m4.x, mk[4 * a4 + 1] = m4.y, mk[4 * a4 + 2] = m4.z, mk[4 * a4 + 3] = m4.w;
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int key = k0 + 8 * (r >> 2) + 4 * g + (r & 3);
+      mk[r] = a.mask[(query < a.L && key < a.L) ? (long)query * a.L + key : 0];
+    }
+  }
+}
+
+template <int DB, int NWV>
+__global__ __launch_bounds__(NWV * 64) void attn_flash_fwd_kernel(FlashArgs a) {
+  touch_kernel_arguments<sizeof(FlashArgs)>();
+  constexpr int D = 32 * DB, P = D + 8;
+  constexpr bool PREFETCH = DB <= 2;  // next block's K / V in registers while this one is worked on
+  __shared__ __attribute__((aligned(16))) bf16_t tiles[NWV][3][kSeqMax * P];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, li = lane & 31, g = lane >> 5;
+  const FlashItem it = flash_locate(a, NWV);
+  const int qb = a.nblk - 1 - it.blk;  // the long (causal) items first
+  const int q0 = qb * kSeqMax, query = q0 + li;
+  const bool qlive = query < a.L;
+  bf16_t* Qs = tiles[wave][0];
+  bf16_t* Ks = tiles[wave][1];
+  bf16_t* Vs = tiles[wave][2];
+  const long kv_step = (long)kSeqMax * a.s_l;
+  const bf16_t* kbase = a.k + it.qkv_off;
+  const bf16_t* vbase = a.v + it.qkv_off;
+  {
+    TileRegs<D, 1> rq;
+    const bf16_t* const src[1] = {a.q + it.qkv_off + (long)q0 * a.s_l};
+    const long sl[1] = {a.s_l};
+    rq.fetch(src, sl, a.L - q0, lane);
+    bf16_t* const tl[1] = {Qs};
+    rq.commit(tl, a.L - q0, lane);
+  }
+  const int kb_end = a.causal ? qb : a.nblk - 1;
+  TileRegs<D, 2> rkv;
+  const long sl2[2] = {a.s_l, a.s_l};
+  bf16_t* const tl2[2] = {Ks, Vs};
+  if (PREFETCH) {
+    const bf16_t* const src[2] = {kbase, vbase};
+    rkv.fetch(src, sl2, a.L, lane);
+  }
+  float m_run = -INFINITY, l_run = 0.0f;
+  f32x16 acc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[db][r] = 0.0f;
+  for (int kb = 0; kb <= kb_end; ++kb) {
+    const int k0 = kb * kSeqMax;
+    if (!PREFETCH) {
+      const bf16_t* const src[2] = {kbase + kb * kv_step, vbase + kb * kv_step};
+      rkv.fetch(src, sl2, a.L - k0, lane);
+    }
+    wave_sync();  // the previous block's fragment reads are done
+    rkv.commit(tl2, a.L - k0, lane);
+    wave_sync();
+    if (PREFETCH && kb < kb_end) {
+      const bf16_t* const src[2] = {kbase + (kb + 1) * kv_step, vbase + (kb + 1) * kv_step};
+      rkv.fetch(src, sl2, a.L - k0 - kSeqMax, lane);
+    }
+    float mk[16];
+    flash_mask(a, query, k0, g, mk);
+    f32x16 s;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = 0.0f;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks)
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rowmajor(Ks, P, li, g, ks), frag_rowmajor(Qs, P, li, g, ks), s,
+                                                  0, 0, 0);
+    float val[16];
+    float bm = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int key = k0 + 8 * (r >> 2) + 4 * g + (r & 3);
+      const bool visible = key < a.L && (!a.causal || key <= query);
+      val[r] = visible ? s[r] * a.scale + mk[r] : -INFINITY;
+      bm = fmaxf(bm, val[r]);
+    }
+    bm = fmaxf(bm, __shfl_xor(bm, 32, kWave));
+    const float m_new = fmaxf(m_run, bm);
+    const float alpha = m_run == -INFINITY ? 0.0f : expf(m_run - m_new);
+    float rs = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      val[r] = val[r] == -INFINITY ? 0.0f : expf(val[r] - m_new);
+      rs += val[r];
+    }
+    rs += __shfl_xor(rs, 32, kWave);
+    l_run = l_run * alpha + rs;
+    m_run = m_new;
+    bf16x8 pb[2];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) pb[r >> 3][r & 7] = from_f32<bf16_t>(val[r]);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[db][r] *= alpha;
+#pragma unroll
+      for (int m = 0; m < 2; ++m)
+        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_acc_order(Vs, P, 32 * db + li, m, g), pb[m], acc[db],
+                                                          0, 0, 0);
+    }
+  }
+  const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+  if (it.live && qlive) {
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[db][r] *= inv;
+      store_transposed(a.o + it.o_off + (long)query * a.o_l, db, g, acc[db]);
+    }
+    if (g == 0) a.lse[it.z * a.L + query] = l_run > 0.0f ? m_run + logf(l_run) : 0.0f;
+  }
+}
+
+// Recomputed probabilities and score gradients of one (query block, key block) pair, lane (li, g) = query q0 + li:
+// p[r] = exp(scale * s + mask - lse), ds[r] = scale * p * (dp - delta) for the 16 keys of the lane.
+template <int D>
+__device__ __forceinline__ void flash_p_ds(const FlashArgs& a, const bf16_t* Qs, const bf16_t* Ks, const bf16_t* Vs,
+                                           const bf16_t* Gs, int query, int k0, int li, int g, float lse, float delta,
+                                           float (&pv)[16], float (&ds)[16]) {
+  constexpr int P = D + 8;
+  float mk[16];
+  flash_mask(a, query, k0, g, mk);
+  f32x16 s, dp;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.0f;
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ++ks) {
+    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rowmajor(Ks, P, li, g, ks), frag_rowmajor(Qs, P, li, g, ks), s, 0,
+                                                0, 0);
+    dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rowmajor(Vs, P, li, g, ks), frag_rowmajor(Gs, P, li, g, ks), dp,
+                                                 0, 0, 0);
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int key = k0 + 8 * (r >> 2) + 4 * g + (r & 3);
+    const bool visible = query < a.L && key < a.L && (!a.causal || key <= query);
+    pv[r] = visible ? expf(s[r] * a.scale + mk[r] - lse) : 0.0f;
+    ds[r] = a.scale * pv[r] * (dp[r] - delta);
+  }
+}
+
+template <int DB, int NWV>
+__global__ __launch_bounds__(NWV * 64) void attn_flash_dq_kernel(FlashArgs a) {
+  touch_kernel_arguments<sizeof(FlashArgs)>();
+  constexpr int D = 32 * DB, P = D + 8;
+  constexpr bool PREFETCH = DB <= 2;
+  __shared__ __attribute__((aligned(16))) bf16_t tiles[NWV][4][kSeqMax * P];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, li = lane & 31, g = lane >> 5;
+  const FlashItem it = flash_locate(a, NWV);
+  const int qb = a.nblk - 1 - it.blk;
+  const int q0 = qb * kSeqMax, query = q0 + li;
+  const bool qlive = query < a.L;
+  bf16_t* Qs = tiles[wave][0];
+  bf16_t* Ks = tiles[wave][1];
+  bf16_t* Vs = tiles[wave][2];
+  bf16_t* Gs = tiles[wave][3];  // dO
+  const long kv_step = (long)kSeqMax * a.s_l;
+  const bf16_t* kbase = a.k + it.qkv_off;
+  const bf16_t* vbase = a.v + it.qkv_off;
+  {
+    // Q, dO and (in the K tile's place) O of the query block; delta = sum_d dO * O per query
+    TileRegs<D, 3> r3;
+    const bf16_t* const src[3] = {a.q + it.qkv_off + (long)q0 * a.s_l, a.dout + it.o_off + (long)q0 * a.o_l,
+                                  a.o + it.o_off + (long)q0 * a.o_l};
+    const long sl[3] = {a.s_l, a.o_l, a.o_l};
+    r3.fetch(src, sl, a.L - q0, lane);
+    bf16_t* const tl[3] = {Qs, Gs, Ks};
+    r3.commit(tl, a.L - q0, lane);
+  }
+  wave_sync();
+  float delta = 0.0f;
+#pragma unroll
+  for (int c = 0; c < D / 2; c += 8) {
+    const bf16x8 gv = *reinterpret_cast<const bf16x8*>(Gs + li * P + g * (D / 2) + c);
+    const bf16x8 ov = *reinterpret_cast<const bf16x8*>(Ks + li * P + g * (D / 2) + c);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) delta += to_f32(gv[e]) * to_f32(ov[e]);
+  }
+  delta += __shfl_xor(delta, 32, kWave);
+  if (it.live && qlive && g == 0) a.delta[it.z * a.L + query] = delta;
+  const float lse = a.lse[it.z * a.L + (qlive ? query : 0)];
+  const int kb_end = a.causal ? qb : a.nblk - 1;
+  TileRegs<D, 2> rkv;
+  const long sl2[2] = {a.s_l, a.s_l};
+  bf16_t* const tl2[2] = {Ks, Vs};
+  if (PREFETCH) {
+    const bf16_t* const src[2] = {kbase, vbase};
+    rkv.fetch(src, sl2, a.L, lane);
+  }
+  f32x16 acc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[db][r] = 0.0f;
+  for (int kb = 0; kb <= kb_end; ++kb) {
+    const int k0 = kb * kSeqMax;
+    if (!PREFETCH) {
+      const bf16_t* const src[2] = {kbase + kb * kv_step, vbase + kb * kv_step};
+      rkv.fetch(src, sl2, a.L - k0, lane);
+    }
+    wave_sync();
+    rkv.commit(tl2, a.L - k0, lane);
+    wave_sync();
+    if (PREFETCH && kb < kb_end) {
+      const bf16_t* const src[2] = {kbase + (kb + 1) * kv_step, vbase + (kb + 1) * kv_step};
+      rkv.fetch(src, sl2, a.L - k0 - kSeqMax, lane);
+    }
+    float pv[16], ds[16];
+    flash_p_ds<D>(a, Qs, Ks, Vs, Gs, query, k0, li, g, lse, delta, pv, ds);
+    bf16x8 dsb[2];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dsb[r >> 3][r & 7] = from_f32<bf16_t>(ds[r]);
+    // dQ^T[dd][query] += sum_key K[key][dd] dS[query][key]
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int m = 0; m < 2; ++m)
+        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_acc_order(Ks, P, 32 * db + li, m, g), dsb[m], acc[db],
+                                                          0, 0, 0);
+  }
+  if (it.live && qlive) {
+#pragma unroll
+    for (int db = 0; db < DB; ++db) store_transposed(a.dq + it.qkv_off + (long)query * a.s_l, db, g, acc[db]);
+  }
+}
+
+template <int DB, int NWV>
+__global__ __launch_bounds__(NWV * 64) void attn_flash_dkv_kernel(FlashArgs a) {
+  touch_kernel_arguments<sizeof(FlashArgs)>();
+  constexpr int D = 32 * DB, P = D + 8;
+  constexpr bool PREFETCH = DB <= 2;
+  __shared__ __attribute__((aligned(16))) bf16_t tiles[NWV][4][kSeqMax * P];
+  __shared__ __attribute__((aligned(16))) bf16_t ptiles[NWV][2][kSeqMax * kPPitch];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, li = lane & 31, g = lane >> 5;
+  const FlashItem it = flash_locate(a, NWV);
+  const int kb = it.blk;  // causal: key block 0 meets every query block, so the long items come first
+  const int k0 = kb * kSeqMax, key_row = k0 + li;
+  bf16_t* Qs = tiles[wave][0];
+  bf16_t* Ks = tiles[wave][1];
+  bf16_t* Vs = tiles[wave][2];
+  bf16_t* Gs = tiles[wave][3];  // dO
+  bf16_t* DSs = ptiles[wave][0];
+  bf16_t* Ps = ptiles[wave][1];
+  {
+    TileRegs<D, 2> r2;
+    const bf16_t* const src[2] = {a.k + it.qkv_off + (long)k0 * a.s_l, a.v + it.qkv_off + (long)k0 * a.s_l};
+    const long sl[2] = {a.s_l, a.s_l};
+    r2.fetch(src, sl, a.L - k0, lane);
+    bf16_t* const tl[2] = {Ks, Vs};
+    r2.commit(tl, a.L - k0, lane);
+  }
+  const int qb_start = a.causal ? kb : 0;
+  const long q_step = (long)kSeqMax * a.s_l, g_step = (long)kSeqMax * a.o_l;
+  const bf16_t* qbase = a.q + it.qkv_off;
+  const bf16_t* gbase = a.dout + it.o_off;
+  TileRegs<D, 2> rqg;
+  const long sl2[2] = {a.s_l, a.o_l};
+  bf16_t* const tl2[2] = {Qs, Gs};
+  if (PREFETCH) {
+    const bf16_t* const src[2] = {qbase + qb_start * q_step, gbase + qb_start * g_step};
+    rqg.fetch(src, sl2, a.L - qb_start * kSeqMax, lane);
+  }
+  f32x16 dk[DB], dv[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dk[db][r] = dv[db][r] = 0.0f;
+  for (int qb = qb_start; qb < a.nblk; ++qb) {
+    const int q0 = qb * kSeqMax, query = q0 + li;
+    if (!PREFETCH) {
+      const bf16_t* const src[2] = {qbase + qb * q_step, gbase + qb * g_step};
+      rqg.fetch(src, sl2, a.L - q0, lane);
+    }
+    wave_sync();  // the previous block's gathers are done
+    rqg.commit(tl2, a.L - q0, lane);
+    wave_sync();
+    if (PREFETCH && qb + 1 < a.nblk) {
+      const bf16_t* const src[2] = {qbase + (qb + 1) * q_step, gbase + (qb + 1) * g_step};
+      rqg.fetch(src, sl2, a.L - q0 - kSeqMax, lane);
+    }
+    const long qi = it.z * a.L + (query < a.L ? query : 0);
+    const float lse = a.lse[qi], delta = a.delta[qi];
+    float pv[16], ds[16];
+    flash_p_ds<D>(a, Qs, Ks, Vs, Gs, query, k0, li, g, lse, delta, pv, ds);
+    // dS and P as [query][key] tiles for the products that contract over the queries
+#pragma unroll
+    for (int a4 = 0; a4 < 4; ++a4) {
+      union {
+        uint2 u;
+        bf16_t e[4];
+      } d4, p4;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        d4.e[e] = from_f32<bf16_t>(ds[4 * a4 + e]);
+        p4.e[e] = from_f32<bf16_t>(pv[4 * a4 + e]);
+      }
+      *reinterpret_cast<uint2*>(DSs + li * kPPitch + 8 * a4 + 4 * g) = d4.u;
+      *reinterpret_cast<uint2*>(Ps + li * kPPitch + 8 * a4 + 4 * g) = p4.u;
+    }
+    wave_sync();
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int m = 0; m < 2; ++m) {
+        // dK^T[dd][key] += sum_query Q[query][dd] dS[query][key];  dV^T[dd][key] += sum_query dO[query][dd] P[query][key]
+        dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_natural(Qs, P, 32 * db + li, m, g),
+                                                         gather_natural(DSs, kPPitch, li, m, g), dk[db], 0, 0, 0);
+        dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_natural(Gs, P, 32 * db + li, m, g),
+                                                         gather_natural(Ps, kPPitch, li, m, g), dv[db], 0, 0, 0);
+      }
+    }
+  }
+  if (it.live && key_row < a.L) {
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      store_transposed(a.dk + it.qkv_off + (long)key_row * a.s_l, db, g, dk[db]);
+      store_transposed(a.dv + it.qkv_off + (long)key_row * a.s_l, db, g, dv[db]);
+    }
+  }
+}
+
 static bool aligned8(int64_t v) { return v % 8 == 0; }
 
 static int check_common(const char* who, int dtype, int64_t L, int64_t N, int64_t H, int64_t D, int64_t G, int64_t s_l,
-                        int64_t s_b, int64_t s_h, int64_t s_g, int64_t o_l, int64_t o_b, int64_t o_h, int64_t o_g) {
+                        int64_t s_b, int64_t s_h, int64_t s_g, int64_t o_l, int64_t o_b, int64_t o_h, int64_t o_g,
+                        int64_t max_len = kSeqMax) {
   RTP_REQUIRE(dtype == RTP_BF16, "%s: only bf16 is implemented (dtype %d)", who, dtype);
-  RTP_REQUIRE(L >= 1 && L <= kSeqMax, "%s: sequence length %lld not in 1..%d", who, (long long)L, kSeqMax);
+  RTP_REQUIRE(L >= 1 && L <= max_len, "%s: sequence length %lld not in 1..%lld", who, (long long)L, (long long)max_len);
   RTP_REQUIRE(D == 32 || D == 64 || D == 128, "%s: head dimension %lld not in {32, 64, 128}", who, (long long)D);
   RTP_REQUIRE(N >= 1 && H >= 1 && G >= 1, "%s: batch, heads and groups must be >= 1", who);
   RTP_REQUIRE(aligned8(s_l) && aligned8(s_b) && aligned8(s_h) && aligned8(s_g) && aligned8(o_l) && aligned8(o_b) &&
@@ -427,4 +815,94 @@ extern "C" int rtp_attn_bwd(void* stream, int dtype, const void* q, const void* 
     hipLaunchKernelGGL((attn_bwd_small_kernel<4, 2>), dim3((unsigned)ceil_div(a.nprob, 2)), dim3(128), 0, st, a);
   RTP_LAUNCH_CHECK();
   return RTP_OK;
+}
+
+// ---- any sequence length (running softmax over 32-key blocks) ----
+
+static constexpr int64_t kFlashMaxLen = 1 << 20;
+
+extern "C" int rtp_attn_flash_supported(int dtype, int64_t L, int64_t D) {
+  return dtype == RTP_BF16 && L >= 1 && L <= kFlashMaxLen && (D == 32 || D == 64 || D == 128);
+}
+
+template <template <int, int> class Launcher>
+static int flash_dispatch(int64_t D, const FlashArgs& a, hipStream_t st) {
+  const long items = a.nprob * a.nblk;
+  if (D == 32)
+    Launcher<1, 4>::run(a, st, items);
+  else if (D == 64)
+    Launcher<2, 4>::run(a, st, items);
+  else
+    Launcher<4, 2>::run(a, st, items);
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
+}
+#define RTP_FLASH_LAUNCHER(NAME, KERNEL)                                                                       \
+  template <int DB, int NWV>                                                                                   \
+  struct NAME {                                                                                                \
+    static void run(const FlashArgs& a, hipStream_t st, long items) {                                          \
+      hipLaunchKernelGGL((KERNEL<DB, NWV>), dim3((unsigned)ceil_div(items, NWV)), dim3(NWV * 64), 0, st, a);   \
+    }                                                                                                          \
+  };
+RTP_FLASH_LAUNCHER(FlashFwd, attn_flash_fwd_kernel)
+RTP_FLASH_LAUNCHER(FlashDq, attn_flash_dq_kernel)
+RTP_FLASH_LAUNCHER(FlashDkv, attn_flash_dkv_kernel)
+
+static int flash_args(const char* who, FlashArgs& a, int dtype, int64_t s_l, int64_t s_b, int64_t s_h, int64_t s_g,
+                      int64_t o_l, int64_t o_b, int64_t o_h, int64_t o_g, const float* mask, int causal, float scale,
+                      int64_t L, int64_t N, int64_t H, int64_t D, int64_t G) {
+  if (int rc = check_common(who, dtype, L, N, H, D, G, s_l, s_b, s_h, s_g, o_l, o_b, o_h, o_g, kFlashMaxLen)) return rc;
+  a.s_l = s_l, a.s_b = s_b, a.s_h = s_h, a.s_g = s_g;
+  a.o_l = o_l, a.o_b = o_b, a.o_h = o_h, a.o_g = o_g;
+  a.mask = mask, a.causal = causal, a.scale = scale;
+  a.L = (int)L, a.N = (int)N, a.H = (int)H, a.nblk = (int)ceil_div(L, kSeqMax), a.nprob = G * N * H;
+  RTP_REQUIRE(ceil_div(a.nprob * a.nblk, 2) < (1ll << 31), "%s: too many (head, block) work items", who);
+  return RTP_OK;
+}
+
+extern "C" int rtp_attn_flash_fwd(void* stream, int dtype, const void* q, const void* k, const void* v, int64_t s_l,
+                                  int64_t s_b, int64_t s_h, int64_t s_g, void* o, int64_t o_l, int64_t o_b,
+                                  int64_t o_h, int64_t o_g, float* lse, const float* mask, int causal, float scale,
+                                  int64_t L, int64_t N, int64_t H, int64_t D, int64_t G) {
+  RTP_REQUIRE(q && k && v && o && lse, "rtp_attn_flash_fwd: null pointer");
+  RTP_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o) % 16 == 0,
+              "rtp_attn_flash_fwd: q, k, v, o must be 16-byte aligned");
+  FlashArgs a{};
+  if (int rc = flash_args("rtp_attn_flash_fwd", a, dtype, s_l, s_b, s_h, s_g, o_l, o_b, o_h, o_g, mask, causal, scale,
+                          L, N, H, D, G))
+    return rc;
+  a.q = (const bf16_t*)q, a.k = (const bf16_t*)k, a.v = (const bf16_t*)v;
+  a.o = (bf16_t*)o, a.lse = lse;
+  hipStream_t st = (hipStream_t)stream;
+  const double np = (double)a.nprob, vis = causal ? 0.5 : 1.0;
+  ProfileScope prof(st, "attn_flash_fwd", 4.0 * np * L * L * D * vis, np * (4.0 * L * D * 2.0 + 4.0 * L));
+  return flash_dispatch<FlashFwd>(D, a, st);
+}
+
+extern "C" int rtp_attn_flash_bwd(void* stream, int dtype, const void* q, const void* k, const void* v, int64_t s_l,
+                                  int64_t s_b, int64_t s_h, int64_t s_g, const void* o, const void* dout, int64_t o_l,
+                                  int64_t o_b, int64_t o_h, int64_t o_g, const float* lse, float* delta, void* dq,
+                                  void* dk, void* dv, const float* mask, int causal, float scale, int64_t L,
+                                  int64_t N, int64_t H, int64_t D, int64_t G) {
+  RTP_REQUIRE(q && k && v && o && dout && lse && delta && dq && dk && dv, "rtp_attn_flash_bwd: null pointer");
+  RTP_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o | (uintptr_t)dout | (uintptr_t)dq |
+               (uintptr_t)dk | (uintptr_t)dv) % 16 == 0,
+              "rtp_attn_flash_bwd: q, k, v, o, dout, dq, dk, dv must be 16-byte aligned");
+  FlashArgs a{};
+  if (int rc = flash_args("rtp_attn_flash_bwd", a, dtype, s_l, s_b, s_h, s_g, o_l, o_b, o_h, o_g, mask, causal, scale,
+                          L, N, H, D, G))
+    return rc;
+  a.q = (const bf16_t*)q, a.k = (const bf16_t*)k, a.v = (const bf16_t*)v;
+  a.dq = (bf16_t*)dq, a.dk = (bf16_t*)dk, a.dv = (bf16_t*)dv;
+  a.o = (bf16_t*)const_cast<void*>(o), a.dout = (const bf16_t*)dout;
+  a.lse = const_cast<float*>(lse), a.delta = delta;
+  hipStream_t st = (hipStream_t)stream;
+  const double np = (double)a.nprob, vis = causal ? 0.5 : 1.0;
+  {
+    // the query-block pass writes delta, the key-block pass reads it: same stream, in this order
+    ProfileScope prof(st, "attn_flash_dq", 6.0 * np * L * L * D * vis, np * (5.0 * L * D * 2.0 + 8.0 * L));
+    if (int rc = flash_dispatch<FlashDq>(D, a, st)) return rc;
+  }
+  ProfileScope prof(st, "attn_flash_dkv", 8.0 * np * L * L * D * vis, np * (6.0 * L * D * 2.0 + 8.0 * L));
+  return flash_dispatch<FlashDkv>(D, a, st);
 }

@@ -100,7 +100,12 @@ def _bmm(dtype, *, a, a_off, lda, a_kc, a_s, a_sg, b, b_off, ldb, b_kc, b_s, b_s
 class _AttentionFn(torch.autograd.Function):
     """Buffers hold all head groups side by side: qkv [L*N, ws*3E_s] (group g at column block g, inside it
     Q | K | V of that group), p [ws*N*h_s, L, L], o [L*N, E] (= the unsharded head order).  A (group,
-    batch, head) triple is addressed by strides inside the batched GEMM, so nothing is re-laid out."""
+    batch, head) triple is addressed by strides inside the batched GEMM, so nothing is re-laid out.
+
+    The core runs in one of three forms: bf16 with L <= 32 in one launch that keeps the scores in registers and
+    stores p; bf16 with longer sequences in a running-softmax launch that stores only the log-sum-exp per
+    query (not when the caller wants the attention weights back); otherwise as batched products and a softmax
+    kernel with p in memory."""
 
     @staticmethod
     def forward(ctx, x, anchor, layer, mask, causal, want_weights, residual_grad=False):
@@ -114,11 +119,15 @@ class _AttentionFn(torch.autograd.Function):
         off = store.offsets
         b_in_off, w_o_off, b_o_off = (off[1], off[2], off[3]) if layer.has_bias else (None, off[1], None)
         qkv = torch.empty(rows, ws * 3 * e_s, dtype=dt, device=dev)
-        p = torch.empty(ws * Z, L, L, dtype=dt, device=dev)
         o = torch.empty(rows, E, dtype=dt, device=dev)
         out = torch.empty(rows, E, dtype=dt, device=dev)
         ldq = N * ws * 3 * e_s
         fused = ops.attn_supported(dt, L, d)
+        flash = not fused and not want_weights and ops.attn_flash_supported(dt, L, d)
+        if flash:
+            p = torch.empty(ws * Z, L, dtype=torch.float32, device=dev)  # log-sum-exp in place of probabilities
+        else:
+            p = torch.empty(ws * Z, L, L, dtype=dt, device=dev)
         order = ring_order(layer.rank, ws)
         rot = Rotation(store.home, order, group=store.stage_group)
         acc = ops.ShardSum(out, sum(len(w) for w in rot.windows))
@@ -132,6 +141,14 @@ class _AttentionFn(torch.autograd.Function):
                     ops.attn_fwd(qkv, q0, q0 + e_s, q0 + 2 * e_s, (ldq, ws * 3 * e_s, d, 3 * e_s), o, first * e_s,
                                  (N * E, E, d, e_s), p[first * Z:(first + cnt) * Z], mask, causal, scale, L, N, h_s,
                                  d, cnt)
+                    c_out, c_in = acc.target(i)
+                    S.row_fwd(o, flat, w_o_off, E, e_s, b_o_off, c_out, first * e_s, c_in=c_in)
+                    i += 1
+                    continue
+                if flash:
+                    ops.attn_flash_fwd(qkv, q0, q0 + e_s, q0 + 2 * e_s, (ldq, ws * 3 * e_s, d, 3 * e_s), o,
+                                       first * e_s, (N * E, E, d, e_s), p[first * Z:(first + cnt) * Z], mask, causal,
+                                       scale, L, N, h_s, d, cnt)
                     c_out, c_in = acc.target(i)
                     S.row_fwd(o, flat, w_o_off, E, e_s, b_o_off, c_out, first * e_s, c_in=c_in)
                     i += 1
@@ -158,6 +175,7 @@ class _AttentionFn(torch.autograd.Function):
         ctx.layer = layer
         ctx.dims = (L, N, E)
         ctx.residual_grad = residual_grad
+        ctx.flash = (mask, causal) if flash else None
         ctx.save_for_backward(x2, qkv, p, o)
         ctx.mark_non_differentiable(*([weights] if weights is not None else []))
         return out.view(L, N, E), weights
@@ -181,6 +199,7 @@ class _AttentionFn(torch.autograd.Function):
         dqkv = torch.empty(rows, ws * 3 * e_s, dtype=dt, device=dev)
         ldq = N * ws * 3 * e_s
         fused = ops.attn_supported(dt, L, d)
+        delta = torch.empty_like(p) if ctx.flash is not None else None
         order = ring_order(layer.rank, ws, reverse=True)
         rot = Rotation(store.home, order, group=store.stage_group)
         # residual_grad: the caller's y = norm(x + attention(x)) sends x's whole gradient through this function,
@@ -196,6 +215,17 @@ class _AttentionFn(torch.autograd.Function):
                 if fused:
                     ops.attn_bwd(qkv, q0, q0 + e_s, q0 + 2 * e_s, (ldq, ws * 3 * e_s, d, 3 * e_s), do, first * e_s,
                                  (N * E, E, d, e_s), p[first * Z:(first + cnt) * Z], dqkv, scale, L, N, h_s, d, cnt)
+                    if need_dx:
+                        c_out, c_in = acc.target(i)
+                        S.col_dgrad(dqkv, flat, 0, 3 * e_s, E, c_out, q0, c_in=c_in)
+                    i += 1
+                    continue
+                if ctx.flash is not None:
+                    mask, causal = ctx.flash
+                    ops.attn_flash_bwd(qkv, q0, q0 + e_s, q0 + 2 * e_s, (ldq, ws * 3 * e_s, d, 3 * e_s), o, do,
+                                       first * e_s, (N * E, E, d, e_s), p[first * Z:(first + cnt) * Z],
+                                       delta[first * Z:(first + cnt) * Z], dqkv, mask, causal, scale, L, N, h_s, d,
+                                       cnt)
                     if need_dx:
                         c_out, c_in = acc.target(i)
                         S.col_dgrad(dqkv, flat, 0, 3 * e_s, E, c_out, q0, c_in=c_in)

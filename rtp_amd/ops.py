@@ -316,6 +316,68 @@ def attn_bwd(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, qkv_strides,
                                    L, N, H, d, G))
 
 
+def attn_flash_supported(dtype: torch.dtype, L: int, d: int) -> bool:
+    """Whether the running-softmax attention core handles this shape (bf16, any L, d in {32, 64, 128})."""
+    if dtype != torch.bfloat16:
+        return False
+    return bool(_lib.load().rtp_attn_flash_supported(dtype_code(dtype), L, d))
+
+
+def _flash_rows(name: str, t: torch.Tensor, G: int, N: int, H: int, L: int) -> None:
+    if t.dtype != torch.float32 or not t.is_contiguous() or t.numel() != G * N * H * L:
+        raise ValueError(f"{name} must be a contiguous fp32 [G*N*H, L] tensor")
+
+
+def _flash_mask(mask: Optional[torch.Tensor], L: int):
+    if mask is None:
+        return None
+    if mask.dtype != torch.float32 or tuple(mask.shape) != (L, L) or not mask.is_contiguous():
+        raise ValueError("attention mask must be a contiguous fp32 [L, L] tensor")
+    return mask.data_ptr()
+
+
+def attn_flash_fwd(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, qkv_strides, o: torch.Tensor, o_off: int,
+                   o_strides, lse: torch.Tensor, mask: Optional[torch.Tensor], causal: bool, scale: float, L: int,
+                   N: int, H: int, d: int, G: int) -> None:
+    """attn_fwd for any L: o = softmax(scale q k^T + mask) v without storing the probabilities; lse [G*N*H, L]
+    fp32 receives the log-sum-exp of each query's scores."""
+    _dev(qkv)
+    esz = qkv.element_size()
+    if o.dtype != qkv.dtype:
+        raise ValueError("attn_flash_fwd: o must share the operand dtype")
+    _flash_rows("attn_flash_fwd: lse", lse, G, N, H, L)
+    mask_ptr = _flash_mask(mask, L)
+    _lib.require_device()
+    base = qkv.data_ptr()
+    check(_lib.load().rtp_attn_flash_fwd(_stream(), dtype_code(qkv.dtype), base + q_off * esz, base + k_off * esz,
+                                         base + v_off * esz, *qkv_strides, o.data_ptr() + o_off * esz, *o_strides,
+                                         lse.data_ptr(), mask_ptr, int(causal), scale, L, N, H, d, G))
+
+
+def attn_flash_bwd(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, qkv_strides, o: torch.Tensor,
+                   dout: torch.Tensor, o_off: int, o_strides, lse: torch.Tensor, delta: torch.Tensor,
+                   dqkv: torch.Tensor, mask: Optional[torch.Tensor], causal: bool, scale: float, L: int, N: int,
+                   H: int, d: int, G: int) -> None:
+    """Backward of attn_flash_fwd: writes dq, dk, dv into `dqkv` (layout and offsets of `qkv`); `o` and `dout`
+    share layout and offset; `delta` [G*N*H, L] fp32 is scratch."""
+    _dev(qkv)
+    esz = qkv.element_size()
+    if dqkv.dtype != qkv.dtype or dqkv.shape != qkv.shape or dqkv.stride() != qkv.stride():
+        raise ValueError("attn_flash_bwd: dqkv must match qkv")
+    if dout.dtype != qkv.dtype or o.dtype != qkv.dtype or dout.shape != o.shape or dout.stride() != o.stride():
+        raise ValueError("attn_flash_bwd: o and dout must share dtype and layout")
+    _flash_rows("attn_flash_bwd: lse", lse, G, N, H, L)
+    _flash_rows("attn_flash_bwd: delta", delta, G, N, H, L)
+    mask_ptr = _flash_mask(mask, L)
+    _lib.require_device()
+    base, dbase = qkv.data_ptr(), dqkv.data_ptr()
+    check(_lib.load().rtp_attn_flash_bwd(_stream(), dtype_code(qkv.dtype), base + q_off * esz, base + k_off * esz,
+                                         base + v_off * esz, *qkv_strides, o.data_ptr() + o_off * esz,
+                                         dout.data_ptr() + o_off * esz, *o_strides, lse.data_ptr(), delta.data_ptr(),
+                                         dbase + q_off * esz, dbase + k_off * esz, dbase + v_off * esz, mask_ptr,
+                                         int(causal), scale, L, N, H, d, G))
+
+
 def layernorm_supported(dtype: torch.dtype, cols: int) -> bool:
     if dtype not in (torch.float32, torch.bfloat16):
         return False

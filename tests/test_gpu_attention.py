@@ -164,3 +164,101 @@ def test_attn_core_rejects_unsupported():
     with pytest.raises(RtpError):
         ops.attn_fwd(qkv, 0, 64, 128, (192, 192, 64, 192), o, 0, (64, 64, 64, 64), p, None, False, 0.125, 33, 1, 1,
                      64, 1)
+
+
+@pytest.mark.parametrize("L,d,causal,mask_kind", [
+    (33, 64, False, None),        # one full key block and a block of a single key
+    (64, 32, True, None),
+    (100, 64, True, None),        # ragged last block, causal: block counts differ per wavefront
+    (100, 128, False, "float"),
+    (96, 64, False, "neg_inf"),   # the causal pattern handed over as a -inf float mask (L % 4 == 0: 16-byte loads)
+    (97, 32, False, "neg_inf"),   # same, scalar mask loads
+    (17, 128, True, "float"),     # shorter than one block
+    (512, 64, True, None),
+])
+def test_attn_flash_core_against_torch_fp32(L, d, causal, mask_kind):
+    """rtp_attn_flash_fwd / rtp_attn_flash_bwd through the C ABI on a packed [L, N, G*3*H*d] projection, against
+    plain fp32 torch attention on the same bf16 inputs (tolerance 2e-2 of the largest reference entry); the
+    log-sum-exp against torch.logsumexp to 1e-3."""
+    from rtp_amd import ops
+    gen = torch.Generator().manual_seed(L * 131 + d)
+    N, H, G = 2, 3, 2
+    e_s = H * d
+    qkv = (torch.randn(L, N, G * 3 * e_s, generator=gen) * 0.5).to(torch.bfloat16)
+    dout = torch.randn(L, N, G * e_s, generator=gen).to(torch.bfloat16)
+    mask = {None: None, "float": torch.randn(L, L, generator=gen) * 2.0, "neg_inf": _causal(L)}[mask_kind]
+    scale = 1.0 / d ** 0.5
+    x = qkv.float().view(L, N, G, 3, H, d).requires_grad_()
+    q, k, v = x[:, :, :, 0], x[:, :, :, 1], x[:, :, :, 2]
+    s = torch.einsum("lnghd,mnghd->nghlm", q, k) * scale
+    if mask is not None:
+        s = s + mask
+    if causal:
+        s = s + _causal(L)
+    p_ref = torch.softmax(s, dim=-1)
+    lse_ref = torch.logsumexp(s.detach(), dim=-1).permute(1, 0, 2, 3)       # [G, N, H, L]
+    o_ref = torch.einsum("nghlm,mnghd->lnghd", p_ref, v).reshape(L, N, G * e_s)
+    o_ref.backward(dout.float())
+    qd, dd = qkv.to(DEV), dout.to(DEV)
+    o = torch.empty(L, N, G * e_s, dtype=torch.bfloat16, device=DEV)
+    lse = torch.empty(G * N * H, L, dtype=torch.float32, device=DEV)
+    delta = torch.empty_like(lse)
+    dqkv = torch.zeros_like(qd)
+    ld = G * 3 * e_s
+    qs, os_ = (N * ld, ld, d, 3 * e_s), (N * G * e_s, G * e_s, d, e_s)
+    md = None if mask is None else mask.to(DEV)
+    assert ops.attn_flash_supported(torch.bfloat16, L, d)
+    ops.attn_flash_fwd(qd, 0, e_s, 2 * e_s, qs, o, 0, os_, lse, md, causal, scale, L, N, H, d, G)
+    ops.attn_flash_bwd(qd, 0, e_s, 2 * e_s, qs, o, dd, 0, os_, lse, delta, dqkv, md, causal, scale, L, N, H, d, G)
+    assert_close(o, o_ref, torch.bfloat16, "o")
+    assert (lse.cpu().view(G, N, H, L) - lse_ref).abs().max().item() < 1e-3
+    delta_ref = (dout.float() * o.float().cpu()).view(L, N, G, H, d).sum(-1).permute(2, 1, 3, 0)
+    assert (delta.cpu().view(G, N, H, L) - delta_ref).abs().max().item() < 1e-3 * max(1.0, delta_ref.abs().max().item())
+    assert_close(dqkv, x.grad.reshape(L, N, ld), torch.bfloat16, "dqkv")
+
+
+def test_attn_flash_matches_short_sequence_core():
+    """On a sequence both cores take (L <= 32) they agree to bf16 rounding of the same fp32 results."""
+    from rtp_amd import ops
+    gen = torch.Generator().manual_seed(77)
+    L, N, H, G, d = 29, 2, 2, 1, 64
+    e_s, ld = H * d, 3 * H * d
+    qd = (torch.randn(L, N, ld, generator=gen) * 0.5).to(torch.bfloat16).to(DEV)
+    dd = torch.randn(L, N, e_s, generator=gen).to(torch.bfloat16).to(DEV)
+    qs, os_ = (N * ld, ld, d, 3 * e_s), (N * e_s, e_s, d, e_s)
+    o1, o2 = (torch.empty(L, N, e_s, dtype=torch.bfloat16, device=DEV) for _ in range(2))
+    p = torch.empty(N * H, L, L, dtype=torch.bfloat16, device=DEV)
+    lse = torch.empty(N * H, L, dtype=torch.float32, device=DEV)
+    d1, d2 = torch.zeros_like(qd), torch.zeros_like(qd)
+    ops.attn_fwd(qd, 0, e_s, 2 * e_s, qs, o1, 0, os_, p, None, True, 0.125, L, N, H, d, G)
+    ops.attn_bwd(qd, 0, e_s, 2 * e_s, qs, dd, 0, os_, p, d1, 0.125, L, N, H, d, G)
+    ops.attn_flash_fwd(qd, 0, e_s, 2 * e_s, qs, o2, 0, os_, lse, None, True, 0.125, L, N, H, d, G)
+    ops.attn_flash_bwd(qd, 0, e_s, 2 * e_s, qs, o2, dd, 0, os_, lse, torch.empty_like(lse), d2, None, True, 0.125, L,
+                       N, H, d, G)
+    assert_close(o2, o1.float(), torch.bfloat16, "o")
+    assert_close(d2, d1.float(), torch.bfloat16, "dqkv")
+
+
+@pytest.mark.parametrize("E,H,L,N,ws,masked,need_weights", [
+    (256, 4, 100, 3, 2, True, False),    # running-softmax core, ragged last block, -inf float mask
+    (512, 4, 70, 2, 4, False, False),    # head_dim 128
+    (128, 4, 48, 2, 2, True, True),      # returned weights: the products-and-softmax form with p in memory
+])
+def test_attention_long_sequence_bf16(E, H, L, N, ws, masked, need_weights):
+    _run(E, H, L, N, ws, torch.bfloat16, masked, need_weights, seed=6)
+
+
+def test_attn_flash_rejects_unsupported():
+    from rtp_amd import ops
+    from rtp_amd._lib import RtpError
+    assert not ops.attn_flash_supported(torch.float32, 64, 64)
+    assert not ops.attn_flash_supported(torch.bfloat16, 64, 48)
+    qkv = torch.zeros(40, 1, 3 * 64, dtype=torch.bfloat16, device=DEV)
+    o = torch.zeros(40, 1, 64, dtype=torch.bfloat16, device=DEV)
+    lse = torch.zeros(1, 40, dtype=torch.float32, device=DEV)
+    with pytest.raises(RtpError):   # stride not a multiple of 8 elements
+        ops.attn_flash_fwd(qkv, 0, 64, 128, (192, 192, 60, 192), o, 0, (64, 64, 64, 64), lse, None, False, 0.125, 40, 1,
+                           1, 64, 1)
+    with pytest.raises(ValueError):
+        ops.attn_flash_fwd(qkv, 0, 64, 128, (192, 192, 64, 192), o, 0, (64, 64, 64, 64), lse[:, :39], None, False,
+                           0.125, 40, 1, 1, 64, 1)
