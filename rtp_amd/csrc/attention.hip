@@ -70,20 +70,32 @@ struct TileRegs {
 __device__ __forceinline__ bf16x8 frag_rowmajor(const bf16_t* tile, int pitch, int li, int g, int ks) {
   return *reinterpret_cast<const bf16x8*>(tile + li * pitch + 16 * ks + 8 * g);
 }
-// Contraction index = tile row, in ACCUMULATOR order: slot e of instruction m in lane group g is row
-// 8*(2m + e/4) + 4g + e%4 (the row that accumulator register 8m + e of that lane group holds).
-__device__ __forceinline__ bf16x8 gather_acc_order(const bf16_t* tile, int pitch, int col, int m, int g) {
-  bf16x8 f;
-#pragma unroll
-  for (int e = 0; e < 8; ++e) f[e] = tile[(8 * (2 * m + (e >> 2)) + 4 * g + (e & 3)) * pitch + col];
-  return f;
+// Operand fragments whose contraction index is the tile ROW come through the LDS's transposing read: per group of
+// 16 lanes it takes a 4 x 16 block (lane t supplies the address of 4 consecutive elements of row t/4 at column
+// 4*(t%4)) and hands lane t the 4 elements of column t.  Two of them make the 8 contraction slots of a lane.
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+__device__ __forceinline__ s16x4 lds_transposed4(const bf16_t* tile, int pitch, int row0, int col0, int t) {
+  typedef __attribute__((address_space(3))) s16x4* lds_ptr;
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(tile + (row0 + (t >> 2)) * pitch + col0 + 4 * (t & 3)));
 }
-// Contraction index = tile row, in natural order: slot e of instruction m in lane group g is row 16m + 8g + e.
-__device__ __forceinline__ bf16x8 gather_natural(const bf16_t* tile, int pitch, int col, int m, int g) {
-  bf16x8 f;
-#pragma unroll
-  for (int e = 0; e < 8; ++e) f[e] = tile[(16 * m + 8 * g + e) * pitch + col];
-  return f;
+__device__ __forceinline__ bf16x8 join(s16x4 lo, s16x4 hi) {
+  union {
+    s16x4 h[2];
+    bf16x8 f;
+  } u;
+  u.h[0] = lo, u.h[1] = hi;
+  return u.f;
+}
+// Fragment of the lane that owns tile column col0 + (lane & 31).  ACCUMULATOR order: slot e of instruction m in lane
+// group g is row 8*(2m + e/4) + 4g + e%4 (the row that accumulator register 8m + e of that lane group holds).
+__device__ __forceinline__ bf16x8 gather_acc_order(const bf16_t* tile, int pitch, int col0, int m, int lane) {
+  const int t = lane & 15, c = col0 + (lane & 16), g = lane >> 5;
+  return join(lds_transposed4(tile, pitch, 16 * m + 4 * g, c, t), lds_transposed4(tile, pitch, 16 * m + 8 + 4 * g, c, t));
+}
+// Natural order: slot e of instruction m in lane group g is row 16m + 8g + e.
+__device__ __forceinline__ bf16x8 gather_natural(const bf16_t* tile, int pitch, int col0, int m, int lane) {
+  const int t = lane & 15, c = col0 + (lane & 16), g = lane >> 5;
+  return join(lds_transposed4(tile, pitch, 16 * m + 8 * g, c, t), lds_transposed4(tile, pitch, 16 * m + 8 * g + 4, c, t));
 }
 
 // Accumulator (rows = feature dd, columns = sequence position li) -> dst[li][32*db + dd], 4 consecutive dd
@@ -227,7 +239,7 @@ __global__ __launch_bounds__(NWV * 64) void attn_fwd_small_kernel(AttnArgs a) {
     for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
 #pragma unroll
     for (int m = 0; m < 2; ++m)
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_acc_order(Vs, P, 32 * db + li, m, g), pb[m], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_acc_order(Vs, P, 32 * db, m, lane), pb[m], acc, 0, 0, 0);
     if (pr.live && qlive) store_transposed(a.o + pr.o_off + li * a.o_l, db, g, acc);
   }
 }
@@ -328,23 +340,23 @@ __global__ __launch_bounds__(NWV * 64) void attn_bwd_small_kernel(AttnArgs a) {
     for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
 #pragma unroll
     for (int m = 0; m < 2; ++m)
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_acc_order(Ks, P, 32 * db + li, m, g), dsb[m], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_acc_order(Ks, P, 32 * db, m, lane), dsb[m], acc, 0, 0, 0);
     if (store) store_transposed(a.dq + pr.qkv_off + li * a.s_l, db, g, acc);
     // dK^T[dd][key] = sum_query Q[query][dd] dS[query][key]
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
 #pragma unroll
     for (int m = 0; m < 2; ++m)
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_natural(Qs, P, 32 * db + li, m, g),
-                                                    gather_natural(DSs, kPPitch, li, m, g), acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_natural(Qs, P, 32 * db, m, lane),
+                                                    gather_natural(DSs, kPPitch, 0, m, lane), acc, 0, 0, 0);
     if (store) store_transposed(a.dk + pr.qkv_off + li * a.s_l, db, g, acc);
     // dV^T[dd][key] = sum_query dO[query][dd] P[query][key]
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
 #pragma unroll
     for (int m = 0; m < 2; ++m)
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_natural(Gs, P, 32 * db + li, m, g),
-                                                    gather_natural(Ps, kPPitch, li, m, g), acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_natural(Gs, P, 32 * db, m, lane),
+                                                    gather_natural(Ps, kPPitch, 0, m, lane), acc, 0, 0, 0);
     if (store) store_transposed(a.dv + pr.qkv_off + li * a.s_l, db, g, acc);
   }
 }
@@ -512,7 +524,7 @@ __global__ __launch_bounds__(NWV * 64) void attn_flash_fwd_kernel(FlashArgs a) {
       for (int r = 0; r < 16; ++r) acc[db][r] *= alpha;
 #pragma unroll
       for (int m = 0; m < 2; ++m)
-        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_acc_order(Vs, P, 32 * db + li, m, g), pb[m], acc[db],
+        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_acc_order(Vs, P, 32 * db, m, lane), pb[m], acc[db],
                                                           0, 0, 0);
     }
   }
@@ -632,7 +644,7 @@ __global__ __launch_bounds__(NWV * 64) void attn_flash_dq_kernel(FlashArgs a) {
     for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int m = 0; m < 2; ++m)
-        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_acc_order(Ks, P, 32 * db + li, m, g), dsb[m], acc[db],
+        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_acc_order(Ks, P, 32 * db, m, lane), dsb[m], acc[db],
                                                           0, 0, 0);
   }
   if (it.live && qlive) {
@@ -720,10 +732,10 @@ __global__ __launch_bounds__(NWV * 64) void attn_flash_dkv_kernel(FlashArgs a) {
 #pragma unroll
       for (int m = 0; m < 2; ++m) {
         // dK^T[dd][key] += sum_query Q[query][dd] dS[query][key];  dV^T[dd][key] += sum_query dO[query][dd] P[query][key]
-        dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_natural(Qs, P, 32 * db + li, m, g),
-                                                         gather_natural(DSs, kPPitch, li, m, g), dk[db], 0, 0, 0);
-        dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_natural(Gs, P, 32 * db + li, m, g),
-                                                         gather_natural(Ps, kPPitch, li, m, g), dv[db], 0, 0, 0);
+        dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_natural(Qs, P, 32 * db, m, lane),
+                                                         gather_natural(DSs, kPPitch, 0, m, lane), dk[db], 0, 0, 0);
+        dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_natural(Gs, P, 32 * db, m, lane),
+                                                         gather_natural(Ps, kPPitch, 0, m, lane), dv[db], 0, 0, 0);
       }
     }
   }
