@@ -367,6 +367,12 @@ __global__ __launch_bounds__(NWV * 64) void attn_bwd_small_kernel(AttnArgs a) {
 // recomputes the probabilities from it, once in a pass that owns a query block (dQ, and the row dot products
 // delta = sum_d dO*O) and once in a pass that owns a key block (dK, dV): no atomics, fixed summation order.
 // A wave works on its own LDS tiles and never meets another wave, so block counts may differ per wave (causal).
+//
+// The loops are bound by vector-ALU issue, not by the matrix cores (16 scores per lane and block against 8 MFMAs
+// at D = 64), so the per-score work is kept to a handful of instructions: scores live in the log2 domain
+// (scale * log2(e) folded into one FMA, the hardware 2^x), visibility tests only run in blocks that touch the
+// end of the sequence or the causal diagonal, the running output is rescaled only when some query's maximum
+// moved, and the loop-invariant operand fragments stay in registers.
 struct FlashArgs {
   const bf16_t *q, *k, *v;
   bf16_t *dq, *dk, *dv;
@@ -380,8 +386,11 @@ struct FlashArgs {
   int causal;
   float scale;
   int L, N, H, nblk;  // nblk = ceil(L / 32)
-  long nprob;         // G * N * H
+  int nprob;          // G * N * H; nprob * nblk < 2^31
 };
+
+constexpr float kLog2e = 1.44269504088896340736f;
+constexpr float kLn2 = 0.69314718055994530942f;
 
 // Orders a wave's LDS writes before its own later LDS reads of other lanes' data (no instruction is needed for
 // that, the LDS serves a wave's accesses in order; this keeps the compiler from reordering them).
@@ -392,45 +401,105 @@ __device__ __forceinline__ void wave_sync() {
 }
 
 struct FlashItem {
-  long z, qkv_off, o_off;
-  int blk;
+  int z, blk;
+  long qkv_off, o_off;
   bool live;
 };
-__device__ __forceinline__ FlashItem flash_locate(const FlashArgs& a, int waves_per_block) {
+// `wave` is wave-uniform (scalar), so the whole item and every base address derived from it stay in scalar registers.
+__device__ __forceinline__ FlashItem flash_locate(const FlashArgs& a, int wave, int waves_per_block) {
   FlashItem it;
-  long w = (long)blockIdx.x * waves_per_block + (threadIdx.x >> 6);
-  const long total = a.nprob * a.nblk;
+  const unsigned total = (unsigned)a.nprob * (unsigned)a.nblk;
+  unsigned w = blockIdx.x * (unsigned)waves_per_block + (unsigned)wave;
   it.live = w < total;
   if (!it.live) w = total - 1;  // idle waves redo the last item and store nothing
-  it.z = w / a.nblk;
-  it.blk = (int)(w - it.z * a.nblk);
-  const long h = it.z % a.H, b = (it.z / a.H) % a.N, g = it.z / ((long)a.H * a.N);
-  it.qkv_off = b * a.s_b + h * a.s_h + g * a.s_g;
-  it.o_off = b * a.o_b + h * a.o_h + g * a.o_g;
+  const unsigned z = w / (unsigned)a.nblk;
+  it.z = (int)z;
+  it.blk = (int)(w - z * (unsigned)a.nblk);
+  const unsigned zh = z / (unsigned)a.H, h = z - zh * (unsigned)a.H;
+  const unsigned g = zh / (unsigned)a.N, b = zh - g * (unsigned)a.N;
+  it.qkv_off = (long)b * a.s_b + (long)h * a.s_h + (long)g * a.s_g;
+  it.o_off = (long)b * a.o_b + (long)h * a.o_h + (long)g * a.o_g;
   return it;
 }
 
-// The 16 additive mask values of lane (li, g) for queries q0 + li and keys k0 + 8*(r/4) + 4*g + r%4; entries outside
-// the sequence read element 0 (their scores are discarded anyway).
-__device__ __forceinline__ void flash_mask(const FlashArgs& a, int query, int k0, int g, float (&mk)[16]) {
+// NT tiles of one 32-row block, global -> registers -> LDS like TileRegs, for a loop: the lane's byte offsets inside
+// a block are computed once (`prepare`), the block's base is a scalar, and rows beyond the sequence are redirected to
+// row 0 only in the one ragged block.
+template <int D, int NT>
+struct BlockRegs {
+  static constexpr int CPR = D / 8, NIT = kSeqMax * CPR / kWave;
+  uint4 val[NT][NIT];
+  unsigned ofs[NT][NIT];
+  __device__ __forceinline__ void prepare(const long (&s_l)[NT], int lane) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) {
+        const int c = lane + it * kWave, row = c / CPR, cc = c % CPR;
+        ofs[t][it] = (unsigned)((row * s_l[t] + cc * 8) * (long)sizeof(bf16_t));
+      }
+  }
+  __device__ __forceinline__ void fetch(const bf16_t* const (&base)[NT], int rows, int lane) {
+    if (rows >= kSeqMax) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int it = 0; it < NIT; ++it)
+          val[t][it] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(base[t]) + ofs[t][it]);
+    } else {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+          const int c = lane + it * kWave, row = c / CPR, cc = c % CPR;
+          const unsigned o = row < rows ? ofs[t][it] : (unsigned)(cc * 8 * sizeof(bf16_t));
+          val[t][it] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(base[t]) + o);
+        }
+    }
+  }
+  __device__ __forceinline__ void commit(bf16_t* const (&tile)[NT], int rows, int lane) const {
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) {
+        const int c = lane + it * kWave, row = c / CPR, cc = c % CPR;
+        *reinterpret_cast<uint4*>(tile[t] + row * (D + 8) + cc * 8) = row < rows ? val[t][it] : make_uint4(0u, 0u, 0u, 0u);
+      }
+  }
+};
+
+// The 16 additive mask values of lane (li, g), times log2(e), for one query and the keys k0 + 8*(r/4) + 4*g + r%4
+// (`keys_in_regs`), or for one key and the queries q0 + 8*(r/4) + 4*g + r%4; entries outside the sequence read
+// element 0 (their scores are discarded anyway).
+template <bool KEYS_IN_REGS>
+__device__ __forceinline__ void flash_mask(const FlashArgs& a, int mine, int base, int g, float (&mk)[16]) {
 #pragma unroll
   for (int r = 0; r < 16; ++r) mk[r] = 0.0f;
   if (!a.mask) return;
-  if (a.L % 4 == 0 && reinterpret_cast<uintptr_t>(a.mask) % 16 == 0) {
+  if (KEYS_IN_REGS && a.L % 4 == 0 && reinterpret_cast<uintptr_t>(a.mask) % 16 == 0) {
 #pragma unroll
     for (int a4 = 0; a4 < 4; ++a4) {
-      const int key0 = k0 + 8 * a4 + 4 * g;
+      const int key0 = base + 8 * a4 + 4 * g;
       const float4 m4 =
-          *reinterpret_cast<const float4*>(a.mask + ((query < a.L && key0 < a.L) ? (long)query * a.L + key0 : 0));
+          *reinterpret_cast<const float4*>(a.mask + ((mine < a.L && key0 < a.L) ? (long)mine * a.L + key0 : 0));
       mk[4 * a4 + 0] = m4.x, mk[4 * a4 + 1] = m4.y, mk[4 * a4 + 2] = m4.z, mk[4 * a4 + 3] = m4.w;
     }
   } else {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const int key = k0 + 8 * (r >> 2) + 4 * g + (r & 3);
-      mk[r] = a.mask[(query < a.L && key < a.L) ? (long)query * a.L + key : 0];
+      const int other = base + 8 * (r >> 2) + 4 * g + (r & 3);
+      const long at = KEYS_IN_REGS ? (long)mine * a.L + other : (long)other * a.L + mine;
+      mk[r] = a.mask[(mine < a.L && other < a.L) ? at : 0];
     }
   }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) mk[r] *= kLog2e;
+}
+
+template <int D>
+__device__ __forceinline__ void load_frags(const bf16_t* tile, int li, int g, bf16x8 (&f)[D / 16]) {
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ++ks) f[ks] = frag_rowmajor(tile, D + 8, li, g, ks);
 }
 
 template <int DB, int NWV>
@@ -438,35 +507,44 @@ __global__ __launch_bounds__(NWV * 64) void attn_flash_fwd_kernel(FlashArgs a) {
   touch_kernel_arguments<sizeof(FlashArgs)>();
   constexpr int D = 32 * DB, P = D + 8;
   constexpr bool PREFETCH = DB <= 2;  // next block's K / V in registers while this one is worked on
-  __shared__ __attribute__((aligned(16))) bf16_t tiles[NWV][3][kSeqMax * P];
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, li = lane & 31, g = lane >> 5;
-  const FlashItem it = flash_locate(a, NWV);
+  __shared__ __attribute__((aligned(16))) bf16_t tiles[NWV][2][kSeqMax * P];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63, li = lane & 31, g = lane >> 5;
+  const FlashItem it = flash_locate(a, wave, NWV);
   const int qb = a.nblk - 1 - it.blk;  // the long (causal) items first
   const int q0 = qb * kSeqMax, query = q0 + li;
   const bool qlive = query < a.L;
-  bf16_t* Qs = tiles[wave][0];
-  bf16_t* Ks = tiles[wave][1];
-  bf16_t* Vs = tiles[wave][2];
+  bf16_t* Ks = tiles[wave][0];
+  bf16_t* Vs = tiles[wave][1];
   const long kv_step = (long)kSeqMax * a.s_l;
   const bf16_t* kbase = a.k + it.qkv_off;
   const bf16_t* vbase = a.v + it.qkv_off;
+  BlockRegs<D, 2> rkv;
   {
-    TileRegs<D, 1> rq;
-    const bf16_t* const src[1] = {a.q + it.qkv_off + (long)q0 * a.s_l};
+    const long sl2[2] = {a.s_l, a.s_l};
+    rkv.prepare(sl2, lane);
+  }
+  bf16_t* const tl2[2] = {Ks, Vs};
+  // the query block's fragments stay in registers; its tile only passes through the K tile's place
+  bf16x8 qf[D / 16];
+  {
+    BlockRegs<D, 1> rq;
     const long sl[1] = {a.s_l};
-    rq.fetch(src, sl, a.L - q0, lane);
-    bf16_t* const tl[1] = {Qs};
+    rq.prepare(sl, lane);
+    const bf16_t* const src[1] = {a.q + it.qkv_off + (long)q0 * a.s_l};
+    bf16_t* const tl[1] = {Ks};
+    rq.fetch(src, a.L - q0, lane);
     rq.commit(tl, a.L - q0, lane);
+    wave_sync();
+    load_frags<D>(Ks, li, g, qf);
   }
   const int kb_end = a.causal ? qb : a.nblk - 1;
-  TileRegs<D, 2> rkv;
-  const long sl2[2] = {a.s_l, a.s_l};
-  bf16_t* const tl2[2] = {Ks, Vs};
   if (PREFETCH) {
     const bf16_t* const src[2] = {kbase, vbase};
-    rkv.fetch(src, sl2, a.L, lane);
+    rkv.fetch(src, a.L, lane);
   }
-  float m_run = -INFINITY, l_run = 0.0f;
+  const float scale2 = a.scale * kLog2e;
+  float m_run = -INFINITY, l_run = 0.0f;  // running maximum (log2 domain) and sum
   f32x16 acc[DB];
 #pragma unroll
   for (int db = 0; db < DB; ++db)
@@ -476,40 +554,45 @@ __global__ __launch_bounds__(NWV * 64) void attn_flash_fwd_kernel(FlashArgs a) {
     const int k0 = kb * kSeqMax;
     if (!PREFETCH) {
       const bf16_t* const src[2] = {kbase + kb * kv_step, vbase + kb * kv_step};
-      rkv.fetch(src, sl2, a.L - k0, lane);
+      rkv.fetch(src, a.L - k0, lane);
     }
     wave_sync();  // the previous block's fragment reads are done
     rkv.commit(tl2, a.L - k0, lane);
     wave_sync();
     if (PREFETCH && kb < kb_end) {
       const bf16_t* const src[2] = {kbase + (kb + 1) * kv_step, vbase + (kb + 1) * kv_step};
-      rkv.fetch(src, sl2, a.L - k0 - kSeqMax, lane);
+      rkv.fetch(src, a.L - k0 - kSeqMax, lane);
     }
     float mk[16];
-    flash_mask(a, query, k0, g, mk);
+    flash_mask<true>(a, query, k0, g, mk);
     f32x16 s;
 #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = 0.0f;
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks)
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rowmajor(Ks, P, li, g, ks), frag_rowmajor(Qs, P, li, g, ks), s,
-                                                  0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rowmajor(Ks, P, li, g, ks), qf[ks], s, 0, 0, 0);
     float val[16];
-    float bm = -INFINITY;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int key = k0 + 8 * (r >> 2) + 4 * g + (r & 3);
-      const bool visible = key < a.L && (!a.causal || key <= query);
-      val[r] = visible ? s[r] * a.scale + mk[r] : -INFINITY;
-      bm = fmaxf(bm, val[r]);
+    for (int r = 0; r < 16; ++r) val[r] = fmaf(s[r], scale2, mk[r]);
+    if (k0 + kSeqMax > a.L || (a.causal && kb == qb)) {  // wave-uniform: only these blocks hold hidden keys
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = k0 + 8 * (r >> 2) + 4 * g + (r & 3);
+        const bool visible = key < a.L && (!a.causal || key <= query);
+        val[r] = visible ? val[r] : -INFINITY;
+      }
     }
+    float bm = val[0];
+#pragma unroll
+    for (int r = 1; r < 16; ++r) bm = fmaxf(bm, val[r]);
     bm = fmaxf(bm, __shfl_xor(bm, 32, kWave));
     const float m_new = fmaxf(m_run, bm);
-    const float alpha = m_run == -INFINITY ? 0.0f : expf(m_run - m_new);
+    const float m_ref = m_new == -INFINITY ? 0.0f : m_new;  // everything hidden so far: 2^(-inf - 0) = 0 all round
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
     float rs = 0.0f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      val[r] = val[r] == -INFINITY ? 0.0f : expf(val[r] - m_new);
+      val[r] = __builtin_amdgcn_exp2f(val[r] - m_ref);
       rs += val[r];
     }
     rs += __shfl_xor(rs, 32, kWave);
@@ -518,15 +601,18 @@ __global__ __launch_bounds__(NWV * 64) void attn_flash_fwd_kernel(FlashArgs a) {
     bf16x8 pb[2];
 #pragma unroll
     for (int r = 0; r < 16; ++r) pb[r >> 3][r & 7] = from_f32<bf16_t>(val[r]);
+    if (__any(alpha != 1.0f)) {
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
+      for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[db][r] *= alpha;
+        for (int r = 0; r < 16; ++r) acc[db][r] *= alpha;
+    }
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int m = 0; m < 2; ++m)
-        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_acc_order(Vs, P, 32 * db, m, lane), pb[m], acc[db],
-                                                          0, 0, 0);
-    }
+        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_acc_order(Vs, P, 32 * db, m, lane), pb[m], acc[db], 0,
+                                                          0, 0);
   }
   const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
   if (it.live && qlive) {
@@ -536,36 +622,34 @@ __global__ __launch_bounds__(NWV * 64) void attn_flash_fwd_kernel(FlashArgs a) {
       for (int r = 0; r < 16; ++r) acc[db][r] *= inv;
       store_transposed(a.o + it.o_off + (long)query * a.o_l, db, g, acc[db]);
     }
-    if (g == 0) a.lse[it.z * a.L + query] = l_run > 0.0f ? m_run + logf(l_run) : 0.0f;
+    if (g == 0) a.lse[(long)it.z * a.L + query] = l_run > 0.0f ? (m_run + __builtin_amdgcn_logf(l_run)) * kLn2 : 0.0f;
   }
 }
 
-// Recomputed probabilities and score gradients of one (query block, key block) pair, lane (li, g) = query q0 + li:
-// p[r] = exp(scale * s + mask - lse), ds[r] = scale * p * (dp - delta) for the 16 keys of the lane.
-template <int D>
-__device__ __forceinline__ void flash_p_ds(const FlashArgs& a, const bf16_t* Qs, const bf16_t* Ks, const bf16_t* Vs,
-                                           const bf16_t* Gs, int query, int k0, int li, int g, float lse, float delta,
-                                           float (&pv)[16], float (&ds)[16]) {
-  constexpr int P = D + 8;
-  float mk[16];
-  flash_mask(a, query, k0, g, mk);
-  f32x16 s, dp;
+// Recomputed probabilities and score gradients of one (query block, key block) pair from the two accumulators
+// s (scores) and dp: p[r] = 2^(scale2 * s + mask2 - lse2), ds[r] = p * (scale * dp - scale * delta).  lse2 / sdelta
+// are per lane (KEYS_IN_REGS: the lane is a query) or per register (the lane is a key, registers run over queries).
+struct FlashRowStats {
+  float lse2, sdelta;  // log-sum-exp * log2(e), scale * delta
+};
+template <bool KEYS_IN_REGS>
+__device__ __forceinline__ void flash_p_ds(const FlashArgs& a, const f32x16& s, const f32x16& dp, const float (&mk)[16],
+                                           float scale2, int mine, int base, int g, bool edge,
+                                           const FlashRowStats (&st)[KEYS_IN_REGS ? 1 : 16], float (&pv)[16],
+                                           float (&ds)[16]) {
 #pragma unroll
-  for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.0f;
+  for (int r = 0; r < 16; ++r) pv[r] = __builtin_amdgcn_exp2f(fmaf(s[r], scale2, mk[r]) - st[KEYS_IN_REGS ? 0 : r].lse2);
+  if (edge) {
 #pragma unroll
-  for (int ks = 0; ks < D / 16; ++ks) {
-    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rowmajor(Ks, P, li, g, ks), frag_rowmajor(Qs, P, li, g, ks), s, 0,
-                                                0, 0);
-    dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rowmajor(Vs, P, li, g, ks), frag_rowmajor(Gs, P, li, g, ks), dp,
-                                                 0, 0, 0);
+    for (int r = 0; r < 16; ++r) {
+      const int other = base + 8 * (r >> 2) + 4 * g + (r & 3);
+      const int query = KEYS_IN_REGS ? mine : other, key = KEYS_IN_REGS ? other : mine;
+      const bool visible = query < a.L && key < a.L && (!a.causal || key <= query);
+      pv[r] = visible ? pv[r] : 0.0f;
+    }
   }
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int key = k0 + 8 * (r >> 2) + 4 * g + (r & 3);
-    const bool visible = query < a.L && key < a.L && (!a.causal || key <= query);
-    pv[r] = visible ? expf(s[r] * a.scale + mk[r] - lse) : 0.0f;
-    ds[r] = a.scale * pv[r] * (dp[r] - delta);
-  }
+  for (int r = 0; r < 16; ++r) ds[r] = pv[r] * fmaf(dp[r], a.scale, -st[KEYS_IN_REGS ? 0 : r].sdelta);
 }
 
 template <int DB, int NWV>
@@ -573,49 +657,65 @@ __global__ __launch_bounds__(NWV * 64) void attn_flash_dq_kernel(FlashArgs a) {
   touch_kernel_arguments<sizeof(FlashArgs)>();
   constexpr int D = 32 * DB, P = D + 8;
   constexpr bool PREFETCH = DB <= 2;
-  __shared__ __attribute__((aligned(16))) bf16_t tiles[NWV][4][kSeqMax * P];
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, li = lane & 31, g = lane >> 5;
-  const FlashItem it = flash_locate(a, NWV);
+  __shared__ __attribute__((aligned(16))) bf16_t tiles[NWV][2][kSeqMax * P];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63, li = lane & 31, g = lane >> 5;
+  const FlashItem it = flash_locate(a, wave, NWV);
   const int qb = a.nblk - 1 - it.blk;
   const int q0 = qb * kSeqMax, query = q0 + li;
   const bool qlive = query < a.L;
-  bf16_t* Qs = tiles[wave][0];
-  bf16_t* Ks = tiles[wave][1];
-  bf16_t* Vs = tiles[wave][2];
-  bf16_t* Gs = tiles[wave][3];  // dO
+  bf16_t* Ks = tiles[wave][0];
+  bf16_t* Vs = tiles[wave][1];
   const long kv_step = (long)kSeqMax * a.s_l;
   const bf16_t* kbase = a.k + it.qkv_off;
   const bf16_t* vbase = a.v + it.qkv_off;
-  {
-    // Q, dO and (in the K tile's place) O of the query block; delta = sum_d dO * O per query
-    TileRegs<D, 3> r3;
-    const bf16_t* const src[3] = {a.q + it.qkv_off + (long)q0 * a.s_l, a.dout + it.o_off + (long)q0 * a.o_l,
-                                  a.o + it.o_off + (long)q0 * a.o_l};
-    const long sl[3] = {a.s_l, a.o_l, a.o_l};
-    r3.fetch(src, sl, a.L - q0, lane);
-    bf16_t* const tl[3] = {Qs, Gs, Ks};
-    r3.commit(tl, a.L - q0, lane);
-  }
-  wave_sync();
-  float delta = 0.0f;
-#pragma unroll
-  for (int c = 0; c < D / 2; c += 8) {
-    const bf16x8 gv = *reinterpret_cast<const bf16x8*>(Gs + li * P + g * (D / 2) + c);
-    const bf16x8 ov = *reinterpret_cast<const bf16x8*>(Ks + li * P + g * (D / 2) + c);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) delta += to_f32(gv[e]) * to_f32(ov[e]);
-  }
-  delta += __shfl_xor(delta, 32, kWave);
-  if (it.live && qlive && g == 0) a.delta[it.z * a.L + query] = delta;
-  const float lse = a.lse[it.z * a.L + (qlive ? query : 0)];
-  const int kb_end = a.causal ? qb : a.nblk - 1;
-  TileRegs<D, 2> rkv;
-  const long sl2[2] = {a.s_l, a.s_l};
   bf16_t* const tl2[2] = {Ks, Vs};
+  // Q and dO fragments of the query block stay in registers; dO and O pass through the tiles for delta
+  bf16x8 qf[D / 16], gf[D / 16];
+  float delta = 0.0f;
+  {
+    BlockRegs<D, 2> rgo;
+    const long sl[2] = {a.o_l, a.o_l};
+    rgo.prepare(sl, lane);
+    const bf16_t* const src[2] = {a.dout + it.o_off + (long)q0 * a.o_l, a.o + it.o_off + (long)q0 * a.o_l};
+    rgo.fetch(src, a.L - q0, lane);
+    rgo.commit(tl2, a.L - q0, lane);
+    wave_sync();
+    load_frags<D>(Ks, li, g, gf);
+#pragma unroll
+    for (int c = 0; c < D / 2; c += 8) {
+      const bf16x8 gv = *reinterpret_cast<const bf16x8*>(Ks + li * P + g * (D / 2) + c);
+      const bf16x8 ov = *reinterpret_cast<const bf16x8*>(Vs + li * P + g * (D / 2) + c);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) delta += to_f32(gv[e]) * to_f32(ov[e]);
+    }
+    delta += __shfl_xor(delta, 32, kWave);
+    if (it.live && qlive && g == 0) a.delta[(long)it.z * a.L + query] = delta;
+  }
+  BlockRegs<D, 2> rkv;
+  {
+    const long sl2[2] = {a.s_l, a.s_l};
+    rkv.prepare(sl2, lane);
+    BlockRegs<D, 1> rq;
+    const long sl[1] = {a.s_l};
+    rq.prepare(sl, lane);
+    const bf16_t* const src[1] = {a.q + it.qkv_off + (long)q0 * a.s_l};
+    bf16_t* const tl[1] = {Ks};
+    rq.fetch(src, a.L - q0, lane);
+    wave_sync();  // the delta reads are done
+    rq.commit(tl, a.L - q0, lane);
+    wave_sync();
+    load_frags<D>(Ks, li, g, qf);
+  }
+  FlashRowStats st[1];
+  st[0].lse2 = a.lse[(long)it.z * a.L + (qlive ? query : 0)] * kLog2e;
+  st[0].sdelta = a.scale * delta;
+  const int kb_end = a.causal ? qb : a.nblk - 1;
   if (PREFETCH) {
     const bf16_t* const src[2] = {kbase, vbase};
-    rkv.fetch(src, sl2, a.L, lane);
+    rkv.fetch(src, a.L, lane);
   }
+  const float scale2 = a.scale * kLog2e;
   f32x16 acc[DB];
 #pragma unroll
   for (int db = 0; db < DB; ++db)
@@ -625,17 +725,28 @@ __global__ __launch_bounds__(NWV * 64) void attn_flash_dq_kernel(FlashArgs a) {
     const int k0 = kb * kSeqMax;
     if (!PREFETCH) {
       const bf16_t* const src[2] = {kbase + kb * kv_step, vbase + kb * kv_step};
-      rkv.fetch(src, sl2, a.L - k0, lane);
+      rkv.fetch(src, a.L - k0, lane);
     }
     wave_sync();
     rkv.commit(tl2, a.L - k0, lane);
     wave_sync();
     if (PREFETCH && kb < kb_end) {
       const bf16_t* const src[2] = {kbase + (kb + 1) * kv_step, vbase + (kb + 1) * kv_step};
-      rkv.fetch(src, sl2, a.L - k0 - kSeqMax, lane);
+      rkv.fetch(src, a.L - k0 - kSeqMax, lane);
     }
+    float mk[16];
+    flash_mask<true>(a, query, k0, g, mk);
+    f32x16 s, dp;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.0f;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rowmajor(Ks, P, li, g, ks), qf[ks], s, 0, 0, 0);
+      dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rowmajor(Vs, P, li, g, ks), gf[ks], dp, 0, 0, 0);
+    }
+    const bool edge = q0 + kSeqMax > a.L || k0 + kSeqMax > a.L || (a.causal && kb == qb);
     float pv[16], ds[16];
-    flash_p_ds<D>(a, Qs, Ks, Vs, Gs, query, k0, li, g, lse, delta, pv, ds);
+    flash_p_ds<true>(a, s, dp, mk, scale2, query, k0, g, edge, st, pv, ds);
     bf16x8 dsb[2];
 #pragma unroll
     for (int r = 0; r < 16; ++r) dsb[r >> 3][r & 7] = from_f32<bf16_t>(ds[r]);
@@ -644,8 +755,8 @@ __global__ __launch_bounds__(NWV * 64) void attn_flash_dq_kernel(FlashArgs a) {
     for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int m = 0; m < 2; ++m)
-        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_acc_order(Ks, P, 32 * db, m, lane), dsb[m], acc[db],
-                                                          0, 0, 0);
+        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_acc_order(Ks, P, 32 * db, m, lane), dsb[m], acc[db], 0,
+                                                          0, 0);
   }
   if (it.live && qlive) {
 #pragma unroll
@@ -653,97 +764,130 @@ __global__ __launch_bounds__(NWV * 64) void attn_flash_dq_kernel(FlashArgs a) {
   }
 }
 
+// Key-block pass.  Scores are formed as S[query][key] (A = Q rows, B = K rows), so a lane is a KEY and its 16
+// accumulator registers run over the queries of the block: P and dS are then, as they stand, the B operands
+// "lane = key, slots = queries" of dV^T = dO^T P and dK^T = Q^T dS, and the per-query statistics come in as 16
+// values per lane.
 template <int DB, int NWV>
 __global__ __launch_bounds__(NWV * 64) void attn_flash_dkv_kernel(FlashArgs a) {
   touch_kernel_arguments<sizeof(FlashArgs)>();
   constexpr int D = 32 * DB, P = D + 8;
   constexpr bool PREFETCH = DB <= 2;
-  __shared__ __attribute__((aligned(16))) bf16_t tiles[NWV][4][kSeqMax * P];
-  __shared__ __attribute__((aligned(16))) bf16_t ptiles[NWV][2][kSeqMax * kPPitch];
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, li = lane & 31, g = lane >> 5;
-  const FlashItem it = flash_locate(a, NWV);
+  __shared__ __attribute__((aligned(16))) bf16_t tiles[NWV][2][kSeqMax * P];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63, li = lane & 31, g = lane >> 5;
+  const FlashItem it = flash_locate(a, wave, NWV);
   const int kb = it.blk;  // causal: key block 0 meets every query block, so the long items come first
-  const int k0 = kb * kSeqMax, key_row = k0 + li;
+  const int k0 = kb * kSeqMax, key = k0 + li;
   bf16_t* Qs = tiles[wave][0];
-  bf16_t* Ks = tiles[wave][1];
-  bf16_t* Vs = tiles[wave][2];
-  bf16_t* Gs = tiles[wave][3];  // dO
-  bf16_t* DSs = ptiles[wave][0];
-  bf16_t* Ps = ptiles[wave][1];
+  bf16_t* Gs = tiles[wave][1];  // dO
+  bf16_t* const tl2[2] = {Qs, Gs};
+  // K and V fragments of the key block stay in registers; their tiles pass through the Q / dO tiles' place
+  bf16x8 kf[D / 16], vf[D / 16];
   {
-    TileRegs<D, 2> r2;
-    const bf16_t* const src[2] = {a.k + it.qkv_off + (long)k0 * a.s_l, a.v + it.qkv_off + (long)k0 * a.s_l};
+    BlockRegs<D, 2> rkv;
     const long sl[2] = {a.s_l, a.s_l};
-    r2.fetch(src, sl, a.L - k0, lane);
-    bf16_t* const tl[2] = {Ks, Vs};
-    r2.commit(tl, a.L - k0, lane);
+    rkv.prepare(sl, lane);
+    const bf16_t* const src[2] = {a.k + it.qkv_off + (long)k0 * a.s_l, a.v + it.qkv_off + (long)k0 * a.s_l};
+    rkv.fetch(src, a.L - k0, lane);
+    rkv.commit(tl2, a.L - k0, lane);
+    wave_sync();
+    load_frags<D>(Qs, li, g, kf);
+    load_frags<D>(Gs, li, g, vf);
   }
   const int qb_start = a.causal ? kb : 0;
   const long q_step = (long)kSeqMax * a.s_l, g_step = (long)kSeqMax * a.o_l;
   const bf16_t* qbase = a.q + it.qkv_off;
   const bf16_t* gbase = a.dout + it.o_off;
-  TileRegs<D, 2> rqg;
-  const long sl2[2] = {a.s_l, a.o_l};
-  bf16_t* const tl2[2] = {Qs, Gs};
+  const float* lse_row = a.lse + (long)it.z * a.L;
+  const float* delta_row = a.delta + (long)it.z * a.L;
+  // queries come in runs of 4: with L % 4 == 0 whole runs are inside or outside the sequence (16-byte loads)
+  const bool stat_quads = a.L % 4 == 0 && (reinterpret_cast<uintptr_t>(a.lse) | reinterpret_cast<uintptr_t>(a.delta)) % 16 == 0;
+  BlockRegs<D, 2> rqg;
+  {
+    const long sl2[2] = {a.s_l, a.o_l};
+    rqg.prepare(sl2, lane);
+  }
   if (PREFETCH) {
     const bf16_t* const src[2] = {qbase + qb_start * q_step, gbase + qb_start * g_step};
-    rqg.fetch(src, sl2, a.L - qb_start * kSeqMax, lane);
+    rqg.fetch(src, a.L - qb_start * kSeqMax, lane);
   }
+  const float scale2 = a.scale * kLog2e;
   f32x16 dk[DB], dv[DB];
 #pragma unroll
   for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int r = 0; r < 16; ++r) dk[db][r] = dv[db][r] = 0.0f;
   for (int qb = qb_start; qb < a.nblk; ++qb) {
-    const int q0 = qb * kSeqMax, query = q0 + li;
+    const int q0 = qb * kSeqMax;
     if (!PREFETCH) {
       const bf16_t* const src[2] = {qbase + qb * q_step, gbase + qb * g_step};
-      rqg.fetch(src, sl2, a.L - q0, lane);
+      rqg.fetch(src, a.L - q0, lane);
     }
-    wave_sync();  // the previous block's gathers are done
+    // statistics of the 16 queries of this lane's registers (the same for every key: broadcast loads)
+    float lse_q[16], delta_q[16];
+    if (stat_quads) {
+#pragma unroll
+      for (int a4 = 0; a4 < 4; ++a4) {
+        const int query0 = q0 + 8 * a4 + 4 * g;
+        const float4 l4 = *reinterpret_cast<const float4*>(lse_row + (query0 < a.L ? query0 : 0));
+        const float4 d4 = *reinterpret_cast<const float4*>(delta_row + (query0 < a.L ? query0 : 0));
+        lse_q[4 * a4 + 0] = l4.x, lse_q[4 * a4 + 1] = l4.y, lse_q[4 * a4 + 2] = l4.z, lse_q[4 * a4 + 3] = l4.w;
+        delta_q[4 * a4 + 0] = d4.x, delta_q[4 * a4 + 1] = d4.y, delta_q[4 * a4 + 2] = d4.z, delta_q[4 * a4 + 3] = d4.w;
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int query = q0 + 8 * (r >> 2) + 4 * g + (r & 3);
+        lse_q[r] = lse_row[query < a.L ? query : 0];
+        delta_q[r] = delta_row[query < a.L ? query : 0];
+      }
+    }
+    wave_sync();  // the previous block's reads are done
     rqg.commit(tl2, a.L - q0, lane);
     wave_sync();
     if (PREFETCH && qb + 1 < a.nblk) {
       const bf16_t* const src[2] = {qbase + (qb + 1) * q_step, gbase + (qb + 1) * g_step};
-      rqg.fetch(src, sl2, a.L - q0 - kSeqMax, lane);
+      rqg.fetch(src, a.L - q0 - kSeqMax, lane);
     }
-    const long qi = it.z * a.L + (query < a.L ? query : 0);
-    const float lse = a.lse[qi], delta = a.delta[qi];
+    float mk[16];
+    flash_mask<false>(a, key, q0, g, mk);
+    f32x16 s, dp;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.0f;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rowmajor(Qs, P, li, g, ks), kf[ks], s, 0, 0, 0);
+      dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rowmajor(Gs, P, li, g, ks), vf[ks], dp, 0, 0, 0);
+    }
+    FlashRowStats st[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) st[r].lse2 = lse_q[r] * kLog2e, st[r].sdelta = delta_q[r] * a.scale;
+    const bool edge = q0 + kSeqMax > a.L || k0 + kSeqMax > a.L || (a.causal && kb == qb);
     float pv[16], ds[16];
-    flash_p_ds<D>(a, Qs, Ks, Vs, Gs, query, k0, li, g, lse, delta, pv, ds);
-    // dS and P as [query][key] tiles for the products that contract over the queries
+    flash_p_ds<false>(a, s, dp, mk, scale2, key, q0, g, edge, st, pv, ds);
+    bf16x8 pb[2], dsb[2];
 #pragma unroll
-    for (int a4 = 0; a4 < 4; ++a4) {
-      union {
-        uint2 u;
-        bf16_t e[4];
-      } d4, p4;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        d4.e[e] = from_f32<bf16_t>(ds[4 * a4 + e]);
-        p4.e[e] = from_f32<bf16_t>(pv[4 * a4 + e]);
-      }
-      *reinterpret_cast<uint2*>(DSs + li * kPPitch + 8 * a4 + 4 * g) = d4.u;
-      *reinterpret_cast<uint2*>(Ps + li * kPPitch + 8 * a4 + 4 * g) = p4.u;
+    for (int r = 0; r < 16; ++r) {
+      pb[r >> 3][r & 7] = from_f32<bf16_t>(pv[r]);
+      dsb[r >> 3][r & 7] = from_f32<bf16_t>(ds[r]);
     }
-    wave_sync();
+    // dK^T[dd][key] += sum_query Q[query][dd] dS[query][key];  dV^T[dd][key] += sum_query dO[query][dd] P[query][key]
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
+    for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int m = 0; m < 2; ++m) {
-        // dK^T[dd][key] += sum_query Q[query][dd] dS[query][key];  dV^T[dd][key] += sum_query dO[query][dd] P[query][key]
-        dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_natural(Qs, P, 32 * db, m, lane),
-                                                         gather_natural(DSs, kPPitch, 0, m, lane), dk[db], 0, 0, 0);
-        dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_natural(Gs, P, 32 * db, m, lane),
-                                                         gather_natural(Ps, kPPitch, 0, m, lane), dv[db], 0, 0, 0);
+        dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_acc_order(Qs, P, 32 * db, m, lane), dsb[m], dk[db], 0, 0,
+                                                         0);
+        dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gather_acc_order(Gs, P, 32 * db, m, lane), pb[m], dv[db], 0, 0,
+                                                         0);
       }
-    }
   }
-  if (it.live && key_row < a.L) {
+  if (it.live && key < a.L) {
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
-      store_transposed(a.dk + it.qkv_off + (long)key_row * a.s_l, db, g, dk[db]);
-      store_transposed(a.dv + it.qkv_off + (long)key_row * a.s_l, db, g, dv[db]);
+      store_transposed(a.dk + it.qkv_off + (long)key * a.s_l, db, g, dk[db]);
+      store_transposed(a.dv + it.qkv_off + (long)key * a.s_l, db, g, dv[db]);
     }
   }
 }
@@ -839,7 +983,7 @@ extern "C" int rtp_attn_flash_supported(int dtype, int64_t L, int64_t D) {
 
 template <template <int, int> class Launcher>
 static int flash_dispatch(int64_t D, const FlashArgs& a, hipStream_t st) {
-  const long items = a.nprob * a.nblk;
+  const long items = (long)a.nprob * a.nblk;
   if (D == 32)
     Launcher<1, 4>::run(a, st, items);
   else if (D == 64)
@@ -867,8 +1011,10 @@ static int flash_args(const char* who, FlashArgs& a, int dtype, int64_t s_l, int
   a.s_l = s_l, a.s_b = s_b, a.s_h = s_h, a.s_g = s_g;
   a.o_l = o_l, a.o_b = o_b, a.o_h = o_h, a.o_g = o_g;
   a.mask = mask, a.causal = causal, a.scale = scale;
-  a.L = (int)L, a.N = (int)N, a.H = (int)H, a.nblk = (int)ceil_div(L, kSeqMax), a.nprob = G * N * H;
-  RTP_REQUIRE(ceil_div(a.nprob * a.nblk, 2) < (1ll << 31), "%s: too many (head, block) work items", who);
+  RTP_REQUIRE(G * N * H * ceil_div(L, kSeqMax) < (1ll << 31), "%s: too many (head, block) work items", who);
+  // a lane's byte offsets inside one 32-row block are kept in 32 bits
+  RTP_REQUIRE(s_l < (1ll << 25) && o_l < (1ll << 25) && s_l >= 0 && o_l >= 0, "%s: sequence stride out of range", who);
+  a.L = (int)L, a.N = (int)N, a.H = (int)H, a.nblk = (int)ceil_div(L, kSeqMax), a.nprob = (int)(G * N * H);
   return RTP_OK;
 }
 
