@@ -627,18 +627,16 @@ __global__ __launch_bounds__(NWV * 64) void attn_flash_fwd_kernel(FlashArgs a) {
 }
 
 // Recomputed probabilities and score gradients of one (query block, key block) pair from the two accumulators
-// s (scores) and dp: p[r] = 2^(scale2 * s + mask2 - lse2), ds[r] = p * (scale * dp - scale * delta).  lse2 / sdelta
-// are per lane (KEYS_IN_REGS: the lane is a query) or per register (the lane is a key, registers run over queries).
-struct FlashRowStats {
-  float lse2, sdelta;  // log-sum-exp * log2(e), scale * delta
-};
+// s (scores) and dp: p[r] = 2^(scale2 * s + e[r]) with e = mask * log2(e) - lse * log2(e) prepared before the
+// products, ds[r] = p * (scale * dp - sdelta) with sdelta = scale * delta per lane (KEYS_IN_REGS: the lane is a
+// query) or per register (the lane is a key, registers run over queries).
 template <bool KEYS_IN_REGS>
-__device__ __forceinline__ void flash_p_ds(const FlashArgs& a, const f32x16& s, const f32x16& dp, const float (&mk)[16],
+__device__ __forceinline__ void flash_p_ds(const FlashArgs& a, const f32x16& s, const f32x16& dp, const float (&e)[16],
                                            float scale2, int mine, int base, int g, bool edge,
-                                           const FlashRowStats (&st)[KEYS_IN_REGS ? 1 : 16], float (&pv)[16],
+                                           const float (&sdelta)[KEYS_IN_REGS ? 1 : 16], float (&pv)[16],
                                            float (&ds)[16]) {
 #pragma unroll
-  for (int r = 0; r < 16; ++r) pv[r] = __builtin_amdgcn_exp2f(fmaf(s[r], scale2, mk[r]) - st[KEYS_IN_REGS ? 0 : r].lse2);
+  for (int r = 0; r < 16; ++r) pv[r] = __builtin_amdgcn_exp2f(fmaf(s[r], scale2, e[r]));
   if (edge) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -649,7 +647,7 @@ __device__ __forceinline__ void flash_p_ds(const FlashArgs& a, const f32x16& s, 
     }
   }
 #pragma unroll
-  for (int r = 0; r < 16; ++r) ds[r] = pv[r] * fmaf(dp[r], a.scale, -st[KEYS_IN_REGS ? 0 : r].sdelta);
+  for (int r = 0; r < 16; ++r) ds[r] = pv[r] * fmaf(dp[r], a.scale, -sdelta[KEYS_IN_REGS ? 0 : r]);
 }
 
 template <int DB, int NWV>
@@ -707,9 +705,8 @@ __global__ __launch_bounds__(NWV * 64) void attn_flash_dq_kernel(FlashArgs a) {
     wave_sync();
     load_frags<D>(Ks, li, g, qf);
   }
-  FlashRowStats st[1];
-  st[0].lse2 = a.lse[(long)it.z * a.L + (qlive ? query : 0)] * kLog2e;
-  st[0].sdelta = a.scale * delta;
+  const float lse2 = a.lse[(long)it.z * a.L + (qlive ? query : 0)] * kLog2e;
+  const float sdelta[1] = {a.scale * delta};
   const int kb_end = a.causal ? qb : a.nblk - 1;
   if (PREFETCH) {
     const bf16_t* const src[2] = {kbase, vbase};
@@ -736,6 +733,8 @@ __global__ __launch_bounds__(NWV * 64) void attn_flash_dq_kernel(FlashArgs a) {
     }
     float mk[16];
     flash_mask<true>(a, query, k0, g, mk);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) mk[r] -= lse2;
     f32x16 s, dp;
 #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.0f;
@@ -746,7 +745,7 @@ __global__ __launch_bounds__(NWV * 64) void attn_flash_dq_kernel(FlashArgs a) {
     }
     const bool edge = q0 + kSeqMax > a.L || k0 + kSeqMax > a.L || (a.causal && kb == qb);
     float pv[16], ds[16];
-    flash_p_ds<true>(a, s, dp, mk, scale2, query, k0, g, edge, st, pv, ds);
+    flash_p_ds<true>(a, s, dp, mk, scale2, query, k0, g, edge, sdelta, pv, ds);
     bf16x8 dsb[2];
 #pragma unroll
     for (int r = 0; r < 16; ++r) dsb[r >> 3][r & 7] = from_f32<bf16_t>(ds[r]);
@@ -769,7 +768,7 @@ __global__ __launch_bounds__(NWV * 64) void attn_flash_dq_kernel(FlashArgs a) {
 // "lane = key, slots = queries" of dV^T = dO^T P and dK^T = Q^T dS, and the per-query statistics come in as 16
 // values per lane.
 template <int DB, int NWV>
-__global__ __launch_bounds__(NWV * 64) void attn_flash_dkv_kernel(FlashArgs a) {
+__global__ __launch_bounds__(NWV * 64) __attribute__((amdgpu_waves_per_eu(DB <= 2 ? 2 : 1))) void attn_flash_dkv_kernel(FlashArgs a) {
   touch_kernel_arguments<sizeof(FlashArgs)>();
   constexpr int D = 32 * DB, P = D + 8;
   constexpr bool PREFETCH = DB <= 2;
@@ -850,8 +849,10 @@ __global__ __launch_bounds__(NWV * 64) void attn_flash_dkv_kernel(FlashArgs a) {
       const bf16_t* const src[2] = {qbase + (qb + 1) * q_step, gbase + (qb + 1) * g_step};
       rqg.fetch(src, a.L - q0 - kSeqMax, lane);
     }
-    float mk[16];
+    float mk[16], sdelta[16];
     flash_mask<false>(a, key, q0, g, mk);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) mk[r] = fmaf(lse_q[r], -kLog2e, mk[r]), sdelta[r] = delta_q[r] * a.scale;
     f32x16 s, dp;
 #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.0f;
@@ -860,12 +861,9 @@ __global__ __launch_bounds__(NWV * 64) void attn_flash_dkv_kernel(FlashArgs a) {
       s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rowmajor(Qs, P, li, g, ks), kf[ks], s, 0, 0, 0);
       dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rowmajor(Gs, P, li, g, ks), vf[ks], dp, 0, 0, 0);
     }
-    FlashRowStats st[16];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) st[r].lse2 = lse_q[r] * kLog2e, st[r].sdelta = delta_q[r] * a.scale;
     const bool edge = q0 + kSeqMax > a.L || k0 + kSeqMax > a.L || (a.causal && kb == qb);
     float pv[16], ds[16];
-    flash_p_ds<false>(a, s, dp, mk, scale2, key, q0, g, edge, st, pv, ds);
+    flash_p_ds<false>(a, s, dp, mk, scale2, key, q0, g, edge, sdelta, pv, ds);
     bf16x8 pb[2], dsb[2];
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
