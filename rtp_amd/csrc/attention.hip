@@ -503,7 +503,7 @@ __device__ __forceinline__ void load_frags(const bf16_t* tile, int li, int g, bf
 }
 
 template <int DB, int NWV>
-__global__ __launch_bounds__(NWV * 64) void attn_flash_fwd_kernel(FlashArgs a) {
+__global__ __launch_bounds__(NWV * 64) __attribute__((amdgpu_waves_per_eu(DB <= 2 ? 3 : 1))) void attn_flash_fwd_kernel(FlashArgs a) {
   touch_kernel_arguments<sizeof(FlashArgs)>();
   constexpr int D = 32 * DB, P = D + 8;
   constexpr bool PREFETCH = DB <= 2;  // next block's K / V in registers while this one is worked on
@@ -651,10 +651,10 @@ __device__ __forceinline__ void flash_p_ds(const FlashArgs& a, const f32x16& s, 
 }
 
 template <int DB, int NWV>
-__global__ __launch_bounds__(NWV * 64) void attn_flash_dq_kernel(FlashArgs a) {
+__global__ __launch_bounds__(NWV * 64) __attribute__((amdgpu_waves_per_eu(DB <= 2 ? 3 : 1))) void attn_flash_dq_kernel(FlashArgs a) {
   touch_kernel_arguments<sizeof(FlashArgs)>();
   constexpr int D = 32 * DB, P = D + 8;
-  constexpr bool PREFETCH = DB <= 2;
+  constexpr bool PREFETCH = false;
   __shared__ __attribute__((aligned(16))) bf16_t tiles[NWV][2][kSeqMax * P];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63, li = lane & 31, g = lane >> 5;
