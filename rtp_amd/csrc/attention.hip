@@ -412,9 +412,12 @@ __device__ __forceinline__ FlashItem flash_locate(const FlashArgs& a, int wave, 
   unsigned w = blockIdx.x * (unsigned)waves_per_block + (unsigned)wave;
   it.live = w < total;
   if (!it.live) w = total - 1;  // idle waves redo the last item and store nothing
-  const unsigned z = w / (unsigned)a.nblk;
+  // Block index major: with a causal mask the items of one block index are equally long, so the grid runs from the
+  // longest items to the shortest, and the workgroups that share a CU (launch order modulo the CU count) differ in
+  // length by whole strata instead of all being long or all being short.
+  const unsigned blk = w / (unsigned)a.nprob, z = w - blk * (unsigned)a.nprob;
   it.z = (int)z;
-  it.blk = (int)(w - z * (unsigned)a.nblk);
+  it.blk = (int)blk;
   const unsigned zh = z / (unsigned)a.H, h = z - zh * (unsigned)a.H;
   const unsigned g = zh / (unsigned)a.N, b = zh - g * (unsigned)a.N;
   it.qkv_off = (long)b * a.s_b + (long)h * a.s_h + (long)g * a.s_g;
@@ -503,10 +506,10 @@ __device__ __forceinline__ void load_frags(const bf16_t* tile, int li, int g, bf
 }
 
 template <int DB, int NWV>
-__global__ __launch_bounds__(NWV * 64) __attribute__((amdgpu_waves_per_eu(DB <= 2 ? 3 : 1))) void attn_flash_fwd_kernel(FlashArgs a) {
+__global__ __launch_bounds__(NWV * 64) __attribute__((amdgpu_waves_per_eu(DB <= 2 ? 4 : 1))) void attn_flash_fwd_kernel(FlashArgs a) {
   touch_kernel_arguments<sizeof(FlashArgs)>();
   constexpr int D = 32 * DB, P = D + 8;
-  constexpr bool PREFETCH = DB <= 2;  // next block's K / V in registers while this one is worked on
+  constexpr bool PREFETCH = false;  // next block's K / V in registers while this one is worked on
   __shared__ __attribute__((aligned(16))) bf16_t tiles[NWV][2][kSeqMax * P];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63, li = lane & 31, g = lane >> 5;
