@@ -229,6 +229,9 @@ def main():
     ap.add_argument("--no-wgrad-overlap", dest="wgrad_overlap", action="store_false",
                     help="launch weight / bias gradient kernels on the compute stream instead of a second stream "
                          "beside the input-gradient chain")
+    ap.add_argument("--optimizer", default="sgd", choices=["sgd", "adam"],
+                    help="sgd: the headline configuration (default); adam: the reference harness's own optimiser "
+                         "(clip 0.05, Adam lr 1e-3), fp32 moments beside the fp32 master")
     ap.add_argument("--no-graph", dest="graph", action="store_false",
                     help="launch every kernel eagerly instead of replaying the step from a captured HIP graph")
     args = ap.parse_args()
@@ -245,14 +248,17 @@ def main():
     import torch.nn.functional as F
     from rtp_amd import _lib, ring, rotated_weight_bytes, staging_bytes
     from rtp_amd.module.loss import cross_entropy
-    from rtp_amd.optim import RotatedSGD
+    from rtp_amd.optim import RotatedAdam, RotatedSGD
 
     dev = torch.device("cuda", 0)
     ring.set_wgrad_overlap(args.wgrad_overlap)
     torch.cuda.set_device(dev)
     c = CFG
     lm = build(c, dev, torch.bfloat16)
-    opt = RotatedSGD(lm, lr=1e-3, clip_value=0.05, overlap_backward=args.sgd_overlap)
+    if args.optimizer == "adam":
+        opt = RotatedAdam(lm, lr=1e-3, clip_value=0.05)
+    else:
+        opt = RotatedSGD(lm, lr=1e-3, clip_value=0.05, overlap_backward=args.sgd_overlap)
     gen = torch.Generator().manual_seed(0)
     ids = torch.randint(0, c["vocab"], (c["seq"], c["batch"]), generator=gen).to(dev)
     tgt = torch.randint(0, c["vocab"], (c["seq"], c["batch"]), generator=gen).to(dev)
@@ -322,10 +328,11 @@ def main():
         "value": tokens / dt, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "10-layer RTP transformer LM fwd+bwd+SGD step: vocab 10240, ninp 2048, nhid 2048, "
+        "config": {"workload": f"10-layer RTP transformer LM fwd+bwd+{args.optimizer.upper()} step: vocab 10240, ninp 2048, nhid 2048, "
                                "32 heads, seq 32, batch 32, bf16 weights + fp32 master, 8 rotation shards emulated on "
                                "one GPU, uniform random token ids, weights U(-0.1,0.1), dropout 0, lr 1e-3, clip 0.05",
                    "tokens_per_step": tokens, "rotation_shards": c["shards"], "hip_graph": bool(args.graph),
+                   "optimizer": args.optimizer,
                    "sgd_overlapped_with_backward": bool(args.sgd_overlap),
                    "wgrad_on_second_stream": bool(args.wgrad_overlap)},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK["bf16_mfma_tflops"], "unit": "TFLOP/s",

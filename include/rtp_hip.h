@@ -352,6 +352,20 @@ int rtp_moe_combine_dweight(void* stream, int dtype, const void* dout, int64_t l
 int rtp_sgd_step(void* stream, int dtype, float* master, const void* grad, void* shadow, int64_t n,
                  float lr, float clip);
 
+/* Adam on a flat shard buffer (reference harness: clip_grad_value_(0.05) then torch.optim.Adam(lr 1e-3),
+ * benchmarks/rtp_benchmark.py:41-42 and :185-186), torch.optim.Adam's arithmetic without amsgrad / maximize:
+ *   g = clamp(grad, -clip, clip) if clip > 0;  g += weight_decay * master if weight_decay != 0
+ *   exp_avg += (1 - beta1) * (g - exp_avg);  exp_avg_sq = beta2 * exp_avg_sq + (1 - beta2) * g * g
+ *   master -= lr / (1 - beta1^step) * exp_avg / (sqrt(exp_avg_sq) / sqrt(1 - beta2^step) + eps)
+ *   shadow = (dtype) master
+ * master, exp_avg, exp_avg_sq fp32 (the state starts at zero, `step` counts from 1); grad and shadow `dtype`
+ * (shadow may be NULL when dtype is fp32 and the master is the weight itself).  step_dev non-NULL: the step
+ * count is read from this device location when the kernel runs and `step` is ignored, so that a launch
+ * recorded into a HIP graph follows a counter the caller advances (on the same stream, before the launch). */
+int rtp_adam_step(void* stream, int dtype, float* master, const void* grad, void* shadow, float* exp_avg,
+                  float* exp_avg_sq, int64_t n, double lr, double beta1, double beta2, double eps,
+                  double weight_decay, int64_t step, const int64_t* step_dev, double clip);
+
 /* The same update for many buffers in one launch.  `chunks` is a table in DEVICE memory, one entry per
  * workgroup: 16-byte aligned pointers into the buffers and a parameter count that is a multiple of 4 (the
  * caller cuts its buffers into chunks of, say, 16384 parameters).  total_params only feeds the profiler. */

@@ -103,6 +103,8 @@ PROTOTYPES = {
     "rtp_moe_combine": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64]),
     "rtp_moe_combine_dweight": (_i, [_vp, _i, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "rtp_sgd_step": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _f, _f]),
+    "rtp_adam_step": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i64, C.c_double, C.c_double, C.c_double, C.c_double,
+                           C.c_double, _i64, _vp, C.c_double]),
     "rtp_sgd_step_multi": (_i, [_vp, _i, _vp, _i64, _f, _f, C.c_double]),
     "rtp_cast": (_i, [_vp, _i, _vp, _i, _vp, _i64]),
     "rtp_profile_enable": (_i, [_i]),

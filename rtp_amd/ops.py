@@ -492,6 +492,32 @@ def sgd_step(master: torch.Tensor, grad: torch.Tensor, shadow: Optional[torch.Te
                                    _ptr(shadow), master.numel(), lr, clip))
 
 
+def adam_step(master: torch.Tensor, grad: torch.Tensor, shadow: Optional[torch.Tensor], exp_avg: torch.Tensor,
+              exp_avg_sq: torch.Tensor, step, lr: float, betas=(0.9, 0.999), eps: float = 1e-8,
+              weight_decay: float = 0.0, clip: float = 0.0) -> None:
+    """One torch.optim.Adam update (optionally preceded by clip_grad_value_) of a flat fp32 master buffer and
+    its fp32 moments; `shadow` receives the master rounded to the gradient's dtype.  `step` counts from 1: an int,
+    or a one-element int64 device tensor that the kernel reads when it runs (for launches recorded into a graph)."""
+    _dev(master)
+    n = master.numel()
+    for name, t in (("master", master), ("exp_avg", exp_avg), ("exp_avg_sq", exp_avg_sq)):
+        if t.dtype != torch.float32 or not t.is_contiguous() or t.numel() != n:
+            raise ValueError(f"adam_step: {name} must be contiguous fp32 of the master's length")
+    if not grad.is_contiguous() or grad.numel() != n:
+        raise ValueError("adam_step: grad must be contiguous and of the master's length")
+    if shadow is not None and (shadow.dtype != grad.dtype or shadow.numel() != n or not shadow.is_contiguous()):
+        raise ValueError("adam_step: shadow must match grad dtype and master length")
+    step_dev = None
+    if isinstance(step, torch.Tensor):
+        if step.dtype != torch.int64 or step.numel() != 1 or step.device != master.device:
+            raise ValueError("adam_step: a device step count must be one int64 element on the master's device")
+        step_dev, step = step.data_ptr(), 0
+    _lib.require_device()
+    check(_lib.load().rtp_adam_step(_stream(), dtype_code(grad.dtype), master.data_ptr(), grad.data_ptr(),
+                                    _ptr(shadow), exp_avg.data_ptr(), exp_avg_sq.data_ptr(), n, lr, betas[0],
+                                    betas[1], eps, weight_decay, int(step), step_dev, clip))
+
+
 SGD_CHUNK = 16384  # parameters per workgroup of the multi-buffer update
 
 

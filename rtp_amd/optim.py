@@ -190,3 +190,51 @@ class RotatedSGD:
                 ops.sgd_step(self.flat_master, self.flat_grad, self.flat, self.lr, self.clip_value)
         if self.stores:
             ring.fence(self.stores[0].home.device)  # staging copies of the next step must see the new weights
+
+
+class RotatedAdam(RotatedSGD):
+    """The reference harness's optimiser (benchmarks/rtp_benchmark.py:41-42: torch.optim.Adam(lr 1e-3) after
+    clip_grad_value_(0.05)) over the same flat buffers as RotatedSGD: one launch per rotated layer and one for
+    the parameters outside rotated layers, fp32 moments beside the fp32 master.  The step count lives in device
+    memory and the kernels form the bias corrections 1 - beta^step themselves, so step() may be recorded into a HIP
+    graph and replayed (`steps` then only counts the eager calls)."""
+
+    def __init__(self, model: nn.Module, lr: float = 1e-3, betas=(0.9, 0.999), eps: float = 1e-8,
+                 weight_decay: float = 0.0, clip_value: float = 0.0):
+        super().__init__(model, lr, clip_value, overlap_backward=False)
+        self.betas, self.eps, self.weight_decay = (float(betas[0]), float(betas[1])), float(eps), float(weight_decay)
+        self.steps = 0
+        self._step_dev = None
+        self._moments = {}
+
+    def state_bytes(self) -> int:
+        return sum(m.numel() * 4 + v.numel() * 4 for m, v in self._moments.values())
+
+    def _adam(self, key, weights: torch.Tensor, grads: torch.Tensor, master: Optional[torch.Tensor]) -> None:
+        target = weights if master is None else master.view(-1)
+        if key not in self._moments:
+            self._moments[key] = (torch.zeros_like(target), torch.zeros_like(target))
+        m, v = self._moments[key]
+        ops.adam_step(target, grads, None if master is None else weights, m, v, self._step_dev, self.lr, self.betas,
+                      self.eps, self.weight_decay, self.clip_value)
+
+    @torch.no_grad()
+    def step(self) -> None:
+        if self.stores:
+            ring.join_wgrad(self.stores[0].home.device)
+        if self._step_dev is None:
+            buffers = [st.home for st in self.stores] + ([self.flat] if self.flat is not None else [])
+            if not buffers:
+                return
+            self._step_dev = torch.zeros(1, dtype=torch.int64, device=buffers[0].device)
+        self.steps += 1
+        self._step_dev += 1
+        for i, (st, master) in enumerate(zip(self.stores, self.masters)):
+            if st.grads is None:
+                continue
+            self._adam(i, st.home.view(-1), st.grads.view(-1), master)
+        if self.flat is not None:
+            self._fold_other_grads()
+            self._adam("flat", self.flat, self.flat_grad, self.flat_master)
+        if self.stores:
+            ring.fence(self.stores[0].home.device)  # staging copies of the next step must see the new weights
