@@ -90,6 +90,15 @@ class RotatedSGD:
                 off += n
         self.flat_master = None if p0.dtype == torch.float32 else self.flat.float()
 
+    @torch.no_grad()
+    def reload_masters(self) -> None:
+        """Re-read the fp32 master copies from the weights (after a checkpoint was loaded into the model)."""
+        for st, master in zip(self.stores, self.masters):
+            if master is not None:
+                master.copy_(st.home)
+        if self.flat_master is not None:
+            self.flat_master.copy_(self.flat)
+
     def master_bytes(self) -> int:
         n = sum(m.numel() * 4 for m in self.masters if m is not None)
         return n + (self.flat_master.numel() * 4 if self.flat_master is not None else 0)

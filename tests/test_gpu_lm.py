@@ -227,3 +227,34 @@ def test_lm_weight_gradients_on_second_stream_are_bit_identical():
         ring.set_wgrad_overlap(False)
     for (na, pa), (nb, pb) in zip(lm_a.named_parameters(), lm_b.named_parameters()):
         assert torch.equal(pa.grad, pb.grad), f"grad of {na} differs"
+
+
+def test_lm_rank_state_dicts_round_trip_on_device():
+    """Per-rank state dicts in the reference's layout, saved from one LM and loaded into another: same logits bit for
+    bit; the optimiser's fp32 masters re-read; the MoE variant's expert and gate keys."""
+    from rtp_amd.checkpoint import load_rank_state_dicts, rank_state_dict
+    from rtp_amd.models.transformer_lm_rtp import TransformerLM
+    from rtp_amd.optim import RotatedSGD
+    V, D, H, Fd, n_dec, L, N, ws = 64, 32, 4, 32, 1, 6, 3, 4
+    a, _ = build_pair(V, D, H, Fd, n_dec, ws, torch.bfloat16, seed=7)
+    b, _ = build_pair(V, D, H, Fd, n_dec, ws, torch.bfloat16, seed=8)
+    opt_b = RotatedSGD(b, lr=0.1)
+    ids = torch.randint(0, V, (L, N)).to(DEV)
+    assert not torch.equal(a(ids), b(ids))
+    dicts = [{k: v.detach().cpu().clone() for k, v in rank_state_dict(a, r).items()} for r in range(ws)]
+    assert "2.self_attn.MultiheadAttention.in_proj_weight" in dicts[1] and "0.embedding.embedding.weight" in dicts[1]
+    assert f"{len(a) - 1}.linear.linear.bias" in dicts[1]
+    load_rank_state_dicts(b, dicts)
+    assert torch.equal(a(ids), b(ids))
+    opt_b.reload_masters()
+    for st, master in zip(opt_b.stores, opt_b.masters):
+        assert torch.equal(master.view(-1).to(torch.bfloat16), st.home.view(-1))
+    moe = TransformerLM(64, 32, 4, 48, 0.0, 0.1, 1, 4, 0, is_moe=True, device=DEV)
+    keys = list(rank_state_dict(moe, 3).keys())
+    assert any(k.endswith("moe_layer.gate.wg.weight") for k in keys), keys
+    assert any(".moe_layer.experts.0." in k for k in keys), keys
+    assert not any(".shards." in k for k in keys)
+    moe2 = TransformerLM(64, 32, 4, 48, 0.0, 0.1, 1, 4, 0, is_moe=True, device=DEV)
+    load_rank_state_dicts(moe2, [rank_state_dict(moe, r) for r in range(4)])
+    for (ka, ta), (kb, tb) in zip(moe.state_dict().items(), moe2.state_dict().items()):
+        assert ka == kb and torch.equal(ta, tb)

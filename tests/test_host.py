@@ -140,3 +140,56 @@ def test_forward_without_gpu_fails_loudly():
 def test_constructor_signatures_match_reference(cls, expected):
     params = [p for p in inspect.signature(cls.__init__).parameters if p != "self"]
     assert params == expected
+
+
+def test_rank_state_dicts_follow_the_reference_layout_and_round_trip():
+    """What rank r of the reference saves (its own shard under the home attribute's name, rtp/module/linear.py:187:
+    only `self.linear` is a registered submodule) and loading ws such dicts back into all shards held here."""
+    from rtp_amd.checkpoint import load_rank_state_dicts, rank_state_dict, world_size_of
+
+    class Net(nn.Module):
+        def __init__(self, lin, mha, emb):
+            super().__init__()
+            self.emb = embedding.ParallelEmbedding(10, 8, 4, 0, Embedding_layer=emb)
+            self.attn = attention.ParallelMultiheadAttention(8, 4, 4, 0, MultiheadAttention_layer=mha)
+            with emulate_shards(4):
+                self.fc = linear.ColumnParallelLinear(8, 12, linear_layer=lin)
+            self.norm = nn.LayerNorm(8)
+
+    torch.manual_seed(0)
+    lin, mha, emb = nn.Linear(8, 12), nn.MultiheadAttention(8, 4), nn.Embedding(10, 8)
+    net = Net(lin, mha, emb)
+    assert world_size_of(net) == 4
+    dicts = [rank_state_dict(net, r) for r in range(4)]
+    assert list(dicts[2].keys()) == [
+        "emb.embedding.weight", "attn.MultiheadAttention.in_proj_weight", "attn.MultiheadAttention.in_proj_bias",
+        "attn.MultiheadAttention.out_proj.weight", "attn.MultiheadAttention.out_proj.bias", "fc.linear.weight",
+        "fc.linear.bias", "norm.weight", "norm.bias"]
+    for r in range(4):
+        assert torch.equal(dicts[r]["fc.linear.weight"], lin.weight[3 * r:3 * r + 3])          # output rows
+        assert torch.equal(dicts[r]["fc.linear.bias"], lin.bias[3 * r:3 * r + 3])
+        assert torch.equal(dicts[r]["emb.embedding.weight"], emb.weight[:, 2 * r:2 * r + 2])   # embedding columns
+        assert torch.equal(dicts[r]["attn.MultiheadAttention.out_proj.weight"], mha.out_proj.weight[:, 2 * r:2 * r + 2])
+        w = O.attention_shard_params(mha.in_proj_weight.detach(), mha.in_proj_bias.detach(),
+                                     mha.out_proj.weight.detach(), mha.out_proj.bias.detach(), 4, r)
+        assert torch.equal(dicts[r]["attn.MultiheadAttention.in_proj_weight"], w[0])
+    # into a differently initialised model of the same architecture
+    other = Net(nn.Linear(8, 12), nn.MultiheadAttention(8, 4), nn.Embedding(10, 8))
+    saved = [{k: v.clone() for k, v in d.items()} for d in dicts]
+    load_rank_state_dicts(other, saved)
+    for (ka, a), (kb, b) in zip(net.state_dict().items(), other.state_dict().items()):
+        assert ka == kb and torch.equal(a, b)
+    st = other.fc._store
+    assert other.fc.linears[1].weight.data_ptr() == st.home[1].data_ptr()   # still views of the flat buffer
+    # strictness: a replicated entry that differs between ranks, a missing rank, a foreign key
+    saved[3]["norm.weight"] = saved[3]["norm.weight"] + 1
+    with pytest.raises(ValueError):
+        load_rank_state_dicts(other, saved)
+    with pytest.raises(ValueError):
+        load_rank_state_dicts(other, saved[:3])
+    saved[3]["norm.weight"] = saved[0]["norm.weight"]
+    saved[0]["nope.weight"] = torch.zeros(1)
+    with pytest.raises(KeyError):
+        load_rank_state_dicts(other, saved)
+    with pytest.raises(ValueError):
+        rank_state_dict(net, 4)
