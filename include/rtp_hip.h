@@ -343,6 +343,30 @@ int rtp_moe_combine_dweight(void* stream, int dtype, const void* dout, int64_t l
                             float* dweight);
 
 /* ---------------------------------------------------------------------------------------------
+ * Out-channel-sharded 2-D convolution (reference: the per-shard `self.layers[index](input_)` = F.conv2d of
+ * ColumnParallelConv2d, rtp/module/conv.py:108, and its autograd backward) as a column-sharded product on
+ * rtp_gemm:  Y[N*Ho*Wo, Co_s] = patches[N*Ho*Wo, Ci*kh*kw] x W_s^T + b_s  (a shard's weight [Co_s, Ci, kh, kw] is,
+ * as stored, that row-major operand), dW_s = dY_s^T patches, dpatches = sum_s dY_s W_s.  These two entry points
+ * build the patch matrix and fold patch gradients back (zero padding, groups = 1):
+ *   im2col: patches[(n*Ho+ho)*Wo+wo][(ci*kh+i)*kw+j] = x[n][ci][ho*sh-ph+i*dh][wo*sw-pw+j*dw], 0 outside; x is
+ *           addressed by element strides (any memory format), columns beyond Ci*kh*kw up to ld_cols are zeroed
+ *   col2im: dx[n][ci][h][w] (contiguous NCHW) = sum of the patch-gradient entries that read x[n][ci][h][w],
+ *           fp32, ascending (i, j)
+ * ho / wo must equal floor((h + 2*ph - dh*(kh-1) - 1) / sh) + 1 (and likewise for w).
+ * --------------------------------------------------------------------------------------------- */
+typedef struct {
+  int64_t n, c, h, w;   /* input: batch, channels, height, width */
+  int64_t kh, kw;       /* kernel */
+  int64_t sh, sw;       /* stride */
+  int64_t ph, pw;       /* zero padding on each side */
+  int64_t dh, dw;       /* dilation */
+  int64_t ho, wo;       /* output height, width */
+} rtp_conv_geom;
+int rtp_im2col(void* stream, int dtype, const void* x, int64_t sx_n, int64_t sx_c, int64_t sx_h, int64_t sx_w,
+               const rtp_conv_geom* geom, void* cols, int64_t ld_cols);
+int rtp_col2im(void* stream, int dtype, const void* dcols, int64_t ld_dcols, const rtp_conv_geom* geom, void* dx);
+
+/* ---------------------------------------------------------------------------------------------
  * Optimiser step on a flat shard buffer (reference harness: clip_grad_value_ + optimizer.step,
  * benchmarks/rtp_benchmark.py:185-186; SGD as the headline configuration asks).
  *   g = clamp(grad, -clip, clip) if clip > 0;  master -= lr * g;  shadow = (dtype) master.

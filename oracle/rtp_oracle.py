@@ -21,6 +21,9 @@ float32 unless the caller passes float64 tensors.  How each function is pinned (
   moe_layer                                      == golden vectors written from the reference's WeightMOELayer run on a
                                                     2-rank gloo ring (tests/golden/moe_ws2.npz), and the closed form
                                                     out[s] = w1*y[e1,slot1] + w2*y[e2,slot2]
+  column_parallel_conv2d / conv_patches / conv_fold
+                                                 == torch.nn.functional.conv2d on the unsharded problem, F.unfold / F.fold,
+                                                    and python loops over a tiny input (patch layout and zero padding)
   transformer_lm                                 == assembled from stock torch layers exactly as
                                                     rtp/models/transformer_lm_rtp.py:19-242 assembles the rotated ones
 """
@@ -174,6 +177,32 @@ def parallel_multihead_attention(x, in_w, in_b, out_w, out_b, num_heads: int, ws
 # ------------------------------------------------------------------------------------------------
 # Top-2 gating (rtp/module/top2gate.py:43-105)
 # ------------------------------------------------------------------------------------------------
+def column_parallel_conv2d(x, weight, bias, ws: int, stride=1, padding=0, dilation=1, rank: int = 0):
+    """Out-channel shards visited in ring order, outputs concatenated on dim 1 in shard order
+    (rtp/module/conv.py:99-114; shard = rows [s*Co/ws, (s+1)*Co/ws) of weight and bias, conv.py:43-47)."""
+    n_s = weight.shape[0] // ws
+    assert n_s * ws == weight.shape[0]
+    outs: List[Optional[torch.Tensor]] = [None] * ws
+    for s in ring_order(rank, ws):
+        b = None if bias is None else bias[s * n_s:(s + 1) * n_s]
+        outs[s] = F.conv2d(x, weight[s * n_s:(s + 1) * n_s], b, stride, padding, dilation)
+    return torch.cat(outs, dim=1).contiguous()
+
+
+def conv_patches(x, kernel_size, stride, padding, dilation):
+    """Patch matrix [N*Ho*Wo, Ci*kh*kw] of an NCHW input: row (n, ho, wo), column (ci, i, j), zero padding --
+    the operand with which conv2d is the product patches @ weight.view(Co, -1).T (+ bias)."""
+    u = F.unfold(x, kernel_size, dilation, padding, stride)        # [N, Ci*kh*kw, Ho*Wo]
+    return u.transpose(1, 2).reshape(-1, u.shape[1])
+
+
+def conv_fold(dpatches, x_shape, kernel_size, stride, padding, dilation):
+    """Transpose of conv_patches: patch gradients [N*Ho*Wo, Ci*kh*kw] summed back onto the NCHW input."""
+    n, c, h, w = x_shape
+    u = dpatches.reshape(n, -1, dpatches.shape[1]).transpose(1, 2)
+    return F.fold(u, (h, w), kernel_size, dilation, padding, stride)
+
+
 def gumbel_noise(shape, generator: torch.Generator) -> torch.Tensor:
     """-log(-log U), U ~ Uniform(tiny, 1-eps): torch.distributions.Gumbel(0,1).rsample (top2gate.py:25-32)
     with an explicit CPU generator so the noise is an input."""

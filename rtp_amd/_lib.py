@@ -27,6 +27,11 @@ class RtpError(RuntimeError):
     """A call into librtp_hip.so returned a negative status."""
 
 
+class ConvGeom(C.Structure):
+    """rtp_conv_geom of include/rtp_hip.h."""
+    _fields_ = [(n, C.c_int64) for n in ("n", "c", "h", "w", "kh", "kw", "sh", "sw", "ph", "pw", "dh", "dw", "ho", "wo")]
+
+
 class GemmDesc(C.Structure):
     _fields_ = [
         ("a", C.c_void_p), ("b", C.c_void_p), ("c_out", C.c_void_p), ("c_in", C.c_void_p),
@@ -102,6 +107,8 @@ PROTOTYPES = {
     "rtp_moe_dispatch": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64]),
     "rtp_moe_combine": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64]),
     "rtp_moe_combine_dweight": (_i, [_vp, _i, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "rtp_im2col": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _i64, C.POINTER(ConvGeom), _vp, _i64]),
+    "rtp_col2im": (_i, [_vp, _i, _vp, _i64, C.POINTER(ConvGeom), _vp]),
     "rtp_sgd_step": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _f, _f]),
     "rtp_adam_step": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i64, C.c_double, C.c_double, C.c_double, C.c_double,
                            C.c_double, _i64, _vp, C.c_double]),

@@ -492,6 +492,40 @@ def sgd_step(master: torch.Tensor, grad: torch.Tensor, shadow: Optional[torch.Te
                                    _ptr(shadow), master.numel(), lr, clip))
 
 
+def conv_geom(x_shape, kernel_size, stride, padding, dilation) -> "_lib.ConvGeom":
+    """Geometry record of a zero-padded 2-D convolution over an NCHW input (output size as torch computes it)."""
+    n, c, h, w = (int(v) for v in x_shape)
+    (kh, kw), (sh, sw), (ph, pw), (dh, dw) = kernel_size, stride, padding, dilation
+    ho = (h + 2 * ph - dh * (kh - 1) - 1) // sh + 1
+    wo = (w + 2 * pw - dw * (kw - 1) - 1) // sw + 1
+    if ho < 1 or wo < 1:
+        raise ValueError(f"convolution kernel {kh}x{kw} (dilation {dh},{dw}) larger than the padded input {h}x{w}")
+    return _lib.ConvGeom(n, c, h, w, kh, kw, sh, sw, ph, pw, dh, dw, ho, wo)
+
+
+def im2col(x: torch.Tensor, geom, cols: torch.Tensor) -> None:
+    """cols[N*Ho*Wo, ld] <- the patch matrix of NCHW `x` (any strides); columns beyond C*kh*kw are zeroed."""
+    _dev(x)
+    if x.dim() != 4 or cols.dim() != 2 or cols.dtype != x.dtype or cols.stride(1) != 1 or \
+            cols.shape[0] != geom.n * geom.ho * geom.wo or cols.stride(0) != cols.shape[1]:
+        raise ValueError("im2col: need a 4-D input and a dense [N*Ho*Wo, ld] patch matrix of its dtype")
+    _lib.require_device()
+    check(_lib.load().rtp_im2col(_stream(), dtype_code(x.dtype), x.data_ptr(), *x.stride(), geom, cols.data_ptr(),
+                                 cols.shape[1]))
+
+
+def col2im(dcols: torch.Tensor, geom, dx: torch.Tensor) -> None:
+    """dx (contiguous NCHW) <- patch gradients dcols[N*Ho*Wo, ld] folded back onto the input."""
+    _dev(dcols)
+    if dcols.dim() != 2 or dcols.stride(1) != 1 or dcols.stride(0) != dcols.shape[1] or dx.dtype != dcols.dtype or \
+            not dx.is_contiguous() or tuple(dx.shape) != (geom.n, geom.c, geom.h, geom.w) or \
+            dcols.shape[0] != geom.n * geom.ho * geom.wo:
+        raise ValueError("col2im: need a dense [N*Ho*Wo, ld] patch-gradient matrix and a contiguous NCHW output")
+    _lib.require_device()
+    check(_lib.load().rtp_col2im(_stream(), dtype_code(dcols.dtype), dcols.data_ptr(), dcols.shape[1], geom,
+                                 dx.data_ptr()))
+
+
 def adam_step(master: torch.Tensor, grad: torch.Tensor, shadow: Optional[torch.Tensor], exp_avg: torch.Tensor,
               exp_avg_sq: torch.Tensor, step, lr: float, betas=(0.9, 0.999), eps: float = 1e-8,
               weight_decay: float = 0.0, clip: float = 0.0) -> None:

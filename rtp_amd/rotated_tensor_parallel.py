@@ -1,4 +1,4 @@
-"""RotatedTensorParallel: shard the nn.Linear / nn.Embedding / nn.MultiheadAttention leaves of an
+"""RotatedTensorParallel: shard the nn.Linear / nn.Conv2d / nn.Embedding / nn.MultiheadAttention leaves of an
 existing model in place and run them as rotated layers (counterpart of
 rtp/rotated_tensor_parallel.py:296-571).
 
@@ -6,6 +6,8 @@ Sharding rules (rotated_tensor_parallel.py:454-529):
   nn.Linear              out_features % ws == 0 -> column shards (weight rows, bias slice), outputs side by side;
                          elif in_features % ws == 0 -> row shards (weight columns, bias/ws), outputs summed;
                          else ValueError.
+  nn.Conv2d              out_channels % ws == 0 -> output-channel shards, outputs concatenated on dim 1, else
+                         ValueError (rotated_tensor_parallel.py:472-483).
   nn.Embedding           embedding_dim % ws == 0 -> column blocks of the table, else ValueError.
   nn.MultiheadAttention  head groups: in-projection blocks [r, r+ws, r+2ws] of a 3*ws row split,
                          out-projection column block r, out bias / ws; outputs summed.
@@ -20,6 +22,7 @@ import torch.nn as nn
 
 from .module.attention import ParallelMultiheadAttention
 from .module.collectives import emulate_shards, resolve_world
+from .module.conv import ColumnParallelConv2d
 from .module.embedding import ParallelEmbedding
 from .module.linear import ColumnParallelLinear, RowParallelLinear
 
@@ -91,7 +94,12 @@ class RotatedTensorParallel(nn.Module):
                     raise ValueError("The input or output features of the linear layer must be divisible by the "
                                      "world size.")
             elif isinstance(module, nn.Conv2d):
-                raise NotImplementedError("RotatedTensorParallel: nn.Conv2d sharding is not built")
+                if module.out_channels % ws != 0:
+                    raise ValueError("The input or output channels of the conv layer must be divisible by the world "
+                                     "size.")
+                wrapped = FlyweightWarpper(ColumnParallelConv2d(
+                    module.in_channels, module.out_channels, module.kernel_size, module.stride, module.padding,
+                    module.dilation, module.groups, module.bias is not None, module.padding_mode, Conv2d_layer=module))
             elif isinstance(module, nn.Embedding):
                 if module.embedding_dim % ws != 0:
                     raise ValueError("The embedding_dim of the embedding layer must be divisible by the world size.")

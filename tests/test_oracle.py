@@ -260,3 +260,43 @@ def test_transformer_lm_structure_and_param_count():
     ids2 = ids.clone()
     ids2[5:] = (ids2[5:] + 1) % 50
     torch.testing.assert_close(small(ids2)[:5], out[:5])
+
+
+@pytest.mark.parametrize("ws", [1, 2, 4])
+@pytest.mark.parametrize("stride,padding,dilation", [(1, 0, 1), (2, 1, 1), ((1, 2), (2, 0), (2, 1))])
+def test_column_conv2d_matches_unsharded_conv_and_patch_product(ws, stride, padding, dilation):
+    """Shards along the output channels concatenate to stock conv2d (the reference's oracle for its Conv2d rule,
+    test_net.py); the patch matrix times the flattened weight is the same convolution; its transpose is F.fold."""
+    torch.manual_seed(ws)
+    x = torch.randn(2, 3, 9, 8, dtype=torch.float64)
+    conv = torch.nn.Conv2d(3, 8, (3, 2), stride, padding, dilation).double()
+    ref = conv(x)
+    out = O.column_parallel_conv2d(x, conv.weight.detach(), conv.bias.detach(), ws, stride, padding, dilation)
+    assert torch.allclose(out, ref, rtol=1e-12, atol=1e-12)
+    p = O.conv_patches(x, (3, 2), conv.stride, conv.padding, conv.dilation)
+    y = (p @ conv.weight.detach().view(8, -1).T + conv.bias.detach()).view(2, ref.shape[2], ref.shape[3], 8)
+    assert torch.allclose(y.permute(0, 3, 1, 2), ref, rtol=1e-12, atol=1e-12)
+    # fold is the transpose of the patch map: <patches(x), g> == <x, fold(g)>
+    g = torch.randn_like(p)
+    lhs = (p * g).sum()
+    rhs = (x * O.conv_fold(g, x.shape, (3, 2), conv.stride, conv.padding, conv.dilation)).sum()
+    assert abs(float(lhs - rhs)) < 1e-9 * max(1.0, abs(float(lhs)))
+
+
+def test_conv_patches_layout_by_loops():
+    """Row (n, ho, wo), column (ci, i, j), zeros outside the image: python loops on a tiny input."""
+    x = torch.arange(2 * 2 * 4 * 5, dtype=torch.float32).view(2, 2, 4, 5) + 1
+    kh, kw, sh, sw, ph, pw, dh, dw = 2, 3, 2, 1, 1, 2, 1, 2
+    ho = (4 + 2 * ph - dh * (kh - 1) - 1) // sh + 1
+    wo = (5 + 2 * pw - dw * (kw - 1) - 1) // sw + 1
+    p = O.conv_patches(x, (kh, kw), (sh, sw), (ph, pw), (dh, dw))
+    assert p.shape == (2 * ho * wo, 2 * kh * kw)
+    for n in range(2):
+        for a in range(ho):
+            for b in range(wo):
+                for ci in range(2):
+                    for i in range(kh):
+                        for j in range(kw):
+                            h, w = a * sh - ph + i * dh, b * sw - pw + j * dw
+                            want = float(x[n, ci, h, w]) if 0 <= h < 4 and 0 <= w < 5 else 0.0
+                            assert float(p[(n * ho + a) * wo + b, (ci * kh + i) * kw + j]) == want
