@@ -8,7 +8,7 @@ import torch.nn as nn
 
 from oracle import rtp_oracle as O
 from rtp_amd import emulate_shards
-from rtp_amd.module import attention, collectives, embedding, linear, moe, top2gate, utils
+from rtp_amd.module import attention, collectives, conv, embedding, linear, moe, top2gate, utils
 from rtp_amd.ring import ring_order
 
 
@@ -136,6 +136,9 @@ def test_forward_without_gpu_fails_loudly():
                                             "dtype", "MultiheadAttention_layer"]),
     (top2gate.WeightTop2Gate, ["model_dim", "num_experts", "gate", "device", "dtype"]),
     (moe.WeightMOELayer, ["gate", "experts", "group", "device", "dtype", "original_experts"]),
+    (conv.ColumnParallelConv2d, ["in_channels", "out_channels", "kernel_size", "stride", "padding", "dilation",
+                                 "groups", "bias", "padding_mode", "device", "dtype", "group", "gather_output",
+                                 "Conv2d_layer"]),
 ])
 def test_constructor_signatures_match_reference(cls, expected):
     params = [p for p in inspect.signature(cls.__init__).parameters if p != "self"]
