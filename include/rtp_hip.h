@@ -343,6 +343,28 @@ int rtp_moe_combine_dweight(void* stream, int dtype, const void* dout, int64_t l
                             float* dweight);
 
 /* ---------------------------------------------------------------------------------------------
+ * Gate projection with few experts (reference: `logits = self.wg(input)` of the rotated gate,
+ * rtp/module/top2gate.py:195-207 -- an nn.Linear without bias whose expert rows are sharded -- and its autograd
+ * backward).  With E <= 16 output columns these are streaming passes over the tokens, not tiled products:
+ *   fwd:   logits[s][e] = sum_m x[s][m] * w[e][m]                  fp32 logits
+ *   dgrad: dx[s][m]     = sum_e dlogits[s][e] * w[e][m]            fp32 dlogits, e ascending, rounded once
+ *   wgrad: dw[e][m]   (+)= sum_s dlogits[s][e] * x[s][m]           partial sums of 64 token rows, then summed in order
+ * x [S, M], w and dw [E, M] in `dtype` with element row pitches; rtp_gate_supported says whether (E, M) qualify
+ * (E <= 16, M a multiple of 16 bytes); x, w, dx must be 16-byte aligned with pitches that keep rows so.  The rows
+ * of w / dw of consecutive shards are consecutive rows of one matrix when a shard's flat buffer is exactly its
+ * [E/ws, M] weight.  Otherwise use rtp_gemm.
+ * --------------------------------------------------------------------------------------------- */
+int rtp_gate_supported(int dtype, int64_t experts, int64_t model_dim);
+int rtp_gate_fwd(void* stream, int dtype, const void* x, int64_t ldx, const void* w, int64_t ldw, int64_t S,
+                 int64_t M, int64_t E, float* logits, int64_t ld_logits);
+int rtp_gate_dgrad(void* stream, int dtype, const float* dlogits, int64_t ld_dlogits, const void* w, int64_t ldw,
+                   int64_t S, int64_t M, int64_t E, void* dx, int64_t ldx);
+size_t rtp_gate_wgrad_workspace_bytes(int64_t S, int64_t M, int64_t E);
+int rtp_gate_wgrad(void* stream, int dtype, const float* dlogits, int64_t ld_dlogits, const void* x, int64_t ldx,
+                   int64_t S, int64_t M, int64_t E, void* dw, int64_t ld_dw, int accumulate, void* workspace,
+                   size_t workspace_bytes);
+
+/* ---------------------------------------------------------------------------------------------
  * Out-channel-sharded 2-D convolution (reference: the per-shard `self.layers[index](input_)` = F.conv2d of
  * ColumnParallelConv2d, rtp/module/conv.py:108, and its autograd backward) as a column-sharded product on
  * rtp_gemm:  Y[N*Ho*Wo, Co_s] = patches[N*Ho*Wo, Ci*kh*kw] x W_s^T + b_s  (a shard's weight [Co_s, Ci, kh, kw] is,

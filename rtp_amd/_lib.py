@@ -107,6 +107,11 @@ PROTOTYPES = {
     "rtp_moe_dispatch": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64]),
     "rtp_moe_combine": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64]),
     "rtp_moe_combine_dweight": (_i, [_vp, _i, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "rtp_gate_supported": (_i, [_i, _i64, _i64]),
+    "rtp_gate_fwd": (_i, [_vp, _i, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64]),
+    "rtp_gate_dgrad": (_i, [_vp, _i, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64]),
+    "rtp_gate_wgrad_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "rtp_gate_wgrad": (_i, [_vp, _i, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i, _vp, _sz]),
     "rtp_im2col": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _i64, C.POINTER(ConvGeom), _vp, _i64]),
     "rtp_col2im": (_i, [_vp, _i, _vp, _i64, C.POINTER(ConvGeom), _vp]),
     "rtp_sgd_step": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _f, _f]),

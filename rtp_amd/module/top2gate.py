@@ -72,8 +72,17 @@ def top2gating(logits: Tensor, noise: Optional[Tensor] = None) -> Tuple[Tensor, 
     return l_aux.to(logits.dtype), combine, dispatch
 
 
+def _run_rows(flat: Tensor, e_s: int, m: int) -> Optional[Tensor]:
+    """The expert rows of a run of staged gate shards as one [cnt * e_s, M] matrix: a gate shard's flat buffer is
+    exactly its [e_s, M] weight, so consecutive shards are consecutive rows."""
+    if flat.shape[1] != e_s * m or not flat.is_contiguous():
+        return None
+    return flat.view(flat.shape[0] * e_s, m)
+
+
 class _GateProjectionFn(torch.autograd.Function):
-    """logits[S,E] = x[S,M] @ wg^T with wg's expert rows sharded and rotated; fp32 logits."""
+    """logits[S,E] = x[S,M] @ wg^T with wg's expert rows sharded and rotated; fp32 logits.  Runs of at most 16
+    experts take the streaming gate kernels (one pass over the tokens each way), others the tiled product."""
 
     @staticmethod
     def forward(ctx, x, anchor, layer):
@@ -84,7 +93,11 @@ class _GateProjectionFn(torch.autograd.Function):
         rot = Rotation(store.home, ring_order(layer.rank, ws), group=store.stage_group)
         for j in range(rot.steps):
             for flat, first, cnt in rot.acquire(j):
-                S.col_fwd(x2, flat, 0, e_s, layer.model_dim, None, logits, first * e_s)
+                rows = _run_rows(flat, e_s, layer.model_dim)
+                if rows is not None and ops.gate_supported(x2, rows):
+                    ops.gate_fwd(x2, rows, logits, first * e_s)
+                else:
+                    S.col_fwd(x2, flat, 0, e_s, layer.model_dim, None, logits, first * e_s)
             rot.release(j)
         ctx.layer = layer
         ctx.save_for_backward(x2)
@@ -96,23 +109,41 @@ class _GateProjectionFn(torch.autograd.Function):
         (x2,) = ctx.saved_tensors
         store = layer._store
         ws, e_s = layer.world_size, layer.num_local_experts
-        dl = d_logits.to(x2.dtype).contiguous()
+        m = layer.model_dim
+        dl32 = d_logits.float().contiguous()
+        dl = None  # the tiled products take the gradient in the weights' dtype; made only if one of them runs
+
+        def low():
+            nonlocal dl
+            if dl is None:
+                dl = dl32.to(x2.dtype)
+            return dl
+
         need_dx = ctx.needs_input_grad[0]
         order = ring_order(layer.rank, ws, reverse=True)
         dx = None
         if need_dx:
             dx = torch.empty_like(x2)
             rot = Rotation(store.home, order, group=store.stage_group)
-            acc = ops.ShardSum(dx, sum(len(w) for w in rot.windows))
+            steps = sum(len(w) for w in rot.windows)
+            acc = ops.ShardSum(dx, steps)
             i = 0
             for j in range(rot.steps):
                 for flat, first, cnt in rot.acquire(j):
-                    c_out, c_in = acc.target(i)
-                    S.col_dgrad(dl, flat, 0, e_s, layer.model_dim, c_out, first * e_s, c_in=c_in)
+                    rows = _run_rows(flat, e_s, m)
+                    if steps == 1 and rows is not None and ops.gate_supported(dx, rows):
+                        ops.gate_dgrad(dl32, first * e_s, rows, dx)   # the only run: dx needs no summing
+                    else:
+                        c_out, c_in = acc.target(i)
+                        S.col_dgrad(low(), flat, 0, e_s, m, c_out, first * e_s, c_in=c_in)
                     i += 1
                 rot.release(j)
         for first, cnt, accumulate in store.grad_runs(order):
-            S.col_wgrad(dl, x2, store.grads, first, 0, e_s, layer.model_dim, first * e_s, cnt, accumulate)
+            rows = _run_rows(store.grads[first:first + cnt], e_s, m)
+            if rows is not None and ops.gate_supported(x2, rows):
+                ops.gate_wgrad(dl32, first * e_s, x2, rows, accumulate)
+            else:
+                S.col_wgrad(low(), x2, store.grads, first, 0, e_s, m, first * e_s, cnt, accumulate)
         store.grads_ready()
         return dx, None, None
 

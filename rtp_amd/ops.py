@@ -492,6 +492,56 @@ def sgd_step(master: torch.Tensor, grad: torch.Tensor, shadow: Optional[torch.Te
                                    _ptr(shadow), master.numel(), lr, clip))
 
 
+def gate_supported(x2: torch.Tensor, w_rows: torch.Tensor) -> bool:
+    """Whether the streaming gate kernels take logits = x2 @ w_rows^T: at most 16 expert rows, model dimension a
+    multiple of 16 bytes, 16-byte aligned rows on both sides."""
+    if x2.dtype not in (torch.float32, torch.bfloat16) or w_rows.dtype != x2.dtype or x2.dim() != 2 or w_rows.dim() != 2:
+        return False
+    vec = 16 // x2.element_size()
+    ok = all(t.stride(1) == 1 and t.stride(0) % vec == 0 and t.data_ptr() % 16 == 0 for t in (x2, w_rows))
+    return ok and bool(_lib.load().rtp_gate_supported(dtype_code(x2.dtype), w_rows.shape[0], x2.shape[1]))
+
+
+def gate_fwd(x2: torch.Tensor, w_rows: torch.Tensor, logits: torch.Tensor, col0: int) -> None:
+    """logits[:, col0 : col0 + E] = x2 @ w_rows^T (fp32 logits, E = w_rows.shape[0] <= 16)."""
+    _dev(x2)
+    if logits.dtype != torch.float32 or logits.stride(1) != 1 or logits.shape[0] != x2.shape[0] or \
+            col0 + w_rows.shape[0] > logits.shape[1]:
+        raise ValueError("gate_fwd: logits must be fp32 [S, >= col0 + E]")
+    _lib.require_device()
+    check(_lib.load().rtp_gate_fwd(_stream(), dtype_code(x2.dtype), x2.data_ptr(), x2.stride(0), w_rows.data_ptr(),
+                                   w_rows.stride(0), x2.shape[0], x2.shape[1], w_rows.shape[0],
+                                   logits.data_ptr() + 4 * col0, logits.stride(0)))
+
+
+def gate_dgrad(d_logits: torch.Tensor, col0: int, w_rows: torch.Tensor, dx: torch.Tensor) -> None:
+    """dx = d_logits[:, col0 : col0 + E] @ w_rows (d_logits fp32; dx in the weights' dtype, fully overwritten)."""
+    _dev(dx)
+    if d_logits.dtype != torch.float32 or d_logits.stride(1) != 1 or dx.dtype != w_rows.dtype or dx.stride(1) != 1 or \
+            d_logits.shape[0] != dx.shape[0] or dx.shape[1] != w_rows.shape[1]:
+        raise ValueError("gate_dgrad: need fp32 d_logits [S, E] and dx [S, M] of the weights' dtype")
+    _lib.require_device()
+    check(_lib.load().rtp_gate_dgrad(_stream(), dtype_code(dx.dtype), d_logits.data_ptr() + 4 * col0, d_logits.stride(0),
+                                     w_rows.data_ptr(), w_rows.stride(0), dx.shape[0], dx.shape[1], w_rows.shape[0],
+                                     dx.data_ptr(), dx.stride(0)))
+
+
+def gate_wgrad(d_logits: torch.Tensor, col0: int, x2: torch.Tensor, dw_rows: torch.Tensor, accumulate: bool) -> None:
+    """dw_rows[E, M] (+)= d_logits[:, col0 : col0 + E]^T @ x2, summed over the tokens in a fixed order."""
+    _dev(x2)
+    e, m = dw_rows.shape
+    if d_logits.dtype != torch.float32 or d_logits.stride(1) != 1 or dw_rows.dtype != x2.dtype or \
+            dw_rows.stride(1) != 1 or x2.shape[1] != m or d_logits.shape[0] != x2.shape[0]:
+        raise ValueError("gate_wgrad: need fp32 d_logits [S, E], x2 [S, M] and dw_rows [E, M] of x2's dtype")
+    lib = _lib.load()
+    nbytes = lib.rtp_gate_wgrad_workspace_bytes(x2.shape[0], m, e)
+    ws = torch.empty(nbytes // 4, dtype=torch.float32, device=x2.device)
+    _lib.require_device()
+    check(lib.rtp_gate_wgrad(_stream(), dtype_code(x2.dtype), d_logits.data_ptr() + 4 * col0, d_logits.stride(0),
+                             x2.data_ptr(), x2.stride(0), x2.shape[0], m, e, dw_rows.data_ptr(), dw_rows.stride(0),
+                             int(accumulate), ws.data_ptr(), nbytes))
+
+
 def conv_geom(x_shape, kernel_size, stride, padding, dilation) -> "_lib.ConvGeom":
     """Geometry record of a zero-padded 2-D convolution over an NCHW input (output size as torch computes it)."""
     n, c, h, w = (int(v) for v in x_shape)

@@ -171,3 +171,45 @@ def test_gate_module_dense_api():
     assert combine.shape == (32, 4, 16) and dispatch.dtype == torch.bool
     assert torch.equal(dispatch.cpu(), g["dispatch_mask"])
     assert rel_err(combine, g["combine_weights"]) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype,S,M,E", [(torch.float32, 100, 64, 3), (torch.bfloat16, 4096, 2048, 8),
+                                         (torch.bfloat16, 33, 136, 16), (torch.float32, 5, 4, 1)])
+def test_gate_streaming_kernels_against_torch(dtype, S, M, E):
+    """rtp_gate_fwd / dgrad / wgrad through the C ABI against fp32 torch products on the same inputs: the gate
+    projection of the reference (an nn.Linear without bias, rtp/module/top2gate.py:202) and its backward."""
+    from rtp_amd import ops
+    from gpu_util import assert_close
+    gen = torch.Generator().manual_seed(S + M + E)
+    x = torch.randn(S, M, generator=gen).to(dtype)
+    w = (torch.randn(E, M, generator=gen) * 0.1).to(dtype)
+    dl = torch.randn(S, E + 2, generator=gen)                     # the run's columns sit at offset 1 of a wider matrix
+    xd, wd, dld = x.to(DEV), w.to(DEV), dl.to(DEV)
+    assert ops.gate_supported(xd, wd)
+    logits = torch.full((S, E + 2), 7.0, device=DEV)
+    ops.gate_fwd(xd, wd, logits, 1)
+    assert_close(logits[:, 1:E + 1], x.float() @ w.float().T, torch.float32 if dtype == torch.float32 else dtype, "logits")
+    assert bool((logits[:, 0] == 7).all()) and bool((logits[:, E + 1] == 7).all())
+    dx = torch.empty(S, M, dtype=dtype, device=DEV)
+    ops.gate_dgrad(dld, 1, wd, dx)
+    assert_close(dx, dl[:, 1:E + 1] @ w.float(), dtype, "dx")
+    dw = torch.zeros(E, M, dtype=dtype, device=DEV)
+    ops.gate_wgrad(dld, 1, xd, dw, False)
+    want = dl[:, 1:E + 1].T @ x.float()
+    assert_close(dw, want, dtype, "dw")
+    first = dw.clone()
+    ops.gate_wgrad(dld, 1, xd, dw, True)
+    assert_close(dw, first.float().cpu() + want, dtype, "dw accumulated")
+    ops.gate_wgrad(dld, 1, xd, dw, False)
+    assert torch.equal(dw, first)                                  # fixed summation order: bit-identical repeat
+
+
+def test_gate_streaming_kernels_limits():
+    from rtp_amd import ops
+    from rtp_amd._lib import RtpError
+    x = torch.zeros(8, 64, dtype=torch.bfloat16, device=DEV)
+    assert not ops.gate_supported(x, torch.zeros(17, 64, dtype=torch.bfloat16, device=DEV))   # too many experts
+    assert not ops.gate_supported(x[:, :60], torch.zeros(4, 60, dtype=torch.bfloat16, device=DEV))  # 60 % 8 != 0
+    assert not ops.gate_supported(x[:, 1:9], torch.zeros(4, 8, dtype=torch.bfloat16, device=DEV))   # misaligned rows
+    with pytest.raises(RtpError):
+        ops.gate_fwd(x, torch.zeros(17, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(8, 17, device=DEV), 0)
