@@ -357,7 +357,7 @@ class _DecoderLayer(nn.Module):
 
     def forward(self, x):
         L = x.shape[0]
-        mask = torch.triu(torch.full((L, L), float("-inf")), diagonal=1)      # :201-204
+        mask = torch.triu(torch.full((L, L), float("-inf"), dtype=x.dtype), diagonal=1)      # :201-204
         x = self.norm1(x + self.self_attn(x, x, x, attn_mask=mask, need_weights=False)[0])
         return self.norm2(x + self.linear2(F.relu(self.linear1(x))))
 

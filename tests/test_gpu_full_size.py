@@ -1,0 +1,173 @@
+"""BASELINE's full-size configurations 4 (10-layer LM) and 5 (MoE layer) on the GPU: parity with the CPU oracle where
+it finishes in seconds, and size-independent properties (causality, shard-count invariance, determinism, a descent
+step).  One rotation schedule (all shards of a layer staged together), since each case is large."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from gpu_util import DEV, assert_close, rel_err
+from oracle import rtp_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def test_lm_headline_config_full_size_fp32_against_oracle():
+    """vocab 10240, d_model 2048, 32 heads, d_ff 2048, 10 layers, seq 32, batch 32, 8 shards, fp32: loss, logits and
+    the gradients against the CPU oracle.  Loss and logits: 1e-5.  Gradients: at this size a handful of the 21 million
+    ReLU inputs sit within fp32 rounding of zero, and a unit that is on in one fp32 evaluation and off in another
+    moves a weight-gradient row by one token's contribution -- two correct fp32 implementations then differ by
+    ~1e-3 of the largest entry.  So the yardstick is the oracle evaluated in fp64: every gradient must be within 5e-5
+    of it, or within 3x the worst distance of the stock fp32 CPU evaluation from it (which units flip differs between
+    two evaluations, so the bound is the worst over all parameters, not per parameter).  A wrong shard, a missing term
+    or a wrong scale is an O(1) error and still fails."""
+    import copy
+    from test_gpu_lm import build_pair, gathered_grads, ref_grads
+    V, D, H, Fd, n_dec, L, N, ws = 10240, 2048, 32, 2048, 10, 32, 32, 8
+    lm, ref = build_pair(V, D, H, Fd, n_dec, ws, torch.float32, seed=11)
+    assert sum(p.numel() for p in ref.parameters()) == 293_816_320
+    gen = torch.Generator().manual_seed(12)
+    ids = torch.randint(0, V, (L, N), generator=gen)
+    tgt = torch.randint(0, V, (L, N), generator=gen)
+    logits = lm(ids.to(DEV))
+    loss = F.cross_entropy(logits.view(-1, V), tgt.to(DEV).view(-1))
+    loss.backward()
+    ref64 = copy.deepcopy(ref).double()
+    ref_logits = ref(ids)
+    ref_loss = F.cross_entropy(ref_logits.view(-1, V), tgt.view(-1))
+    ref_loss.backward()
+    F.cross_entropy(ref64(ids).view(-1, V), tgt.view(-1)).backward()
+    assert abs(float(loss.detach()) - float(ref_loss.detach())) <= 1e-5 * abs(float(ref_loss.detach()))
+    assert_close(logits, ref_logits, torch.float32, "logits")
+    mine, cpu32, truth = gathered_grads(lm, ws), ref_grads(ref), ref_grads(ref64)
+    rows = sorted(((rel_err(mine[k], truth[k]), rel_err(cpu32[k], truth[k]), k) for k in truth), reverse=True)
+    print("gradient error vs fp64 (device fp32, CPU fp32):", [(f"{a:.1e}", f"{b:.1e}", k) for a, b, k in rows[:4]])
+    bound = max(5e-5, 3.0 * max(cpu_err for _, cpu_err, _ in rows))
+    assert bound < 5e-2, f"the fp32 oracle itself is {bound / 3:.1e} from fp64: the comparison would prove nothing"
+    for dev_err, cpu_err, k in rows:
+        assert dev_err <= bound, f"{k}: device {dev_err:.3e}, CPU fp32 {cpu_err:.3e}, bound {bound:.1e}"
+
+
+def test_lm_headline_config_full_size_bf16():
+    """The benchmark's configuration itself (bf16 weights, fp32 accumulation): loss, logits and the last layers'
+    gradients against the fp32 oracle to the bf16 bound (2e-2) -- deeper gradients are not compared with fp32, a bf16
+    activation that crosses a ReLU kink or tips a near-one-hot softmax moves them by more than rounding --, then
+    size-independent properties: causality, determinism, shard-count invariance, a descent step."""
+    from test_gpu_lm import build_pair, gathered_grads, load_unsharded, ref_grads
+    from rtp_amd.models.transformer_lm_rtp import TransformerLM
+    from rtp_amd.module.loss import cross_entropy
+    from rtp_amd.optim import RotatedSGD
+    V, D, H, Fd, n_dec, L, N, ws = 10240, 2048, 32, 2048, 10, 32, 32, 8
+    lm, ref = build_pair(V, D, H, Fd, n_dec, ws, torch.bfloat16, seed=11)
+    gen = torch.Generator().manual_seed(12)
+    ids = torch.randint(0, V, (L, N), generator=gen)
+    tgt = torch.randint(0, V, (L, N), generator=gen)
+    idd, tgd = ids.to(DEV), tgt.to(DEV)
+    logits = lm(idd)
+    loss = cross_entropy(logits.view(-1, V), tgd.view(-1))
+    loss.backward()
+    ref_logits = ref(ids)
+    ref_loss = F.cross_entropy(ref_logits.view(-1, V), tgt.view(-1))
+    ref_loss.backward()
+    assert abs(float(loss.detach()) - float(ref_loss.detach())) <= 2e-2 * abs(float(ref_loss.detach()))
+    assert_close(logits, ref_logits, torch.bfloat16, "logits")
+    mine, theirs = gathered_grads(lm, ws), ref_grads(ref)
+    for k in ("head_w", "head_b", "l9.w2", "l9.b2"):
+        assert_close(mine[k], theirs[k], torch.bfloat16, k)
+    with torch.no_grad():
+        # causality: another token at the last position leaves every earlier position's logits bit for bit
+        ids2 = idd.clone()
+        ids2[-1] = (ids2[-1] + 1) % V
+        assert torch.equal(lm(ids2)[:-1], logits[:-1])
+        # determinism
+        assert torch.equal(lm(idd), logits)
+        # the same master weights cut into 2 shards instead of 8: sums are re-associated, nothing else changes
+        lm2 = TransformerLM(V, D, H, Fd, 0.0, 0.1, n_dec, 2, 0, device=DEV, dtype=torch.bfloat16)
+        load_unsharded(lm2, ref)
+        assert_close(lm2(idd), logits.float(), torch.bfloat16, "2 shards vs 8 shards")
+        del lm2
+    # a descent step on the same batch lowers the loss
+    opt = RotatedSGD(lm, lr=0.05)
+    opt.step()
+    with torch.no_grad():
+        after = cross_entropy(lm(idd).view(-1, V), tgd.view(-1))
+    assert float(after) < float(loss.detach())
+
+
+def _moe_config5(dtype, seed=31):
+    from test_gpu_moe import _moe_from_tensors
+    gen = torch.Generator().manual_seed(seed)
+    E, M, Fd, S, ws = 8, 2048, 8192, 4096, 8
+    wg = (torch.rand(E, M, generator=gen) * 0.2 - 0.1).to(dtype).float()
+    experts = [tuple((torch.rand(s, generator=gen) * 0.04 - 0.02).to(dtype).float()
+                     for s in ((Fd, M), (Fd,), (M, Fd), (M,))) for _ in range(E)]
+    x = torch.randn(8, S // 8, M, generator=gen).to(dtype)
+    coef = torch.randn(8, S // 8, M, generator=gen).to(dtype)
+    noise = O.gumbel_noise((S, E), gen)
+    return wg, experts, x, coef, noise, _moe_from_tensors(wg, experts, ws, dtype), ws
+
+
+def _close_but_for_relu_flips(a, b, tol, what):
+    """Entry-wise |a - b| <= tol * max|b| for all but 1 % of the entries, and nowhere beyond 0.5 * max|b|.  Among the
+    67 million ReLU inputs of this configuration a few dozen sit within fp32 rounding of zero; which side such a unit
+    falls on differs between two correct fp32 evaluations and moves one row of a weight gradient (or one token's input
+    gradient) by that token's whole contribution -- up to ~10 % of the largest entry.  A wrong shard, scale or term
+    moves most entries."""
+    a, b = a.detach().double().cpu().flatten(), b.detach().double().cpu().flatten()
+    err = (a - b).abs() / b.abs().max()
+    k = max(1, int(0.99 * err.numel()))
+    q99 = float(torch.kthvalue(err, k).values)
+    assert q99 <= tol, f"{what}: 99th percentile of the error {q99:.3e} > {tol:.0e}"
+    assert float(err.max()) <= 0.5, f"{what}: largest error {float(err.max()):.3e} of the largest entry"
+
+
+def test_moe_headline_config_full_size_fp32_against_oracle():
+    """8 experts in 8 shards, top-2, d_model 2048, d_ff 8192, 4096 tokens, fp32, against the dense-einsum oracle:
+    output and l_aux to 1e-5 / 1e-6, gradients that do not pass a ReLU to 1e-5, the others to 1e-5 but for ReLU flips."""
+    wg, experts, x, coef, noise, layer, ws = _moe_config5(torch.float32)
+    xd = x.to(DEV).requires_grad_()
+    out = layer(xd, noise=noise.to(DEV))
+    ((out * coef.to(DEV)).sum() + layer.l_aux).backward()
+    wgo = wg.clone().requires_grad_()
+    eo = [tuple(p.clone().requires_grad_() for p in e) for e in experts]
+    xo = x.clone().requires_grad_()
+    ref, l_aux = O.moe_layer(xo, wgo, eo, noise, ws)
+    ((ref * coef).sum() + l_aux).backward()
+    assert_close(out, ref, torch.float32, "output")
+    assert abs(float(layer.l_aux.detach()) - float(l_aux.detach())) <= 1e-6
+    _close_but_for_relu_flips(xd.grad, xo.grad, 1e-5, "input grad")
+    for s in (0, 5):
+        w1, b1, w2, b2 = layer.experts_list[s].parameters()
+        _close_but_for_relu_flips(w1.grad, eo[s][0].grad, 1e-5, f"expert {s} linear1.weight grad")
+        _close_but_for_relu_flips(b1.grad, eo[s][1].grad, 1e-5, f"expert {s} linear1.bias grad")
+        assert_close(w2.grad, eo[s][2].grad, torch.float32, f"expert {s} linear2.weight grad")
+        assert_close(b2.grad, eo[s][3].grad, torch.float32, f"expert {s} linear2.bias grad")
+    _close_but_for_relu_flips(torch.cat([w.weight.grad for w in layer.gate.wgs], 0), wgo.grad, 1e-5, "gate grad")
+
+
+def test_moe_headline_config_full_size_bf16_properties():
+    """The same configuration in bf16: bit-identical repeat, routing within capacity, every kept token's output is
+    the weighted sum of its two experts' rows (checked on the device's own routing with the oracle's expert FFN)."""
+    from rtp_amd.module.top2gate import top2_route
+    wg, experts, x, coef, noise, layer, ws = _moe_config5(torch.bfloat16)
+    xd = x.to(DEV)
+    with torch.no_grad():
+        out = layer(xd, noise=noise.to(DEV))
+        assert torch.equal(layer(xd, noise=noise.to(DEV)), out)
+        r, weight, _ = layer.gate.route(xd.view(-1, x.shape[-1]), noise.to(DEV))
+    S, E = noise.shape
+    expert, slot, keep = r.expert.cpu().long(), r.slot.cpu().long(), r.keep.cpu().bool()
+    assert expert.shape == (S, 2) and int(r.capacity) == 2 * S // E
+    assert bool((slot[keep] < r.capacity).all()) and bool((expert[:, 0] != expert[:, 1]).all())
+    # (expert, slot) pairs of kept assignments are unique: no two tokens share a capacity slot
+    flat = (expert * int(r.capacity) + slot)[keep]
+    assert flat.unique().numel() == flat.numel()
+    # a sample of tokens against the closed form out[s] = w1 * ffn_e1(x[s]) + w2 * ffn_e2(x[s])
+    w = weight.float().cpu()
+    xs = x.view(-1, x.shape[-1]).float()
+    sample = torch.arange(0, S, 97)
+    want = torch.zeros(sample.numel(), x.shape[-1])
+    for i, s in enumerate(sample.tolist()):
+        for c in range(2):
+            if keep[s, c]:
+                want[i] += w[s, c] * O.expert_ffn(xs[s:s + 1], *experts[int(expert[s, c])])[0]
+    assert_close(out.view(-1, x.shape[-1])[sample.to(DEV)], want, torch.bfloat16, "sampled outputs")
