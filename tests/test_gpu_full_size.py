@@ -1,4 +1,4 @@
-"""BASELINE's full-size configurations 4 (10-layer LM) and 5 (MoE layer) on the GPU: parity with the CPU oracle where
+"""The benchmark configurations at full size -- the 10-layer LM and the MoE layer -- on the GPU: parity with the CPU oracle where
 it finishes in seconds, and size-independent properties (causality, shard-count invariance, determinism, a descent
 step).  One rotation schedule (all shards of a layer staged together), since each case is large."""
 import pytest
