@@ -279,6 +279,21 @@ int rtp_layernorm_bwd(void* stream, int dtype, const void* dy, const void* z, co
                       const float* mean, const float* rstd, int64_t rows, int64_t cols, void* dz,
                       void* dgamma, void* dbeta, void* workspace, size_t workspace_bytes);
 
+/* Deferred parameter gradients: rtp_layernorm_bwd with dgamma == NULL writes dz and leaves the per-block partial
+ * sums [rtp_layernorm_bwd_blocks(rows)][2][cols] (fp32) in `workspace`; rtp_layernorm_bwd_finalize then reduces the
+ * partial sums of MANY LayerNorms (same dtype) in one launch -- a caller that only needs dgamma / dbeta when the
+ * backward pass ends saves a launch per layer.  `items` is a table in DEVICE memory; max_cols = the widest entry. */
+typedef struct {
+  const float* part; /* the workspace of that layer's rtp_layernorm_bwd call */
+  int64_t nblocks;   /* rtp_layernorm_bwd_blocks(rows) */
+  int64_t cols;
+  void* dgamma;
+  void* dbeta; /* may be NULL */
+} rtp_ln_final_item;
+int64_t rtp_layernorm_bwd_blocks(int64_t rows);
+int rtp_layernorm_bwd_finalize(void* stream, int dtype, const rtp_ln_final_item* items, int64_t n_items,
+                               int64_t max_cols);
+
 /* ---------------------------------------------------------------------------------------------
  * Softmax cross-entropy over the vocabulary axis of the LM's logits (reference harness:
  * nn.CrossEntropyLoss()(outputs.view(-1, vocab_size), labels.view(-1)), test_transformer.py:195-197,

@@ -98,6 +98,8 @@ PROTOTYPES = {
     "rtp_layernorm_supported": (_i, [_i, _i64]),
     "rtp_add_layernorm_fwd": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _f, _i64, _i64, _vp, _vp, _vp, _vp]),
     "rtp_layernorm_bwd_workspace_bytes": (_sz, [_i64, _i64]),
+    "rtp_layernorm_bwd_blocks": (_i64, [_i64]),
+    "rtp_layernorm_bwd_finalize": (_i, [_vp, _i, _vp, _i64, _i64]),
     "rtp_layernorm_bwd": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _sz]),
     "rtp_softmax_xent_fwd": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _vp, _vp, _vp]),
     "rtp_softmax_xent_bwd": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _i64]),

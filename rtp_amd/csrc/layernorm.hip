@@ -214,8 +214,7 @@ __global__ __launch_bounds__(kLnThreads) void layernorm_bwd_kernel(const T* dy, 
 // 32 columns of the [2][cols] sums per workgroup: 8 groups of threads each add an eighth of the blocks (a fixed
 // order, sixteen loads in flight), then the eighths are added in order.
 template <typename T>
-__global__ __launch_bounds__(256) void layernorm_bwd_final_kernel(const float* part, long nblocks, int cols, T* dgamma,
-                                                                  T* dbeta) {
+__device__ __forceinline__ void ln_final_columns(const float* part, long nblocks, int cols, T* dgamma, T* dbeta) {
   __shared__ float eighth[8][32];
   const int cl = threadIdx.x & 31, grp = threadIdx.x >> 5;
   const int c = blockIdx.x * 32 + cl;  // column of the [2 * cols] row
@@ -248,6 +247,26 @@ __global__ __launch_bounds__(256) void layernorm_bwd_final_kernel(const float* p
       dbeta[c - cols] = from_f32<T>(s);
     }
   }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void layernorm_bwd_final_kernel(const float* part, long nblocks, int cols, T* dgamma,
+                                                                  T* dbeta) {
+  ln_final_columns<T>(part, nblocks, cols, dgamma, dbeta);
+}
+
+// The same reduction for many LayerNorms in one launch: blockIdx.y picks the entry of a device-resident table.  Their
+// parameter gradients are not needed before the backward pass ends, so one launch there replaces one per layer.
+struct LnFinalItem {
+  const float* part;
+  long nblocks, cols;
+  void *dgamma, *dbeta;
+};
+template <typename T>
+__global__ __launch_bounds__(256) void layernorm_bwd_final_many_kernel(const LnFinalItem* items) {
+  const LnFinalItem it = items[blockIdx.y];
+  if ((long)blockIdx.x * 32 >= 2 * it.cols) return;  // the grid is sized for the widest entry
+  ln_final_columns<T>(it.part, it.nblocks, (int)it.cols, (T*)it.dgamma, (T*)it.dbeta);
 }
 
 static int ln_nv(int dtype, int64_t cols) {
@@ -308,7 +327,8 @@ extern "C" size_t rtp_layernorm_bwd_workspace_bytes(int64_t rows, int64_t cols) 
 extern "C" int rtp_layernorm_bwd(void* stream, int dtype, const void* dy, const void* z, const void* gamma,
                                  const float* mean, const float* rstd, int64_t rows, int64_t cols, void* dz,
                                  void* dgamma, void* dbeta, void* workspace, size_t workspace_bytes) {
-  RTP_REQUIRE(dy && z && gamma && mean && rstd && dz && dgamma && workspace, "rtp_layernorm_bwd: null pointer");
+  RTP_REQUIRE(dy && z && gamma && mean && rstd && dz && workspace, "rtp_layernorm_bwd: null pointer");
+  RTP_REQUIRE(dgamma || !dbeta, "rtp_layernorm_bwd: dbeta without dgamma");
   RTP_REQUIRE(rows >= 1 && rows < (1ll << 31), "rtp_layernorm_bwd: row count %lld out of range", (long long)rows);
   const int nv = ln_nv(dtype, cols);
   RTP_REQUIRE((dtype == RTP_F32 || dtype == RTP_BF16) && nv,
@@ -328,14 +348,39 @@ extern "C" int rtp_layernorm_bwd(void* stream, int dtype, const void* dy, const 
   if (dtype == RTP_F32) {
     RTP_LN_DISPATCH(layernorm_bwd_kernel, float, nv, grid, block, lds, st, (const float*)dy, (const float*)z,
                     (const float*)gamma, mean, rstd, (long)rows, (int)cols, (float*)dz, part)
-    hipLaunchKernelGGL(layernorm_bwd_final_kernel<float>, dim3((unsigned)ceil_div(2 * cols, 32)), block, 0, st, part,
-                       (long)nblocks, (int)cols, (float*)dgamma, (float*)dbeta);
+    if (dgamma)
+      hipLaunchKernelGGL(layernorm_bwd_final_kernel<float>, dim3((unsigned)ceil_div(2 * cols, 32)), block, 0, st, part,
+                         (long)nblocks, (int)cols, (float*)dgamma, (float*)dbeta);
   } else {
     RTP_LN_DISPATCH(layernorm_bwd_kernel, bf16_t, nv, grid, block, lds, st, (const bf16_t*)dy, (const bf16_t*)z,
                     (const bf16_t*)gamma, mean, rstd, (long)rows, (int)cols, (bf16_t*)dz, part)
-    hipLaunchKernelGGL(layernorm_bwd_final_kernel<bf16_t>, dim3((unsigned)ceil_div(2 * cols, 32)), block, 0, st, part,
-                       (long)nblocks, (int)cols, (bf16_t*)dgamma, (bf16_t*)dbeta);
+    if (dgamma)
+      hipLaunchKernelGGL(layernorm_bwd_final_kernel<bf16_t>, dim3((unsigned)ceil_div(2 * cols, 32)), block, 0, st, part,
+                         (long)nblocks, (int)cols, (bf16_t*)dgamma, (bf16_t*)dbeta);
   }
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
+}
+
+extern "C" int64_t rtp_layernorm_bwd_blocks(int64_t rows) { return rows <= 0 ? 0 : ceil_div(rows, kLnBwdRows); }
+
+extern "C" int rtp_layernorm_bwd_finalize(void* stream, int dtype, const rtp_ln_final_item* items, int64_t n_items,
+                                          int64_t max_cols) {
+  static_assert(sizeof(rtp_ln_final_item) == sizeof(LnFinalItem), "rtp_ln_final_item layout");
+  RTP_REQUIRE(items, "rtp_layernorm_bwd_finalize: null table");
+  RTP_REQUIRE(dtype == RTP_F32 || dtype == RTP_BF16, "rtp_layernorm_bwd_finalize: unknown dtype %d", dtype);
+  RTP_REQUIRE(n_items >= 0 && n_items < 65536, "rtp_layernorm_bwd_finalize: %lld entries out of range", (long long)n_items);
+  RTP_REQUIRE(max_cols >= 1 && max_cols <= kLnMaxCols, "rtp_layernorm_bwd_finalize: widest entry %lld out of range",
+              (long long)max_cols);
+  if (n_items == 0) return RTP_OK;
+  hipStream_t st = (hipStream_t)stream;
+  ProfileScope prof(st, "layernorm_bwd_finalize", 0.0, 0.0);
+  const dim3 grid((unsigned)ceil_div(2 * max_cols, 32), (unsigned)n_items);
+  const LnFinalItem* table = reinterpret_cast<const LnFinalItem*>(items);
+  if (dtype == RTP_F32)
+    hipLaunchKernelGGL(layernorm_bwd_final_many_kernel<float>, grid, dim3(256), 0, st, table);
+  else
+    hipLaunchKernelGGL(layernorm_bwd_final_many_kernel<bf16_t>, grid, dim3(256), 0, st, table);
   RTP_LAUNCH_CHECK();
   return RTP_OK;
 }

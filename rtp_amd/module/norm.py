@@ -3,10 +3,60 @@ norm1(x + sa_block(x)) / norm2(x + ff_block(x)) with two ATen calls each way,
 rtp/models/transformer_lm_rtp.py:176-177).  The LayerNorm parameters stay ordinary nn.LayerNorm parameters."""
 from __future__ import annotations
 
+import os
+
 import torch
 import torch.nn as nn
 
 from .. import ops
+
+
+class _DeferredParamGrads:
+    """LayerNorm parameter gradients whose reduction waits for the end of the backward pass: each layer's backward
+    leaves per-block partial sums in a buffer of its own, and ONE launch reduces all of them when autograd is done
+    (nobody reads a parameter gradient earlier).  Only for gradients that go straight into an optimiser's persistent
+    slices; the device table is rebuilt only when a buffer moved."""
+
+    def __init__(self):
+        self.pending = {}   # device index -> [(part, rows, cols, dgamma, dbeta, weight)]
+        self.armed = set()  # device indices with a callback queued in the running backward pass
+        self.tables = {}    # (device index, dtype) -> (key, table, max_cols)
+
+    def add(self, device: torch.device, item) -> bool:
+        idx = device.index if device.index is not None else torch.cuda.current_device()
+        if idx not in self.armed:
+            try:
+                torch.autograd.Variable._execution_engine.queue_callback(lambda: self.flush(idx))
+            except RuntimeError:
+                return False  # not inside a backward pass: the caller reduces at once
+            self.armed.add(idx)
+        self.pending.setdefault(idx, []).append(item)
+        item[5]._rtp_ln_pending = True
+        return True
+
+    def flush(self, idx: int) -> None:
+        self.armed.discard(idx)
+        items = self.pending.pop(idx, [])
+        if not items:
+            return
+        for it in items:
+            it[5]._rtp_ln_pending = False
+        by_dtype = {}
+        for it in items:
+            by_dtype.setdefault(it[3].dtype, []).append(it)
+        for dtype, group in by_dtype.items():
+            key = tuple((it[0].data_ptr(), it[1], it[2], it[3].data_ptr(), it[4].data_ptr() if it[4] is not None else 0)
+                        for it in group)
+            cached = self.tables.get((idx, dtype))
+            if cached is None or cached[0] != key:
+                cached = (key, ops.layernorm_final_table([it[:5] for it in group], group[0][0].device),
+                          max(it[2] for it in group))
+                self.tables[(idx, dtype)] = cached
+            ops.layernorm_finalize(cached[1], dtype, cached[2])
+
+
+_deferred = _DeferredParamGrads()
+_DEFER = os.environ.get("RTP_LN_DEFER", "1") != "0"  # 0: reduce each LayerNorm's parameter gradients in its own backward
 
 
 class _AddLayerNormFn(torch.autograd.Function):
@@ -39,7 +89,22 @@ class _AddLayerNormFn(torch.autograd.Function):
         else:
             dgamma = torch.empty_like(weight)
             dbeta = torch.empty_like(weight) if bias is not None else None
-        ops.layernorm_bwd(dy.contiguous(), z, weight, mean, rstd, dz, dgamma, dbeta)
+        if direct and not _DEFER:
+            ops.layernorm_bwd(dy.contiguous(), z, weight, mean, rstd, dz, dgamma, dbeta)
+        elif direct:
+            # reduced together with every other LayerNorm's when the backward pass ends
+            part = ops.layernorm_bwd_deferred(dy.contiguous(), z, weight, mean, rstd, dz,
+                                              getattr(weight, "_rtp_ln_part", None))
+            weight._rtp_ln_part = part
+            done = _deferred.add(z.device, (part, z.numel() // z.shape[-1], z.shape[-1], dgamma, dbeta, weight))
+            if not done:
+                ops.layernorm_finalize(ops.layernorm_final_table(
+                    [(part, z.numel() // z.shape[-1], z.shape[-1], dgamma, dbeta)], z.device), z.dtype, z.shape[-1])
+        else:
+            if getattr(weight, "_rtp_ln_pending", False):
+                # the same LayerNorm applied twice: its first gradient must be in place before autograd adds this one
+                _deferred.flush(z.device.index if z.device.index is not None else torch.cuda.current_device())
+            ops.layernorm_bwd(dy.contiguous(), z, weight, mean, rstd, dz, dgamma, dbeta)
         if direct:
             ws.overwrite = False
             weight.grad = ws.view

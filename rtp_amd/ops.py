@@ -423,6 +423,45 @@ def layernorm_bwd(dy: torch.Tensor, z: torch.Tensor, gamma: torch.Tensor, mean: 
                                 dbeta.data_ptr() if dbeta is not None else None, ws.data_ptr(), nbytes))
 
 
+def layernorm_bwd_deferred(dy: torch.Tensor, z: torch.Tensor, gamma: torch.Tensor, mean: torch.Tensor,
+                           rstd: torch.Tensor, dz: torch.Tensor, part: Optional[torch.Tensor]) -> torch.Tensor:
+    """layernorm_bwd without the reduction of the parameter gradients: writes dz and leaves the per-block partial sums
+    in `part` (allocated when None or too small; the caller keeps it until layernorm_finalize has run)."""
+    _dev(dy)
+    cols = z.shape[-1]
+    rows = z.numel() // max(cols, 1)
+    if any(t.dtype != z.dtype or t.shape != z.shape or not t.is_contiguous() for t in (dy, dz)) or \
+            not z.is_contiguous():
+        raise ValueError("layernorm_bwd_deferred: dy, z, dz must be contiguous, of one shape and dtype")
+    _lib.require_device()
+    lib = _lib.load()
+    nbytes = lib.rtp_layernorm_bwd_workspace_bytes(rows, cols)
+    if part is None or part.numel() < nbytes or part.device != z.device:
+        part = torch.empty(nbytes, dtype=torch.uint8, device=z.device)
+    check(lib.rtp_layernorm_bwd(_stream(), dtype_code(z.dtype), dy.data_ptr(), z.data_ptr(), gamma.data_ptr(),
+                                mean.data_ptr(), rstd.data_ptr(), rows, cols, dz.data_ptr(), None, None,
+                                part.data_ptr(), part.numel()))
+    return part
+
+
+def layernorm_final_table(items, device) -> torch.Tensor:
+    """Device table for layernorm_finalize: items = [(part, rows, cols, dgamma, dbeta or None), ...]."""
+    lib = _lib.load()
+    rows = []
+    for part, n_rows, cols, dgamma, dbeta in items:
+        rows.append([part.data_ptr(), lib.rtp_layernorm_bwd_blocks(n_rows), cols, dgamma.data_ptr(),
+                     dbeta.data_ptr() if dbeta is not None else 0])
+    return torch.tensor(rows, dtype=torch.int64).to(device)
+
+
+def layernorm_finalize(table: torch.Tensor, dtype: torch.dtype, max_cols: int) -> None:
+    """dgamma / dbeta of every LayerNorm in `table` from its partial sums, one launch."""
+    _dev(table)
+    _lib.require_device()
+    check(_lib.load().rtp_layernorm_bwd_finalize(_stream(), dtype_code(dtype), table.data_ptr(), table.shape[0],
+                                                 max_cols))
+
+
 def softmax_xent_supported(logits: torch.Tensor) -> bool:
     if logits.dtype not in (torch.float32, torch.bfloat16) or logits.dim() != 2 or not logits.is_cuda:
         return False

@@ -53,3 +53,42 @@ def test_add_layer_norm_falls_back_for_unsupported_rows():
     x = torch.randn(4, 38, device=DEV)
     r = torch.randn(4, 38, device=DEV)
     assert torch.equal(add_layer_norm(x, r, norm), norm(x + r))
+
+
+def test_layer_norm_parameter_gradients_reduced_at_the_end_of_backward():
+    """With an optimiser's persistent gradient slices, every LayerNorm's backward leaves partial sums and one launch
+    at the end of the backward pass reduces all of them: same gradients as torch, also for a LayerNorm applied twice
+    in one forward pass (its second gradient is accumulated by autograd after the first is in place) and over
+    repeated steps (the device table is reused)."""
+    import torch.nn as nn
+    from rtp_amd.module.norm import add_layer_norm
+    from rtp_amd.optim import RotatedSGD
+
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.n1, self.n2 = nn.LayerNorm(64), nn.LayerNorm(64)
+
+        def forward(self, x, fused):
+            f = (lambda a, b, n: add_layer_norm(a, b, n)) if fused else (lambda a, b, n: n(a + b))
+            h = f(x, x * 0.5, self.n1)
+            h = f(h, x, self.n2)
+            return f(h, h * 2.0, self.n1)            # n1 a second time
+
+    torch.manual_seed(0)
+    ref = Net()
+    with torch.no_grad():
+        for p in ref.parameters():
+            p.add_(torch.randn_like(p) * 0.1)
+    net = Net().to(DEV)
+    net.load_state_dict(ref.state_dict())
+    opt = RotatedSGD(net, lr=0.0)
+    for step in range(3):
+        x = torch.randn(40, 64)
+        g = torch.randn(40, 64)
+        opt.zero_grad()
+        ref.zero_grad()
+        net(x.to(DEV), True).backward(g.to(DEV))
+        ref(x, False).backward(g)
+        for (k, p), q in zip(net.named_parameters(), ref.parameters()):
+            assert_close(p.grad, q.grad, torch.float32, f"step {step} {k}")
