@@ -206,13 +206,16 @@ int rtp_embedding_scatter_add_det(void* stream, int dtype, const void* grad_out,
 /* ---------------------------------------------------------------------------------------------
  * Attention softmax (reference: rtp/module/functional.py:779-792 baddbmm+softmax, :825
  * scaled_dot_product_attention with an additive float mask).
- *   fwd: p[z,i,j] = softmax_j( scale*s[z,i,j] + mask[i,j] )  (and j <= i + (S-L) only, if causal)
- *        s fp32 [Z,L,S] contiguous, mask fp32 [L,S] or NULL, p `dtype` [Z,L,S].
+ *   fwd: p[z,i,j] = softmax_j( scale*s[z,i,j] + mask[i,j] + key_bias[b,j] )  (and j <= i + (S-L) only, if causal)
+ *        s fp32 [Z,L,S] contiguous, mask fp32 [L,S] or NULL, p `dtype` [Z,L,S]; key_bias fp32 [n_batch,S] or NULL is
+ *        the key padding mask (0 / -inf, functional.py:760-768 merges it into the mask per batch), with
+ *        z = (group * n_batch + b) * heads + head.
  *   bwd: ds[z,i,j] = scale * p * (dp - sum_j dp*p)           dp fp32, ds `dtype`.
  * One wavefront per row, fp32 max/sum by cross-lane reduction.
  * --------------------------------------------------------------------------------------------- */
-int rtp_softmax_fwd(void* stream, int dtype, const float* s, const float* mask, int causal,
-                    float scale, int64_t z, int64_t l, int64_t skv, void* p);
+int rtp_softmax_fwd(void* stream, int dtype, const float* s, const float* mask, const float* key_bias,
+                    int64_t n_batch, int64_t heads, int causal, float scale, int64_t z, int64_t l, int64_t skv,
+                    void* p);
 int rtp_softmax_bwd(void* stream, int dtype, const void* p, const float* dp, float scale,
                     int64_t z, int64_t l, int64_t skv, void* ds);
 
@@ -225,15 +228,16 @@ int rtp_softmax_bwd(void* stream, int dtype, const void* p, const float* dp, flo
  * stored p.  Element (l, b, h, g, dd) of q/k/v/dq/dk/dv is at base + l*s_l + b*s_b + h*s_h + g*s_g + dd, of
  * o/dout at base + l*o_l + b*o_b + h*o_h + g*o_g + dd (strides in elements, multiples of 8; bases 16-byte
  * aligned).  p is [G][N][H][L][L] bf16, written by fwd and read by bwd.  mask: additive fp32 [L][L] or
- * NULL; causal != 0 hides keys j > i.  scale multiplies the scores before the mask is added.
- *   fwd: p = softmax(scale * q k^T + mask), o = p v
+ * NULL; key_bias: additive fp32 [N][L] per (batch, key) or NULL (the key padding mask: 0 / -inf); causal != 0
+ * hides keys j > i.  scale multiplies the scores before the masks are added.
+ *   fwd: p = softmax(scale * q k^T + mask + key_bias), o = p v
  *   bwd: dv = p^T dout, dp = dout v^T, ds = scale * p o (dp - rowsum(dp o p)), dq = ds k, dk = ds^T q
  * --------------------------------------------------------------------------------------------- */
 int rtp_attn_supported(int dtype, int64_t L, int64_t D);
 int rtp_attn_fwd(void* stream, int dtype, const void* q, const void* k, const void* v, int64_t s_l,
                  int64_t s_b, int64_t s_h, int64_t s_g, void* o, int64_t o_l, int64_t o_b, int64_t o_h,
-                 int64_t o_g, void* p, const float* mask, int causal, float scale, int64_t L, int64_t N,
-                 int64_t H, int64_t D, int64_t G);
+                 int64_t o_g, void* p, const float* mask, const float* key_bias, int causal, float scale,
+                 int64_t L, int64_t N, int64_t H, int64_t D, int64_t G);
 int rtp_attn_bwd(void* stream, int dtype, const void* q, const void* k, const void* v, int64_t s_l,
                  int64_t s_b, int64_t s_h, int64_t s_g, const void* dout, int64_t o_l, int64_t o_b,
                  int64_t o_h, int64_t o_g, const void* p, void* dq, void* dk, void* dv, float scale,
@@ -242,7 +246,7 @@ int rtp_attn_bwd(void* stream, int dtype, const void* q, const void* k, const vo
 /* ---------------------------------------------------------------------------------------------
  * Fused attention core for any sequence length (reference: the same per-head-group core,
  * rtp/module/functional.py:779-800 and :815-830, there bmm -> softmax -> bmm with the [L, L] probabilities
- * in memory).  bf16 only, D in {32, 64, 128}; addressing, mask, causal and scale as for rtp_attn_fwd.  One
+ * in memory).  bf16 only, D in {32, 64, 128}; addressing, mask, key_bias, causal and scale as for rtp_attn_fwd.  One
  * wavefront per (group, batch, head, 32-query block) walks the keys in blocks of 32 with a running softmax;
  * the probabilities are never stored.  lse and delta are fp32 [G][N][H][L].
  *   fwd: o = softmax(scale * q k^T + mask) v,  lse = log sum_j exp(scale * q k_j + mask_j)
@@ -253,13 +257,13 @@ int rtp_attn_bwd(void* stream, int dtype, const void* q, const void* k, const vo
 int rtp_attn_flash_supported(int dtype, int64_t L, int64_t D);
 int rtp_attn_flash_fwd(void* stream, int dtype, const void* q, const void* k, const void* v, int64_t s_l,
                        int64_t s_b, int64_t s_h, int64_t s_g, void* o, int64_t o_l, int64_t o_b, int64_t o_h,
-                       int64_t o_g, float* lse, const float* mask, int causal, float scale, int64_t L,
-                       int64_t N, int64_t H, int64_t D, int64_t G);
+                       int64_t o_g, float* lse, const float* mask, const float* key_bias, int causal, float scale,
+                       int64_t L, int64_t N, int64_t H, int64_t D, int64_t G);
 int rtp_attn_flash_bwd(void* stream, int dtype, const void* q, const void* k, const void* v, int64_t s_l,
                        int64_t s_b, int64_t s_h, int64_t s_g, const void* o, const void* dout, int64_t o_l,
                        int64_t o_b, int64_t o_h, int64_t o_g, const float* lse, float* delta, void* dq,
-                       void* dk, void* dv, const float* mask, int causal, float scale, int64_t L, int64_t N,
-                       int64_t H, int64_t D, int64_t G);
+                       void* dk, void* dv, const float* mask, const float* key_bias, int causal, float scale,
+                       int64_t L, int64_t N, int64_t H, int64_t D, int64_t G);
 
 /* ---------------------------------------------------------------------------------------------
  * Residual add + LayerNorm of the post-LN decoder layer (reference: norm1(x + sa_block(x)) and

@@ -83,18 +83,18 @@ PROTOTYPES = {
     "rtp_embedding_sort_ids": (_i, [_vp, _vp, _i64, _vp, _sz]),
     "rtp_embedding_scatter_add_det": (_i, [_vp, _i, _vp, _i64, _i64, _vp, _vp, _i64, _i, _i64, _i64, _i64,
                                            _i64, _i, _i, _i64, _i64, _i64]),
-    "rtp_softmax_fwd": (_i, [_vp, _i, _vp, _vp, _i, _f, _i64, _i64, _i64, _vp]),
+    "rtp_softmax_fwd": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _i64, _i, _f, _i64, _i64, _i64, _vp]),
     "rtp_softmax_bwd": (_i, [_vp, _i, _vp, _vp, _f, _i64, _i64, _i64, _vp]),
     "rtp_attn_supported": (_i, [_i, _i64, _i64]),
-    "rtp_attn_fwd": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _i, _f,
-                          _i64, _i64, _i64, _i64, _i64]),
+    "rtp_attn_fwd": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _i,
+                          _f, _i64, _i64, _i64, _i64, _i64]),
     "rtp_attn_bwd": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp,
                           _f, _i64, _i64, _i64, _i64, _i64]),
     "rtp_attn_flash_supported": (_i, [_i, _i64, _i64]),
-    "rtp_attn_flash_fwd": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _i,
-                                _f, _i64, _i64, _i64, _i64, _i64]),
+    "rtp_attn_flash_fwd": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp,
+                                _i, _f, _i64, _i64, _i64, _i64, _i64]),
     "rtp_attn_flash_bwd": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _vp,
-                                _vp, _vp, _vp, _vp, _vp, _i, _f, _i64, _i64, _i64, _i64, _i64]),
+                                _vp, _vp, _vp, _vp, _vp, _vp, _i, _f, _i64, _i64, _i64, _i64, _i64]),
     "rtp_layernorm_supported": (_i, [_i, _i64]),
     "rtp_add_layernorm_fwd": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _f, _i64, _i64, _vp, _vp, _vp, _vp]),
     "rtp_layernorm_bwd_workspace_bytes": (_sz, [_i64, _i64]),

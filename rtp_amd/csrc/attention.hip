@@ -28,7 +28,8 @@ struct AttnArgs {
   const bf16_t* dout;
   long o_l, o_b, o_h, o_g;
   bf16_t* p;          // probabilities [G][N][H][L][L]
-  const float* mask;  // additive [L][L] or null
+  const float* mask;   // additive [L][L] or null
+  const float* kbias;  // additive per (batch, key) [N][L] or null (a key padding mask: 0 / -inf)
   int causal;
   float scale;
   int L, N, H;
@@ -115,6 +116,7 @@ __device__ __forceinline__ void store_transposed(bf16_t* dst_row, int db, int g,
 
 struct Problem {
   long z, qkv_off, o_off;
+  int b;
   bool live;
 };
 __device__ __forceinline__ Problem locate(const AttnArgs& a, int waves_per_block) {
@@ -125,6 +127,7 @@ __device__ __forceinline__ Problem locate(const AttnArgs& a, int waves_per_block
   const long h = pr.z % a.H, b = (pr.z / a.H) % a.N, g = pr.z / ((long)a.H * a.N);
   pr.qkv_off = b * a.s_b + h * a.s_h + g * a.s_g;
   pr.o_off = b * a.o_b + h * a.o_h + g * a.o_g;
+  pr.b = (int)b;
   return pr;
 }
 
@@ -169,6 +172,16 @@ __global__ __launch_bounds__(NWV * 64) void attn_fwd_small_kernel(AttnArgs a) {
       }
     }
   }
+  float kb[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) kb[r] = 0.0f;
+  if (a.kbias) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int key = 8 * (r >> 2) + 4 * g + (r & 3);
+      kb[r] = a.kbias[(long)pr.b * a.L + (key < a.L ? key : 0)];
+    }
+  }
   {
     bf16_t* const tl[3] = {Qs, Ks, Vs};
     regs.commit(tl, a.L, lane);
@@ -191,7 +204,7 @@ __global__ __launch_bounds__(NWV * 64) void attn_fwd_small_kernel(AttnArgs a) {
   for (int r = 0; r < 16; ++r) {
     const int key = 8 * (r >> 2) + 4 * g + (r & 3);
     const bool visible = key < a.L && (!a.causal || key <= li);
-    const float x = s[r] * a.scale + ((qlive && key < a.L) ? mk[r] : 0.0f);  // outside: an unrelated mask entry
+    const float x = s[r] * a.scale + ((qlive && key < a.L) ? mk[r] + kb[r] : 0.0f);  // outside: unrelated entries
     val[r] = visible ? x : -INFINITY;
     mx = fmaxf(mx, val[r]);
   }
@@ -383,6 +396,7 @@ struct FlashArgs {
   float* lse;               // [G*N*H][L] log-sum-exp of the scaled, masked scores
   float* delta;             // [G*N*H][L] row dot products dO . O (written by the dQ pass, read by the dK/dV pass)
   const float* mask;        // additive [L][L] or null
+  const float* kbias;       // additive per (batch, key) [N][L] or null
   int causal;
   float scale;
   int L, N, H, nblk;  // nblk = ceil(L / 32)
@@ -401,7 +415,7 @@ __device__ __forceinline__ void wave_sync() {
 }
 
 struct FlashItem {
-  int z, blk;
+  int z, blk, b;
   long qkv_off, o_off;
   bool live;
 };
@@ -422,6 +436,7 @@ __device__ __forceinline__ FlashItem flash_locate(const FlashArgs& a, int wave, 
   const unsigned g = zh / (unsigned)a.N, b = zh - g * (unsigned)a.N;
   it.qkv_off = (long)b * a.s_b + (long)h * a.s_h + (long)g * a.s_g;
   it.o_off = (long)b * a.o_b + (long)h * a.o_h + (long)g * a.o_g;
+  it.b = (int)b;
   return it;
 }
 
@@ -472,27 +487,43 @@ struct BlockRegs {
 };
 
 // The 16 additive mask values of lane (li, g), times log2(e), for one query and the keys k0 + 8*(r/4) + 4*g + r%4
-// (`keys_in_regs`), or for one key and the queries q0 + 8*(r/4) + 4*g + r%4; entries outside the sequence read
-// element 0 (their scores are discarded anyway).
+// (`keys_in_regs`), or for one key and the queries q0 + 8*(r/4) + 4*g + r%4: the [L][L] mask plus the per-(batch, key)
+// bias.  Entries outside the sequence read element 0 (their scores are discarded anyway).
 template <bool KEYS_IN_REGS>
-__device__ __forceinline__ void flash_mask(const FlashArgs& a, int mine, int base, int g, float (&mk)[16]) {
+__device__ __forceinline__ void flash_mask(const FlashArgs& a, int batch, int mine, int base, int g, float (&mk)[16]) {
 #pragma unroll
   for (int r = 0; r < 16; ++r) mk[r] = 0.0f;
-  if (!a.mask) return;
-  if (KEYS_IN_REGS && a.L % 4 == 0 && reinterpret_cast<uintptr_t>(a.mask) % 16 == 0) {
+  if (!a.mask && !a.kbias) return;
+  if (a.mask) {
+    if (KEYS_IN_REGS && a.L % 4 == 0 && reinterpret_cast<uintptr_t>(a.mask) % 16 == 0) {
 #pragma unroll
-    for (int a4 = 0; a4 < 4; ++a4) {
-      const int key0 = base + 8 * a4 + 4 * g;
-      const float4 m4 =
-          *reinterpret_cast<const float4*>(a.mask + ((mine < a.L && key0 < a.L) ? (long)mine * a.L + key0 : 0));
-      mk[4 * a4 + 0] = m4.x, mk[4 * a4 + 1] = m4.y, mk[4 * a4 + 2] = m4.z, mk[4 * a4 + 3] = m4.w;
+      for (int a4 = 0; a4 < 4; ++a4) {
+        const int key0 = base + 8 * a4 + 4 * g;
+        const float4 m4 =
+            *reinterpret_cast<const float4*>(a.mask + ((mine < a.L && key0 < a.L) ? (long)mine * a.L + key0 : 0));
+        mk[4 * a4 + 0] = m4.x, mk[4 * a4 + 1] = m4.y, mk[4 * a4 + 2] = m4.z, mk[4 * a4 + 3] = m4.w;
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int other = base + 8 * (r >> 2) + 4 * g + (r & 3);
+        const long at = KEYS_IN_REGS ? (long)mine * a.L + other : (long)other * a.L + mine;
+        mk[r] = a.mask[(mine < a.L && other < a.L) ? at : 0];
+      }
     }
-  } else {
+  }
+  if (a.kbias) {
+    const float* row = a.kbias + (long)batch * a.L;
+    if (KEYS_IN_REGS) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int other = base + 8 * (r >> 2) + 4 * g + (r & 3);
-      const long at = KEYS_IN_REGS ? (long)mine * a.L + other : (long)other * a.L + mine;
-      mk[r] = a.mask[(mine < a.L && other < a.L) ? at : 0];
+      for (int r = 0; r < 16; ++r) {
+        const int key = base + 8 * (r >> 2) + 4 * g + (r & 3);
+        mk[r] += row[key < a.L ? key : 0];
+      }
+    } else {
+      const float kb = row[mine < a.L ? mine : 0];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mk[r] += kb;
     }
   }
 #pragma unroll
@@ -567,7 +598,7 @@ __global__ __launch_bounds__(NWV * 64) __attribute__((amdgpu_waves_per_eu(DB <= 
       rkv.fetch(src, a.L - k0 - kSeqMax, lane);
     }
     float mk[16];
-    flash_mask<true>(a, query, k0, g, mk);
+    flash_mask<true>(a, it.b, query, k0, g, mk);
     f32x16 s;
 #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = 0.0f;
@@ -735,7 +766,7 @@ __global__ __launch_bounds__(NWV * 64) __attribute__((amdgpu_waves_per_eu(DB <= 
       rkv.fetch(src, a.L - k0 - kSeqMax, lane);
     }
     float mk[16];
-    flash_mask<true>(a, query, k0, g, mk);
+    flash_mask<true>(a, it.b, query, k0, g, mk);
 #pragma unroll
     for (int r = 0; r < 16; ++r) mk[r] -= lse2;
     f32x16 s, dp;
@@ -853,7 +884,7 @@ __global__ __launch_bounds__(NWV * 64) __attribute__((amdgpu_waves_per_eu(DB <= 
       rqg.fetch(src, a.L - q0 - kSeqMax, lane);
     }
     float mk[16], sdelta[16];
-    flash_mask<false>(a, key, q0, g, mk);
+    flash_mask<false>(a, it.b, key, q0, g, mk);
 #pragma unroll
     for (int r = 0; r < 16; ++r) mk[r] = fmaf(lse_q[r], -kLog2e, mk[r]), sdelta[r] = delta_q[r] * a.scale;
     f32x16 s, dp;
@@ -919,8 +950,8 @@ extern "C" int rtp_attn_supported(int dtype, int64_t L, int64_t D) {
 
 extern "C" int rtp_attn_fwd(void* stream, int dtype, const void* q, const void* k, const void* v, int64_t s_l,
                             int64_t s_b, int64_t s_h, int64_t s_g, void* o, int64_t o_l, int64_t o_b, int64_t o_h,
-                            int64_t o_g, void* p, const float* mask, int causal, float scale, int64_t L, int64_t N,
-                            int64_t H, int64_t D, int64_t G) {
+                            int64_t o_g, void* p, const float* mask, const float* key_bias, int causal, float scale,
+                            int64_t L, int64_t N, int64_t H, int64_t D, int64_t G) {
   RTP_REQUIRE(q && k && v && o && p, "rtp_attn_fwd: null pointer");
   if (int rc = check_common("rtp_attn_fwd", dtype, L, N, H, D, G, s_l, s_b, s_h, s_g, o_l, o_b, o_h, o_g)) return rc;
   RTP_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o) % 16 == 0,
@@ -929,7 +960,7 @@ extern "C" int rtp_attn_fwd(void* stream, int dtype, const void* q, const void* 
   a.q = (const bf16_t*)q, a.k = (const bf16_t*)k, a.v = (const bf16_t*)v;
   a.s_l = s_l, a.s_b = s_b, a.s_h = s_h, a.s_g = s_g;
   a.o = (bf16_t*)o, a.o_l = o_l, a.o_b = o_b, a.o_h = o_h, a.o_g = o_g;
-  a.p = (bf16_t*)p, a.mask = mask, a.causal = causal, a.scale = scale;
+  a.p = (bf16_t*)p, a.mask = mask, a.kbias = key_bias, a.causal = causal, a.scale = scale;
   a.L = (int)L, a.N = (int)N, a.H = (int)H, a.nprob = G * N * H;
   hipStream_t st = (hipStream_t)stream;
   const double np = (double)a.nprob;
@@ -1006,12 +1037,12 @@ RTP_FLASH_LAUNCHER(FlashDq, attn_flash_dq_kernel)
 RTP_FLASH_LAUNCHER(FlashDkv, attn_flash_dkv_kernel)
 
 static int flash_args(const char* who, FlashArgs& a, int dtype, int64_t s_l, int64_t s_b, int64_t s_h, int64_t s_g,
-                      int64_t o_l, int64_t o_b, int64_t o_h, int64_t o_g, const float* mask, int causal, float scale,
-                      int64_t L, int64_t N, int64_t H, int64_t D, int64_t G) {
+                      int64_t o_l, int64_t o_b, int64_t o_h, int64_t o_g, const float* mask, const float* key_bias,
+                      int causal, float scale, int64_t L, int64_t N, int64_t H, int64_t D, int64_t G) {
   if (int rc = check_common(who, dtype, L, N, H, D, G, s_l, s_b, s_h, s_g, o_l, o_b, o_h, o_g, kFlashMaxLen)) return rc;
   a.s_l = s_l, a.s_b = s_b, a.s_h = s_h, a.s_g = s_g;
   a.o_l = o_l, a.o_b = o_b, a.o_h = o_h, a.o_g = o_g;
-  a.mask = mask, a.causal = causal, a.scale = scale;
+  a.mask = mask, a.kbias = key_bias, a.causal = causal, a.scale = scale;
   RTP_REQUIRE(G * N * H * ceil_div(L, kSeqMax) < (1ll << 31), "%s: too many (head, block) work items", who);
   // a lane's byte offsets inside one 32-row block are kept in 32 bits
   RTP_REQUIRE(s_l < (1ll << 25) && o_l < (1ll << 25) && s_l >= 0 && o_l >= 0, "%s: sequence stride out of range", who);
@@ -1021,14 +1052,14 @@ static int flash_args(const char* who, FlashArgs& a, int dtype, int64_t s_l, int
 
 extern "C" int rtp_attn_flash_fwd(void* stream, int dtype, const void* q, const void* k, const void* v, int64_t s_l,
                                   int64_t s_b, int64_t s_h, int64_t s_g, void* o, int64_t o_l, int64_t o_b,
-                                  int64_t o_h, int64_t o_g, float* lse, const float* mask, int causal, float scale,
-                                  int64_t L, int64_t N, int64_t H, int64_t D, int64_t G) {
+                                  int64_t o_h, int64_t o_g, float* lse, const float* mask, const float* key_bias,
+                                  int causal, float scale, int64_t L, int64_t N, int64_t H, int64_t D, int64_t G) {
   RTP_REQUIRE(q && k && v && o && lse, "rtp_attn_flash_fwd: null pointer");
   RTP_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o) % 16 == 0,
               "rtp_attn_flash_fwd: q, k, v, o must be 16-byte aligned");
   FlashArgs a{};
-  if (int rc = flash_args("rtp_attn_flash_fwd", a, dtype, s_l, s_b, s_h, s_g, o_l, o_b, o_h, o_g, mask, causal, scale,
-                          L, N, H, D, G))
+  if (int rc = flash_args("rtp_attn_flash_fwd", a, dtype, s_l, s_b, s_h, s_g, o_l, o_b, o_h, o_g, mask, key_bias, causal,
+                          scale, L, N, H, D, G))
     return rc;
   a.q = (const bf16_t*)q, a.k = (const bf16_t*)k, a.v = (const bf16_t*)v;
   a.o = (bf16_t*)o, a.lse = lse;
@@ -1041,15 +1072,15 @@ extern "C" int rtp_attn_flash_fwd(void* stream, int dtype, const void* q, const 
 extern "C" int rtp_attn_flash_bwd(void* stream, int dtype, const void* q, const void* k, const void* v, int64_t s_l,
                                   int64_t s_b, int64_t s_h, int64_t s_g, const void* o, const void* dout, int64_t o_l,
                                   int64_t o_b, int64_t o_h, int64_t o_g, const float* lse, float* delta, void* dq,
-                                  void* dk, void* dv, const float* mask, int causal, float scale, int64_t L,
-                                  int64_t N, int64_t H, int64_t D, int64_t G) {
+                                  void* dk, void* dv, const float* mask, const float* key_bias, int causal, float scale,
+                                  int64_t L, int64_t N, int64_t H, int64_t D, int64_t G) {
   RTP_REQUIRE(q && k && v && o && dout && lse && delta && dq && dk && dv, "rtp_attn_flash_bwd: null pointer");
   RTP_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o | (uintptr_t)dout | (uintptr_t)dq |
                (uintptr_t)dk | (uintptr_t)dv) % 16 == 0,
               "rtp_attn_flash_bwd: q, k, v, o, dout, dq, dk, dv must be 16-byte aligned");
   FlashArgs a{};
-  if (int rc = flash_args("rtp_attn_flash_bwd", a, dtype, s_l, s_b, s_h, s_g, o_l, o_b, o_h, o_g, mask, causal, scale,
-                          L, N, H, D, G))
+  if (int rc = flash_args("rtp_attn_flash_bwd", a, dtype, s_l, s_b, s_h, s_g, o_l, o_b, o_h, o_g, mask, key_bias, causal,
+                          scale, L, N, H, D, G))
     return rc;
   a.q = (const bf16_t*)q, a.k = (const bf16_t*)k, a.v = (const bf16_t*)v;
   a.dq = (bf16_t*)dq, a.dk = (bf16_t*)dk, a.dv = (bf16_t*)dv;

@@ -7,7 +7,8 @@ namespace rtp {
 constexpr int kRowsPerBlock = 4;
 
 template <typename T>
-__global__ __launch_bounds__(256) void softmax_fwd_kernel(const float* s, const float* mask, int causal, float scale,
+__global__ __launch_bounds__(256) void softmax_fwd_kernel(const float* s, const float* mask, const float* kbias,
+                                                          long n_batch, long heads, int causal, float scale,
                                                           long rows, long l, long skv, T* p) {
   const int lane = threadIdx.x & 63;
   const long row = (long)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
@@ -15,6 +16,8 @@ __global__ __launch_bounds__(256) void softmax_fwd_kernel(const float* s, const 
   const long i = row % l;
   const float* srow = s + row * skv;
   const float* mrow = mask ? mask + i * skv : nullptr;
+  // per-(batch, key) bias: problem index row / l = (group * n_batch + batch) * heads + head
+  const float* krow = kbias ? kbias + ((row / l / heads) % n_batch) * skv : nullptr;
   T* prow = p + row * skv;
   const long jmax = causal ? (i + (skv - l) + 1 < skv ? i + (skv - l) + 1 : skv) : skv;  // columns [0, jmax) are visible
 
@@ -22,6 +25,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_kernel(const float* s, const 
   for (long j = lane; j < jmax; j += kWave) {
     float v = srow[j] * scale;
     if (mrow) v += mrow[j];
+    if (krow) v += krow[j];
     mx = fmaxf(mx, v);
   }
   mx = wave_max(mx);
@@ -29,6 +33,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_kernel(const float* s, const 
   for (long j = lane; j < jmax; j += kWave) {
     float v = srow[j] * scale;
     if (mrow) v += mrow[j];
+    if (krow) v += krow[j];
     sum += expf(v - mx);
   }
   sum = wave_sum(sum);
@@ -38,6 +43,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_kernel(const float* s, const 
     if (j < jmax) {
       float v = srow[j] * scale;
       if (mrow) v += mrow[j];
+      if (krow) v += krow[j];
       o = expf(v - mx) * inv;
     }
     prow[j] = from_f32<T>(o);
@@ -66,9 +72,13 @@ __global__ __launch_bounds__(256) void softmax_bwd_kernel(const T* p, const floa
 
 using namespace rtp;
 
-extern "C" int rtp_softmax_fwd(void* stream, int dtype, const float* s, const float* mask, int causal, float scale,
-                               int64_t z, int64_t l, int64_t skv, void* p) {
+extern "C" int rtp_softmax_fwd(void* stream, int dtype, const float* s, const float* mask, const float* key_bias,
+                               int64_t n_batch, int64_t heads, int causal, float scale, int64_t z, int64_t l,
+                               int64_t skv, void* p) {
   RTP_REQUIRE(s && p, "rtp_softmax_fwd: null pointer");
+  RTP_REQUIRE(!key_bias || (n_batch >= 1 && heads >= 1 && z % (n_batch * heads) == 0),
+              "rtp_softmax_fwd: a key bias needs z = groups * n_batch * heads (z=%lld n_batch=%lld heads=%lld)",
+              (long long)z, (long long)n_batch, (long long)heads);
   RTP_REQUIRE(z >= 0 && l >= 0 && skv >= 1, "rtp_softmax_fwd: bad shape z=%lld l=%lld s=%lld", (long long)z,
               (long long)l, (long long)skv);
   const int64_t rows = z * l;
@@ -78,11 +88,11 @@ extern "C" int rtp_softmax_fwd(void* stream, int dtype, const float* s, const fl
   hipStream_t st = (hipStream_t)stream;
   ProfileScope prof(st, "softmax_fwd", 0.0, (double)rows * skv * (4.0 + (dtype == RTP_F32 ? 4 : 2)));
   if (dtype == RTP_F32)
-    hipLaunchKernelGGL(softmax_fwd_kernel<float>, grid, dim3(256), 0, st, s, mask, causal, scale, (long)rows, (long)l,
-                       (long)skv, (float*)p);
+    hipLaunchKernelGGL(softmax_fwd_kernel<float>, grid, dim3(256), 0, st, s, mask, key_bias, (long)n_batch, (long)heads,
+                       causal, scale, (long)rows, (long)l, (long)skv, (float*)p);
   else if (dtype == RTP_BF16)
-    hipLaunchKernelGGL(softmax_fwd_kernel<bf16_t>, grid, dim3(256), 0, st, s, mask, causal, scale, (long)rows,
-                       (long)l, (long)skv, (bf16_t*)p);
+    hipLaunchKernelGGL(softmax_fwd_kernel<bf16_t>, grid, dim3(256), 0, st, s, mask, key_bias, (long)n_batch, (long)heads,
+                       causal, scale, (long)rows, (long)l, (long)skv, (bf16_t*)p);
   else
     return fail(RTP_ERR_ARG, "rtp_softmax_fwd: unknown dtype %d", dtype);
   RTP_LAUNCH_CHECK();

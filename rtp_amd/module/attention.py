@@ -108,7 +108,7 @@ class _AttentionFn(torch.autograd.Function):
     kernel with p in memory."""
 
     @staticmethod
-    def forward(ctx, x, anchor, layer, mask, causal, want_weights, residual_grad=False):
+    def forward(ctx, x, anchor, layer, mask, causal, want_weights, residual_grad=False, key_bias=None):
         store = layer._store
         L, N, E = x.shape
         ws, h_s, d, e_s = layer.world_size, layer.num_heads_per_partition, layer.head_dim, layer.embed_dim_per_partition
@@ -140,7 +140,7 @@ class _AttentionFn(torch.autograd.Function):
                     # scores, softmax and p v in one launch, one wavefront per (group, batch, head)
                     ops.attn_fwd(qkv, q0, q0 + e_s, q0 + 2 * e_s, (ldq, ws * 3 * e_s, d, 3 * e_s), o, first * e_s,
                                  (N * E, E, d, e_s), p[first * Z:(first + cnt) * Z], mask, causal, scale, L, N, h_s,
-                                 d, cnt)
+                                 d, cnt, key_bias=key_bias)
                     c_out, c_in = acc.target(i)
                     S.row_fwd(o, flat, w_o_off, E, e_s, b_o_off, c_out, first * e_s, c_in=c_in)
                     i += 1
@@ -148,7 +148,7 @@ class _AttentionFn(torch.autograd.Function):
                 if flash:
                     ops.attn_flash_fwd(qkv, q0, q0 + e_s, q0 + 2 * e_s, (ldq, ws * 3 * e_s, d, 3 * e_s), o,
                                        first * e_s, (N * E, E, d, e_s), p[first * Z:(first + cnt) * Z], mask, causal,
-                                       scale, L, N, h_s, d, cnt)
+                                       scale, L, N, h_s, d, cnt, key_bias=key_bias)
                     c_out, c_in = acc.target(i)
                     S.row_fwd(o, flat, w_o_off, E, e_s, b_o_off, c_out, first * e_s, c_in=c_in)
                     i += 1
@@ -159,7 +159,7 @@ class _AttentionFn(torch.autograd.Function):
                      c_s=(h_s * L * L, L * L), c_sg=Z * L * L, m=L, n=L, k=d, batch=Z, zdiv=h_s, groups=cnt,
                      out_f32=True)
                 p_run = p[first * Z:(first + cnt) * Z]
-                ops.softmax_fwd(scores, p_run, mask=mask, causal=causal, scale=scale)
+                ops.softmax_fwd(scores, p_run, mask=mask, causal=causal, scale=scale, key_bias=key_bias, heads=h_s)
                 del scores
                 _bmm(dt, a=p, a_off=first * Z * L * L, lda=L, a_kc=True, a_s=(h_s * L * L, L * L), a_sg=Z * L * L,
                      b=qkv, b_off=q0 + 2 * e_s, ldb=ldq, b_kc=False, b_s=(ws * 3 * e_s, d), b_sg=3 * e_s, c=o,
@@ -175,7 +175,7 @@ class _AttentionFn(torch.autograd.Function):
         ctx.layer = layer
         ctx.dims = (L, N, E)
         ctx.residual_grad = residual_grad
-        ctx.flash = (mask, causal) if flash else None
+        ctx.flash = (mask, causal, key_bias) if flash else None
         ctx.save_for_backward(x2, qkv, p, o)
         ctx.mark_non_differentiable(*([weights] if weights is not None else []))
         return out.view(L, N, E), weights
@@ -221,11 +221,11 @@ class _AttentionFn(torch.autograd.Function):
                     i += 1
                     continue
                 if ctx.flash is not None:
-                    mask, causal = ctx.flash
+                    mask, causal, key_bias = ctx.flash
                     ops.attn_flash_bwd(qkv, q0, q0 + e_s, q0 + 2 * e_s, (ldq, ws * 3 * e_s, d, 3 * e_s), o, do,
                                        first * e_s, (N * E, E, d, e_s), p[first * Z:(first + cnt) * Z],
                                        delta[first * Z:(first + cnt) * Z], dqkv, mask, causal, scale, L, N, h_s, d,
-                                       cnt)
+                                       cnt, key_bias=key_bias)
                     if need_dx:
                         c_out, c_in = acc.target(i)
                         S.col_dgrad(dqkv, flat, 0, 3 * e_s, E, c_out, q0, c_in=c_in)
@@ -269,13 +269,14 @@ class _AttentionFn(torch.autograd.Function):
             store.grads_ready()
 
         run_wgrad(dev, param_grads, (dout2, o, dqkv, x2))
-        return (dx.view(L, N, E) if need_dx else None), None, None, None, None, None, None
+        return (dx.view(L, N, E) if need_dx else None), None, None, None, None, None, None, None
 
 
 class ParallelMultiheadAttention(RotatedLayer):
     """Signature follows rtp/module/attention.py:192-193; `MultiheadAttention_layer` imports the weights
     of an unsharded nn.MultiheadAttention.  Self-attention only (query, key and value must be the same
-    tensor); key_padding_mask, 3-D masks and attention dropout are not implemented and raise."""
+    tensor); 3-D masks and attention dropout are not implemented and raise.  key_padding_mask [batch, keys] (bool or
+    float, functional.py:615-623 and :760-768) reaches the kernels as a per-(batch, key) additive bias."""
 
     def __init__(self, embed_dim, num_heads, world_size, rank, dropout=0., bias=True, add_bias_kv=False,
                  add_zero_attn=False, kdim=None, vdim=None, batch_first=False, device=None, dtype=None,
@@ -308,8 +309,6 @@ class ParallelMultiheadAttention(RotatedLayer):
             if not (key.data_ptr() == query.data_ptr() == value.data_ptr() and key.shape == query.shape == value.shape
                     and key.stride() == query.stride() == value.stride()):
                 raise NotImplementedError("rotated attention implements self-attention only (query is key is value)")
-        if key_padding_mask is not None:
-            raise NotImplementedError("rotated attention: key_padding_mask is not implemented")
         if self.dropout > 0.0 and self.training:
             raise NotImplementedError("rotated attention: attention dropout is not implemented (use dropout=0)")
         if query.dim() != 3:
@@ -326,7 +325,19 @@ class ParallelMultiheadAttention(RotatedLayer):
             mask = mask.to(device=x.device, dtype=torch.float32).contiguous()
         elif is_causal:
             causal = True
-        out, weights = _AttentionFn.apply(x, self._anchor, self, mask, causal, bool(need_weights), bool(residual_grad))
+        key_bias = None
+        if key_padding_mask is not None:
+            # functional.py:615-623, :760-768: a bool mask hides the keys where it is True, a float mask is added to the
+            # scores; merged into the attention mask per batch there, handed to the kernels as a [batch, key] bias here
+            if key_padding_mask.dim() != 2 or tuple(key_padding_mask.shape) != (x.shape[1], L):
+                raise ValueError(f"key_padding_mask must be [batch, keys] = {(x.shape[1], L)}, got "
+                                 f"{tuple(key_padding_mask.shape)}")
+            key_bias = F._canonical_mask(mask=key_padding_mask, mask_name="key_padding_mask",
+                                         other_type=F._none_or_dtype(attn_mask), other_name="attn_mask",
+                                         target_type=torch.float32)
+            key_bias = key_bias.to(device=x.device, dtype=torch.float32).contiguous()
+        out, weights = _AttentionFn.apply(x, self._anchor, self, mask, causal, bool(need_weights), bool(residual_grad),
+                                          key_bias)
         if need_weights and weights is not None and average_attn_weights:
             weights = weights.float().mean(dim=1).to(out.dtype)
         if self.batch_first:

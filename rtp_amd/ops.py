@@ -246,9 +246,18 @@ def embedding_scatter_add(grad_out: torch.Tensor, n_ids: int, workspace: torch.T
         grad_table_sg))
 
 
+def _key_bias_ptr(who: str, key_bias: Optional[torch.Tensor], n_batch: int, keys: int):
+    if key_bias is None:
+        return None
+    if key_bias.dtype != torch.float32 or tuple(key_bias.shape) != (n_batch, keys) or not key_bias.is_contiguous():
+        raise ValueError(f"{who}: key_bias must be a contiguous fp32 [batch, keys] tensor")
+    return key_bias.data_ptr()
+
+
 def softmax_fwd(scores: torch.Tensor, p: torch.Tensor, *, mask: Optional[torch.Tensor], causal: bool,
-                scale: float) -> None:
-    """p[Z,L,S] = softmax(scale*scores + mask) row-wise; scores fp32, mask fp32 [L,S] or None."""
+                scale: float, key_bias: Optional[torch.Tensor] = None, heads: int = 1) -> None:
+    """p[Z,L,S] = softmax(scale*scores + mask + key_bias[b]) row-wise; scores fp32, mask fp32 [L,S] or None,
+    key_bias fp32 [N,S] or None with Z = groups * N * heads (problem z belongs to batch (z // heads) % N)."""
     _dev(scores)
     _dev(p)
     if scores.dtype != torch.float32 or scores.dim() != 3 or not scores.is_contiguous() or \
@@ -258,9 +267,11 @@ def softmax_fwd(scores: torch.Tensor, p: torch.Tensor, *, mask: Optional[torch.T
     if mask is not None:
         if mask.dtype != torch.float32 or tuple(mask.shape) != (l, s) or not mask.is_contiguous():
             raise ValueError("softmax_fwd: mask must be contiguous fp32 [L,S]")
+    n_batch = key_bias.shape[0] if key_bias is not None else 1
+    kb = _key_bias_ptr("softmax_fwd", key_bias, n_batch, s)
     _lib.require_device()
-    check(_lib.load().rtp_softmax_fwd(_stream(), dtype_code(p.dtype), scores.data_ptr(), _ptr(mask), int(causal),
-                                      scale, z, l, s, p.data_ptr()))
+    check(_lib.load().rtp_softmax_fwd(_stream(), dtype_code(p.dtype), scores.data_ptr(), _ptr(mask), kb, n_batch, heads,
+                                      int(causal), scale, z, l, s, p.data_ptr()))
 
 
 def softmax_bwd(p: torch.Tensor, dp: torch.Tensor, ds: torch.Tensor, scale: float) -> None:
@@ -283,7 +294,7 @@ def attn_supported(dtype: torch.dtype, L: int, d: int) -> bool:
 
 def attn_fwd(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, qkv_strides, o: torch.Tensor, o_off: int,
              o_strides, p: torch.Tensor, mask: Optional[torch.Tensor], causal: bool, scale: float, L: int, N: int,
-             H: int, d: int, G: int) -> None:
+             H: int, d: int, G: int, key_bias: Optional[torch.Tensor] = None) -> None:
     """Fused q k^T -> softmax -> p v for G*N*H (group, batch, head) problems addressed by element strides
     (s_l, s_b, s_h, s_g) into the packed projection `qkv` (offsets in elements) and `o`; p [G*N*H, L, L]."""
     _dev(qkv)
@@ -296,8 +307,8 @@ def attn_fwd(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, qkv_strides,
     base = qkv.data_ptr()
     check(_lib.load().rtp_attn_fwd(_stream(), dtype_code(qkv.dtype), base + q_off * esz, base + k_off * esz,
                                    base + v_off * esz, *qkv_strides, o.data_ptr() + o_off * esz, *o_strides,
-                                   p.data_ptr(), mask.data_ptr() if mask is not None else None, int(causal), scale,
-                                   L, N, H, d, G))
+                                   p.data_ptr(), mask.data_ptr() if mask is not None else None,
+                                   _key_bias_ptr("attn_fwd", key_bias, N, L), int(causal), scale, L, N, H, d, G))
 
 
 def attn_bwd(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, qkv_strides, dout: torch.Tensor, o_off: int,
@@ -338,7 +349,7 @@ def _flash_mask(mask: Optional[torch.Tensor], L: int):
 
 def attn_flash_fwd(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, qkv_strides, o: torch.Tensor, o_off: int,
                    o_strides, lse: torch.Tensor, mask: Optional[torch.Tensor], causal: bool, scale: float, L: int,
-                   N: int, H: int, d: int, G: int) -> None:
+                   N: int, H: int, d: int, G: int, key_bias: Optional[torch.Tensor] = None) -> None:
     """attn_fwd for any L: o = softmax(scale q k^T + mask) v without storing the probabilities; lse [G*N*H, L]
     fp32 receives the log-sum-exp of each query's scores."""
     _dev(qkv)
@@ -351,13 +362,14 @@ def attn_flash_fwd(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, qkv_st
     base = qkv.data_ptr()
     check(_lib.load().rtp_attn_flash_fwd(_stream(), dtype_code(qkv.dtype), base + q_off * esz, base + k_off * esz,
                                          base + v_off * esz, *qkv_strides, o.data_ptr() + o_off * esz, *o_strides,
-                                         lse.data_ptr(), mask_ptr, int(causal), scale, L, N, H, d, G))
+                                         lse.data_ptr(), mask_ptr, _key_bias_ptr("attn_flash_fwd", key_bias, N, L),
+                                         int(causal), scale, L, N, H, d, G))
 
 
 def attn_flash_bwd(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, qkv_strides, o: torch.Tensor,
                    dout: torch.Tensor, o_off: int, o_strides, lse: torch.Tensor, delta: torch.Tensor,
                    dqkv: torch.Tensor, mask: Optional[torch.Tensor], causal: bool, scale: float, L: int, N: int,
-                   H: int, d: int, G: int) -> None:
+                   H: int, d: int, G: int, key_bias: Optional[torch.Tensor] = None) -> None:
     """Backward of attn_flash_fwd: writes dq, dk, dv into `dqkv` (layout and offsets of `qkv`); `o` and `dout`
     share layout and offset; `delta` [G*N*H, L] fp32 is scratch."""
     _dev(qkv)
@@ -375,7 +387,8 @@ def attn_flash_bwd(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, qkv_st
                                          base + v_off * esz, *qkv_strides, o.data_ptr() + o_off * esz,
                                          dout.data_ptr() + o_off * esz, *o_strides, lse.data_ptr(), delta.data_ptr(),
                                          dbase + q_off * esz, dbase + k_off * esz, dbase + v_off * esz, mask_ptr,
-                                         int(causal), scale, L, N, H, d, G))
+                                         _key_bias_ptr("attn_flash_bwd", key_bias, N, L), int(causal), scale, L, N, H,
+                                         d, G))
 
 
 def layernorm_supported(dtype: torch.dtype, cols: int) -> bool:

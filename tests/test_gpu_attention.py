@@ -94,8 +94,8 @@ def test_attention_unsupported_raise():
     x = torch.randn(4, 2, 8, device=DEV)
     with pytest.raises(NotImplementedError):
         layer(x, x.clone(), x)
-    with pytest.raises(NotImplementedError):
-        layer(x, x, x, key_padding_mask=torch.zeros(2, 4, dtype=torch.bool, device=DEV))
+    with pytest.raises(ValueError):
+        layer(x, x, x, key_padding_mask=torch.zeros(3, 4, dtype=torch.bool, device=DEV))   # [batch, keys] = [2, 4]
     with pytest.raises(NotImplementedError):
         ParallelMultiheadAttention(8, 2, 2, 0, kdim=4, device=DEV)
 
@@ -262,3 +262,52 @@ def test_attn_flash_rejects_unsupported():
     with pytest.raises(ValueError):
         ops.attn_flash_fwd(qkv, 0, 64, 128, (192, 192, 64, 192), o, 0, (64, 64, 64, 64), lse[:, :39], None, False,
                            0.125, 40, 1, 1, 64, 1)
+
+
+@pytest.mark.parametrize("E,H,L,N,ws,dtype,masked,need_weights", [
+    (128, 4, 20, 3, 2, torch.bfloat16, False, False),   # short-sequence core
+    (128, 4, 20, 3, 2, torch.bfloat16, True, True),     # ... with the causal float mask, weights returned
+    (256, 4, 100, 3, 2, torch.bfloat16, False, False),  # running-softmax core
+    (256, 4, 100, 3, 4, torch.bfloat16, True, False),
+    (64, 4, 40, 2, 2, torch.float32, True, False),      # products and softmax kernel
+    (128, 4, 48, 2, 2, torch.bfloat16, False, True),    # weights returned beyond 32 positions
+])
+def test_attention_key_padding_mask(E, H, L, N, ws, dtype, masked, need_weights):
+    """key_padding_mask [batch, keys] (bool: True hides the key) against nn.MultiheadAttention; each batch row pads a
+    different tail, key 0 stays visible so no query loses all its keys."""
+    from rtp_amd.module.attention import ParallelMultiheadAttention
+    gen = torch.Generator().manual_seed(8)
+    mha = _master(E, H, dtype, gen)
+    x = torch.randn(L, N, E, generator=gen).to(dtype)
+    g = torch.randn(L, N, E, generator=gen).to(dtype)
+    kpm = torch.zeros(N, L, dtype=torch.bool)
+    for b in range(N):
+        kpm[b, L - 1 - 3 * b:] = True
+    mask = _causal(L) if masked else None
+    layer = ParallelMultiheadAttention(E, H, ws, 0, MultiheadAttention_layer=mha, device=DEV, dtype=dtype)
+    xd = x.to(DEV).requires_grad_()
+    out, w = layer(xd, xd, xd, attn_mask=None if mask is None else mask.to(DEV), key_padding_mask=kpm.to(DEV),
+                   need_weights=need_weights)
+    out.backward(g.to(DEV))
+    ref_m = nn.MultiheadAttention(E, H, bias=True)
+    ref_m.load_state_dict({k: v.float() for k, v in mha.state_dict().items()})
+    xo = x.float().requires_grad_()
+    ref, w_ref = ref_m(xo, xo, xo, attn_mask=mask, key_padding_mask=kpm, need_weights=True, average_attn_weights=False)
+    ref.backward(g.float())
+    assert_close(out, ref, dtype, "output")
+    assert_close(xd.grad, xo.grad, dtype, "input grad")
+    assert_close(O.attention_grad_reinterleave([l.in_proj_weight.grad for l in layer.layers], ws),
+                 ref_m.in_proj_weight.grad, dtype, "in_proj_weight grad")
+    assert_close(torch.cat([l.out_proj.weight.grad for l in layer.layers], dim=1), ref_m.out_proj.weight.grad, dtype,
+                 "out_proj.weight grad")
+    if need_weights:
+        h_s = H // ws
+        assert_close(w, w_ref[:, (ws - 1) * h_s:].mean(1), dtype, "attention weights of the last shard")
+        hidden = kpm.to(DEV)[:, None, :].expand(N, L, L)
+        assert not w[hidden].any()                        # padded keys get exactly zero weight
+    # a float key_padding_mask is added to the scores: the same -inf pattern gives the same result
+    xf = x.to(DEV)
+    with torch.no_grad():
+        out_f, _ = layer(xf, xf, xf, attn_mask=None if mask is None else mask.to(DEV), need_weights=need_weights,
+                         key_padding_mask=torch.zeros(N, L).masked_fill(kpm, float("-inf")).to(DEV))
+    assert torch.equal(out_f, out.detach())
