@@ -119,14 +119,19 @@ struct Problem {
   int b;
   bool live;
 };
+// The wave index is made scalar and the problem index is split by 32-bit divisions (the host keeps nprob below 2^31):
+// 64-bit divisions are software loops of ~140 instructions each, in front of the kernel's first load.
 __device__ __forceinline__ Problem locate(const AttnArgs& a, int waves_per_block) {
   Problem pr;
-  pr.z = (long)blockIdx.x * waves_per_block + (threadIdx.x >> 6);
-  pr.live = pr.z < a.nprob;
-  if (!pr.live) pr.z = a.nprob - 1;  // idle waves redo the last problem and store nothing
-  const long h = pr.z % a.H, b = (pr.z / a.H) % a.N, g = pr.z / ((long)a.H * a.N);
-  pr.qkv_off = b * a.s_b + h * a.s_h + g * a.s_g;
-  pr.o_off = b * a.o_b + h * a.o_h + g * a.o_g;
+  const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  unsigned z = blockIdx.x * (unsigned)waves_per_block + wave;
+  pr.live = z < (unsigned)a.nprob;
+  if (!pr.live) z = (unsigned)a.nprob - 1;  // idle waves redo the last problem and store nothing
+  pr.z = z;
+  const unsigned zh = z / (unsigned)a.H, h = z - zh * (unsigned)a.H;
+  const unsigned g = zh / (unsigned)a.N, b = zh - g * (unsigned)a.N;
+  pr.qkv_off = (long)b * a.s_b + (long)h * a.s_h + (long)g * a.s_g;
+  pr.o_off = (long)b * a.o_b + (long)h * a.o_h + (long)g * a.o_g;
   pr.b = (int)b;
   return pr;
 }
@@ -197,14 +202,17 @@ __global__ __launch_bounds__(NWV * 64) void attn_fwd_small_kernel(AttnArgs a) {
     s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rowmajor(Ks, P, li, g, ks), frag_rowmajor(Qs, P, li, g, ks), s, 0,
                                                 0, 0);
 
-  // softmax over the keys of query li
+  // softmax over the keys of query li, in the log2 domain (scale * log2 e in one FMA, the hardware 2^x)
+  constexpr float kLog2eSmall = 1.44269504088896340736f;
+  const float scale2 = a.scale * kLog2eSmall;
   float val[16];
   float mx = -INFINITY;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int key = 8 * (r >> 2) + 4 * g + (r & 3);
     const bool visible = key < a.L && (!a.causal || key <= li);
-    const float x = s[r] * a.scale + ((qlive && key < a.L) ? mk[r] + kb[r] : 0.0f);  // outside: unrelated entries
+    // outside the sequence: unrelated mask entries
+    const float x = fmaf(s[r], scale2, ((qlive && key < a.L) ? (mk[r] + kb[r]) * kLog2eSmall : 0.0f));
     val[r] = visible ? x : -INFINITY;
     mx = fmaxf(mx, val[r]);
   }
@@ -212,9 +220,7 @@ __global__ __launch_bounds__(NWV * 64) void attn_fwd_small_kernel(AttnArgs a) {
   float sum = 0.0f;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
-    const int key = 8 * (r >> 2) + 4 * g + (r & 3);
-    const bool visible = key < a.L && (!a.causal || key <= li);
-    val[r] = visible ? expf(val[r] - mx) : 0.0f;
+    val[r] = __builtin_amdgcn_exp2f(val[r] - mx);  // hidden keys: 2^(-inf) = 0; every key hidden: NaN, as torch gives
     sum += val[r];
   }
   sum += __shfl_xor(sum, 32, kWave);
@@ -936,7 +942,7 @@ static int check_common(const char* who, int dtype, int64_t L, int64_t N, int64_
   RTP_REQUIRE(aligned8(s_l) && aligned8(s_b) && aligned8(s_h) && aligned8(s_g) && aligned8(o_l) && aligned8(o_b) &&
                   aligned8(o_h) && aligned8(o_g),
               "%s: strides must be multiples of 8 elements", who);
-  RTP_REQUIRE(ceil_div(G * N * H, 2) < (1ll << 31), "%s: too many problems", who);
+  RTP_REQUIRE(G * N * H < (1ll << 31), "%s: too many problems", who);
   return RTP_OK;
 }
 
