@@ -443,6 +443,21 @@ typedef struct {
 int rtp_sgd_step_multi(void* stream, int dtype, const rtp_sgd_chunk* chunks, int64_t n_chunks, float lr,
                        float clip, double total_params);
 
+/* Adam for many buffers in one launch, like rtp_sgd_step_multi: `chunks` is a table in DEVICE memory, one entry per
+ * workgroup (16-byte aligned pointers, a parameter count that is a multiple of 4); the other arguments as for
+ * rtp_adam_step.  total_params only feeds the profiler. */
+typedef struct {
+  float* master;
+  const void* grad;
+  void* shadow; /* NULL: the master is the weight */
+  float* exp_avg;
+  float* exp_avg_sq;
+  int64_t n;
+} rtp_adam_chunk;
+int rtp_adam_step_multi(void* stream, int dtype, const rtp_adam_chunk* chunks, int64_t n_chunks, double lr,
+                        double beta1, double beta2, double eps, double weight_decay, int64_t step,
+                        const int64_t* step_dev, double clip, double total_params);
+
 /* dst(dtype_dst)[i] = src(dtype_src)[i]  (fp32 <-> bf16 conversion, round to nearest even). */
 int rtp_cast(void* stream, int dtype_src, const void* src, int dtype_dst, void* dst, int64_t n);
 

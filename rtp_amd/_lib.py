@@ -119,6 +119,8 @@ PROTOTYPES = {
     "rtp_sgd_step": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _f, _f]),
     "rtp_adam_step": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i64, C.c_double, C.c_double, C.c_double, C.c_double,
                            C.c_double, _i64, _vp, C.c_double]),
+    "rtp_adam_step_multi": (_i, [_vp, _i, _vp, _i64, C.c_double, C.c_double, C.c_double, C.c_double, C.c_double, _i64, _vp,
+                                 C.c_double, C.c_double]),
     "rtp_sgd_step_multi": (_i, [_vp, _i, _vp, _i64, _f, _f, C.c_double]),
     "rtp_cast": (_i, [_vp, _i, _vp, _i, _vp, _i64]),
     "rtp_profile_enable": (_i, [_i]),

@@ -216,6 +216,49 @@ __global__ __launch_bounds__(256) void adam_vec4_kernel(float4* master, const T*
   }
 }
 
+// Adam for many buffers in one launch: workgroup b updates chunk b of a device-resident table.
+struct AdamChunk {
+  float* master;
+  const void* grad;
+  void* shadow;  // may be null
+  float *exp_avg, *exp_avg_sq;
+  long n;  // parameters in the chunk, a multiple of 4; the pointers are 16-byte aligned
+};
+template <typename T>
+__global__ __launch_bounds__(256) void adam_multi_kernel(const AdamChunk* chunks, AdamScalars c) {
+  using P = typename Sgd4<T>::Pack;
+  adam_bias_corrections(c);
+  const AdamChunk ch = chunks[blockIdx.x];
+  float4* master = reinterpret_cast<float4*>(ch.master);
+  float4* m4 = reinterpret_cast<float4*>(ch.exp_avg);
+  float4* v4 = reinterpret_cast<float4*>(ch.exp_avg_sq);
+  const T* grad = reinterpret_cast<const T*>(ch.grad);
+  T* shadow = reinterpret_cast<T*>(ch.shadow);
+  const long n4 = ch.n >> 2;
+  auto one = [&](long i, const P& g, float4 w, float4 m, float4 v) {
+    float *wf = reinterpret_cast<float*>(&w), *mf = reinterpret_cast<float*>(&m), *vf = reinterpret_cast<float*>(&v);
+    P sh;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      adam_update(wf[e], mf[e], vf[e], to_f32(g.e[e]), c);
+      sh.e[e] = from_f32<T>(wf[e]);
+    }
+    nt_store(w, master + i), nt_store(m, m4 + i), nt_store(v, v4 + i);
+    if (shadow) Sgd4<T>::store(shadow, i, sh);
+  };
+  long i = threadIdx.x;
+  for (; i + 256 < n4; i += 512) {
+    const long k = i + 256;
+    const P g0 = Sgd4<T>::load(grad, i), g1 = Sgd4<T>::load(grad, k);
+    const float4 w0 = nt_load(master + i), w1 = nt_load(master + k);
+    const float4 a0 = nt_load(m4 + i), a1 = nt_load(m4 + k);
+    const float4 b0 = nt_load(v4 + i), b1 = nt_load(v4 + k);
+    one(i, g0, w0, a0, b0);
+    one(k, g1, w1, a1, b1);
+  }
+  for (; i < n4; i += 256) one(i, Sgd4<T>::load(grad, i), nt_load(master + i), nt_load(m4 + i), nt_load(v4 + i));
+}
+
 template <typename S, typename D>
 __global__ __launch_bounds__(256) void cast_kernel(const S* src, D* dst, long n) {
   const long stride = (long)gridDim.x * blockDim.x;
@@ -314,6 +357,36 @@ extern "C" int rtp_adam_step(void* stream, int dtype, float* master, const void*
     launch_adam<float>(s, vec4, master, grad, shadow, exp_avg, exp_avg_sq, n, c);
   else
     launch_adam<bf16_t>(s, vec4, master, grad, shadow, exp_avg, exp_avg_sq, n, c);
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
+}
+
+extern "C" int rtp_adam_step_multi(void* stream, int dtype, const rtp_adam_chunk* chunks, int64_t n_chunks, double lr,
+                                   double beta1, double beta2, double eps, double weight_decay, int64_t step,
+                                   const int64_t* step_dev, double clip, double total_params) {
+  static_assert(sizeof(rtp_adam_chunk) == sizeof(AdamChunk), "rtp_adam_chunk layout");
+  RTP_REQUIRE(chunks, "rtp_adam_step_multi: null chunk table");
+  RTP_REQUIRE(n_chunks >= 0 && n_chunks < (1ll << 31), "rtp_adam_step_multi: chunk count %lld out of range",
+              (long long)n_chunks);
+  RTP_REQUIRE(dtype == RTP_F32 || dtype == RTP_BF16, "rtp_adam_step_multi: unknown dtype %d", dtype);
+  RTP_REQUIRE(step_dev || step >= 1, "rtp_adam_step_multi: step counts from 1 (got %lld)", (long long)step);
+  RTP_REQUIRE(beta1 >= 0.0 && beta1 < 1.0 && beta2 >= 0.0 && beta2 < 1.0 && eps >= 0.0 && lr >= 0.0,
+              "rtp_adam_step_multi: need 0 <= beta < 1, eps >= 0, lr >= 0");
+  if (n_chunks == 0) return RTP_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const double t = step_dev ? 1.0 : (double)step;
+  const double bc1 = 1.0 - std::pow(beta1, t), bc2 = 1.0 - std::pow(beta2, t);
+  AdamScalars c{};
+  c.step_dev = reinterpret_cast<const long*>(step_dev), c.lr = lr, c.beta1 = beta1, c.beta2d = beta2;
+  c.w1 = (float)(1.0 - beta1), c.beta2 = (float)beta2, c.w2 = (float)(1.0 - beta2);
+  c.bc2_sqrt = (float)std::sqrt(bc2), c.eps = (float)eps, c.neg_step_size = (float)(-(lr / bc1));
+  c.weight_decay = (float)weight_decay, c.clip = (float)clip;
+  ProfileScope prof(s, "adam_step", 12.0 * total_params, total_params * (dtype == RTP_F32 ? 32.0 : 28.0));
+  const AdamChunk* table = reinterpret_cast<const AdamChunk*>(chunks);
+  if (dtype == RTP_F32)
+    hipLaunchKernelGGL(adam_multi_kernel<float>, dim3((unsigned)n_chunks), dim3(256), 0, s, table, c);
+  else
+    hipLaunchKernelGGL(adam_multi_kernel<bf16_t>, dim3((unsigned)n_chunks), dim3(256), 0, s, table, c);
   RTP_LAUNCH_CHECK();
   return RTP_OK;
 }

@@ -676,6 +676,42 @@ def sgd_chunk_table(items, device) -> Optional[torch.Tensor]:
     return torch.tensor(rows, dtype=torch.int64).to(device)
 
 
+def adam_chunk_table(items, device) -> Optional[torch.Tensor]:
+    """Device table for adam_step_multi from (master, grad, shadow-or-None, exp_avg, exp_avg_sq) tuples of flat
+    tensors, or None when some buffer does not allow 16-byte accesses (then update the buffers one by one)."""
+    rows = []
+    for master, grad, shadow, m, v in items:
+        n = master.numel()
+        ptrs = [master.data_ptr(), grad.data_ptr(), m.data_ptr(), v.data_ptr()] + \
+               ([shadow.data_ptr()] if shadow is not None else [])
+        if n % 4 or any(p % 16 for p in ptrs) or any(t.numel() != n for t in (grad, m, v)) or \
+                (shadow is not None and shadow.numel() != n):
+            return None
+        gs = grad.element_size()
+        for off in range(0, n, SGD_CHUNK):
+            cnt = min(SGD_CHUNK, n - off)
+            rows.append((master.data_ptr() + off * 4, grad.data_ptr() + off * gs,
+                         shadow.data_ptr() + off * gs if shadow is not None else 0, m.data_ptr() + off * 4,
+                         v.data_ptr() + off * 4, cnt))
+    if not rows:
+        return None
+    return torch.tensor(rows, dtype=torch.int64).to(device)
+
+
+def adam_step_multi(table: torch.Tensor, dtype: torch.dtype, step, lr: float, betas, eps: float, weight_decay: float,
+                    clip: float, total_params: int) -> None:
+    """adam_step for every chunk of `table` in one launch; `step` as for adam_step."""
+    _dev(table)
+    step_dev = None
+    if isinstance(step, torch.Tensor):
+        if step.dtype != torch.int64 or step.numel() != 1 or step.device != table.device:
+            raise ValueError("adam_step_multi: a device step count must be one int64 element on the table's device")
+        step_dev, step = step.data_ptr(), 0
+    _lib.require_device()
+    check(_lib.load().rtp_adam_step_multi(_stream(), dtype_code(dtype), table.data_ptr(), table.shape[0], lr, betas[0],
+                                          betas[1], eps, weight_decay, int(step), step_dev, clip, float(total_params)))
+
+
 def sgd_step_multi(table: torch.Tensor, dtype: torch.dtype, lr: float, clip: float, total_params: int) -> None:
     _dev(table)
     _lib.require_device()

@@ -203,8 +203,9 @@ class RotatedSGD:
 
 class RotatedAdam(RotatedSGD):
     """The reference harness's optimiser (benchmarks/rtp_benchmark.py:41-42: torch.optim.Adam(lr 1e-3) after
-    clip_grad_value_(0.05)) over the same flat buffers as RotatedSGD: one launch per rotated layer and one for
-    the parameters outside rotated layers, fp32 moments beside the fp32 master.  The step count lives in device
+    clip_grad_value_(0.05)) over the same flat buffers as RotatedSGD, fp32 moments beside the fp32 master: one launch
+    over a device chunk table for all of them (or one per buffer where a buffer is not 16-byte aligned or the buffers
+    differ in dtype).  The step count lives in device
     memory and the kernels form the bias corrections 1 - beta^step themselves, so step() may be recorded into a HIP
     graph and replayed (`steps` then only counts the eager calls)."""
 
@@ -215,17 +216,45 @@ class RotatedAdam(RotatedSGD):
         self.steps = 0
         self._step_dev = None
         self._moments = {}
+        self._adam_table = self._adam_key = None
+        self._adam_params, self._adam_dtype = 0, None
 
     def state_bytes(self) -> int:
         return sum(m.numel() * 4 + v.numel() * 4 for m, v in self._moments.values())
 
-    def _adam(self, key, weights: torch.Tensor, grads: torch.Tensor, master: Optional[torch.Tensor]) -> None:
-        target = weights if master is None else master.view(-1)
+    def _state(self, key, target: torch.Tensor):
         if key not in self._moments:
             self._moments[key] = (torch.zeros_like(target), torch.zeros_like(target))
-        m, v = self._moments[key]
-        ops.adam_step(target, grads, None if master is None else weights, m, v, self._step_dev, self.lr, self.betas,
-                      self.eps, self.weight_decay, self.clip_value)
+        return self._moments[key]
+
+    def _buffers(self):
+        """(key, update target, gradients, weights to refresh or None) of every buffer that has gradients."""
+        out = []
+        for i, (st, master) in enumerate(zip(self.stores, self.masters)):
+            if st.grads is None:
+                continue
+            home, grads = st.home.view(-1), st.grads.view(-1)
+            out.append((i, home, grads, None) if master is None else (i, master.view(-1), grads, home))
+        if self.flat is not None:
+            out.append(("flat", self.flat, self.flat_grad, None) if self.flat_master is None
+                       else ("flat", self.flat_master, self.flat_grad, self.flat))
+        return out
+
+    def _multi_adam_table(self, buffers):
+        """Chunk table over every buffer, rebuilt only when a buffer moved; None when one launch cannot cover them."""
+        if len({g.dtype for _, _, g, _ in buffers}) != 1:
+            return None
+        items = []
+        for key, target, grads, shadow in buffers:
+            m, v = self._state(key, target)
+            items.append((target, grads, shadow, m, v))
+        ptr_key = tuple(t.data_ptr() for it in items for t in it if t is not None)
+        if ptr_key != self._adam_key:
+            self._adam_key = ptr_key
+            self._adam_table = ops.adam_chunk_table(items, items[0][0].device)
+            self._adam_params = sum(it[0].numel() for it in items)
+            self._adam_dtype = items[0][1].dtype
+        return self._adam_table
 
     @torch.no_grad()
     def step(self) -> None:
@@ -238,12 +267,17 @@ class RotatedAdam(RotatedSGD):
             self._step_dev = torch.zeros(1, dtype=torch.int64, device=buffers[0].device)
         self.steps += 1
         self._step_dev += 1
-        for i, (st, master) in enumerate(zip(self.stores, self.masters)):
-            if st.grads is None:
-                continue
-            self._adam(i, st.home.view(-1), st.grads.view(-1), master)
         if self.flat is not None:
             self._fold_other_grads()
-            self._adam("flat", self.flat, self.flat_grad, self.flat_master)
+        buffers = self._buffers()
+        table = self._multi_adam_table(buffers) if buffers else None
+        if table is not None:
+            ops.adam_step_multi(table, self._adam_dtype, self._step_dev, self.lr, self.betas, self.eps,
+                                self.weight_decay, self.clip_value, self._adam_params)
+        else:
+            for key, target, grads, shadow in buffers:
+                m, v = self._state(key, target)
+                ops.adam_step(target, grads, shadow, m, v, self._step_dev, self.lr, self.betas, self.eps,
+                              self.weight_decay, self.clip_value)
         if self.stores:
             ring.fence(self.stores[0].home.device)  # staging copies of the next step must see the new weights
