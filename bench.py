@@ -23,7 +23,7 @@ if ROOT not in sys.path:
 CFG = dict(vocab=10240, ninp=2048, nhid=2048, nhead=32, layers=10, seq=32, batch=32, shards=8)
 PEAK = {"bf16_mfma_tflops": 2500.0, "fp32_mfma_tflops": 157.3, "hbm_gbs": 8000.0}
 # Memory-side traffic per launch of the GEMM variants of this workload, KiB, averaged over the launches of a step:
-# FETCH_SIZE * 1.9937 + WRITE_SIZE * 1.0000 from two rocprofv3 --pmc runs of this script; the factors are what the same
+# FETCH_SIZE * 1.9927 + WRITE_SIZE * 1.0000 from two rocprofv3 --pmc runs of this script; the factors are what the same
 # counters read for the library's plain copy kernel on a copy of known size (profiles/lm_step_pmc_fetch_write.txt).
 MEASURED_TRAFFIC_KIB = {
     "gemm_bf16_128x128_rc_rc": 45027.6, "gemm_bf16_128x64_kc_rc": 59061.3, "gemm_bf16_128x64_kc_kc": 36972.4,
