@@ -67,10 +67,11 @@ struct GemmArgs {
   char* a_rowsum;  // bias gradient output (sum over k of A's rows), or null
   long rowsum_sg;
   // wave-specialised kernel: tile mapping without run-time divisions
-  // A brick is mbk x nbk tiles; its tiles are handed out panel by panel, a panel being all mbk tile rows of `panel`
-  // consecutive tile columns with the row running fastest -- see the kernel.
-  FastDiv d_batch, d_zdiv, d_tiles_n, d_brick, d_panel, d_mbk;  // divisors mbk*nbk, mbk*panel, mbk
-  int nbk, panel;
+  // A brick is mbk x nbk tiles; its tiles are handed out panel by panel, a panel being prow x pcol tiles with the
+  // row running fastest, and the panels of a strip of pcol tile columns follow each other down the rows before
+  // the next strip starts -- see the kernel.
+  FastDiv d_batch, d_zdiv, d_tiles_n, d_brick, d_panel, d_prow, d_pm;  // divisors mbk*nbk, prow*pcol, prow, mbk/prow
+  int mbk, nbk, prow, pcol;
   int xn_shift, xm_shift, zbk;  // log2 of xn and xm, batch*groups entries per brick
 };
 
@@ -725,13 +726,16 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   const unsigned id = blockIdx.x + blockIdx.y * gridDim.x;
   const unsigned xcd = id & 7, slot = id >> 3;
   // The ~32 workgroups an XCD runs at a time should cover a compact block of the brick, not a row of it: they
-  // share the XCD's L2, and a 4 x 8 block of tiles reads 12 tile-operands where a 1 x 32 row reads 33.
+  // share the XCD's L2, and a 4 x 8 block of tiles reads 12 tile-operands where a 1 x 32 row reads 33.  Over the
+  // rounds of a long launch the panels walk down a strip of pcol tile columns, whose B operand stays in the L2
+  // while the A rows stream past once per strip.
   const unsigned zl = fast_div(slot, p.d_brick);  // entry of the batch*groups axis inside the brick
   const unsigned t = slot - zl * p.d_brick.d;      // tile inside the mbk x nbk brick
-  const unsigned pn = fast_div(t, p.d_panel), r = t - pn * p.d_panel.d;
-  const unsigned cn = fast_div(r, p.d_mbk), cm = r - cn * p.d_mbk.d;
-  const int tile_n_x = (int)((xcd & ((1u << p.xn_shift) - 1)) * p.nbk + pn * p.panel + cn);
-  const int tile_m_x = (int)(((xcd >> p.xn_shift) & ((1u << p.xm_shift) - 1)) * p.d_mbk.d + cm);
+  const unsigned q = fast_div(t, p.d_panel), r = t - q * p.d_panel.d;  // panel, tile inside the panel
+  const unsigned cn = fast_div(r, p.d_prow), cm = r - cn * p.d_prow.d;
+  const unsigned qn = fast_div(q, p.d_pm), qm = q - qn * p.d_pm.d;     // strip, panel inside the strip
+  const int tile_n_x = (int)((xcd & ((1u << p.xn_shift) - 1)) * p.nbk + qn * p.pcol + cn);
+  const int tile_m_x = (int)(((xcd >> p.xn_shift) & ((1u << p.xm_shift) - 1)) * p.mbk + qm * p.prow + cm);
   const int z_x = (int)((xcd >> (p.xn_shift + p.xm_shift)) * p.zbk + zl);
   const int tile_m_p = (int)fast_div(blockIdx.x, p.d_tiles_n);
   const int tile_n_p = (int)(blockIdx.x - tile_m_p * p.d_tiles_n.d);
@@ -1209,14 +1213,23 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   a.d_tiles_n = make_fastdiv((unsigned)a.tiles_n);
   {
     const int nbk = a.xg ? a.tiles_n / a.xn : 1, mbk = a.xg ? a.tiles_m / a.xm : 1;
-    // panel width: the largest power of two that divides nbk and keeps a panel (mbk rows) within ~32 tiles
-    int panel = 1;
-    while (panel * 2 * mbk <= 32 && nbk % (panel * 2) == 0) panel *= 2;
-    a.nbk = nbk;
-    a.panel = panel;
+    // Panel = prow x pcol tiles, about one round of an XCD's 32 CUs.  pcol: the widest divisor of nbk (at most 32)
+    // whose strip of B tiles (pcol * BN rows x all of K) stays within ~3 MB of the XCD's 4 MB L2 -- the A rows stream
+    // past the strip once, so the L2 fills are about A * nbk / pcol + B per brick.  prow: the tallest divisor of mbk
+    // that keeps the panel within 32 tiles.
+    const double b_tile_bytes = (double)ts.bn * (double)d->k * (double)d->ksegs * sizeof(T);
+    int pcol = 1;
+    for (int c = 2; c <= 32 && c <= nbk; ++c)
+      if (nbk % c == 0 && c * b_tile_bytes <= 3.0 * 1024 * 1024) pcol = c;
+    int prow = 1;
+    for (int r = 2; r * pcol <= 32 && r <= mbk; ++r)
+      if (mbk % r == 0) prow = r;
+    a.mbk = mbk, a.nbk = nbk;
+    a.prow = prow, a.pcol = pcol;
     a.d_brick = make_fastdiv((unsigned)(nbk * mbk));
-    a.d_panel = make_fastdiv((unsigned)(mbk * panel));
-    a.d_mbk = make_fastdiv((unsigned)mbk);
+    a.d_panel = make_fastdiv((unsigned)(prow * pcol));
+    a.d_prow = make_fastdiv((unsigned)prow);
+    a.d_pm = make_fastdiv((unsigned)(mbk / prow));
   }
   a.xn_shift = a.xn == 8 ? 3 : a.xn == 4 ? 2 : a.xn == 2 ? 1 : 0;
   a.xm_shift = a.xm == 8 ? 3 : a.xm == 4 ? 2 : a.xm == 2 ? 1 : 0;
