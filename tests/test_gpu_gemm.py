@@ -258,3 +258,32 @@ def test_gemm_wide_tile_shapes(dtype, akc, m, n, k):
                  ldb=k, ldc=n, a_kcontig=akc, b_kcontig=True, bias=biasd.data_ptr())
     torch.cuda.synchronize()
     assert rel_err(out, ref) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("m,n,k,groups,akc,bkc", [
+    (3072, 1536, 256, 1, True, True),      # 12 x 12 tiles of 256 x 128 (or 24 x 12 of 128 x 128): odd divisors
+    (1280, 3840, 192, 1, True, False),     # 5 / 10 tile rows
+    (2048, 1152, 1024, 2, False, False),   # 2 groups, 9 tile columns of 128: panels of 1 x 9 or 3 x 3
+    (4096, 2048, 2048, 4, False, False),   # long K: a strip of B tiles must fit the L2, narrow panels
+    (1792, 2560, 64, 3, True, True),       # 3 groups: no even split over the 8 XCDs
+])
+def test_gemm_many_rounds_tile_order(m, n, k, groups, akc, bkc):
+    """Launches of several rounds of tiles per CU: the order in which an XCD's tiles are handed out (bricks, panels of
+    prow x pcol tiles walked down strips of tile columns) must cover every tile exactly once whatever the divisors of
+    the tile counts are.  Output starts as NaN, so a tile that is never written shows; bf16 against fp64."""
+    ops = _ops()
+    dtype = torch.bfloat16
+    gen = torch.Generator().manual_seed(m + n + k + groups)
+    a = _rand((groups, m, k) if akc else (groups, k, m), dtype, gen)
+    b = _rand((groups, n, k) if bkc else (groups, k, n), dtype, gen)
+    A = a.double() if akc else a.double().transpose(1, 2)
+    B = b.double() if bkc else b.double().transpose(1, 2)
+    ref = A @ B.transpose(1, 2)
+    ad, bd = a.to(DEV), b.to(DEV)
+    out = torch.full((groups, m, n), float("nan"), dtype=dtype, device=DEV)
+    ops.gemm_raw(dtype, a=ad.data_ptr(), b=bd.data_ptr(), c_out=out.data_ptr(), m=m, n=n, k=k, lda=ad.stride(1),
+                 ldb=bd.stride(1), ldc=n, a_kcontig=akc, b_kcontig=bkc, groups=groups, a_sg=ad.stride(0),
+                 b_sg=bd.stride(0), c_sg=m * n)
+    torch.cuda.synchronize()
+    assert not torch.isnan(out).any()
+    assert rel_err(out, ref) <= TOL[dtype]
