@@ -190,6 +190,17 @@ int rtp_embedding_gather(void* stream, int dtype, const void* table, int64_t ld_
                          int64_t n_ids, void* out, int64_t ld_out, int64_t groups, int64_t table_sg,
                          int64_t out_sg);
 
+/* The gather fused with the two element-wise steps the language model applies to it (reference:
+ * rtp/models/transformer_lm_rtp.py:27-28 `embedding(src) * sqrt(ninp)` and :49 `x + pe[:x.size(0)]`):
+ *   out[t, c] = T( T(table[ids[t], c] * scale) + pos[t / batch, c] ), each step rounded to the element type as
+ * the separate operations round.  Tokens are laid out [sequence, batch] so t / batch is the position; shard g reads
+ * the positional table at pos + g*pos_sg (leading dimension ld_pos). */
+int rtp_embedding_gather_scale_pos(void* stream, int dtype, const void* table, int64_t ld_table,
+                                   int64_t row_begin, int64_t row_count, int64_t cols, const int64_t* ids,
+                                   int64_t n_ids, void* out, int64_t ld_out, int64_t groups, int64_t table_sg,
+                                   int64_t out_sg, float scale, const void* pos, int64_t ld_pos, int64_t pos_sg,
+                                   int64_t batch);
+
 size_t rtp_embedding_scatter_workspace_bytes(int64_t n_ids);
 
 /* Sorts (id, position) once; the result in `workspace` is reused by every shard of the layer. */
@@ -202,6 +213,15 @@ int rtp_embedding_scatter_add_det(void* stream, int dtype, const void* grad_out,
                                   int64_t row_count, int64_t cols, int64_t padding_idx,
                                   int scale_by_freq, int zero_fill, int64_t groups, int64_t grad_out_sg,
                                   int64_t grad_table_sg);
+
+/* Backward of rtp_embedding_gather_scale_pos: the same ordered sum over T(grad_out[t, :] * grad_scale), the
+ * gradient the multiplication by the scale hands to the embedding (transformer_lm_rtp.py:27-28). */
+int rtp_embedding_scatter_add_scaled(void* stream, int dtype, const void* grad_out, int64_t ld_grad_out,
+                                     int64_t n_ids, const void* workspace, void* grad_table,
+                                     int64_t ld_grad_table, int grad_table_f32, int64_t row_begin,
+                                     int64_t row_count, int64_t cols, int64_t padding_idx,
+                                     int scale_by_freq, int zero_fill, int64_t groups, int64_t grad_out_sg,
+                                     int64_t grad_table_sg, float grad_scale);
 
 /* ---------------------------------------------------------------------------------------------
  * Attention softmax (reference: rtp/module/functional.py:779-792 baddbmm+softmax, :825

@@ -79,10 +79,14 @@ PROTOTYPES = {
     "rtp_shard_copy_async": (_i, [_vp, _vp, _vp, _sz]),
     "rtp_zero_async": (_i, [_vp, _vp, _sz]),
     "rtp_embedding_gather": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _i64, _i64]),
+    "rtp_embedding_gather_scale_pos": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _i64, _i64,
+                                            _i64, _f, _vp, _i64, _i64, _i64]),
     "rtp_embedding_scatter_workspace_bytes": (_sz, [_i64]),
     "rtp_embedding_sort_ids": (_i, [_vp, _vp, _i64, _vp, _sz]),
     "rtp_embedding_scatter_add_det": (_i, [_vp, _i, _vp, _i64, _i64, _vp, _vp, _i64, _i, _i64, _i64, _i64,
                                            _i64, _i, _i, _i64, _i64, _i64]),
+    "rtp_embedding_scatter_add_scaled": (_i, [_vp, _i, _vp, _i64, _i64, _vp, _vp, _i64, _i, _i64, _i64, _i64,
+                                              _i64, _i, _i, _i64, _i64, _i64, _f]),
     "rtp_softmax_fwd": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _i64, _i, _f, _i64, _i64, _i64, _vp]),
     "rtp_softmax_bwd": (_i, [_vp, _i, _vp, _vp, _f, _i64, _i64, _i64, _vp]),
     "rtp_attn_supported": (_i, [_i, _i64, _i64]),

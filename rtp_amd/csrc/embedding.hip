@@ -8,16 +8,28 @@
 namespace rtp {
 
 // One workgroup per (token, 4 KiB column chunk); 16-byte lanes when the shard rectangle allows it.
+// With `pos` the row is scaled and a positional row added on the way: out = T(T(table * scale) + pos[t / batch]),
+// each step rounded to T as the two separate element-wise operations would round it.
 template <typename T>
 __global__ __launch_bounds__(256) void gather_kernel(const T* table, long ld_table, long row_begin, long row_count,
                                                      long cols, const int64_t* ids, T* out, long ld_out, int vec,
-                                                     long table_sg, long out_sg) {
+                                                     long table_sg, long out_sg, float scale, const T* pos, long ld_pos,
+                                                     long pos_sg, long batch) {
   const long t = blockIdx.x;
   const long row = ids[t] - row_begin;
   if (row < 0 || row >= row_count) return;
   const T* src = table + blockIdx.z * table_sg + row * ld_table;
   T* dst = out + blockIdx.z * out_sg + t * ld_out;
   constexpr int VEC = 16 / sizeof(T);
+  if (pos) {
+    const T* prow = pos + (t / batch) * ld_pos + blockIdx.z * pos_sg;
+    for (long i = (long)blockIdx.y * 256 + threadIdx.x; i < cols; i += (long)gridDim.y * 256) {
+#pragma clang fp contract(off)
+      const float a = to_f32(from_f32<T>(to_f32(src[i]) * scale));
+      dst[i] = from_f32<T>(a + to_f32(prow[i]));
+    }
+    return;
+  }
   if (vec) {
     const long nvec = cols / VEC;
     const uint4* s = reinterpret_cast<const uint4*>(src);
@@ -57,7 +69,7 @@ template <typename T, typename G>
 __global__ __launch_bounds__(256) void scatter_kernel(const T* grad_out, long ld_go, long n, const int* keys,
                                                       const int* vals, G* grad_table, long ld_gt, long row_begin,
                                                       long row_count, long cols, long padding_idx, int scale_by_freq,
-                                                      int overwrite, long go_sg, long gt_sg) {
+                                                      int overwrite, long go_sg, long gt_sg, float grad_scale) {
   grad_out += blockIdx.z * go_sg;  // group = shard: its column block of the upstream gradient, its own table
   grad_table += blockIdx.z * gt_sg;
   const long i = blockIdx.x;
@@ -71,7 +83,15 @@ __global__ __launch_bounds__(256) void scatter_kernel(const T* grad_out, long ld
   const float inv = scale_by_freq ? 1.0f / (float)(end - i) : 1.0f;
   for (long c = (long)blockIdx.y * 256 + threadIdx.x; c < cols; c += (long)gridDim.y * 256) {
     float acc = 0.0f;
-    for (long j = i; j < end; ++j) acc += to_f32(grad_out[(long)vals[j] * ld_go + c]);
+    if (grad_scale == 1.0f) {
+      for (long j = i; j < end; ++j) acc += to_f32(grad_out[(long)vals[j] * ld_go + c]);
+    } else {
+#pragma clang fp contract(off)
+      // the upstream gradient of a scaled embedding: T(grad * scale), rounded as the separate multiplication would
+      // (no fused multiply-add: the product is rounded before it joins the sum)
+      for (long j = i; j < end; ++j)
+        acc += to_f32(from_f32<T>(to_f32(grad_out[(long)vals[j] * ld_go + c]) * grad_scale));
+    }
     if (scale_by_freq) acc *= inv;
     G* dst = grad_table + row * ld_gt + c;
     if (!overwrite) acc = to_f32(*dst) + acc;
@@ -103,9 +123,10 @@ static SortLayout sort_layout(int64_t n) {
 
 using namespace rtp;
 
-extern "C" int rtp_embedding_gather(void* stream, int dtype, const void* table, int64_t ld_table, int64_t row_begin,
-                                    int64_t row_count, int64_t cols, const int64_t* ids, int64_t n_ids, void* out,
-                                    int64_t ld_out, int64_t groups, int64_t table_sg, int64_t out_sg) {
+static int gather_impl(void* stream, int dtype, const void* table, int64_t ld_table, int64_t row_begin,
+                       int64_t row_count, int64_t cols, const int64_t* ids, int64_t n_ids, void* out, int64_t ld_out,
+                       int64_t groups, int64_t table_sg, int64_t out_sg, float scale, const void* pos, int64_t ld_pos,
+                       int64_t pos_sg, int64_t batch) {
   RTP_REQUIRE(table && ids && out, "rtp_embedding_gather: null pointer");
   RTP_REQUIRE(cols >= 0 && ld_table >= cols && ld_out >= cols && row_count >= 0 && n_ids >= 0,
               "rtp_embedding_gather: bad shape cols=%lld ld_table=%lld ld_out=%lld", (long long)cols,
@@ -125,13 +146,32 @@ extern "C" int rtp_embedding_gather(void* stream, int dtype, const void* table, 
   if (dtype == RTP_F32)
     hipLaunchKernelGGL(gather_kernel<float>, grid, dim3(256), 0, s, (const float*)table, (long)ld_table,
                        (long)row_begin, (long)row_count, (long)cols, ids, (float*)out, (long)ld_out, vec,
-                       (long)table_sg, (long)out_sg);
+                       (long)table_sg, (long)out_sg, scale, (const float*)pos, (long)ld_pos, (long)pos_sg,
+                       (long)batch);
   else
     hipLaunchKernelGGL(gather_kernel<bf16_t>, grid, dim3(256), 0, s, (const bf16_t*)table, (long)ld_table,
                        (long)row_begin, (long)row_count, (long)cols, ids, (bf16_t*)out, (long)ld_out, vec,
-                       (long)table_sg, (long)out_sg);
+                       (long)table_sg, (long)out_sg, scale, (const bf16_t*)pos, (long)ld_pos, (long)pos_sg,
+                       (long)batch);
   RTP_LAUNCH_CHECK();
   return RTP_OK;
+}
+
+extern "C" int rtp_embedding_gather(void* stream, int dtype, const void* table, int64_t ld_table, int64_t row_begin,
+                                    int64_t row_count, int64_t cols, const int64_t* ids, int64_t n_ids, void* out,
+                                    int64_t ld_out, int64_t groups, int64_t table_sg, int64_t out_sg) {
+  return gather_impl(stream, dtype, table, ld_table, row_begin, row_count, cols, ids, n_ids, out, ld_out, groups,
+                     table_sg, out_sg, 1.0f, nullptr, 0, 0, 1);
+}
+
+extern "C" int rtp_embedding_gather_scale_pos(void* stream, int dtype, const void* table, int64_t ld_table,
+                                              int64_t row_begin, int64_t row_count, int64_t cols, const int64_t* ids,
+                                              int64_t n_ids, void* out, int64_t ld_out, int64_t groups,
+                                              int64_t table_sg, int64_t out_sg, float scale, const void* pos,
+                                              int64_t ld_pos, int64_t pos_sg, int64_t batch) {
+  RTP_REQUIRE(pos && batch >= 1 && ld_pos >= cols, "rtp_embedding_gather_scale_pos: need a positional table and batch >= 1");
+  return gather_impl(stream, dtype, table, ld_table, row_begin, row_count, cols, ids, n_ids, out, ld_out, groups,
+                     table_sg, out_sg, scale, pos, ld_pos, pos_sg, batch);
 }
 
 extern "C" size_t rtp_embedding_scatter_workspace_bytes(int64_t n_ids) {
@@ -160,12 +200,10 @@ extern "C" int rtp_embedding_sort_ids(void* stream, const int64_t* ids, int64_t 
   return RTP_OK;
 }
 
-extern "C" int rtp_embedding_scatter_add_det(void* stream, int dtype, const void* grad_out, int64_t ld_grad_out,
-                                             int64_t n_ids, const void* workspace, void* grad_table,
-                                             int64_t ld_grad_table, int grad_table_f32, int64_t row_begin,
-                                             int64_t row_count, int64_t cols, int64_t padding_idx, int scale_by_freq,
-                                             int zero_fill, int64_t groups, int64_t grad_out_sg,
-                                             int64_t grad_table_sg) {
+static int scatter_impl(void* stream, int dtype, const void* grad_out, int64_t ld_grad_out, int64_t n_ids,
+                        const void* workspace, void* grad_table, int64_t ld_grad_table, int grad_table_f32,
+                        int64_t row_begin, int64_t row_count, int64_t cols, int64_t padding_idx, int scale_by_freq,
+                        int zero_fill, int64_t groups, int64_t grad_out_sg, int64_t grad_table_sg, float grad_scale) {
   RTP_REQUIRE(grad_out && workspace && grad_table, "rtp_embedding_scatter_add_det: null pointer");
   RTP_REQUIRE(groups >= 1 && groups < 65536, "rtp_embedding_scatter_add_det: groups %lld not in 1..65535",
               (long long)groups);
@@ -204,7 +242,8 @@ extern "C" int rtp_embedding_scatter_add_det(void* stream, int dtype, const void
 #define RTP_SCATTER(T, G)                                                                                         \
   hipLaunchKernelGGL((scatter_kernel<T, G>), grid, dim3(256), 0, s, (const T*)grad_out, (long)ld_grad_out,         \
                      (long)n_ids, keys, vals, (G*)grad_table, (long)ld_grad_table, (long)row_begin, (long)row_count, \
-                     (long)cols, (long)padding_idx, scale_by_freq, overwrite, (long)grad_out_sg, (long)grad_table_sg)
+                     (long)cols, (long)padding_idx, scale_by_freq, overwrite, (long)grad_out_sg, (long)grad_table_sg,  \
+                     grad_scale)
   // algorithmic bytes: read every upstream row once, write (or read-modify-write) every touched row once
   ProfileScope prof(s, "embedding_scatter_add", (double)groups * n_ids * cols,
                     (double)groups * n_ids * cols * ((dtype == RTP_F32 ? 4.0 : 2.0) + (zero_fill ? 1.0 : 2.0) * gsz) + 8.0 * n_ids);
@@ -217,4 +256,26 @@ extern "C" int rtp_embedding_scatter_add_det(void* stream, int dtype, const void
 #undef RTP_SCATTER
   RTP_LAUNCH_CHECK();
   return RTP_OK;
+}
+
+extern "C" int rtp_embedding_scatter_add_det(void* stream, int dtype, const void* grad_out, int64_t ld_grad_out,
+                                             int64_t n_ids, const void* workspace, void* grad_table,
+                                             int64_t ld_grad_table, int grad_table_f32, int64_t row_begin,
+                                             int64_t row_count, int64_t cols, int64_t padding_idx, int scale_by_freq,
+                                             int zero_fill, int64_t groups, int64_t grad_out_sg,
+                                             int64_t grad_table_sg) {
+  return scatter_impl(stream, dtype, grad_out, ld_grad_out, n_ids, workspace, grad_table, ld_grad_table, grad_table_f32,
+                      row_begin, row_count, cols, padding_idx, scale_by_freq, zero_fill, groups, grad_out_sg,
+                      grad_table_sg, 1.0f);
+}
+
+extern "C" int rtp_embedding_scatter_add_scaled(void* stream, int dtype, const void* grad_out, int64_t ld_grad_out,
+                                                int64_t n_ids, const void* workspace, void* grad_table,
+                                                int64_t ld_grad_table, int grad_table_f32, int64_t row_begin,
+                                                int64_t row_count, int64_t cols, int64_t padding_idx,
+                                                int scale_by_freq, int zero_fill, int64_t groups, int64_t grad_out_sg,
+                                                int64_t grad_table_sg, float grad_scale) {
+  return scatter_impl(stream, dtype, grad_out, ld_grad_out, n_ids, workspace, grad_table, ld_grad_table, grad_table_f32,
+                      row_begin, row_count, cols, padding_idx, scale_by_freq, zero_fill, groups, grad_out_sg,
+                      grad_table_sg, grad_scale);
 }

@@ -5,6 +5,7 @@ Residual add + LayerNorm is one fused kernel each way (module/norm.py); the FFN'
 from __future__ import annotations
 
 import math
+import os
 
 import torch
 import torch.nn as nn
@@ -27,9 +28,21 @@ class EmbeddingLayer(nn.Module):
             for shard in self.embedding.embeddings:
                 shard.weight.data.uniform_(-initrange, initrange)
         self.ninp_sqrt = math.sqrt(ninp)
+        self.positional = None  # set by adopt_positional
+
+    def adopt_positional(self, layer: "PositionalEncodingLayer") -> None:
+        """Take over the addition of the positional rows from the layer that follows (which then only applies its
+        dropout), so that scale and addition ride on the gather instead of two passes over the activations."""
+        object.__setattr__(self, "positional", layer)  # plain attribute: the layer stays registered once, in the model
+        layer.added_upstream = True
 
     def forward(self, src):
-        return self.embedding(src) * self.ninp_sqrt
+        pos = self.positional
+        if pos is None:
+            return self.embedding(src) * self.ninp_sqrt
+        if src.dim() == 2 and pos.pe.dtype == self.embedding._store.home.dtype:
+            return self.embedding.forward_scaled_positional(src, self.ninp_sqrt, pos.pe[:, 0, :])
+        return self.embedding(src) * self.ninp_sqrt + pos.pe[: src.size(0), :]
 
 
 class PositionalEncodingLayer(nn.Module):
@@ -43,9 +56,11 @@ class PositionalEncodingLayer(nn.Module):
         pe[:, 1::2] = torch.cos(position * div_term)
         pe = pe.unsqueeze(0).transpose(0, 1)
         self.register_buffer("pe", pe.to(device=device, dtype=dtype))
+        self.added_upstream = False  # True once the embedding layer before this one adds the rows itself
 
     def forward(self, x):
-        x = x + self.pe[: x.size(0), :]
+        if not self.added_upstream:
+            x = x + self.pe[: x.size(0), :]
         return self.dropout(x)
 
 
@@ -193,3 +208,5 @@ class TransformerLM(nn.Sequential):
                                                   world_size=world_size, rank=rank, device=device, dtype=dtype))
         layers.append(LinearLayer(ninp, ntokens, initrange, world_size, rank, device=device, dtype=dtype))
         super().__init__(*layers)
+        if os.environ.get("RTP_EMBED_FUSE", "1") != "0":
+            layers[0].adopt_positional(layers[1])

@@ -42,19 +42,23 @@ class ModelParallelEmbedding(nn.Embedding):
 
 class _EmbeddingFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, ids, anchor, layer):
+    def forward(ctx, ids, anchor, layer, scale=1.0, pos=None):
         store = layer._store
         d_s, ws = layer.embedding_dim_per_partition, layer.world_size
         flat_ids = ids.reshape(-1).contiguous()
         out = torch.empty(flat_ids.numel(), layer.embedding_dim, dtype=store.home.dtype, device=store.home.device)
         rot = Rotation(store.home, ring_order(layer.rank, ws), group=store.stage_group)
+        # tokens are [sequence, batch, ...]: every id of one position shares a positional row
+        batch = flat_ids.numel() // ids.shape[0] if pos is not None else 1
         for j in range(rot.steps):
             for flat, first, cnt in rot.acquire(j):
                 table = flat[0].view(layer.num_embeddings, d_s)
-                ops.embedding_gather(table, flat_ids, out[:, first * d_s:(first + 1) * d_s], groups=cnt,
-                                     table_sg=store.numel, out_sg=d_s)
+                cols = slice(first * d_s, (first + 1) * d_s)
+                ops.embedding_gather(table, flat_ids, out[:, cols], groups=cnt, table_sg=store.numel, out_sg=d_s,
+                                     scale=scale, pos=None if pos is None else pos[:, cols], pos_sg=d_s, batch=batch)
             rot.release(j)
         ctx.layer = layer
+        ctx.grad_scale = scale
         ctx.save_for_backward(flat_ids)
         return out.view(*ids.shape, layer.embedding_dim)
 
@@ -77,9 +81,9 @@ class _EmbeddingFn(torch.autograd.Function):
             ops.embedding_scatter_add(g2[:, first * d_s:(first + 1) * d_s], flat_ids.numel(), workspace, table,
                                       padding_idx=pad, scale_by_freq=layer.scale_grad_by_freq,
                                       zero_fill=not accumulate, groups=cnt, grad_out_sg=d_s,
-                                      grad_table_sg=store.grads.shape[1])
+                                      grad_table_sg=store.grads.shape[1], grad_scale=ctx.grad_scale)
         store.grads_ready()
-        return None, None, None
+        return None, None, None, None, None
 
 
 class ParallelEmbedding(RotatedLayer):
@@ -129,3 +133,15 @@ class ParallelEmbedding(RotatedLayer):
         if input_.dtype != torch.int64:
             input_ = input_.long()
         return _EmbeddingFn.apply(input_, self._anchor, self)
+
+    def forward_scaled_positional(self, input_: torch.Tensor, scale: float, pos: torch.Tensor) -> torch.Tensor:
+        """(self(input_) * scale) + pos[:input_.size(0), None, :] in one gather per shard group, with the rounding
+        of the separate operations; `input_` is [sequence, batch], `pos` a [positions, embedding_dim] table of the
+        layer's dtype that needs no gradient (rtp/models/transformer_lm_rtp.py:27-28 and :49)."""
+        if input_.dim() != 2 or pos.dim() != 2 or pos.shape[1] != self.embedding_dim or pos.requires_grad:
+            raise ValueError("forward_scaled_positional: ids must be [sequence, batch] and pos [positions, dim]")
+        if input_.shape[0] > pos.shape[0]:
+            raise ValueError("forward_scaled_positional: sequence longer than the positional table")
+        if input_.dtype != torch.int64:
+            input_ = input_.long()
+        return _EmbeddingFn.apply(input_, self._anchor, self, float(scale), pos)

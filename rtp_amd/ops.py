@@ -194,9 +194,12 @@ def zero_(t: torch.Tensor) -> None:
 
 
 def embedding_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, row_begin: int = 0, groups: int = 1,
-                     table_sg: int = 0, out_sg: int = 0) -> None:
+                     table_sg: int = 0, out_sg: int = 0, *, scale: float = 1.0, pos: Optional[torch.Tensor] = None,
+                     pos_sg: int = 0, batch: int = 1) -> None:
     """out[t, :] = table[ids[t] - row_begin, :] for ids inside the shard's row range.  With groups > 1,
-    `table` / `out` are shard 0's table and output block; shard g sits table_sg / out_sg elements further."""
+    `table` / `out` are shard 0's table and output block; shard g sits table_sg / out_sg elements further.
+    With `pos` ([positions, cols] block of a positional table, shard g at pos_sg elements further) the row is
+    scaled and the positional row of token t (position t // batch) added, rounding after each step."""
     for t in (table, ids, out):
         _dev(t)
     rows, cols, ld_t = _mat(table, "table")
@@ -205,6 +208,17 @@ def embedding_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, 
             out.dtype != table.dtype:
         raise ValueError("embedding_gather: ids must be contiguous int64 with one id per output row")
     _lib.require_device()
+    if pos is not None:
+        _dev(pos)
+        p_rows, p_cols, ld_p = _mat(pos, "pos")
+        if pos.dtype != table.dtype or p_cols != cols or batch < 1 or (n + batch - 1) // batch > p_rows:
+            raise ValueError("embedding_gather: pos must hold one row of the table's dtype per position")
+        check(_lib.load().rtp_embedding_gather_scale_pos(
+            _stream(), dtype_code(table.dtype), table.data_ptr(), ld_t, row_begin, rows, cols, ids.data_ptr(), n,
+            out.data_ptr(), ld_o, groups, table_sg, out_sg, float(scale), pos.data_ptr(), ld_p, pos_sg, batch))
+        return
+    if scale != 1.0:
+        raise ValueError("embedding_gather: a scale needs the positional table")
     check(_lib.load().rtp_embedding_gather(_stream(), dtype_code(table.dtype), table.data_ptr(), ld_t, row_begin,
                                            rows, cols, ids.data_ptr(), n, out.data_ptr(), ld_o, groups, table_sg,
                                            out_sg))
@@ -226,10 +240,11 @@ def embedding_sort_ids(ids: torch.Tensor) -> torch.Tensor:
 def embedding_scatter_add(grad_out: torch.Tensor, n_ids: int, workspace: torch.Tensor, grad_table: torch.Tensor,
                           *, row_begin: int = 0, padding_idx: int = -1, scale_by_freq: bool = False,
                           zero_fill: bool = True, groups: int = 1, grad_out_sg: int = 0,
-                          grad_table_sg: int = 0) -> None:
+                          grad_table_sg: int = 0, grad_scale: float = 1.0) -> None:
     """grad_table[id] (+)= sum of the grad_out rows whose token is id, in ascending position order.  With
     groups > 1, group g reads grad_out + g*grad_out_sg and writes grad_table + g*grad_table_sg (elements):
-    all shards of an embedding in one launch."""
+    all shards of an embedding in one launch.  grad_scale != 1 sums grad_out * grad_scale, each product rounded
+    to grad_out's dtype first (the gradient a scaled embedding receives)."""
     for t in (grad_out, workspace, grad_table):
         _dev(t)
     n, cols, ld_go = _mat(grad_out, "grad_out")
@@ -239,11 +254,14 @@ def embedding_scatter_add(grad_out: torch.Tensor, n_ids: int, workspace: torch.T
     if grad_table.dtype not in (grad_out.dtype, torch.float32):
         raise TypeError("embedding_scatter_add: grad_table must be the grad dtype or float32")
     _lib.require_device()
-    check(_lib.load().rtp_embedding_scatter_add_det(
-        _stream(), dtype_code(grad_out.dtype), grad_out.data_ptr(), ld_go, n_ids, workspace.data_ptr(),
-        grad_table.data_ptr(), ld_gt, int(grad_table.dtype == torch.float32), row_begin, rows, cols,
-        -1 if padding_idx is None else padding_idx, int(scale_by_freq), int(zero_fill), groups, grad_out_sg,
-        grad_table_sg))
+    args = (_stream(), dtype_code(grad_out.dtype), grad_out.data_ptr(), ld_go, n_ids, workspace.data_ptr(),
+            grad_table.data_ptr(), ld_gt, int(grad_table.dtype == torch.float32), row_begin, rows, cols,
+            -1 if padding_idx is None else padding_idx, int(scale_by_freq), int(zero_fill), groups, grad_out_sg,
+            grad_table_sg)
+    if grad_scale != 1.0:
+        check(_lib.load().rtp_embedding_scatter_add_scaled(*args, float(grad_scale)))
+    else:
+        check(_lib.load().rtp_embedding_scatter_add_det(*args))
 
 
 def _key_bias_ptr(who: str, key_bias: Optional[torch.Tensor], n_batch: int, keys: int):

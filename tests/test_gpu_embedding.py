@@ -77,3 +77,37 @@ def test_embedding_unsupported_options_raise():
         ParallelEmbedding(8, 8, 2, 0, max_norm=1.0, device=DEV)
     with pytest.raises(NotImplementedError):
         ParallelEmbedding(8, 8, 2, 0, sparse=True, device=DEV)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("ws", [1, 4])
+def test_embedding_scaled_positional_is_bit_exact(dtype, ws):
+    """(embedding(ids) * sqrt(d) + pe[:L]) and its backward, as the language model applies them
+    (rtp/models/transformer_lm_rtp.py:27-28, :49), against the same three torch CPU operations: each step
+    rounds to the element type, so equality is exact in fp32 and in bf16."""
+    import math
+    gen = torch.Generator().manual_seed(3)
+    v, d, seq, batch = 37, 48, 11, 5
+    master = nn.Embedding(v, d).to(dtype)
+    pe = torch.randn(seq + 3, d, generator=gen).to(dtype)
+    ids = torch.randint(0, v, (seq, batch), generator=gen)
+    g = torch.randn(seq, batch, d, generator=gen).to(dtype)
+    scale = math.sqrt(d)
+    layer = _layer(master, ws, dtype)
+    out = layer.forward_scaled_positional(ids.to(DEV), scale, pe.to(DEV))
+    ref = master(ids) * scale + pe[:seq, None, :]
+    assert out.dtype == dtype and torch.equal(out.cpu(), ref.detach())
+    out.backward(g.to(DEV))
+    ref.backward(g)
+    dw = torch.cat([e.weight.grad for e in layer.embeddings], dim=1).cpu()
+    if dtype == torch.float32:
+        assert torch.equal(dw, master.weight.grad)
+    else:
+        # torch's CPU bf16 index_add_ rounds the running sum after every add; the device sums in fp32 and rounds
+        # once, so compare with the fp32 ordered sum of the bf16-rounded scaled rows
+        scaled = (g * scale).float().numpy()
+        want = O.embedding_backward_sequential(ids.numpy(), scaled, v, None)
+        want_t = torch.from_numpy(want).to(dw.dtype)  # the gradient buffer is fp32 or the layer's dtype
+        assert torch.equal(dw, want_t)
+    with pytest.raises(ValueError):
+        layer.forward_scaled_positional(ids.to(DEV), scale, pe[:seq - 1].to(DEV))

@@ -258,3 +258,24 @@ def test_lm_rank_state_dicts_round_trip_on_device():
     load_rank_state_dicts(moe2, [rank_state_dict(moe, r) for r in range(4)])
     for (ka, ta), (kb, tb) in zip(moe.state_dict().items(), moe2.state_dict().items()):
         assert ka == kb and torch.equal(ta, tb)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_lm_embedding_scale_and_positions_on_the_gather_are_bit_identical(dtype, monkeypatch):
+    """The model lets the embedding gather apply * sqrt(ninp) and + pe (transformer_lm_rtp.py:27-28, :49); with
+    RTP_EMBED_FUSE=0 the three steps run as separate operations.  Logits and every gradient must not change."""
+    V, D, H, Fd, n_dec, L, N = 96, 64, 4, 64, 2, 12, 5
+    gen = torch.Generator().manual_seed(1)
+    ids = torch.randint(0, V, (L, N), generator=gen).to(DEV)
+    tgt = torch.randint(0, V, (L, N), generator=gen).to(DEV)
+    results = []
+    for fuse in ("1", "0"):
+        monkeypatch.setenv("RTP_EMBED_FUSE", fuse)
+        lm, _ = build_pair(V, D, H, Fd, n_dec, 4, dtype)
+        assert lm[1].added_upstream == (fuse == "1")
+        logits = lm(ids)
+        F.cross_entropy(logits.float().view(-1, V), tgt.view(-1)).backward()
+        results.append((logits.detach(), gathered_grads(lm, 4)))
+    assert torch.equal(results[0][0], results[1][0])
+    for k, g in results[0][1].items():
+        assert torch.equal(g, results[1][1][k]), k
