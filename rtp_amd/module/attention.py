@@ -29,7 +29,8 @@ from .utils import (affine_weight, affine_weight_attention, as_rows, attention_b
 
 class SubParallelMultiheadAttention(nn.Module):
     """Parameters of one head group (rtp/module/attention.py:17-104).  Declaration order fixes the
-    flat-shard layout: in_proj_weight, in_proj_bias, out_proj.weight, out_proj.bias."""
+    flat-shard layout: in_proj_weight (or q_proj_weight, k_proj_weight, v_proj_weight when keys or values have
+    their own width), in_proj_bias, out_proj.weight, out_proj.bias."""
 
     def __init__(self, embed_dim, num_heads, world_size, rank, dropout=0., bias=True, add_bias_kv=False,
                  add_zero_attn=False, kdim=None, vdim=None, batch_first=False, device=None, dtype=None) -> None:
@@ -39,11 +40,13 @@ class SubParallelMultiheadAttention(nn.Module):
         super().__init__()
         kdim = embed_dim if kdim is None else kdim
         vdim = embed_dim if vdim is None else vdim
-        if kdim != embed_dim or vdim != embed_dim or add_bias_kv or add_zero_attn:
-            raise NotImplementedError("rotated attention: kdim/vdim != embed_dim, add_bias_kv and add_zero_attn "
-                                      "are not implemented")
+        if add_bias_kv:
+            # the reference keeps bias_k / bias_v at full width [1, 1, embed_dim] in every shard and concatenates
+            # them to keys of width embed_dim / ws (attention.py:70-72, functional.py:711-716): that only runs
+            # with one shard, so there is no sharded behaviour to reproduce
+            raise NotImplementedError("rotated attention: add_bias_kv is not implemented")
         self.embed_dim, self.kdim, self.vdim = embed_dim, kdim, vdim
-        self._qkv_same_embed_dim = True
+        self._qkv_same_embed_dim = kdim == embed_dim and vdim == embed_dim
         self.num_heads = num_heads
         self.dropout = dropout
         self.batch_first = batch_first
@@ -54,7 +57,14 @@ class SubParallelMultiheadAttention(nn.Module):
         self.embed_dim_per_partition = divide_and_check_no_remainder(embed_dim, world_size)
         e_s = self.embed_dim_per_partition
         kw = {"device": device, "dtype": dtype}
-        self.in_proj_weight = Parameter(torch.empty((3 * e_s, embed_dim), **kw))
+        if self._qkv_same_embed_dim:
+            self.in_proj_weight = Parameter(torch.empty((3 * e_s, embed_dim), **kw))
+        else:
+            # attention.py:51-55: three separate row blocks when keys or values have their own width
+            self.q_proj_weight = Parameter(torch.empty((e_s, embed_dim), **kw))
+            self.k_proj_weight = Parameter(torch.empty((e_s, kdim), **kw))
+            self.v_proj_weight = Parameter(torch.empty((e_s, vdim), **kw))
+            self.register_parameter("in_proj_weight", None)
         self.bias = bias
         if bias:
             self.in_proj_bias = Parameter(torch.empty(3 * e_s, **kw))
@@ -68,7 +78,11 @@ class SubParallelMultiheadAttention(nn.Module):
     def _reset_parameters(self) -> None:
         # The reference leaves in_proj_* as torch.empty (attention.py:57,64); give them the
         # nn.MultiheadAttention defaults instead of uninitialised memory.
-        nn.init.xavier_uniform_(self.in_proj_weight)
+        if self._qkv_same_embed_dim:
+            nn.init.xavier_uniform_(self.in_proj_weight)
+        else:
+            for w in (self.q_proj_weight, self.k_proj_weight, self.v_proj_weight):
+                nn.init.xavier_uniform_(w)
         if self.in_proj_bias is not None:
             nn.init.constant_(self.in_proj_bias, 0.)
             nn.init.constant_(self.out_proj.bias, 0.)
@@ -78,7 +92,12 @@ class SubParallelMultiheadAttention(nn.Module):
             return
         idx = attention_block_index(self.rank, self.world_size)
         e_s = self.embed_dim_per_partition
-        affine_weight_attention(self.in_proj_weight, mha.in_proj_weight, idx, e_s, 0, self.world_size, self.rank)
+        if self._qkv_same_embed_dim:
+            affine_weight_attention(self.in_proj_weight, mha.in_proj_weight, idx, e_s, 0, self.world_size, self.rank)
+        else:
+            for mine, theirs in ((self.q_proj_weight, mha.q_proj_weight), (self.k_proj_weight, mha.k_proj_weight),
+                                 (self.v_proj_weight, mha.v_proj_weight)):
+                affine_weight(mine, theirs, e_s, 0, self.world_size, self.rank)
         if self.bias:
             affine_weight_attention(self.in_proj_bias, mha.in_proj_bias, idx, e_s, 0, self.world_size, self.rank)
         affine_weight(self.out_proj.weight, mha.out_proj.weight, e_s, 1, self.world_size, self.rank)
@@ -272,11 +291,177 @@ class _AttentionFn(torch.autograd.Function):
         return (dx.view(L, N, E) if need_dx else None), None, None, None, None, None, None, None
 
 
+def _shard_layout(layer):
+    """Element offsets inside a flat shard of (W_q, W_k, W_v, b_in, W_o, b_o); b_in / b_o are None without biases."""
+    off = layer._store.offsets
+    e_s, E = layer.embed_dim_per_partition, layer.embed_dim
+    if layer.separate_proj:
+        wq, wk, wv, nxt = off[0], off[1], off[2], 3
+    else:
+        wq, wk, wv, nxt = off[0], off[0] + e_s * E, off[0] + 2 * e_s * E, 1
+    if layer.has_bias:
+        return wq, wk, wv, off[nxt], off[nxt + 1], off[nxt + 2]
+    return wq, wk, wv, None, off[nxt], None
+
+
+class _GeneralAttentionFn(torch.autograd.Function):
+    """Attention whose keys and values come from their own tensors (query [L, N, E], key [S, N, kdim], value
+    [S, N, vdim]; functional.py:575-609 projects them with three row blocks of the shard), optionally with one
+    all-zero key / value appended per batch entry (add_zero_attn, functional.py:746-753).  Three projections per
+    shard run into q [L*N, E], k and v [(S+z)*N, E] (group g at column block g); the core is batched products and
+    the softmax kernel with p [ws*N*h_s, L, S+z] in memory."""
+
+    @staticmethod
+    def forward(ctx, query, key, value, anchor, layer, mask, key_bias, want_weights):
+        store = layer._store
+        L, N, E = query.shape
+        s_in = key.shape[0]
+        zero = 1 if layer.add_zero_attn else 0
+        sk = s_in + zero
+        ws, h_s, d, e_s = layer.world_size, layer.num_heads_per_partition, layer.head_dim, layer.embed_dim_per_partition
+        dt, dev = query.dtype, query.device
+        q2, k2, v2 = as_rows(query, E), as_rows(key, layer.kdim), as_rows(value, layer.vdim)
+        wq, wk, wv, b_in, w_o, b_o = _shard_layout(layer)
+        bq, bk, bv = (b_in, b_in + e_s, b_in + 2 * e_s) if b_in is not None else (None, None, None)
+        Z = N * h_s
+        scale = 1.0 / math.sqrt(d)
+        qb = torch.empty(L * N, E, dtype=dt, device=dev)
+        kb = torch.empty(sk * N, E, dtype=dt, device=dev)
+        vb = torch.empty(sk * N, E, dtype=dt, device=dev)
+        if zero:
+            kb[s_in * N:].zero_()
+            vb[s_in * N:].zero_()
+        o = torch.empty(L * N, E, dtype=dt, device=dev)
+        out = torch.empty(L * N, E, dtype=dt, device=dev)
+        p = torch.empty(ws * Z, L, sk, dtype=dt, device=dev)
+        ld = N * E  # one step along the sequence in q, k, v and o
+        order = ring_order(layer.rank, ws)
+        rot = Rotation(store.home, order, group=store.stage_group)
+        acc = ops.ShardSum(out, sum(len(w) for w in rot.windows))
+        i = 0
+        for j in range(rot.steps):
+            for flat, first, cnt in rot.acquire(j):
+                c0 = first * e_s
+                S.col_fwd(q2, flat, wq, e_s, E, bq, qb, c0)
+                S.col_fwd(k2, flat, wk, e_s, layer.kdim, bk, kb[:s_in * N], c0)
+                S.col_fwd(v2, flat, wv, e_s, layer.vdim, bv, vb[:s_in * N], c0)
+                scores = torch.empty(cnt * Z, L, sk, dtype=torch.float32, device=dev)
+                _bmm(dt, a=qb, a_off=c0, lda=ld, a_kc=True, a_s=(E, d), a_sg=e_s, b=kb, b_off=c0, ldb=ld, b_kc=True,
+                     b_s=(E, d), b_sg=e_s, c=scores, c_off=0, ldc=sk, c_s=(h_s * L * sk, L * sk), c_sg=Z * L * sk,
+                     m=L, n=sk, k=d, batch=Z, zdiv=h_s, groups=cnt, out_f32=True)
+                ops.softmax_fwd(scores, p[first * Z:(first + cnt) * Z], mask=mask, causal=False, scale=scale,
+                                key_bias=key_bias, heads=h_s)
+                del scores
+                _bmm(dt, a=p, a_off=first * Z * L * sk, lda=sk, a_kc=True, a_s=(h_s * L * sk, L * sk),
+                     a_sg=Z * L * sk, b=vb, b_off=c0, ldb=ld, b_kc=False, b_s=(E, d), b_sg=e_s, c=o, c_off=c0, ldc=ld,
+                     c_s=(E, d), c_sg=e_s, m=L, n=d, k=sk, batch=Z, zdiv=h_s, groups=cnt)
+                c_out, c_in = acc.target(i)
+                S.row_fwd(o, flat, w_o, E, e_s, b_o, c_out, c0, c_in=c_in)
+                i += 1
+            rot.release(j)
+        weights = None
+        if want_weights:
+            last = order[-1]
+            weights = p[last * Z:(last + 1) * Z].view(N, h_s, L, sk)
+        ctx.layer = layer
+        ctx.dims = (L, N, E, s_in, sk)
+        ctx.save_for_backward(q2, k2, v2, qb, kb, vb, p, o)
+        ctx.mark_non_differentiable(*([weights] if weights is not None else []))
+        return out.view(L, N, E), weights
+
+    @staticmethod
+    def backward(ctx, dout, _dweights=None):
+        layer = ctx.layer
+        q2, k2, v2, qb, kb, vb, p, o = ctx.saved_tensors
+        store = layer._store
+        L, N, E, s_in, sk = ctx.dims
+        ws, h_s, d, e_s = layer.world_size, layer.num_heads_per_partition, layer.head_dim, layer.embed_dim_per_partition
+        dt, dev = q2.dtype, q2.device
+        wq, wk, wv, b_in, w_o, b_o = _shard_layout(layer)
+        bq, bk, bv = (b_in, b_in + e_s, b_in + 2 * e_s) if b_in is not None else (None, None, None)
+        Z = N * h_s
+        scale = 1.0 / math.sqrt(d)
+        ld = N * E
+        dout2 = as_rows(dout, E)
+        do = torch.empty(L * N, E, dtype=dt, device=dev)
+        dqb = torch.empty(L * N, E, dtype=dt, device=dev)
+        dkb = torch.empty(sk * N, E, dtype=dt, device=dev)
+        dvb = torch.empty(sk * N, E, dtype=dt, device=dev)
+        order = ring_order(layer.rank, ws, reverse=True)
+        rot = Rotation(store.home, order, group=store.stage_group)
+        parts = sum(len(w) for w in rot.windows)
+        # input gradients of the three projections, each summed over the shards; the rows of an appended zero key
+        # belong to no input
+        sums = []
+        for need, src, rows, width, w_off in ((ctx.needs_input_grad[0], dqb, L * N, E, wq),
+                                              (ctx.needs_input_grad[1], dkb, s_in * N, layer.kdim, wk),
+                                              (ctx.needs_input_grad[2], dvb, s_in * N, layer.vdim, wv)):
+            if need:
+                dx = torch.empty(rows, width, dtype=dt, device=dev)
+                sums.append((dx, ops.ShardSum(dx, parts), src[:rows], width, w_off))
+            else:
+                sums.append(None)
+        i = 0
+        for j in range(rot.steps):
+            for flat, first, cnt in rot.acquire(j):
+                c0 = first * e_s
+                p_off = first * Z * L * sk
+                p_s, p_sg = (h_s * L * sk, L * sk), Z * L * sk
+                S.row_dgrad(dout2, flat, w_o, E, e_s, do, c0)
+                # dP = dO V^T
+                dp = torch.empty(cnt * Z, L, sk, dtype=torch.float32, device=dev)
+                _bmm(dt, a=do, a_off=c0, lda=ld, a_kc=True, a_s=(E, d), a_sg=e_s, b=vb, b_off=c0, ldb=ld, b_kc=True,
+                     b_s=(E, d), b_sg=e_s, c=dp, c_off=0, ldc=sk, c_s=p_s, c_sg=p_sg, m=L, n=sk, k=d, batch=Z,
+                     zdiv=h_s, groups=cnt, out_f32=True)
+                # dV = P^T dO
+                _bmm(dt, a=p, a_off=p_off, lda=sk, a_kc=False, a_s=p_s, a_sg=p_sg, b=do, b_off=c0, ldb=ld, b_kc=False,
+                     b_s=(E, d), b_sg=e_s, c=dvb, c_off=c0, ldc=ld, c_s=(E, d), c_sg=e_s, m=sk, n=d, k=L, batch=Z,
+                     zdiv=h_s, groups=cnt)
+                ds = torch.empty(cnt * Z, L, sk, dtype=dt, device=dev)
+                ops.softmax_bwd(p[first * Z:(first + cnt) * Z], dp, ds, scale)
+                del dp
+                # dQ = dS K
+                _bmm(dt, a=ds, a_off=0, lda=sk, a_kc=True, a_s=p_s, a_sg=p_sg, b=kb, b_off=c0, ldb=ld, b_kc=False,
+                     b_s=(E, d), b_sg=e_s, c=dqb, c_off=c0, ldc=ld, c_s=(E, d), c_sg=e_s, m=L, n=d, k=sk, batch=Z,
+                     zdiv=h_s, groups=cnt)
+                # dK = dS^T Q
+                _bmm(dt, a=ds, a_off=0, lda=sk, a_kc=False, a_s=p_s, a_sg=p_sg, b=qb, b_off=c0, ldb=ld, b_kc=False,
+                     b_s=(E, d), b_sg=e_s, c=dkb, c_off=c0, ldc=ld, c_s=(E, d), c_sg=e_s, m=sk, n=d, k=L, batch=Z,
+                     zdiv=h_s, groups=cnt)
+                for item in sums:
+                    if item is not None:
+                        _, acc, src, width, w_off = item
+                        c_out, c_in = acc.target(i)
+                        S.col_dgrad(src, flat, w_off, e_s, width, c_out, c0, c_in=c_in)
+                i += 1
+            rot.release(j)
+        runs = store.grad_runs(order)
+        dk_in, dv_in = dkb[:s_in * N], dvb[:s_in * N]
+
+        def param_grads():
+            for first, cnt, accumulate in runs:
+                c0 = first * e_s
+                S.row_wgrad(dout2, o, store.grads, first, w_o, E, e_s, c0, cnt, accumulate, b_off=b_o)
+                S.col_wgrad(dqb, q2, store.grads, first, wq, e_s, E, c0, cnt, accumulate, b_off=bq)
+                S.col_wgrad(dk_in, k2, store.grads, first, wk, e_s, layer.kdim, c0, cnt, accumulate, b_off=bk)
+                S.col_wgrad(dv_in, v2, store.grads, first, wv, e_s, layer.vdim, c0, cnt, accumulate, b_off=bv)
+            store.grads_ready()
+
+        run_wgrad(dev, param_grads, (dout2, o, dqb, dk_in, dv_in, q2, k2, v2))
+        grads = [None if item is None else item[0] for item in sums]
+        dq = None if grads[0] is None else grads[0].view(L, N, E)
+        dk = None if grads[1] is None else grads[1].view(s_in, N, layer.kdim)
+        dv = None if grads[2] is None else grads[2].view(s_in, N, layer.vdim)
+        return dq, dk, dv, None, None, None, None, None
+
+
 class ParallelMultiheadAttention(RotatedLayer):
     """Signature follows rtp/module/attention.py:192-193; `MultiheadAttention_layer` imports the weights
-    of an unsharded nn.MultiheadAttention.  Self-attention only (query, key and value must be the same
-    tensor); 3-D masks and attention dropout are not implemented and raise.  key_padding_mask [batch, keys] (bool or
-    float, functional.py:615-623 and :760-768) reaches the kernels as a per-(batch, key) additive bias."""
+    of an unsharded nn.MultiheadAttention.  Self-attention (query, key and value the same tensor) takes the packed
+    projection and the fused cores; keys / values from other tensors, kdim / vdim != embed_dim and add_zero_attn take
+    three projections and the product + softmax core.  3-D masks, add_bias_kv and attention dropout are not
+    implemented and raise.  key_padding_mask [batch, keys] (bool or float, functional.py:615-623 and :760-768) reaches
+    the kernels as a per-(batch, key) additive bias."""
 
     def __init__(self, embed_dim, num_heads, world_size, rank, dropout=0., bias=True, add_bias_kv=False,
                  add_zero_attn=False, kdim=None, vdim=None, batch_first=False, device=None, dtype=None,
@@ -286,9 +471,9 @@ class ParallelMultiheadAttention(RotatedLayer):
         self.embed_dim, self.num_heads = embed_dim, num_heads
         self.dropout, self.batch_first, self.has_bias = dropout, batch_first, bias
         if MultiheadAttention_layer is not None and device is None:
-            device = MultiheadAttention_layer.in_proj_weight.device
+            device = MultiheadAttention_layer.out_proj.weight.device
         if MultiheadAttention_layer is not None and dtype is None:
-            dtype = MultiheadAttention_layer.in_proj_weight.dtype
+            dtype = MultiheadAttention_layer.out_proj.weight.dtype
         layers = []
         for s in range(world_size):
             sub = SubParallelMultiheadAttention(embed_dim, num_heads, world_size, s, dropout, bias, add_bias_kv,
@@ -296,6 +481,9 @@ class ParallelMultiheadAttention(RotatedLayer):
             sub.affine_weight(MultiheadAttention_layer)
             layers.append(sub)
         self.head_dim = layers[0].head_dim
+        self.kdim, self.vdim = layers[0].kdim, layers[0].vdim
+        self.separate_proj = not layers[0]._qkv_same_embed_dim
+        self.add_zero_attn = bool(add_zero_attn)
         self.num_heads_per_partition = layers[0].num_heads_per_partition
         self.embed_dim_per_partition = layers[0].embed_dim_per_partition
         self._init_store(layers)
@@ -305,39 +493,62 @@ class ParallelMultiheadAttention(RotatedLayer):
     def forward(self, query: Tensor, key: Tensor, value: Tensor, key_padding_mask: Optional[Tensor] = None,
                 need_weights: bool = True, attn_mask: Optional[Tensor] = None, average_attn_weights: bool = True,
                 is_causal: bool = False, test_tensor=None, residual_grad: bool = False) -> Tuple[Tensor, Optional[Tensor]]:
-        if not (key is query and value is query):
-            if not (key.data_ptr() == query.data_ptr() == value.data_ptr() and key.shape == query.shape == value.shape
-                    and key.stride() == query.stride() == value.stride()):
-                raise NotImplementedError("rotated attention implements self-attention only (query is key is value)")
+        same = key is query and value is query
+        if not same:
+            same = (key.data_ptr() == query.data_ptr() == value.data_ptr() and key.shape == query.shape == value.shape
+                    and key.stride() == query.stride() == value.stride())
+        general = not same or self.separate_proj or self.add_zero_attn
         if self.dropout > 0.0 and self.training:
             raise NotImplementedError("rotated attention: attention dropout is not implemented (use dropout=0)")
-        if query.dim() != 3:
-            raise NotImplementedError("rotated attention expects a batched [L, N, E] (or batch_first) input")
+        if query.dim() != 3 or key.dim() != 3 or value.dim() != 3:
+            raise NotImplementedError("rotated attention expects batched [L, N, E] (or batch_first) inputs")
         x = query.transpose(0, 1) if self.batch_first else query
-        L = x.shape[0]
+        L, keys = x.shape[0], (key.shape[1] if self.batch_first else key.shape[0])
         mask = None
         causal = False
         if attn_mask is not None:
-            if attn_mask.dim() != 2 or tuple(attn_mask.shape) != (L, L):
-                raise NotImplementedError("rotated attention: only a 2-D [L, L] attn_mask is implemented")
+            if attn_mask.dim() != 2 or tuple(attn_mask.shape) != (L, keys):
+                raise NotImplementedError(f"rotated attention: only a 2-D [queries, keys] = {(L, keys)} attn_mask is "
+                                          f"implemented, got {tuple(attn_mask.shape)}")
             mask = F._canonical_mask(mask=attn_mask, mask_name="attn_mask", other_type=None, other_name="",
                                      target_type=torch.float32)
             mask = mask.to(device=x.device, dtype=torch.float32).contiguous()
         elif is_causal:
+            if general:
+                # functional.py:623-628
+                raise RuntimeError("Need attn_mask if specifying the is_causal hint.")
             causal = True
         key_bias = None
         if key_padding_mask is not None:
             # functional.py:615-623, :760-768: a bool mask hides the keys where it is True, a float mask is added to the
             # scores; merged into the attention mask per batch there, handed to the kernels as a [batch, key] bias here
-            if key_padding_mask.dim() != 2 or tuple(key_padding_mask.shape) != (x.shape[1], L):
-                raise ValueError(f"key_padding_mask must be [batch, keys] = {(x.shape[1], L)}, got "
+            if key_padding_mask.dim() != 2 or tuple(key_padding_mask.shape) != (x.shape[1], keys):
+                raise ValueError(f"key_padding_mask must be [batch, keys] = {(x.shape[1], keys)}, got "
                                  f"{tuple(key_padding_mask.shape)}")
             key_bias = F._canonical_mask(mask=key_padding_mask, mask_name="key_padding_mask",
                                          other_type=F._none_or_dtype(attn_mask), other_name="attn_mask",
                                          target_type=torch.float32)
             key_bias = key_bias.to(device=x.device, dtype=torch.float32).contiguous()
-        out, weights = _AttentionFn.apply(x, self._anchor, self, mask, causal, bool(need_weights), bool(residual_grad),
-                                          key_bias)
+        if general:
+            if residual_grad:
+                raise ValueError("residual_grad is for self-attention (the residual is the attention's own input)")
+            k_in, v_in = (key.transpose(0, 1), value.transpose(0, 1)) if self.batch_first else (key, value)
+            if k_in.shape[0] != v_in.shape[0] or k_in.shape[1] != x.shape[1] or v_in.shape[1] != x.shape[1] or \
+                    x.shape[2] != self.embed_dim or k_in.shape[2] != self.kdim or v_in.shape[2] != self.vdim:
+                raise ValueError(f"rotated attention: query {tuple(query.shape)}, key {tuple(key.shape)} and value "
+                                 f"{tuple(value.shape)} do not fit embed_dim / kdim / vdim = "
+                                 f"{(self.embed_dim, self.kdim, self.vdim)} and a common batch and key count")
+            if self.add_zero_attn:
+                # functional.py:746-753: the appended all-zero key is visible to every query
+                if mask is not None:
+                    mask = F.pad(mask, (0, 1))
+                if key_bias is not None:
+                    key_bias = F.pad(key_bias, (0, 1))
+            out, weights = _GeneralAttentionFn.apply(x, k_in, v_in, self._anchor, self, mask, key_bias,
+                                                     bool(need_weights))
+        else:
+            out, weights = _AttentionFn.apply(x, self._anchor, self, mask, causal, bool(need_weights),
+                                              bool(residual_grad), key_bias)
         if need_weights and weights is not None and average_attn_weights:
             weights = weights.float().mean(dim=1).to(out.dtype)
         if self.batch_first:

@@ -93,11 +93,11 @@ def test_attention_unsupported_raise():
     layer = ParallelMultiheadAttention(8, 2, 2, 0, device=DEV)
     x = torch.randn(4, 2, 8, device=DEV)
     with pytest.raises(NotImplementedError):
-        layer(x, x.clone(), x)
+        layer(x, x, x, attn_mask=torch.zeros(4, 4, 4, device=DEV))  # 3-D masks
     with pytest.raises(ValueError):
         layer(x, x, x, key_padding_mask=torch.zeros(3, 4, dtype=torch.bool, device=DEV))   # [batch, keys] = [2, 4]
     with pytest.raises(NotImplementedError):
-        ParallelMultiheadAttention(8, 2, 2, 0, kdim=4, device=DEV)
+        ParallelMultiheadAttention(8, 2, 2, 0, add_bias_kv=True, device=DEV)
 
 
 @pytest.mark.parametrize("E,H,L,N,ws,masked,need_weights", [

@@ -62,3 +62,34 @@ def test_wrapper_indivisible_linear_raises():
     from rtp_amd.rotated_tensor_parallel import RotatedTensorParallel
     with emulate_shards(4), pytest.raises(ValueError):
         RotatedTensorParallel(nn.Sequential(nn.Linear(6, 7)))
+
+
+def test_wrapper_on_stock_transformer_decoder_layer():
+    """torch.nn.TransformerDecoderLayer wrapped in place: its self-attention, its attention over the encoder memory
+    (keys and values from another tensor, with a key padding mask) and both feed-forward projections become rotated
+    layers; output and the gradients reaching both inputs must match the untouched copy."""
+    from rtp_amd import emulate_shards
+    from rtp_amd.rotated_tensor_parallel import RotatedTensorParallel
+    torch.manual_seed(0)
+    ref = nn.TransformerDecoderLayer(d_model=32, nhead=4, dim_feedforward=64, dropout=0.0)
+    with emulate_shards(4):
+        model = RotatedTensorParallel(copy.deepcopy(ref)).to(DEV)
+    kinds = sorted(type(w.rotated).__name__ for w in model.FlyweightModule_list)
+    assert kinds == ["ColumnParallelLinear", "ColumnParallelLinear", "ParallelMultiheadAttention",
+                     "ParallelMultiheadAttention"]
+    tgt, mem, g = torch.randn(6, 3, 32), torch.randn(9, 3, 32), torch.randn(6, 3, 32)
+    causal = torch.triu(torch.full((6, 6), float("-inf")), diagonal=1)
+    mem_pad = torch.zeros(3, 9, dtype=torch.bool)
+    mem_pad[1, 7:] = True
+    a, b = tgt.to(DEV).requires_grad_(), mem.to(DEV).requires_grad_()
+    out = model(a, b, tgt_mask=causal.to(DEV), memory_key_padding_mask=mem_pad.to(DEV))
+    out.backward(g.to(DEV))
+    ra, rb = tgt.clone().requires_grad_(), mem.clone().requires_grad_()
+    want = ref(ra, rb, tgt_mask=causal, memory_key_padding_mask=mem_pad)
+    want.backward(g)
+    assert_close(out, want, torch.float32, "output")
+    assert_close(a.grad, ra.grad, torch.float32, "target grad")
+    assert_close(b.grad, rb.grad, torch.float32, "memory grad")
+    m = model.module
+    assert_close(O.attention_grad_reinterleave([s.in_proj_weight.grad for s in m.multihead_attn.module_list], 4),
+                 ref.multihead_attn.in_proj_weight.grad, torch.float32, "memory attention in_proj")

@@ -34,6 +34,29 @@ def test_resolve_world_precedence(monkeypatch):
             pass
 
 
+def test_attention_with_own_key_and_value_widths_keeps_three_projection_blocks():
+    """kdim / vdim != embed_dim (rtp/module/attention.py:51-55, :81-84): q / k / v_proj_weight row blocks of shard s,
+    the packed bias re-interleaved as for the packed weight, and the rank state dict under the reference's names."""
+    from rtp_amd.checkpoint import rank_state_dict
+    mha = nn.MultiheadAttention(8, 4, kdim=6, vdim=10)
+    with torch.no_grad():
+        mha.in_proj_bias.copy_(torch.randn(24))
+    layer = attention.ParallelMultiheadAttention(8, 4, 2, 0, kdim=6, vdim=10, MultiheadAttention_layer=mha)
+    assert layer._store.names == ["q_proj_weight", "k_proj_weight", "v_proj_weight", "in_proj_bias", "out_proj.weight",
+                                  "out_proj.bias"]
+    for s, sub in enumerate(layer.layers):
+        rows = slice(4 * s, 4 * s + 4)
+        assert torch.equal(sub.q_proj_weight, mha.q_proj_weight[rows]) and sub.in_proj_weight is None
+        assert torch.equal(sub.k_proj_weight, mha.k_proj_weight[rows]) and sub.k_proj_weight.shape == (4, 6)
+        assert torch.equal(sub.v_proj_weight, mha.v_proj_weight[rows]) and sub.v_proj_weight.shape == (4, 10)
+        b = mha.in_proj_bias.detach().view(3, 2, 4)[:, s].reshape(-1)
+        assert torch.equal(sub.in_proj_bias, b)
+    holder = nn.Module()
+    holder.attn = layer
+    sd = rank_state_dict(holder, 1)
+    assert torch.equal(sd["attn.MultiheadAttention.k_proj_weight"], mha.k_proj_weight[4:8])
+
+
 def test_column_row_shard_layouts_match_oracle():
     master = nn.Linear(12, 8)
     with emulate_shards(4):
