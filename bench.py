@@ -132,7 +132,7 @@ def attainable_peaks(dev):
             "note": "same GEMM kernel / the shard-copy kernel, run alone on this GPU; copy counts bytes read + written"}
 
 
-def layer_workload(name, steps, warmup):
+def layer_workload(name, steps, warmup, graph=True):
     """The reference's other configurations (single rotated layers), fwd+bwd, timed with the same event
     bracketing; one JSON line with the layer's own algorithmic work and the dominant kernel's roofline."""
     import torch
@@ -216,12 +216,29 @@ def layer_workload(name, steps, warmup):
     else:
         raise SystemExit(f"unknown workload {name}")
 
-    for _ in range(max(warmup, 1)):
-        fn()
+    from rtp_amd import ring
+    # warm-up on a side stream, then the layer's forward + backward recorded once into a HIP graph and replayed
+    # (as for the language-model step); --no-graph times eager launches, CPU launch overhead included
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(max(warmup, 1)):
+            fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    ring.fence(dev)
+    run, launch_mode = fn, "eager (CPU launch overhead included)"
+    if graph:
+        cg = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(cg):
+            fn()
+        ring.fence(dev)
+        run, launch_mode = cg.replay, "HIP graph replay"
+        run()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
-        fn()
+        run()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / steps
     _lib.profile_enable(True)
@@ -244,7 +261,7 @@ def layer_workload(name, steps, warmup):
     out = {"metric": f"fwd+bwd time of one rotated layer ({name})", "value": dt * 1e3, "unit": "ms", "n_gpus": 1,
            "steps": steps, "warmup": warmup, "ms_per_step": dt * 1e3, "higher_is_better": False, "scaling": "weak",
            "vs_baseline": None, "dtype": work["dtype"], "data": "synthetic",
-           "config": {"workload": work["desc"], "launch_mode": "eager (CPU launch overhead included)"},
+           "config": {"workload": work["desc"], "launch_mode": launch_mode},
            "roofline": {"bound": work["bound"], "achieved": achieved, "peak": work["peak"], "unit": unit,
                         "frac": achieved / work["peak"], "traffic": None, "kernel": dom_name,
                         "avg_launch_us": avg_ms * 1e3},
@@ -280,7 +297,7 @@ def main():
         sys.exit(2)
 
     if args.workload != "lm":
-        layer_workload(args.workload, args.steps, args.warmup)
+        layer_workload(args.workload, args.steps, args.warmup, args.graph)
         return
 
     import torch
