@@ -93,6 +93,17 @@ def cpu_baseline(c, steps=2):
             f"({dt * 1e3:.0f} ms/step, os.cpu_count()={os.cpu_count()})"}
 
 
+def _time_cpu(one, steps):
+    """Median wall time of `one()` over `steps` calls after one warm-up call."""
+    one()
+    times = []
+    for _ in range(steps):
+        t0 = time.perf_counter()
+        one()
+        times.append(time.perf_counter() - t0)
+    return sorted(times)[len(times) // 2]
+
+
 def attainable_peaks(dev):
     """What this box's GPU actually delivers for the two kernel families the step is made of, measured here and now:
     a large bf16 product (4096^3, the same GEMM kernel, random operands) and a 1 GiB device-to-device copy (the
@@ -132,30 +143,45 @@ def attainable_peaks(dev):
             "note": "same GEMM kernel / the shard-copy kernel, run alone on this GPU; copy counts bytes read + written"}
 
 
-def layer_workload(name, steps, warmup, graph=True):
+def layer_workload(name, steps, warmup, graph=True, cpu=True):
     """The reference's other configurations (single rotated layers), fwd+bwd, timed with the same event
     bracketing; one JSON line with the layer's own algorithmic work and the dominant kernel's roofline."""
     import torch
     import torch.nn as nn
     from rtp_amd import _lib, emulate_shards
 
-    dev = torch.device("cuda", 0)
-    torch.cuda.set_device(dev)
     gen = torch.Generator().manual_seed(0)
 
     def uni(*shape):
         return torch.rand(*shape, generator=gen) * 0.2 - 0.1
 
-    if name == "linear":  # fp32 column-parallel Linear [1024,2048] x [2048,2048], 2 shards
-        from rtp_amd.module.linear import ColumnParallelLinear
+    ring_result = None
+    if name == "linear":
         master = nn.Linear(2048, 2048)
         with torch.no_grad():
             master.weight.copy_(uni(2048, 2048)), master.bias.zero_()
+        x_cpu, g_cpu = torch.randn(1024, 2048, generator=gen), torch.randn(1024, 2048, generator=gen)
+        if cpu:
+            # The reference's own execution of this configuration: two gloo ranks on the host cores, each with half
+            # of the batch rows and one home shard, the shards (and their gradients) travelling the ring.  The rank
+            # processes are started here, before this process has touched the GPU.
+            from oracle import gloo_ring
+            threads = max(1, torch.get_num_threads() // 2)
+            res = gloo_ring.column_linear_ring(x_cpu, master.weight.detach(), master.bias.detach(), g_cpu, ws=2,
+                                               steps=5, warmup=2, threads_per_rank=threads)
+            ring_result = (sorted(res["times"])[2], 2 * threads,
+                           "median of 5 fwd+bwd passes after 2 warm-ups, 2 gloo ranks on loopback")
+
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    if name == "linear":  # fp32 column-parallel Linear [1024,2048] x [2048,2048], 2 shards
+        from rtp_amd.module.linear import ColumnParallelLinear
         with emulate_shards(2):
             layer = ColumnParallelLinear(2048, 2048, linear_layer=master, device=dev, dtype=torch.float32)
-        x = torch.randn(1024, 2048, generator=gen).to(dev).requires_grad_()
-        g = torch.randn(1024, 2048, generator=gen).to(dev)
+        x = x_cpu.to(dev).requires_grad_()
+        g = g_cpu.to(dev)
         fn = lambda: layer(x).backward(g)
+        cpu_fn = lambda: ring_result
         work = {"flops": 3 * 2.0 * 1024 * 2048 * 2048, "bytes": None, "bound": "mfma", "peak": PEAK["fp32_mfma_tflops"],
                 "dtype": "f32", "desc": "column-parallel Linear fwd+bwd, X [1024,2048], W [2048,2048], 2 shards, fp32"}
     elif name == "embedding":  # table [10240,2048] fp32, 4 shards, ids [32,32]
@@ -164,9 +190,18 @@ def layer_workload(name, steps, warmup, graph=True):
         with torch.no_grad():
             master.weight.copy_(uni(10240, 2048))
         layer = ParallelEmbedding(10240, 2048, 4, 0, Embedding_layer=master, device=dev, dtype=torch.float32)
-        ids = torch.randint(0, 10240, (32, 32), generator=gen).to(dev)
-        g = torch.randn(32, 32, 2048, generator=gen).to(dev)
+        ids_cpu, g_cpu = torch.randint(0, 10240, (32, 32), generator=gen), torch.randn(32, 32, 2048, generator=gen)
+        ids, g = ids_cpu.to(dev), g_cpu.to(dev)
         fn = lambda: layer(ids).backward(g)
+
+        def cpu_fn():
+            from oracle import rtp_oracle as O
+            table = master.weight.detach().clone().requires_grad_()
+
+            def one():
+                table.grad = None
+                O.parallel_embedding(ids_cpu, table, 4).backward(g_cpu)
+            return _time_cpu(one, 5), torch.get_num_threads(), "median of 5 fwd+bwd passes after 1 warm-up"
         # gather 16 MiB + scatter-add <= 24 MiB of algorithmic traffic (the 80 MiB dense zero fill is not counted)
         work = {"flops": None, "bytes": (16 + 24) * 2.0 ** 20, "bound": "hbm", "peak": PEAK["hbm_gbs"], "dtype": "f32",
                 "desc": "vocab-sharded Embedding fwd+bwd, table [10240,2048] fp32 in 4 shards, ids [32,32]"}
@@ -178,9 +213,23 @@ def layer_workload(name, steps, warmup, graph=True):
                 p_.copy_(uni(*p_.shape))
         layer = ParallelMultiheadAttention(2048, 32, 8, 0, MultiheadAttention_layer=mha.to(torch.bfloat16), device=dev,
                                            dtype=torch.bfloat16)
-        x = torch.randn(512, 8, 2048, generator=gen).to(dev, torch.bfloat16).requires_grad_()
-        g = torch.randn(512, 8, 2048, generator=gen).to(dev, torch.bfloat16)
+        x_cpu, g_cpu = torch.randn(512, 8, 2048, generator=gen), torch.randn(512, 8, 2048, generator=gen)
+        x = x_cpu.to(dev, torch.bfloat16).requires_grad_()
+        g = g_cpu.to(dev, torch.bfloat16)
         fn = lambda: layer(x, x, x, is_causal=True, need_weights=False)[0].backward(g)
+
+        def cpu_fn():
+            from oracle import rtp_oracle as O
+            ps = [p_.detach().float().clone().requires_grad_() for p_ in
+                  (mha.in_proj_weight, mha.in_proj_bias, mha.out_proj.weight, mha.out_proj.bias)]
+            xc = x_cpu.clone().requires_grad_()
+            mask = torch.triu(torch.full((512, 512), float("-inf")), diagonal=1)
+
+            def one():
+                for t in ps + [xc]:
+                    t.grad = None
+                O.parallel_multihead_attention(xc, *ps, 32, 8, mask=mask)[0].backward(g_cpu)
+            return _time_cpu(one, 3), torch.get_num_threads(), "median of 3 fwd+bwd passes after 1 warm-up, fp32"
         proj = 2.0 * 4096 * 2048 * (6144 + 2048)
         core = 4.0 * 8 * 32 * 512 * 512 * 64
         work = {"flops": 3 * proj + 3.5 * core, "bytes": None, "bound": "mfma", "peak": PEAK["bf16_mfma_tflops"],
@@ -205,11 +254,26 @@ def layer_workload(name, steps, warmup, graph=True):
             local = nn.ModuleList([FeedForwardLayer_expert(2048, 8192, nn.ReLU(), 0.0)])
             layer = WeightMOELayer(gate, local, device=dev, dtype=torch.bfloat16,
                                    original_experts=[nn.ModuleList([m]) for m in masters])
-        x = torch.randn(8, 512, 2048, generator=gen).to(dev, torch.bfloat16).requires_grad_()
-        g = torch.randn(8, 512, 2048, generator=gen).to(dev, torch.bfloat16)
+        x_cpu, g_cpu = torch.randn(8, 512, 2048, generator=gen), torch.randn(8, 512, 2048, generator=gen)
+        x = x_cpu.to(dev, torch.bfloat16).requires_grad_()
+        g = g_cpu.to(dev, torch.bfloat16)
         u = torch.rand(4096, 8, generator=gen).clamp(min=torch.finfo(torch.float32).tiny, max=1 - torch.finfo(torch.float32).eps)
-        noise = (-torch.log(-torch.log(u))).to(dev)  # Gumbel(0,1) routing noise, drawn on the host
+        noise_cpu = -torch.log(-torch.log(u))  # Gumbel(0,1) routing noise, drawn on the host
+        noise = noise_cpu.to(dev)
         fn = lambda: (layer(x, noise=noise) * g).sum().backward()
+
+        def cpu_fn():
+            from oracle import rtp_oracle as O
+            wg = mg.wg.weight.detach().float().clone().requires_grad_()
+            experts = [tuple(p_.detach().float().clone().requires_grad_() for p_ in m.parameters()) for m in masters]
+            xc = x_cpu.clone().requires_grad_()
+
+            def one():
+                for t in [wg, xc] + [t for e in experts for t in e]:
+                    t.grad = None
+                (O.moe_layer(xc, wg, experts, noise_cpu, 8)[0] * g_cpu).sum().backward()
+            return _time_cpu(one, 1), torch.get_num_threads(), "1 fwd+bwd pass after 1 warm-up, fp32, the " \
+                "reference's dense dispatch / combine einsums"
         work = {"flops": 3 * 8192 * 2.0 * 2 * 2048 * 8192, "bytes": None, "bound": "mfma", "peak": PEAK["bf16_mfma_tflops"],
                 "dtype": "bf16", "desc": "expert-sharded MoE layer fwd+bwd, 8 experts, top-2, d_model 2048, d_ff 8192, "
                 "4096 tokens, bf16 (flops for 8192 routed pairs, i.e. nothing dropped)"}
@@ -267,6 +331,13 @@ def layer_workload(name, steps, warmup, graph=True):
                         "avg_launch_us": avg_ms * 1e3},
            "whole_layer": {"achieved": whole, "unit": unit, "frac": whole / work["peak"]},
            "kernels": kernels}
+    if cpu:
+        # the CPU restatement of the same layer on this box's host cores: a reported baseline, not a target
+        del layer
+        torch.cuda.empty_cache()
+        sec, cores, sample = cpu_fn()
+        out["cpu_baseline"] = {"value": sec * 1e3, "unit": "ms", "cores": cores, "kind": "port",
+                               "sample": f"{sample} (os.cpu_count()={os.cpu_count()})"}
     print(json.dumps(out))
 
 
@@ -297,7 +368,7 @@ def main():
         sys.exit(2)
 
     if args.workload != "lm":
-        layer_workload(args.workload, args.steps, args.warmup, args.graph)
+        layer_workload(args.workload, args.steps, args.warmup, args.graph, not args.no_cpu_baseline)
         return
 
     import torch

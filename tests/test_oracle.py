@@ -300,3 +300,25 @@ def test_conv_patches_layout_by_loops():
                             h, w = a * sh - ph + i * dh, b * sw - pw + j * dw
                             want = float(x[n, ci, h, w]) if 0 <= h < 4 and 0 <= w < 5 else 0.0
                             assert float(p[(n * ho + a) * wo + b, (ci * kh + i) * kw + j]) == want
+
+
+@pytest.mark.parametrize("ws", [2, 4])
+def test_gloo_ring_column_linear_equals_unsharded_linear(ws):
+    """The reference's actual execution (ws gloo ranks, shards travelling the ring with their gradients) restated in
+    oracle/gloo_ring.py gives torch.nn.functional.linear on the unsharded problem: outputs, input gradients and the
+    gathered weight / bias gradients (the comparison of the reference's tests/test_linear.py:134-165)."""
+    from oracle import gloo_ring
+    gen = torch.Generator().manual_seed(ws)
+    x, w, b = torch.randn(8 * ws, 12, generator=gen), torch.randn(4 * ws, 12, generator=gen), torch.randn(4 * ws, generator=gen)
+    dy = torch.randn(8 * ws, 4 * ws, generator=gen)
+    res = gloo_ring.column_linear_ring(x, w, b, dy, ws=ws, steps=2)
+    xr, wr, br = x.clone().requires_grad_(), w.clone().requires_grad_(), b.clone().requires_grad_()
+    y = torch.nn.functional.linear(xr, wr, br)
+    y.backward(dy)
+    torch.testing.assert_close(res["y"], y.detach())
+    torch.testing.assert_close(res["dx"], xr.grad)
+    torch.testing.assert_close(res["dw"], wr.grad)
+    torch.testing.assert_close(res["db"], br.grad)
+    assert len(res["times"]) == 2 and all(t > 0 for t in res["times"])
+    # and the one-process shard loop used by the device parity tests agrees with it
+    torch.testing.assert_close(O.column_parallel_linear(x, w, b, ws), res["y"])
