@@ -127,7 +127,7 @@ class _AttentionFn(torch.autograd.Function):
     kernel with p in memory."""
 
     @staticmethod
-    def forward(ctx, x, anchor, layer, mask, causal, want_weights, residual_grad=False, key_bias=None):
+    def forward(ctx, x, anchor, layer, mask, causal, want_weights, residual_grad=False, key_bias=None, drop_p=0.0):
         store = layer._store
         L, N, E = x.shape
         ws, h_s, d, e_s = layer.world_size, layer.num_heads_per_partition, layer.head_dim, layer.embed_dim_per_partition
@@ -141,12 +141,16 @@ class _AttentionFn(torch.autograd.Function):
         o = torch.empty(rows, E, dtype=dt, device=dev)
         out = torch.empty(rows, E, dtype=dt, device=dev)
         ldq = N * ws * 3 * e_s
-        fused = ops.attn_supported(dt, L, d)
-        flash = not fused and not want_weights and ops.attn_flash_supported(dt, L, d)
+        # attention dropout works on the probabilities in memory: the product + softmax form of the core
+        fused = drop_p == 0.0 and ops.attn_supported(dt, L, d)
+        flash = drop_p == 0.0 and not fused and not want_weights and ops.attn_flash_supported(dt, L, d)
         if flash:
             p = torch.empty(ws * Z, L, dtype=torch.float32, device=dev)  # log-sum-exp in place of probabilities
         else:
             p = torch.empty(ws * Z, L, L, dtype=dt, device=dev)
+        # drop: per-probability multiplier 0 or 1 / (1 - drop_p); pv: the probabilities that meet V
+        drop = torch.empty(ws * Z, L, L, dtype=torch.float32, device=dev) if drop_p > 0.0 else None
+        pv = torch.empty_like(p) if drop_p > 0.0 else p
         order = ring_order(layer.rank, ws)
         rot = Rotation(store.home, order, group=store.stage_group)
         acc = ops.ShardSum(out, sum(len(w) for w in rot.windows))
@@ -180,7 +184,10 @@ class _AttentionFn(torch.autograd.Function):
                 p_run = p[first * Z:(first + cnt) * Z]
                 ops.softmax_fwd(scores, p_run, mask=mask, causal=causal, scale=scale, key_bias=key_bias, heads=h_s)
                 del scores
-                _bmm(dt, a=p, a_off=first * Z * L * L, lda=L, a_kc=True, a_s=(h_s * L * L, L * L), a_sg=Z * L * L,
+                if drop is not None:
+                    _apply_dropout(layer, drop_p, p_run, drop[first * Z:(first + cnt) * Z],
+                                   pv[first * Z:(first + cnt) * Z])
+                _bmm(dt, a=pv, a_off=first * Z * L * L, lda=L, a_kc=True, a_s=(h_s * L * L, L * L), a_sg=Z * L * L,
                      b=qkv, b_off=q0 + 2 * e_s, ldb=ldq, b_kc=False, b_s=(ws * 3 * e_s, d), b_sg=3 * e_s, c=o,
                      c_off=first * e_s, ldc=N * E, c_s=(E, d), c_sg=e_s, m=L, n=d, k=L, batch=Z, zdiv=h_s, groups=cnt)
                 c_out, c_in = acc.target(i)
@@ -190,19 +197,22 @@ class _AttentionFn(torch.autograd.Function):
         weights = None
         if want_weights:
             last = order[-1]
-            weights = p[last * Z:(last + 1) * Z].view(N, h_s, L, L)
+            weights = pv[last * Z:(last + 1) * Z].view(N, h_s, L, L)  # functional.py:789-792: after dropout
         ctx.layer = layer
         ctx.dims = (L, N, E)
         ctx.residual_grad = residual_grad
         ctx.flash = (mask, causal, key_bias) if flash else None
-        ctx.save_for_backward(x2, qkv, p, o)
+        ctx.fused = fused
+        ctx.dropped = drop is not None
+        ctx.save_for_backward(x2, qkv, p, o, *((drop, pv) if drop is not None else ()))
         ctx.mark_non_differentiable(*([weights] if weights is not None else []))
         return out.view(L, N, E), weights
 
     @staticmethod
     def backward(ctx, dout, _dweights=None):
         layer = ctx.layer
-        x2, qkv, p, o = ctx.saved_tensors
+        x2, qkv, p, o = ctx.saved_tensors[:4]
+        drop, pv = ctx.saved_tensors[4:] if ctx.dropped else (None, p)
         store = layer._store
         L, N, E = ctx.dims
         ws, h_s, d, e_s = layer.world_size, layer.num_heads_per_partition, layer.head_dim, layer.embed_dim_per_partition
@@ -217,7 +227,7 @@ class _AttentionFn(torch.autograd.Function):
         do = torch.empty(rows, E, dtype=dt, device=dev)
         dqkv = torch.empty(rows, ws * 3 * e_s, dtype=dt, device=dev)
         ldq = N * ws * 3 * e_s
-        fused = ops.attn_supported(dt, L, d)
+        fused = ctx.fused
         delta = torch.empty_like(p) if ctx.flash is not None else None
         order = ring_order(layer.rank, ws, reverse=True)
         rot = Rotation(store.home, order, group=store.stage_group)
@@ -257,9 +267,11 @@ class _AttentionFn(torch.autograd.Function):
                      c_s=(h_s * L * L, L * L), c_sg=Z * L * L, m=L, n=L, k=d, batch=Z, zdiv=h_s, groups=cnt, out_f32=True)
                 p_off = first * Z * L * L
                 # dV = P^T dO
-                _bmm(dt, a=p, a_off=p_off, lda=L, a_kc=False, a_s=(h_s * L * L, L * L), a_sg=Z * L * L, b=do,
+                _bmm(dt, a=pv, a_off=p_off, lda=L, a_kc=False, a_s=(h_s * L * L, L * L), a_sg=Z * L * L, b=do,
                      b_off=first * e_s, ldb=N * E, b_kc=False, b_s=(E, d), b_sg=e_s, c=dqkv, c_off=q0 + 2 * e_s, ldc=ldq,
                      c_s=(ws * 3 * e_s, d), c_sg=3 * e_s, m=L, n=d, k=L, batch=Z, zdiv=h_s, groups=cnt)
+                if drop is not None:
+                    dp.mul_(drop[first * Z:(first + cnt) * Z])
                 ds = torch.empty(cnt * Z, L, L, dtype=dt, device=dev)
                 ops.softmax_bwd(p[first * Z:(first + cnt) * Z], dp, ds, scale)
                 del dp
@@ -288,7 +300,25 @@ class _AttentionFn(torch.autograd.Function):
             store.grads_ready()
 
         run_wgrad(dev, param_grads, (dout2, o, dqkv, x2))
-        return (dx.view(L, N, E) if need_dx else None), None, None, None, None, None, None, None
+        return (dx.view(L, N, E) if need_dx else None), None, None, None, None, None, None, None, None
+
+
+def _apply_dropout(layer, drop_p: float, p: Tensor, drop: Tensor, out: Tensor) -> None:
+    """Attention dropout (functional.py:789-792 / the dropout_p of :825): every probability is kept with chance
+    1 - drop_p and scaled by 1 / (1 - drop_p).  `drop` receives the fp32 multipliers (0 or 1 / (1 - drop_p)) for the
+    backward pass, `out` the probabilities that meet V.  The draw itself is torch's device generator (an ordinary
+    torch op, like the model's other dropouts); `layer.dropout_keep_fn`, if set, supplies the 0 / 1 keep mask instead."""
+    keep = 1.0 - drop_p
+    fn = getattr(layer, "dropout_keep_fn", None)
+    if fn is not None:
+        drop.copy_(fn(tuple(drop.shape)))
+    else:
+        drop.bernoulli_(keep)
+    drop.div_(keep)
+    if out.dtype == torch.float32:
+        torch.mul(p, drop, out=out)
+    else:
+        out.copy_(p.float().mul_(drop))
 
 
 def _shard_layout(layer):
@@ -312,7 +342,7 @@ class _GeneralAttentionFn(torch.autograd.Function):
     the softmax kernel with p [ws*N*h_s, L, S+z] in memory."""
 
     @staticmethod
-    def forward(ctx, query, key, value, anchor, layer, mask, key_bias, want_weights):
+    def forward(ctx, query, key, value, anchor, layer, mask, key_bias, want_weights, drop_p=0.0):
         store = layer._store
         L, N, E = query.shape
         s_in = key.shape[0]
@@ -334,6 +364,8 @@ class _GeneralAttentionFn(torch.autograd.Function):
         o = torch.empty(L * N, E, dtype=dt, device=dev)
         out = torch.empty(L * N, E, dtype=dt, device=dev)
         p = torch.empty(ws * Z, L, sk, dtype=dt, device=dev)
+        drop = torch.empty(ws * Z, L, sk, dtype=torch.float32, device=dev) if drop_p > 0.0 else None
+        pv = torch.empty_like(p) if drop_p > 0.0 else p
         ld = N * E  # one step along the sequence in q, k, v and o
         order = ring_order(layer.rank, ws)
         rot = Rotation(store.home, order, group=store.stage_group)
@@ -352,7 +384,10 @@ class _GeneralAttentionFn(torch.autograd.Function):
                 ops.softmax_fwd(scores, p[first * Z:(first + cnt) * Z], mask=mask, causal=False, scale=scale,
                                 key_bias=key_bias, heads=h_s)
                 del scores
-                _bmm(dt, a=p, a_off=first * Z * L * sk, lda=sk, a_kc=True, a_s=(h_s * L * sk, L * sk),
+                if drop is not None:
+                    _apply_dropout(layer, drop_p, p[first * Z:(first + cnt) * Z], drop[first * Z:(first + cnt) * Z],
+                                   pv[first * Z:(first + cnt) * Z])
+                _bmm(dt, a=pv, a_off=first * Z * L * sk, lda=sk, a_kc=True, a_s=(h_s * L * sk, L * sk),
                      a_sg=Z * L * sk, b=vb, b_off=c0, ldb=ld, b_kc=False, b_s=(E, d), b_sg=e_s, c=o, c_off=c0, ldc=ld,
                      c_s=(E, d), c_sg=e_s, m=L, n=d, k=sk, batch=Z, zdiv=h_s, groups=cnt)
                 c_out, c_in = acc.target(i)
@@ -362,17 +397,19 @@ class _GeneralAttentionFn(torch.autograd.Function):
         weights = None
         if want_weights:
             last = order[-1]
-            weights = p[last * Z:(last + 1) * Z].view(N, h_s, L, sk)
+            weights = pv[last * Z:(last + 1) * Z].view(N, h_s, L, sk)
         ctx.layer = layer
         ctx.dims = (L, N, E, s_in, sk)
-        ctx.save_for_backward(q2, k2, v2, qb, kb, vb, p, o)
+        ctx.dropped = drop is not None
+        ctx.save_for_backward(q2, k2, v2, qb, kb, vb, p, o, *((drop, pv) if drop is not None else ()))
         ctx.mark_non_differentiable(*([weights] if weights is not None else []))
         return out.view(L, N, E), weights
 
     @staticmethod
     def backward(ctx, dout, _dweights=None):
         layer = ctx.layer
-        q2, k2, v2, qb, kb, vb, p, o = ctx.saved_tensors
+        q2, k2, v2, qb, kb, vb, p, o = ctx.saved_tensors[:8]
+        drop, pv = ctx.saved_tensors[8:] if ctx.dropped else (None, p)
         store = layer._store
         L, N, E, s_in, sk = ctx.dims
         ws, h_s, d, e_s = layer.world_size, layer.num_heads_per_partition, layer.head_dim, layer.embed_dim_per_partition
@@ -414,9 +451,11 @@ class _GeneralAttentionFn(torch.autograd.Function):
                      b_s=(E, d), b_sg=e_s, c=dp, c_off=0, ldc=sk, c_s=p_s, c_sg=p_sg, m=L, n=sk, k=d, batch=Z,
                      zdiv=h_s, groups=cnt, out_f32=True)
                 # dV = P^T dO
-                _bmm(dt, a=p, a_off=p_off, lda=sk, a_kc=False, a_s=p_s, a_sg=p_sg, b=do, b_off=c0, ldb=ld, b_kc=False,
+                _bmm(dt, a=pv, a_off=p_off, lda=sk, a_kc=False, a_s=p_s, a_sg=p_sg, b=do, b_off=c0, ldb=ld, b_kc=False,
                      b_s=(E, d), b_sg=e_s, c=dvb, c_off=c0, ldc=ld, c_s=(E, d), c_sg=e_s, m=sk, n=d, k=L, batch=Z,
                      zdiv=h_s, groups=cnt)
+                if drop is not None:
+                    dp.mul_(drop[first * Z:(first + cnt) * Z])
                 ds = torch.empty(cnt * Z, L, sk, dtype=dt, device=dev)
                 ops.softmax_bwd(p[first * Z:(first + cnt) * Z], dp, ds, scale)
                 del dp
@@ -452,15 +491,15 @@ class _GeneralAttentionFn(torch.autograd.Function):
         dq = None if grads[0] is None else grads[0].view(L, N, E)
         dk = None if grads[1] is None else grads[1].view(s_in, N, layer.kdim)
         dv = None if grads[2] is None else grads[2].view(s_in, N, layer.vdim)
-        return dq, dk, dv, None, None, None, None, None
+        return dq, dk, dv, None, None, None, None, None, None
 
 
 class ParallelMultiheadAttention(RotatedLayer):
     """Signature follows rtp/module/attention.py:192-193; `MultiheadAttention_layer` imports the weights
     of an unsharded nn.MultiheadAttention.  Self-attention (query, key and value the same tensor) takes the packed
     projection and the fused cores; keys / values from other tensors, kdim / vdim != embed_dim and add_zero_attn take
-    three projections and the product + softmax core.  3-D masks, add_bias_kv and attention dropout are not
-    implemented and raise.  key_padding_mask [batch, keys] (bool or float, functional.py:615-623 and :760-768) reaches
+    three projections and the product + softmax core, and so does attention dropout while training (the probabilities
+    are dropped in memory).  3-D masks and add_bias_kv are not implemented and raise.  key_padding_mask [batch, keys] (bool or float, functional.py:615-623 and :760-768) reaches
     the kernels as a per-(batch, key) additive bias."""
 
     def __init__(self, embed_dim, num_heads, world_size, rank, dropout=0., bias=True, add_bias_kv=False,
@@ -498,8 +537,9 @@ class ParallelMultiheadAttention(RotatedLayer):
             same = (key.data_ptr() == query.data_ptr() == value.data_ptr() and key.shape == query.shape == value.shape
                     and key.stride() == query.stride() == value.stride())
         general = not same or self.separate_proj or self.add_zero_attn
-        if self.dropout > 0.0 and self.training:
-            raise NotImplementedError("rotated attention: attention dropout is not implemented (use dropout=0)")
+        drop_p = float(self.dropout) if self.training else 0.0
+        if not 0.0 <= drop_p < 1.0:
+            raise ValueError(f"attention dropout probability has to be in [0, 1), got {drop_p}")
         if query.dim() != 3 or key.dim() != 3 or value.dim() != 3:
             raise NotImplementedError("rotated attention expects batched [L, N, E] (or batch_first) inputs")
         x = query.transpose(0, 1) if self.batch_first else query
@@ -545,10 +585,10 @@ class ParallelMultiheadAttention(RotatedLayer):
                 if key_bias is not None:
                     key_bias = F.pad(key_bias, (0, 1))
             out, weights = _GeneralAttentionFn.apply(x, k_in, v_in, self._anchor, self, mask, key_bias,
-                                                     bool(need_weights))
+                                                     bool(need_weights), drop_p)
         else:
             out, weights = _AttentionFn.apply(x, self._anchor, self, mask, causal, bool(need_weights),
-                                              bool(residual_grad), key_bias)
+                                              bool(residual_grad), key_bias, drop_p)
         if need_weights and weights is not None and average_attn_weights:
             weights = weights.float().mean(dim=1).to(out.dtype)
         if self.batch_first:

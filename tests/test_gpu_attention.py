@@ -311,3 +311,110 @@ def test_attention_key_padding_mask(E, H, L, N, ws, dtype, masked, need_weights)
         out_f, _ = layer(xf, xf, xf, attn_mask=None if mask is None else mask.to(DEV), need_weights=need_weights,
                          key_padding_mask=torch.zeros(N, L).masked_fill(kpm, float("-inf")).to(DEV))
     assert torch.equal(out_f, out.detach())
+
+
+def _attention_with_keep_masks(x, mha, H, ws, keep, drop_p, mask):
+    """Per-shard attention (functional.py:779-800) with the given 0 / 1 keep mask [ws * N * H/ws, L, L] applied to the
+    softmax probabilities and scaled by 1 / (1 - drop_p), on the CPU with autograd."""
+    import math
+    import torch.nn.functional as F
+    L, N, E = x.shape
+    h_s, e_s = H // ws, E // ws
+    d = E // H
+    Z = N * h_s
+    out = 0
+    for g in range(ws):
+        w_in, b_in, w_o, b_o = O.attention_shard_params(mha.in_proj_weight, mha.in_proj_bias, mha.out_proj.weight,
+                                                         mha.out_proj.bias, ws, g)
+        q, k, v = F.linear(x, w_in, b_in).split(e_s, dim=-1)
+        q, k, v = (t.reshape(L, Z, d).transpose(0, 1) for t in (q, k, v))
+        s = torch.bmm(q / math.sqrt(d), k.transpose(1, 2))
+        p = torch.softmax(s if mask is None else s + mask, dim=-1) * keep[g * Z:(g + 1) * Z] / (1.0 - drop_p)
+        o = torch.bmm(p, v).transpose(0, 1).reshape(L * N, e_s)
+        out = out + F.linear(o, w_o, b_o).view(L, N, E)
+    return out
+
+
+@pytest.mark.parametrize("ws", [1, 2, 4])
+def test_attention_dropout_with_recorded_masks(ws):
+    """Attention dropout while training: the layer draws keep masks (recorded here through dropout_keep_fn), the CPU
+    restatement applies the same masks; output and every gradient must agree.  eval() switches dropout off."""
+    from rtp_amd.module.attention import ParallelMultiheadAttention
+    E, H, L, N, drop_p = 32, 4, 6, 3, 0.3
+    gen = torch.Generator().manual_seed(11)
+    mha = _master(E, H, torch.float32, gen)
+    layer = ParallelMultiheadAttention(E, H, ws, 0, dropout=drop_p, MultiheadAttention_layer=mha, device=DEV)
+    drawn = []
+    mask_gen = torch.Generator().manual_seed(12)
+
+    def keep_fn(shape):
+        m = (torch.rand(shape, generator=mask_gen) >= drop_p).float()
+        drawn.append(m)
+        return m.to(DEV)
+    layer.dropout_keep_fn = keep_fn
+    x = torch.randn(L, N, E, generator=gen)
+    g = torch.randn(L, N, E, generator=gen)
+    xd = x.to(DEV).requires_grad_()
+    out, w = layer(xd, xd, xd, attn_mask=_causal(L).to(DEV), need_weights=True, average_attn_weights=False)
+    out.backward(g.to(DEV))
+    keep = torch.cat(drawn, 0)  # ring order of home rank 0 = ascending shard index
+    assert keep.shape == (N * H, L, L)
+    xo = x.clone().requires_grad_()
+    want = _attention_with_keep_masks(xo, mha, H, ws, keep, drop_p, _causal(L))
+    want.backward(g)
+    assert_close(out, want, torch.float32, "output")
+    assert_close(xd.grad, xo.grad, torch.float32, "input grad")
+    assert_close(O.attention_grad_reinterleave([l.in_proj_weight.grad for l in layer.layers], ws),
+                 mha.in_proj_weight.grad, torch.float32, "in_proj_weight grad")
+    assert_close(torch.cat([l.out_proj.weight.grad for l in layer.layers], dim=1), mha.out_proj.weight.grad,
+                 torch.float32, "out_proj.weight grad")
+    # the returned weights are the dropped ones of the last shard visited (functional.py:789-800)
+    h_s = H // ws
+    zero_where_dropped = w.cpu()[keep[(ws - 1) * N * h_s:].view(N, h_s, L, L) == 0]
+    assert torch.count_nonzero(zero_where_dropped) == 0
+    # without the hook the device generator draws: about drop_p of the visible probabilities become zero
+    layer.dropout_keep_fn = None
+    _, w2 = layer(xd, xd, xd, need_weights=True, average_attn_weights=False)
+    frac = float((w2 == 0).float().mean())
+    assert 0.15 < frac < 0.45, frac
+    layer.eval()
+    a, _ = layer(xd, xd, xd, attn_mask=_causal(L).to(DEV), need_weights=False)
+    ref, _ = mha(x, x, x, attn_mask=_causal(L), need_weights=False)
+    assert_close(a, ref, torch.float32, "eval output")
+
+
+def test_attention_dropout_bf16_and_other_key_tensor():
+    """bf16, and keys / values from another tensor: with an all-ones keep mask the probabilities are only scaled by
+    1 / (1 - p), so (out - b_o) is the dropout-free result divided by (1 - p)."""
+    from rtp_amd.module.attention import ParallelMultiheadAttention
+    E, H, drop_p = 64, 4, 0.25
+    gen = torch.Generator().manual_seed(13)
+    mha = _master(E, H, torch.bfloat16, gen)
+    layer = ParallelMultiheadAttention(E, H, 2, 0, dropout=drop_p, MultiheadAttention_layer=mha, device=DEV,
+                                       dtype=torch.bfloat16)
+    layer.dropout_keep_fn = lambda shape: torch.ones(shape, device=DEV)
+    q = torch.randn(9, 2, E, generator=gen).to(torch.bfloat16)
+    k = torch.randn(14, 2, E, generator=gen).to(torch.bfloat16)
+    ref_m = nn.MultiheadAttention(E, H)
+    ref_m.load_state_dict({n: v.float() for n, v in mha.state_dict().items()})
+    for key in (q, k):
+        out, _ = layer(q.to(DEV), key.to(DEV), key.to(DEV), need_weights=False)
+        ref, _ = ref_m(q.float(), key.float(), key.float(), need_weights=False)
+        b_o = ref_m.out_proj.bias.detach()
+        assert_close(out.float().cpu() - b_o, (ref.detach() - b_o) / (1 - drop_p), torch.bfloat16, "scaled output")
+
+
+def test_lm_trains_with_dropout():
+    """The language model with the reference's default dropout 0.1 (transformer_lm_rtp.py:128, :139 hands it to the
+    attention as well): a training step runs and the loss is finite; eval() is deterministic."""
+    import torch.nn.functional as F
+    from rtp_amd.models.transformer_lm_rtp import TransformerLM
+    torch.manual_seed(0)
+    lm = TransformerLM(64, 32, 4, 32, 0.1, 0.1, 2, 2, 0, device=DEV)
+    ids = torch.randint(0, 64, (10, 3), device=DEV)
+    loss = F.cross_entropy(lm(ids).view(-1, 64), ids.view(-1))
+    loss.backward()
+    assert torch.isfinite(loss)
+    assert all(torch.isfinite(p.grad).all() for p in lm.parameters() if p.grad is not None)
+    lm.eval()
+    assert torch.equal(lm(ids), lm(ids))
