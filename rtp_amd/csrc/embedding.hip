@@ -22,7 +22,25 @@ __global__ __launch_bounds__(256) void gather_kernel(const T* table, long ld_tab
   T* dst = out + blockIdx.z * out_sg + t * ld_out;
   constexpr int VEC = 16 / sizeof(T);
   if (pos) {
-    const T* prow = pos + (t / batch) * ld_pos + blockIdx.z * pos_sg;
+    const T* prow = pos + (long)((unsigned)t / (unsigned)batch) * ld_pos + blockIdx.z * pos_sg;
+    if (vec) {
+      const long nvec = cols / VEC;
+      union Pack {
+        uint4 u;
+        T e[VEC];
+      };
+      for (long i = (long)blockIdx.y * 256 + threadIdx.x; i < nvec; i += (long)gridDim.y * 256) {
+#pragma clang fp contract(off)
+        Pack a, b, r;
+        a.u = reinterpret_cast<const uint4*>(src)[i];
+        b.u = reinterpret_cast<const uint4*>(prow)[i];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e)
+          r.e[e] = from_f32<T>(to_f32(from_f32<T>(to_f32(a.e[e]) * scale)) + to_f32(b.e[e]));
+        reinterpret_cast<uint4*>(dst)[i] = r.u;
+      }
+      return;
+    }
     for (long i = (long)blockIdx.y * 256 + threadIdx.x; i < cols; i += (long)gridDim.y * 256) {
 #pragma clang fp contract(off)
       const float a = to_f32(from_f32<T>(to_f32(src[i]) * scale));
@@ -138,7 +156,8 @@ static int gather_impl(void* stream, int dtype, const void* table, int64_t ld_ta
   RTP_REQUIRE(dtype == RTP_F32 || dtype == RTP_BF16, "rtp_embedding_gather: unknown dtype %d", dtype);
   const int vec = ((uintptr_t)table % 16 == 0) && ((uintptr_t)out % 16 == 0) && (ld_table * esz) % 16 == 0 &&
                   (ld_out * esz) % 16 == 0 && (cols * esz) % 16 == 0 && (table_sg * esz) % 16 == 0 &&
-                  (out_sg * esz) % 16 == 0;
+                  (out_sg * esz) % 16 == 0 &&
+                  (!pos || ((uintptr_t)pos % 16 == 0 && (ld_pos * esz) % 16 == 0 && (pos_sg * esz) % 16 == 0));
   const unsigned chunks = (unsigned)std::min<int64_t>(16, std::max<int64_t>(1, ceil_div(cols * (int64_t)esz, 4096)));
   dim3 grid((unsigned)n_ids, chunks, (unsigned)groups);
   hipStream_t s = (hipStream_t)stream;
@@ -169,7 +188,8 @@ extern "C" int rtp_embedding_gather_scale_pos(void* stream, int dtype, const voi
                                               int64_t n_ids, void* out, int64_t ld_out, int64_t groups,
                                               int64_t table_sg, int64_t out_sg, float scale, const void* pos,
                                               int64_t ld_pos, int64_t pos_sg, int64_t batch) {
-  RTP_REQUIRE(pos && batch >= 1 && ld_pos >= cols, "rtp_embedding_gather_scale_pos: need a positional table and batch >= 1");
+  RTP_REQUIRE(pos && batch >= 1 && batch < (1ll << 31) && ld_pos >= cols,
+              "rtp_embedding_gather_scale_pos: need a positional table and 1 <= batch < 2^31");
   return gather_impl(stream, dtype, table, ld_table, row_begin, row_count, cols, ids, n_ids, out, ld_out, groups,
                      table_sg, out_sg, scale, pos, ld_pos, pos_sg, batch);
 }
