@@ -219,3 +219,14 @@ def test_rank_state_dicts_follow_the_reference_layout_and_round_trip():
         load_rank_state_dicts(other, saved)
     with pytest.raises(ValueError):
         rank_state_dict(net, 4)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asking for more exits with a message instead of a number."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                         timeout=120)
+    assert res.returncode == 2 and "one GPU" in res.stderr and res.stdout.strip() == ""
