@@ -15,12 +15,14 @@ class _DeferredParamGrads:
     """LayerNorm parameter gradients whose reduction waits for the end of the backward pass: each layer's backward
     leaves per-block partial sums in a buffer of its own, and ONE launch reduces all of them when autograd is done
     (nobody reads a parameter gradient earlier).  Only for gradients that go straight into an optimiser's persistent
-    slices; the device table is rebuilt only when a buffer moved."""
+    slices.  The device table of one set of buffers is built once and kept for good: a captured graph holds its
+    address, and another model's backward pass must neither replace it nor force a host-to-device copy into a
+    capture (the first, eager, step of a model builds its table)."""
 
     def __init__(self):
         self.pending = {}   # device index -> [(part, rows, cols, dgamma, dbeta, weight)]
         self.armed = set()  # device indices with a callback queued in the running backward pass
-        self.tables = {}    # (device index, dtype) -> (key, table, max_cols)
+        self.tables = {}    # (device index, dtype, buffer addresses and shapes) -> (table, max_cols)
 
     def add(self, device: torch.device, item) -> bool:
         idx = device.index if device.index is not None else torch.cuda.current_device()
@@ -47,12 +49,12 @@ class _DeferredParamGrads:
         for dtype, group in by_dtype.items():
             key = tuple((it[0].data_ptr(), it[1], it[2], it[3].data_ptr(), it[4].data_ptr() if it[4] is not None else 0)
                         for it in group)
-            cached = self.tables.get((idx, dtype))
-            if cached is None or cached[0] != key:
-                cached = (key, ops.layernorm_final_table([it[:5] for it in group], group[0][0].device),
+            cached = self.tables.get((idx, dtype, key))
+            if cached is None:
+                cached = (ops.layernorm_final_table([it[:5] for it in group], group[0][0].device),
                           max(it[2] for it in group))
-                self.tables[(idx, dtype)] = cached
-            ops.layernorm_finalize(cached[1], dtype, cached[2])
+                self.tables[(idx, dtype, key)] = cached
+            ops.layernorm_finalize(cached[0], dtype, cached[1])
 
 
 _deferred = _DeferredParamGrads()
