@@ -124,12 +124,17 @@ class DeviceRing:
         self.next_slot = 0
         self.epoch = 0
         self.holder: List[Optional["StageGroup"]] = [None, None]
+        self.retired: List[torch.Tensor] = []
 
     def reserve(self, nbytes: int) -> None:
         if nbytes <= self.slot_bytes:
             return
         # Work queued on the side stream may still read the old slots.
         torch.cuda.synchronize(self.device)
+        if self.staging is not None:
+            # a graph captured earlier holds addresses inside the old slots and may be replayed again: the memory
+            # stays allocated (and nobody else's) for the life of the process
+            self.retired.append(self.staging)
         self.slot_bytes = (nbytes + _SLOT_ALIGN - 1) // _SLOT_ALIGN * _SLOT_ALIGN
         self.staging = torch.empty(2 * self.slot_bytes, dtype=torch.uint8, device=self.device)
         self.fence()
