@@ -26,8 +26,8 @@ PEAK = {"bf16_mfma_tflops": 2500.0, "fp32_mfma_tflops": 157.3, "hbm_gbs": 8000.0
 # FETCH_SIZE * 1.9927 + WRITE_SIZE * 1.0000 from two rocprofv3 --pmc runs of this script; the factors are what the same
 # counters read for the library's plain copy kernel on a copy of known size (profiles/lm_step_pmc_fetch_write.txt).
 MEASURED_TRAFFIC_KIB = {
-    "gemm_bf16_128x128_rc_rc": 46071.0, "gemm_bf16_128x64_kc_rc": 59047.4, "gemm_bf16_128x64_kc_kc": 36974.4,
-    "gemm_bf16_128x192_kc_kc": 74867.5,
+    "gemm_bf16_128x128_rc_rc": 45809.5, "gemm_bf16_128x64_kc_rc": 59047.3, "gemm_bf16_128x64_kc_kc": 36974.4,
+    "gemm_bf16_128x192_kc_kc": 74863.4,
 }
 
 
