@@ -93,6 +93,30 @@ def test_lm_headline_config_full_size_bf16():
     assert float(after) < float(loss.detach())
 
 
+def test_lm_headline_config_graph_replays_equal_eager_steps():
+    """The benchmark's measurement mode at the benchmark's size: the 10-layer bf16 step recorded into a HIP graph
+    (weight gradients on their second stream, as bench.py runs it) and replayed with new token ids stays
+    bit-identical, weights and loss, to a twin model that takes the same steps eagerly."""
+    from test_gpu_lm import graph_replays_against_eager_twin
+    from rtp_amd import ring
+    from rtp_amd.models.transformer_lm_rtp import TransformerLM
+    V, D, H, Fd, n_dec, L, N, ws = 10240, 2048, 32, 2048, 10, 32, 32, 8
+    twins = []
+    for _ in range(2):
+        torch.manual_seed(21)
+        twins.append(TransformerLM(V, D, H, Fd, 0.0, 0.1, n_dec, ws, 0, device=DEV, dtype=torch.bfloat16))
+    with torch.no_grad():
+        for pa, pb in zip(twins[0].parameters(), twins[1].parameters()):
+            pb.copy_(pa)
+    before = ring.wgrad_overlap()
+    ring.set_wgrad_overlap(True)
+    try:
+        loss = graph_replays_against_eager_twin(twins, V, L, N, replays=3, lr=1e-3)
+    finally:
+        ring.set_wgrad_overlap(before)
+    assert 0.0 < loss < 20.0
+
+
 def _moe_config5(dtype, seed=31):
     from test_gpu_moe import _moe_from_tensors
     gen = torch.Generator().manual_seed(seed)

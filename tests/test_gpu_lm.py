@@ -281,66 +281,72 @@ def test_lm_embedding_scale_and_positions_on_the_gather_are_bit_identical(dtype,
         assert torch.equal(g, results[1][1][k]), k
 
 
-@pytest.mark.parametrize("overlap", [False, True])
-def test_lm_step_replayed_from_a_graph_matches_eager_steps(overlap):
-    """The whole training step (zero grads, forward, cross-entropy, backward on both streams, clip + SGD, the rotation
-    copies on their side stream) recorded once into a HIP graph, as the benchmark times it: every replay, with new
-    token ids, eager work and synchronisation in between, must leave exactly the weights and the loss that a twin
-    model reaches by taking the same steps eagerly."""
+def graph_replays_against_eager_twin(twin_lms, V, L, N, replays, lr=1e-2):
+    """Record one whole training step of twin_lms[0] into a HIP graph and replay it `replays` times with new token ids,
+    eager work and synchronisation in between; twin_lms[1] (same weights) takes the same steps eagerly.  Losses and
+    all weights must stay bit-identical."""
     from rtp_amd import ring
     from rtp_amd.module.loss import cross_entropy
     from rtp_amd.optim import RotatedSGD
+    twins = [(lm, RotatedSGD(lm, lr=lr, clip_value=0.05)) for lm in twin_lms]
+    gen = torch.Generator().manual_seed(5)
+    ids = torch.randint(0, V, (L, N), generator=gen).to(DEV)
+    tgt = torch.randint(0, V, (L, N), generator=gen).to(DEV)
+    losses = [None, None]
+
+    def step(i):
+        lm, opt = twins[i]
+        opt.zero_grad()
+        loss = cross_entropy(lm(ids).view(-1, V), tgt.view(-1))
+        loss.backward()
+        opt.step()
+        losses[i] = loss.detach()
+
+    def same_state(what):
+        assert torch.equal(losses[0], losses[1]), what
+        for (na, pa), (_, pb) in zip(twins[0][0].named_parameters(), twins[1][0].named_parameters()):
+            assert torch.equal(pa, pb), f"{what}: {na}"
+
+    # both twins take their first step eagerly on a side stream (gradient accumulators are created there)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(0)
+        step(1)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    ring.fence(DEV)
+    same_state("first eager step")
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(0)
+    ring.fence(DEV)
+    # the capture recorded the step without running it: twin 0 is still one step behind until the first replay
+    for r in range(replays):
+        if r:
+            ids.copy_(torch.randint(0, V, (L, N), generator=gen))
+            tgt.copy_(torch.randint(0, V, (L, N), generator=gen))
+        graph.replay()
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            step(1)
+        torch.cuda.synchronize()
+        same_state(f"replay {r}")
+        _ = (twins[0][0][2].norm1.weight.float() * 2).sum().item()  # unrelated eager work between replays
+    return float(losses[0])
+
+
+@pytest.mark.parametrize("overlap", [False, True])
+def test_lm_step_replayed_from_a_graph_matches_eager_steps(overlap):
+    """The whole training step (zero grads, forward, cross-entropy, backward on both streams, clip + SGD, the rotation
+    copies on their side stream) recorded once into a HIP graph, as the benchmark times it: every replay must leave
+    exactly the weights and the loss that a twin model reaches by taking the same steps eagerly."""
+    from rtp_amd import ring
     V, D, H, Fd, n_dec, L, N, ws = 96, 64, 4, 64, 2, 12, 5, 4
     before = ring.wgrad_overlap()
     ring.set_wgrad_overlap(overlap)
     try:
-        twins = []
-        for _ in range(2):
-            lm, _ = build_pair(V, D, H, Fd, n_dec, ws, torch.bfloat16)
-            twins.append((lm, RotatedSGD(lm, lr=1e-2, clip_value=0.05)))
-        gen = torch.Generator().manual_seed(5)
-        ids = torch.randint(0, V, (L, N), generator=gen).to(DEV)
-        tgt = torch.randint(0, V, (L, N), generator=gen).to(DEV)
-        losses = [None, None]
-
-        def step(i):
-            lm, opt = twins[i]
-            opt.zero_grad()
-            loss = cross_entropy(lm(ids).view(-1, V), tgt.view(-1))
-            loss.backward()
-            opt.step()
-            losses[i] = loss.detach()
-
-        def same_state(what):
-            assert torch.equal(losses[0], losses[1]), what
-            for (na, pa), (_, pb) in zip(twins[0][0].named_parameters(), twins[1][0].named_parameters()):
-                assert torch.equal(pa, pb), f"{what}: {na}"
-
-        # both twins take their first step eagerly on a side stream (gradient accumulators are created there)
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            step(0)
-            step(1)
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        ring.fence(DEV)
-        same_state("first eager step")
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            step(0)
-        ring.fence(DEV)
-        # the capture recorded the step without running it: twin 0 is still one step behind after this replay
-        for r in range(4):
-            if r:
-                ids.copy_(torch.randint(0, V, (L, N), generator=gen))
-                tgt.copy_(torch.randint(0, V, (L, N), generator=gen))
-            graph.replay()
-            torch.cuda.synchronize()
-            with torch.cuda.stream(side):
-                step(1)
-            torch.cuda.synchronize()
-            same_state(f"replay {r}")
-            _ = (twins[0][0][2].norm1.weight.float() * 2).sum().item()  # unrelated eager work between replays
+        twins = [build_pair(V, D, H, Fd, n_dec, ws, torch.bfloat16)[0] for _ in range(2)]
+        graph_replays_against_eager_twin(twins, V, L, N, replays=4)
     finally:
         ring.set_wgrad_overlap(before)
