@@ -129,6 +129,9 @@ class DeviceRing:
     def reserve(self, nbytes: int) -> None:
         if nbytes <= self.slot_bytes:
             return
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("rotation staging slots have to grow while a graph is being captured: run one eager "
+                               "step of every model first, so that the slots have their final size")
         # Work queued on the side stream may still read the old slots.
         torch.cuda.synchronize(self.device)
         if self.staging is not None:

@@ -127,3 +127,33 @@ def test_stage_group_partial_use_and_restage():
     finally:
         ring.set_rotation_window(saved)
     torch.cuda.synchronize()
+
+
+def test_staging_growth_during_capture_is_refused():
+    """A layer whose shards do not fit the staging slots yet cannot take its first step inside a graph capture (the
+    slots would have to be reallocated under the graph): a clear error, nothing recorded, and the layer works
+    eagerly afterwards."""
+    from rtp_amd import emulate_shards, ring
+    from rtp_amd.module.linear import ColumnParallelLinear
+    dev = torch.device(DEV)
+    slot = ring.device_ring(dev).slot_bytes
+    n = max(512, (int((slot / 4) ** 0.5) // 256 + 2) * 256)  # an fp32 [n, n] weight larger than one slot
+    with emulate_shards(2):
+        layer = ColumnParallelLinear(n, n, device=DEV, dtype=torch.float32)
+    x = torch.randn(8, n, device=DEV)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        _ = x * 2  # the capture below needs a warmed-up allocator, not a warmed-up layer
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError, match="eager step"):
+        with torch.cuda.graph(graph):
+            layer(x)
+    torch.cuda.synchronize()
+    y = layer(x)
+    ref = torch.nn.functional.linear(x.cpu(), torch.cat([l.weight for l in layer.linears], 0).cpu(),
+                                     torch.cat([l.bias for l in layer.linears], 0).cpu())
+    torch.testing.assert_close(y.cpu(), ref, rtol=1e-4, atol=1e-4)
+    assert ring.device_ring(dev).slot_bytes >= n * n * 4
