@@ -475,6 +475,15 @@ def layernorm_bwd_deferred(dy: torch.Tensor, z: torch.Tensor, gamma: torch.Tenso
     return part
 
 
+def _device_table(rows, device) -> torch.Tensor:
+    """int64 rows -> device tensor.  The upload cannot be recorded into a graph: a model's first step, which builds
+    its tables, has to run eagerly."""
+    if torch.cuda.is_current_stream_capturing():
+        raise RuntimeError("a device table (optimiser chunks / LayerNorm reduction) has to be built while a graph is "
+                           "being captured: run one eager step of the model and its optimiser first")
+    return torch.tensor(rows, dtype=torch.int64).to(device)
+
+
 def layernorm_final_table(items, device) -> torch.Tensor:
     """Device table for layernorm_finalize: items = [(part, rows, cols, dgamma, dbeta or None), ...]."""
     lib = _lib.load()
@@ -482,7 +491,7 @@ def layernorm_final_table(items, device) -> torch.Tensor:
     for part, n_rows, cols, dgamma, dbeta in items:
         rows.append([part.data_ptr(), lib.rtp_layernorm_bwd_blocks(n_rows), cols, dgamma.data_ptr(),
                      dbeta.data_ptr() if dbeta is not None else 0])
-    return torch.tensor(rows, dtype=torch.int64).to(device)
+    return _device_table(rows, device)
 
 
 def layernorm_finalize(table: torch.Tensor, dtype: torch.dtype, max_cols: int) -> None:
@@ -691,7 +700,7 @@ def sgd_chunk_table(items, device) -> Optional[torch.Tensor]:
                          shadow.data_ptr() + off * gs if shadow is not None else 0, cnt))
     if not rows:
         return None
-    return torch.tensor(rows, dtype=torch.int64).to(device)
+    return _device_table(rows, device)
 
 
 def adam_chunk_table(items, device) -> Optional[torch.Tensor]:
@@ -713,7 +722,7 @@ def adam_chunk_table(items, device) -> Optional[torch.Tensor]:
                          v.data_ptr() + off * 4, cnt))
     if not rows:
         return None
-    return torch.tensor(rows, dtype=torch.int64).to(device)
+    return _device_table(rows, device)
 
 
 def adam_step_multi(table: torch.Tensor, dtype: torch.dtype, step, lr: float, betas, eps: float, weight_decay: float,
