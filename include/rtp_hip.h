@@ -236,6 +236,11 @@ int rtp_embedding_scatter_add_scaled(void* stream, int dtype, const void* grad_o
 int rtp_softmax_fwd(void* stream, int dtype, const float* s, const float* mask, const float* key_bias,
                     int64_t n_batch, int64_t heads, int causal, float scale, int64_t z, int64_t l, int64_t skv,
                     void* p);
+/* The same with one mask per problem (the 3-D attn_mask [batch * heads, L, S] of functional.py:701-704): mask is fp32
+ * [mask_problems, L, S] and problem z takes mask[z % mask_problems]; mask_problems <= 1 is the single-mask form. */
+int rtp_softmax_fwd_masks(void* stream, int dtype, const float* s, const float* mask, int64_t mask_problems,
+                          const float* key_bias, int64_t n_batch, int64_t heads, int causal, float scale, int64_t z,
+                          int64_t l, int64_t skv, void* p);
 int rtp_softmax_bwd(void* stream, int dtype, const void* p, const float* dp, float scale,
                     int64_t z, int64_t l, int64_t skv, void* ds);
 

@@ -88,6 +88,7 @@ PROTOTYPES = {
     "rtp_embedding_scatter_add_scaled": (_i, [_vp, _i, _vp, _i64, _i64, _vp, _vp, _i64, _i, _i64, _i64, _i64,
                                               _i64, _i, _i, _i64, _i64, _i64, _f]),
     "rtp_softmax_fwd": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _i64, _i, _f, _i64, _i64, _i64, _vp]),
+    "rtp_softmax_fwd_masks": (_i, [_vp, _i, _vp, _vp, _i64, _vp, _i64, _i64, _i, _f, _i64, _i64, _i64, _vp]),
     "rtp_softmax_bwd": (_i, [_vp, _i, _vp, _vp, _f, _i64, _i64, _i64, _vp]),
     "rtp_attn_supported": (_i, [_i, _i64, _i64]),
     "rtp_attn_fwd": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _i,

@@ -9,13 +9,14 @@ constexpr int kRowsPerBlock = 4;
 template <typename T>
 __global__ __launch_bounds__(256) void softmax_fwd_kernel(const float* s, const float* mask, const float* kbias,
                                                           long n_batch, long heads, int causal, float scale,
-                                                          long rows, long l, long skv, T* p) {
+                                                          long rows, long l, long skv, T* p, long mask_mod) {
   const int lane = threadIdx.x & 63;
   const long row = (long)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
   if (row >= rows) return;
   const long i = row % l;
   const float* srow = s + row * skv;
-  const float* mrow = mask ? mask + i * skv : nullptr;
+  // one [l, skv] mask for every problem, or mask_mod of them: problem z takes mask[z % mask_mod]
+  const float* mrow = mask ? mask + (mask_mod > 1 ? ((row / l) % mask_mod) * l * skv : 0) + i * skv : nullptr;
   // per-(batch, key) bias: problem index row / l = (group * n_batch + batch) * heads + head
   const float* krow = kbias ? kbias + ((row / l / heads) % n_batch) * skv : nullptr;
   T* prow = p + row * skv;
@@ -72,10 +73,12 @@ __global__ __launch_bounds__(256) void softmax_bwd_kernel(const T* p, const floa
 
 using namespace rtp;
 
-extern "C" int rtp_softmax_fwd(void* stream, int dtype, const float* s, const float* mask, const float* key_bias,
-                               int64_t n_batch, int64_t heads, int causal, float scale, int64_t z, int64_t l,
-                               int64_t skv, void* p) {
+extern "C" int rtp_softmax_fwd_masks(void* stream, int dtype, const float* s, const float* mask, int64_t mask_problems,
+                                     const float* key_bias, int64_t n_batch, int64_t heads, int causal, float scale,
+                                     int64_t z, int64_t l, int64_t skv, void* p) {
   RTP_REQUIRE(s && p, "rtp_softmax_fwd: null pointer");
+  RTP_REQUIRE(mask_problems >= 0 && (mask_problems <= 1 || (mask && z % mask_problems == 0)),
+              "rtp_softmax_fwd: %lld masks do not divide z=%lld problems", (long long)mask_problems, (long long)z);
   RTP_REQUIRE(!key_bias || (n_batch >= 1 && heads >= 1 && z % (n_batch * heads) == 0),
               "rtp_softmax_fwd: a key bias needs z = groups * n_batch * heads (z=%lld n_batch=%lld heads=%lld)",
               (long long)z, (long long)n_batch, (long long)heads);
@@ -89,14 +92,20 @@ extern "C" int rtp_softmax_fwd(void* stream, int dtype, const float* s, const fl
   ProfileScope prof(st, "softmax_fwd", 0.0, (double)rows * skv * (4.0 + (dtype == RTP_F32 ? 4 : 2)));
   if (dtype == RTP_F32)
     hipLaunchKernelGGL(softmax_fwd_kernel<float>, grid, dim3(256), 0, st, s, mask, key_bias, (long)n_batch, (long)heads,
-                       causal, scale, (long)rows, (long)l, (long)skv, (float*)p);
+                       causal, scale, (long)rows, (long)l, (long)skv, (float*)p, (long)mask_problems);
   else if (dtype == RTP_BF16)
     hipLaunchKernelGGL(softmax_fwd_kernel<bf16_t>, grid, dim3(256), 0, st, s, mask, key_bias, (long)n_batch, (long)heads,
-                       causal, scale, (long)rows, (long)l, (long)skv, (bf16_t*)p);
+                       causal, scale, (long)rows, (long)l, (long)skv, (bf16_t*)p, (long)mask_problems);
   else
     return fail(RTP_ERR_ARG, "rtp_softmax_fwd: unknown dtype %d", dtype);
   RTP_LAUNCH_CHECK();
   return RTP_OK;
+}
+
+extern "C" int rtp_softmax_fwd(void* stream, int dtype, const float* s, const float* mask, const float* key_bias,
+                               int64_t n_batch, int64_t heads, int causal, float scale, int64_t z, int64_t l,
+                               int64_t skv, void* p) {
+  return rtp_softmax_fwd_masks(stream, dtype, s, mask, 1, key_bias, n_batch, heads, causal, scale, z, l, skv, p);
 }
 
 extern "C" int rtp_softmax_bwd(void* stream, int dtype, const void* p, const float* dp, float scale, int64_t z,

@@ -141,9 +141,10 @@ class _AttentionFn(torch.autograd.Function):
         o = torch.empty(rows, E, dtype=dt, device=dev)
         out = torch.empty(rows, E, dtype=dt, device=dev)
         ldq = N * ws * 3 * e_s
-        # attention dropout works on the probabilities in memory: the product + softmax form of the core
-        fused = drop_p == 0.0 and ops.attn_supported(dt, L, d)
-        flash = drop_p == 0.0 and not fused and not want_weights and ops.attn_flash_supported(dt, L, d)
+        # attention dropout and per-head masks work on the probabilities in memory: the product + softmax form
+        plain = drop_p == 0.0 and (mask is None or mask.dim() == 2)
+        fused = plain and ops.attn_supported(dt, L, d)
+        flash = plain and not fused and not want_weights and ops.attn_flash_supported(dt, L, d)
         if flash:
             p = torch.empty(ws * Z, L, dtype=torch.float32, device=dev)  # log-sum-exp in place of probabilities
         else:
@@ -498,8 +499,8 @@ class ParallelMultiheadAttention(RotatedLayer):
     """Signature follows rtp/module/attention.py:192-193; `MultiheadAttention_layer` imports the weights
     of an unsharded nn.MultiheadAttention.  Self-attention (query, key and value the same tensor) takes the packed
     projection and the fused cores; keys / values from other tensors, kdim / vdim != embed_dim and add_zero_attn take
-    three projections and the product + softmax core, and so does attention dropout while training (the probabilities
-    are dropped in memory).  3-D masks and add_bias_kv are not implemented and raise.  key_padding_mask [batch, keys] (bool or float, functional.py:615-623 and :760-768) reaches
+    three projections and the product + softmax core, and so do attention dropout while training (the probabilities
+    are dropped in memory) and 3-D masks [batch * heads / ws, L, S].  add_bias_kv is not implemented and raises.  key_padding_mask [batch, keys] (bool or float, functional.py:615-623 and :760-768) reaches
     the kernels as a per-(batch, key) additive bias."""
 
     def __init__(self, embed_dim, num_heads, world_size, rank, dropout=0., bias=True, add_bias_kv=False,
@@ -547,9 +548,12 @@ class ParallelMultiheadAttention(RotatedLayer):
         mask = None
         causal = False
         if attn_mask is not None:
-            if attn_mask.dim() != 2 or tuple(attn_mask.shape) != (L, keys):
-                raise NotImplementedError(f"rotated attention: only a 2-D [queries, keys] = {(L, keys)} attn_mask is "
-                                          f"implemented, got {tuple(attn_mask.shape)}")
+            # functional.py:690-704: [L, S], or one mask per (batch, head of a shard) [N * heads / ws, L, S], which
+            # every head group of the rotation then shares
+            per_head = (x.shape[1] * self.num_heads_per_partition, L, keys)
+            if tuple(attn_mask.shape) not in ((L, keys), per_head):
+                raise RuntimeError(f"The shape of the attn_mask is {tuple(attn_mask.shape)}, but should be "
+                                   f"{(L, keys)} or {per_head}.")
             mask = F._canonical_mask(mask=attn_mask, mask_name="attn_mask", other_type=None, other_name="",
                                      target_type=torch.float32)
             mask = mask.to(device=x.device, dtype=torch.float32).contiguous()

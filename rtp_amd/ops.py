@@ -274,22 +274,29 @@ def _key_bias_ptr(who: str, key_bias: Optional[torch.Tensor], n_batch: int, keys
 
 def softmax_fwd(scores: torch.Tensor, p: torch.Tensor, *, mask: Optional[torch.Tensor], causal: bool,
                 scale: float, key_bias: Optional[torch.Tensor] = None, heads: int = 1) -> None:
-    """p[Z,L,S] = softmax(scale*scores + mask + key_bias[b]) row-wise; scores fp32, mask fp32 [L,S] or None,
-    key_bias fp32 [N,S] or None with Z = groups * N * heads (problem z belongs to batch (z // heads) % N)."""
+    """p[Z,L,S] = softmax(scale*scores + mask + key_bias[b]) row-wise; scores fp32, mask fp32 [L,S] (one for all
+    problems) or [M,L,S] (problem z takes mask[z % M]) or None, key_bias fp32 [N,S] or None with
+    Z = groups * N * heads (problem z belongs to batch (z // heads) % N)."""
     _dev(scores)
     _dev(p)
     if scores.dtype != torch.float32 or scores.dim() != 3 or not scores.is_contiguous() or \
             p.shape != scores.shape or not p.is_contiguous():
         raise ValueError("softmax_fwd: scores must be contiguous fp32 [Z,L,S] and p the same shape")
     z, l, s = scores.shape
+    masks = 1
     if mask is not None:
-        if mask.dtype != torch.float32 or tuple(mask.shape) != (l, s) or not mask.is_contiguous():
-            raise ValueError("softmax_fwd: mask must be contiguous fp32 [L,S]")
+        if mask.dtype != torch.float32 or tuple(mask.shape[-2:]) != (l, s) or mask.dim() not in (2, 3) or \
+                not mask.is_contiguous():
+            raise ValueError("softmax_fwd: mask must be contiguous fp32 [L,S] or [M,L,S]")
+        if mask.dim() == 3:
+            masks = mask.shape[0]
+            if masks < 1 or z % masks:
+                raise ValueError(f"softmax_fwd: {masks} masks do not divide {z} problems")
     n_batch = key_bias.shape[0] if key_bias is not None else 1
     kb = _key_bias_ptr("softmax_fwd", key_bias, n_batch, s)
     _lib.require_device()
-    check(_lib.load().rtp_softmax_fwd(_stream(), dtype_code(p.dtype), scores.data_ptr(), _ptr(mask), kb, n_batch, heads,
-                                      int(causal), scale, z, l, s, p.data_ptr()))
+    check(_lib.load().rtp_softmax_fwd_masks(_stream(), dtype_code(p.dtype), scores.data_ptr(), _ptr(mask), masks, kb,
+                                            n_batch, heads, int(causal), scale, z, l, s, p.data_ptr()))
 
 
 def softmax_bwd(p: torch.Tensor, dp: torch.Tensor, ds: torch.Tensor, scale: float) -> None:

@@ -92,8 +92,8 @@ def test_attention_unsupported_raise():
     from rtp_amd.module.attention import ParallelMultiheadAttention
     layer = ParallelMultiheadAttention(8, 2, 2, 0, device=DEV)
     x = torch.randn(4, 2, 8, device=DEV)
-    with pytest.raises(NotImplementedError):
-        layer(x, x, x, attn_mask=torch.zeros(4, 4, 4, device=DEV))  # 3-D masks
+    with pytest.raises(RuntimeError):
+        layer(x, x, x, attn_mask=torch.zeros(4, 4, 4, device=DEV))  # a 3-D mask is [batch * heads / ws, L, S] = [2, 4, 4]
     with pytest.raises(ValueError):
         layer(x, x, x, key_padding_mask=torch.zeros(3, 4, dtype=torch.bool, device=DEV))   # [batch, keys] = [2, 4]
     with pytest.raises(NotImplementedError):

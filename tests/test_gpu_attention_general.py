@@ -149,7 +149,43 @@ def test_general_attention_argument_checks():
         layer(q, k, torch.randn(8, 2, 32, device=DEV))  # keys and values must pair up
     with pytest.raises(ValueError):
         layer(q, k, k, key_padding_mask=torch.zeros(2, 5, dtype=torch.bool, device=DEV))
-    with pytest.raises(NotImplementedError):
-        layer(q, k, k, attn_mask=torch.zeros(8, 5, 7, device=DEV))
+    with pytest.raises(RuntimeError):
+        layer(q, k, k, attn_mask=torch.zeros(8, 5, 7, device=DEV))  # 3-D masks are [batch * heads / ws, L, S]
     with pytest.raises(NotImplementedError):
         ParallelMultiheadAttention(32, 4, 2, 0, add_bias_kv=True, device=DEV)
+
+
+@pytest.mark.parametrize("ws", [1, 2, 4])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_one_mask_per_batch_entry_and_head(ws, dtype):
+    """3-D attn_mask (functional.py:701-704).  A shard sees heads / ws heads, so the mask is [batch * heads / ws, L, S]
+    and every head group of the rotation shares it; the unsharded layer gets the same masks laid out over all heads.
+    Keys from another tensor (fp32) and self-attention (also bf16, where 2-D masks would take the fused core)."""
+    from rtp_amd.module.attention import ParallelMultiheadAttention
+    E, H, L, N = 64, 4, 7, 3
+    h_s = H // ws
+    gen = torch.Generator().manual_seed(20 + ws)
+    ref = _master(E, H, gen, dtype)
+    layer = ParallelMultiheadAttention(E, H, ws, 0, MultiheadAttention_layer=ref.to(dtype) if dtype != torch.float32 else ref,
+                                       device=DEV, dtype=dtype)
+    ref = ref.float()
+    for S, same in ((L, True), (10, False)):
+        m = torch.where(torch.rand(N * h_s, L, S, generator=gen) < 0.3, float("-inf"), 0.0)
+        m += torch.randn(N * h_s, L, S, generator=gen)
+        m[:, :, 0] = 0.0
+        full = m.view(N, 1, h_s, L, S).expand(N, ws, h_s, L, S).reshape(N * H, L, S)
+        q = torch.randn(L, N, E, generator=gen).to(dtype)
+        k = q if same else torch.randn(S, N, E, generator=gen).to(dtype)
+        g = torch.randn(L, N, E, generator=gen).to(dtype)
+        qd = q.to(DEV).requires_grad_()
+        kd = qd if same else k.to(DEV).requires_grad_()
+        out, _ = layer(qd, kd, kd, attn_mask=m.to(DEV), need_weights=False)
+        out.backward(g.to(DEV))
+        qo = q.float().requires_grad_()
+        ko = qo if same else k.float().requires_grad_()
+        want, _ = ref(qo, ko, ko, attn_mask=full, need_weights=False)
+        want.backward(g.float())
+        assert_close(out, want, dtype, "output")
+        assert_close(qd.grad, qo.grad, dtype, "query grad")
+        if not same:
+            assert_close(kd.grad, ko.grad, dtype, "key grad")
