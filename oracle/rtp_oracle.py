@@ -24,8 +24,10 @@ float32 unless the caller passes float64 tensors.  How each function is pinned (
   column_parallel_conv2d / conv_patches / conv_fold
                                                  == torch.nn.functional.conv2d on the unsharded problem, F.unfold / F.fold,
                                                     and python loops over a tiny input (patch layout and zero padding)
-  transformer_lm                                 == assembled from stock torch layers exactly as
-                                                    rtp/models/transformer_lm_rtp.py:19-242 assembles the rotated ones
+  TransformerLM (with and without MoE blocks)    == golden vectors written from the reference's own TransformerLM run on
+                                                    a 2-rank gloo ring (tests/golden/lm_ws2.npz, lm_moe_ws2.npz: logits,
+                                                    losses, l_aux and every home-shard gradient), plus parameter count
+                                                    and causality
 """
 from __future__ import annotations
 
@@ -345,31 +347,50 @@ class _PositionalEncoding(nn.Module):
 
 
 class _DecoderLayer(nn.Module):
-    """Post-LN block x = LN1(x + SA(x)); x = LN2(x + FFN(x)) (transformer_lm_rtp.py:176-177), dropout 0."""
+    """Post-LN block x = LN1(x + SA(x)); x = LN2(x + FFN(x)) (transformer_lm_rtp.py:176-177), dropout 0.  With
+    `num_experts` > 0 the feed-forward block is the MoE layer (:151-158, :191-195): gate projection `wg`, experts
+    `experts[e]` = (linear1, linear2); the routing noise is the attribute `noise` ([S, E], zeros if unset -- with two
+    experts the noise cannot change the routing) and the layer keeps `l_aux` as the reference's moe_layer does."""
 
-    def __init__(self, ninp, nhead, nhid):
+    def __init__(self, ninp, nhead, nhid, num_experts=0, ws=1):
         super().__init__()
         self.self_attn = nn.MultiheadAttention(ninp, nhead, dropout=0.0)
         self.norm1 = nn.LayerNorm(ninp)
         self.norm2 = nn.LayerNorm(ninp)
-        self.linear1 = nn.Linear(ninp, nhid)
-        self.linear2 = nn.Linear(nhid, ninp)
+        self.num_experts, self.ws, self.noise, self.l_aux = num_experts, ws, None, None
+        if num_experts:
+            self.wg = nn.Linear(ninp, num_experts, bias=False)
+            self.experts = nn.ModuleList(nn.ModuleList([nn.Linear(ninp, nhid), nn.Linear(nhid, ninp)])
+                                         for _ in range(num_experts))
+        else:
+            self.linear1 = nn.Linear(ninp, nhid)
+            self.linear2 = nn.Linear(nhid, ninp)
+
+    def _ff(self, x):
+        if not self.num_experts:
+            return self.linear2(F.relu(self.linear1(x)))
+        S = x.shape[0] * x.shape[1]
+        noise = self.noise if self.noise is not None else torch.zeros(S, self.num_experts, dtype=x.dtype)
+        experts = [(e[0].weight, e[0].bias, e[1].weight, e[1].bias) for e in self.experts]
+        out, self.l_aux = moe_layer(x, self.wg.weight, experts, noise, self.ws)
+        return out
 
     def forward(self, x):
         L = x.shape[0]
         mask = torch.triu(torch.full((L, L), float("-inf"), dtype=x.dtype), diagonal=1)      # :201-204
         x = self.norm1(x + self.self_attn(x, x, x, attn_mask=mask, need_weights=False)[0])
-        return self.norm2(x + self.linear2(F.relu(self.linear1(x))))
+        return self.norm2(x + self._ff(x))
 
 
 class TransformerLM(nn.Sequential):
     """Unsharded LM with the rotated LM's structure; weights are copied in by the tests so both sides
-    start from identical values."""
+    start from identical values.  num_experts > 0 builds the is_moe=True model (one gate + `num_experts` experts per
+    decoder layer, `ws` shards in the MoE layer's ring order)."""
 
-    def __init__(self, ntokens, ninp, nhead, nhid, ndecoder):
+    def __init__(self, ntokens, ninp, nhead, nhid, ndecoder, num_experts=0, ws=1):
         self.ninp = ninp
         layers = [nn.Embedding(ntokens, ninp), _PositionalEncoding(ninp)]
-        layers += [_DecoderLayer(ninp, nhead, nhid) for _ in range(ndecoder)]
+        layers += [_DecoderLayer(ninp, nhead, nhid, num_experts, ws) for _ in range(ndecoder)]
         layers.append(nn.Linear(ninp, ntokens))
         super().__init__(*layers)
 

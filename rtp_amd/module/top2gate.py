@@ -148,15 +148,24 @@ class _GateProjectionFn(torch.autograd.Function):
         return dx, None, None
 
 
-class Top2Gate(nn.Module):
-    """Unsharded gate (rtp/module/top2gate.py:109-137): the master a WeightTop2Gate can be built from."""
+class Top2Gate(RotatedLayer):
+    """Unsharded gate (rtp/module/top2gate.py:109-137): forward(input[S,M]) = top2gating(wg(input)), and the master a
+    WeightTop2Gate can be built from.  The projection is the rotated gate's with a single shard holding every expert
+    row, so it runs on the same kernels."""
 
     def __init__(self, model_dim: int, num_experts: int) -> None:
         super().__init__()
-        self.wg = nn.Linear(model_dim, num_experts, bias=False)
+        self.model_dim = model_dim
+        self.num_experts = num_experts
+        self.world_size, self.rank, self.num_local_experts = 1, 0, num_experts
+        self._init_store([nn.Linear(model_dim, num_experts, bias=False)])
+        self.wg = self.shards[0]
 
     def forward(self, input: Tensor, noise: Optional[Tensor] = None) -> Tuple[Tensor, Tensor, Tensor]:
-        raise NotImplementedError("Top2Gate only carries master weights here; use WeightTop2Gate(gate=...)")
+        logits = _GateProjectionFn.apply(input, self._anchor, self)
+        r, weight, l_aux = top2_route(logits, noise)
+        combine, dispatch = dense_from_routing(r, weight, input.dtype)
+        return l_aux.to(input.dtype), combine, dispatch
 
 
 class WeightTop2Gate(RotatedLayer):

@@ -60,3 +60,21 @@ def test_ops_refuse_cpu_tensors():
         ops.linear_fwd(torch.zeros(2, 2), torch.zeros(2, 2), torch.zeros(2, 2))
     with pytest.raises(_lib.RtpError):
         ops.embedding_gather(torch.zeros(2, 2), torch.zeros(2, dtype=torch.long), torch.zeros(2, 2))
+
+
+def test_integration_stub_struct_matches_the_library():
+    """The ctypes GemmDesc a maintainer would paste from INTEGRATION.md has the layout of rtp_gemm_desc: same size as
+    the library reports and the same field names, order and offsets as the package's own binding."""
+    from rtp_amd import _lib
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    m = re.search(r"^class GemmDesc\(C\.Structure\):.*?(?=^assert _lib\.rtp_gemm_desc_size)", text, flags=re.S | re.M)
+    assert m, "INTEGRATION.md no longer holds the GemmDesc stub"
+    scope = {"C": ctypes}
+    exec(m.group(0), scope)
+    stub = scope["GemmDesc"]
+    assert ctypes.sizeof(stub) == ctypes.sizeof(_lib.GemmDesc)
+    mine = [(n, getattr(_lib.GemmDesc, n).offset, getattr(_lib.GemmDesc, n).size) for n, _ in _lib.GemmDesc._fields_]
+    theirs = [(n, getattr(stub, n).offset, getattr(stub, n).size) for n, _ in stub._fields_]
+    assert mine == theirs
+    if os.path.exists(_lib.LIB_PATH):
+        assert _lib.load().rtp_gemm_desc_size() == ctypes.sizeof(stub)

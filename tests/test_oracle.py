@@ -322,3 +322,69 @@ def test_gloo_ring_column_linear_equals_unsharded_linear(ws):
     assert len(res["times"]) == 2 and all(t > 0 for t in res["times"])
     # and the one-process shard loop used by the device parity tests agrees with it
     torch.testing.assert_close(O.column_parallel_linear(x, w, b, ws), res["y"])
+
+
+# ---- LM against the reference's own TransformerLM on a 2-rank gloo ring (tests/golden/make_lm_golden.py) ----
+@pytest.mark.parametrize("name", ["lm_ws2.npz", "lm_moe_ws2.npz"])
+def test_transformer_lm_matches_reference_golden(name):
+    """Logits, loss (and l_aux) of each rank's batch; every home-shard gradient == the matching slice of the
+    gradient of the SUM of the ranks' losses; LayerNorm gradients == the gradient of that rank's loss alone."""
+    import lm_golden as G
+    fix = G.load(name)
+    c = fix["cfg"]
+    ref = G.oracle_lm(fix)
+    per_rank_ln = []
+    total = {}
+    for r in range(c["WS"]):
+        for p in ref.parameters():
+            p.grad = None
+        logits = ref(fix["ids"][r])
+        torch.testing.assert_close(logits, fix[f"rank{r}.logits"])
+        loss = F.cross_entropy(logits.view(-1, c["V"]), fix["tgt"][r].view(-1))
+        if c["moe"]:
+            l_aux = torch.stack([ref[2 + i].l_aux for i in range(c["NDEC"])])
+            torch.testing.assert_close(l_aux, fix[f"rank{r}.l_aux"])
+            loss = loss + l_aux.sum()
+        torch.testing.assert_close(loss, fix[f"rank{r}.loss"])
+        loss.backward()
+        g = {k: v.clone() for k, v in G.oracle_full_grads(ref, c).items()}
+        per_rank_ln.append({k: v for k, v in g.items() if ".ln" in k})
+        for k, v in g.items():
+            total[k] = total[k] + v if k in total else v
+    for r in range(c["WS"]):
+        for k, v in G.shard_slices(total, c, r).items():
+            torch.testing.assert_close(fix[f"rank{r}.grad.{k}"], v, msg=lambda m, k=k, r=r: f"rank {r} {k}: {m}")
+        for k, v in per_rank_ln[r].items():
+            torch.testing.assert_close(fix[f"rank{r}.grad.{k}"], v, msg=lambda m, k=k, r=r: f"rank {r} {k}: {m}")
+
+
+def test_transformer_lm_golden_catches_structural_mistakes():
+    """The fixture separates the reference's structure from near misses: no sqrt(ninp) scale, sin/cos swapped in the
+    positions, pre-LN blocks -- each moves the logits far outside the comparison's tolerance."""
+    import lm_golden as G
+    fix = G.load("lm_ws2.npz")
+    ref = G.oracle_lm(fix)
+    want = fix["rank0.logits"]
+    ids = fix["ids"][0]
+
+    def run(scale=True, swap_pe=False, pre_ln=False):
+        x = ref[0](ids) * (math.sqrt(ref.ninp) if scale else 1.0)
+        pe = ref[1].pe[: x.size(0), :]
+        if swap_pe:
+            pe = torch.stack([pe[..., 1::2], pe[..., 0::2]], dim=-1).flatten(-2)
+        x = x + pe
+        for d in list(ref)[2:-1]:
+            L = x.shape[0]
+            mask = torch.triu(torch.full((L, L), float("-inf")), diagonal=1)
+            if pre_ln:
+                h = d.norm1(x)
+                x = x + d.self_attn(h, h, h, attn_mask=mask, need_weights=False)[0]
+                x = x + d._ff(d.norm2(x))
+            else:
+                x = d.norm1(x + d.self_attn(x, x, x, attn_mask=mask, need_weights=False)[0])
+                x = d.norm2(x + d._ff(x))
+        return ref[-1](x)
+
+    torch.testing.assert_close(run(), want)
+    for kw in (dict(scale=False), dict(swap_pe=True), dict(pre_ln=True)):
+        assert (run(**kw) - want).abs().max() > 1e-2, kw
