@@ -359,6 +359,10 @@ def main():
     ap.add_argument("--optimizer", default="sgd", choices=["sgd", "adam"],
                     help="sgd: the headline configuration (default); adam: the reference harness's own optimiser "
                          "(clip 0.05, Adam lr 1e-3), fp32 moments beside the fp32 master")
+    ap.add_argument("--rotation", default="direct", choices=["direct", "staged"],
+                    help="direct (default): the products read every shard from its home row, the LDS stage ring of the "
+                         "product kernel is the rotation's double buffer; staged: shards are first copied into two HBM "
+                         "slots on a side stream (the transport of a multi-GPU ring)")
     ap.add_argument("--no-graph", dest="graph", action="store_false",
                     help="launch every kernel eagerly instead of replaying the step from a captured HIP graph")
     args = ap.parse_args()
@@ -379,6 +383,7 @@ def main():
 
     dev = torch.device("cuda", 0)
     ring.set_wgrad_overlap(args.wgrad_overlap)
+    ring.set_rotation_mode(args.rotation)
     torch.cuda.set_device(dev)
     c = CFG
     lm = build(c, dev, torch.bfloat16)
@@ -460,7 +465,7 @@ def main():
                                "32 heads, seq 32, batch 32, bf16 weights + fp32 master, 8 rotation shards emulated on "
                                "one GPU, uniform random token ids, weights U(-0.1,0.1), dropout 0, lr 1e-3, clip 0.05",
                    "tokens_per_step": tokens, "rotation_shards": c["shards"], "hip_graph": bool(args.graph),
-                   "optimizer": args.optimizer,
+                   "optimizer": args.optimizer, "rotation": args.rotation,
                    "sgd_overlapped_with_backward": bool(args.sgd_overlap),
                    "wgrad_on_second_stream": bool(args.wgrad_overlap)},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK["bf16_mfma_tflops"], "unit": "TFLOP/s",

@@ -36,6 +36,27 @@ def rotation_window() -> Optional[int]:
     return _window
 
 
+# ---- where a shard waits for its turn ----------------------------------------------------------------
+# "direct" (default): the products read every shard straight from its home row.  The double buffer of the rotation is
+# then the LDS stage ring inside the product kernel: its loader waves stream the tiles of the next (shard, tile) work
+# item from home into LDS while the MFMA waves work on the current one, so no second copy of a shard ever exists in
+# HBM (resident weights = 1.0x the model) and the weights cross the memory bus once per pass.
+# "staged": every window of shards is first copied home -> staging slot by the copy kernel on the side stream while
+# the previous window computes (two slots in HBM; the transport a multi-GPU ring would fill from its neighbour).
+_mode = os.environ.get("RTP_ROTATION", "direct")
+
+
+def set_rotation_mode(mode: str) -> None:
+    global _mode
+    if mode not in ("direct", "staged"):
+        raise ValueError("rotation mode must be 'direct' or 'staged'")
+    _mode = mode
+
+
+def rotation_mode() -> str:
+    return _mode
+
+
 # ---- weight gradients on a second stream -----------------------------------------------------------
 # A layer's weight / bias gradients are needed only by the optimiser, while its input gradient is needed by
 # the next layer of the backward pass.  With the switch on, the gradient products of the parameters are
@@ -298,6 +319,9 @@ class Rotation:
                     start = b
             self.windows.append(runs)
         self.steps = len(self.windows)
+        self.direct = _mode == "direct"
+        if self.direct:
+            return
         self.ring = device_ring(home.device)
         self.lib = _lib.load()
         self.stream = torch.cuda.current_stream(home.device).cuda_stream
@@ -321,6 +345,8 @@ class Rotation:
             dst += count * self.nbytes
 
     def acquire(self, j: int) -> List[Run]:
+        if self.direct:
+            return [(self.home[first:first + count], first, count) for first, count in self.windows[j]]
         if self.group is not None:
             g = self.group
             if not g.acquired:
@@ -342,6 +368,8 @@ class Rotation:
         return out
 
     def release(self, j: int) -> None:
+        if self.direct:
+            return
         if self.group is not None:
             g = self.group
             g.remaining.discard(self.member)

@@ -20,12 +20,17 @@ def _seed():
     yield
 
 
-@pytest.fixture(params=[None, 1, 3], ids=["window=all", "window=1", "window=3"])
+@pytest.fixture(params=[("direct", None), ("staged", None), ("staged", 1), ("staged", 3), ("direct", 3)],
+                ids=["direct", "window=all", "window=1", "window=3", "direct-window=3"])
 def rotation_window(request):
-    """Runs a GPU test under three rotation schedules: all shards of a layer staged together (one grouped
-    launch per layer), one shard per ring step (the reference's schedule), and a window that does not
-    divide the shard count (ragged last window)."""
-    from rtp_amd.ring import set_rotation_window
-    set_rotation_window(request.param)
-    yield request.param
+    """Runs a GPU test under the rotation schedules: shards read from their home rows by one grouped launch per
+    layer (the default); and, staged through the two HBM slots, all shards of a layer together, one shard per ring
+    step (the reference's schedule) and a window that does not divide the shard count (ragged last window); the
+    ragged window once more without staging."""
+    from rtp_amd.ring import set_rotation_mode, set_rotation_window
+    mode, window = request.param
+    set_rotation_mode(mode)
+    set_rotation_window(window)
+    yield window
     set_rotation_window(None)
+    set_rotation_mode("direct")

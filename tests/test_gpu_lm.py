@@ -156,7 +156,9 @@ def test_lm_bf16_master_weights_and_weight_bytes():
     n_rot = sum(p.numel() for n, p in lm.named_parameters() if "norm" not in n)
     assert rotated_weight_bytes(lm) == 2 * n_rot  # every shard resident exactly once, in bf16
     largest = max(m._store.numel for m in lm.modules() if hasattr(m, "_store")) * 2
-    assert staging_bytes() >= 2 * largest
+    from rtp_amd import ring
+    if ring.rotation_mode() == "staged":
+        assert staging_bytes() >= 2 * largest
 
 
 def test_lm_moe_variant_runs_and_backprops():

@@ -8,6 +8,15 @@ from gpu_util import DEV
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def _staged_mode():
+    """These tests are about the two HBM slots; the last one checks the direct schedule."""
+    from rtp_amd import ring
+    ring.set_rotation_mode("staged")
+    yield
+    ring.set_rotation_mode("direct")
+
+
 @pytest.mark.parametrize("window", [1, 3, None])
 def test_rotation_delivers_each_shard_in_ring_order(window):
     from rtp_amd.ring import Rotation, ring_order
@@ -157,3 +166,29 @@ def test_staging_growth_during_capture_is_refused():
                                      torch.cat([l.bias for l in layer.linears], 0).cpu())
     torch.testing.assert_close(y.cpu(), ref, rtol=1e-4, atol=1e-4)
     assert ring.device_ring(dev).slot_bytes >= n * n * 4
+
+
+@pytest.mark.parametrize("window", [None, 1, 3])
+def test_direct_rotation_reads_home_rows_and_stages_nothing(window):
+    """In the direct schedule a window's shards are handed out as views of their home rows, in the same window /
+    run structure as the staged schedule, and no staging memory is touched or reserved."""
+    from rtp_amd import ring
+    from rtp_amd.ring import Rotation, ring_order
+    ring.set_rotation_mode("direct")
+    before = ring.staging_bytes()
+    ws, numel = 8, 1000
+    home = torch.randn(ws, numel, device=DEV)
+    for rank in (0, 5):
+        order = ring_order(rank, ws)
+        rot = Rotation(home, order, window=window)
+        visited = []
+        for j in range(rot.steps):
+            for flat, first, cnt in rot.acquire(j):
+                assert flat.data_ptr() == home[first].data_ptr() and flat.shape == (cnt, numel)
+                visited += list(range(first, first + cnt))
+            rot.release(j)
+        assert sorted(visited) == list(range(ws))
+        w = window or ws
+        for j, win in enumerate(rot.windows):
+            assert sorted(s for f, c in win for s in range(f, f + c)) == sorted(order[j * w:(j + 1) * w])
+    assert ring.staging_bytes() == before
