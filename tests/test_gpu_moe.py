@@ -194,7 +194,7 @@ def test_unsharded_top2gate_forward_matches_reference_golden(path):
     x[:, :E] = logits
     l_aux, combine, dispatch = gate(x.to(DEV), noise=noise.to(DEV))
     assert np.array_equal(dispatch.cpu().numpy(), z["dispatch_mask"])
-    np.testing.assert_allclose(combine.cpu().numpy(), z["combine_weights"], rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(combine.detach().cpu().numpy(), z["combine_weights"], rtol=1e-5, atol=1e-7)
     assert abs(float(l_aux) - float(z["l_aux"])) <= 1e-6
 
 
