@@ -408,6 +408,17 @@ int rtp_gate_wgrad(void* stream, int dtype, const float* dlogits, int64_t ld_dlo
                    int64_t S, int64_t M, int64_t E, void* dw, int64_t ld_dw, int accumulate, void* workspace,
                    size_t workspace_bytes);
 
+/* rtp_gate_wgrad for callers that cannot allocate (code under HIP-graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as rtp_gate_wgrad without the
+ * workspace: the partial sums go to a buffer built into the library (RTP_GATE_WGRAD_STATIC_MAX_BYTES = 8 MiB of device
+ * memory per GPU, held until the process ends), so ceil(S / 64) * E * M * 4 bytes must not exceed that size -- larger
+ * problems are refused with RTP_ERR_ARG and belong to rtp_gate_wgrad.  The call allocates and frees nothing.  Every
+ * call on a GPU uses that GPU's one buffer: calls that may overlap on one GPU (different streams) race; calls on one
+ * stream, or ordered by events, do not.  Nothing in the buffer has to be cleared between calls. */
+#define RTP_GATE_WGRAD_STATIC_MAX_BYTES ((size_t)8 << 20)
+int rtp_gate_wgrad_static(void* stream, int dtype, const float* dlogits, int64_t ld_dlogits, const void* x,
+                          int64_t ldx, int64_t S, int64_t M, int64_t E, void* dw, int64_t ld_dw, int accumulate);
+
 /* ---------------------------------------------------------------------------------------------
  * Out-channel-sharded 2-D convolution (reference: the per-shard `self.layers[index](input_)` = F.conv2d of
  * ColumnParallelConv2d, rtp/module/conv.py:108, and its autograd backward) as a column-sharded product on

@@ -21,6 +21,7 @@ GEMM_CIN_F32 = 2
 GEMM_RELU = 4
 GEMM_STREAM_OUT = 8
 GEMM_ROWSUM_ACCUM = 16
+GATE_WGRAD_STATIC_MAX_BYTES = 8 << 20  # RTP_GATE_WGRAD_STATIC_MAX_BYTES of include/rtp_hip.h
 
 
 class RtpError(RuntimeError):
@@ -119,6 +120,7 @@ PROTOTYPES = {
     "rtp_gate_dgrad": (_i, [_vp, _i, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64]),
     "rtp_gate_wgrad_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "rtp_gate_wgrad": (_i, [_vp, _i, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i, _vp, _sz]),
+    "rtp_gate_wgrad_static": (_i, [_vp, _i, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i]),
     "rtp_im2col": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _i64, C.POINTER(ConvGeom), _vp, _i64]),
     "rtp_col2im": (_i, [_vp, _i, _vp, _i64, C.POINTER(ConvGeom), _vp]),
     "rtp_sgd_step": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _f, _f]),

@@ -97,6 +97,10 @@ __device__ __forceinline__ void nt_store(uint4 a, uint4* p) {
   __builtin_nontemporal_store(v, reinterpret_cast<nt_u32x4*>(p));
 }
 
+// Resolves, for the current device, the address of the scratch buffer built into the library for
+// rtp_gate_wgrad_static (gate.hip).  Part of rtp_device_check.
+int gate_static_setup();
+
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Reads one word of every 64-byte line of a kernel's BYTES bytes of arguments (and of the launch dimensions that

@@ -4,6 +4,8 @@
 // token row is read (or written) once.
 #include "common.h"
 
+#include <mutex>
+
 #include "rtp_hip.h"
 
 namespace rtp {
@@ -272,24 +274,14 @@ extern "C" size_t rtp_gate_wgrad_workspace_bytes(int64_t S, int64_t M, int64_t E
   return (size_t)ceil_div(S, kGateWgradRows) * (size_t)E * (size_t)M * sizeof(float);
 }
 
-extern "C" int rtp_gate_wgrad(void* stream, int dtype, const float* dlogits, int64_t ld_dlogits, const void* x,
-                              int64_t ldx, int64_t S, int64_t M, int64_t E, void* dw, int64_t ld_dw, int accumulate,
-                              void* workspace, size_t workspace_bytes) {
-  if (int rc = gate_check("rtp_gate_wgrad", dtype, S, M, E)) return rc;
-  const int64_t vec = dtype == RTP_F32 ? 4 : 8;
-  RTP_REQUIRE(dlogits && x && dw && workspace, "rtp_gate_wgrad: null pointer");
-  RTP_REQUIRE(aligned16(x) && aligned16(workspace) && ldx % vec == 0 && ldx >= M && ld_dw >= M && ld_dlogits >= E,
-              "rtp_gate_wgrad: x and the workspace must be 16-byte aligned, row pitches >= M (x: a multiple of %lld)",
-              (long long)vec);
-  RTP_REQUIRE(workspace_bytes >= rtp_gate_wgrad_workspace_bytes(S, M, E), "rtp_gate_wgrad: workspace of %zu bytes, need %zu",
-              workspace_bytes, rtp_gate_wgrad_workspace_bytes(S, M, E));
-  hipStream_t st = (hipStream_t)stream;
-  const double esz = dtype == RTP_F32 ? 4.0 : 2.0;
+// The two launches of the weight gradient; `part` holds ceil(S / 64) * E * M floats, every one of which the first
+// kernel writes before the second reads it (nothing has to start at zero).
+static int gate_wgrad_launch(hipStream_t st, int dtype, const float* dlogits, int64_t ld_dlogits, const void* x,
+                             int64_t ldx, int64_t S, int64_t M, int64_t E, void* dw, int64_t ld_dw, int accumulate,
+                             float* part) {
   const long nrb = ceil_div(S, kGateWgradRows);
-  ProfileScope prof(st, "gate_wgrad", 2.0 * S * M * E, esz * ((double)S * M + (double)E * M) + 4.0 * S * E + 8.0 * nrb * E * M);
   const dim3 grid((unsigned)ceil_div(M / 4, 256), (unsigned)nrb);
   const dim3 fgrid((unsigned)ceil_div(E * (M / 4), 256));
-  float* part = (float*)workspace;
   if (dtype == RTP_F32) {
     RTP_GATE_LAUNCH(gate_wgrad_partial_kernel, float, E, grid, st, dlogits, (long)ld_dlogits, (const float*)x, (long)ldx,
                     (long)S, (int)M, (int)E, part);
@@ -303,4 +295,79 @@ extern "C" int rtp_gate_wgrad(void* stream, int dtype, const float* dlogits, int
   }
   RTP_LAUNCH_CHECK();
   return RTP_OK;
+}
+
+static int gate_wgrad_check(const char* who, int dtype, const float* dlogits, int64_t ld_dlogits, const void* x,
+                            int64_t ldx, int64_t S, int64_t M, int64_t E, void* dw, int64_t ld_dw) {
+  if (int rc = gate_check(who, dtype, S, M, E)) return rc;
+  const int64_t vec = dtype == RTP_F32 ? 4 : 8;
+  RTP_REQUIRE(dlogits && x && dw, "%s: null pointer", who);
+  RTP_REQUIRE(aligned16(x) && ldx % vec == 0 && ldx >= M && ld_dw >= M && ld_dlogits >= E,
+              "%s: x must be 16-byte aligned, row pitches >= M (x: a multiple of %lld)", who, (long long)vec);
+  return RTP_OK;
+}
+
+extern "C" int rtp_gate_wgrad(void* stream, int dtype, const float* dlogits, int64_t ld_dlogits, const void* x,
+                              int64_t ldx, int64_t S, int64_t M, int64_t E, void* dw, int64_t ld_dw, int accumulate,
+                              void* workspace, size_t workspace_bytes) {
+  if (int rc = gate_wgrad_check("rtp_gate_wgrad", dtype, dlogits, ld_dlogits, x, ldx, S, M, E, dw, ld_dw)) return rc;
+  RTP_REQUIRE(workspace && aligned16(workspace), "rtp_gate_wgrad: the workspace must be a 16-byte aligned pointer");
+  RTP_REQUIRE(workspace_bytes >= rtp_gate_wgrad_workspace_bytes(S, M, E), "rtp_gate_wgrad: workspace of %zu bytes, need %zu",
+              workspace_bytes, rtp_gate_wgrad_workspace_bytes(S, M, E));
+  hipStream_t st = (hipStream_t)stream;
+  const double esz = dtype == RTP_F32 ? 4.0 : 2.0;
+  const long nrb = ceil_div(S, kGateWgradRows);
+  ProfileScope prof(st, "gate_wgrad", 2.0 * S * M * E, esz * ((double)S * M + (double)E * M) + 4.0 * S * E + 8.0 * nrb * E * M);
+  return gate_wgrad_launch(st, dtype, dlogits, ld_dlogits, x, ldx, S, M, E, dw, ld_dw, accumulate, (float*)workspace);
+}
+
+// ---- the same weight gradient for callers that cannot allocate -------------------------------------------------
+// The partial sums go to a buffer that is part of the library's code object instead of a caller's workspace.  In host
+// code the array's name is only a stand-in for the symbol: the device address of each GPU's own copy is asked for
+// once per device (with that device current) and kept; kernels and everything else only ever see that address.
+namespace rtp {
+constexpr size_t kGateStaticScratchBytes = RTP_GATE_WGRAD_STATIC_MAX_BYTES;
+static __device__ __align__(256) unsigned char gate_wgrad_scratch[kGateStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::mutex gate_scratch_mutex;
+static void* gate_scratch_ptr[kMaxDevices];  // per device, nullptr until resolved
+
+static int gate_scratch_for_current_device(float** out) {
+  int dev = -1;
+  RTP_HIP_TRY(hipGetDevice(&dev));
+  RTP_REQUIRE(dev >= 0 && dev < kMaxDevices, "rtp_gate_wgrad_static: device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(gate_scratch_mutex);
+  if (!gate_scratch_ptr[dev]) {
+    void* p = nullptr;
+    RTP_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(gate_wgrad_scratch)));
+    RTP_REQUIRE(p != nullptr, "rtp_gate_wgrad_static: the scratch symbol has no address on device %d", dev);
+    gate_scratch_ptr[dev] = p;
+  }
+  *out = (float*)gate_scratch_ptr[dev];
+  return RTP_OK;
+}
+
+// Called by rtp_device_check (the library's per-device set-up call) so that the address is known before a caller's
+// first rtp_gate_wgrad_static; that entry point resolves it itself on a device nobody checked.
+int gate_static_setup() {
+  float* p = nullptr;
+  return gate_scratch_for_current_device(&p);
+}
+
+}  // namespace rtp
+
+extern "C" int rtp_gate_wgrad_static(void* stream, int dtype, const float* dlogits, int64_t ld_dlogits, const void* x,
+                                     int64_t ldx, int64_t S, int64_t M, int64_t E, void* dw, int64_t ld_dw,
+                                     int accumulate) {
+  if (int rc = gate_wgrad_check("rtp_gate_wgrad_static", dtype, dlogits, ld_dlogits, x, ldx, S, M, E, dw, ld_dw))
+    return rc;
+  const size_t need = rtp_gate_wgrad_workspace_bytes(S, M, E);
+  RTP_REQUIRE(need <= kGateStaticScratchBytes,
+              "rtp_gate_wgrad_static: ceil(S / 64) * E * M * 4 = %zu bytes of partial sums exceed the built-in %zu; use "
+              "rtp_gate_wgrad with a workspace",
+              need, kGateStaticScratchBytes);
+  float* part = nullptr;
+  if (int rc = gate_scratch_for_current_device(&part)) return rc;
+  return gate_wgrad_launch((hipStream_t)stream, dtype, dlogits, ld_dlogits, x, ldx, S, M, E, dw, ld_dw, accumulate, part);
 }

@@ -149,7 +149,8 @@ extern "C" int rtp_device_check(char* name_out, int name_len) {
   }
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return fail(RTP_ERR_DEVICE, "device %d is %s; this library is built for gfx950 only", dev, prop.gcnArchName);
-  return RTP_OK;
+  // per-device set-up: the address of the built-in scratch of rtp_gate_wgrad_static on this device
+  return gate_static_setup();
 }
 
 extern "C" int rtp_ring_create(void** ring_out) {
