@@ -153,6 +153,15 @@ class ShardStore:
         if self.grads is not None:
             self._overwrite = set(range(self.world_size))
 
+    def settle_overwrite(self) -> None:
+        """Before an optimiser reads `grads`: a shard still marked for overwriting took no part in any backward since
+        zero_grad (a layer that was not used), so its row holds the previous step's gradient; torch would apply a
+        zero (or no) gradient, so the row is cleared."""
+        if self.grads is not None:
+            for s in sorted(self._overwrite):
+                self.grads[s].zero_()
+        self._overwrite.clear()
+
     def grad_runs(self, order: Sequence[int]):
         if self.on_backward is not None:
             self.on_backward(self)
@@ -201,7 +210,17 @@ class RotatedLayer(nn.Module):
     def _init_store(self, shard_modules: Sequence[nn.Module]) -> None:
         self.shards = nn.ModuleList(shard_modules)
         self._store = ShardStore(shard_modules)
+        self.register_load_state_dict_post_hook(RotatedLayer._after_load_state_dict)
         self._anchor = torch.zeros((), dtype=torch.float32, device=self._store.home.device, requires_grad=True)
+
+    @staticmethod
+    def _after_load_state_dict(module, incompatible_keys) -> None:
+        """load_state_dict copied new values into the home rows on the current stream: staged copies made from now
+        on must wait for that."""
+        home = module._store.home
+        if home is not None and home.is_cuda:
+            from .. import ring
+            ring.fence(home.device)
 
     def _apply(self, fn, recurse=True):
         super()._apply(fn, recurse)

@@ -177,6 +177,8 @@ class RotatedSGD:
     def step(self) -> None:
         if self.stores:
             ring.join_wgrad(self.stores[0].home.device)
+        for st in self.stores:
+            st.settle_overwrite()
         table = None if (self._early or self.overlap_backward) else self._multi_table()
         if table is not None:
             self._fold_other_grads()
@@ -260,6 +262,8 @@ class RotatedAdam(RotatedSGD):
     def step(self) -> None:
         if self.stores:
             ring.join_wgrad(self.stores[0].home.device)
+        for st in self.stores:
+            st.settle_overwrite()
         if self._step_dev is None:
             buffers = [st.home for st in self.stores] + ([self.flat] if self.flat is not None else [])
             if not buffers:

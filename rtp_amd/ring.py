@@ -86,6 +86,7 @@ def join_wgrad(device: Optional[torch.device] = None) -> None:
     second stream."""
     idx = torch.cuda.current_device() if device is None or device.index is None else device.index
     _flush_wgrad(idx)
+    _wgrad_task.pop(idx, None)
     if _wgrad_dirty.get(idx):
         torch.cuda.current_stream(idx).wait_stream(_wgrad_streams[idx])
         _wgrad_dirty[idx] = False
@@ -99,11 +100,27 @@ def _flush_wgrad(idx: int) -> None:
     aux = _wgrad_streams.get(idx)
     if aux is None:
         aux = _wgrad_streams[idx] = torch.cuda.Stream(device=idx)  # default priority
+        _install_optimizer_hooks()
     aux.wait_stream(torch.cuda.current_stream(idx))
+    _wgrad_dirty[idx] = True
     with torch.cuda.stream(aux):
         for fn in pending:
             fn()
     pending.clear()
+
+
+_wgrad_task: Dict[int, int] = {}  # device -> id of the backward pass whose end-of-pass join is armed
+
+
+def _abandon_wgrad(idx: int) -> None:
+    """A backward pass ended without its join (it raised part-way): what it deferred is dropped unlaunched -- its
+    gradients are incomplete anyway -- and what it already launched on the second stream is waited for."""
+    _wgrad_pending.get(idx, []).clear()
+    if _wgrad_dirty.get(idx):
+        torch.cuda.current_stream(idx).wait_stream(_wgrad_streams[idx])
+        _wgrad_dirty[idx] = False
+    _wgrad_keepalive.get(idx, []).clear()
+    _wgrad_task.pop(idx, None)
 
 
 def run_wgrad(device: torch.device, fn, tensors: Sequence[torch.Tensor] = ()) -> None:
@@ -111,21 +128,23 @@ def run_wgrad(device: torch.device, fn, tensors: Sequence[torch.Tensor] = ()) ->
     current stream.  With it: deferred until `_WGRAD_BATCH` layers have queued up (or the backward pass ends) and
     then on the second stream -- one fork of the compute stream per batch, since every fork and join between
     two hardware queues idles the compute stream for several microseconds.  `tensors` are the operands `fn`
-    reads that autograd may free or reuse when the layer's backward returns."""
-    if not _wgrad_overlap:
+    reads that autograd may free or reuse when the layer's backward returns.  The join at the end of the pass is
+    armed once per backward pass (by the id of the autograd engine's running task); outside a backward pass the
+    launches happen at once, on the current stream."""
+    task = torch._C._current_graph_task_id() if _wgrad_overlap else -1
+    if task < 0:
         fn()
         return
     idx = device.index if device.index is not None else torch.cuda.current_device()
+    if _wgrad_task.get(idx) != task:
+        if idx in _wgrad_task or _wgrad_pending.get(idx) or _wgrad_dirty.get(idx):
+            _abandon_wgrad(idx)  # leftovers of a pass that never reached its join
+        torch.autograd.Variable._execution_engine.queue_callback(lambda: join_wgrad(torch.device("cuda", idx)))
+        _wgrad_task[idx] = task
     # Hold the operands until the compute stream has rejoined: while a second reference exists autograd
     # neither frees a gradient buffer nor accumulates into it in place under the second stream's reads.
     _wgrad_keepalive.setdefault(idx, []).extend(t for t in tensors if t is not None)
     _wgrad_pending.setdefault(idx, []).append(fn)
-    if not _wgrad_dirty.get(idx):
-        _wgrad_dirty[idx] = True
-        try:  # rejoin when the running backward pass ends
-            torch.autograd.Variable._execution_engine.queue_callback(lambda: join_wgrad(torch.device("cuda", idx)))
-        except RuntimeError:
-            pass  # not inside a backward pass: the caller joins explicitly
     if len(_wgrad_pending[idx]) >= _WGRAD_BATCH:
         _flush_wgrad(idx)
 
@@ -194,6 +213,30 @@ class DeviceRing:
 
 
 _rings: Dict[int, DeviceRing] = {}
+_hooks_installed = False
+
+
+def _install_optimizer_hooks() -> None:
+    """Any torch.optim optimiser rewrites home shards in place: before its step the deferred weight gradients are
+    joined, after it every ring is fenced, so that the next staging copy is ordered after the update without the
+    caller having to know about the side stream (RotatedSGD / RotatedAdam do the same themselves)."""
+    global _hooks_installed
+    if _hooks_installed:
+        return
+    _hooks_installed = True
+    from torch.optim.optimizer import register_optimizer_step_post_hook, register_optimizer_step_pre_hook
+
+    def pre(optimizer, args, kwargs):
+        for idx in list(_wgrad_pending) + list(_wgrad_dirty):
+            join_wgrad(torch.device("cuda", idx))
+
+    def post(optimizer, args, kwargs):
+        for r in _rings.values():
+            with torch.cuda.device(r.device):
+                r.fence()
+
+    register_optimizer_step_pre_hook(pre)
+    register_optimizer_step_post_hook(post)
 
 
 def device_ring(device: torch.device) -> DeviceRing:
@@ -201,6 +244,7 @@ def device_ring(device: torch.device) -> DeviceRing:
     ring = _rings.get(idx)
     if ring is None:
         ring = _rings[idx] = DeviceRing(torch.device("cuda", idx))
+        _install_optimizer_hooks()
     return ring
 
 

@@ -4,7 +4,7 @@ import pytest
 import torch
 import torch.nn as nn
 
-from gpu_util import DEV, assert_close
+from gpu_util import DEV, assert_close, rel_err
 from oracle import rtp_oracle as O
 
 pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("rotation_window")]
@@ -154,3 +154,69 @@ def test_column_relu_mlp_matches_separate_modules(dtype, ws):
     for layer, r in ((l1, r1), (l2, r2)):
         assert_close(torch.cat([l.weight.grad for l in layer.linears], dim=0), r.weight.grad, dtype, "weight grad")
         assert_close(torch.cat([l.bias.grad for l in layer.linears], dim=0), r.bias.grad, dtype, "bias grad")
+
+
+def test_unused_layer_gets_no_stale_gradient_after_zero_grad():
+    """RotatedSGD.zero_grad keeps the gradient rows attached and lets the next backward overwrite them; a rotated
+    layer that takes no part in that backward must then be stepped with a zero gradient, not with last step's."""
+    from rtp_amd import emulate_shards
+    from rtp_amd.module.linear import ColumnParallelLinear
+    from rtp_amd.optim import RotatedSGD
+    with emulate_shards(2):
+        used = ColumnParallelLinear(8, 8, device=DEV)
+        idle = ColumnParallelLinear(8, 8, device=DEV)
+    model = nn.ModuleList([used, idle])
+    opt = RotatedSGD(model, lr=0.5)
+    x = torch.randn(4, 8, device=DEV)
+    (used(x).sum() + idle(x).sum()).backward()
+    opt.step()
+    w_idle = torch.cat([l.weight.detach().clone() for l in idle.linears], 0)
+    w_used = torch.cat([l.weight.detach().clone() for l in used.linears], 0)
+    opt.zero_grad()
+    used(x).sum().backward()       # `idle` is not part of this step
+    opt.step()
+    torch.cuda.synchronize()
+    assert torch.equal(torch.cat([l.weight.detach() for l in idle.linears], 0), w_idle)
+    assert not torch.equal(torch.cat([l.weight.detach() for l in used.linears], 0), w_used)
+
+
+def test_backward_that_raises_leaves_no_deferred_weight_gradients_behind():
+    """With weight gradients deferred to the second stream, a backward pass that raises part-way never reaches its
+    end-of-pass join; the next pass must not launch the dead pass's closures nor skip its own join."""
+    from rtp_amd import emulate_shards, ring
+    from rtp_amd.module.linear import ColumnParallelLinear
+
+    class Boom(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, x):
+            return x.clone()
+
+        @staticmethod
+        def backward(ctx, g):
+            raise ValueError("boom")
+
+    with emulate_shards(2):
+        a = ColumnParallelLinear(8, 8, device=DEV)
+        b = ColumnParallelLinear(8, 8, device=DEV)
+    x = torch.randn(4, 8, device=DEV)
+    ring.set_wgrad_overlap(True)
+    try:
+        with pytest.raises(ValueError, match="boom"):
+            b(Boom.apply(a(x))).sum().backward()     # b's backward defers its gradients, then the pass dies
+        for l in a.linears + b.linears:
+            l.weight.grad = l.bias.grad = None
+        x2 = torch.randn(4, 8, device=DEV)
+        b(a(x2)).sum().backward()
+        torch.cuda.synchronize()
+        assert not ring._wgrad_pending.get(0) and not ring._wgrad_dirty.get(0) and 0 not in ring._wgrad_task
+        wa = torch.cat([l.weight.detach() for l in a.linears], 0)
+        ba = torch.cat([l.bias.detach() for l in a.linears], 0)
+        wb = torch.cat([l.weight.detach() for l in b.linears], 0)
+        h = x2 @ wa.T + ba
+        want_b = torch.ones(4, 8, device=DEV).T @ h
+        got_b = torch.cat([l.weight.grad for l in b.linears], 0)
+        assert rel_err(got_b, want_b) <= 1e-5
+        want_a = (torch.ones(4, 8, device=DEV) @ wb).T @ x2
+        assert rel_err(torch.cat([l.weight.grad for l in a.linears], 0), want_a) <= 1e-5
+    finally:
+        ring.set_wgrad_overlap(False)

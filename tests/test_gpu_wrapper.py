@@ -93,3 +93,60 @@ def test_wrapper_on_stock_transformer_decoder_layer():
     m = model.module
     assert_close(O.attention_grad_reinterleave([s.in_proj_weight.grad for s in m.multihead_attn.module_list], 4),
                  ref.multihead_attn.in_proj_weight.grad, torch.float32, "memory attention in_proj")
+
+
+@pytest.mark.parametrize("overlap", [False, True])
+def test_wrapped_model_trains_with_a_stock_optimizer(overlap):
+    """Three steps of torch.optim.SGD + clip_grad_value_ on model.parameters() (what the reference harness does,
+    benchmarks/rtp_benchmark.py:185-186) against the untouched copy on the CPU: nobody calls ring.fence() or
+    join_wgrad() here, the optimiser hooks order the staging copies and the second-stream weight gradients."""
+    from rtp_amd import emulate_shards, ring
+    from rtp_amd.rotated_tensor_parallel import RotatedTensorParallel
+    class ColumnNet(nn.Module):
+        """Only layers whose shards partition the parameters: a row-parallel bias (and the attention's output bias)
+        is held as bias/ws by every shard and each copy receives the whole gradient (rtp/module/linear.py:133-135),
+        so after an optimiser step such a model no longer equals its unsharded twin -- in the reference as here."""
+
+        def __init__(self):
+            super().__init__()
+            self.emb = nn.Embedding(40, 16)
+            self.norm = nn.LayerNorm(16)
+            self.fc1 = nn.Linear(16, 24)
+            self.fc2 = nn.Linear(24, 8)
+
+        def forward(self, ids):
+            return self.fc2(torch.relu(self.fc1(self.norm(self.emb(ids)))))
+
+    ws = 4
+    torch.manual_seed(3)
+    ref = ColumnNet()
+    with emulate_shards(ws):
+        model = RotatedTensorParallel(copy.deepcopy(ref)).to(DEV)
+    assert [type(w.rotated).__name__ for w in model.FlyweightModule_list] == \
+        ["ParallelEmbedding", "ColumnParallelLinear", "ColumnParallelLinear"]
+    opt = torch.optim.SGD(model.parameters(), lr=0.1)
+    ref_opt = torch.optim.SGD(ref.parameters(), lr=0.1)
+    gen = torch.Generator().manual_seed(5)
+    ring.set_wgrad_overlap(overlap)
+    try:
+        for step in range(3):
+            ids = torch.randint(0, 40, (7, 3), generator=gen)
+            g = torch.randn(7, 3, 8, generator=gen)
+            big = torch.randn(2048, 2048, device=DEV)
+            (big @ big).sum()  # the compute stream is busy when the step starts: the side stream runs ahead of it
+            opt.zero_grad()
+            out = model(ids.to(DEV))
+            out.backward(g.to(DEV))
+            torch.nn.utils.clip_grad_value_(model.parameters(), 0.05)
+            opt.step()
+            ref_opt.zero_grad()
+            ref_out = ref(ids)
+            ref_out.backward(g)
+            torch.nn.utils.clip_grad_value_(ref.parameters(), 0.05)
+            ref_opt.step()
+            assert_close(out, ref_out, torch.float32, f"step {step} output")
+    finally:
+        ring.set_wgrad_overlap(False)
+    m = model.module
+    assert_close(torch.cat([s.weight for s in m.fc1.module_list], 0), ref.fc1.weight, torch.float32, "fc1 after 3 steps")
+    assert_close(torch.cat([s.weight for s in m.emb.module_list], 1), ref.emb.weight, torch.float32, "emb after 3 steps")
