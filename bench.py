@@ -6,9 +6,11 @@ MI355X, bf16 weights with fp32 master, 8 rotation shards emulated on the device,
     python bench.py --gpus 1 --steps K --warmup W
 
 Prints one JSON line.  `value` is tokens/s over K timed steps with inputs resident in HBM.  `roofline`
-is the dominant kernel of the step (by summed duration), timed per launch with HIP events on the stream
-it runs on, during extra profiled steps that follow the timed region (so the events do not perturb
-`value`).  `cpu_baseline` is the CPU oracle (stock torch layers, fp32) timed on this box's host cores.
+is the dominant kernel of the step (the GEMM variant with the largest summed duration), timed per launch in
+the timed mode itself: the step is captured once more with every GEMM launch carrying a device time-stamp
+slot and replayed after the timed region (so the stamps do not perturb `value`).  `kernels` lists every
+kernel of the library timed with HIP events on two further eager steps.  `cpu_baseline` is the CPU oracle
+(stock torch layers, fp32) timed on this box's host cores.
 """
 import argparse
 import json
@@ -58,9 +60,10 @@ def build(c, device, dtype):
     return lm
 
 
-def cpu_baseline(c, steps=2):
+def cpu_baseline(c, steps=5, warmup=2):
     """The oracle LM (stock nn.Embedding / nn.MultiheadAttention / nn.Linear / nn.LayerNorm, fp32) on the host
-    cores: same shapes, same step (zero grads, fwd, CE, bwd, clip, SGD)."""
+    cores: same shapes, same step (zero grads, fwd, CE, bwd, clip, SGD).  It is the UNSHARDED stock model, which
+    does the same arithmetic as the reference's shard loop without its per-shard launches and concatenations."""
     import torch
     import torch.nn.functional as F
     from oracle import rtp_oracle as O
@@ -83,14 +86,17 @@ def cpu_baseline(c, steps=2):
             for p in ref.parameters():
                 p.add_(p.grad.clamp_(-0.05, 0.05), alpha=-1e-3)
 
-    one()
-    t0 = time.perf_counter()
-    for _ in range(steps):
+    for _ in range(warmup):
         one()
-    dt = (time.perf_counter() - t0) / steps
+    times = []
+    for _ in range(steps):
+        t0 = time.perf_counter()
+        one()
+        times.append(time.perf_counter() - t0)
+    dt = sorted(times)[len(times) // 2]
     return {"value": c["seq"] * c["batch"] / dt, "unit": "tokens/s", "cores": torch.get_num_threads(),
-            "kind": "port", "sample": f"{steps} full steps of the same configuration in fp32 after 1 warm-up "
-            f"({dt * 1e3:.0f} ms/step, os.cpu_count()={os.cpu_count()})"}
+            "kind": "port", "sample": f"median of {steps} full steps of the same configuration after {warmup} warm-ups, "
+            f"fp32, unsharded stock model ({dt * 1e3:.0f} ms/step, os.cpu_count()={os.cpu_count()})"}
 
 
 def _time_cpu(one, steps):
@@ -138,9 +144,26 @@ def attainable_peaks(dev):
 
     t_gemm = timed(gemm, 10)
     t_copy = timed(lambda: ops.shard_copy(dst, src), 5)
-    return {"gemm_bf16_4096_cubed_tflops": 2.0 * n ** 3 / t_gemm / 1e12,
-            "device_copy_1GiB_gbs": 2.0 * src.numel() / t_copy / 1e9,
-            "note": "same GEMM kernel / the shard-copy kernel, run alone on this GPU; copy counts bytes read + written"}
+    out = {"gemm_bf16_4096_cubed_tflops": 2.0 * n ** 3 / t_gemm / 1e12,
+           "device_copy_1GiB_gbs": 2.0 * src.numel() / t_copy / 1e9,
+           "note": "same GEMM kernel / the shard-copy kernel, run alone on this GPU; copy counts bytes read + written"}
+    del src, dst
+    # Yardstick outside the product path: the vendor library (torch.matmul -> hipBLASLt) on the same random data,
+    # for the large product and for the LM's per-layer shapes, beside this library's own time for each.
+    yard = {}
+    for (m_, n_, k_) in ((4096, 4096, 4096), (1024, 2048, 2048), (1024, 6144, 2048), (1024, 10240, 2048)):
+        x = torch.randn(m_, k_, generator=gen).to(torch.bfloat16).to(dev)
+        w = torch.randn(n_, k_, generator=gen).to(torch.bfloat16).to(dev)
+        y = torch.empty(m_, n_, dtype=torch.bfloat16, device=dev)
+        wt = w.t()
+        t_lib = timed(lambda: ops.gemm_raw(torch.bfloat16, a=x.data_ptr(), b=w.data_ptr(), c_out=y.data_ptr(), m=m_, n=n_,
+                                           k=k_, lda=k_, ldb=k_, ldc=n_, a_kcontig=True, b_kcontig=True), 20)
+        t_ven = timed(lambda: torch.matmul(x, wt, out=y), 20)
+        fl = 2.0 * m_ * n_ * k_
+        yard[f"{m_}x{n_}x{k_}"] = {"this_library_us": t_lib * 1e6, "this_library_tflops": fl / t_lib / 1e12,
+                                   "torch_matmul_us": t_ven * 1e6, "torch_matmul_tflops": fl / t_ven / 1e12}
+    out["yardstick_torch_matmul_same_data"] = yard
+    return out
 
 
 def layer_workload(name, steps, warmup, graph=True, cpu=True):
@@ -436,7 +459,39 @@ def main():
     dt = (time.perf_counter() - t0) / args.steps
     last_loss = float(loss_box[0])
 
-    # Per-kernel timing with HIP events around every launch, on two extra eager steps.
+    # The dominant kernel in the TIMED mode (graph replay, both streams live): the step is captured a second time
+    # with the GEMM launches carrying device time-stamp slots (HIP timing events do not work inside a replayed
+    # graph), replayed, and the per-launch durations read back after every replay.
+    graph_stats, instr_ms = None, None
+    if args.graph:
+        _lib.profile_enable(2)
+        g2 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g2):
+            step()
+        ring.fence(dev)
+        _lib.profile_enable(0)
+        stream = torch.cuda.current_stream().cuda_stream
+        g2.replay()
+        torch.cuda.synchronize()
+        reps, graph_stats = 5, {}
+        t_i = 0.0
+        for _ in range(reps):
+            _lib.profile_reset_stamps(stream)
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            g2.replay()
+            torch.cuda.synchronize()
+            t_i += time.perf_counter() - t1
+            for k, v in _lib.profile_collect(clear=False).items():
+                acc = graph_stats.setdefault(k, {"launches": 0, "total_ms": 0.0, "flops": 0.0, "bytes": 0.0})
+                for f in acc:
+                    acc[f] += v[f]
+        instr_ms = t_i / reps * 1e3
+        _lib.profile_collect()
+        del g2
+
+    # Per-kernel timing with HIP events around every launch, on two extra EAGER steps (every kernel of the library,
+    # but launched from Python: the second stream is mostly idle then, so these are not the timed mode's durations).
     _lib.profile_enable(True)
     prof_steps = 2
     for _ in range(prof_steps):
@@ -444,15 +499,21 @@ def main():
     stats = _lib.profile_collect()
     _lib.profile_enable(False)
     gemms = {k: v for k, v in stats.items() if k.startswith("gemm_")}
-    dom_name, dom = max(gemms.items(), key=lambda kv: kv[1]["total_ms"])
+    timed_gemms = {k: v for k, v in (graph_stats or stats).items() if k.startswith("gemm_")}
+    dom_name, dom = max(timed_gemms.items(), key=lambda kv: kv[1]["total_ms"])
     avg_ms = dom["total_ms"] / dom["launches"]
     achieved = dom["flops"] / dom["launches"] / (avg_ms * 1e-3) / 1e12
+    eager = gemms[dom_name]
+    achieved_eager = eager["flops"] / eager["total_ms"] / 1e9
     all_gemm_ms = sum(v["total_ms"] for v in gemms.values()) / prof_steps
     all_gemm_tflops = sum(v["flops"] for v in gemms.values()) / prof_steps / (all_gemm_ms * 1e-3) / 1e12
     copy = stats.get("shard_copy")
     kernels = {k: {"launches_per_step": v["launches"] // prof_steps, "ms_per_step": round(v["total_ms"] / prof_steps, 4),
                    "tflops": round(v["flops"] / max(v["total_ms"], 1e-9) / 1e9, 2),
                    "gbs": round(v["bytes"] / max(v["total_ms"], 1e-9) / 1e6, 1)} for k, v in sorted(stats.items())}
+    graph_gemms = None if graph_stats is None else {
+        k: {"launches_per_step": v["launches"] // 5, "avg_launch_us": round(v["total_ms"] / v["launches"] * 1e3, 3),
+            "tflops": round(v["flops"] / max(v["total_ms"], 1e-9) / 1e9, 2)} for k, v in sorted(graph_stats.items())}
 
     flops = step_flops(c)
     peaks = attainable_peaks(dev)
@@ -473,8 +534,14 @@ def main():
                      "traffic": (MEASURED_TRAFFIC_KIB[dom_name] * 1024.0 if dom_name in MEASURED_TRAFFIC_KIB else None),
                      "traffic_unit": "bytes per launch (counter runs, see profiles/)",
                      "algorithmic_bytes_per_launch": dom["bytes"] / dom["launches"], "kernel": dom_name,
-                     "avg_launch_us": avg_ms * 1e3, "launches_per_step": dom["launches"] // prof_steps,
-                     "flops_per_launch": dom["flops"] / dom["launches"]},
+                     "avg_launch_us": avg_ms * 1e3,
+                     "launches_per_step": dom["launches"] // (5 if graph_stats is not None else prof_steps),
+                     "flops_per_launch": dom["flops"] / dom["launches"],
+                     "timed_in": ("HIP-graph replay of the step, both streams live, device time stamps per launch"
+                                  if graph_stats is not None else "eager launches, HIP events"),
+                     "frac_standalone_eager": achieved_eager / PEAK["bf16_mfma_tflops"],
+                     "instrumented_replay_ms_per_step": instr_ms},
+        "gemm_kernels_in_graph_replay": graph_gemms,
         "measured_attainable": dict(peaks, dominant_kernel_frac_of_measured_gemm=achieved / peaks["gemm_bf16_4096_cubed_tflops"]),
         "step_mfma_frac": flops / dt / (PEAK["bf16_mfma_tflops"] * 1e12),
         "step_algorithmic_tflop": flops / 1e12,

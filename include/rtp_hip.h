@@ -503,8 +503,11 @@ int rtp_cast(void* stream, int dtype_src, const void* src, int dtype_dst, void* 
  * library is bracketed by two HIP timing events on the stream it is launched on and booked under
  * its kernel-variant name with the algorithmic flops and bytes of that launch.  rtp_profile_collect
  * synchronises the device, sums the event durations per name into `out` (at most `max_out`
- * entries, *n_out receives the count) and clears the records.  Must be off while a stream is being
- * captured into a HIP graph.
+ * entries, *n_out receives the count) and clears the records.  rtp_profile_read does the same without
+ * clearing them.  Profiling may be on while a stream is captured into a HIP graph: the events then become
+ * nodes of that graph, every replay stamps them again, and rtp_profile_read after a replay returns the
+ * durations of that replay -- per-kernel times of the graph-replayed schedule, all streams live.  Call
+ * rtp_profile_collect only when the graph will not be replayed again (it destroys the events).
  * --------------------------------------------------------------------------------------------- */
 typedef struct {
   char name[64];
@@ -514,8 +517,15 @@ typedef struct {
   double bytes; /* algorithmic, summed over launches */
 } rtp_kernel_stat;
 
-int rtp_profile_enable(int on);
+int rtp_profile_enable(int mode); /* 0 off, 1 HIP events around every launch, 2 device time stamps (see below) */
+/* Mode 2 is for launches recorded into a HIP graph, where timing events do not work: every rtp_gemm launch made
+ * while it is on carries the address of a two-word slot in device memory, where its workgroups leave the earliest
+ * start and the latest end of the device's constant-rate wall clock, at every replay.  rtp_profile_reset_stamps
+ * (a small kernel on `stream`) clears the slots before a replay; rtp_profile_read after it returns that replay's
+ * durations per kernel variant.  Other kernels are not timed in this mode. */
+int rtp_profile_reset_stamps(void* stream);
 int rtp_profile_collect(rtp_kernel_stat* out, int max_out, int* n_out);
+int rtp_profile_read(rtp_kernel_stat* out, int max_out, int* n_out);
 
 #ifdef __cplusplus
 }

@@ -132,6 +132,8 @@ PROTOTYPES = {
     "rtp_cast": (_i, [_vp, _i, _vp, _i, _vp, _i64]),
     "rtp_profile_enable": (_i, [_i]),
     "rtp_profile_collect": (_i, [C.POINTER(KernelStat), _i, C.POINTER(_i)]),
+    "rtp_profile_reset_stamps": (_i, [_vp]),
+    "rtp_profile_read": (_i, [C.POINTER(KernelStat), _i, C.POINTER(_i)]),
 }
 
 _lib: Optional[C.CDLL] = None
@@ -175,14 +177,22 @@ def require_device() -> None:
         _device_checked = True
 
 
-def profile_enable(on: bool) -> None:
+def profile_enable(on) -> None:
+    """False / 0: off; True / 1: HIP events around every launch; 2: device time stamps in the GEMM kernels (the mode
+    that works for launches recorded into a HIP graph)."""
     check(load().rtp_profile_enable(int(on)))
 
 
-def profile_collect():
-    """{kernel variant: {launches, total_ms, flops, bytes}} since profiling was enabled; clears the records."""
+def profile_reset_stamps(stream: int) -> None:
+    check(load().rtp_profile_reset_stamps(stream))
+
+
+def profile_collect(clear: bool = True):
+    """{kernel variant: {launches, total_ms, flops, bytes}} since profiling was enabled; clears the records unless
+    clear=False (events recorded into a captured graph stay valid for its later replays)."""
     buf = (KernelStat * 64)()
     n = C.c_int(0)
-    check(load().rtp_profile_collect(buf, 64, C.byref(n)))
+    lib = load()
+    check((lib.rtp_profile_collect if clear else lib.rtp_profile_read)(buf, 64, C.byref(n)))
     return {buf[i].name.decode(): {"launches": buf[i].launches, "total_ms": buf[i].total_ms, "flops": buf[i].flops,
                                    "bytes": buf[i].bytes} for i in range(n.value)}

@@ -126,6 +126,9 @@ __device__ __forceinline__ void touch_kernel_arguments() {
 struct ProfileScope {
   ProfileScope(hipStream_t stream, const char* name, double flops, double bytes);
   ~ProfileScope();
+  // With device time stamps switched on (rtp_profile_enable(2)): books this launch and returns the address of its
+  // two-word stamp slot for the kernel to fill (earliest start, latest end of the wall clock); otherwise null.
+  unsigned long long* trace_slot();
   ProfileScope(const ProfileScope&) = delete;
   ProfileScope& operator=(const ProfileScope&) = delete;
 

@@ -73,6 +73,7 @@ struct GemmArgs {
   FastDiv d_batch, d_zdiv, d_tiles_n, d_brick, d_panel, d_prow, d_pm;  // divisors mbk*nbk, prow*pcol, prow, mbk/prow
   int mbk, nbk, prow, pcol;
   int xn_shift, xm_shift, zbk;  // log2 of xn and xm, batch*groups entries per brick
+  unsigned long long* trace;    // null, or two words: earliest start / latest end of the launch on the wall clock
 };
 
 constexpr int kThreads = 256;
@@ -713,6 +714,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
 
   touch_kernel_arguments<sizeof(GemmArgs)>();
   const int tid = threadIdx.x;
+  if (p.trace != nullptr && tid == 0) atomicMin(p.trace, (unsigned long long)wall_clock64());
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = (wave >> 1) & 1, wn = wave & 1;
@@ -939,6 +941,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   }
   __syncthreads();
   finish_tile<T, BM, BN, 512>(p, ct, m0, n0, tid, grp, zo, zi);
+  if (p.trace != nullptr && tid == 0) atomicMax(p.trace + 1, (unsigned long long)wall_clock64());
 }
 
 template <typename T, int BM, int BN, int NSTAGE, int SB, int PD>
@@ -1127,6 +1130,7 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   const int64_t nz = d->batch * d->groups;
   a.a_rowsum = (char*)d->a_rowsum;
   a.rowsum_sg = d->rowsum_sg;
+  a.trace = nullptr;
   RTP_REQUIRE(!d->a_rowsum || rowsum_fused<T>(d),
               "rtp_gemm: a_rowsum needs A stored K x M, batch == 1 and vector-aligned operands (rtp_gemm_rowsum_fused)");
   if (is_tiny(d)) {
@@ -1248,6 +1252,7 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   const double cin_sz = d->c_in ? ((d->flags & RTP_GEMM_CIN_F32) ? 4.0 : (double)sizeof(T)) : 0.0;
   const double bytes = ((double)d->m + (double)d->n) * kk * nz * sizeof(T) + mn * (out_sz + cin_sz);
   ProfileScope prof(s, name, 2.0 * mn * kk, bytes);
+  a.trace = fast ? prof.trace_slot() : nullptr;
   if (!fast) return launch_layout<T, 64, 64, 1, false>(s, a, akc, bkc, grid);
   switch (shape) {
     case 0:

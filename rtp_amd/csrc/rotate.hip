@@ -16,17 +16,25 @@ char* error_buffer() {
 }
 
 struct ProfileRecord {
-  hipEvent_t start, stop;
+  hipEvent_t start, stop;  // host-recorded timing events, or null when the launch stamps a device slot
+  int slot;                // index into the device stamp buffer, or -1
   const char* name;
   double flops, bytes;
 };
 static std::mutex g_profile_mutex;
-static bool g_profile_on = false;
+static int g_profile_mode = 0;  // 0 off, 1 HIP events around every launch, 2 device time stamps (GEMM kernels)
 static std::vector<ProfileRecord> g_profile_records;
+// Mode 2: a launch that supports it receives a slot of two 64-bit words in device memory; its first workgroup to
+// start stores the earliest value of the constant-rate wall clock there (atomic min), its last to end the latest
+// (atomic max).  The slot address is a kernel argument, so a launch recorded into a HIP graph stamps its slot at
+// every replay -- which HIP timing events recorded during a capture do not do.
+constexpr int kTraceSlots = 8192;
+static unsigned long long* g_trace_buf = nullptr;
+static int g_trace_next = 0;
 
 ProfileScope::ProfileScope(hipStream_t stream, const char* name, double flops, double bytes)
     : stream_(stream), name_(name), flops_(flops), bytes_(bytes) {
-  if (!g_profile_on) return;
+  if (g_profile_mode != 1) return;
   if (hipEventCreate(&start_) != hipSuccess) {
     start_ = nullptr;
     return;
@@ -43,7 +51,24 @@ ProfileScope::~ProfileScope() {
   }
   (void)hipEventRecord(stop, stream_);
   std::lock_guard<std::mutex> lock(g_profile_mutex);
-  g_profile_records.push_back({start_, stop, name_, flops_, bytes_});
+  g_profile_records.push_back({start_, stop, -1, name_, flops_, bytes_});
+}
+
+unsigned long long* ProfileScope::trace_slot() {
+  if (g_profile_mode != 2) return nullptr;
+  std::lock_guard<std::mutex> lock(g_profile_mutex);
+  if (!g_trace_buf || g_trace_next >= kTraceSlots) return nullptr;
+  const int slot = g_trace_next++;
+  g_profile_records.push_back({nullptr, nullptr, slot, name_, flops_, bytes_});
+  return g_trace_buf + 2 * (size_t)slot;
+}
+
+__global__ void trace_reset_kernel(unsigned long long* buf, int slots) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < slots) {
+    buf[2 * i] = ~0ull;
+    buf[2 * i + 1] = 0ull;
+  }
 }
 
 struct Ring {
@@ -252,22 +277,59 @@ extern "C" int rtp_zero_async(void* stream, void* dst, size_t bytes) {
   return RTP_OK;
 }
 
-extern "C" int rtp_profile_enable(int on) {
+extern "C" int rtp_profile_enable(int mode) {
+  RTP_REQUIRE(mode >= 0 && mode <= 2, "rtp_profile_enable: mode 0 (off), 1 (events) or 2 (device time stamps)");
   std::lock_guard<std::mutex> lock(g_profile_mutex);
-  g_profile_on = on != 0;
+  if (mode == 2 && !g_trace_buf) {
+    RTP_HIP_TRY(hipMalloc((void**)&g_trace_buf, sizeof(unsigned long long) * 2 * kTraceSlots));
+    hipLaunchKernelGGL(trace_reset_kernel, dim3((kTraceSlots + 255) / 256), dim3(256), 0, nullptr, g_trace_buf, kTraceSlots);
+    RTP_LAUNCH_CHECK();
+    RTP_HIP_TRY(hipDeviceSynchronize());
+  }
+  g_profile_mode = mode;
   return RTP_OK;
 }
 
-extern "C" int rtp_profile_collect(rtp_kernel_stat* out, int max_out, int* n_out) {
+extern "C" int rtp_profile_reset_stamps(void* stream) {
+  std::lock_guard<std::mutex> lock(g_profile_mutex);
+  if (!g_trace_buf || g_trace_next == 0) return RTP_OK;
+  hipLaunchKernelGGL(trace_reset_kernel, dim3((g_trace_next + 255) / 256), dim3(256), 0, (hipStream_t)stream, g_trace_buf,
+                     g_trace_next);
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
+}
+
+// Sums the recorded launches per kernel name.  `clear`: destroy the event pairs afterwards.  Without it they stay
+// valid -- what a HIP graph needs whose capture recorded them as event nodes: every replay stamps them anew, and a
+// read after a replay returns that replay's durations.
+static int profile_sum(rtp_kernel_stat* out, int max_out, int* n_out, bool clear) {
   RTP_REQUIRE(out && n_out && max_out > 0, "rtp_profile_collect: bad arguments");
   RTP_HIP_TRY(hipDeviceSynchronize());
   std::lock_guard<std::mutex> lock(g_profile_mutex);
+  std::vector<unsigned long long> stamps;
+  double ticks_per_ms = 1e5;  // the wall clock runs at 100 MHz unless the device says otherwise
+  if (g_trace_buf && g_trace_next > 0) {
+    stamps.resize(2 * (size_t)g_trace_next);
+    RTP_HIP_TRY(hipMemcpy(stamps.data(), g_trace_buf, stamps.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost));
+    int dev = 0, khz = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) == hipSuccess && khz > 0)
+      ticks_per_ms = (double)khz;
+  }
   std::map<std::string, rtp_kernel_stat> agg;
   for (const ProfileRecord& r : g_profile_records) {
     float ms = 0.0f;
-    if (hipEventElapsedTime(&ms, r.start, r.stop) != hipSuccess) ms = 0.0f;
-    (void)hipEventDestroy(r.start);
-    (void)hipEventDestroy(r.stop);
+    if (r.slot >= 0) {
+      const unsigned long long t0 = stamps[2 * (size_t)r.slot], t1 = stamps[2 * (size_t)r.slot + 1];
+      if (t1 < t0) continue;  // the launch did not run since the last reset
+      ms = (float)((double)(t1 - t0) / ticks_per_ms);
+    } else {
+      if (hipEventElapsedTime(&ms, r.start, r.stop) != hipSuccess) ms = 0.0f;
+      if (clear) {
+        (void)hipEventDestroy(r.start);
+        (void)hipEventDestroy(r.stop);
+      }
+    }
     rtp_kernel_stat& st = agg[r.name];
     if (st.launches == 0) {
       memset(&st, 0, sizeof(st));
@@ -278,7 +340,10 @@ extern "C" int rtp_profile_collect(rtp_kernel_stat* out, int max_out, int* n_out
     st.flops += r.flops;
     st.bytes += r.bytes;
   }
-  g_profile_records.clear();
+  if (clear) {
+    g_profile_records.clear();
+    g_trace_next = 0;
+  }
   int n = 0;
   for (auto& kv : agg) {
     if (n >= max_out) break;
@@ -286,4 +351,12 @@ extern "C" int rtp_profile_collect(rtp_kernel_stat* out, int max_out, int* n_out
   }
   *n_out = n;
   return RTP_OK;
+}
+
+extern "C" int rtp_profile_collect(rtp_kernel_stat* out, int max_out, int* n_out) {
+  return profile_sum(out, max_out, n_out, true);
+}
+
+extern "C" int rtp_profile_read(rtp_kernel_stat* out, int max_out, int* n_out) {
+  return profile_sum(out, max_out, n_out, false);
 }
