@@ -376,6 +376,10 @@ def main():
     ap.add_argument("--sgd-overlap", dest="sgd_overlap", action="store_true",
                     help="apply each rotated layer's SGD update right after that layer's backward, on a second stream "
                          "(measured: no gain, the update and the backward compete for memory bandwidth)")
+    ap.add_argument("--no-sgd-fused", dest="sgd_fused", action="store_false",
+                    help="one clip + SGD launch over all parameters after the backward pass, instead of applying the "
+                         "update of every weight matrix in the epilogue of its weight-gradient product (the default: "
+                         "bit-identical weights, the gradients of those matrices are never written or read back)")
     ap.add_argument("--no-wgrad-overlap", dest="wgrad_overlap", action="store_false",
                     help="launch weight / bias gradient kernels on the compute stream instead of a second stream "
                          "beside the input-gradient chain")
@@ -413,7 +417,8 @@ def main():
     if args.optimizer == "adam":
         opt = RotatedAdam(lm, lr=1e-3, clip_value=0.05)
     else:
-        opt = RotatedSGD(lm, lr=1e-3, clip_value=0.05, overlap_backward=args.sgd_overlap)
+        opt = RotatedSGD(lm, lr=1e-3, clip_value=0.05, overlap_backward=args.sgd_overlap,
+                         fused_backward=args.sgd_fused and not args.sgd_overlap)
     gen = torch.Generator().manual_seed(0)
     ids = torch.randint(0, c["vocab"], (c["seq"], c["batch"]), generator=gen).to(dev)
     tgt = torch.randint(0, c["vocab"], (c["seq"], c["batch"]), generator=gen).to(dev)
@@ -528,6 +533,7 @@ def main():
                    "tokens_per_step": tokens, "rotation_shards": c["shards"], "hip_graph": bool(args.graph),
                    "optimizer": args.optimizer, "rotation": args.rotation,
                    "sgd_overlapped_with_backward": bool(args.sgd_overlap),
+                   "sgd_fused_into_weight_gradient_products": bool(args.sgd_fused),
                    "wgrad_on_second_stream": bool(args.wgrad_overlap)},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK["bf16_mfma_tflops"], "unit": "TFLOP/s",
                      "frac": achieved / PEAK["bf16_mfma_tflops"],

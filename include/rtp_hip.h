@@ -90,7 +90,8 @@ enum {
   RTP_GEMM_CIN_F32 = 2,
   RTP_GEMM_RELU = 4,
   RTP_GEMM_STREAM_OUT = 8, /* c_out is not read again soon (weight gradients): non-temporal stores */
-  RTP_GEMM_ROWSUM_ACCUM = 16 /* a_rowsum is added to, not overwritten */
+  RTP_GEMM_ROWSUM_ACCUM = 16, /* a_rowsum is added to, not overwritten */
+  RTP_GEMM_SGD_SKIP_OUT = 32  /* with sgd_master: the product is consumed by the update, c_out is not written */
 };
 
 typedef struct {
@@ -112,12 +113,27 @@ typedef struct {
   int32_t a_kcontig, b_kcontig;
   void* a_rowsum;    /* may be NULL; length M per group */
   int64_t rowsum_sg; /* per-group element stride of a_rowsum */
+  /* Clip + SGD applied to the product where it is produced (a weight-gradient product whose result would only be
+   * read once more, by the optimiser: benchmarks/rtp_benchmark.py:185-186).  sgd_master (may be NULL: no update) is
+   * the fp32 parameter buffer, sgd_weights (may be NULL) the `dtype` copy of it that the layers read; both are
+   * indexed exactly like c_out (ldc, c_so, c_si, c_sg).  Per element: g = the product rounded to `dtype` (what
+   * c_out receives), clamped to +-sgd_clip if sgd_clip > 0; master -= sgd_lr * g (product and difference rounded
+   * separately, as rtp_sgd_step does); weights = master rounded to `dtype`.  Results are bit-identical to rtp_gemm
+   * followed by rtp_sgd_step.  Needs vector-aligned operands, an output in `dtype` and a plain epilogue (no c_in,
+   * bias, ReLU or gate); ask rtp_gemm_sgd_fused whether a descriptor qualifies. */
+  void* sgd_master;
+  void* sgd_weights;
+  float sgd_lr, sgd_clip;
 } rtp_gemm_desc;
 
 int rtp_gemm(void* stream, int dtype, const rtp_gemm_desc* d);
 
 /* 1 if rtp_gemm would produce d->a_rowsum for this descriptor (the pointer itself may still be NULL), else 0. */
 int rtp_gemm_rowsum_fused(int dtype, const rtp_gemm_desc* d);
+
+/* 1 if rtp_gemm would apply the fused update (sgd_master, sgd_weights) for this descriptor, else 0 (rtp_gemm then
+ * refuses a descriptor that asks for it). */
+int rtp_gemm_sgd_fused(int dtype, const rtp_gemm_desc* d);
 
 /* sizeof(rtp_gemm_desc) as this library was compiled: lets a binding verify its struct layout. */
 size_t rtp_gemm_desc_size(void);

@@ -21,6 +21,7 @@ GEMM_CIN_F32 = 2
 GEMM_RELU = 4
 GEMM_STREAM_OUT = 8
 GEMM_ROWSUM_ACCUM = 16
+GEMM_SGD_SKIP_OUT = 32
 GATE_WGRAD_STATIC_MAX_BYTES = 8 << 20  # RTP_GATE_WGRAD_STATIC_MAX_BYTES of include/rtp_hip.h
 
 
@@ -50,6 +51,7 @@ class GemmDesc(C.Structure):
         ("bias_sk", C.c_int64),
         ("alpha", C.c_float), ("flags", C.c_int32), ("a_kcontig", C.c_int32), ("b_kcontig", C.c_int32),
         ("a_rowsum", C.c_void_p), ("rowsum_sg", C.c_int64),
+        ("sgd_master", C.c_void_p), ("sgd_weights", C.c_void_p), ("sgd_lr", C.c_float), ("sgd_clip", C.c_float),
     ]
 
 
@@ -67,7 +69,7 @@ PROTOTYPES = {
     "rtp_device_check": (_i, [C.c_char_p, _i]),
     "rtp_gemm": (_i, [_vp, _i, C.POINTER(GemmDesc)]),
     "rtp_gemm_rowsum_fused": (_i, [_i, C.POINTER(GemmDesc)]),
-    "rtp_gemm_rowsum_fused": (_i, [_i, C.POINTER(GemmDesc)]),
+    "rtp_gemm_sgd_fused": (_i, [_i, C.POINTER(GemmDesc)]),
     "rtp_gemm_desc_size": (_sz, []),
     "rtp_colsum_workspace_bytes": (_sz, [_i64, _i64]),
     "rtp_colsum": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _vp, _i, _i, _i64, _i64, _vp, _sz]),

@@ -110,13 +110,13 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 template <size_t BYTES>
 __device__ __forceinline__ void touch_kernel_arguments() {
   constexpr int LINES = (int)(BYTES / 64) + 1;
-  static_assert(LINES <= 8, "at most 512 bytes of kernel arguments");
+  static_assert(LINES <= 10, "at most 640 bytes of kernel arguments");
   typedef const __attribute__((address_space(4))) int* kernarg_t;
   kernarg_t ka = (kernarg_t)__builtin_amdgcn_kernarg_segment_ptr();
   const int w0 = ka[0], w1 = ka[LINES > 1 ? 16 : 0], w2 = ka[LINES > 2 ? 32 : 0], w3 = ka[LINES > 3 ? 48 : 0];
   const int w4 = ka[LINES > 4 ? 64 : 0], w5 = ka[LINES > 5 ? 80 : 0], w6 = ka[LINES > 6 ? 96 : 0];
-  const int w7 = ka[LINES > 7 ? 112 : 0];
-  asm volatile("" ::"s"(w0), "s"(w1), "s"(w2), "s"(w3), "s"(w4), "s"(w5), "s"(w6), "s"(w7));
+  const int w7 = ka[LINES > 7 ? 112 : 0], w8 = ka[LINES > 8 ? 128 : 0], w9 = ka[LINES > 9 ? 144 : 0];
+  asm volatile("" ::"s"(w0), "s"(w1), "s"(w2), "s"(w3), "s"(w4), "s"(w5), "s"(w6), "s"(w7), "s"(w8), "s"(w9));
 }
 
 

@@ -74,6 +74,9 @@ struct GemmArgs {
   int mbk, nbk, prow, pcol;
   int xn_shift, xm_shift, zbk;  // log2 of xn and xm, batch*groups entries per brick
   unsigned long long* trace;    // null, or two words: earliest start / latest end of the launch on the wall clock
+  float* sgd_master;            // null, or the fp32 parameters the product updates (indexed like c_out)
+  char* sgd_w;                  // null, or the compute-dtype copy of the parameters
+  float sgd_lr, sgd_clip;
 };
 
 constexpr int kThreads = 256;
@@ -451,6 +454,19 @@ __device__ __forceinline__ void store8(T* dst, const float (&v)[8], bool stream)
   }
 }
 
+// Clip + SGD on one element: g is the gradient as the output dtype holds it.  Two roundings (product, then
+// difference), no fused multiply-add: the arithmetic of sgd_kernel in optim.hip.
+template <typename T>
+__device__ __forceinline__ float sgd_update(float w, float v, float lr, float clip) {
+  float g = to_f32(from_f32<T>(v));
+  if (clip > 0.0f) g = fminf(fmaxf(g, -clip), clip);
+  {
+#pragma clang fp contract(off)
+    const float step = lr * g;
+    return w - step;
+  }
+}
+
 template <typename T, int BM, int BN, int NTHR>
 __device__ __forceinline__ void finish_tile(const GemmArgs& p, const float* ct, int m0, int n0, int tid, int grp,
                                             long zo, long zi) {
@@ -467,6 +483,10 @@ __device__ __forceinline__ void finish_tile(const GemmArgs& p, const float* ct, 
   const T* gate =
       p.gate ? reinterpret_cast<const T*>(p.gate) + grp * p.gate_sg + zo * p.gate_so + zi * p.gate_si : nullptr;
   const int nb_seg = p.bias_sk ? p.ksegs : 1;  // a bias per K segment is summed in segment order
+  const long zoff = grp * p.c_sg + zo * p.c_so + zi * p.c_si;
+  float* master = p.sgd_master ? p.sgd_master + zoff : nullptr;
+  T* wcopy = p.sgd_w ? reinterpret_cast<T*>(p.sgd_w) + zoff : nullptr;
+  const bool skip_out = p.flags & RTP_GEMM_SGD_SKIP_OUT;
 
   for (int c = tid; c < CHUNKS; c += NTHR) {
     const int lr = c / CPR, lc = (c % CPR) * 8;
@@ -510,10 +530,20 @@ __device__ __forceinline__ void finish_tile(const GemmArgs& p, const float* ct, 
         for (int e = 0; e < 8; ++e) v[e] = t[e] > 0.0f ? v[e] : 0.0f;
       }
       const long off = (long)row * p.ldc + col;
-      if (out_f32)
-        store8(reinterpret_cast<float*>(cbase) + off, v, stream_out);
-      else
-        store8(reinterpret_cast<T*>(cbase) + off, v, stream_out);
+      if (master) {
+        float w[8];
+        load8(master + off, w);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) w[e] = sgd_update<T>(w[e], v[e], p.sgd_lr, p.sgd_clip);
+        store8(master + off, w, true);
+        if (wcopy) store8(wcopy + off, w, true);
+      }
+      if (!skip_out) {
+        if (out_f32)
+          store8(reinterpret_cast<float*>(cbase) + off, v, stream_out);
+        else
+          store8(reinterpret_cast<T*>(cbase) + off, v, stream_out);
+      }
     } else {
       for (int e = 0; e < 8 && col + e < p.n; ++e) {
         float x = v[e];
@@ -529,11 +559,67 @@ __device__ __forceinline__ void finish_tile(const GemmArgs& p, const float* ct, 
         if (relu) x = fmaxf(x, 0.0f);
         if (gate) x = to_f32(gate[(long)row * p.ld_gate + col + e]) > 0.0f ? x : 0.0f;
         const long off = (long)row * p.ldc + col + e;
+        if (master) {
+          const float w = sgd_update<T>(master[off], x, p.sgd_lr, p.sgd_clip);
+          master[off] = w;
+          if (wcopy) wcopy[off] = from_f32<T>(w);
+        }
+        if (skip_out) continue;
         if (out_f32)
           reinterpret_cast<float*>(cbase)[off] = x;
         else
           reinterpret_cast<T*>(cbase)[off] = from_f32<T>(x);
       }
+    }
+  }
+}
+
+// Epilogue of a product whose result is consumed by the fused clip + SGD update (a weight gradient: no c_in, bias,
+// ReLU or mask; 16-byte aligned operands, checked by the host).  The fp32 parameters of up to four of the thread's
+// chunks are requested before the first of them is needed, so the trips to memory overlap instead of following
+// each other; rows / columns outside the problem read a clamped address and store nothing.
+template <typename T, int BM, int BN, int NTHR>
+__device__ __forceinline__ void finish_tile_sgd(const GemmArgs& p, const float* ct, int m0, int n0, int tid, int grp,
+                                                long zo, long zi) {
+  constexpr int CP = BN + 4, CPR = BN / 8, CHUNKS = BM * CPR, NCH = CHUNKS / NTHR;
+  constexpr int BATCH = NCH % 4 == 0 ? 4 : (NCH % 3 == 0 ? 3 : (NCH % 2 == 0 ? 2 : 1));
+  static_assert(CHUNKS % NTHR == 0 && NCH % BATCH == 0, "every thread owns the same number of chunks");
+  const bool stream_out = p.flags & RTP_GEMM_STREAM_OUT;
+  const bool skip_out = p.flags & RTP_GEMM_SGD_SKIP_OUT;
+  const long zoff = grp * p.c_sg + zo * p.c_so + zi * p.c_si;
+  T* cbase = reinterpret_cast<T*>(p.c_out) + zoff;
+  float* master = p.sgd_master + zoff;
+  T* wcopy = p.sgd_w ? reinterpret_cast<T*>(p.sgd_w) + zoff : nullptr;
+#pragma unroll
+  for (int b0 = 0; b0 < NCH; b0 += BATCH) {
+    float w[BATCH][8];
+    long off[BATCH];
+    bool live[BATCH];
+#pragma unroll
+    for (int i = 0; i < BATCH; ++i) {
+      const int c = tid + (b0 + i) * NTHR;
+      const int row = m0 + c / CPR, col = n0 + (c % CPR) * 8;
+      live[i] = row < p.m && col < p.n;
+      off[i] = (long)(row < p.m ? row : p.m - 1) * p.ldc + (col < p.n ? col : 0);
+      load8(master + off[i], w[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < BATCH; ++i) {
+      const int c = tid + (b0 + i) * NTHR;
+      const int lr = c / CPR, lc = (c % CPR) * 8;
+      float v[8];
+      const float4 lo = *reinterpret_cast<const float4*>(ct + lr * CP + lc);
+      const float4 hi = *reinterpret_cast<const float4*>(ct + lr * CP + lc + 4);
+      v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w, v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        v[e] *= p.alpha;
+        w[i][e] = sgd_update<T>(w[i][e], v[e], p.sgd_lr, p.sgd_clip);
+      }
+      if (!live[i]) continue;
+      store8(master + off[i], w[i], true);
+      if (wcopy) store8(wcopy + off[i], w[i], true);
+      if (!skip_out) store8(cbase + off[i], v, stream_out);
     }
   }
 }
@@ -940,7 +1026,10 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
           ct[(wm * WM + i * 32 + 8 * (r >> 2) + 4 * g + (r & 3)) * CP + wn * WN + j * 32 + li] = acc[i][j][r];
   }
   __syncthreads();
-  finish_tile<T, BM, BN, 512>(p, ct, m0, n0, tid, grp, zo, zi);
+  if (p.sgd_master != nullptr && p.vec_c)
+    finish_tile_sgd<T, BM, BN, 512>(p, ct, m0, n0, tid, grp, zo, zi);
+  else
+    finish_tile<T, BM, BN, 512>(p, ct, m0, n0, tid, grp, zo, zi);
   if (p.trace != nullptr && tid == 0) atomicMax(p.trace + 1, (unsigned long long)wall_clock64());
 }
 
@@ -1076,6 +1165,13 @@ static bool takes_dma_kernel(const rtp_gemm_desc* d) {
          (bkc || mult(d->n, VEC)) && d->k > 0 && d->lda <= ld_max && d->ldb <= ld_max;
 }
 
+// The fused clip + SGD lives in the epilogue of the wave-specialised kernel; the gradient keeps the compute dtype.
+template <typename T>
+static bool sgd_fused(const rtp_gemm_desc* d) {
+  return !is_tiny(d) && takes_dma_kernel<T>(d) && !(d->flags & (RTP_GEMM_OUT_F32 | RTP_GEMM_RELU)) && !d->c_in &&
+         !d->bias && !d->gate;
+}
+
 template <typename T>
 static bool rowsum_fused(const rtp_gemm_desc* d) {
   return !d->a_kcontig && d->batch == 1 && !is_tiny(d) && takes_dma_kernel<T>(d);
@@ -1131,6 +1227,18 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   a.a_rowsum = (char*)d->a_rowsum;
   a.rowsum_sg = d->rowsum_sg;
   a.trace = nullptr;
+  a.sgd_master = (float*)d->sgd_master;
+  a.sgd_w = (char*)d->sgd_weights;
+  a.sgd_lr = d->sgd_lr;
+  a.sgd_clip = d->sgd_clip;
+  RTP_REQUIRE(!d->sgd_master || sgd_fused<T>(d),
+              "rtp_gemm: sgd_master needs vector-aligned operands, an output in the compute dtype and no c_in / bias / "
+              "ReLU / mask (rtp_gemm_sgd_fused)");
+  RTP_REQUIRE(d->sgd_master || (!d->sgd_weights && !(d->flags & RTP_GEMM_SGD_SKIP_OUT)),
+              "rtp_gemm: sgd_weights / RTP_GEMM_SGD_SKIP_OUT without sgd_master");
+  if (d->sgd_master)  // the update's 16-byte accesses: 8 fp32 columns are two of them
+    a.vec_c = a.vec_c && mult((int64_t)(uintptr_t)d->sgd_master, 16) &&
+              (!d->sgd_weights || mult((int64_t)(uintptr_t)d->sgd_weights, 16));
   RTP_REQUIRE(!d->a_rowsum || rowsum_fused<T>(d),
               "rtp_gemm: a_rowsum needs A stored K x M, batch == 1 and vector-aligned operands (rtp_gemm_rowsum_fused)");
   if (is_tiny(d)) {
@@ -1408,6 +1516,14 @@ extern "C" int rtp_gemm_rowsum_fused(int dtype, const rtp_gemm_desc* d) {
   if (!d || !d->a || !d->b || d->m <= 0 || d->n <= 0 || d->k <= 0 || d->groups < 1 || d->ksegs < 1) return 0;
   if (dtype == RTP_F32) return rowsum_fused<float>(d) ? 1 : 0;
   if (dtype == RTP_BF16) return rowsum_fused<bf16_t>(d) ? 1 : 0;
+  return 0;
+}
+
+extern "C" int rtp_gemm_sgd_fused(int dtype, const rtp_gemm_desc* d) {
+  using namespace rtp;
+  if (!d || !d->a || !d->b || d->m <= 0 || d->n <= 0 || d->k <= 0 || d->groups < 1 || d->ksegs < 1) return 0;
+  if (dtype == RTP_F32) return sgd_fused<float>(d) ? 1 : 0;
+  if (dtype == RTP_BF16) return sgd_fused<bf16_t>(d) ? 1 : 0;
   return 0;
 }
 

@@ -295,9 +295,9 @@ class _AttentionFn(torch.autograd.Function):
         def param_grads():
             for first, cnt, accumulate in runs:
                 S.row_wgrad(dout2, o, store.grads, first, w_o_off, E, e_s, first * e_s, cnt, accumulate,
-                            b_off=b_o_off if layer.has_bias else None)
+                            b_off=b_o_off if layer.has_bias else None, store=store)
                 S.col_wgrad(dqkv, x2, store.grads, first, 0, 3 * e_s, E, first * 3 * e_s, cnt, accumulate,
-                            b_off=b_in_off if layer.has_bias else None)
+                            b_off=b_in_off if layer.has_bias else None, store=store)
             store.grads_ready()
 
         run_wgrad(dev, param_grads, (dout2, o, dqkv, x2))
@@ -481,10 +481,10 @@ class _GeneralAttentionFn(torch.autograd.Function):
         def param_grads():
             for first, cnt, accumulate in runs:
                 c0 = first * e_s
-                S.row_wgrad(dout2, o, store.grads, first, w_o, E, e_s, c0, cnt, accumulate, b_off=b_o)
-                S.col_wgrad(dqb, q2, store.grads, first, wq, e_s, E, c0, cnt, accumulate, b_off=bq)
-                S.col_wgrad(dk_in, k2, store.grads, first, wk, e_s, layer.kdim, c0, cnt, accumulate, b_off=bk)
-                S.col_wgrad(dv_in, v2, store.grads, first, wv, e_s, layer.vdim, c0, cnt, accumulate, b_off=bv)
+                S.row_wgrad(dout2, o, store.grads, first, w_o, E, e_s, c0, cnt, accumulate, b_off=b_o, store=store)
+                S.col_wgrad(dqb, q2, store.grads, first, wq, e_s, E, c0, cnt, accumulate, b_off=bq, store=store)
+                S.col_wgrad(dk_in, k2, store.grads, first, wk, e_s, layer.kdim, c0, cnt, accumulate, b_off=bk, store=store)
+                S.col_wgrad(dv_in, v2, store.grads, first, wv, e_s, layer.vdim, c0, cnt, accumulate, b_off=bv, store=store)
             store.grads_ready()
 
         run_wgrad(dev, param_grads, (dout2, o, dqb, dk_in, dv_in, q2, k2, v2))

@@ -77,6 +77,7 @@ class ShardStore:
         self.grads: Optional[torch.Tensor] = None
         self._overwrite = set()
         self.stage_group = None  # set by ring.group_stores
+        self.fused_sgd = None  # set by an optimiser that applies its update inside the weight-gradient products
         self.on_grads_ready = None  # optional callable(store): the layer's backward has written every gradient row
         self.on_backward = None     # optional callable(store): the layer's backward has started (called at once)
         self.pack()

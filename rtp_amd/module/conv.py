@@ -110,7 +110,7 @@ class _ColumnConvFn(torch.autograd.Function):
         def param_grads():
             for first, cnt, accumulate in runs:
                 S.col_wgrad(dy2, cols, store.grads, first, 0, n_s, k, first * n_s, cnt, accumulate,
-                            b_off=n_s * k if layer.has_bias else None)
+                            b_off=n_s * k if layer.has_bias else None, store=store)
             store.grads_ready()
 
         run_wgrad(dy2.device, param_grads, (dy2, cols))

@@ -108,7 +108,7 @@ class _ColumnLinearFn(torch.autograd.Function):
         def param_grads():
             for first, cnt, accumulate in runs:
                 S.col_wgrad(dy2, x2, store.grads, first, 0, n_s, k, first * n_s, cnt, accumulate,
-                            b_off=n_s * k if layer.has_bias else None)
+                            b_off=n_s * k if layer.has_bias else None, store=store)
             store.grads_ready()
 
         run_wgrad(dy2.device, param_grads, (dy2, x2))
@@ -173,7 +173,7 @@ class _ColumnReluMlpFn(torch.autograd.Function):
             def param_grads(lin=lin, store=store, g=g, inp=inp, runs=runs, n_s=n_s, k=k):
                 for first, cnt, accumulate in runs:
                     S.col_wgrad(g, inp, store.grads, first, 0, n_s, k, first * n_s, cnt, accumulate,
-                                b_off=n_s * k if lin.has_bias else None)
+                                b_off=n_s * k if lin.has_bias else None, store=store)
                 store.grads_ready()
 
             run_wgrad(g.device, param_grads, (g, inp))
@@ -236,7 +236,7 @@ class _RowLinearFn(torch.autograd.Function):
         def param_grads():
             for first, cnt, accumulate in runs:
                 S.row_wgrad(dy2, x2, store.grads, first, 0, n, k_s, first * k_s, cnt, accumulate,
-                            b_off=n * k_s if layer.has_bias else None)
+                            b_off=n * k_s if layer.has_bias else None, store=store)
             store.grads_ready()
 
         run_wgrad(dy2.device, param_grads, (dy2, x2))

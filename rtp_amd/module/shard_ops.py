@@ -46,9 +46,29 @@ def col_dgrad(dy2, flat, w_off, n_s, k, out, col0, c_in: Optional[torch.Tensor] 
                  b_sk=numel, **kw)
 
 
-def col_wgrad(dy2, x2, grads, first, w_off, n_s, k, col0, cnt, accumulate, b_off: Optional[int] = None):
+def _fused(store, accumulate, first, cnt, w_off, length):
+    """Keyword arguments that make a weight-gradient product of `store` apply the optimiser's update itself (when
+    an optimiser has asked for that, RotatedSGD(fused_backward=True)), and the note of what it covers."""
+    f = getattr(store, "fused_sgd", None) if store is not None else None
+    if f is None:
+        return {}
+    if accumulate:
+        raise RuntimeError("RotatedSGD(fused_backward=True): a rotated layer produced gradients twice before step(); "
+                           "use fused_backward=False for gradient accumulation or shared layers")
+    return f.bind(store, first, cnt, w_off, length)
+
+
+def _fused_done(store, kw):
+    """After the launch: if the library could not fuse the update for these operands, take the note back (the
+    optimiser then updates that range itself)."""
+    if kw:
+        store.fused_sgd.confirm()
+
+
+def col_wgrad(dy2, x2, grads, first, w_off, n_s, k, col0, cnt, accumulate, b_off: Optional[int] = None, store=None):
     """grads[first+g, w_off : w_off + n_s*k] (+)= dy2[:, col0 + g*n_s : ...]^T @ x2, g < cnt; with `b_off` also the
-    bias gradients grads[first+g, b_off : b_off + n_s] (+)= column sums of the same block of dy2."""
+    bias gradients grads[first+g, b_off : b_off + n_s] (+)= column sums of the same block of dy2.  `store`: the
+    layer's ShardStore, for an optimiser that applies its update inside this launch."""
     numel = grads.shape[1]
     es = grads.element_size()
     m, _, lda = _rows(dy2)
@@ -65,10 +85,12 @@ def col_wgrad(dy2, x2, grads, first, w_off, n_s, k, col0, cnt, accumulate, b_off
         return
     # the bias gradient is the row sum of the product's first operand dy^T: the same launch adds it up
     rs = None if b_off is None else grads.data_ptr() + (first * numel + b_off) * es
+    kw = _fused(store, accumulate, first, cnt, w_off, n_s * k)
     fused = ops.gemm_raw(grads.dtype, a=dy2.data_ptr() + col0 * es, b=x2.data_ptr(), c_out=c, m=n_s, n=k, k=m, lda=lda,
                          ldb=ldb, ldc=k, a_kcontig=False, b_kcontig=False, groups=cnt, a_sg=n_s, c_sg=numel,
                          c_in=c if accumulate else None, ld_cin=k, cin_sg=numel, stream_out=True,
-                         rowsum=rs, rowsum_sg=numel, rowsum_accum=accumulate)
+                         rowsum=rs, rowsum_sg=numel, rowsum_accum=accumulate, **kw)
+    _fused_done(store, kw)
     if b_off is not None and not fused:
         col_bgrad(dy2, grads, first, b_off, n_s, col0, cnt, accumulate)
 
@@ -104,7 +126,7 @@ def row_dgrad(dy2, flat, w_off, n, k_s, out, col0):
                  c_sg=k_s)
 
 
-def row_wgrad(dy2, x2, grads, first, w_off, n, k_s, col0, cnt, accumulate, b_off: Optional[int] = None):
+def row_wgrad(dy2, x2, grads, first, w_off, n, k_s, col0, cnt, accumulate, b_off: Optional[int] = None, store=None):
     """grads[first+g, w_off : w_off + n*k_s] (+)= dy2^T @ x2[:, col0 + g*k_s : ...]; with `b_off` also the bias
     gradients grads[first+g, b_off : b_off + n] (+)= column sums of dy2 (every shard of a row-style layer stores
     bias/ws and receives the full sum, tests/test_linear.py:181-186)."""
@@ -114,10 +136,12 @@ def row_wgrad(dy2, x2, grads, first, w_off, n, k_s, col0, cnt, accumulate, b_off
     _, _, ldb = _rows(x2)
     c = grads.data_ptr() + (first * numel + w_off) * es
     rs = None if b_off is None else grads.data_ptr() + (first * numel + b_off) * es
+    kw = _fused(store, accumulate, first, cnt, w_off, n * k_s)
     fused = ops.gemm_raw(grads.dtype, a=dy2.data_ptr(), b=x2.data_ptr() + col0 * es, c_out=c, m=n, n=k_s, k=m, lda=lda,
                          ldb=ldb, ldc=k_s, a_kcontig=False, b_kcontig=False, groups=cnt, b_sg=k_s, c_sg=numel,
                          c_in=c if accumulate else None, ld_cin=k_s, cin_sg=numel, stream_out=True,
-                         rowsum=rs, rowsum_sg=numel, rowsum_accum=accumulate)
+                         rowsum=rs, rowsum_sg=numel, rowsum_accum=accumulate, **kw)
+    _fused_done(store, kw)
     if b_off is not None and not fused:
         row_bgrad(dy2, grads, first, b_off, n, cnt, accumulate)
 

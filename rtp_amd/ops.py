@@ -50,8 +50,13 @@ def gemm_raw(dtype: torch.dtype, *, a: int, b: int, c_out: int, m: int, n: int, 
              a_s=(0, 0), b_s=(0, 0), c_s=(0, 0), cin_s=(0, 0), gate_s=(0, 0), bias_s=(0, 0), groups: int = 1,
              a_sg: int = 0, b_sg: int = 0, c_sg: int = 0, cin_sg: int = 0, gate_sg: int = 0, bias_sg: int = 0,
              ksegs: int = 1, a_sk: int = 0, b_sk: int = 0, bias_sk: int = 0, stream_out: bool = False,
-             rowsum: Optional[int] = None, rowsum_sg: int = 0, rowsum_accum: bool = False) -> bool:
+             rowsum: Optional[int] = None, rowsum_sg: int = 0, rowsum_accum: bool = False,
+             sgd: Optional["FusedSgd"] = None, sgd_master: int = 0, sgd_weights: int = 0) -> bool:
     """One rtp_gemm call on raw device addresses (see include/rtp_hip.h for the operand rules).
+
+    `sgd` (with the addresses of the fp32 parameters and of their compute-dtype copy that match c_out) asks for the
+    clip + SGD update in the product's epilogue; if the library cannot fuse it for these operands the product runs
+    without it and `sgd.missed` is set.
 
     `rowsum` asks for the row sums of A (the bias gradient of a weight-gradient product) from the same launch.
     Returns whether they were produced: False means the library cannot fuse them for these operands, the
@@ -76,6 +81,14 @@ def gemm_raw(dtype: torch.dtype, *, a: int, b: int, c_out: int, m: int, n: int, 
         (GEMM_STREAM_OUT if stream_out else 0) | (GEMM_ROWSUM_ACCUM if rowsum_accum else 0)
     d.a_kcontig, d.b_kcontig = int(a_kcontig), int(b_kcontig)
     lib = _lib.load()
+    if sgd is not None:
+        if lib.rtp_gemm_sgd_fused(dtype_code(dtype), C.byref(d)):
+            d.sgd_master, d.sgd_weights = sgd_master, (sgd_weights or None)
+            d.sgd_lr, d.sgd_clip = sgd.lr, sgd.clip
+            if not sgd.keep_grads:
+                d.flags |= _lib.GEMM_SGD_SKIP_OUT
+        else:
+            sgd.missed = True
     fused = rowsum is not None and bool(lib.rtp_gemm_rowsum_fused(dtype_code(dtype), C.byref(d)))
     d.a_rowsum, d.rowsum_sg = (rowsum, rowsum_sg) if fused else (None, 0)
     check(lib.rtp_gemm(_stream(), dtype_code(dtype), C.byref(d)))
@@ -761,6 +774,15 @@ def cast(src: torch.Tensor, dst: torch.Tensor) -> None:
     _lib.require_device()
     check(_lib.load().rtp_cast(_stream(), dtype_code(src.dtype), src.data_ptr(), dtype_code(dst.dtype),
                                dst.data_ptr(), src.numel()))
+
+
+class FusedSgd:
+    """What a weight-gradient product needs to apply clip + SGD in its own epilogue: the step's scalars, whether the
+    gradient is still to be stored, and the record of what was (or could not be) updated this way."""
+
+    def __init__(self, lr: float, clip: float, keep_grads: bool = False):
+        self.lr, self.clip, self.keep_grads = float(lr), float(clip), bool(keep_grads)
+        self.missed = False
 
 
 class ShardSum:

@@ -34,11 +34,51 @@ class GradSink:
         self.overwrite = False  # True after zero_grad(): the next gradient replaces the slice's contents
 
 
+class _FusedBinding:
+    """Per rotated layer: where the fp32 parameters and their compute-dtype copy live, and which parameter ranges
+    of which shards the weight-gradient products of the running backward pass have already updated."""
+
+    def __init__(self, ctx: ops.FusedSgd, master: Optional[torch.Tensor]):
+        self.ctx = ctx
+        self.master = master       # [ws, numel] fp32, or None when the weights are fp32 themselves
+        self.applied = {}          # (offset, length) -> set of shard indices
+        self._last = None
+
+    def bind(self, store: ShardStore, first: int, cnt: int, w_off: int, length: int):
+        numel = store.numel
+        if self.master is None:
+            mptr, wptr = store.home.data_ptr() + (first * numel + w_off) * 4, 0
+        else:
+            mptr = self.master.data_ptr() + (first * numel + w_off) * 4
+            wptr = store.home.data_ptr() + (first * numel + w_off) * store.home.element_size()
+        self._last = ((w_off, length), range(first, first + cnt))
+        self.ctx.missed = False
+        return dict(sgd=self.ctx, sgd_master=mptr, sgd_weights=wptr)
+
+    def confirm(self) -> None:
+        key, shards = self._last
+        self._last = None
+        if self.ctx.missed:
+            self.ctx.missed = False
+            return
+        self.applied.setdefault(key, set()).update(shards)
+
+
 class RotatedSGD:
-    def __init__(self, model: nn.Module, lr: float, clip_value: float = 0.0, overlap_backward: bool = False):
+    """`fused_backward=True`: clip + SGD of every weight matrix of the rotated layers is applied in the epilogue of
+    the weight-gradient product that computes its gradient (the gradient is consumed where it is produced: it is not
+    written to memory unless keep_grads=True, and never read back); step() then only updates what no product
+    covers -- biases, embedding tables, gate weights, LayerNorm.  Same arithmetic, bit-identical weights.  As with
+    overlap_backward the weights change during backward(), and exactly one backward per step is allowed."""
+
+    def __init__(self, model: nn.Module, lr: float, clip_value: float = 0.0, overlap_backward: bool = False,
+                 fused_backward: bool = False, keep_grads: bool = False):
         self.lr = float(lr)
         self.clip_value = float(clip_value)
         self.overlap_backward = bool(overlap_backward)
+        self.fused_backward = bool(fused_backward)
+        if self.fused_backward and self.overlap_backward:
+            raise ValueError("RotatedSGD: fused_backward and overlap_backward exclude each other")
         self.stores: List[ShardStore] = []
         rotated_params = set()
         for m in model.modules():
@@ -54,6 +94,12 @@ class RotatedSGD:
         self._table = self._table_key = None
         self._table_params, self._table_dtype = 0, None
         self._aux = None
+        self._rest_table = self._rest_key = None
+        self._rest_params = 0
+        if self.fused_backward:
+            ctx = ops.FusedSgd(self.lr, self.clip_value, keep_grads)
+            for st, master in zip(self.stores, self.masters):
+                st.fused_sgd = _FusedBinding(ctx, master)
         if self.overlap_backward and self.stores:
             self._aux = torch.cuda.Stream(device=self.stores[0].home.device)  # default priority
             for st in self.stores:
@@ -173,12 +219,49 @@ class RotatedSGD:
             self._table_dtype = dtype
         return self._table
 
+    def _step_rest(self) -> None:
+        """fused_backward: update every parameter range the weight-gradient products of this pass did not."""
+        items = []
+        for st, master in zip(self.stores, self.masters):
+            if st.grads is None:
+                continue
+            done = st.fused_sgd.applied
+            for off, n in zip(st.offsets, st.numels):
+                for s in range(st.world_size):
+                    if s in done.get((off, n), ()):
+                        continue
+                    g, h = st.grads[s, off:off + n], st.home[s, off:off + n]
+                    items.append((h, g, None) if master is None else (master[s, off:off + n], g, h))
+            done.clear()
+        if self.flat is not None:
+            self._fold_other_grads()
+            items.append((self.flat, self.flat_grad, None) if self.flat_master is None
+                         else (self.flat_master, self.flat_grad, self.flat))
+        if not items:
+            return
+        key = tuple(t.data_ptr() for it in items for t in it if t is not None)
+        if key != self._rest_key:
+            same = len({it[1].dtype for it in items}) == 1
+            self._rest_key = key
+            self._rest_table = ops.sgd_chunk_table(items, items[0][0].device) if same else None
+            self._rest_params = sum(it[0].numel() for it in items)
+        if self._rest_table is not None:
+            ops.sgd_step_multi(self._rest_table, items[0][1].dtype, self.lr, self.clip_value, self._rest_params)
+        else:
+            for m, g, sh in items:
+                ops.sgd_step(m, g, sh, self.lr, self.clip_value)
+
     @torch.no_grad()
     def step(self) -> None:
         if self.stores:
             ring.join_wgrad(self.stores[0].home.device)
         for st in self.stores:
             st.settle_overwrite()
+        if self.fused_backward:
+            self._step_rest()
+            if self.stores:
+                ring.fence(self.stores[0].home.device)
+            return
         table = None if (self._early or self.overlap_backward) else self._multi_table()
         if table is not None:
             self._fold_other_grads()

@@ -352,3 +352,52 @@ def test_lm_step_replayed_from_a_graph_matches_eager_steps(overlap):
         graph_replays_against_eager_twin(twins, V, L, N, replays=4)
     finally:
         ring.set_wgrad_overlap(before)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("wgrad_overlap", [False, True])
+def test_lm_sgd_fused_into_weight_gradient_products_is_bit_identical(dtype, wgrad_overlap):
+    """fused_backward=True applies clip + SGD in the epilogue of every weight-gradient product (the gradient is
+    never stored); after step() every weight and master equals the sequential optimiser's, step after step, and
+    with keep_grads=True so does every gradient."""
+    from rtp_amd import ring
+    from rtp_amd.optim import RotatedSGD
+    # more than 256 tokens and widths of whole 16-byte vectors: the products take the kernel that carries the update
+    V, D, H, Fd, n_dec, L, N, ws = 128, 64, 4, 128, 2, 16, 20, 4
+    lms = [build_pair(V, D, H, Fd, n_dec, ws, dtype, seed=5)[0] for _ in range(3)]
+    opts = [RotatedSGD(lms[0], lr=0.05, clip_value=0.05),
+            RotatedSGD(lms[1], lr=0.05, clip_value=0.05, fused_backward=True),
+            RotatedSGD(lms[2], lr=0.05, clip_value=0.05, fused_backward=True, keep_grads=True)]
+    gen = torch.Generator().manual_seed(0)
+    ring.set_wgrad_overlap(wgrad_overlap)
+    try:
+        for step in range(3):
+            ids = torch.randint(0, V, (L, N), generator=gen).to(DEV)
+            for lm, opt in zip(lms, opts):
+                opt.zero_grad()
+                F.cross_entropy(lm(ids).float().view(-1, V), ids.view(-1)).backward()
+                opt.step()
+            torch.cuda.synchronize()
+            for other, opt_o, grads_too in ((lms[1], opts[1], False), (lms[2], opts[2], True)):
+                for (na, pa), (nb, pb) in zip(lms[0].named_parameters(), other.named_parameters()):
+                    assert na == nb and torch.equal(pa, pb), f"step {step}: {na} differs"
+                    if grads_too:
+                        assert torch.equal(pa.grad, pb.grad), f"step {step}: grad of {na} differs"
+                for ma, mb in zip(opts[0].masters, opt_o.masters):
+                    assert (ma is None and mb is None) or torch.equal(ma, mb)
+    finally:
+        ring.set_wgrad_overlap(False)
+    # the products did cover the weight matrices: what step() still updates is a small remainder
+    n_all = sum(st.world_size * st.numel for st in opts[1].stores)
+    assert 0 < opts[1]._rest_params < 0.35 * n_all
+
+
+def test_lm_sgd_fused_rejects_gradient_accumulation():
+    from rtp_amd.optim import RotatedSGD
+    V, D, H, Fd, n_dec, L, N, ws = 64, 32, 2, 32, 1, 6, 3, 2
+    lm, _ = build_pair(V, D, H, Fd, n_dec, ws, torch.float32, seed=2)
+    RotatedSGD(lm, lr=0.1, fused_backward=True)
+    ids = torch.randint(0, V, (L, N)).to(DEV)
+    F.cross_entropy(lm(ids).view(-1, V), ids.view(-1)).backward()
+    with pytest.raises(RuntimeError, match="fused_backward"):
+        F.cross_entropy(lm(ids).view(-1, V), ids.view(-1)).backward()
