@@ -247,6 +247,9 @@ int rtp_embedding_scatter_add_scaled(void* stream, int dtype, const void* grad_o
  *        the key padding mask (0 / -inf, functional.py:760-768 merges it into the mask per batch), with
  *        z = (group * n_batch + b) * heads + head.
  *   bwd: ds[z,i,j] = scale * p * (dp - sum_j dp*p)           dp fp32, ds `dtype`.
+ * Attention dropout (functional.py:789-792 / the dropout_p of :825): `keep` fp32 [Z,L,S] holds 0 or 1 / (1 - rate) per
+ * probability (the draw is the caller's).  fwd then also writes p_dropped = p * keep, the operand of the product with
+ * V; bwd takes dp as the gradient of p_dropped and multiplies it by keep first.  Both NULL: no dropout.
  * One wavefront per row, fp32 max/sum by cross-lane reduction.
  * --------------------------------------------------------------------------------------------- */
 int rtp_softmax_fwd(void* stream, int dtype, const float* s, const float* mask, const float* key_bias,
@@ -256,8 +259,8 @@ int rtp_softmax_fwd(void* stream, int dtype, const float* s, const float* mask, 
  * [mask_problems, L, S] and problem z takes mask[z % mask_problems]; mask_problems <= 1 is the single-mask form. */
 int rtp_softmax_fwd_masks(void* stream, int dtype, const float* s, const float* mask, int64_t mask_problems,
                           const float* key_bias, int64_t n_batch, int64_t heads, int causal, float scale, int64_t z,
-                          int64_t l, int64_t skv, void* p);
-int rtp_softmax_bwd(void* stream, int dtype, const void* p, const float* dp, float scale,
+                          int64_t l, int64_t skv, void* p, const float* keep, void* p_dropped);
+int rtp_softmax_bwd(void* stream, int dtype, const void* p, const float* dp, const float* keep, float scale,
                     int64_t z, int64_t l, int64_t skv, void* ds);
 
 /* ---------------------------------------------------------------------------------------------
@@ -345,18 +348,26 @@ int rtp_layernorm_bwd_finalize(void* stream, int dtype, const rtp_ln_final_item*
  * there a log-softmax, a gather and their backward over an fp32 copy of the logits).
  *   fwd: stats[r] = {m, s}, m = max_j logits[r, j], s = sum_j exp(logits[r, j] - m) (fp32 [rows, 2]);
  *        loss[r] = (m - logits[r, target[r]]) + log s (fp32 [rows]).
- *   bwd: dlogits[r, j] = (exp(logits[r, j] - m) / s - [j == target[r]]) * dloss[r * dloss_stride],
- *        dloss fp32 (dloss_stride 0: one scalar for all rows, 1: one value per row).
- * A row whose target lies outside [0, cols) has loss 0 and gradient 0 (an ignored row).
- * fp32 or bf16 logits, statistics in fp32; cols and both leading dimensions multiples of 16 bytes, cols at
- * most 8192 vectors of 16 bytes (65536 bf16 or 32768 fp32 classes: a row is held in registers).
+ *   bwd: dlogits[r, j] = (exp(logits[r, j] - m) / s - [j == target[r]]) * dloss[r * dloss_stride] * scale[0],
+ *        dloss fp32 (dloss_stride 0: one scalar for all rows, 1: one value per row); scale: a device scalar, may
+ *        be NULL for 1.
+ *   reduce: out[0] = sum_r loss[r], divided by the number of rows with target != ignore_index when `mean`;
+ *        scale[0] = 1 / that number (1 without `mean`) -- the `scale` of the backward pass of a mean loss.  One
+ *        workgroup, fixed summation order; no rows at all or all ignored gives NaN, as torch does.
+ * A row whose target equals ignore_index has loss 0 and gradient 0.  Any other target outside [0, cols) is the
+ * caller's error (torch asserts on the device): its loss is NaN, which shows in every sum over the rows, and its
+ * gradient 0.  fp32 or bf16 logits, statistics in fp32.  Rows of whole 16-byte vectors (cols and both leading
+ * dimensions multiples of 16 bytes, 16-byte aligned, at most 8192 vectors: 65536 bf16 or 32768 fp32 classes) are
+ * held in registers and read once; anything else takes element-wise kernels with the same results.
  * dlogits may alias logits.
  * --------------------------------------------------------------------------------------------- */
 int rtp_softmax_xent_fwd(void* stream, int dtype, const void* logits, int64_t ld, int64_t rows, int64_t cols,
-                         const int64_t* target, float* loss, float* stats);
+                         const int64_t* target, int64_t ignore_index, float* loss, float* stats);
+int rtp_softmax_xent_reduce(void* stream, const float* loss, const int64_t* target, int64_t ignore_index,
+                            int64_t rows, int mean, float* out, float* scale);
 int rtp_softmax_xent_bwd(void* stream, int dtype, const void* logits, int64_t ld, int64_t rows, int64_t cols,
                          const int64_t* target, const float* stats, const float* dloss, int64_t dloss_stride,
-                         void* dlogits, int64_t ld_dlogits);
+                         const float* scale, void* dlogits, int64_t ld_dlogits);
 
 /* ---------------------------------------------------------------------------------------------
  * Top-2 routing (reference: top2gating, rtp/module/top2gate.py:43-105).

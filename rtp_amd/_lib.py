@@ -91,8 +91,8 @@ PROTOTYPES = {
     "rtp_embedding_scatter_add_scaled": (_i, [_vp, _i, _vp, _i64, _i64, _vp, _vp, _i64, _i, _i64, _i64, _i64,
                                               _i64, _i, _i, _i64, _i64, _i64, _f]),
     "rtp_softmax_fwd": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _i64, _i, _f, _i64, _i64, _i64, _vp]),
-    "rtp_softmax_fwd_masks": (_i, [_vp, _i, _vp, _vp, _i64, _vp, _i64, _i64, _i, _f, _i64, _i64, _i64, _vp]),
-    "rtp_softmax_bwd": (_i, [_vp, _i, _vp, _vp, _f, _i64, _i64, _i64, _vp]),
+    "rtp_softmax_fwd_masks": (_i, [_vp, _i, _vp, _vp, _i64, _vp, _i64, _i64, _i, _f, _i64, _i64, _i64, _vp, _vp, _vp]),
+    "rtp_softmax_bwd": (_i, [_vp, _i, _vp, _vp, _vp, _f, _i64, _i64, _i64, _vp]),
     "rtp_attn_supported": (_i, [_i, _i64, _i64]),
     "rtp_attn_fwd": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _i,
                           _f, _i64, _i64, _i64, _i64, _i64]),
@@ -109,8 +109,9 @@ PROTOTYPES = {
     "rtp_layernorm_bwd_blocks": (_i64, [_i64]),
     "rtp_layernorm_bwd_finalize": (_i, [_vp, _i, _vp, _i64, _i64]),
     "rtp_layernorm_bwd": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _sz]),
-    "rtp_softmax_xent_fwd": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _vp, _vp, _vp]),
-    "rtp_softmax_xent_bwd": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _i64]),
+    "rtp_softmax_xent_fwd": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _vp]),
+    "rtp_softmax_xent_reduce": (_i, [_vp, _vp, _vp, _i64, _i64, _i, _vp, _vp]),
+    "rtp_softmax_xent_bwd": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _i64]),
     "rtp_top2_route_workspace_bytes": (_sz, [_i64, _i64]),
     "rtp_top2_route": (_i, [_vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz]),
     "rtp_top2_route_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),

@@ -8,7 +8,8 @@
 namespace rtp {
 
 constexpr int kLnThreads = 256;
-constexpr int kLnMaxCols = 2048;  // at most 2 vectors per thread (fp32), 1 (bf16)
+constexpr int kLnMaxVectors = 4;   // 16-byte vectors per thread: rows of up to 8192 bf16 or 4096 fp32 columns
+constexpr int kLnMaxCols = kLnMaxVectors * kLnThreads * 8;
 constexpr int kLnBwdRows = 4;     // rows per workgroup in the backward
 
 template <typename T>
@@ -271,8 +272,9 @@ __global__ __launch_bounds__(256) void layernorm_bwd_final_many_kernel(const LnF
 
 static int ln_nv(int dtype, int64_t cols) {
   const int vec = dtype == RTP_F32 ? 4 : 8;
-  if (cols <= 0 || cols % vec || cols > kLnMaxCols) return 0;
-  return (int)ceil_div(cols / vec, kLnThreads);  // 1 or 2
+  if (cols <= 0 || cols % vec || cols / vec > (int64_t)kLnMaxVectors * kLnThreads) return 0;
+  const int nv = (int)ceil_div(cols / vec, kLnThreads);
+  return nv == 3 ? 4 : nv;  // instantiated for 1, 2 and 4
 }
 
 }  // namespace rtp
@@ -286,8 +288,10 @@ extern "C" int rtp_layernorm_supported(int dtype, int64_t cols) {
 #define RTP_LN_DISPATCH(KERNEL, T, NVV, ...)                          \
   if ((NVV) == 1) {                                                   \
     hipLaunchKernelGGL((KERNEL<T, 1>), __VA_ARGS__);                  \
-  } else {                                                            \
+  } else if ((NVV) == 2) {                                            \
     hipLaunchKernelGGL((KERNEL<T, 2>), __VA_ARGS__);                  \
+  } else {                                                            \
+    hipLaunchKernelGGL((KERNEL<T, 4>), __VA_ARGS__);                  \
   }
 
 extern "C" int rtp_add_layernorm_fwd(void* stream, int dtype, const void* x, const void* r, const void* gamma,
@@ -297,8 +301,8 @@ extern "C" int rtp_add_layernorm_fwd(void* stream, int dtype, const void* x, con
   RTP_REQUIRE(rows >= 0 && rows < (1ll << 31), "rtp_add_layernorm_fwd: row count %lld out of range", (long long)rows);
   const int nv = ln_nv(dtype, cols);
   RTP_REQUIRE((dtype == RTP_F32 || dtype == RTP_BF16) && nv,
-              "rtp_add_layernorm_fwd: dtype %d with %lld columns is not supported (16-byte vectors, at most %d columns)",
-              dtype, (long long)cols, kLnMaxCols);
+              "rtp_add_layernorm_fwd: dtype %d with %lld columns is not supported (whole 16-byte vectors, at most %d of them)",
+              dtype, (long long)cols, kLnMaxVectors * kLnThreads);
   RTP_REQUIRE(((uintptr_t)x | (uintptr_t)r | (uintptr_t)gamma | (uintptr_t)beta | (uintptr_t)z_out | (uintptr_t)y) % 16 == 0,
               "rtp_add_layernorm_fwd: operands must be 16-byte aligned");
   if (rows == 0) return RTP_OK;

@@ -1,11 +1,12 @@
 """GPT-2 style nn.Sequential language model built from the rotated layers (counterpart of
 rtp/models/transformer_lm_rtp.py:19-242): embedding * sqrt(ninp) -> sinusoidal positions -> N post-LN
 decoder layers (rotated self-attention + rotated ReLU FFN or rotated MoE) -> rotated logits projection.
-Residual add + LayerNorm is one fused kernel each way (module/norm.py); the FFN's ReLU is folded into its two products (module/linear.py); dropout is an ordinary torch op."""
+Residual add + LayerNorm is one fused kernel each way (module/norm.py); the FFN's ReLU is folded into its two
+products (module/linear.py); the embedding's scale and the positional rows ride on its gather; dropout masks are
+drawn by torch's device generator and applied element-wise."""
 from __future__ import annotations
 
 import math
-import os
 
 import torch
 import torch.nn as nn
@@ -38,11 +39,11 @@ class EmbeddingLayer(nn.Module):
 
     def forward(self, src):
         pos = self.positional
-        if pos is None:
+        if pos is None:  # on its own, as the reference's layer: the next layer adds the positions
             return self.embedding(src) * self.ninp_sqrt
-        if src.dim() == 2 and pos.pe.dtype == self.embedding._store.home.dtype:
-            return self.embedding.forward_scaled_positional(src, self.ninp_sqrt, pos.pe[:, 0, :])
-        return self.embedding(src) * self.ninp_sqrt + pos.pe[: src.size(0), :]
+        if src.dim() != 2:
+            raise ValueError("EmbeddingLayer: token ids must be [sequence, batch]")
+        return self.embedding.forward_scaled_positional(src, self.ninp_sqrt, pos.pe[:, 0, :])
 
 
 class PositionalEncodingLayer(nn.Module):
@@ -80,8 +81,15 @@ class FeedForwardLayer_expert(nn.Module):
 
 
 class FeedForwardLayer(nn.Module):
+    """Linear -> ReLU -> dropout -> Linear -> dropout over two rotated column-parallel layers
+    (rtp/models/transformer_lm_rtp.py:77-89).  The ReLU lives in the epilogues of the two layers' products, so the
+    activation must be nn.ReLU (what the reference's TransformerLM always passes)."""
+
     def __init__(self, d_model, dim_feedforward, activation, dropout, world_size, rank, device=None, dtype=None):
         super().__init__()
+        if not isinstance(activation, nn.ReLU):
+            raise NotImplementedError("FeedForwardLayer: the rotated feed-forward block computes ReLU inside its products; "
+                                      f"got activation {type(activation).__name__}")
         with emulate_shards(world_size):
             self.linear1 = ColumnParallelLinear(d_model, dim_feedforward, device=device, dtype=dtype)
             self.linear2 = ColumnParallelLinear(dim_feedforward, d_model, device=device, dtype=dtype)
@@ -89,17 +97,10 @@ class FeedForwardLayer(nn.Module):
         self.dropout1 = nn.Dropout(dropout)
         self.dropout2 = nn.Dropout(dropout)
 
-    def fusable(self, x) -> bool:
-        return isinstance(self.activation, nn.ReLU) and not (self.training and self.dropout1.p > 0) and x.is_cuda
-
     def forward(self, x, residual_grad=False):
-        if self.fusable(x):
-            # ReLU folded into the epilogues of the two rotated products
-            y = column_relu_mlp(x, self.linear1, self.linear2, residual_grad=residual_grad)
-            return y if self.dropout2.p == 0.0 or not self.training else self.dropout2(y)
-        if residual_grad:
-            raise RuntimeError("FeedForwardLayer: residual_grad needs the fused ReLU path")
-        return self.dropout2(self.linear2(self.dropout1(self.activation(self.linear1(x)))))
+        p1 = self.dropout1.p if self.training else 0.0
+        y = column_relu_mlp(x, self.linear1, self.linear2, residual_grad=residual_grad, dropout_p=p1)
+        return y if self.dropout2.p == 0.0 or not self.training else self.dropout2(y)
 
 
 class TransformerEncoderLayer(nn.Module):
@@ -145,8 +146,7 @@ class TransformerEncoderLayer(nn.Module):
             via = layer_norm_fusable(x, self.norm1) and x.requires_grad and torch.is_grad_enabled() and no_drop
             x = add_layer_norm(x, self._sa_block(x, src_mask, src_key_padding_mask, residual_grad=via), self.norm1,
                                x_grad_via_branch=via)
-            via = (via and not self.is_moe and self.ff_block.fusable(x)
-                   and (self.ff_block.dropout2.p == 0.0 or not self.training))
+            via = via and not self.is_moe and (self.ff_block.dropout2.p == 0.0 or not self.training)
             x = add_layer_norm(x, self.ff_block(x, residual_grad=True) if via else self._ff_block(x), self.norm2,
                                x_grad_via_branch=via)
         return x
@@ -208,5 +208,4 @@ class TransformerLM(nn.Sequential):
                                                   world_size=world_size, rank=rank, device=device, dtype=dtype))
         layers.append(LinearLayer(ninp, ntokens, initrange, world_size, rank, device=device, dtype=dtype))
         super().__init__(*layers)
-        if os.environ.get("RTP_EMBED_FUSE", "1") != "0":
-            layers[0].adopt_positional(layers[1])
+        layers[0].adopt_positional(layers[1])

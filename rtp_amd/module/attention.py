@@ -183,11 +183,13 @@ class _AttentionFn(torch.autograd.Function):
                      c_s=(h_s * L * L, L * L), c_sg=Z * L * L, m=L, n=L, k=d, batch=Z, zdiv=h_s, groups=cnt,
                      out_f32=True)
                 p_run = p[first * Z:(first + cnt) * Z]
-                ops.softmax_fwd(scores, p_run, mask=mask, causal=causal, scale=scale, key_bias=key_bias, heads=h_s)
-                del scores
                 if drop is not None:
-                    _apply_dropout(layer, drop_p, p_run, drop[first * Z:(first + cnt) * Z],
-                                   pv[first * Z:(first + cnt) * Z])
+                    ops.softmax_fwd(scores, p_run, mask=mask, causal=causal, scale=scale, key_bias=key_bias, heads=h_s,
+                                    keep=_draw_keep(layer, drop_p, drop[first * Z:(first + cnt) * Z]),
+                                    p_dropped=pv[first * Z:(first + cnt) * Z])
+                else:
+                    ops.softmax_fwd(scores, p_run, mask=mask, causal=causal, scale=scale, key_bias=key_bias, heads=h_s)
+                del scores
                 _bmm(dt, a=pv, a_off=first * Z * L * L, lda=L, a_kc=True, a_s=(h_s * L * L, L * L), a_sg=Z * L * L,
                      b=qkv, b_off=q0 + 2 * e_s, ldb=ldq, b_kc=False, b_s=(ws * 3 * e_s, d), b_sg=3 * e_s, c=o,
                      c_off=first * e_s, ldc=N * E, c_s=(E, d), c_sg=e_s, m=L, n=d, k=L, batch=Z, zdiv=h_s, groups=cnt)
@@ -271,10 +273,9 @@ class _AttentionFn(torch.autograd.Function):
                 _bmm(dt, a=pv, a_off=p_off, lda=L, a_kc=False, a_s=(h_s * L * L, L * L), a_sg=Z * L * L, b=do,
                      b_off=first * e_s, ldb=N * E, b_kc=False, b_s=(E, d), b_sg=e_s, c=dqkv, c_off=q0 + 2 * e_s, ldc=ldq,
                      c_s=(ws * 3 * e_s, d), c_sg=3 * e_s, m=L, n=d, k=L, batch=Z, zdiv=h_s, groups=cnt)
-                if drop is not None:
-                    dp.mul_(drop[first * Z:(first + cnt) * Z])
                 ds = torch.empty(cnt * Z, L, L, dtype=dt, device=dev)
-                ops.softmax_bwd(p[first * Z:(first + cnt) * Z], dp, ds, scale)
+                ops.softmax_bwd(p[first * Z:(first + cnt) * Z], dp, ds, scale,
+                                keep=None if drop is None else drop[first * Z:(first + cnt) * Z])
                 del dp
                 # dQ = dS K
                 _bmm(dt, a=ds, a_off=0, lda=L, a_kc=True, a_s=(h_s * L * L, L * L), a_sg=Z * L * L, b=qkv,
@@ -304,22 +305,18 @@ class _AttentionFn(torch.autograd.Function):
         return (dx.view(L, N, E) if need_dx else None), None, None, None, None, None, None, None, None
 
 
-def _apply_dropout(layer, drop_p: float, p: Tensor, drop: Tensor, out: Tensor) -> None:
+def _draw_keep(layer, drop_p: float, drop: Tensor) -> Tensor:
     """Attention dropout (functional.py:789-792 / the dropout_p of :825): every probability is kept with chance
-    1 - drop_p and scaled by 1 / (1 - drop_p).  `drop` receives the fp32 multipliers (0 or 1 / (1 - drop_p)) for the
-    backward pass, `out` the probabilities that meet V.  The draw itself is torch's device generator (an ordinary
-    torch op, like the model's other dropouts); `layer.dropout_keep_fn`, if set, supplies the 0 / 1 keep mask instead."""
+    1 - drop_p and scaled by 1 / (1 - drop_p).  Fills `drop` with the fp32 multipliers (0 or 1 / (1 - drop_p)) that the
+    softmax kernels apply, forward and backward.  The draw itself is torch's device generator (like the model's
+    other dropouts); `layer.dropout_keep_fn`, if set, supplies the 0 / 1 keep mask instead."""
     keep = 1.0 - drop_p
     fn = getattr(layer, "dropout_keep_fn", None)
     if fn is not None:
         drop.copy_(fn(tuple(drop.shape)))
     else:
         drop.bernoulli_(keep)
-    drop.div_(keep)
-    if out.dtype == torch.float32:
-        torch.mul(p, drop, out=out)
-    else:
-        out.copy_(p.float().mul_(drop))
+    return drop.div_(keep)
 
 
 def _shard_layout(layer):
@@ -382,12 +379,15 @@ class _GeneralAttentionFn(torch.autograd.Function):
                 _bmm(dt, a=qb, a_off=c0, lda=ld, a_kc=True, a_s=(E, d), a_sg=e_s, b=kb, b_off=c0, ldb=ld, b_kc=True,
                      b_s=(E, d), b_sg=e_s, c=scores, c_off=0, ldc=sk, c_s=(h_s * L * sk, L * sk), c_sg=Z * L * sk,
                      m=L, n=sk, k=d, batch=Z, zdiv=h_s, groups=cnt, out_f32=True)
-                ops.softmax_fwd(scores, p[first * Z:(first + cnt) * Z], mask=mask, causal=False, scale=scale,
-                                key_bias=key_bias, heads=h_s)
-                del scores
                 if drop is not None:
-                    _apply_dropout(layer, drop_p, p[first * Z:(first + cnt) * Z], drop[first * Z:(first + cnt) * Z],
-                                   pv[first * Z:(first + cnt) * Z])
+                    ops.softmax_fwd(scores, p[first * Z:(first + cnt) * Z], mask=mask, causal=False, scale=scale,
+                                    key_bias=key_bias, heads=h_s,
+                                    keep=_draw_keep(layer, drop_p, drop[first * Z:(first + cnt) * Z]),
+                                    p_dropped=pv[first * Z:(first + cnt) * Z])
+                else:
+                    ops.softmax_fwd(scores, p[first * Z:(first + cnt) * Z], mask=mask, causal=False, scale=scale,
+                                    key_bias=key_bias, heads=h_s)
+                del scores
                 _bmm(dt, a=pv, a_off=first * Z * L * sk, lda=sk, a_kc=True, a_s=(h_s * L * sk, L * sk),
                      a_sg=Z * L * sk, b=vb, b_off=c0, ldb=ld, b_kc=False, b_s=(E, d), b_sg=e_s, c=o, c_off=c0, ldc=ld,
                      c_s=(E, d), c_sg=e_s, m=L, n=d, k=sk, batch=Z, zdiv=h_s, groups=cnt)
@@ -455,10 +455,9 @@ class _GeneralAttentionFn(torch.autograd.Function):
                 _bmm(dt, a=pv, a_off=p_off, lda=sk, a_kc=False, a_s=p_s, a_sg=p_sg, b=do, b_off=c0, ldb=ld, b_kc=False,
                      b_s=(E, d), b_sg=e_s, c=dvb, c_off=c0, ldc=ld, c_s=(E, d), c_sg=e_s, m=sk, n=d, k=L, batch=Z,
                      zdiv=h_s, groups=cnt)
-                if drop is not None:
-                    dp.mul_(drop[first * Z:(first + cnt) * Z])
                 ds = torch.empty(cnt * Z, L, sk, dtype=dt, device=dev)
-                ops.softmax_bwd(p[first * Z:(first + cnt) * Z], dp, ds, scale)
+                ops.softmax_bwd(p[first * Z:(first + cnt) * Z], dp, ds, scale,
+                                keep=None if drop is None else drop[first * Z:(first + cnt) * Z])
                 del dp
                 # dQ = dS K
                 _bmm(dt, a=ds, a_off=0, lda=sk, a_kc=True, a_s=p_s, a_sg=p_sg, b=kb, b_off=c0, ldb=ld, b_kc=False,

@@ -121,7 +121,7 @@ class _ColumnReluMlpFn(torch.autograd.Function):
     input-gradient product.  Same values as the three separate modules."""
 
     @staticmethod
-    def forward(ctx, x, anchor1, anchor2, lin1, lin2, residual_grad=False):
+    def forward(ctx, x, anchor1, anchor2, lin1, lin2, residual_grad=False, keep=None):
         k1, f, n2 = lin1.in_features, lin1.out_features, lin2.out_features
         x2 = as_rows(x, k1)
         rows, dt, dev = x2.shape[0], x2.dtype, x2.device
@@ -135,9 +135,12 @@ class _ColumnReluMlpFn(torch.autograd.Function):
                 for flat, first, cnt in rot.acquire(j):
                     S.col_fwd(src, flat, 0, n_s, k, b_off, dst, first * n_s, relu=relu)
                 rot.release(j)
+            if relu and keep is not None:
+                h.mul_(keep)  # dropout on the hidden activations: 0 or 1 / (1 - p) per element
         ctx.layers = (lin1, lin2)
         ctx.x_shape = x.shape
         ctx.residual_grad = residual_grad
+        ctx.keep = keep
         ctx.save_for_backward(x2, h)
         return y.view(*x.shape[:-1], n2)
 
@@ -168,6 +171,8 @@ class _ColumnReluMlpFn(torch.autograd.Function):
                                     gate=gate if i == steps - 1 else None)
                         i += 1
                     rot.release(j)
+                if lin is lin2 and ctx.keep is not None:
+                    dh.mul_(ctx.keep)  # h > 0 already implies a kept element; what is left is the 1 / (1 - p)
             runs = store.grad_runs(order)
 
             def param_grads(lin=lin, store=store, g=g, inp=inp, runs=runs, n_s=n_s, k=k):
@@ -177,19 +182,25 @@ class _ColumnReluMlpFn(torch.autograd.Function):
                 store.grads_ready()
 
             run_wgrad(g.device, param_grads, (g, inp))
-        return (dx.view(ctx.x_shape) if need_dx else None), None, None, None, None, None
+        return (dx.view(ctx.x_shape) if need_dx else None), None, None, None, None, None, None
 
 
 def column_relu_mlp(x: torch.Tensor, lin1: "ColumnParallelLinear", lin2: "ColumnParallelLinear",
-                    residual_grad: bool = False) -> torch.Tensor:
-    """lin2(relu(lin1(x))) with the ReLU fused into the products of the two rotated layers.  residual_grad: the
-    backward returns dy + mlp'(dy), for a caller whose residual connection does not propagate x's gradient itself
-    (add_layer_norm(..., x_grad_via_branch=True))."""
+                    residual_grad: bool = False, dropout_p: float = 0.0) -> torch.Tensor:
+    """lin2(dropout(relu(lin1(x)))) with the ReLU fused into the products of the two rotated layers.  residual_grad:
+    the backward returns dy + mlp'(dy), for a caller whose residual connection does not propagate x's gradient itself
+    (add_layer_norm(..., x_grad_via_branch=True)).  dropout_p > 0: the hidden activations are multiplied by a keep
+    mask drawn from torch's device generator (0 or 1 / (1 - p)), and so is their gradient."""
     if lin1.out_features != lin2.in_features:
         raise ValueError("column_relu_mlp: lin1.out_features must equal lin2.in_features")
     if residual_grad and lin2.out_features != lin1.in_features:
         raise ValueError("column_relu_mlp: residual_grad needs an output of the input's width")
-    return _ColumnReluMlpFn.apply(x, lin1._anchor, lin2._anchor, lin1, lin2, bool(residual_grad))
+    keep = None
+    if dropout_p > 0.0:
+        rows = x.numel() // x.shape[-1]
+        keep = torch.empty(rows, lin1.out_features, dtype=x.dtype, device=x.device).bernoulli_(1.0 - dropout_p)
+        keep.mul_(1.0 / (1.0 - dropout_p))
+    return _ColumnReluMlpFn.apply(x, lin1._anchor, lin2._anchor, lin1, lin2, bool(residual_grad), keep)
 
 
 class _RowLinearFn(torch.autograd.Function):

@@ -125,13 +125,15 @@ def layer_norm_fusable(x: torch.Tensor, norm: nn.LayerNorm) -> bool:
 
 
 def add_layer_norm(x: torch.Tensor, r: torch.Tensor, norm: nn.LayerNorm, x_grad_via_branch: bool = False) -> torch.Tensor:
-    """norm(x + r).  Fused on the device when the row length qualifies, else the two torch calls.
+    """norm(x + r) in one kernel each way.  Rows must be whole 16-byte vectors, at most 1024 of them (8192 bf16 /
+    4096 fp32 features), over the last dimension with an elementwise affine: anything else raises (there is no
+    second implementation behind this one).
     x_grad_via_branch: r = f(x) was computed by a rotated layer called with residual_grad=True, whose backward
     already returns the residual part of x's gradient (added in the epilogue of its last product), so this
-    function gives x no gradient of its own.  Only valid when layer_norm_fusable(x, norm)."""
-    fused = layer_norm_fusable(x, norm) and x.shape == r.shape and x.dtype == r.dtype
-    if not fused:
-        if x_grad_via_branch:
-            raise RuntimeError("add_layer_norm: x_grad_via_branch needs the fused path (check layer_norm_fusable)")
-        return norm(x + r)
+    function gives x no gradient of its own."""
+    if not (layer_norm_fusable(x, norm) and x.shape == r.shape and x.dtype == r.dtype):
+        from .._lib import RtpError
+        raise RtpError(f"add_layer_norm: x {tuple(x.shape)} {x.dtype} on {x.device}, branch {tuple(r.shape)} {r.dtype}, "
+                       f"LayerNorm{tuple(norm.normalized_shape)}: needs device tensors of one dtype, a LayerNorm over "
+                       "the last dimension with elementwise affine, rows of whole 16-byte vectors (at most 1024)")
     return _AddLayerNormFn.apply(x, r, norm.weight, norm.bias, norm.eps, bool(x_grad_via_branch))

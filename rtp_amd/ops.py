@@ -285,11 +285,21 @@ def _key_bias_ptr(who: str, key_bias: Optional[torch.Tensor], n_batch: int, keys
     return key_bias.data_ptr()
 
 
+def _keep_ptr(who: str, keep: Optional[torch.Tensor], like: torch.Tensor):
+    if keep is None:
+        return None
+    if keep.dtype != torch.float32 or keep.shape != like.shape or not keep.is_contiguous() or keep.device != like.device:
+        raise ValueError(f"{who}: keep must be a contiguous fp32 tensor of the probabilities' shape")
+    return keep.data_ptr()
+
+
 def softmax_fwd(scores: torch.Tensor, p: torch.Tensor, *, mask: Optional[torch.Tensor], causal: bool,
-                scale: float, key_bias: Optional[torch.Tensor] = None, heads: int = 1) -> None:
+                scale: float, key_bias: Optional[torch.Tensor] = None, heads: int = 1,
+                keep: Optional[torch.Tensor] = None, p_dropped: Optional[torch.Tensor] = None) -> None:
     """p[Z,L,S] = softmax(scale*scores + mask + key_bias[b]) row-wise; scores fp32, mask fp32 [L,S] (one for all
     problems) or [M,L,S] (problem z takes mask[z % M]) or None, key_bias fp32 [N,S] or None with
-    Z = groups * N * heads (problem z belongs to batch (z // heads) % N)."""
+    Z = groups * N * heads (problem z belongs to batch (z // heads) % N).  Attention dropout: `keep` (fp32, 0 or
+    1 / (1 - rate) per probability) and `p_dropped` (receives p * keep) go together."""
     _dev(scores)
     _dev(p)
     if scores.dtype != torch.float32 or scores.dim() != 3 or not scores.is_contiguous() or \
@@ -308,19 +318,27 @@ def softmax_fwd(scores: torch.Tensor, p: torch.Tensor, *, mask: Optional[torch.T
     n_batch = key_bias.shape[0] if key_bias is not None else 1
     kb = _key_bias_ptr("softmax_fwd", key_bias, n_batch, s)
     _lib.require_device()
+    if (keep is None) != (p_dropped is None):
+        raise ValueError("softmax_fwd: keep and p_dropped go together")
+    if p_dropped is not None and (p_dropped.shape != p.shape or p_dropped.dtype != p.dtype or
+                                  not p_dropped.is_contiguous()):
+        raise ValueError("softmax_fwd: p_dropped must match p")
     check(_lib.load().rtp_softmax_fwd_masks(_stream(), dtype_code(p.dtype), scores.data_ptr(), _ptr(mask), masks, kb,
-                                            n_batch, heads, int(causal), scale, z, l, s, p.data_ptr()))
+                                            n_batch, heads, int(causal), scale, z, l, s, p.data_ptr(),
+                                            _keep_ptr("softmax_fwd", keep, p), _ptr(p_dropped)))
 
 
-def softmax_bwd(p: torch.Tensor, dp: torch.Tensor, ds: torch.Tensor, scale: float) -> None:
+def softmax_bwd(p: torch.Tensor, dp: torch.Tensor, ds: torch.Tensor, scale: float,
+                keep: Optional[torch.Tensor] = None) -> None:
+    """ds = scale * p * (g - sum_j g * p) with g = dp, or dp * keep when the probabilities were dropped."""
     _dev(p)
     if dp.dtype != torch.float32 or p.dim() != 3 or dp.shape != p.shape or ds.shape != p.shape or \
             ds.dtype != p.dtype or not (p.is_contiguous() and dp.is_contiguous() and ds.is_contiguous()):
         raise ValueError("softmax_bwd: need contiguous p/ds [Z,L,S] of one dtype and fp32 dp")
     z, l, s = p.shape
     _lib.require_device()
-    check(_lib.load().rtp_softmax_bwd(_stream(), dtype_code(p.dtype), p.data_ptr(), dp.data_ptr(), scale, z, l, s,
-                                      ds.data_ptr()))
+    check(_lib.load().rtp_softmax_bwd(_stream(), dtype_code(p.dtype), p.data_ptr(), dp.data_ptr(),
+                                      _keep_ptr("softmax_bwd", keep, p), scale, z, l, s, ds.data_ptr()))
 
 
 def attn_supported(dtype: torch.dtype, L: int, d: int) -> bool:
@@ -522,58 +540,71 @@ def layernorm_finalize(table: torch.Tensor, dtype: torch.dtype, max_cols: int) -
                                                  max_cols))
 
 
-def softmax_xent_supported(logits: torch.Tensor) -> bool:
-    if logits.dtype not in (torch.float32, torch.bfloat16) or logits.dim() != 2 or not logits.is_cuda:
-        return False
-    vec = 16 // logits.element_size()
-    # a row is held in registers: at most 32 vectors of 16 bytes per thread of a 256-thread workgroup
-    return bool(logits.stride(1) == 1 and vec <= logits.shape[1] <= 32 * 256 * vec and logits.shape[1] % vec == 0
-                and logits.stride(0) >= logits.shape[1] and logits.stride(0) % vec == 0
-                and logits.data_ptr() % 16 == 0)
-
-
 def _xent_check(who: str, logits: torch.Tensor, target: torch.Tensor) -> None:
     _dev(logits)
-    if not softmax_xent_supported(logits):
-        raise ValueError(f"{who}: logits must be fp32/bf16 [rows, cols], unit column stride, cols and the row "
-                         "stride multiples of 16 bytes")
+    if logits.dtype not in (torch.float32, torch.bfloat16) or logits.dim() != 2 or logits.shape[1] < 1 or \
+            (logits.shape[1] > 1 and logits.stride(1) != 1) or \
+            (logits.shape[0] > 1 and logits.stride(0) < logits.shape[1]):
+        raise ValueError(f"{who}: logits must be fp32 / bf16 [rows, classes] with unit column stride")
     if target.dtype != torch.int64 or target.numel() != logits.shape[0] or not target.is_contiguous() or \
             target.device != logits.device:
         raise ValueError(f"{who}: target must be contiguous int64 [rows] on the logits' device")
 
 
-def softmax_xent_fwd(logits: torch.Tensor, target: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Per-row cross-entropy loss (fp32 [rows]) and softmax statistics {max, sum exp} (fp32 [rows, 2])."""
+def softmax_xent_fwd(logits: torch.Tensor, target: torch.Tensor,
+                     ignore_index: int = -100) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-row cross-entropy loss (fp32 [rows]; 0 where target == ignore_index, NaN for any other target outside
+    the classes) and softmax statistics {max, sum exp} (fp32 [rows, 2])."""
     _xent_check("softmax_xent_fwd", logits, target)
     rows, cols = logits.shape
     loss = torch.empty(rows, dtype=torch.float32, device=logits.device)
     stats = torch.empty((rows, 2), dtype=torch.float32, device=logits.device)
     _lib.require_device()
-    check(_lib.load().rtp_softmax_xent_fwd(_stream(), dtype_code(logits.dtype), logits.data_ptr(), logits.stride(0),
-                                           rows, cols, target.data_ptr(), loss.data_ptr(), stats.data_ptr()))
+    check(_lib.load().rtp_softmax_xent_fwd(_stream(), dtype_code(logits.dtype), logits.data_ptr(),
+                                           logits.stride(0) if rows > 1 else cols, rows, cols, target.data_ptr(),
+                                           int(ignore_index), loss.data_ptr(), stats.data_ptr()))
     return loss, stats
 
 
+def softmax_xent_reduce(loss_rows: torch.Tensor, target: torch.Tensor, ignore_index: int,
+                        mean: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(fp32 scalar, fp32 [1]): the sum of the per-row losses (their mean over the rows not ignored when `mean`), and
+    the factor the backward pass scales with (1 / number of rows not ignored, or 1)."""
+    _dev(loss_rows)
+    if loss_rows.dtype != torch.float32 or not loss_rows.is_contiguous() or target.numel() != loss_rows.numel():
+        raise ValueError("softmax_xent_reduce: loss_rows must be contiguous fp32 [rows] and target int64 [rows]")
+    out = torch.empty((), dtype=torch.float32, device=loss_rows.device)
+    scale = torch.empty(1, dtype=torch.float32, device=loss_rows.device)
+    _lib.require_device()
+    check(_lib.load().rtp_softmax_xent_reduce(_stream(), loss_rows.data_ptr(), target.data_ptr(), int(ignore_index),
+                                              loss_rows.numel(), int(mean), out.data_ptr(), scale.data_ptr()))
+    return out, scale
+
+
 def softmax_xent_bwd(logits: torch.Tensor, target: torch.Tensor, stats: torch.Tensor, dloss: torch.Tensor,
-                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """dlogits = (softmax(logits) - onehot(target)) * dloss[row]; dloss fp32 [rows], stride 0 or 1."""
+                     out: Optional[torch.Tensor] = None, scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """dlogits = (softmax(logits) - onehot(target)) * dloss[row] (* scale[0]); dloss fp32 [rows] with stride 0 or
+    1, or one element for all rows; scale: an fp32 device scalar."""
     _xent_check("softmax_xent_bwd", logits, target)
     rows, cols = logits.shape
-    if dloss.dtype != torch.float32 or dloss.numel() != rows or dloss.dim() != 1:
-        raise ValueError("softmax_xent_bwd: dloss must be fp32 [rows]")
+    if dloss.dtype != torch.float32 or dloss.numel() not in (1, rows) or dloss.dim() > 1:
+        raise ValueError("softmax_xent_bwd: dloss must be fp32 [rows] or a single fp32 element")
     if stats.dtype != torch.float32 or stats.shape != (rows, 2) or not stats.is_contiguous():
         raise ValueError("softmax_xent_bwd: stats must be the contiguous fp32 [rows, 2] of softmax_xent_fwd")
-    if rows > 1 and dloss.stride(0) not in (0, 1):
-        dloss = dloss.contiguous()
-    stride = dloss.stride(0) if rows > 1 else 0
+    stride = 0 if (dloss.numel() == 1 or dloss.dim() == 0) else dloss.stride(0)
+    if rows > 1 and stride not in (0, 1):
+        raise ValueError("softmax_xent_bwd: dloss stride must be 0 or 1")
+    if scale is not None and (scale.dtype != torch.float32 or scale.numel() != 1 or scale.device != logits.device):
+        raise ValueError("softmax_xent_bwd: scale must be one fp32 element on the logits' device")
     if out is None:
-        out = torch.empty((rows, cols), dtype=logits.dtype, device=logits.device)
-    elif out.shape != logits.shape or out.dtype != logits.dtype or not softmax_xent_supported(out):
-        raise ValueError("softmax_xent_bwd: out must match logits")
+        out = torch.empty(rows, cols, dtype=logits.dtype, device=logits.device)
+    elif out.shape != logits.shape or out.dtype != logits.dtype or (cols > 1 and out.stride(1) != 1):
+        raise ValueError("softmax_xent_bwd: out must match the logits' shape and dtype")
     _lib.require_device()
-    check(_lib.load().rtp_softmax_xent_bwd(_stream(), dtype_code(logits.dtype), logits.data_ptr(), logits.stride(0),
-                                           rows, cols, target.data_ptr(), stats.data_ptr(), dloss.data_ptr(), stride,
-                                           out.data_ptr(), out.stride(0)))
+    check(_lib.load().rtp_softmax_xent_bwd(_stream(), dtype_code(logits.dtype), logits.data_ptr(),
+                                           logits.stride(0) if rows > 1 else cols, rows, cols, target.data_ptr(),
+                                           stats.data_ptr(), dloss.data_ptr(), 0 if rows <= 1 else stride,
+                                           _ptr(scale), out.data_ptr(), out.stride(0) if rows > 1 else cols))
     return out
 
 

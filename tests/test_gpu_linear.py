@@ -220,3 +220,33 @@ def test_backward_that_raises_leaves_no_deferred_weight_gradients_behind():
         assert rel_err(torch.cat([l.weight.grad for l in a.linears], 0), want_a) <= 1e-5
     finally:
         ring.set_wgrad_overlap(False)
+
+
+def test_column_relu_mlp_with_dropout_on_the_hidden_activations():
+    """lin2(dropout(relu(lin1(x)))) (rtp/models/transformer_lm_rtp.py:88-89 with dropout > 0): the keep mask is drawn
+    by torch's device generator inside the function; redrawing it from the same generator state gives the
+    reference computation on the CPU."""
+    from rtp_amd import emulate_shards
+    from rtp_amd.module.linear import ColumnParallelLinear, column_relu_mlp
+    torch.manual_seed(4)
+    m1, m2 = nn.Linear(32, 48), nn.Linear(48, 32)
+    with emulate_shards(4):
+        l1 = ColumnParallelLinear(32, 48, linear_layer=m1, device=DEV)
+        l2 = ColumnParallelLinear(48, 32, linear_layer=m2, device=DEV)
+    x, g = torch.randn(10, 32), torch.randn(10, 32)
+    p = 0.25
+    torch.cuda.manual_seed(77)
+    xd = x.to(DEV).requires_grad_()
+    y = column_relu_mlp(xd, l1, l2, dropout_p=p)
+    y.backward(g.to(DEV))
+    torch.cuda.manual_seed(77)
+    keep = torch.empty(10, 48, device=DEV).bernoulli_(1.0 - p).mul_(1.0 / (1.0 - p)).cpu()
+    assert 0 < int((keep == 0).sum()) < keep.numel()
+    xr = x.clone().requires_grad_()
+    ref = m2(torch.relu(m1(xr)) * keep)
+    ref.backward(g)
+    assert_close(y, ref, torch.float32, "output")
+    assert_close(xd.grad, xr.grad, torch.float32, "dx")
+    assert_close(torch.cat([s.weight.grad for s in l1.linears], 0), m1.weight.grad, torch.float32, "dW1")
+    assert_close(torch.cat([s.weight.grad for s in l2.linears], 0), m2.weight.grad, torch.float32, "dW2")
+    assert_close(torch.cat([s.bias.grad for s in l1.linears], 0), m1.bias.grad, torch.float32, "db1")

@@ -263,18 +263,21 @@ def test_lm_rank_state_dicts_round_trip_on_device():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_lm_embedding_scale_and_positions_on_the_gather_are_bit_identical(dtype, monkeypatch):
-    """The model lets the embedding gather apply * sqrt(ninp) and + pe (transformer_lm_rtp.py:27-28, :49); with
-    RTP_EMBED_FUSE=0 the three steps run as separate operations.  Logits and every gradient must not change."""
+def test_lm_embedding_scale_and_positions_on_the_gather_are_bit_identical(dtype):
+    """The model lets the embedding gather apply * sqrt(ninp) and + pe (transformer_lm_rtp.py:27-28, :49).  A twin
+    whose embedding layer has not adopted the positional layer runs the three steps as the reference does (gather,
+    multiply, add: separate operations); logits and every gradient must be the same bits."""
     V, D, H, Fd, n_dec, L, N = 96, 64, 4, 64, 2, 12, 5
     gen = torch.Generator().manual_seed(1)
     ids = torch.randint(0, V, (L, N), generator=gen).to(DEV)
     tgt = torch.randint(0, V, (L, N), generator=gen).to(DEV)
     results = []
-    for fuse in ("1", "0"):
-        monkeypatch.setenv("RTP_EMBED_FUSE", fuse)
+    for fused in (True, False):
         lm, _ = build_pair(V, D, H, Fd, n_dec, 4, dtype)
-        assert lm[1].added_upstream == (fuse == "1")
+        assert lm[1].added_upstream and lm[0].positional is lm[1]
+        if not fused:
+            object.__setattr__(lm[0], "positional", None)
+            lm[1].added_upstream = False
         logits = lm(ids)
         F.cross_entropy(logits.float().view(-1, V), tgt.view(-1)).backward()
         results.append((logits.detach(), gathered_grads(lm, 4)))

@@ -70,12 +70,45 @@ def test_cross_entropy_extreme_logits_stay_finite():
     assert_close(xd.grad, ref_in.grad, torch.float32, "dlogits")
 
 
-def test_cross_entropy_falls_back_for_unsupported_layouts():
-    from rtp_amd import ops
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,cols", [(6, 37), (3, 1), (17, 1001)])
+def test_cross_entropy_ragged_class_counts(dtype, rows, cols):
+    """Class counts that are not whole 16-byte vectors take the element-wise kernels: same results, no torch path."""
     from rtp_amd.module.loss import cross_entropy
-    x = torch.randn(6, 37, device=DEV)
-    t = torch.randint(0, 37, (6,), device=DEV)
-    assert not ops.softmax_xent_supported(x)
-    assert torch.equal(cross_entropy(x, t), F.cross_entropy(x, t))
-    with pytest.raises(ValueError):
-        ops.softmax_xent_fwd(x, t)
+    store, target = _case(rows, cols, dtype, 3 * rows + cols)
+    ref_in = store.float().clone().requires_grad_()
+    ref = F.cross_entropy(ref_in, target)
+    ref.backward()
+    x = store.to(DEV).requires_grad_()
+    loss = cross_entropy(x, target.to(DEV).int())     # int32 class indices are accepted
+    loss.backward()
+    assert abs(loss.item() - ref.item()) <= 1e-5 * max(abs(ref.item()), 1e-3)
+    assert_close(x.grad, ref_in.grad, dtype, "dlogits")
+
+
+def test_cross_entropy_default_ignore_index_and_invalid_targets():
+    """-100 is ignored by default and the mean runs over the other rows (nn.CrossEntropyLoss's defaults); a target
+    outside the classes that is not the ignore index poisons the loss with NaN instead of being skipped silently."""
+    from rtp_amd._lib import RtpError
+    from rtp_amd.module.loss import CrossEntropyLoss, cross_entropy
+    rows, cols = 40, 64
+    store, target = _case(rows, cols, torch.float32, 9)
+    target[::4] = -100
+    ref_in = store.clone().requires_grad_()
+    ref = torch.nn.CrossEntropyLoss()(ref_in, target)
+    ref.backward()
+    x = store.to(DEV).requires_grad_()
+    out = CrossEntropyLoss()(x, target.to(DEV))
+    out.backward()
+    assert_close(out, ref, torch.float32, "loss")
+    assert_close(x.grad, ref_in.grad, torch.float32, "dlogits")
+    bad = target.clone()
+    bad[1] = cols + 3
+    assert torch.isnan(cross_entropy(store.to(DEV), bad.to(DEV)))
+    rows_loss = cross_entropy(store.to(DEV), bad.to(DEV), reduction="none")
+    assert torch.isnan(rows_loss[1]) and torch.isfinite(rows_loss[2])
+    all_ignored = torch.full((rows,), -100)
+    assert torch.isnan(cross_entropy(store.to(DEV), all_ignored.to(DEV)))          # 0 / 0, as torch
+    assert float(cross_entropy(store.to(DEV), all_ignored.to(DEV), reduction="sum")) == 0.0
+    with pytest.raises(RtpError):
+        cross_entropy(store, target)                                             # CPU tensors: no fallback

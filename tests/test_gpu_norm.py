@@ -10,7 +10,7 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("rows,cols", [(37, 2048), (5, 64), (1024, 512), (3, 8), (9, 1288)])
+@pytest.mark.parametrize("rows,cols", [(37, 2048), (5, 64), (1024, 512), (3, 8), (9, 1288), (6, 4096), (5, 3080)])
 def test_add_layer_norm_matches_torch(dtype, rows, cols):
     from rtp_amd import ops
     from rtp_amd.module.norm import add_layer_norm
@@ -43,16 +43,23 @@ def test_add_layer_norm_matches_torch(dtype, rows, cols):
     assert_close(dev_norm.bias.grad, b.grad, dtype, "dbeta")
 
 
-def test_add_layer_norm_falls_back_for_unsupported_rows():
+def test_add_layer_norm_refuses_rows_the_kernels_cannot_take():
+    """There is one implementation: rows that are not whole 16-byte vectors, or wider than the kernels hold in
+    registers, raise instead of going through torch."""
     from rtp_amd import ops
+    from rtp_amd._lib import RtpError
     from rtp_amd.module.norm import add_layer_norm
+    assert ops.layernorm_supported(torch.bfloat16, 8192) and ops.layernorm_supported(torch.float32, 4096)
     assert not ops.layernorm_supported(torch.float32, 4100)
     assert not ops.layernorm_supported(torch.bfloat16, 36)
     assert not ops.layernorm_supported(torch.float32, 38)
     norm = nn.LayerNorm(38).to(DEV)
     x = torch.randn(4, 38, device=DEV)
     r = torch.randn(4, 38, device=DEV)
-    assert torch.equal(add_layer_norm(x, r, norm), norm(x + r))
+    with pytest.raises(RtpError, match="16-byte"):
+        add_layer_norm(x, r, norm)
+    with pytest.raises(RtpError):
+        add_layer_norm(torch.randn(4, 64), torch.randn(4, 64), nn.LayerNorm(64))     # CPU tensors
 
 
 def test_layer_norm_parameter_gradients_reduced_at_the_end_of_backward():
