@@ -66,6 +66,39 @@ __global__ __launch_bounds__(256) void sort_prep_kernel(const int64_t* ids, long
   }
 }
 
+// (id, position) pairs of up to kSortLdsMax token ids sorted by one workgroup in LDS: a bitonic network over the
+// 64-bit words id << 32 | position (all different, so the order is total and the result is the stable sort by id).
+// A step's 1024 ids take 55 compare-exchange rounds of a few hundred nanoseconds each; a device-wide radix sort
+// spends several launches on them.  Slots beyond n hold the largest word and stay at the end.
+constexpr int kSortLdsMax = 8192;  // 64 KiB of LDS
+constexpr int kSortThreads = 1024;
+__global__ __launch_bounds__(kSortThreads) void sort_ids_lds_kernel(const int64_t* ids, int n, int npow2, int* keys,
+                                                                    int* vals) {
+  extern __shared__ unsigned long long sort_words[];
+  for (int i = threadIdx.x; i < npow2; i += kSortThreads)
+    sort_words[i] = i < n ? ((unsigned long long)(unsigned)(int)ids[i] << 32) | (unsigned)i : ~0ull;
+  __syncthreads();
+  for (int k = 2; k <= npow2; k <<= 1) {
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      for (int t = threadIdx.x; t < (npow2 >> 1); t += kSortThreads) {
+        const int lo = ((t & ~(j - 1)) << 1) | (t & (j - 1)), hi = lo | j;
+        const unsigned long long a = sort_words[lo], b = sort_words[hi];
+        const bool ascending = (lo & k) == 0;
+        if ((a > b) == ascending) {
+          sort_words[lo] = b;
+          sort_words[hi] = a;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  for (int i = threadIdx.x; i < n; i += kSortThreads) {
+    const unsigned long long w = sort_words[i];
+    keys[i] = (int)(unsigned)(w >> 32);
+    vals[i] = (int)(unsigned)(w & 0xffffffffull);
+  }
+}
+
 __global__ __launch_bounds__(256) void zero_rows_kernel(char* base, long ld_bytes, long row_bytes, long rows,
                                                         long group_bytes) {
   const long r = blockIdx.x;
@@ -210,6 +243,16 @@ extern "C" int rtp_embedding_sort_ids(void* stream, const int64_t* ids, int64_t 
     return fail(RTP_ERR_WORKSPACE, "rtp_embedding_sort_ids: workspace %zu < required %zu", workspace_bytes, L.total);
   char* w = (char*)workspace;
   hipStream_t s = (hipStream_t)stream;
+  if (n_ids <= kSortLdsMax) {
+    int npow2 = 2;
+    while (npow2 < n_ids) npow2 <<= 1;
+    ProfileScope prof(s, "embedding_sort_ids", 0.0, 16.0 * (double)n_ids);
+    hipLaunchKernelGGL(sort_ids_lds_kernel, dim3(1), dim3(kSortThreads), (size_t)npow2 * 8, s, ids, (int)n_ids, npow2,
+                       (int*)(w + L.keys_out), (int*)(w + L.vals_out));
+    RTP_LAUNCH_CHECK();
+    return RTP_OK;
+  }
+  // more ids than one workgroup's LDS holds: the device-wide radix sort of rocPRIM
   hipLaunchKernelGGL(sort_prep_kernel, dim3((unsigned)ceil_div(n_ids, 256)), dim3(256), 0, s, ids, (long)n_ids,
                      (int*)(w + L.keys_in), (int*)(w + L.vals_in));
   RTP_LAUNCH_CHECK();

@@ -111,3 +111,25 @@ def test_embedding_scaled_positional_is_bit_exact(dtype, ws):
         assert torch.equal(dw, want_t)
     with pytest.raises(ValueError):
         layer.forward_scaled_positional(ids.to(DEV), scale, pe[:seq - 1].to(DEV))
+
+
+@pytest.mark.parametrize("n,vocab", [(1, 5), (2, 3), (1000, 7), (1024, 10240), (4097, 50), (8192, 1 << 30), (8193, 100),
+                                     (40000, 977)])
+def test_sorted_token_ids_are_the_stable_sort_by_id(n, vocab):
+    """rtp_embedding_sort_ids leaves (id, position) pairs ordered by id, equal ids by ascending position -- the order
+    the scatter-add sums in.  Up to 8192 ids are sorted by one workgroup in LDS, more by the device-wide radix sort."""
+    from rtp_amd import _lib
+    gen = torch.Generator().manual_seed(n)
+    ids = torch.randint(0, vocab, (n,), generator=gen)
+    lib = _lib.load()
+    _lib.require_device()
+    nbytes = lib.rtp_embedding_scatter_workspace_bytes(n)
+    ws = torch.zeros(nbytes, dtype=torch.uint8, device=DEV)
+    dev_ids = ids.to(DEV)
+    _lib.check(lib.rtp_embedding_sort_ids(torch.cuda.current_stream().cuda_stream, dev_ids.data_ptr(), n, ws.data_ptr(),
+                                          nbytes))
+    arr = (n * 4 + 255) // 256 * 256
+    keys = ws[2 * arr:2 * arr + 4 * n].view(torch.int32).cpu()
+    vals = ws[3 * arr:3 * arr + 4 * n].view(torch.int32).cpu()
+    order = torch.sort(ids, stable=True).indices
+    assert torch.equal(keys.long(), ids[order]) and torch.equal(vals.long(), order)
