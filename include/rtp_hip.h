@@ -45,6 +45,61 @@ int rtp_abi_version(void);
 int rtp_device_check(char* name_out, int name_len);
 
 /* ---------------------------------------------------------------------------------------------
+ * One rotated column-parallel Linear, all shards, one launch per product (reference: the per-layer ring loop of
+ * ColumnParallelLinear.forward, rtp/module/linear.py:211-222 -- fetch the next shard, multiply, concatenate -- and its
+ * backward through _WeightParallelRegion_before/_after, rtp/module/collectives.py:264-317).  The layer is described by
+ * where its shards live: `home` is [shards, numel] flat shard buffers in `dtype` (shard g at home + g * numel), each
+ * holding the weight [n_s, k] at element w_off and, if bias_off >= 0, the bias [n_s] there.  The product kernel
+ * walks (shard, tile) work items in the ring order of rank 0 and streams every shard straight from home through
+ * its LDS stages: nothing is copied or staged in device memory.
+ *   fwd: y[rows, shards * n_s] (column block g) = x[rows, k] W_g^T + b_g; flags: RTP_GEMM_RELU (through a ReLU),
+ *        RTP_GEMM_OUT_F32 (y is fp32 although the shards are bf16).
+ *   bwd: either half may be left out (dx == NULL / grads == NULL), so that the two can go to different streams.
+ *        dx[rows, k] = (dx_init +) sum_g dy[:, block g] W_g, optionally masked by relu_gate > 0 (the layer's input
+ *        when it came out of a ReLU); dx_flags: RTP_GEMM_OUT_F32 / RTP_GEMM_CIN_F32 when dx / dx_init are fp32
+ *        running sums of a layer whose shards arrive in several runs; grads is [shards, numel] like home: weight gradient dy[:, block g]^T x at
+ *        w_off and the bias gradient at bias_off of row g, added to what is there when `accumulate`.  sgd_master /
+ *        sgd_weights ([shards, numel] fp32 / `dtype`, laid out like home) ask for the clip + SGD update of rtp_gemm's
+ *        fused epilogue; sgd_skip_grad_store then leaves the weight gradient unwritten.  colsum_workspace is only
+ *        read when the bias gradient cannot ride in the weight-gradient launch (rtp_colsum_workspace_bytes(rows,
+ *        shards * n_s) bytes).  What operands of odd alignment could not get is reported instead of refused when
+ *        `done` (host memory, may be NULL) is given: it receives RTP_ROTATED_BIAS_DONE if the bias gradient was
+ *        produced (always, given a workspace) and RTP_ROTATED_SGD_DONE if the update was applied; the caller then
+ *        does the missing part itself (rtp_colsum, rtp_sgd_step).  Without `done` a part that cannot be done is
+ *        an error.
+ * --------------------------------------------------------------------------------------------- */
+typedef struct {
+  const void* home;
+  int64_t numel, shards;
+  int64_t w_off, bias_off; /* bias_off < 0: no bias */
+  int64_t n_s, k;
+} rtp_rotated_linear;
+
+typedef struct {
+  void* dx; /* may be NULL */
+  int64_t ld_dx;
+  const void* dx_init; /* may be NULL */
+  int64_t ld_dx_init;
+  const void* relu_gate; /* may be NULL */
+  int64_t ld_relu_gate;
+  int64_t dx_flags;
+  void* grads; /* may be NULL */
+  int32_t accumulate, sgd_skip_grad_store;
+  void* sgd_master;  /* may be NULL */
+  void* sgd_weights; /* may be NULL */
+  float sgd_lr, sgd_clip;
+  void* colsum_workspace; /* may be NULL */
+  size_t colsum_workspace_bytes;
+  int32_t* done; /* may be NULL */
+} rtp_rotated_linear_bwd_args;
+enum { RTP_ROTATED_BIAS_DONE = 1, RTP_ROTATED_SGD_DONE = 2 };
+
+int rtp_rotated_linear_fwd(void* stream, int dtype, const rtp_rotated_linear* layer, const void* x, int64_t ldx,
+                           int64_t rows, void* y, int64_t ldy, int flags);
+int rtp_rotated_linear_bwd(void* stream, int dtype, const rtp_rotated_linear* layer, const void* dy, int64_t ldy,
+                           const void* x, int64_t ldx, int64_t rows, const rtp_rotated_linear_bwd_args* args);
+
+/* ---------------------------------------------------------------------------------------------
  * GEMM   C[z][m,n] = epilogue( alpha * sum_k A[z](m,k) * B[z](n,k) )
  *
  * Stands in for F.linear inside the shard modules (rtp/module/linear.py:216, :385;

@@ -22,6 +22,7 @@ GEMM_RELU = 4
 GEMM_STREAM_OUT = 8
 GEMM_ROWSUM_ACCUM = 16
 GEMM_SGD_SKIP_OUT = 32
+ROTATED_BIAS_DONE, ROTATED_SGD_DONE = 1, 2
 GATE_WGRAD_STATIC_MAX_BYTES = 8 << 20  # RTP_GATE_WGRAD_STATIC_MAX_BYTES of include/rtp_hip.h
 
 
@@ -55,6 +56,22 @@ class GemmDesc(C.Structure):
     ]
 
 
+class RotatedLinear(C.Structure):
+    """rtp_rotated_linear of include/rtp_hip.h: where the shards of a column-parallel layer live."""
+    _fields_ = [("home", C.c_void_p), ("numel", C.c_int64), ("shards", C.c_int64), ("w_off", C.c_int64),
+                ("bias_off", C.c_int64), ("n_s", C.c_int64), ("k", C.c_int64)]
+
+
+class RotatedLinearBwdArgs(C.Structure):
+    """rtp_rotated_linear_bwd_args of include/rtp_hip.h."""
+    _fields_ = [("dx", C.c_void_p), ("ld_dx", C.c_int64), ("dx_init", C.c_void_p), ("ld_dx_init", C.c_int64),
+                ("relu_gate", C.c_void_p), ("ld_relu_gate", C.c_int64), ("dx_flags", C.c_int64), ("grads", C.c_void_p),
+                ("accumulate", C.c_int32), ("sgd_skip_grad_store", C.c_int32), ("sgd_master", C.c_void_p),
+                ("sgd_weights", C.c_void_p), ("sgd_lr", C.c_float), ("sgd_clip", C.c_float),
+                ("colsum_workspace", C.c_void_p), ("colsum_workspace_bytes", C.c_size_t),
+                ("done", C.POINTER(C.c_int32))]
+
+
 class KernelStat(C.Structure):
     _fields_ = [("name", C.c_char * 64), ("launches", C.c_int64), ("total_ms", C.c_double),
                 ("flops", C.c_double), ("bytes", C.c_double)]
@@ -67,6 +84,9 @@ PROTOTYPES = {
     "rtp_last_error": (C.c_char_p, []),
     "rtp_abi_version": (_i, []),
     "rtp_device_check": (_i, [C.c_char_p, _i]),
+    "rtp_rotated_linear_fwd": (_i, [_vp, _i, C.POINTER(RotatedLinear), _vp, _i64, _i64, _vp, _i64, _i]),
+    "rtp_rotated_linear_bwd": (_i, [_vp, _i, C.POINTER(RotatedLinear), _vp, _i64, _vp, _i64, _i64,
+                                    C.POINTER(RotatedLinearBwdArgs)]),
     "rtp_gemm": (_i, [_vp, _i, C.POINTER(GemmDesc)]),
     "rtp_gemm_rowsum_fused": (_i, [_i, C.POINTER(GemmDesc)]),
     "rtp_gemm_sgd_fused": (_i, [_i, C.POINTER(GemmDesc)]),

@@ -161,7 +161,7 @@ using namespace rtp;
 
 extern "C" const char* rtp_last_error(void) { return error_buffer(); }
 
-extern "C" int rtp_abi_version(void) { return 1; }
+extern "C" int rtp_abi_version(void) { return 2; }
 
 extern "C" int rtp_device_check(char* name_out, int name_len) {
   int dev = 0;

@@ -12,7 +12,7 @@ from typing import Optional
 
 import torch
 
-from .. import ops
+from .. import _lib, ops
 
 
 def _rows(t: torch.Tensor):
@@ -21,29 +21,14 @@ def _rows(t: torch.Tensor):
 
 
 def col_fwd(x2, flat, w_off, n_s, k, bias_off, out, col0, *, relu=False):
-    """out[:, col0 + g*n_s : col0 + (g+1)*n_s] = x2 @ W_g^T (+ b_g), g over the run."""
-    cnt, numel = flat.shape
-    es = flat.element_size()
-    m, _, lda = _rows(x2)
-    _, _, ldc = _rows(out)
-    out_f32 = out.dtype == torch.float32 and flat.dtype != torch.float32
-    osz = 4 if out_f32 else es
-    ops.gemm_raw(flat.dtype, a=x2.data_ptr(), b=flat.data_ptr() + w_off * es, c_out=out.data_ptr() + col0 * osz,
-                 bias=None if bias_off is None else flat.data_ptr() + bias_off * es, m=m, n=n_s, k=k, lda=lda, ldb=k,
-                 ldc=ldc, a_kcontig=True, b_kcontig=True, relu=relu, out_f32=out_f32, groups=cnt, b_sg=numel,
-                 bias_sg=numel, c_sg=n_s)
+    """out[:, col0 + g*n_s : col0 + (g+1)*n_s] = x2 @ W_g^T (+ b_g), g over the run: the run is a rotated
+    column-parallel layer of its own (rtp_rotated_linear_fwd) whose outputs start at column col0."""
+    ops.rotated_linear_fwd(x2, flat, w_off, bias_off, n_s, k, out[:, col0:], relu=relu)
 
 
 def col_dgrad(dy2, flat, w_off, n_s, k, out, col0, c_in: Optional[torch.Tensor] = None, gate=None):
     """out[M, k] = (c_in +) sum_g dy2[:, col0 + g*n_s : ...] @ W_g   (contraction segmented over shards)."""
-    cnt, numel = flat.shape
-    es = flat.element_size()
-    m, _, lda = _rows(dy2)
-    _, _, ldc = _rows(out)
-    kw = ops._epilogue_args(flat.dtype, out, c_in, None, gate)
-    ops.gemm_raw(flat.dtype, a=dy2.data_ptr() + col0 * es, b=flat.data_ptr() + w_off * es, c_out=out.data_ptr(), m=m,
-                 n=k, k=n_s, lda=lda, ldb=k, ldc=ldc, a_kcontig=True, b_kcontig=False, ksegs=cnt, a_sk=n_s,
-                 b_sk=numel, **kw)
+    ops.rotated_linear_bwd(dy2[:, col0:], None, flat, w_off, None, n_s, k, dx=out, dx_init=c_in, relu_gate=gate)
 
 
 def _fused(store, accumulate, first, cnt, w_off, length):
@@ -83,15 +68,19 @@ def col_wgrad(dy2, x2, grads, first, w_off, n_s, k, col0, cnt, accumulate, b_off
         if b_off is not None:
             col_bgrad(dy2, grads, first, b_off, n_s, col0, cnt, accumulate)
         return
-    # the bias gradient is the row sum of the product's first operand dy^T: the same launch adds it up
-    rs = None if b_off is None else grads.data_ptr() + (first * numel + b_off) * es
+    # one launch for the run (rtp_rotated_linear_bwd): the weight gradients, the bias gradients as the row sums of the
+    # product's first operand dy^T, and the optimiser's update where one asked for it
     kw = _fused(store, accumulate, first, cnt, w_off, n_s * k)
-    fused = ops.gemm_raw(grads.dtype, a=dy2.data_ptr() + col0 * es, b=x2.data_ptr(), c_out=c, m=n_s, n=k, k=m, lda=lda,
-                         ldb=ldb, ldc=k, a_kcontig=False, b_kcontig=False, groups=cnt, a_sg=n_s, c_sg=numel,
-                         c_in=c if accumulate else None, ld_cin=k, cin_sg=numel, stream_out=True,
-                         rowsum=rs, rowsum_sg=numel, rowsum_accum=accumulate, **kw)
-    _fused_done(store, kw)
-    if b_off is not None and not fused:
+    if kw:  # bound to the weight's own address; the entry point takes the run's base and adds w_off itself
+        kw = dict(sgd=kw["sgd"], sgd_master=kw["sgd_master"] - w_off * 4,
+                  sgd_weights=kw["sgd_weights"] - w_off * es if kw["sgd_weights"] else 0)
+    run = grads[first:first + cnt]  # the weight-gradient half reads no weights: the gradient rows give the layout
+    done = ops.rotated_linear_bwd(dy2[:, col0:], x2, run, w_off, b_off, n_s, k, grads=run, accumulate=accumulate, **kw)
+    if kw:
+        if not done & _lib.ROTATED_SGD_DONE:
+            kw["sgd"].missed = True
+        _fused_done(store, kw)
+    if b_off is not None and not done & _lib.ROTATED_BIAS_DONE:
         col_bgrad(dy2, grads, first, b_off, n_s, col0, cnt, accumulate)
 
 

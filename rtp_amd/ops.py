@@ -95,6 +95,80 @@ def gemm_raw(dtype: torch.dtype, *, a: int, b: int, c_out: int, m: int, n: int, 
     return fused
 
 
+def _rotated_layer(home: torch.Tensor, w_off: int, bias_off: Optional[int], n_s: int, k: int) -> "_lib.RotatedLinear":
+    if home.dim() != 2 or not home.is_contiguous():
+        raise ValueError("rotated_linear: home must be the contiguous [shards, numel] buffer of the layer")
+    _dev(home)
+    return _lib.RotatedLinear(home.data_ptr(), home.shape[1], home.shape[0], w_off, -1 if bias_off is None else bias_off,
+                              n_s, k)
+
+
+def rotated_linear_fwd(x2: torch.Tensor, home: torch.Tensor, w_off: int, bias_off: Optional[int], n_s: int, k: int,
+                       y: torch.Tensor, relu: bool = False) -> None:
+    """y[rows, shards * n_s] = x2 @ W_g^T + b_g for every shard g of `home` [shards, numel], one launch; y in the
+    shards' dtype or fp32."""
+    layer = _rotated_layer(home, w_off, bias_off, n_s, k)
+    rows, kk, ldx = _mat(x2, "x")
+    ry, ny, ldy = _mat(y, "y")
+    if kk != k or ry != rows or ny < n_s * home.shape[0] or x2.dtype != home.dtype or \
+            y.dtype not in (home.dtype, torch.float32):
+        raise ValueError("rotated_linear_fwd: x [rows, k] in the shards' dtype, y [rows, >= shards * n_s] (or fp32)")
+    flags = (GEMM_RELU if relu else 0) | (GEMM_OUT_F32 if y.dtype != home.dtype else 0)
+    _lib.require_device()
+    check(_lib.load().rtp_rotated_linear_fwd(_stream(), dtype_code(home.dtype), C.byref(layer), x2.data_ptr(), ldx, rows,
+                                             y.data_ptr(), ldy, flags))
+
+
+def rotated_linear_bwd(dy2: torch.Tensor, x2: Optional[torch.Tensor], home: torch.Tensor, w_off: int,
+                       bias_off: Optional[int], n_s: int, k: int, *, dx: Optional[torch.Tensor] = None,
+                       dx_init: Optional[torch.Tensor] = None, relu_gate: Optional[torch.Tensor] = None,
+                       grads: Optional[torch.Tensor] = None, accumulate: bool = False, sgd: Optional["FusedSgd"] = None,
+                       sgd_master: int = 0, sgd_weights: int = 0) -> int:
+    """The backward of rotated_linear_fwd, either half or both: dx [rows, k] (= dx_init + sum over the shards, masked
+    where relu_gate <= 0) and / or the gradient rows `grads` [shards, numel] (weights, and the bias where the layer
+    has one), with the clip + SGD update `sgd` applied in the same launch to the fp32 parameters at address
+    sgd_master and their compute-dtype copy at sgd_weights (both laid out like home).  Returns the library's
+    done flags (ROTATED_BIAS_DONE, ROTATED_SGD_DONE): what is missing there is left to the caller."""
+    layer = _rotated_layer(home, w_off, bias_off, n_s, k)
+    rows, ny, ldy = _mat(dy2, "dy")
+    if ny < n_s * home.shape[0] or dy2.dtype != home.dtype:
+        raise ValueError("rotated_linear_bwd: dy must be [rows, >= shards * n_s] in the shards' dtype")
+    a = _lib.RotatedLinearBwdArgs()
+    done = C.c_int32(0)
+    a.done = C.pointer(done)
+    if dx is not None:
+        r, c, ld = _mat(dx, "dx")
+        if (r, c) != (rows, k):
+            raise ValueError("rotated_linear_bwd: dx must be [rows, k]")
+        a.dx, a.ld_dx = dx.data_ptr(), ld
+        for name, t in (("dx_init", dx_init), ("relu_gate", relu_gate)):
+            if t is not None:
+                r, c, ld = _mat(t, name)
+                if (r, c) != (rows, k):
+                    raise ValueError(f"rotated_linear_bwd: {name} must match dx")
+                setattr(a, name, t.data_ptr())
+                setattr(a, "ld_" + name, ld)
+        for t, what in ((dx, "dx"), (dx_init, "dx_init")):
+            if t is not None and t.dtype not in (home.dtype, torch.float32):
+                raise TypeError(f"rotated_linear_bwd: {what} must be {home.dtype} or float32")
+        if relu_gate is not None and relu_gate.dtype != home.dtype:
+            raise TypeError("rotated_linear_bwd: relu_gate must be in the shards' dtype")
+        a.dx_flags = (GEMM_OUT_F32 if dx.dtype != home.dtype else 0) | \
+            (GEMM_CIN_F32 if dx_init is not None and dx_init.dtype != home.dtype else 0)
+    if grads is not None:
+        if grads.shape != home.shape or grads.dtype != home.dtype or not grads.is_contiguous() or x2 is None:
+            raise ValueError("rotated_linear_bwd: grads must be laid out like home, and the layer's input is needed")
+        a.grads, a.accumulate = grads.data_ptr(), int(accumulate)
+        if sgd is not None:
+            a.sgd_master, a.sgd_weights = sgd_master, (sgd_weights or None)
+            a.sgd_lr, a.sgd_clip, a.sgd_skip_grad_store = sgd.lr, sgd.clip, int(not sgd.keep_grads)
+    xr = _mat(x2, "x") if x2 is not None else (rows, k, k)
+    _lib.require_device()
+    check(_lib.load().rtp_rotated_linear_bwd(_stream(), dtype_code(home.dtype), C.byref(layer), dy2.data_ptr(), ldy,
+                                             _ptr(x2), xr[2], rows, C.byref(a)))
+    return done.value
+
+
 def _epilogue_args(dtype, out, c_in, bias, gate):
     kw = {}
     if out.dtype == torch.float32 and dtype != torch.float32:

@@ -3,6 +3,7 @@ reference tests' gather rules for the gradients (tests/test_linear.py:117-186)."
 import pytest
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 from gpu_util import DEV, assert_close, rel_err
 from oracle import rtp_oracle as O
@@ -250,3 +251,56 @@ def test_column_relu_mlp_with_dropout_on_the_hidden_activations():
     assert_close(torch.cat([s.weight.grad for s in l1.linears], 0), m1.weight.grad, torch.float32, "dW1")
     assert_close(torch.cat([s.weight.grad for s in l2.linears], 0), m2.weight.grad, torch.float32, "dW2")
     assert_close(torch.cat([s.bias.grad for s in l1.linears], 0), m1.bias.grad, torch.float32, "db1")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,n_s,k,ws,bias", [(1024, 256, 2048, 8, True), (320, 32, 64, 4, True), (64, 24, 8, 1, False),
+                                                (77, 40, 72, 3, True)])
+def test_rotated_linear_entry_points_against_torch(dtype, rows, n_s, k, ws, bias):
+    """rtp_rotated_linear_fwd / _bwd through the C ABI on a flat [shards, numel] layer (the reference's per-layer ring
+    loop, rtp/module/linear.py:211-222, and its backward) against F.linear on the unsharded weight: outputs, input
+    gradient with an initial value and a ReLU mask, weight and bias gradients, and the fused clip + SGD update."""
+    from rtp_amd import _lib, ops
+    gen = torch.Generator().manual_seed(rows + n_s)
+    numel = n_s * k + (n_s if bias else 0) + 8            # some unrelated tail in every flat shard
+    home = (torch.randn(ws, numel, generator=gen) * 0.1).to(dtype)
+    w = home[:, :n_s * k].reshape(ws * n_s, k).float()
+    b = home[:, n_s * k:n_s * k + n_s].reshape(-1).float() if bias else None
+    x = torch.randn(rows, k, generator=gen).to(dtype)
+    dy = torch.randn(rows, ws * n_s, generator=gen).to(dtype)
+    init = torch.randn(rows, k, generator=gen).to(dtype)
+    gate = torch.randn(rows, k, generator=gen).to(dtype)
+    hd, xd, dyd = home.to(DEV), x.to(DEV), dy.to(DEV)
+    b_off = n_s * k if bias else None
+    y = torch.empty(rows, ws * n_s, dtype=dtype, device=DEV)
+    ops.rotated_linear_fwd(xd, hd, 0, b_off, n_s, k, y, relu=True)
+    assert_close(y, torch.relu(F.linear(x.float(), w, b)), dtype, "relu(x W^T + b)")
+    dx = torch.empty(rows, k, dtype=dtype, device=DEV)
+    ops.rotated_linear_bwd(dyd, None, hd, 0, b_off, n_s, k, dx=dx, dx_init=init.to(DEV), relu_gate=gate.to(DEV))
+    want = (init.float() + dy.float() @ w) * (gate.float() > 0)
+    assert_close(dx, want, dtype, "dx")
+    grads = torch.full((ws, numel), 7.0, dtype=dtype, device=DEV)
+    done = ops.rotated_linear_bwd(dyd, xd, hd, 0, b_off, n_s, k, grads=grads)
+    dw = (dy.float().T @ x.float()).view(ws, n_s * k)
+    assert_close(grads[:, :n_s * k], dw, dtype, "dW")
+    if bias:
+        if done & _lib.ROTATED_BIAS_DONE:
+            assert_close(grads[:, n_s * k:n_s * k + n_s], dy.float().sum(0).view(ws, n_s), dtype, "db")
+    assert bool((grads[:, -8:] == 7.0).all())            # nothing beyond the layer's own slices is touched
+    # the same launch with the optimiser's update in its epilogue: fp32 parameters and their copy
+    master = hd.float().clone()
+    weights = hd.clone()
+    sgd = ops.FusedSgd(lr=0.05, clip=0.5, keep_grads=False)
+    grads2 = torch.full((ws, numel), 7.0, dtype=dtype, device=DEV)
+    done = ops.rotated_linear_bwd(dyd, xd, hd, 0, b_off, n_s, k, grads=grads2, sgd=sgd, sgd_master=master.data_ptr(),
+                                  sgd_weights=weights.data_ptr() if dtype != torch.float32 else 0)
+    if done & _lib.ROTATED_SGD_DONE:
+        g = grads[:, :n_s * k].float().clamp(-0.5, 0.5)          # the gradient as the dtype holds it
+        want_m = hd.float()[:, :n_s * k] - 0.05 * g
+        assert torch.equal(master[:, :n_s * k], want_m)
+        assert torch.equal(master[:, n_s * k:], hd.float()[:, n_s * k:])
+        if dtype != torch.float32:
+            assert torch.equal(weights[:, :n_s * k], want_m.to(dtype))
+        assert bool((grads2[:, :n_s * k] == 7.0).all())          # consumed, not stored
+    else:
+        assert rows == 64 or k % 8                               # only shapes the vector kernel does not take
