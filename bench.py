@@ -380,6 +380,10 @@ def main():
                     help="one clip + SGD launch over all parameters after the backward pass, instead of applying the "
                          "update of every weight matrix in the epilogue of its weight-gradient product (the default: "
                          "bit-identical weights, the gradients of those matrices are never written or read back)")
+    ap.add_argument("--fused-head-loss", dest="fused_head_loss", action="store_true",
+                    help="logits layer and cross-entropy as one operation whose [tokens, vocab] logits never reach "
+                         "memory (statistics from the forward product's epilogue, the gradient from a second run of the "
+                         "product); measured slower than writing the logits once at this token count, so not the default")
     ap.add_argument("--no-wgrad-overlap", dest="wgrad_overlap", action="store_false",
                     help="launch weight / bias gradient kernels on the compute stream instead of a second stream "
                          "beside the input-gradient chain")
@@ -405,7 +409,7 @@ def main():
     import torch
     import torch.nn.functional as F
     from rtp_amd import _lib, ring, rotated_weight_bytes, staging_bytes
-    from rtp_amd.module.loss import cross_entropy
+    from rtp_amd.module.loss import cross_entropy, linear_cross_entropy
     from rtp_amd.optim import RotatedAdam, RotatedSGD
 
     dev = torch.device("cuda", 0)
@@ -427,8 +431,14 @@ def main():
 
     def step():
         opt.zero_grad()
-        logits = lm(ids)
-        loss = cross_entropy(logits.view(-1, c["vocab"]), tgt.view(-1))
+        if args.fused_head_loss:
+            hidden = ids
+            for layer in list(lm)[:-1]:
+                hidden = layer(hidden)
+            loss = linear_cross_entropy(hidden, lm[-1].linear, tgt.view(-1))
+        else:
+            logits = lm(ids)
+            loss = cross_entropy(logits.view(-1, c["vocab"]), tgt.view(-1))
         loss.backward()
         opt.step()
         loss_box[0] = loss.detach()  # detached: a live autograd graph would pin last step's AccumulateGrad nodes
@@ -534,6 +544,7 @@ def main():
                    "optimizer": args.optimizer, "rotation": args.rotation,
                    "sgd_overlapped_with_backward": bool(args.sgd_overlap),
                    "sgd_fused_into_weight_gradient_products": bool(args.sgd_fused),
+                   "logits_and_loss_fused": bool(args.fused_head_loss),
                    "wgrad_on_second_stream": bool(args.wgrad_overlap)},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK["bf16_mfma_tflops"], "unit": "TFLOP/s",
                      "frac": achieved / PEAK["bf16_mfma_tflops"],

@@ -99,6 +99,24 @@ int rtp_rotated_linear_fwd(void* stream, int dtype, const rtp_rotated_linear* la
 int rtp_rotated_linear_bwd(void* stream, int dtype, const rtp_rotated_linear* layer, const void* dy, int64_t ldy,
                            const void* x, int64_t ldx, int64_t rows, const rtp_rotated_linear_bwd_args* args);
 
+/* The logits layer together with its loss (reference: LinearLayer, rtp/models/transformer_lm_rtp.py:214-228, feeding
+ * nn.CrossEntropyLoss()(output.view(-1, ntokens), targets), benchmarks/rtp_benchmark.py:182): the [rows, classes]
+ * logits never reach memory.
+ *   xent_fwd: loss[r] and stats[r] = {max, sum exp} of row r's logits x[r] W^T + b over all shards (fp32 [rows],
+ *        fp32 [rows, 2]); loss and ignore_index as rtp_softmax_xent_fwd.  The logits product's epilogue leaves the
+ *        statistics of every 64-column block in the workspace (rtp_rotated_linear_xent_workspace_bytes, 8-byte
+ *        aligned) and a second small kernel combines them.  Feed loss to rtp_softmax_xent_reduce for a mean.
+ *   xent_bwd: dlogits[rows, classes] = (softmax - onehot(target)) * dloss[0] * scale[0] (scale may be NULL), from
+ *        the same product run once more with the row statistics; hand dlogits to rtp_rotated_linear_bwd as dy.
+ * A shard's column count n_s must be a multiple of 64; operands vector-aligned as for the fused update. */
+size_t rtp_rotated_linear_xent_workspace_bytes(const rtp_rotated_linear* layer, int64_t rows);
+int rtp_rotated_linear_xent_fwd(void* stream, int dtype, const rtp_rotated_linear* layer, const void* x, int64_t ldx,
+                                int64_t rows, const int64_t* target, int64_t ignore_index, float* loss, float* stats,
+                                void* workspace, size_t workspace_bytes);
+int rtp_rotated_linear_xent_bwd(void* stream, int dtype, const rtp_rotated_linear* layer, const void* x, int64_t ldx,
+                                int64_t rows, const int64_t* target, int64_t ignore_index, const float* stats,
+                                const float* dloss, const float* scale, void* dlogits, int64_t ld_dlogits);
+
 /* ---------------------------------------------------------------------------------------------
  * GEMM   C[z][m,n] = epilogue( alpha * sum_k A[z](m,k) * B[z](n,k) )
  *
@@ -179,6 +197,20 @@ typedef struct {
   void* sgd_master;
   void* sgd_weights;
   float sgd_lr, sgd_clip;
+  /* Softmax cross-entropy over the rows of the product, for a product that is the logits of a column-parallel layer
+   * (groups of n columns side by side, n a multiple of 64): what rtp_rotated_linear_xent_fwd / _bwd set up.
+   * xent_mode 1: instead of the logits, {max, sum exp} of every 64-column block go to xent_part [m][groups*n/64] (pairs
+   * of floats) and the logit of target[row] to xent_tlogit [m].  xent_mode 2: the logits are turned into
+   * (softmax - onehot(target)) * xent_dloss[0] * xent_scale[0] before they are stored, with xent_stats [m] = {max,
+   * sum exp} of each whole row; rows whose target equals xent_ignore (or lies outside the classes) get zeros. */
+  int32_t xent_mode, xent_reserved;
+  const int64_t* xent_target;
+  int64_t xent_ignore;
+  float* xent_part;
+  float* xent_tlogit;
+  const float* xent_stats;
+  const float* xent_dloss;
+  const float* xent_scale; /* may be NULL */
 } rtp_gemm_desc;
 
 int rtp_gemm(void* stream, int dtype, const rtp_gemm_desc* d);
@@ -418,6 +450,10 @@ int rtp_layernorm_bwd_finalize(void* stream, int dtype, const rtp_ln_final_item*
  * --------------------------------------------------------------------------------------------- */
 int rtp_softmax_xent_fwd(void* stream, int dtype, const void* logits, int64_t ld, int64_t rows, int64_t cols,
                          const int64_t* target, int64_t ignore_index, float* loss, float* stats);
+/* loss / stats of every row from the {max, sum exp} pairs of its 64-column blocks (part [rows, blocks] pairs) and the
+ * target's logit tlogit [rows]: the second step of rtp_rotated_linear_xent_fwd. */
+int rtp_softmax_xent_combine(void* stream, const float* part, int64_t blocks, const float* tlogit,
+                             const int64_t* target, int64_t ignore_index, int64_t rows, float* loss, float* stats);
 int rtp_softmax_xent_reduce(void* stream, const float* loss, const int64_t* target, int64_t ignore_index,
                             int64_t rows, int mean, float* out, float* scale);
 int rtp_softmax_xent_bwd(void* stream, int dtype, const void* logits, int64_t ld, int64_t rows, int64_t cols,

@@ -53,6 +53,9 @@ class GemmDesc(C.Structure):
         ("alpha", C.c_float), ("flags", C.c_int32), ("a_kcontig", C.c_int32), ("b_kcontig", C.c_int32),
         ("a_rowsum", C.c_void_p), ("rowsum_sg", C.c_int64),
         ("sgd_master", C.c_void_p), ("sgd_weights", C.c_void_p), ("sgd_lr", C.c_float), ("sgd_clip", C.c_float),
+        ("xent_mode", C.c_int32), ("xent_reserved", C.c_int32), ("xent_target", C.c_void_p), ("xent_ignore", C.c_int64),
+        ("xent_part", C.c_void_p), ("xent_tlogit", C.c_void_p), ("xent_stats", C.c_void_p), ("xent_dloss", C.c_void_p),
+        ("xent_scale", C.c_void_p),
     ]
 
 
@@ -87,6 +90,11 @@ PROTOTYPES = {
     "rtp_rotated_linear_fwd": (_i, [_vp, _i, C.POINTER(RotatedLinear), _vp, _i64, _i64, _vp, _i64, _i]),
     "rtp_rotated_linear_bwd": (_i, [_vp, _i, C.POINTER(RotatedLinear), _vp, _i64, _vp, _i64, _i64,
                                     C.POINTER(RotatedLinearBwdArgs)]),
+    "rtp_rotated_linear_xent_workspace_bytes": (_sz, [C.POINTER(RotatedLinear), _i64]),
+    "rtp_rotated_linear_xent_fwd": (_i, [_vp, _i, C.POINTER(RotatedLinear), _vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _sz]),
+    "rtp_rotated_linear_xent_bwd": (_i, [_vp, _i, C.POINTER(RotatedLinear), _vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _vp,
+                                         _i64]),
+    "rtp_softmax_xent_combine": (_i, [_vp, _vp, _i64, _vp, _vp, _i64, _i64, _vp, _vp]),
     "rtp_gemm": (_i, [_vp, _i, C.POINTER(GemmDesc)]),
     "rtp_gemm_rowsum_fused": (_i, [_i, C.POINTER(GemmDesc)]),
     "rtp_gemm_sgd_fused": (_i, [_i, C.POINTER(GemmDesc)]),

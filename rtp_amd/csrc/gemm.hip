@@ -77,6 +77,17 @@ struct GemmArgs {
   float* sgd_master;            // null, or the fp32 parameters the product updates (indexed like c_out)
   char* sgd_w;                  // null, or the compute-dtype copy of the parameters
   float sgd_lr, sgd_clip;
+  // softmax cross-entropy over the product's rows (the product is the logits of a column-parallel layer):
+  // mode 1 leaves per-(row, 64-column block) {max, sum exp} and the target's logit instead of the logits,
+  // mode 2 turns the logits into their gradient before they are stored
+  int xent_mode, xent_blocks;   // blocks: 64-column blocks per row over all groups
+  const long* xent_target;
+  long xent_ignore;
+  float2* xent_part;            // mode 1: [m][xent_blocks]
+  float* xent_tlogit;           // mode 1: [m]
+  const float2* xent_stats;     // mode 2: [m] {max, sum exp} of the whole row
+  const float* xent_dloss;      // mode 2: upstream gradient, one scalar
+  const float* xent_scale;      // mode 2: second scalar factor (1 / rows counted), or null
 };
 
 constexpr int kThreads = 256;
@@ -529,6 +540,22 @@ __device__ __forceinline__ void finish_tile(const GemmArgs& p, const float* ct, 
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] = t[e] > 0.0f ? v[e] : 0.0f;
       }
+      if (p.xent_mode == 2) {
+        // logits -> their cross-entropy gradient: (softmax - onehot(target)) * dloss (* scale); rows whose target
+        // is the ignore index or outside the classes get zeros
+        const long tg = p.xent_target[row];
+        const bool live = tg != p.xent_ignore && tg >= 0 && tg < (long)p.xent_blocks * 64;
+        const float2 st = p.xent_stats[row];
+        const float inv = 1.0f / st.y;
+        const float sc = live ? p.xent_dloss[0] * (p.xent_scale ? p.xent_scale[0] : 1.0f) : 0.0f;
+        const long gcol = (long)grp * p.n + col;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float gq = expf(to_f32(from_f32<T>(v[e])) - st.x) * inv;
+          if (gcol + e == tg) gq -= 1.0f;
+          v[e] = gq * sc;
+        }
+      }
       const long off = (long)row * p.ldc + col;
       if (master) {
         float w[8];
@@ -571,6 +598,47 @@ __device__ __forceinline__ void finish_tile(const GemmArgs& p, const float* ct, 
           reinterpret_cast<T*>(cbase)[off] = from_f32<T>(x);
       }
     }
+  }
+}
+
+// Epilogue of a logits product whose rows only feed a softmax cross-entropy (mode 1): thread r of the first BM
+// threads walks row r of the tile in LDS, 64 columns at a time, and leaves {max, sum exp(v - max)} of every
+// 64-column block in part[row][block] -- the block index runs over the layer's whole output row, group after
+// group, so the layout does not depend on the tile shape -- and the logit of the row's target where this tile
+// holds it.  The logits themselves are not stored.  v = alpha * acc + bias, rounded to T as the stored logits would
+// be, so that loss and gradient are those of the logits a separate product would have written.
+template <typename T, int BM, int BN, int NTHR>
+__device__ __forceinline__ void finish_tile_xent_stats(const GemmArgs& p, const float* ct, int m0, int n0, int tid,
+                                                       int grp) {
+  static_assert(BN % 64 == 0 && BM <= NTHR, "64-column blocks, one thread per tile row");
+  constexpr int CP = BN + 4;
+  if (tid >= BM) return;
+  const int row = m0 + tid;
+  if (row >= p.m) return;
+  const T* bias = p.bias ? reinterpret_cast<const T*>(p.bias) + grp * p.bias_sg : nullptr;
+  const long t = p.xent_target[row];
+  const long tcol = t - (long)grp * p.n;  // the target's column inside this group, if it is in [0, n)
+  const float* crow = ct + tid * CP;
+#pragma unroll
+  for (int b = 0; b < BN / 64; ++b) {
+    const int col0 = n0 + b * 64;
+    if (col0 >= p.n) break;
+    float mx = -INFINITY;
+    for (int j = 0; j < 64; ++j) {
+      float v = p.alpha * crow[b * 64 + j];
+      if (bias) v += to_f32(bias[col0 + j]);
+      v = to_f32(from_f32<T>(v));
+      mx = fmaxf(mx, v);
+      if (col0 + j == tcol) p.xent_tlogit[row] = v;
+    }
+    float sum = 0.0f;
+    for (int j = 0; j < 64; ++j) {
+      float v = p.alpha * crow[b * 64 + j];
+      if (bias) v += to_f32(bias[col0 + j]);
+      v = to_f32(from_f32<T>(v));
+      sum += expf(v - mx);
+    }
+    p.xent_part[(long)row * p.xent_blocks + ((long)grp * p.n + col0) / 64] = make_float2(mx, sum);
   }
 }
 
@@ -1028,6 +1096,8 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   __syncthreads();
   if (p.sgd_master != nullptr && p.vec_c)
     finish_tile_sgd<T, BM, BN, 512>(p, ct, m0, n0, tid, grp, zo, zi);
+  else if (p.xent_mode == 1)
+    finish_tile_xent_stats<T, BM, BN, 512>(p, ct, m0, n0, tid, grp);
   else
     finish_tile<T, BM, BN, 512>(p, ct, m0, n0, tid, grp, zo, zi);
   if (p.trace != nullptr && tid == 0) atomicMax(p.trace + 1, (unsigned long long)wall_clock64());
@@ -1227,6 +1297,25 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   a.a_rowsum = (char*)d->a_rowsum;
   a.rowsum_sg = d->rowsum_sg;
   a.trace = nullptr;
+  a.xent_mode = d->xent_mode;
+  a.xent_blocks = (int)(d->groups * d->n / 64);
+  a.xent_target = (const long*)d->xent_target;
+  a.xent_ignore = (long)d->xent_ignore;
+  a.xent_part = (float2*)d->xent_part;
+  a.xent_tlogit = d->xent_tlogit;
+  a.xent_stats = (const float2*)d->xent_stats;
+  a.xent_dloss = d->xent_dloss;
+  a.xent_scale = d->xent_scale;
+  if (d->xent_mode) {
+    RTP_REQUIRE(d->xent_mode == 1 || d->xent_mode == 2, "rtp_gemm: xent_mode is 0, 1 or 2");
+    RTP_REQUIRE(takes_dma_kernel<T>(d) && !is_tiny(d) && a.vec_c && d->n % 64 == 0 && d->batch == 1 && d->ksegs >= 1 &&
+                    d->c_sg == d->n && !(d->flags & (RTP_GEMM_OUT_F32 | RTP_GEMM_RELU)) && !d->c_in && !d->gate,
+                "rtp_gemm: the cross-entropy epilogues need vector-aligned operands, groups of a multiple of 64 columns "
+                "laid side by side (c_sg == n), an output in the compute dtype and no c_in / ReLU / mask");
+    RTP_REQUIRE(d->xent_target && (d->xent_mode == 1 ? (d->xent_part && d->xent_tlogit) : (d->xent_stats && d->xent_dloss)),
+                "rtp_gemm: missing cross-entropy operands for mode %d", d->xent_mode);
+    RTP_REQUIRE((uintptr_t)d->xent_part % 8 == 0 && (uintptr_t)d->xent_stats % 8 == 0, "rtp_gemm: 8-byte aligned statistics");
+  }
   a.sgd_master = (float*)d->sgd_master;
   a.sgd_w = (char*)d->sgd_weights;
   a.sgd_lr = d->sgd_lr;

@@ -130,3 +130,73 @@ extern "C" int rtp_rotated_linear_bwd(void* stream, int dtype, const rtp_rotated
   }
   return RTP_OK;
 }
+
+// ---- the logits layer together with its cross-entropy (rtp/models/transformer_lm_rtp.py:223 feeding the harness's
+// nn.CrossEntropyLoss(), benchmarks/rtp_benchmark.py:182) -------------------------------------------------------
+// Forward: the logits product leaves, per row, the softmax statistics of every 64-column block and the target's
+// logit -- the [rows, classes] logits are never written -- and a small kernel turns them into the row's loss and
+// {max, sum exp}.  Backward: the same product once more, its epilogue now writing the logits' gradient
+// (softmax - onehot) * dloss * scale, which the layer's ordinary backward (rtp_rotated_linear_bwd) consumes.
+static void logits_desc(rtp_gemm_desc* d, const rtp_rotated_linear* L, int64_t es, const void* x, int64_t ldx,
+                        int64_t rows, void* out, int64_t ld_out) {
+  clear(d);
+  d->a = x;
+  d->b = (const char*)L->home + L->w_off * es;
+  d->c_out = out;
+  d->bias = L->bias_off >= 0 ? (const char*)L->home + L->bias_off * es : nullptr;
+  d->m = rows, d->n = L->n_s, d->k = L->k;
+  d->lda = ldx, d->ldb = L->k, d->ldc = ld_out;
+  d->groups = L->shards;
+  d->b_sg = d->bias_sg = L->numel;
+  d->c_sg = L->n_s;
+  d->a_kcontig = d->b_kcontig = 1;
+}
+
+extern "C" size_t rtp_rotated_linear_xent_workspace_bytes(const rtp_rotated_linear* L, int64_t rows) {
+  if (!L || rows <= 0 || L->n_s <= 0 || L->shards <= 0) return 256;
+  return (size_t)rows * (size_t)(L->shards * L->n_s / 64) * 8 + (size_t)rows * 4 + 256;
+}
+
+extern "C" int rtp_rotated_linear_xent_fwd(void* stream, int dtype, const rtp_rotated_linear* L, const void* x,
+                                           int64_t ldx, int64_t rows, const int64_t* target, int64_t ignore_index,
+                                           float* loss, float* stats, void* workspace, size_t workspace_bytes) {
+  if (int rc = check_layer("rtp_rotated_linear_xent_fwd", dtype, L)) return rc;
+  RTP_REQUIRE(x && target && loss && stats && workspace && ldx >= L->k, "rtp_rotated_linear_xent_fwd: bad arguments");
+  RTP_REQUIRE(L->n_s % 64 == 0, "rtp_rotated_linear_xent_fwd: a shard's %lld output columns are not a multiple of 64",
+              (long long)L->n_s);
+  RTP_REQUIRE((uintptr_t)workspace % 8 == 0 && workspace_bytes >= rtp_rotated_linear_xent_workspace_bytes(L, rows),
+              "rtp_rotated_linear_xent_fwd: workspace of %zu bytes, need %zu (8-byte aligned)", workspace_bytes,
+              rtp_rotated_linear_xent_workspace_bytes(L, rows));
+  if (rows == 0) return RTP_OK;
+  const int64_t es = dtype == RTP_F32 ? 4 : 2;
+  const int64_t blocks = L->shards * L->n_s / 64;
+  float* part = (float*)workspace;
+  float* tlogit = part + rows * blocks * 2;
+  rtp_gemm_desc d;
+  // c_out is not written in this mode; the pointer only has to be a valid, aligned address for the descriptor checks
+  logits_desc(&d, L, es, x, ldx, rows, workspace, L->n_s * L->shards);
+  d.xent_mode = 1;
+  d.xent_target = target, d.xent_ignore = ignore_index;
+  d.xent_part = part, d.xent_tlogit = tlogit;
+  if (int rc = rtp_gemm(stream, dtype, &d)) return rc;
+  return rtp_softmax_xent_combine(stream, part, blocks, tlogit, target, ignore_index, rows, loss, stats);
+}
+
+extern "C" int rtp_rotated_linear_xent_bwd(void* stream, int dtype, const rtp_rotated_linear* L, const void* x,
+                                           int64_t ldx, int64_t rows, const int64_t* target, int64_t ignore_index,
+                                           const float* stats, const float* dloss, const float* scale, void* dlogits,
+                                           int64_t ld_dlogits) {
+  if (int rc = check_layer("rtp_rotated_linear_xent_bwd", dtype, L)) return rc;
+  RTP_REQUIRE(x && target && stats && dloss && dlogits && ldx >= L->k && ld_dlogits >= L->n_s * L->shards,
+              "rtp_rotated_linear_xent_bwd: bad arguments");
+  RTP_REQUIRE(L->n_s % 64 == 0, "rtp_rotated_linear_xent_bwd: a shard's %lld output columns are not a multiple of 64",
+              (long long)L->n_s);
+  if (rows == 0) return RTP_OK;
+  const int64_t es = dtype == RTP_F32 ? 4 : 2;
+  rtp_gemm_desc d;
+  logits_desc(&d, L, es, x, ldx, rows, dlogits, ld_dlogits);
+  d.xent_mode = 2;
+  d.xent_target = target, d.xent_ignore = ignore_index;
+  d.xent_stats = stats, d.xent_dloss = dloss, d.xent_scale = scale;
+  return rtp_gemm(stream, dtype, &d);
+}

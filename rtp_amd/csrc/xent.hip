@@ -123,6 +123,28 @@ __global__ __launch_bounds__(kXentThreads) void xent_bwd_any_kernel(const T* x, 
   }
 }
 
+// Per-row statistics from the {max, sum exp} of the row's 64-column blocks (left by the logits product's
+// epilogue): one wavefront per row, blocks combined in a fixed order; loss as in xent_fwd_kernel.
+__global__ __launch_bounds__(256) void xent_combine_kernel(const float2* part, long blocks, const float* tlogit,
+                                                           const long* target, long ignore, long rows, long classes,
+                                                           float* loss, float2* stats) {
+  const int lane = threadIdx.x & 63;
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const float2* pr = part + row * blocks;
+  float mx = -INFINITY;
+  for (long b = lane; b < blocks; b += kWave) mx = fmaxf(mx, pr[b].x);
+  mx = wave_max(mx);
+  float sum = 0.0f;
+  for (long b = lane; b < blocks; b += kWave) sum += pr[b].y * expf(pr[b].x - mx);
+  sum = wave_sum(sum);
+  if (lane == 0) {
+    const long t = target[row];
+    stats[row] = make_float2(mx, sum);
+    loss[row] = row_loss(t, ignore, (int)classes, mx, sum, (t >= 0 && t < classes) ? tlogit[row] : 0.0f);
+  }
+}
+
 // out[0] = sum of loss[0..rows) (mean != 0: divided by the number of rows whose target is not `ignore`),
 // scale[0] = 1 / that number (1 for a plain sum).  One workgroup, fixed summation order.
 __global__ __launch_bounds__(kXentThreads) void xent_reduce_kernel(const float* loss, const long* target, long ignore,
@@ -245,6 +267,23 @@ extern "C" int rtp_softmax_xent_fwd(void* stream, int dtype, const void* logits,
   else
     launch_xent_fwd<bf16_t>(nv, grid, st, (const bf16_t*)logits, (long)ld, (int)cols, (const long*)target,
                             (long)ignore_index, loss, (float2*)stats);
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
+}
+
+extern "C" int rtp_softmax_xent_combine(void* stream, const float* part, int64_t blocks, const float* tlogit,
+                                        const int64_t* target, int64_t ignore_index, int64_t rows, float* loss,
+                                        float* stats) {
+  RTP_REQUIRE(part && tlogit && target && loss && stats, "rtp_softmax_xent_combine: null pointer");
+  RTP_REQUIRE(rows >= 0 && rows < (1ll << 31) && blocks >= 1 && blocks < (1ll << 25),
+              "rtp_softmax_xent_combine: rows %lld / blocks %lld out of range", (long long)rows, (long long)blocks);
+  RTP_REQUIRE((uintptr_t)part % 8 == 0 && (uintptr_t)stats % 8 == 0, "rtp_softmax_xent_combine: 8-byte aligned pairs");
+  if (rows == 0) return RTP_OK;
+  hipStream_t st = (hipStream_t)stream;
+  ProfileScope prof(st, "softmax_xent_combine", 0.0, 8.0 * (double)rows * blocks);
+  hipLaunchKernelGGL(xent_combine_kernel, dim3((unsigned)ceil_div(rows, 4)), dim3(256), 0, st, (const float2*)part,
+                     (long)blocks, tlogit, (const long*)target, (long)ignore_index, (long)rows, (long)(blocks * 64), loss,
+                     (float2*)stats);
   RTP_LAUNCH_CHECK();
   return RTP_OK;
 }

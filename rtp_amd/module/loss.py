@@ -45,6 +45,77 @@ class _ReducedLossFn(torch.autograd.Function):
         return ops.softmax_xent_bwd(logits, target, stats, dloss.float().reshape(1), scale=scale), None, None, None
 
 
+class _LinearCrossEntropyFn(torch.autograd.Function):
+    """cross_entropy(layer(x), target) for a rotated column-parallel layer, the logits never stored: the forward
+    product leaves softmax statistics, the backward runs the product once more and writes the logits' gradient,
+    which then takes the layer's ordinary backward."""
+
+    @staticmethod
+    def forward(ctx, x, anchor, layer, target, ignore_index, mean):
+        from ..ring import Rotation, ring_order
+        from .utils import as_rows
+        store = layer._store
+        n_s, k = layer.output_size_per_partition, layer.in_features
+        x2 = as_rows(x, k)
+        rot = Rotation(store.home, ring_order(layer.rank, layer.world_size), group=store.stage_group)
+        runs = rot.acquire(0)
+        if rot.steps != 1 or len(runs) != 1:
+            raise RuntimeError("linear_cross_entropy needs all shards of the layer in one run (rotation window = all)")
+        b_off = n_s * k if layer.has_bias else None
+        rows, stats = ops.rotated_linear_xent_fwd(x2, runs[0][0], 0, b_off, n_s, k, target, ignore_index)
+        rot.release(0)
+        loss, scale = ops.softmax_xent_reduce(rows, target, ignore_index, mean)
+        ctx.layer, ctx.ignore_index, ctx.x_shape = layer, ignore_index, x.shape
+        ctx.save_for_backward(x2, target, stats, scale)
+        return loss
+
+    @staticmethod
+    def backward(ctx, dloss):
+        from ..ring import Rotation, ring_order, run_wgrad
+        from . import shard_ops as S
+        layer = ctx.layer
+        x2, target, stats, scale = ctx.saved_tensors
+        store = layer._store
+        n_s, k, ws = layer.output_size_per_partition, layer.in_features, layer.world_size
+        b_off = n_s * k if layer.has_bias else None
+        order = ring_order(layer.rank, ws, reverse=True)
+        rot = Rotation(store.home, order, group=store.stage_group)
+        flat = rot.acquire(0)[0][0]
+        dlogits = ops.rotated_linear_xent_bwd(x2, flat, 0, b_off, n_s, k, target, ctx.ignore_index, stats,
+                                              dloss.float().reshape(1), scale)
+        dx = None
+        if ctx.needs_input_grad[0]:
+            dx = torch.empty_like(x2)
+            S.col_dgrad(dlogits, flat, 0, n_s, k, dx, 0)
+        rot.release(0)
+        runs = store.grad_runs(order)
+
+        def param_grads():
+            for first, cnt, accumulate in runs:
+                S.col_wgrad(dlogits, x2, store.grads, first, 0, n_s, k, first * n_s, cnt, accumulate, b_off=b_off,
+                            store=store)
+            store.grads_ready()
+
+        run_wgrad(dlogits.device, param_grads, (dlogits, x2))
+        return (dx.view(ctx.x_shape) if dx is not None else None), None, None, None, None, None
+
+
+def linear_cross_entropy(x: torch.Tensor, layer, target: torch.Tensor, ignore_index: int = -100,
+                         reduction: str = "mean") -> torch.Tensor:
+    """cross_entropy(layer(x).view(-1, classes), target) for a ColumnParallelLinear `layer` (the LM's logits layer,
+    rtp/models/transformer_lm_rtp.py:223, and the harness loss, benchmarks/rtp_benchmark.py:182) without the
+    [rows, classes] logits ever reaching memory: their softmax statistics come out of the forward product's epilogue
+    and their gradient out of a second run of that product in the backward pass.  Same values as the two separate
+    calls (the logits are rounded to the layer's dtype before they enter the loss, as the stored ones would be).
+    Needs a shard width that is a multiple of 64 columns and the rotation window that covers the whole layer."""
+    if reduction not in ("mean", "sum"):
+        raise ValueError("linear_cross_entropy: reduction must be 'mean' or 'sum'")
+    if target.dim() != 1 or target.numel() * x.shape[-1] != x.numel():
+        raise ValueError("linear_cross_entropy: target must hold one class index per row of x")
+    target = (target if target.dtype == torch.int64 else target.long()).contiguous()
+    return _LinearCrossEntropyFn.apply(x, layer._anchor, layer, target, int(ignore_index), reduction == "mean")
+
+
 def cross_entropy(logits: torch.Tensor, target: torch.Tensor, ignore_index: int = -100,
                   reduction: str = "mean") -> torch.Tensor:
     """F.cross_entropy(logits.float(), target) for logits [rows, classes] and class-index targets [rows].

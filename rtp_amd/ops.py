@@ -169,6 +169,46 @@ def rotated_linear_bwd(dy2: torch.Tensor, x2: Optional[torch.Tensor], home: torc
     return done.value
 
 
+def rotated_linear_xent_fwd(x2: torch.Tensor, home: torch.Tensor, w_off: int, bias_off: Optional[int], n_s: int, k: int,
+                            target: torch.Tensor, ignore_index: int = -100) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-row cross-entropy loss (fp32 [rows]) and {max, sum exp} (fp32 [rows, 2]) of the logits
+    x2 @ W_g^T + b_g over all shards g of `home`, without the logits reaching memory."""
+    layer = _rotated_layer(home, w_off, bias_off, n_s, k)
+    rows, kk, ldx = _mat(x2, "x")
+    if kk != k or x2.dtype != home.dtype:
+        raise ValueError("rotated_linear_xent_fwd: x must be [rows, k] in the shards' dtype")
+    if target.dtype != torch.int64 or target.numel() != rows or not target.is_contiguous() or target.device != x2.device:
+        raise ValueError("rotated_linear_xent_fwd: target must be contiguous int64 [rows] on the device")
+    lib = _lib.load()
+    nbytes = lib.rtp_rotated_linear_xent_workspace_bytes(C.byref(layer), rows)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x2.device)
+    loss = torch.empty(rows, dtype=torch.float32, device=x2.device)
+    stats = torch.empty(rows, 2, dtype=torch.float32, device=x2.device)
+    _lib.require_device()
+    check(lib.rtp_rotated_linear_xent_fwd(_stream(), dtype_code(home.dtype), C.byref(layer), x2.data_ptr(), ldx, rows,
+                                          target.data_ptr(), int(ignore_index), loss.data_ptr(), stats.data_ptr(),
+                                          ws.data_ptr(), nbytes))
+    return loss, stats
+
+
+def rotated_linear_xent_bwd(x2: torch.Tensor, home: torch.Tensor, w_off: int, bias_off: Optional[int], n_s: int, k: int,
+                            target: torch.Tensor, ignore_index: int, stats: torch.Tensor, dloss: torch.Tensor,
+                            scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The logits' gradient [rows, shards * n_s] = (softmax - onehot(target)) * dloss * scale in the shards' dtype, from
+    the logits product run once more with the rows' statistics."""
+    layer = _rotated_layer(home, w_off, bias_off, n_s, k)
+    rows, kk, ldx = _mat(x2, "x")
+    if kk != k or x2.dtype != home.dtype or stats.shape != (rows, 2) or stats.dtype != torch.float32 or \
+            not stats.is_contiguous() or dloss.dtype != torch.float32 or dloss.numel() != 1:
+        raise ValueError("rotated_linear_xent_bwd: x [rows, k], stats fp32 [rows, 2], dloss one fp32 element")
+    out = torch.empty(rows, n_s * home.shape[0], dtype=home.dtype, device=x2.device)
+    _lib.require_device()
+    check(_lib.load().rtp_rotated_linear_xent_bwd(_stream(), dtype_code(home.dtype), C.byref(layer), x2.data_ptr(), ldx,
+                                                  rows, target.data_ptr(), int(ignore_index), stats.data_ptr(),
+                                                  dloss.data_ptr(), _ptr(scale), out.data_ptr(), out.stride(0)))
+    return out
+
+
 def _epilogue_args(dtype, out, c_in, bias, gate):
     kw = {}
     if out.dtype == torch.float32 and dtype != torch.float32:

@@ -46,9 +46,9 @@ def test_loader_binds_and_reports_version():
 
 def test_gemm_desc_matches_c_layout():
     from rtp_amd import _lib
-    # 6 pointers + 33 int64 + float + 3 int32, the row-sum pointer and its group stride, then the fused update:
-    # two pointers and two floats
-    assert ctypes.sizeof(_lib.GemmDesc) == 6 * 8 + 33 * 8 + 4 + 3 * 4 + 8 + 8 + 8 + 8 + 4 + 4
+    # 6 pointers + 33 int64 + float + 3 int32, the row-sum pointer and its group stride, the fused update (two
+    # pointers and two floats), then the cross-entropy epilogues (two int32, a pointer, an int64, five pointers)
+    assert ctypes.sizeof(_lib.GemmDesc) == 6 * 8 + 33 * 8 + 4 + 3 * 4 + 8 + 8 + (8 + 8 + 4 + 4) + (2 * 4 + 8 + 8 + 5 * 8)
     if os.path.exists(_lib.LIB_PATH):
         assert _lib.load().rtp_gemm_desc_size() == ctypes.sizeof(_lib.GemmDesc)
 

@@ -112,3 +112,53 @@ def test_cross_entropy_default_ignore_index_and_invalid_targets():
     assert float(cross_entropy(store.to(DEV), all_ignored.to(DEV), reduction="sum")) == 0.0
     with pytest.raises(RtpError):
         cross_entropy(store, target)                                             # CPU tensors: no fallback
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,k,vocab,ws", [(1024, 256, 10240, 8), (96, 64, 512, 4), (70, 64, 128, 2), (130, 128, 1344, 3)])
+def test_linear_cross_entropy_matches_separate_layer_and_loss(dtype, rows, k, vocab, ws):
+    """The logits layer fused with its loss (logits never stored) against the same layer followed by the
+    cross-entropy kernels, and against torch on the CPU: loss, input gradient, weight and bias gradients, with
+    ignored rows."""
+    from rtp_amd import emulate_shards
+    from rtp_amd.module.linear import ColumnParallelLinear
+    from rtp_amd.module.loss import cross_entropy, linear_cross_entropy
+    gen = torch.Generator().manual_seed(rows + vocab)
+    master = torch.nn.Linear(k, vocab)
+    with torch.no_grad():
+        master.weight.copy_((torch.rand(vocab, k, generator=gen) * 0.2 - 0.1).to(dtype).float())
+        master.bias.copy_((torch.rand(vocab, generator=gen) * 0.2 - 0.1).to(dtype).float())
+    with emulate_shards(ws):
+        fused = ColumnParallelLinear(k, vocab, linear_layer=master, device=DEV, dtype=dtype)
+        plain = ColumnParallelLinear(k, vocab, linear_layer=master, device=DEV, dtype=dtype)
+    x = (torch.randn(rows, k, generator=gen) * 2.0).to(dtype)
+    target = torch.randint(0, vocab, (rows,), generator=gen)
+    target[::7] = -100
+    xf, xp = x.to(DEV).requires_grad_(), x.to(DEV).requires_grad_()
+    lf = linear_cross_entropy(xf, fused, target.to(DEV))
+    (lf * 1.5).backward()
+    lp = cross_entropy(plain(xp), target.to(DEV))
+    (lp * 1.5).backward()
+    xr = x.float().clone().requires_grad_()
+    lr = F.cross_entropy(master(xr), target)
+    (lr * 1.5).backward()
+    assert abs(float(lf) - float(lr)) <= (1e-5 if dtype == torch.float32 else 2e-2) * abs(float(lr))
+    assert abs(float(lf) - float(lp)) <= 1e-6 * abs(float(lp))     # same rounded logits on both device paths
+    assert_close(xf.grad, xr.grad, dtype, "dx vs torch")
+    assert_close(xf.grad, xp.grad.float().cpu(), dtype, "dx vs separate kernels")
+    gw = torch.cat([s.weight.grad for s in fused.linears], 0)
+    gb = torch.cat([s.bias.grad for s in fused.linears], 0)
+    assert_close(gw, master.weight.grad, dtype, "dW")
+    assert_close(gb, master.bias.grad, dtype, "db")
+    assert torch.count_nonzero(xf.grad[::7]).item() == 0
+
+
+def test_linear_cross_entropy_refuses_shard_widths_it_cannot_block():
+    from rtp_amd import emulate_shards
+    from rtp_amd._lib import RtpError
+    from rtp_amd.module.linear import ColumnParallelLinear
+    from rtp_amd.module.loss import linear_cross_entropy
+    with emulate_shards(2):
+        layer = ColumnParallelLinear(64, 96, device=DEV)          # 48 columns per shard
+    with pytest.raises(RtpError, match="multiple of 64"):
+        linear_cross_entropy(torch.randn(8, 64, device=DEV), layer, torch.zeros(8, dtype=torch.long, device=DEV))
