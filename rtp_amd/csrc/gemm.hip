@@ -1103,6 +1103,245 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   if (p.trace != nullptr && tid == 0) atomicMax(p.trace + 1, (unsigned long long)wall_clock64());
 }
 
+// ---------------------------------------------------------------------------------------------
+// 256 x 256 tiles for large products.  What bounds the kernel above on a large product is the stream of operand
+// bytes from the L2 into the LDS (a product of 4096^3 takes as long with its MFMAs removed), and that stream is
+// (1/BM + 1/BN) bytes per flop: a 256 x 256 tile moves two thirds of what 256 x 128 moves.  Its 256 KiB of fp32
+// accumulators need all eight waves of the workgroup as MFMA waves (2 x 4 wave tiles of 128 x 64, 128 accumulator
+// registers each), so here the waves issue the direct-to-LDS loads themselves, each an eighth of a slab, right
+// after the barrier that frees a stage; the slab is 64 bytes of k per row (32 KiB per stage, 5 stages).  Same
+// barrier protocol as above with both roles in one wave: before barrier k+1 a wave waits for its own loads of slab
+// k+1, after it the wave refills the stage of slab k-1.  The epilogue goes through LDS in four passes of 64 rows.
+template <typename T, bool AKC, bool BKC, int NSTAGE, int SB, int PD>
+__global__ __launch_bounds__(512) void gemm_dma8_kernel(GemmArgs p) {
+  constexpr int BM = 256, BN = 256, NL = 8;
+  using DA = DmaOperand<T, BM, AKC, NL, SB>;
+  using DB = DmaOperand<T, BN, BKC, NL, SB>;
+  constexpr int BK = SB / sizeof(T);
+  constexpr int KS = SB / 32;
+  constexpr int WM = 128, WN = 64, MT = 4, NT = 2;
+  constexpr int STAGE = DA::BYTES + DB::BYTES;
+  constexpr int NI = DA::NI + DB::NI;
+  static_assert((NSTAGE - 2) * NI < 64, "vmcnt is a 6-bit counter");
+  static_assert(NSTAGE >= 3 && NSTAGE * STAGE <= 160 * 1024, "3 or more stages within 160 KiB of LDS");
+  static_assert(64 * (BN + 4) * 4 <= NSTAGE * STAGE, "an epilogue pass stages 64 rows of the fp32 tile");
+  __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE];
+
+  touch_kernel_arguments<sizeof(GemmArgs)>();
+  const int tid = threadIdx.x;
+  if (p.trace != nullptr && tid == 0) atomicMin(p.trace, (unsigned long long)wall_clock64());
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 2, wn = wave & 3;
+  const int li = lane & 31, g = lane >> 5;
+
+  // tile mapping: as in gemm_dma_kernel
+  const unsigned id = blockIdx.x + blockIdx.y * gridDim.x;
+  const unsigned xcd = id & 7, slot = id >> 3;
+  const unsigned zl = fast_div(slot, p.d_brick);
+  const unsigned t_ = slot - zl * p.d_brick.d;
+  const unsigned q_ = fast_div(t_, p.d_panel), r_ = t_ - q_ * p.d_panel.d;
+  const unsigned cn = fast_div(r_, p.d_prow), cm = r_ - cn * p.d_prow.d;
+  const unsigned qn = fast_div(q_, p.d_pm), qm = q_ - qn * p.d_pm.d;
+  const int tile_n_x = (int)((xcd & ((1u << p.xn_shift) - 1)) * p.nbk + qn * p.pcol + cn);
+  const int tile_m_x = (int)(((xcd >> p.xn_shift) & ((1u << p.xm_shift) - 1)) * p.mbk + qm * p.prow + cm);
+  const int z_x = (int)((xcd >> (p.xn_shift + p.xm_shift)) * p.zbk + zl);
+  const int tile_m_p = (int)fast_div(blockIdx.x, p.d_tiles_n);
+  const int tile_n_p = (int)(blockIdx.x - tile_m_p * p.d_tiles_n.d);
+  const bool bricks = p.xg != 0;
+  const int tile_m = bricks ? tile_m_x : tile_m_p, tile_n = bricks ? tile_n_x : tile_n_p;
+  const int z = bricks ? z_x : (int)blockIdx.y;
+  const int m0 = tile_m * BM;
+  const int n0 = tile_n * BN;
+  const int grp = (int)fast_div(z, p.d_batch), zb = z - grp * (int)p.d_batch.d;
+  const long zo = fast_div(zb, p.d_zdiv), zi = zb - (int)zo * (int)p.d_zdiv.d;
+  const int nk_seg = (p.k + BK - 1) / BK;
+  const int nk = nk_seg * p.ksegs;
+
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  float rsum[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) rsum[i] = 0.0f;
+
+  // ---- this wave's share of the loads ----
+  const T* A = reinterpret_cast<const T*>(p.a) + grp * p.a_sg + zo * p.a_so + zi * p.a_si;
+  const T* B = reinterpret_cast<const T*>(p.b) + grp * p.b_sg + zo * p.b_so + zi * p.b_si;
+  DA da;
+  DB db;
+  da.init(p.lda, m0, p.m, wave, lane);
+  db.init(p.ldb, n0, p.n, wave, lane);
+  const char* ca = DA::slab_base(A, p.lda, m0);
+  const char* cb = DB::slab_base(B, p.ldb, n0);
+  constexpr long SZ = (long)sizeof(T);
+  const long step_a = (AKC ? (long)BK : (long)BK * p.lda) * SZ, step_b = (BKC ? (long)BK : (long)BK * p.ldb) * SZ;
+  const long last_a = step_a + p.a_sk * SZ - nk_seg * step_a, last_b = step_b + p.b_sk * SZ - nk_seg * step_b;
+  const int k0_last = (nk_seg - 1) * BK;
+  const bool tail = p.k % BK != 0;
+  const unsigned lds0 = (unsigned)(uintptr_t)(lptr_t)lds;
+  unsigned fill = lds0;
+  int left = nk_seg;
+  auto issue = [&]() {
+    if (left != 1 || !tail) {
+      da.template issue<false>(fill, wave, ca, 0, 0);
+      db.template issue<false>(fill + DA::BYTES, wave, cb, 0, 0);
+    } else {
+      da.template issue<true>(fill, wave, ca, k0_last, p.k);
+      db.template issue<true>(fill + DA::BYTES, wave, cb, k0_last, p.k);
+    }
+    if (left != 1) {
+      ca += step_a;
+      cb += step_b;
+      --left;
+    } else {
+      ca += last_a;
+      cb += last_b;
+      left = nk_seg;
+    }
+    fill += STAGE;
+    if (fill == lds0 + NSTAGE * STAGE) fill = lds0;
+  };
+
+  constexpr int NSET = PD + 1;
+  static_assert(PD >= 1 && PD <= KS, "prefetch distance of 1..KS k-steps");
+  static_assert((NSTAGE * KS) % NSET == 0, "register set of a k-step must not depend on the round");
+  Frag<T> fa[NSET][MT], fb[NSET][NT];
+  const bool rowsum = p.a_rowsum != nullptr && tile_n == 0 && wn == 0;
+  auto read_step = [&](auto S, auto Q, auto SET) {
+    const char* sa = lds + (decltype(S)::value % NSTAGE) * STAGE;
+    const char* sb = sa + DA::BYTES;
+    constexpr int q = decltype(Q)::value, set = decltype(SET)::value;
+#pragma unroll
+    for (int i = 0; i < MT; ++i) fa[set][i] = read_frag_dma<T, BM, AKC, SB>(sa, wm * WM + i * 32, lane, q);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) fb[set][j] = read_frag_dma<T, BN, BKC, SB>(sb, wn * WN + j * 32, lane, q);
+  };
+  auto mma_step = [&](auto SET) {
+    constexpr int set = decltype(SET)::value;
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j) mma(fa[set][i], fb[set][j], acc[i][j]);
+    if (rowsum) {
+#pragma unroll
+      for (int i = 0; i < MT; ++i) rsum[i] = frag_sum(fa[set][i], rsum[i]);
+    }
+  };
+  auto step = [&](auto S, auto Q, int k, auto STEADY) {
+    constexpr bool steady = decltype(STEADY)::value;
+    constexpr int s = decltype(S)::value, q = decltype(Q)::value;
+    constexpr int t = s * KS + q;
+    constexpr int tq = (q + PD) % KS, ds = (q + PD) / KS;
+    if (steady || k + ds < nk) {
+      if (ds == 1 && tq == 0) {
+        // barrier k+1: my loads of slab k+1 have landed; behind it everybody's have, and everybody has consumed
+        // the last fragments of slab k-1, whose stage takes slab k+NSTAGE-1
+        if (k + NSTAGE - 1 < nk) {
+          RTP_WAIT_VM((NSTAGE - 3) * NI);
+        } else {
+          RTP_WAIT_VM(0);
+        }
+        __builtin_amdgcn_s_barrier();
+        if (k + NSTAGE - 1 < nk) issue();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      read_step(std::integral_constant<int, (s + ds) % NSTAGE>{}, std::integral_constant<int, tq>{},
+                std::integral_constant<int, (t + PD) % NSET>{});
+    }
+    mma_step(std::integral_constant<int, t % NSET>{});
+    constexpr int RPF_A = AKC ? 1 : (sizeof(T) == 2 ? 2 : 4), RPF_B = BKC ? 1 : (sizeof(T) == 2 ? 2 : 4);
+    constexpr int NR = MT * RPF_A + NT * RPF_B, NM = MT * NT * (sizeof(T) == 2 ? 1 : 4);
+    constexpr int PER = (NR + NM - 1) / NM;
+    [&]<int... I>(std::integer_sequence<int, I...>) {
+      ((__builtin_amdgcn_sched_group_barrier(0x008, 1, 0),
+        (I * PER < NR ? __builtin_amdgcn_sched_group_barrier(0x100, (I + 1) * PER <= NR ? PER : NR - I * PER, 0)
+                      : (void)0)),
+       ...);
+    }(std::make_integer_sequence<int, NM>{});
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto phase = [&](auto S, int k, auto STEADY) {
+    if (!decltype(STEADY)::value && k >= nk) return;
+    [&]<int... Q>(std::integer_sequence<int, Q...>) {
+      (step(S, std::integral_constant<int, Q>{}, k, STEADY), ...);
+    }(std::make_integer_sequence<int, KS>{});
+  };
+  auto round = [&](int kt, auto STEADY) {
+    [&]<int... S>(std::integer_sequence<int, S...>) {
+      (phase(std::integral_constant<int, S>{}, kt + S, STEADY), ...);
+    }(std::make_integer_sequence<int, NSTAGE>{});
+  };
+
+  // prologue: NSTAGE-1 slabs on their way, slab 0 landed
+  const int ahead = nk < NSTAGE - 1 ? nk : NSTAGE - 1;
+  for (int s_ = 0; s_ < ahead; ++s_) issue();
+  if (nk >= NSTAGE - 1) {
+    RTP_WAIT_VM((NSTAGE - 2) * NI);
+  } else {
+    RTP_WAIT_VM(0);
+  }
+  __builtin_amdgcn_s_barrier();  // barrier 0
+  [&]<int... Q>(std::integer_sequence<int, Q...>) {
+    (read_step(std::integral_constant<int, 0>{}, std::integral_constant<int, Q>{}, std::integral_constant<int, Q>{}), ...);
+  }(std::make_integer_sequence<int, PD>{});
+  __builtin_amdgcn_sched_barrier(0);
+  int kt = 0;
+  for (; kt + NSTAGE < nk; kt += NSTAGE) round(kt, std::true_type{});
+  for (; kt < nk; kt += NSTAGE) round(kt, std::false_type{});
+
+  if (p.a_rowsum != nullptr && tile_n == 0 && wn == 0) {
+    T* dst = reinterpret_cast<T*>(p.a_rowsum) + grp * p.rowsum_sg;
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const float v = rsum[i] + __shfl_xor(rsum[i], 32, 64);
+      const int row = m0 + wm * WM + i * 32 + li;
+      if (g == 0 && row < p.m) dst[row] = from_f32<T>((p.flags & RTP_GEMM_ROWSUM_ACCUM) ? to_f32(dst[row]) + v : v);
+    }
+  }
+
+  // Epilogue in MT passes: pass i stages rows i*32 .. i*32+31 of both tile halves (64 rows of 256 columns, fp32)
+  // in the slab memory; every thread then finishes chunks of 8 columns as in the other kernel.
+  constexpr int CP = BN + 4;
+  float* ct = reinterpret_cast<float*>(lds);
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+    __syncthreads();  // the fragments (first pass) or the previous pass's rows have been read
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        ct[(wm * 32 + 8 * (r >> 2) + 4 * g + (r & 3)) * CP + wn * WN + j * 32 + li] = acc[i][j][r];
+    __syncthreads();
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int mrow = m0 + h * WM + i * 32;
+      if (mrow >= p.m) continue;
+      finish_tile<T, 32, BN, 512>(p, ct + h * 32 * CP, mrow, n0, tid, grp, zo, zi);
+    }
+  }
+  if (p.trace != nullptr && tid == 0) atomicMax(p.trace + 1, (unsigned long long)wall_clock64());
+}
+
+template <typename T, int NSTAGE, int SB, int PD>
+static int launch_dma8(hipStream_t s, const GemmArgs& a, bool akc, bool bkc, dim3 grid) {
+  const dim3 block(512);
+  if (akc && bkc)
+    hipLaunchKernelGGL((gemm_dma8_kernel<T, true, true, NSTAGE, SB, PD>), grid, block, 0, s, a);
+  else if (akc && !bkc)
+    hipLaunchKernelGGL((gemm_dma8_kernel<T, true, false, NSTAGE, SB, PD>), grid, block, 0, s, a);
+  else if (!akc && bkc)
+    hipLaunchKernelGGL((gemm_dma8_kernel<T, false, true, NSTAGE, SB, PD>), grid, block, 0, s, a);
+  else
+    hipLaunchKernelGGL((gemm_dma8_kernel<T, false, false, NSTAGE, SB, PD>), grid, block, 0, s, a);
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
+}
+
 template <typename T, int BM, int BN, int NSTAGE, int SB, int PD>
 static int launch_dma(hipStream_t s, const GemmArgs& a, bool akc, bool bkc, dim3 grid) {
   const dim3 block(512);
@@ -1211,9 +1450,9 @@ struct TileShape {
   int bm, bn;
   const char* tag;
 };
-static const TileShape kShapes[5] = {{256, 128, "256x128"}, {128, 128, "128x128"}, {128, 64, "128x64"}, {64, 64, "64x64"},
-                                     {128, 192, "128x192"}};
-constexpr int kNumShapes = 5;
+static const TileShape kShapes[6] = {{256, 128, "256x128"}, {128, 128, "128x128"}, {128, 64, "128x64"}, {64, 64, "64x64"},
+                                     {128, 192, "128x192"}, {256, 256, "256x256"}};
+constexpr int kNumShapes = 6;
 
 // One wavefront per 32 x 32 block is the better kernel for one attention head at sequence length <= 64.
 static bool is_tiny(const rtp_gemm_desc* d) { return d->m <= 64 && d->n <= 64 && d->k * d->ksegs <= 256; }
@@ -1361,11 +1600,17 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
     const char* e = getenv("RTP_GEMM_TILE");  // debugging aid: index into kShapes
     return e ? atoi(e) : -1;
   }();
-  static const double slab_ns[kNumShapes] = {966.0, 470.0, 283.0, 167.0, 720.0};
-  static const int slab_bytes[kNumShapes] = {128, 128, 128, 128, 128};
+  static const double slab_ns[kNumShapes] = {966.0, 470.0, 283.0, 167.0, 720.0, 840.0};
+  static const int slab_bytes[kNumShapes] = {128, 128, 128, 128, 128, 64};
   int shape = 3;  // 64 x 64 unless the model finds something cheaper
   double best = 0.0;
   for (int i = 0; fast && i < kNumShapes; ++i) {
+    // the 256 x 256 kernel is built for 16-bit operands and the plain epilogue, and pays only on very large
+    // products (measured: +9 % forward, +20 % on the transposed layouts at 8192^3, nothing at 4096^3, a loss
+    // where it leaves CUs without a tile)
+    if (i == 5 && (sizeof(T) != 2 || d->sgd_master || d->xent_mode == 1 ||
+                   ceil_div(d->m, 256) * ceil_div(d->n, 256) * nz < 1024 || d->k * d->ksegs < 2048) && i != forced)
+      continue;
     // never a tile that is mostly padding: a 32 x 32 problem (one attention head at seq 32) stays at 64 x 64
     if ((!akc && (kShapes[i].bm & (kShapes[i].bm - 1))) || (!bkc && (kShapes[i].bn & (kShapes[i].bn - 1)))) continue;
     if (kShapes[i].bm > 64 && kShapes[i].bm > ceil_div(d->m, 64) * 64) continue;
@@ -1460,6 +1705,9 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
       return launch_dma<T, 128, 64, 5, 128, 4>(s, a, akc, bkc, grid);
     case 4:
       return launch_dma<T, 128, 192, 3, 128, 2>(s, a, akc, bkc, grid);
+    case 5:
+      if constexpr (sizeof(T) == 2) return launch_dma8<T, 5, 64, 1>(s, a, akc, bkc, grid);
+      return fail(RTP_ERR_ARG, "gemm: no 256 x 256 kernel for this dtype");
     default:
       return launch_dma<T, 64, 64, 4, 128, 3>(s, a, akc, bkc, grid);
   }

@@ -287,3 +287,33 @@ def test_gemm_many_rounds_tile_order(m, n, k, groups, akc, bkc):
     torch.cuda.synchronize()
     assert not torch.isnan(out).any()
     assert rel_err(out, ref) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("akc,bkc", [(True, True), (True, False), (False, True)])
+def test_gemm_256x256_tile_path(akc, bkc):
+    """A product with more than 1024 tiles of 256 x 256 and a long K takes the eight-wave kernel (checked by its
+    name in the launch records); ragged on every edge, with bias, ReLU and an addend in the epilogue.  The yardstick
+    is torch's fp32 product of the same bf16 values on the device (float64 on the CPU would take minutes)."""
+    from rtp_amd import _lib
+    ops = _ops()
+    dtype = torch.bfloat16
+    gen = torch.Generator().manual_seed(77)
+    m, n, k = 8104, 8200, 2056  # leading dimensions stay multiples of 16 bytes in every layout
+    a = _rand((m, k) if akc else (k, m), dtype, gen).to(DEV)
+    b = _rand((n, k) if bkc else (k, n), dtype, gen).to(DEV)
+    bias, cin = _rand((n,), dtype, gen).to(DEV), _rand((m, n), dtype, gen).to(DEV)
+    A = a.float() if akc else a.float().t()
+    B = b.float() if bkc else b.float().t()
+    ref = torch.relu(A @ B.t() + bias.float() + cin.float())
+    out = torch.full((m, n), float("nan"), dtype=dtype, device=DEV)
+    _lib.profile_enable(1)
+    try:
+        ops.gemm_raw(dtype, a=a.data_ptr(), b=b.data_ptr(), c_out=out.data_ptr(), m=m, n=n, k=k, lda=a.stride(0),
+                     ldb=b.stride(0), ldc=n, a_kcontig=akc, b_kcontig=bkc, bias=bias.data_ptr(), c_in=cin.data_ptr(),
+                     ld_cin=n, relu=True)
+        torch.cuda.synchronize()
+        names = list(_lib.profile_collect())
+    finally:
+        _lib.profile_enable(0)
+    assert any("256x256" in nm for nm in names), names
+    assert rel_err(out, ref) <= TOL[dtype]
