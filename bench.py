@@ -394,6 +394,9 @@ def main():
                     help="direct (default): the products read every shard from its home row, the LDS stage ring of the "
                          "product kernel is the rotation's double buffer; staged: shards are first copied into two HBM "
                          "slots on a side stream (the transport of a multi-GPU ring)")
+    ap.add_argument("--no-warm-ahead", dest="warm_ahead", action="store_false",
+                    help="do not read the next layer's shards into the memory-side cache on a side stream while the "
+                         "current layer computes (direct rotation only)")
     ap.add_argument("--no-graph", dest="graph", action="store_false",
                     help="launch every kernel eagerly instead of replaying the step from a captured HIP graph")
     args = ap.parse_args()
@@ -415,6 +418,7 @@ def main():
     dev = torch.device("cuda", 0)
     ring.set_wgrad_overlap(args.wgrad_overlap)
     ring.set_rotation_mode(args.rotation)
+    ring.set_warm_ahead(args.warm_ahead and args.rotation == "direct")
     torch.cuda.set_device(dev)
     c = CFG
     lm = build(c, dev, torch.bfloat16)
@@ -545,7 +549,8 @@ def main():
                    "sgd_overlapped_with_backward": bool(args.sgd_overlap),
                    "sgd_fused_into_weight_gradient_products": bool(args.sgd_fused),
                    "logits_and_loss_fused": bool(args.fused_head_loss),
-                   "wgrad_on_second_stream": bool(args.wgrad_overlap)},
+                   "wgrad_on_second_stream": bool(args.wgrad_overlap),
+                   "next_layer_shards_read_ahead_into_cache": bool(ring.warm_ahead())},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK["bf16_mfma_tflops"], "unit": "TFLOP/s",
                      "frac": achieved / PEAK["bf16_mfma_tflops"],
                      "traffic": (MEASURED_TRAFFIC_KIB[dom_name] * 1024.0 if dom_name in MEASURED_TRAFFIC_KIB else None),

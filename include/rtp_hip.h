@@ -215,6 +215,17 @@ typedef struct {
 
 int rtp_gemm(void* stream, int dtype, const rtp_gemm_desc* d);
 
+/* "The next shard arrives while the current one computes" (reference: the irecv of the next shard under the current
+ * step's product, rtp/module/linear.py:211-220, rtp/module/collectives.py:240-317) for shards that are read from
+ * their home rows: hands `bytes` at `src` (16-byte aligned; the shards of the layer that runs next) to the next
+ * product that this host thread launches through rtp_gemm or rtp_rotated_linear_* on the wave-specialised kernel.
+ * That launch requests them at its start, so they sit in the GPU's memory-side cache when their own products run
+ * (weights are read once per pass and would otherwise come from HBM at their turn).  Up to 192 KiB per workgroup
+ * of the carrying launch.  A hint: no result depends on it; it ends with that next product launch whether or not
+ * the launch could carry it (other kernels than the wave-specialised one cannot), so `src` has to stay allocated
+ * only until then.  bytes == 0 withdraws a pending hint. */
+int rtp_gemm_warm_next(const void* src, size_t bytes);
+
 /* 1 if rtp_gemm would produce d->a_rowsum for this descriptor (the pointer itself may still be NULL), else 0. */
 int rtp_gemm_rowsum_fused(int dtype, const rtp_gemm_desc* d);
 
@@ -263,6 +274,13 @@ int rtp_ring_fence(void* ring, void* main_stream);
 int rtp_ring_prefetch(void* ring, void* main_stream, int slot, void* dst, const void* src, size_t bytes);
 int rtp_ring_acquire(void* ring, void* main_stream, int slot);
 int rtp_ring_release(void* ring, void* main_stream, int slot);
+
+/* Reads `bytes` at `src` (16-byte aligned) on `stream` and keeps nothing, so that the lines sit in the GPU's
+ * memory-side cache when the products that use them start: the one-GPU form of "the next shard arrives while the
+ * current one computes" (reference: the isend/irecv of the next shard that overlaps the current step's compute,
+ * rtp/module/collectives.py:240-317, rtp/module/linear.py:211-220) when the shards are read from their home rows
+ * and nothing is copied.  A hint: no result depends on it.  flags bit 0: non-temporal loads. */
+int rtp_cache_warm(void* stream, const void* src, size_t bytes, int flags);
 
 /* The copy kernel on its own (16-byte vectorised, grid-stride): dst/src 16-byte aligned or any
  * alignment (falls back to bytes for the ragged ends). */

@@ -96,6 +96,7 @@ PROTOTYPES = {
                                          _i64]),
     "rtp_softmax_xent_combine": (_i, [_vp, _vp, _i64, _vp, _vp, _i64, _i64, _vp, _vp]),
     "rtp_gemm": (_i, [_vp, _i, C.POINTER(GemmDesc)]),
+    "rtp_gemm_warm_next": (_i, [_vp, _sz]),
     "rtp_gemm_rowsum_fused": (_i, [_i, C.POINTER(GemmDesc)]),
     "rtp_gemm_sgd_fused": (_i, [_i, C.POINTER(GemmDesc)]),
     "rtp_gemm_desc_size": (_sz, []),
@@ -105,6 +106,7 @@ PROTOTYPES = {
     "rtp_ring_destroy": (_i, [_vp]),
     "rtp_ring_fence": (_i, [_vp, _vp]),
     "rtp_ring_prefetch": (_i, [_vp, _vp, _i, _vp, _vp, _sz]),
+    "rtp_cache_warm": (_i, [_vp, _vp, _sz, _i]),
     "rtp_ring_acquire": (_i, [_vp, _vp, _i]),
     "rtp_ring_release": (_i, [_vp, _vp, _i]),
     "rtp_shard_copy_async": (_i, [_vp, _vp, _vp, _sz]),

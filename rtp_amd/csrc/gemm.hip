@@ -88,6 +88,9 @@ struct GemmArgs {
   const float2* xent_stats;     // mode 2: [m] {max, sum exp} of the whole row
   const float* xent_dloss;      // mode 2: upstream gradient, one scalar
   const float* xent_scale;      // mode 2: second scalar factor (1 / rows counted), or null
+  // bytes that some later launch will read from HBM (the next layer's shards): requested here, see warm_ahead()
+  const char* warm;
+  long warm_bytes;
 };
 
 constexpr int kThreads = 256;
@@ -811,6 +814,27 @@ struct DmaOperand {
   }
 };
 
+// The next layer's shards arrive while this product computes.  Weights are read once per pass, so at their turn
+// they come from HBM, whose latency the NSTAGE - 1 slabs in flight do not cover: measured on the LM's shapes, a
+// product takes 15 - 30 % longer on weights from HBM than on weights that sit in the 256 MiB memory-side cache.
+// So a product can be handed the bytes that the *next* products will need: its MFMA waves, idle until the first
+// slab has landed, request them right at kernel start, 1 KiB per instruction, straight into 1 KiB of LDS that
+// nothing reads (no registers, and nobody ever waits for these loads: an MFMA wave next waits for vector memory
+// in the epilogue).  Pieces are dealt round-robin over (workgroup, wave), so the launch as a whole reads the region
+// front to back; a wave asks for at most kWarmMax pieces (the counter of outstanding loads has 6 bits), the rest
+// of a larger region stays unread.
+constexpr int kWarmMax = 48;
+__device__ __forceinline__ void warm_ahead(const GemmArgs& p, unsigned lds_dst, unsigned wg, unsigned nwg, int wave,
+                                           int lane) {
+  if (p.warm == nullptr) return;
+  const long pieces = p.warm_bytes >> 10;
+  long piece = (long)wg * 4 + wave;
+  for (int j = 0; j < kWarmMax && piece < pieces; ++j, piece += (long)nwg * 4) {
+    const char* src = p.warm + (piece << 10) + lane * 16;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_dst), "v"(src) : "memory");
+  }
+}
+
 typedef short short4_t __attribute__((ext_vector_type(4)));
 
 // rowbase: first tile row of the 32-row MFMA block; the lane's own row is rowbase + lane % 32.
@@ -861,10 +885,11 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   constexpr int NI = DA::NI + DB::NI;  // loads per loader wave and slab
   static_assert((NSTAGE - 2) * NI < 64, "vmcnt is a 6-bit counter");
   static_assert(NSTAGE >= 3, "at least 3 LDS stages");
-  static_assert(NSTAGE * STAGE <= 160 * 1024, "160 KiB of LDS per workgroup");
+  static_assert(NSTAGE * STAGE + 1024 <= 160 * 1024, "160 KiB of LDS per workgroup");
   static_assert(BM * (BN + 4) * 4 <= NSTAGE * STAGE, "the epilogue stages the fp32 tile in the slab memory");
-  // Stage addresses are compile-time offsets into one array, so LDS reads carry immediate offsets.
-  __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE];
+  // Stage addresses are compile-time offsets into one array, so LDS reads carry immediate offsets.  The last KiB
+  // is where the loads of warm_ahead() land.
+  __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE + 1024];
 
   touch_kernel_arguments<sizeof(GemmArgs)>();
   const int tid = threadIdx.x;
@@ -1056,6 +1081,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
         (phase(std::integral_constant<int, S>{}, kt + S, STEADY), ...);
       }(std::make_integer_sequence<int, NSTAGE>{});
     };
+    warm_ahead(p, (unsigned)(uintptr_t)(lptr_t)lds + NSTAGE * STAGE, id, gridDim.x * gridDim.y, wave, lane);
     __builtin_amdgcn_s_barrier();  // barrier 0
     [&]<int... Q>(std::integer_sequence<int, Q...>) {
       (read_step(std::integral_constant<int, 0>{}, std::integral_constant<int, Q>{}, std::integral_constant<int, Q>{}),
@@ -1486,8 +1512,15 @@ static bool rowsum_fused(const rtp_gemm_desc* d) {
   return !d->a_kcontig && d->batch == 1 && !is_tiny(d) && takes_dma_kernel<T>(d);
 }
 
+// rtp_gemm_warm_next: bytes the next product launched by this host thread requests at its start
+static thread_local const void* t_warm_src = nullptr;
+static thread_local size_t t_warm_bytes = 0;
+
 template <typename T>
 static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
+  // the hint of rtp_gemm_warm_next rides in this launch or ends with it
+  const void* warm_src = t_warm_src;
+  t_warm_src = nullptr;
   constexpr int VEC = 16 / sizeof(T);
   GemmArgs a;
   a.a = (const char*)d->a;
@@ -1695,7 +1728,13 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   const double bytes = ((double)d->m + (double)d->n) * kk * nz * sizeof(T) + mn * (out_sz + cin_sz);
   ProfileScope prof(s, name, 2.0 * mn * kk, bytes);
   a.trace = fast ? prof.trace_slot() : nullptr;
+  a.warm = nullptr;
+  a.warm_bytes = 0;
   if (!fast) return launch_layout<T, 64, 64, 1, false>(s, a, akc, bkc, grid);
+  if (shape != 5 && warm_src != nullptr) {
+    a.warm = (const char*)warm_src;
+    a.warm_bytes = (long)t_warm_bytes;
+  }
   switch (shape) {
     case 0:
       return launch_dma<T, 256, 128, 3, 128, 1>(s, a, akc, bkc, grid);
@@ -1854,6 +1893,13 @@ extern "C" int rtp_gemm_rowsum_fused(int dtype, const rtp_gemm_desc* d) {
   if (dtype == RTP_F32) return rowsum_fused<float>(d) ? 1 : 0;
   if (dtype == RTP_BF16) return rowsum_fused<bf16_t>(d) ? 1 : 0;
   return 0;
+}
+
+extern "C" int rtp_gemm_warm_next(const void* src, size_t bytes) {
+  RTP_REQUIRE(((uintptr_t)src & 15) == 0, "rtp_gemm_warm_next: source must be 16-byte aligned");
+  rtp::t_warm_src = bytes ? src : nullptr;
+  rtp::t_warm_bytes = bytes;
+  return RTP_OK;
 }
 
 extern "C" int rtp_gemm_sgd_fused(int dtype, const rtp_gemm_desc* d) {

@@ -114,6 +114,34 @@ __global__ __launch_bounds__(256) void copy_kernel(char* dst, const char* src, s
   }
 }
 
+// Reads `bytes` at `src` and keeps nothing: the lines end up in the 256 MiB memory-side cache (and pass through the
+// L2), from where the products that need them next take them at cached-operand speed.  Weights are read once per
+// pass, so at their turn they would otherwise come from HBM, whose latency the products' load pipeline does not
+// cover.  One workgroup per CU, like the background copy: the kernel runs under the products of the layer before.
+__global__ __launch_bounds__(256) void warm_kernel(const char* src, size_t bytes, unsigned* sink, int nt) {
+  const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t nthreads = (size_t)gridDim.x * blockDim.x;
+  const size_t nvec = bytes >> 4;
+  const uint4* s = reinterpret_cast<const uint4*>(src);
+  unsigned acc = 0;
+  size_t i = tid;
+  if (nt) {
+    for (; i + 3 * nthreads < nvec; i += 4 * nthreads) {
+      const uint4 v0 = nt_load(s + i), v1 = nt_load(s + i + nthreads), v2 = nt_load(s + i + 2 * nthreads),
+                  v3 = nt_load(s + i + 3 * nthreads);
+      acc |= v0.x & v1.x & v2.x & v3.x;
+    }
+  } else {
+    for (; i + 3 * nthreads < nvec; i += 4 * nthreads) {
+      const uint4 v0 = s[i], v1 = s[i + nthreads], v2 = s[i + 2 * nthreads], v3 = s[i + 3 * nthreads];
+      acc |= v0.x & v1.x & v2.x & v3.x;
+    }
+  }
+  for (; i < nvec; i += nthreads) acc |= s[i].x;
+  // never true for the value the host passes (sink == nullptr): the loads cannot be optimised away
+  if (sink != nullptr && acc == 0x9e3779b9u) *sink = acc;
+}
+
 __global__ __launch_bounds__(256) void zero_kernel(char* dst, size_t bytes, int aligned) {
   const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t nthreads = (size_t)gridDim.x * blockDim.x;
@@ -176,6 +204,17 @@ extern "C" int rtp_device_check(char* name_out, int name_len) {
     return fail(RTP_ERR_DEVICE, "device %d is %s; this library is built for gfx950 only", dev, prop.gcnArchName);
   // per-device set-up: the address of the built-in scratch of rtp_gate_wgrad_static on this device
   return gate_static_setup();
+}
+
+extern "C" int rtp_cache_warm(void* stream, const void* src, size_t bytes, int flags) {
+  if (bytes == 0) return RTP_OK;
+  RTP_REQUIRE(src && ((uintptr_t)src & 15) == 0, "rtp_cache_warm: source must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  ProfileScope prof(s, "cache_warm", 0.0, (double)bytes);
+  hipLaunchKernelGGL(warm_kernel, dim3(copy_grid(bytes, true)), dim3(256), 0, s, (const char*)src, bytes,
+                     (unsigned*)nullptr, flags & 1);
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
 }
 
 extern "C" int rtp_ring_create(void** ring_out) {

@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import ctypes as C
 import os
+import weakref
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
@@ -55,6 +56,60 @@ def set_rotation_mode(mode: str) -> None:
 
 def rotation_mode() -> str:
     return _mode
+
+
+# ---- the next layer's shards arrive while the current layer computes (direct mode) ------------------------
+# Read from their home rows, a layer's weights are touched once per pass, so at their turn they come from HBM, and the
+# products' load pipeline (a few K slabs in flight) does not cover that latency: measured on the LM's shapes, a
+# product takes 15 - 30 % longer on weights from HBM than on weights that sit in the 256 MiB memory-side cache.  With
+# the switch on, a rotation that starts hands the home rows of the layer that followed this one the last time round
+# to its own first product (rtp_gemm_warm_next), whose workgroups request them at their start: the one-GPU form of
+# the reference's irecv of the next shard during the current step (rtp/module/linear.py:211-220).  Which layer
+# follows is learned from the order of the rotations (keyed by the last two layers, so the forward and the backward
+# order are told apart); nothing depends on the guess being right.  No second stream is involved: a read pass on a
+# side stream (rtp_cache_warm) warms as well, but every fork of the compute stream costs ~5 us, more than it gains.
+_warm_ahead = os.environ.get("RTP_WARM_AHEAD", "1") == "1"
+_warm_hist: Dict[int, Tuple[int, int]] = {}
+_warm_next: Dict[Tuple[int, int, int], "weakref.ref"] = {}  # (device, layer before, layer) -> the layer that followed
+_warm_pending: Dict[int, Optional[torch.Tensor]] = {}       # the tensor a hint not yet launched may point into
+
+
+def set_warm_ahead(on: bool) -> None:
+    global _warm_ahead
+    _warm_ahead = bool(on)
+    _warm_hist.clear()
+    _warm_next.clear()
+    if _warm_pending:
+        _lib.load().rtp_gemm_warm_next(None, 0)
+        _warm_pending.clear()
+
+
+def warm_ahead() -> bool:
+    return _warm_ahead
+
+
+def _warm_step(home: torch.Tensor) -> None:
+    """A rotation over `home` starts (direct mode).  The table holds weak references, so it keeps no model alive; the
+    one tensor a pending hint points into is held until the next rotation replaces or withdraws the hint (the
+    library drops a hint with the first product launched after it, carried or not)."""
+    idx = home.device.index if home.device.index is not None else torch.cuda.current_device()
+    prev, cur = _warm_hist.get(idx, (0, 0))
+    here = home.data_ptr()
+    if here == cur:
+        return  # the same layer again (its backward pass right after its forward pass)
+    if len(_warm_next) > 4096:
+        _warm_next.clear()  # far more layers than any model rotates: stale entries of models long gone
+    _warm_next[(idx, prev, cur)] = weakref.ref(home)
+    _warm_hist[idx] = (cur, here)
+    ref = _warm_next.get((idx, cur, here))
+    nxt = ref() if ref is not None else None
+    lib = _lib.load()
+    if nxt is not None and nxt.is_cuda and nxt.data_ptr() != here:
+        _warm_pending[idx] = nxt
+        check(lib.rtp_gemm_warm_next(nxt.data_ptr(), nxt.numel() * nxt.element_size()))
+    elif _warm_pending.get(idx) is not None:
+        _warm_pending[idx] = None
+        check(lib.rtp_gemm_warm_next(None, 0))
 
 
 # ---- weight gradients on a second stream -----------------------------------------------------------
@@ -365,6 +420,8 @@ class Rotation:
         self.steps = len(self.windows)
         self.direct = _mode == "direct"
         if self.direct:
+            if _warm_ahead:
+                _warm_step(home)
             return
         self.ring = device_ring(home.device)
         self.lib = _lib.load()

@@ -317,3 +317,52 @@ def test_gemm_256x256_tile_path(akc, bkc):
         _lib.profile_enable(0)
     assert any("256x256" in nm for nm in names), names
     assert rel_err(out, ref) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("warm_bytes", [16, 1024, 3 * 1024 + 16, 1 << 20, 80 << 20])
+def test_gemm_carries_a_warm_ahead_hint(warm_bytes):
+    """rtp_gemm_warm_next: the next product reads the hinted region at its start and its result is what it is without
+    the hint, bit for bit; regions that are no multiple of the 1 KiB request size, smaller than one request and larger
+    than a launch can take are all fine.  The hint ends with that launch: a second product runs without it."""
+    from rtp_amd import _lib
+    ops = _ops()
+    lib = _lib.load()
+    dtype = torch.bfloat16
+    gen = torch.Generator().manual_seed(3)
+    m, n, k = 300, 520, 200
+    x, w = _rand((m, k), dtype, gen).to(DEV), _rand((n, k), dtype, gen).to(DEV)
+    region = torch.ones(warm_bytes, dtype=torch.uint8, device=DEV)
+    plain = torch.empty(m, n, dtype=dtype, device=DEV)
+    ops.linear_fwd(x, w, plain)
+    hinted = torch.full((m, n), float("nan"), dtype=dtype, device=DEV)
+    _lib.check(lib.rtp_gemm_warm_next(region.data_ptr(), warm_bytes))
+    ops.linear_fwd(x, w, hinted)
+    del region  # the hint is gone with the launch: the next product must not touch the freed region
+    torch.cuda.empty_cache()
+    again = torch.empty(m, n, dtype=dtype, device=DEV)
+    ops.linear_fwd(x, w, again)
+    torch.cuda.synchronize()
+    assert torch.equal(plain, hinted) and torch.equal(plain, again)
+    # a launch that cannot carry the hint (the one-wavefront kernel for tiny products) ends it as well
+    region = torch.ones(4096, dtype=torch.uint8, device=DEV)
+    _lib.check(lib.rtp_gemm_warm_next(region.data_ptr(), 4096))
+    tiny = torch.empty(8, 8, dtype=dtype, device=DEV)
+    ops.linear_fwd(x[:8, :8].contiguous(), w[:8, :8].contiguous(), tiny)
+    del region
+    torch.cuda.empty_cache()
+    ops.linear_fwd(x, w, again)
+    torch.cuda.synchronize()
+    assert torch.equal(plain, again)
+    with pytest.raises(_lib.RtpError):
+        _lib.check(lib.rtp_gemm_warm_next(x.data_ptr() + 2, 64))
+
+
+def test_cache_warm_reads_and_changes_nothing():
+    from rtp_amd import _lib
+    lib = _lib.load()
+    t = torch.arange(1 << 20, dtype=torch.int32, device=DEV)
+    want = t.clone()
+    for nbytes in (0, 16, 4096 + 48, t.numel() * 4):
+        _lib.check(lib.rtp_cache_warm(torch.cuda.current_stream().cuda_stream, t.data_ptr(), nbytes, 0))
+    torch.cuda.synchronize()
+    assert torch.equal(t, want)

@@ -192,3 +192,51 @@ def test_direct_rotation_reads_home_rows_and_stages_nothing(window):
         for j, win in enumerate(rot.windows):
             assert sorted(s for f, c in win for s in range(f, f + c)) == sorted(order[j * w:(j + 1) * w])
     assert ring.staging_bytes() == before
+
+
+def test_warm_ahead_learns_the_layer_order_and_changes_no_result():
+    """Direct rotation with the next layer's shards handed to the current layer's first product: after one pass the
+    table knows, for the forward and for the backward order, which layer follows which; outputs and gradients are
+    bit-identical with the switch off; the table keeps no layer alive."""
+    import gc
+    import weakref
+    from rtp_amd import emulate_shards, ring
+    from rtp_amd.module.linear import ColumnParallelLinear
+    ring.set_rotation_mode("direct")
+    ws, d = 4, 256
+    gen = torch.Generator().manual_seed(11)
+    with emulate_shards(ws):
+        layers = [ColumnParallelLinear(d, d, device=DEV, dtype=torch.bfloat16) for _ in range(3)]
+    x = (torch.randn(130, d, generator=gen) * 0.3).to(torch.bfloat16).to(DEV)
+
+    def run():
+        xi = x.clone().requires_grad_(True)
+        h = xi
+        for lyr in layers:
+            h = lyr(h)
+        h.float().square().mean().backward()
+        out = [h.detach().clone(), xi.grad.clone()] + [p.grad.clone() for lyr in layers for p in lyr.parameters()]
+        for lyr in layers:
+            lyr.zero_grad(set_to_none=True)
+        return out
+
+    try:
+        ring.set_warm_ahead(False)
+        want = run()
+        ring.set_warm_ahead(True)
+        for _ in range(3):
+            got = run()
+            assert all(torch.equal(a, b) for a, b in zip(want, got))
+        homes = [lyr._store.home.data_ptr() for lyr in layers]
+        idx = torch.device(DEV).index or 0
+        follows = {(k[1], k[2]): v().data_ptr() for k, v in ring._warm_next.items() if k[0] == idx and v() is not None}
+        assert follows[(homes[0], homes[1])] == homes[2]       # forward order
+        assert follows[(homes[2], homes[1])] == homes[0]       # backward order
+        probe = weakref.ref(layers[1]._store.home)
+        del layers[:], got, want
+        gc.collect()
+        ring.set_warm_ahead(True)  # clears what may still be pending
+        gc.collect()
+        assert probe() is None
+    finally:
+        ring.set_warm_ahead(True)
