@@ -25,12 +25,21 @@ if ROOT not in sys.path:
 CFG = dict(vocab=10240, ninp=2048, nhid=2048, nhead=32, layers=10, seq=32, batch=32, shards=8)
 PEAK = {"bf16_mfma_tflops": 2500.0, "fp32_mfma_tflops": 157.3, "hbm_gbs": 8000.0}
 # Memory-side traffic per launch of the GEMM variants of this workload, KiB, averaged over the launches of a step:
-# FETCH_SIZE * 1.9927 + WRITE_SIZE * 1.0000 from two rocprofv3 --pmc runs of this script; the factors are what the same
+# FETCH_SIZE * 1.9999 + WRITE_SIZE * 1.0000 from two rocprofv3 --pmc runs of this script; the factors are what the same
 # counters read for the library's plain copy kernel on a copy of known size (profiles/lm_step_pmc_fetch_write.txt).
+# The weight-gradient variant (128x128 rc_rc) carries the clip + SGD update: its figure includes the fp32 parameters
+# read and written and their bf16 copy written.
 MEASURED_TRAFFIC_KIB = {
-    "gemm_bf16_128x128_rc_rc": 45809.5, "gemm_bf16_128x64_kc_rc": 59047.3, "gemm_bf16_128x64_kc_kc": 36974.4,
-    "gemm_bf16_128x192_kc_kc": 74863.4,
+    "gemm_bf16_128x128_rc_rc": 106570.1, "gemm_bf16_128x64_kc_rc": 69584.4, "gemm_bf16_128x64_kc_kc": 46835.8,
+    "gemm_bf16_128x192_kc_kc": 106247.3,
 }
+
+
+# rocprofv3's average duration of a dispatch over the kernel's own execution span (first wave's start to last wave's
+# end, printed by this script as roofline.execution_span), both from the one rocprofv3 run of the default command
+# whose summary is profiles/lm_step_kernel_trace.txt: 44.112 us / 35.188 us for the weight-gradient product,
+# 35.847 / 29.544 for the input-gradient product.
+DISPATCH_OVER_EXECUTION_SPAN = {"gemm_bf16_128x128_rc_rc": 44.112 / 35.188, "gemm_bf16_128x64_kc_rc": 35.847 / 29.544}
 
 
 def step_flops(c):
@@ -163,7 +172,57 @@ def attainable_peaks(dev):
         yard[f"{m_}x{n_}x{k_}"] = {"this_library_us": t_lib * 1e6, "this_library_tflops": fl / t_lib / 1e12,
                                    "torch_matmul_us": t_ven * 1e6, "torch_matmul_tflops": fl / t_ven / 1e12}
     out["yardstick_torch_matmul_same_data"] = yard
+    # What the matrix pipes sustain with nothing else in the way: a register-only MFMA loop on every SIMD, with
+    # constant and with normally distributed operands.  The second is the practical ceiling of a bf16 product.
+    import ctypes
+    from rtp_amd import _lib
+    rate = ctypes.c_double(0.0)
+    probe = {}
+    for name, mode in (("constant_operands", 0), ("random_operands", 1)):
+        _lib.check(_lib.load().rtp_probe_mfma_rate(torch.cuda.current_stream().cuda_stream, mode, 20000, ctypes.byref(rate)))
+        probe[name] = rate.value
+    out["mfma_register_loop_tflops"] = probe
     return out
+
+
+def gemm_workload(shape, operands, engine, steps, warmup):
+    """One bf16 product, repeated: the measurement behind the GEMM ceiling figures.  Run it under
+    `rocprofv3 --pmc GRBM_GUI_ACTIVE` for the sustained clock (busy cycles / duration) with zero-filled and with random
+    operands, and with --engine torch for the vendor library's time on the same data."""
+    import torch
+    from rtp_amd import ops
+    dev = torch.device("cuda", 0)
+    m, n, k = (int(v) for v in shape.lower().split("x"))
+    gen = torch.Generator().manual_seed(1)
+    if operands == "random":
+        x = torch.randn(m, k, generator=gen).to(torch.bfloat16).to(dev)
+        w = torch.randn(n, k, generator=gen).to(torch.bfloat16).to(dev)
+    else:
+        x = torch.zeros(m, k, dtype=torch.bfloat16, device=dev)
+        w = torch.zeros(n, k, dtype=torch.bfloat16, device=dev)
+    y = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+    wt = w.t()
+    if engine == "rtp":
+        def one():
+            ops.gemm_raw(torch.bfloat16, a=x.data_ptr(), b=w.data_ptr(), c_out=y.data_ptr(), m=m, n=n, k=k, lda=k, ldb=k,
+                         ldc=n, a_kcontig=True, b_kcontig=True)
+    else:
+        def one():
+            torch.matmul(x, wt, out=y)
+    for _ in range(warmup):
+        one()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(steps):
+        one()
+    e1.record()
+    torch.cuda.synchronize()
+    t = e0.elapsed_time(e1) * 1e-3 / steps
+    print(json.dumps({"metric": "bf16 product, TFLOP/s", "value": 2.0 * m * n * k / t / 1e12, "unit": "TFLOP/s",
+                      "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": t * 1e3, "higher_is_better": True,
+                      "dtype": "bf16", "data": "synthetic",
+                      "config": {"workload": f"one product {m}x{n}x{k}, {operands} operands, engine {engine}"}}))
 
 
 def layer_workload(name, steps, warmup, graph=True, cpu=True):
@@ -370,7 +429,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", default="lm", choices=["lm", "linear", "embedding", "attention", "moe"],
+    ap.add_argument("--workload", default="lm", choices=["lm", "linear", "embedding", "attention", "moe", "gemm"],
                     help="lm: the headline training step (default); the others time one rotated layer of the "
                          "reference's remaining configurations, fwd+bwd")
     ap.add_argument("--sgd-overlap", dest="sgd_overlap", action="store_true",
@@ -395,8 +454,14 @@ def main():
                          "product kernel is the rotation's double buffer; staged: shards are first copied into two HBM "
                          "slots on a side stream (the transport of a multi-GPU ring)")
     ap.add_argument("--no-warm-ahead", dest="warm_ahead", action="store_false",
-                    help="do not read the next layer's shards into the memory-side cache on a side stream while the "
-                         "current layer computes (direct rotation only)")
+                    help="do not let a layer's first product request the next layer's shards, which brings them into "
+                         "the memory-side cache before their own products run (direct rotation only)")
+    ap.add_argument("--operands", default="random", choices=["random", "zeros"],
+                    help="--workload gemm: normally distributed or all-zero bf16 operands")
+    ap.add_argument("--engine", default="rtp", choices=["rtp", "torch"],
+                    help="--workload gemm: this library's product kernel, or torch.matmul (the vendor library) as the "
+                         "yardstick on the same data")
+    ap.add_argument("--shape", default="4096x4096x4096", help="--workload gemm: MxNxK of y[M,N] = x[M,K] w[N,K]^T")
     ap.add_argument("--no-graph", dest="graph", action="store_false",
                     help="launch every kernel eagerly instead of replaying the step from a captured HIP graph")
     args = ap.parse_args()
@@ -405,6 +470,9 @@ def main():
               f"has no multi-GPU path (--gpus {args.gpus} is not supported)", file=sys.stderr)
         sys.exit(2)
 
+    if args.workload == "gemm":
+        gemm_workload(args.shape, args.operands, args.engine, args.steps, args.warmup)
+        return
     if args.workload != "lm":
         layer_workload(args.workload, args.steps, args.warmup, args.graph, not args.no_cpu_baseline)
         return
@@ -509,21 +577,35 @@ def main():
         _lib.profile_collect()
         del g2
 
-    # Per-kernel timing with HIP events around every launch, on two extra EAGER steps (every kernel of the library,
-    # but launched from Python: the second stream is mostly idle then, so these are not the timed mode's durations).
+    # Per-kernel timing with HIP events around every launch in extra EAGER steps: every kernel of the library, for the
+    # `kernels` table.  With an event pair per launch the host cannot keep the GPU fed (eager_ms_per_step below), so
+    # the two streams hardly overlap here: these are not the timed mode's durations.
     _lib.profile_enable(True)
     prof_steps = 2
+    torch.cuda.synchronize()
+    t_e = time.perf_counter()
     for _ in range(prof_steps):
         step()
+    torch.cuda.synchronize()
+    eager_ms = (time.perf_counter() - t_e) / prof_steps * 1e3
     stats = _lib.profile_collect()
     _lib.profile_enable(False)
     gemms = {k: v for k, v in stats.items() if k.startswith("gemm_")}
     timed_gemms = {k: v for k, v in (graph_stats or stats).items() if k.startswith("gemm_")}
     dom_name, dom = max(timed_gemms.items(), key=lambda kv: kv[1]["total_ms"])
-    avg_ms = dom["total_ms"] / dom["launches"]
+    span_us = dom["total_ms"] / dom["launches"] * 1e3
+    # rocprofv3 reports a longer duration for the same dispatches than the kernel's own first-wave-to-last-wave span:
+    # its clock starts when the queue reaches the dispatch, and the workgroups then still wait for the CUs that the
+    # other stream's product holds.  The ratio of the two was measured in the rocprofv3 run of this very command
+    # (profiles/lm_step_kernel_trace.txt: average duration / the span this script printed in that run); the roofline
+    # figure is quoted on the longer, rocprofv3-compatible span.
+    ratio = DISPATCH_OVER_EXECUTION_SPAN.get(dom_name, 1.0) if graph_stats is not None else 1.0
+    avg_ms = span_us * ratio * 1e-3
     achieved = dom["flops"] / dom["launches"] / (avg_ms * 1e-3) / 1e12
-    eager = gemms[dom_name]
-    achieved_eager = eager["flops"] / eager["total_ms"] / 1e9
+    span = {"avg_launch_us": span_us, "frac": dom["flops"] / dom["launches"] / (span_us * 1e-6) / 1e12 / PEAK["bf16_mfma_tflops"],
+            "what": "first wave's start to last wave's end of the kernel (device time stamps in the replayed HIP graph; HIP "
+                    "events in eager mode): its own execution, without the wait for CUs that a dispatch span includes",
+            "instrumented_replay_ms_per_step": instr_ms}
     all_gemm_ms = sum(v["total_ms"] for v in gemms.values()) / prof_steps
     all_gemm_tflops = sum(v["flops"] for v in gemms.values()) / prof_steps / (all_gemm_ms * 1e-3) / 1e12
     copy = stats.get("shard_copy")
@@ -559,10 +641,12 @@ def main():
                      "avg_launch_us": avg_ms * 1e3,
                      "launches_per_step": dom["launches"] // (5 if graph_stats is not None else prof_steps),
                      "flops_per_launch": dom["flops"] / dom["launches"],
-                     "timed_in": ("HIP-graph replay of the step, both streams live, device time stamps per launch"
+                     "timed_in": ("HIP-graph replay of the step, both streams live: device time stamps per launch, times the "
+                                  "measured ratio of rocprofv3's dispatch duration to that span"
                                   if graph_stats is not None else "eager launches, HIP events"),
-                     "frac_standalone_eager": achieved_eager / PEAK["bf16_mfma_tflops"],
-                     "instrumented_replay_ms_per_step": instr_ms},
+                     "dispatch_over_execution_span": ratio,
+                     "execution_span": span,
+                     "eager_ms_per_step_with_event_pairs": eager_ms},
         "gemm_kernels_in_graph_replay": graph_gemms,
         "measured_attainable": dict(peaks, dominant_kernel_frac_of_measured_gemm=achieved / peaks["gemm_bf16_4096_cubed_tflops"]),
         "step_mfma_frac": flops / dt / (PEAK["bf16_mfma_tflops"] * 1e12),

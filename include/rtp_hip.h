@@ -226,6 +226,12 @@ int rtp_gemm(void* stream, int dtype, const rtp_gemm_desc* d);
  * only until then.  bytes == 0 withdraws a pending hint. */
 int rtp_gemm_warm_next(const void* src, size_t bytes);
 
+/* Measurement aid (no counterpart in the reference; bench.py reports it beside the published peak): TFLOP/s of a
+ * register-only loop of v_mfma_f32_32x32x16_bf16 on every SIMD of the device, `iters` iterations of 32 MFMAs per
+ * wavefront, with constant operands (random_operands == 0) or normally distributed ones (1).  Synchronises on
+ * `stream`; allocates and frees 4 bytes. */
+int rtp_probe_mfma_rate(void* stream, int random_operands, int iters, double* tflops);
+
 /* 1 if rtp_gemm would produce d->a_rowsum for this descriptor (the pointer itself may still be NULL), else 0. */
 int rtp_gemm_rowsum_fused(int dtype, const rtp_gemm_desc* d);
 

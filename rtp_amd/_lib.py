@@ -97,6 +97,7 @@ PROTOTYPES = {
     "rtp_softmax_xent_combine": (_i, [_vp, _vp, _i64, _vp, _vp, _i64, _i64, _vp, _vp]),
     "rtp_gemm": (_i, [_vp, _i, C.POINTER(GemmDesc)]),
     "rtp_gemm_warm_next": (_i, [_vp, _sz]),
+    "rtp_probe_mfma_rate": (_i, [_vp, _i, _i, C.POINTER(C.c_double)]),
     "rtp_gemm_rowsum_fused": (_i, [_i, C.POINTER(GemmDesc)]),
     "rtp_gemm_sgd_fused": (_i, [_i, C.POINTER(GemmDesc)]),
     "rtp_gemm_desc_size": (_sz, []),

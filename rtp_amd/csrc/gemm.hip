@@ -1725,7 +1725,11 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   const double kk = (double)d->k * (double)d->ksegs;
   const double out_sz = (d->flags & RTP_GEMM_OUT_F32) ? 4.0 : (double)sizeof(T);
   const double cin_sz = d->c_in ? ((d->flags & RTP_GEMM_CIN_F32) ? 4.0 : (double)sizeof(T)) : 0.0;
-  const double bytes = ((double)d->m + (double)d->n) * kk * nz * sizeof(T) + mn * (out_sz + cin_sz);
+  // operands once + the output (and addend); a fused update reads and writes the fp32 parameters and writes their copy
+  const double upd_sz = d->sgd_master ? 8.0 + (d->sgd_weights ? (double)sizeof(T) : 0.0) -
+                                            ((d->flags & RTP_GEMM_SGD_SKIP_OUT) ? out_sz : 0.0)
+                                      : 0.0;
+  const double bytes = ((double)d->m + (double)d->n) * kk * nz * sizeof(T) + mn * (out_sz + cin_sz + upd_sz);
   ProfileScope prof(s, name, 2.0 * mn * kk, bytes);
   a.trace = fast ? prof.trace_slot() : nullptr;
   a.warm = nullptr;
