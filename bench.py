@@ -363,6 +363,20 @@ def layer_workload(name, steps, warmup, graph=True, cpu=True):
         raise SystemExit(f"unknown workload {name}")
 
     from rtp_amd import ring
+    from rtp_amd.module.collectives import ShardStore
+    # Every pass starts like a training step, after zero_grad: the rotated gradients are overwritten, not added to
+    # (what RotatedSGD.zero_grad arranges), and the input's gradient is a fresh tensor.
+    stores = [m._store for m in layer.modules() if isinstance(getattr(m, "_store", None), ShardStore)]
+    inputs = [t for t in (locals().get("x"),) if torch.is_tensor(t) and t.requires_grad]
+    body = fn
+
+    def fn():
+        for st in stores:
+            st.mark_overwrite()
+        for t in inputs:
+            t.grad = None
+        body()
+
     # warm-up on a side stream, then the layer's forward + backward recorded once into a HIP graph and replayed
     # (as for the language-model step); --no-graph times eager launches, CPU launch overhead included
     side = torch.cuda.Stream()

@@ -1638,11 +1638,12 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   int shape = 3;  // 64 x 64 unless the model finds something cheaper
   double best = 0.0;
   for (int i = 0; fast && i < kNumShapes; ++i) {
-    // the 256 x 256 kernel is built for 16-bit operands and the plain epilogue, and pays only on very large
-    // products (measured: +9 % forward, +20 % on the transposed layouts at 8192^3, nothing at 4096^3, a loss
-    // where it leaves CUs without a tile)
+    // the 256 x 256 kernel is built for 16-bit operands and the plain epilogue, and pays on products with a long
+    // contraction that give every CU at least one such tile (measured: +9 % forward, +20 % on the transposed
+    // layouts at 8192^3, +10 - 20 % on the expert products of the MoE layer, nothing at 4096^3, a loss where it
+    // leaves CUs without a tile or K is short)
     if (i == 5 && (sizeof(T) != 2 || d->sgd_master || d->xent_mode == 1 ||
-                   ceil_div(d->m, 256) * ceil_div(d->n, 256) * nz < 1024 || d->k * d->ksegs < 2048) && i != forced)
+                   ceil_div(d->m, 256) * ceil_div(d->n, 256) * nz < 256 || d->k * d->ksegs < 2048) && i != forced)
       continue;
     // never a tile that is mostly padding: a 32 x 32 problem (one attention head at seq 32) stays at 64 x 64
     if ((!akc && (kShapes[i].bm & (kShapes[i].bm - 1))) || (!bkc && (kShapes[i].bn & (kShapes[i].bn - 1)))) continue;

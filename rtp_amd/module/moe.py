@@ -131,7 +131,10 @@ class _ExpertsFn(torch.autograd.Function):
                 w1, b1, w2, b2 = store.offsets[4 * le:4 * le + 4]
                 r0 = (first * n_local + le) * c_rows
                 base = g.data_ptr() + first * store.numel * es
-                common = dict(groups=cnt, c_sg=store.numel, cin_sg=store.numel, a_kcontig=False, b_kcontig=False)
+                # stream_out: an expert's gradient (tens of MB per launch) is not read again before the optimiser, and
+                # written with ordinary stores it evicts the launch's own operands from the caches (468 -> 338 us)
+                common = dict(groups=cnt, c_sg=store.numel, cin_sg=store.numel, a_kcontig=False, b_kcontig=False,
+                              stream_out=True)
                 # dW2 = dY^T H ; dW1 = dH^T X  (contraction over the expert's capacity rows); the bias gradients are
                 # the row sums of the first operands and come out of the same launches where the library can fuse them
                 c2 = base + w2 * es
