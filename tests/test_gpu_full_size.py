@@ -93,10 +93,13 @@ def test_lm_headline_config_full_size_bf16():
     assert float(after) < float(loss.detach())
 
 
-def test_lm_headline_config_graph_replays_equal_eager_steps():
+@pytest.mark.parametrize("fused", [False, True], ids=["separate-update", "update-in-wgrad-epilogue"])
+def test_lm_headline_config_graph_replays_equal_eager_steps(fused):
     """The benchmark's measurement mode at the benchmark's size: the 10-layer bf16 step recorded into a HIP graph
-    (weight gradients on their second stream, as bench.py runs it) and replayed with new token ids stays
-    bit-identical, weights and loss, to a twin model that takes the same steps eagerly."""
+    (weight gradients on their second stream, the next layer's shards requested ahead, and -- the benchmark's default
+    -- clip + SGD applied in the epilogues of the weight-gradient products) and replayed with new token ids stays
+    bit-identical, weights and loss, to a twin model that takes the same steps eagerly with the separate update
+    launch."""
     from test_gpu_lm import graph_replays_against_eager_twin
     from rtp_amd import ring
     from rtp_amd.models.transformer_lm_rtp import TransformerLM
@@ -111,7 +114,7 @@ def test_lm_headline_config_graph_replays_equal_eager_steps():
     before = ring.wgrad_overlap()
     ring.set_wgrad_overlap(True)
     try:
-        loss = graph_replays_against_eager_twin(twins, V, L, N, replays=3, lr=1e-3)
+        loss = graph_replays_against_eager_twin(twins, V, L, N, replays=3, lr=1e-3, fused_replayed=fused)
     finally:
         ring.set_wgrad_overlap(before)
     assert 0.0 < loss < 20.0

@@ -286,14 +286,16 @@ def test_lm_embedding_scale_and_positions_on_the_gather_are_bit_identical(dtype)
         assert torch.equal(g, results[1][1][k]), k
 
 
-def graph_replays_against_eager_twin(twin_lms, V, L, N, replays, lr=1e-2):
+def graph_replays_against_eager_twin(twin_lms, V, L, N, replays, lr=1e-2, fused_replayed=False):
     """Record one whole training step of twin_lms[0] into a HIP graph and replay it `replays` times with new token ids,
     eager work and synchronisation in between; twin_lms[1] (same weights) takes the same steps eagerly.  Losses and
-    all weights must stay bit-identical."""
+    all weights must stay bit-identical.  `fused_replayed`: the replayed twin applies clip + SGD in the epilogues of
+    its weight-gradient products while the eager twin keeps the separate update launch."""
     from rtp_amd import ring
     from rtp_amd.module.loss import cross_entropy
     from rtp_amd.optim import RotatedSGD
-    twins = [(lm, RotatedSGD(lm, lr=lr, clip_value=0.05)) for lm in twin_lms]
+    twins = [(lm, RotatedSGD(lm, lr=lr, clip_value=0.05, fused_backward=fused_replayed and i == 0))
+             for i, lm in enumerate(twin_lms)]
     gen = torch.Generator().manual_seed(5)
     ids = torch.randint(0, V, (L, N), generator=gen).to(DEV)
     tgt = torch.randint(0, V, (L, N), generator=gen).to(DEV)
