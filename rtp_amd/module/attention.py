@@ -30,7 +30,13 @@ from .utils import (affine_weight, affine_weight_attention, as_rows, attention_b
 class SubParallelMultiheadAttention(nn.Module):
     """Parameters of one head group (rtp/module/attention.py:17-104).  Declaration order fixes the
     flat-shard layout: in_proj_weight (or q_proj_weight, k_proj_weight, v_proj_weight when keys or values have
-    their own width), in_proj_bias, out_proj.weight, out_proj.bias."""
+    their own width), in_proj_bias, bias_k, bias_v (add_bias_kv), out_proj.weight, out_proj.bias -- torch's own
+    order: a module's parameters before its children's.
+
+    add_bias_kv: the reference declares bias_k / bias_v at full width [1, 1, embed_dim] in every shard and
+    concatenates them to keys of width embed_dim / ws (attention.py:70-72, functional.py:711-716), which only runs
+    with one shard.  Here a shard holds its head group's slice [1, 1, embed_dim / ws] of them, so that the rotated
+    layer equals nn.MultiheadAttention(add_bias_kv=True) for any shard count (and the reference for one)."""
 
     def __init__(self, embed_dim, num_heads, world_size, rank, dropout=0., bias=True, add_bias_kv=False,
                  add_zero_attn=False, kdim=None, vdim=None, batch_first=False, device=None, dtype=None) -> None:
@@ -40,11 +46,6 @@ class SubParallelMultiheadAttention(nn.Module):
         super().__init__()
         kdim = embed_dim if kdim is None else kdim
         vdim = embed_dim if vdim is None else vdim
-        if add_bias_kv:
-            # the reference keeps bias_k / bias_v at full width [1, 1, embed_dim] in every shard and concatenates
-            # them to keys of width embed_dim / ws (attention.py:70-72, functional.py:711-716): that only runs
-            # with one shard, so there is no sharded behaviour to reproduce
-            raise NotImplementedError("rotated attention: add_bias_kv is not implemented")
         self.embed_dim, self.kdim, self.vdim = embed_dim, kdim, vdim
         self._qkv_same_embed_dim = kdim == embed_dim and vdim == embed_dim
         self.num_heads = num_heads
@@ -71,7 +72,11 @@ class SubParallelMultiheadAttention(nn.Module):
         else:
             self.register_parameter("in_proj_bias", None)
         self.out_proj = NonDynamicallyQuantizableLinear(e_s, embed_dim, bias=bias, **kw)
-        self.bias_k = self.bias_v = None
+        if add_bias_kv:
+            self.bias_k = Parameter(torch.empty((1, 1, e_s), **kw))
+            self.bias_v = Parameter(torch.empty((1, 1, e_s), **kw))
+        else:
+            self.bias_k = self.bias_v = None
         self.add_zero_attn = add_zero_attn
         self._reset_parameters()
 
@@ -86,6 +91,9 @@ class SubParallelMultiheadAttention(nn.Module):
         if self.in_proj_bias is not None:
             nn.init.constant_(self.in_proj_bias, 0.)
             nn.init.constant_(self.out_proj.bias, 0.)
+        if self.bias_k is not None:
+            nn.init.xavier_normal_(self.bias_k)
+            nn.init.xavier_normal_(self.bias_v)
 
     def affine_weight(self, mha) -> None:
         if mha is None:
@@ -101,6 +109,12 @@ class SubParallelMultiheadAttention(nn.Module):
         if self.bias:
             affine_weight_attention(self.in_proj_bias, mha.in_proj_bias, idx, e_s, 0, self.world_size, self.rank)
         affine_weight(self.out_proj.weight, mha.out_proj.weight, e_s, 1, self.world_size, self.rank)
+        if self.bias_k is not None:
+            if mha.bias_k is None:
+                raise ValueError("add_bias_kv: the layer to import has no bias_k / bias_v")
+            with torch.no_grad():  # the head group's columns of the appended key / value
+                self.bias_k.copy_(mha.bias_k[..., self.rank * e_s:(self.rank + 1) * e_s])
+                self.bias_v.copy_(mha.bias_v[..., self.rank * e_s:(self.rank + 1) * e_s])
         if self.bias:
             with torch.no_grad():
                 self.out_proj.bias.data.copy_(mha.out_proj.bias.data)
@@ -327,17 +341,26 @@ def _shard_layout(layer):
         wq, wk, wv, nxt = off[0], off[1], off[2], 3
     else:
         wq, wk, wv, nxt = off[0], off[0] + e_s * E, off[0] + 2 * e_s * E, 1
+    kv = 2 if layer.add_bias_kv else 0  # bias_k, bias_v sit between the input projection and the output projection
     if layer.has_bias:
-        return wq, wk, wv, off[nxt], off[nxt + 1], off[nxt + 2]
-    return wq, wk, wv, None, off[nxt], None
+        return wq, wk, wv, off[nxt], off[nxt + 1 + kv], off[nxt + 2 + kv]
+    return wq, wk, wv, None, off[nxt + kv], None
+
+
+def _bias_kv_layout(layer):
+    """Element offsets of (bias_k, bias_v) inside a flat shard."""
+    off = layer._store.offsets
+    nxt = (3 if layer.separate_proj else 1) + (1 if layer.has_bias else 0)
+    return off[nxt], off[nxt + 1]
 
 
 class _GeneralAttentionFn(torch.autograd.Function):
     """Attention whose keys and values come from their own tensors (query [L, N, E], key [S, N, kdim], value
-    [S, N, vdim]; functional.py:575-609 projects them with three row blocks of the shard), optionally with one
-    all-zero key / value appended per batch entry (add_zero_attn, functional.py:746-753).  Three projections per
-    shard run into q [L*N, E], k and v [(S+z)*N, E] (group g at column block g); the core is batched products and
-    the softmax kernel with p [ws*N*h_s, L, S+z] in memory."""
+    [S, N, vdim]; functional.py:575-609 projects them with three row blocks of the shard), optionally with the
+    learned key / value bias_k / bias_v (add_bias_kv, functional.py:711-716) and then one all-zero key / value
+    (add_zero_attn, functional.py:746-753) appended per batch entry.  Three projections per shard run into
+    q [L*N, E], k and v [(S+z)*N, E] (group g at column block g; z appended positions); the core is batched products
+    and the softmax kernel with p [ws*N*h_s, L, S+z] in memory."""
 
     @staticmethod
     def forward(ctx, query, key, value, anchor, layer, mask, key_bias, want_weights, drop_p=0.0):
@@ -345,7 +368,8 @@ class _GeneralAttentionFn(torch.autograd.Function):
         L, N, E = query.shape
         s_in = key.shape[0]
         zero = 1 if layer.add_zero_attn else 0
-        sk = s_in + zero
+        bkv = 1 if layer.add_bias_kv else 0
+        sk = s_in + bkv + zero
         ws, h_s, d, e_s = layer.world_size, layer.num_heads_per_partition, layer.head_dim, layer.embed_dim_per_partition
         dt, dev = query.dtype, query.device
         q2, k2, v2 = as_rows(query, E), as_rows(key, layer.kdim), as_rows(value, layer.vdim)
@@ -357,8 +381,9 @@ class _GeneralAttentionFn(torch.autograd.Function):
         kb = torch.empty(sk * N, E, dtype=dt, device=dev)
         vb = torch.empty(sk * N, E, dtype=dt, device=dev)
         if zero:
-            kb[s_in * N:].zero_()
-            vb[s_in * N:].zero_()
+            kb[(s_in + bkv) * N:].zero_()
+            vb[(s_in + bkv) * N:].zero_()
+        bk_off, bv_off = _bias_kv_layout(layer) if bkv else (None, None)
         o = torch.empty(L * N, E, dtype=dt, device=dev)
         out = torch.empty(L * N, E, dtype=dt, device=dev)
         p = torch.empty(ws * Z, L, sk, dtype=dt, device=dev)
@@ -375,6 +400,9 @@ class _GeneralAttentionFn(torch.autograd.Function):
                 S.col_fwd(q2, flat, wq, e_s, E, bq, qb, c0)
                 S.col_fwd(k2, flat, wk, e_s, layer.kdim, bk, kb[:s_in * N], c0)
                 S.col_fwd(v2, flat, wv, e_s, layer.vdim, bv, vb[:s_in * N], c0)
+                if bkv:  # position s_in of every batch entry: the head groups' slices of bias_k / bias_v
+                    kb[s_in * N:(s_in + 1) * N, c0:c0 + cnt * e_s] = flat[:, bk_off:bk_off + e_s].reshape(1, cnt * e_s)
+                    vb[s_in * N:(s_in + 1) * N, c0:c0 + cnt * e_s] = flat[:, bv_off:bv_off + e_s].reshape(1, cnt * e_s)
                 scores = torch.empty(cnt * Z, L, sk, dtype=torch.float32, device=dev)
                 _bmm(dt, a=qb, a_off=c0, lda=ld, a_kc=True, a_s=(E, d), a_sg=e_s, b=kb, b_off=c0, ldb=ld, b_kc=True,
                      b_s=(E, d), b_sg=e_s, c=scores, c_off=0, ldc=sk, c_s=(h_s * L * sk, L * sk), c_sg=Z * L * sk,
@@ -484,9 +512,14 @@ class _GeneralAttentionFn(torch.autograd.Function):
                 S.col_wgrad(dqb, q2, store.grads, first, wq, e_s, E, c0, cnt, accumulate, b_off=bq, store=store)
                 S.col_wgrad(dk_in, k2, store.grads, first, wk, e_s, layer.kdim, c0, cnt, accumulate, b_off=bk, store=store)
                 S.col_wgrad(dv_in, v2, store.grads, first, wv, e_s, layer.vdim, c0, cnt, accumulate, b_off=bv, store=store)
+                if layer.add_bias_kv:
+                    # the appended position's key / value gradient, summed over the batch entries it was copied to
+                    bk_off, bv_off = _bias_kv_layout(layer)
+                    S.col_bgrad(dkb[s_in * N:(s_in + 1) * N], store.grads, first, bk_off, e_s, c0, cnt, accumulate)
+                    S.col_bgrad(dvb[s_in * N:(s_in + 1) * N], store.grads, first, bv_off, e_s, c0, cnt, accumulate)
             store.grads_ready()
 
-        run_wgrad(dev, param_grads, (dout2, o, dqb, dk_in, dv_in, q2, k2, v2))
+        run_wgrad(dev, param_grads, (dout2, o, dqb, dkb, dvb, q2, k2, v2))
         grads = [None if item is None else item[0] for item in sums]
         dq = None if grads[0] is None else grads[0].view(L, N, E)
         dk = None if grads[1] is None else grads[1].view(s_in, N, layer.kdim)
@@ -499,7 +532,8 @@ class ParallelMultiheadAttention(RotatedLayer):
     of an unsharded nn.MultiheadAttention.  Self-attention (query, key and value the same tensor) takes the packed
     projection and the fused cores; keys / values from other tensors, kdim / vdim != embed_dim and add_zero_attn take
     three projections and the product + softmax core, and so do attention dropout while training (the probabilities
-    are dropped in memory) and 3-D masks [batch * heads / ws, L, S].  add_bias_kv is not implemented and raises.  key_padding_mask [batch, keys] (bool or float, functional.py:615-623 and :760-768) reaches
+    are dropped in memory), 3-D masks [batch * heads / ws, L, S] and add_bias_kv (a shard holds its head group's slice of
+    bias_k / bias_v, see SubParallelMultiheadAttention).  key_padding_mask [batch, keys] (bool or float, functional.py:615-623 and :760-768) reaches
     the kernels as a per-(batch, key) additive bias."""
 
     def __init__(self, embed_dim, num_heads, world_size, rank, dropout=0., bias=True, add_bias_kv=False,
@@ -523,6 +557,7 @@ class ParallelMultiheadAttention(RotatedLayer):
         self.kdim, self.vdim = layers[0].kdim, layers[0].vdim
         self.separate_proj = not layers[0]._qkv_same_embed_dim
         self.add_zero_attn = bool(add_zero_attn)
+        self.add_bias_kv = bool(add_bias_kv)
         self.num_heads_per_partition = layers[0].num_heads_per_partition
         self.embed_dim_per_partition = layers[0].embed_dim_per_partition
         self._init_store(layers)
@@ -536,7 +571,7 @@ class ParallelMultiheadAttention(RotatedLayer):
         if not same:
             same = (key.data_ptr() == query.data_ptr() == value.data_ptr() and key.shape == query.shape == value.shape
                     and key.stride() == query.stride() == value.stride())
-        general = not same or self.separate_proj or self.add_zero_attn
+        general = not same or self.separate_proj or self.add_zero_attn or self.add_bias_kv
         drop_p = float(self.dropout) if self.training else 0.0
         if not 0.0 <= drop_p < 1.0:
             raise ValueError(f"attention dropout probability has to be in [0, 1), got {drop_p}")
@@ -581,12 +616,14 @@ class ParallelMultiheadAttention(RotatedLayer):
                 raise ValueError(f"rotated attention: query {tuple(query.shape)}, key {tuple(key.shape)} and value "
                                  f"{tuple(value.shape)} do not fit embed_dim / kdim / vdim = "
                                  f"{(self.embed_dim, self.kdim, self.vdim)} and a common batch and key count")
-            if self.add_zero_attn:
-                # functional.py:746-753: the appended all-zero key is visible to every query
+            # functional.py:711-716 and :746-753: the appended bias key and the appended all-zero key are visible to
+            # every query (one zero column each in both masks)
+            extra = int(self.add_bias_kv) + int(self.add_zero_attn)
+            if extra:
                 if mask is not None:
-                    mask = F.pad(mask, (0, 1))
+                    mask = F.pad(mask, (0, extra))
                 if key_bias is not None:
-                    key_bias = F.pad(key_bias, (0, 1))
+                    key_bias = F.pad(key_bias, (0, extra))
             out, weights = _GeneralAttentionFn.apply(x, k_in, v_in, self._anchor, self, mask, key_bias,
                                                      bool(need_weights), drop_p)
         else:

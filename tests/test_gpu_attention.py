@@ -97,7 +97,7 @@ def test_attention_unsupported_raise():
     with pytest.raises(ValueError):
         layer(x, x, x, key_padding_mask=torch.zeros(3, 4, dtype=torch.bool, device=DEV))   # [batch, keys] = [2, 4]
     with pytest.raises(NotImplementedError):
-        ParallelMultiheadAttention(8, 2, 2, 0, add_bias_kv=True, device=DEV)
+        layer(x[:, 0], x[:, 0], x[:, 0])  # unbatched [L, E] inputs
 
 
 @pytest.mark.parametrize("E,H,L,N,ws,masked,need_weights", [

@@ -22,10 +22,11 @@ def _master(E, H, gen, dtype, **kw):
 
 
 def _check(E, H, L, S, N, ws, dtype, *, kdim=None, vdim=None, zero=False, shared_kv=False, mask=False, pad=False,
-           need_weights=False, batch_first=False, seed=0):
+           need_weights=False, batch_first=False, seed=0, bias_kv=False):
     from rtp_amd.module.attention import ParallelMultiheadAttention
     gen = torch.Generator().manual_seed(seed)
-    ref = _master(E, H, gen, dtype, kdim=kdim, vdim=vdim, add_zero_attn=zero, batch_first=batch_first)
+    ref = _master(E, H, gen, dtype, kdim=kdim, vdim=vdim, add_zero_attn=zero, batch_first=batch_first,
+                  add_bias_kv=bias_kv)
     kd, vd = ref.kdim, ref.vdim
     shape = (lambda n, w: (N, n, w)) if batch_first else (lambda n, w: (n, N, w))
     q = torch.randn(shape(L, E), generator=gen).to(dtype)
@@ -43,7 +44,7 @@ def _check(E, H, L, S, N, ws, dtype, *, kdim=None, vdim=None, zero=False, shared
         for n in range(N):
             kpm[n, S - (n % 3):] = n % 3 > 0
     layer = ParallelMultiheadAttention(E, H, ws, 0, kdim=kdim, vdim=vdim, add_zero_attn=zero, batch_first=batch_first,
-                                       MultiheadAttention_layer=ref.to(dtype) if dtype != torch.float32 else ref,
+                                       add_bias_kv=bias_kv, MultiheadAttention_layer=ref.to(dtype) if dtype != torch.float32 else ref,
                                        device=DEV, dtype=dtype)
     ref = ref.float()
     qd = q.to(DEV).requires_grad_()
@@ -77,6 +78,9 @@ def _check(E, H, L, S, N, ws, dtype, *, kdim=None, vdim=None, zero=False, shared
                  "out_proj.weight grad")
     for l in subs:
         assert_close(l.out_proj.bias.grad, ref.out_proj.bias.grad, dtype, "out_proj.bias grad")
+    if bias_kv:  # a shard holds its head group's columns of the appended key / value
+        assert_close(torch.cat([l.bias_k.grad for l in subs], dim=2), ref.bias_k.grad, dtype, "bias_k grad")
+        assert_close(torch.cat([l.bias_v.grad for l in subs], dim=2), ref.bias_v.grad, dtype, "bias_v grad")
     if need_weights:
         # per-head weights of the last head group the rotation visits (shard ws-1 when the home rank is 0)
         with torch.no_grad():
@@ -115,6 +119,35 @@ def test_attention_add_zero_attn_fp32(ws):
     _check(32, 4, 5, 12, 2, ws, torch.float32, zero=True, need_weights=True, seed=6)
 
 
+@pytest.mark.parametrize("ws", [1, 2, 4])
+def test_attention_add_bias_kv_fp32(ws):
+    """The learned key / value bias_k / bias_v appended per batch entry (functional.py:711-716), alone, together with
+    the all-zero key, under masks, with own key / value widths; against nn.MultiheadAttention(add_bias_kv=True), which
+    is what the reference computes with one shard (its shards keep bias_k at full width and cannot run with more)."""
+    _check(32, 4, 8, 8, 3, ws, torch.float32, bias_kv=True, mask=True, pad=True, seed=11)
+    _check(32, 4, 5, 12, 2, ws, torch.float32, bias_kv=True, zero=True, need_weights=True, seed=12)
+    if ws <= 2:
+        _check(32, 4, 6, 10, 3, ws, torch.float32, bias_kv=True, kdim=24, vdim=40, pad=True, seed=13)
+
+
+def test_attention_add_bias_kv_bf16_and_self_attention_input():
+    _check(128, 4, 33, 47, 3, 4, torch.bfloat16, bias_kv=True, pad=True, seed=14)
+    from rtp_amd.module.attention import ParallelMultiheadAttention
+    gen = torch.Generator().manual_seed(15)
+    ref = _master(64, 4, gen, torch.float32, add_bias_kv=True)
+    layer = ParallelMultiheadAttention(64, 4, 2, 0, add_bias_kv=True, MultiheadAttention_layer=ref, device=DEV)
+    x = torch.randn(10, 3, 64, generator=gen)
+    xd = x.to(DEV).requires_grad_()
+    out, _ = layer(xd, xd, xd, need_weights=False)
+    out.sum().backward()
+    xo = x.clone().requires_grad_()
+    want, _ = ref(xo, xo, xo, need_weights=False)
+    want.sum().backward()
+    assert_close(out, want, torch.float32, "output")
+    assert_close(xd.grad, xo.grad, torch.float32, "input grad")
+    assert_close(torch.cat([l.bias_k.grad for l in layer.layers], dim=2), ref.bias_k.grad, torch.float32, "bias_k grad")
+
+
 def test_add_zero_attn_on_self_attention_input():
     """query is key is value with add_zero_attn: the general path, same tensor three times."""
     from rtp_amd.module.attention import ParallelMultiheadAttention
@@ -151,8 +184,9 @@ def test_general_attention_argument_checks():
         layer(q, k, k, key_padding_mask=torch.zeros(2, 5, dtype=torch.bool, device=DEV))
     with pytest.raises(RuntimeError):
         layer(q, k, k, attn_mask=torch.zeros(8, 5, 7, device=DEV))  # 3-D masks are [batch * heads / ws, L, S]
-    with pytest.raises(NotImplementedError):
-        ParallelMultiheadAttention(32, 4, 2, 0, add_bias_kv=True, device=DEV)
+    with pytest.raises(ValueError):  # importing a layer without bias_k / bias_v into one that has them
+        ParallelMultiheadAttention(32, 4, 2, 0, add_bias_kv=True, MultiheadAttention_layer=nn.MultiheadAttention(32, 4),
+                                   device=DEV)
 
 
 @pytest.mark.parametrize("ws", [1, 2, 4])
