@@ -350,6 +350,20 @@ int rtp_embedding_scatter_add_scaled(void* stream, int dtype, const void* grad_o
                                      int scale_by_freq, int zero_fill, int64_t groups, int64_t grad_out_sg,
                                      int64_t grad_table_sg, float grad_scale);
 
+/* rtp_embedding_scatter_add_scaled with the optimiser's update applied where a row's gradient is produced
+ * (reference: the embedding's share of `clip_grad_value_` + `optimizer.step()`, benchmarks/rtp_benchmark.py:185-186,
+ * for plain SGD): every table row some token names gets w = master - lr * clamp(T(sum), +-clip) (clip == 0: no
+ * clamp), the arithmetic of rtp_sgd_step on the gradient as its table would hold it; `weights` (may be NULL) receives
+ * the row in `dtype`.  master is fp32, laid out like grad_table (same leading dimension and group stride).  Rows no
+ * token names have a zero gradient, which the update leaves unchanged: they are not touched, and with
+ * store_grad == 0 the dense gradient table is neither filled nor written.  The caller guarantees one backward pass
+ * per update (the sum is the row's whole gradient). */
+int rtp_embedding_scatter_add_sgd(void* stream, int dtype, const void* grad_out, int64_t ld_grad_out, int64_t n_ids,
+                                  const void* workspace, void* grad_table, int64_t ld_grad_table, int64_t row_begin,
+                                  int64_t row_count, int64_t cols, int64_t padding_idx, int scale_by_freq,
+                                  int64_t groups, int64_t grad_out_sg, int64_t grad_table_sg, float grad_scale,
+                                  float* master, void* weights, float lr, float clip, int store_grad);
+
 /* ---------------------------------------------------------------------------------------------
  * Attention softmax (reference: rtp/module/functional.py:779-792 baddbmm+softmax, :825
  * scaled_dot_product_attention with an additive float mask).

@@ -84,6 +84,20 @@ __device__ __forceinline__ float4 nt_load(const float4* p) {
   const nt_f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const nt_f32x4*>(p));
   return make_float4(v.x, v.y, v.z, v.w);
 }
+
+// Clip + SGD on one element: g is the gradient as the output dtype holds it.  Two roundings (product, then
+// difference), no fused multiply-add: the arithmetic of sgd_kernel in optim.hip.
+template <typename T>
+__device__ __forceinline__ float sgd_update(float w, float v, float lr, float clip) {
+  float g = to_f32(from_f32<T>(v));
+  if (clip > 0.0f) g = fminf(fmaxf(g, -clip), clip);
+  {
+#pragma clang fp contract(off)
+    const float step = lr * g;
+    return w - step;
+  }
+}
+
 __device__ __forceinline__ void nt_store(float4 a, float4* p) {
   const nt_f32x4 v = {a.x, a.y, a.z, a.w};
   __builtin_nontemporal_store(v, reinterpret_cast<nt_f32x4*>(p));

@@ -120,9 +120,12 @@ template <typename T, typename G>
 __global__ __launch_bounds__(256) void scatter_kernel(const T* grad_out, long ld_go, long n, const int* keys,
                                                       const int* vals, G* grad_table, long ld_gt, long row_begin,
                                                       long row_count, long cols, long padding_idx, int scale_by_freq,
-                                                      int overwrite, long go_sg, long gt_sg, float grad_scale) {
+                                                      int overwrite, long go_sg, long gt_sg, float grad_scale,
+                                                      float* master, T* weights, float lr, float clip, int store_grad) {
   grad_out += blockIdx.z * go_sg;  // group = shard: its column block of the upstream gradient, its own table
   grad_table += blockIdx.z * gt_sg;
+  if (master != nullptr) master += blockIdx.z * gt_sg;
+  if (weights != nullptr) weights += blockIdx.z * gt_sg;
   const long i = blockIdx.x;
   const int id = keys[i];
   if (i > 0 && keys[i - 1] == id) return;
@@ -145,6 +148,16 @@ __global__ __launch_bounds__(256) void scatter_kernel(const T* grad_out, long ld
     }
     if (scale_by_freq) acc *= inv;
     G* dst = grad_table + row * ld_gt + c;
+    if (master != nullptr) {
+      // clip + SGD applied where the row's gradient is produced (the caller guarantees that this is the row's whole
+      // gradient of the step): the arithmetic of the separate update on the gradient as its table would hold it.
+      // Rows no token names keep a zero gradient, which the update leaves alone, so they are not touched at all.
+      const float w = sgd_update<G>(master[row * ld_gt + c], acc, lr, clip);
+      master[row * ld_gt + c] = w;
+      if (weights != nullptr) weights[row * ld_gt + c] = from_f32<T>(w);
+      if (store_grad) *dst = from_f32<G>(acc);
+      continue;
+    }
     if (!overwrite) acc = to_f32(*dst) + acc;
     *dst = from_f32<G>(acc);
   }
@@ -266,8 +279,16 @@ extern "C" int rtp_embedding_sort_ids(void* stream, const int64_t* ids, int64_t 
 static int scatter_impl(void* stream, int dtype, const void* grad_out, int64_t ld_grad_out, int64_t n_ids,
                         const void* workspace, void* grad_table, int64_t ld_grad_table, int grad_table_f32,
                         int64_t row_begin, int64_t row_count, int64_t cols, int64_t padding_idx, int scale_by_freq,
-                        int zero_fill, int64_t groups, int64_t grad_out_sg, int64_t grad_table_sg, float grad_scale) {
+                        int zero_fill, int64_t groups, int64_t grad_out_sg, int64_t grad_table_sg, float grad_scale,
+                        float* master = nullptr, void* weights = nullptr, float lr = 0.0f, float clip = 0.0f,
+                        int store_grad = 1) {
   RTP_REQUIRE(grad_out && workspace && grad_table, "rtp_embedding_scatter_add_det: null pointer");
+  if (master != nullptr) {
+    // the fused update replaces the dense gradient: nothing to fill unless the gradient is wanted as well
+    RTP_REQUIRE(!grad_table_f32 || dtype == RTP_F32, "rtp_embedding_scatter_add_sgd: the gradient table has the table's dtype");
+    RTP_REQUIRE(zero_fill || !store_grad, "rtp_embedding_scatter_add_sgd: a stored gradient starts from a zero fill");
+    if (!store_grad) zero_fill = 0;
+  }
   RTP_REQUIRE(groups >= 1 && groups < 65536, "rtp_embedding_scatter_add_det: groups %lld not in 1..65535",
               (long long)groups);
   RTP_REQUIRE(dtype == RTP_F32 || dtype == RTP_BF16, "rtp_embedding_scatter_add_det: unknown dtype %d", dtype);
@@ -306,7 +327,7 @@ static int scatter_impl(void* stream, int dtype, const void* grad_out, int64_t l
   hipLaunchKernelGGL((scatter_kernel<T, G>), grid, dim3(256), 0, s, (const T*)grad_out, (long)ld_grad_out,         \
                      (long)n_ids, keys, vals, (G*)grad_table, (long)ld_grad_table, (long)row_begin, (long)row_count, \
                      (long)cols, (long)padding_idx, scale_by_freq, overwrite, (long)grad_out_sg, (long)grad_table_sg,  \
-                     grad_scale)
+                     grad_scale, master, (T*)weights, lr, clip, store_grad)
   // algorithmic bytes: read every upstream row once, write (or read-modify-write) every touched row once
   ProfileScope prof(s, "embedding_scatter_add", (double)groups * n_ids * cols,
                     (double)groups * n_ids * cols * ((dtype == RTP_F32 ? 4.0 : 2.0) + (zero_fill ? 1.0 : 2.0) * gsz) + 8.0 * n_ids);
@@ -341,4 +362,18 @@ extern "C" int rtp_embedding_scatter_add_scaled(void* stream, int dtype, const v
   return scatter_impl(stream, dtype, grad_out, ld_grad_out, n_ids, workspace, grad_table, ld_grad_table, grad_table_f32,
                       row_begin, row_count, cols, padding_idx, scale_by_freq, zero_fill, groups, grad_out_sg,
                       grad_table_sg, grad_scale);
+}
+
+extern "C" int rtp_embedding_scatter_add_sgd(void* stream, int dtype, const void* grad_out, int64_t ld_grad_out,
+                                             int64_t n_ids, const void* workspace, void* grad_table,
+                                             int64_t ld_grad_table, int64_t row_begin, int64_t row_count, int64_t cols,
+                                             int64_t padding_idx, int scale_by_freq, int64_t groups,
+                                             int64_t grad_out_sg, int64_t grad_table_sg, float grad_scale,
+                                             float* master, void* weights, float lr, float clip, int store_grad) {
+  RTP_REQUIRE(master != nullptr, "rtp_embedding_scatter_add_sgd: null master");
+  RTP_REQUIRE(dtype == RTP_F32 ? weights == nullptr || weights == (void*)master : true,
+              "rtp_embedding_scatter_add_sgd: fp32 tables are their own master");
+  return scatter_impl(stream, dtype, grad_out, ld_grad_out, n_ids, workspace, grad_table, ld_grad_table, 0, row_begin,
+                      row_count, cols, padding_idx, scale_by_freq, store_grad ? 1 : 0, groups, grad_out_sg,
+                      grad_table_sg, grad_scale, master, dtype == RTP_F32 ? nullptr : weights, lr, clip, store_grad);
 }

@@ -468,19 +468,6 @@ __device__ __forceinline__ void store8(T* dst, const float (&v)[8], bool stream)
   }
 }
 
-// Clip + SGD on one element: g is the gradient as the output dtype holds it.  Two roundings (product, then
-// difference), no fused multiply-add: the arithmetic of sgd_kernel in optim.hip.
-template <typename T>
-__device__ __forceinline__ float sgd_update(float w, float v, float lr, float clip) {
-  float g = to_f32(from_f32<T>(v));
-  if (clip > 0.0f) g = fminf(fmaxf(g, -clip), clip);
-  {
-#pragma clang fp contract(off)
-    const float step = lr * g;
-    return w - step;
-  }
-}
-
 template <typename T, int BM, int BN, int NTHR>
 __device__ __forceinline__ void finish_tile(const GemmArgs& p, const float* ct, int m0, int n0, int tid, int grp,
                                             long zo, long zi) {

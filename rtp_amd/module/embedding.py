@@ -17,6 +17,7 @@ import torch.nn.init as init
 from .. import ops
 from ..ring import Rotation, ring_order
 from .collectives import RotatedLayer
+from .shard_ops import _fused, _fused_done
 from .utils import affine_weight, divide_and_check_no_remainder
 
 
@@ -78,10 +79,14 @@ class _EmbeddingFn(torch.autograd.Function):
         # runs of consecutive shards with the same overwrite / accumulate state go out as one grouped launch
         for first, cnt, accumulate in store._grad_runs(ring_order(layer.rank, ws, reverse=True)):
             table = store.grads[first, :store.numels[0]].view(store.shapes[0])
+            # an optimiser that applies its update where gradients are produced: the rows the step's tokens name are
+            # updated by the scatter-add itself, the dense [V, D/ws] gradient is neither zero-filled nor written
+            kw = _fused(store, accumulate, first, cnt, store.offsets[0], store.numels[0])
             ops.embedding_scatter_add(g2[:, first * d_s:(first + 1) * d_s], flat_ids.numel(), workspace, table,
                                       padding_idx=pad, scale_by_freq=layer.scale_grad_by_freq,
                                       zero_fill=not accumulate, groups=cnt, grad_out_sg=d_s,
-                                      grad_table_sg=store.grads.shape[1], grad_scale=ctx.grad_scale)
+                                      grad_table_sg=store.grads.shape[1], grad_scale=ctx.grad_scale, **kw)
+            _fused_done(store, kw)
         store.grads_ready()
         return None, None, None, None, None
 

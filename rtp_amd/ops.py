@@ -367,11 +367,16 @@ def embedding_sort_ids(ids: torch.Tensor) -> torch.Tensor:
 def embedding_scatter_add(grad_out: torch.Tensor, n_ids: int, workspace: torch.Tensor, grad_table: torch.Tensor,
                           *, row_begin: int = 0, padding_idx: int = -1, scale_by_freq: bool = False,
                           zero_fill: bool = True, groups: int = 1, grad_out_sg: int = 0,
-                          grad_table_sg: int = 0, grad_scale: float = 1.0) -> None:
+                          grad_table_sg: int = 0, grad_scale: float = 1.0, sgd: Optional["FusedSgd"] = None,
+                          sgd_master: int = 0, sgd_weights: int = 0) -> None:
     """grad_table[id] (+)= sum of the grad_out rows whose token is id, in ascending position order.  With
     groups > 1, group g reads grad_out + g*grad_out_sg and writes grad_table + g*grad_table_sg (elements):
     all shards of an embedding in one launch.  grad_scale != 1 sums grad_out * grad_scale, each product rounded
-    to grad_out's dtype first (the gradient a scaled embedding receives)."""
+    to grad_out's dtype first (the gradient a scaled embedding receives).
+
+    `sgd` (with the addresses of the fp32 table and of its compute-dtype copy that match grad_table): the rows some
+    token names are updated by clip + SGD right here, the others are left alone (their gradient is zero), and the
+    dense gradient is only filled and written when sgd.keep_grads."""
     for t in (grad_out, workspace, grad_table):
         _dev(t)
     n, cols, ld_go = _mat(grad_out, "grad_out")
@@ -385,6 +390,16 @@ def embedding_scatter_add(grad_out: torch.Tensor, n_ids: int, workspace: torch.T
             grad_table.data_ptr(), ld_gt, int(grad_table.dtype == torch.float32), row_begin, rows, cols,
             -1 if padding_idx is None else padding_idx, int(scale_by_freq), int(zero_fill), groups, grad_out_sg,
             grad_table_sg)
+    if sgd is not None:
+        if not zero_fill or grad_table.dtype != grad_out.dtype:
+            raise ValueError("embedding_scatter_add: the fused update takes the whole gradient of the step, in the "
+                             "table's own dtype")
+        check(_lib.load().rtp_embedding_scatter_add_sgd(
+            _stream(), dtype_code(grad_out.dtype), grad_out.data_ptr(), ld_go, n_ids, workspace.data_ptr(),
+            grad_table.data_ptr(), ld_gt, row_begin, rows, cols, -1 if padding_idx is None else padding_idx,
+            int(scale_by_freq), groups, grad_out_sg, grad_table_sg, float(grad_scale), sgd_master, sgd_weights or None,
+            sgd.lr, sgd.clip, int(sgd.keep_grads)))
+        return
     if grad_scale != 1.0:
         check(_lib.load().rtp_embedding_scatter_add_scaled(*args, float(grad_scale)))
     else:

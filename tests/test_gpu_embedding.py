@@ -133,3 +133,36 @@ def test_sorted_token_ids_are_the_stable_sort_by_id(n, vocab):
     vals = ws[3 * arr:3 * arr + 4 * n].view(torch.int32).cpu()
     order = torch.sort(ids, stable=True).indices
     assert torch.equal(keys.long(), ids[order]) and torch.equal(vals.long(), order)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embedding_update_applied_by_the_scatter_add_is_bit_identical(dtype):
+    """RotatedSGD(fused_backward=True): the rows the step's tokens name are updated by the scatter-add itself and the
+    others left alone; weights after two steps equal those of the separate gradient + update launches bit for bit,
+    with a padding row, repeated ids and gradient scaling by frequency."""
+    from rtp_amd.module.embedding import ParallelEmbedding
+    from rtp_amd.optim import RotatedSGD
+    V, D, ws = 300, 64, 4
+    gen = torch.Generator().manual_seed(23)
+    master = torch.nn.Embedding(V, D, padding_idx=7, scale_grad_by_freq=True)
+    with torch.no_grad():
+        master.weight.copy_((torch.randn(V, D, generator=gen) * 0.5).to(dtype).float())
+    twins = []
+    for fused in (False, True):
+        emb = ParallelEmbedding(V, D, ws, 0, padding_idx=7, scale_grad_by_freq=True, Embedding_layer=master,
+                                device=DEV, dtype=dtype)
+        twins.append((emb, RotatedSGD(emb, lr=0.1, clip_value=0.05, fused_backward=fused)))
+    for step in range(2):
+        ids = torch.randint(0, V, (9, 5), generator=gen)
+        ids[0, :3] = 7          # padding rows
+        ids[1:4, 0] = 11        # a repeated id
+        coef = torch.randn(9, 5, D, generator=gen).to(dtype).to(DEV)
+        for emb, opt in twins:
+            opt.zero_grad()
+            (emb(ids.to(DEV)) * coef).sum().backward()
+            opt.step()
+        torch.cuda.synchronize()
+        for (a, _), (b, _) in zip(*[[(p, None) for p in t[0].parameters()] for t in twins]):
+            assert torch.equal(a, b), f"step {step}"
+    # the fused twin never filled or wrote its dense gradient table
+    assert twins[1][0]._store.fused_sgd is not None
