@@ -512,11 +512,20 @@ __device__ __forceinline__ void finish_tile(const GemmArgs& p, const float* ct, 
         for (int e = 0; e < 8; ++e) v[e] += t[e];
       }
       if (bias) {
+        // The per-segment biases of a row-parallel layer sit in eight different home rows, far from any cache: the
+        // loads of eight segments are issued together (segments past the last re-read segment 0 and count as zero)
+        // and then added in segment order -- one trip to memory instead of one per segment.
         float bv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        for (int sgm = 0; sgm < nb_seg; ++sgm) {
-          load8(bias + sgm * p.bias_sk + col, t);
+        for (int s0 = 0; s0 < nb_seg; s0 += 8) {
+          float bt[8][8];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) bv[e] += t[e];
+          for (int j = 0; j < 8; ++j) load8(bias + (s0 + j < nb_seg ? s0 + j : 0) * p.bias_sk + col, bt[j]);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const float on = s0 + j < nb_seg ? 1.0f : 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) bv[e] += on * bt[j][e];
+          }
         }
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] += bv[e];
@@ -1069,6 +1078,39 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
       }(std::make_integer_sequence<int, NSTAGE>{});
     };
     warm_ahead(p, (unsigned)(uintptr_t)(lptr_t)lds + NSTAGE * STAGE, id, gridDim.x * gridDim.y, wave, lane);
+    if (p.bias != nullptr && wave == 0) {
+      // the epilogue's bias values (one vector per K segment of a row-parallel layer, each in another home row) are
+      // requested now and sit in the L2 when the epilogue asks for them
+      const int nb = p.bias_sk ? p.ksegs : 1;
+      const T* bs = reinterpret_cast<const T*>(p.bias) + grp * p.bias_sg + zo * p.bias_so + zi * p.bias_si + n0;
+      constexpr int LPS = (BN * (int)sizeof(T) + 63) / 64;  // lanes per segment: one per 64 bytes of the tile's columns
+      const int sgm = lane / LPS, part = lane % LPS;
+      if (sgm < nb && n0 + part * (64 / (int)sizeof(T)) + 4 / (int)sizeof(T) <= p.n) {  // the 4 bytes read lie inside the vector
+        const char* src = reinterpret_cast<const char*>(bs + (long)sgm * p.bias_sk) + part * 64;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
+                     :
+                     : "s"((unsigned)(uintptr_t)(lptr_t)lds + NSTAGE * STAGE), "v"(src)
+                     : "memory");
+      }
+    }
+    if (p.gate != nullptr && p.vec_c) {
+      // the ReLU mask of the epilogue is an activation saved by the forward pass, long gone from the caches: the
+      // tile's part of it is requested now, 16 bytes per lane
+      constexpr int CPR = BN * (int)sizeof(T) / 16, NCH = BM * CPR;  // 16-byte chunks per tile row, per tile
+      const T* gt = reinterpret_cast<const T*>(p.gate) + grp * p.gate_sg + zo * p.gate_so + zi * p.gate_si;
+#pragma unroll
+      for (int c0 = 0; c0 < NCH; c0 += 256) {
+        const int c = c0 + wave * 64 + lane;
+        const int row = m0 + c / CPR, col = n0 + (c % CPR) * (16 / (int)sizeof(T));
+        if (c < NCH && row < p.m && col + 16 / (int)sizeof(T) <= p.n) {
+          const char* src = reinterpret_cast<const char*>(gt + (long)row * p.ld_gate + col);
+          asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                       :
+                       : "s"((unsigned)(uintptr_t)(lptr_t)lds + NSTAGE * STAGE), "v"(src)
+                       : "memory");
+        }
+      }
+    }
     __builtin_amdgcn_s_barrier();  // barrier 0
     [&]<int... Q>(std::integer_sequence<int, Q...>) {
       (read_step(std::integral_constant<int, 0>{}, std::integral_constant<int, Q>{}, std::integral_constant<int, Q>{}),
