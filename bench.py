@@ -30,16 +30,16 @@ PEAK = {"bf16_mfma_tflops": 2500.0, "fp32_mfma_tflops": 157.3, "hbm_gbs": 8000.0
 # The weight-gradient variant (128x128 rc_rc) carries the clip + SGD update: its figure includes the fp32 parameters
 # read and written and their bf16 copy written.
 MEASURED_TRAFFIC_KIB = {
-    "gemm_bf16_128x128_rc_rc": 106570.1, "gemm_bf16_128x64_kc_rc": 69584.4, "gemm_bf16_128x64_kc_kc": 46835.8,
-    "gemm_bf16_128x192_kc_kc": 106247.3,
+    "gemm_bf16_128x128_rc_rc": 106735.7, "gemm_bf16_128x64_kc_rc": 70131.4, "gemm_bf16_128x64_kc_kc": 46918.2,
+    "gemm_bf16_128x192_kc_kc": 106270.0,
 }
 
 
 # rocprofv3's average duration of a dispatch over the kernel's own execution span (first wave's start to last wave's
 # end, printed by this script as roofline.execution_span), both from the one rocprofv3 run of the default command
-# whose summary is profiles/lm_step_kernel_trace.txt: 44.112 us / 35.188 us for the weight-gradient product,
-# 35.847 / 29.544 for the input-gradient product.
-DISPATCH_OVER_EXECUTION_SPAN = {"gemm_bf16_128x128_rc_rc": 44.112 / 35.188, "gemm_bf16_128x64_kc_rc": 35.847 / 29.544}
+# whose summary is profiles/lm_step_kernel_trace.txt: 44.067 us / 35.301 us for the weight-gradient product,
+# 36.246 / 30.426 for the input-gradient product.
+DISPATCH_OVER_EXECUTION_SPAN = {"gemm_bf16_128x128_rc_rc": 44.067 / 35.301, "gemm_bf16_128x64_kc_rc": 36.246 / 30.426}
 
 
 def step_flops(c):
