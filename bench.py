@@ -367,7 +367,7 @@ def layer_workload(name, steps, warmup, graph=True, cpu=True):
     # Every pass starts like a training step, after zero_grad: the rotated gradients are overwritten, not added to
     # (what RotatedSGD.zero_grad arranges), and the input's gradient is a fresh tensor.
     stores = [m._store for m in layer.modules() if isinstance(getattr(m, "_store", None), ShardStore)]
-    inputs = [t for t in (locals().get("x"),) if torch.is_tensor(t) and t.requires_grad]
+    inputs = [] if name == "embedding" else [x]  # the embedding's input is token ids
     body = fn
 
     def fn():
