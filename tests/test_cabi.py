@@ -64,12 +64,13 @@ def test_ops_refuse_cpu_tensors():
 
 
 def test_integration_stub_struct_matches_the_library():
-    """The ctypes GemmDesc a maintainer would paste from INTEGRATION.md has the layout of rtp_gemm_desc: same size as
-    the library reports and the same field names, order and offsets as the package's own binding."""
+    """The ctypes GemmDesc that the integration notes at the repository root print for a maintainer to paste has the
+    layout of rtp_gemm_desc: same size as the library reports and the same field names, order and offsets as the
+    package's own binding."""
     from rtp_amd import _lib
     text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
     m = re.search(r"^class GemmDesc\(C\.Structure\):.*?(?=^assert _lib\.rtp_gemm_desc_size)", text, flags=re.S | re.M)
-    assert m, "INTEGRATION.md no longer holds the GemmDesc stub"
+    assert m, "the integration notes no longer hold the GemmDesc stub"
     scope = {"C": ctypes}
     exec(m.group(0), scope)
     stub = scope["GemmDesc"]
