@@ -1662,7 +1662,7 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
     const char* e = getenv("RTP_GEMM_TILE");  // debugging aid: index into kShapes
     return e ? atoi(e) : -1;
   }();
-  static const double slab_ns[kNumShapes] = {966.0, 470.0, 283.0, 167.0, 720.0, 840.0};
+  static const double slab_ns[kNumShapes] = {966.0, 470.0, 283.0, 167.0, 800.0, 840.0};
   static const int slab_bytes[kNumShapes] = {128, 128, 128, 128, 128, 64};
   int shape = 3;  // 64 x 64 unless the model finds something cheaper
   double best = 0.0;
