@@ -30,16 +30,16 @@ PEAK = {"bf16_mfma_tflops": 2500.0, "fp32_mfma_tflops": 157.3, "hbm_gbs": 8000.0
 # The weight-gradient variant (128x128 rc_rc) carries the clip + SGD update: its figure includes the fp32 parameters
 # read and written and their bf16 copy written.
 MEASURED_TRAFFIC_KIB = {
-    "gemm_bf16_128x128_rc_rc": 106735.7, "gemm_bf16_128x64_kc_rc": 70131.4, "gemm_bf16_128x64_kc_kc": 46918.2,
-    "gemm_bf16_128x192_kc_kc": 106270.0,
+    "gemm_bf16_128x128_rc_rc": 106667.6, "gemm_bf16_128x64_kc_rc": 70132.1, "gemm_bf16_128x64_kc_kc": 46918.7,
+    "gemm_bf16_128x192_kc_kc": 74478.8, "gemm_bf16_128x128_kc_kc": 169491.2,
 }
 
 
 # rocprofv3's average duration of a dispatch over the kernel's own execution span (first wave's start to last wave's
 # end, printed by this script as roofline.execution_span), both from the one rocprofv3 run of the default command
-# whose summary is profiles/lm_step_kernel_trace.txt: 44.067 us / 35.301 us for the weight-gradient product,
-# 36.246 / 30.426 for the input-gradient product.
-DISPATCH_OVER_EXECUTION_SPAN = {"gemm_bf16_128x128_rc_rc": 44.067 / 35.301, "gemm_bf16_128x64_kc_rc": 36.246 / 30.426}
+# whose summary is profiles/lm_step_kernel_trace.txt: 44.002 us / 34.914 us for the weight-gradient product,
+# 36.490 / 30.317 for the input-gradient product.  Between runs and boxes the ratio moves by about +-3 %.
+DISPATCH_OVER_EXECUTION_SPAN = {"gemm_bf16_128x128_rc_rc": 44.002 / 34.914, "gemm_bf16_128x64_kc_rc": 36.490 / 30.317}
 
 
 def step_flops(c):
@@ -616,7 +616,22 @@ def main():
     ratio = DISPATCH_OVER_EXECUTION_SPAN.get(dom_name, 1.0) if graph_stats is not None else 1.0
     avg_ms = span_us * ratio * 1e-3
     achieved = dom["flops"] / dom["launches"] / (avg_ms * 1e-3) / 1e12
-    span = {"avg_launch_us": span_us, "frac": dom["flops"] / dom["launches"] / (span_us * 1e-6) / 1e12 / PEAK["bf16_mfma_tflops"],
+    # Which roof bounds the kernel: the larger of its two minimum times, flops at the MFMA peak or algorithmic bytes
+    # at the HBM peak.  A weight-gradient product that carries the optimiser's update moves 10 bytes per output
+    # element on top of its operands, against 2 * K flops with K = the step's 1024 tokens: ~125 flop per byte, below
+    # the machine's 312, so its roof is the memory system's; the other products are bound by the matrix pipes.
+    alg_bytes = dom["bytes"] / dom["launches"]
+    mfma_frac = achieved / PEAK["bf16_mfma_tflops"]
+    hbm_gbs = alg_bytes / (avg_ms * 1e-3) / 1e9
+    hbm_frac = hbm_gbs / PEAK["hbm_gbs"]
+    if hbm_frac > mfma_frac:
+        roof = {"bound": "hbm", "achieved": hbm_gbs, "peak": PEAK["hbm_gbs"], "unit": "GB/s", "frac": hbm_frac,
+                "mfma_view": {"achieved": achieved, "peak": PEAK["bf16_mfma_tflops"], "unit": "TFLOP/s", "frac": mfma_frac}}
+    else:
+        roof = {"bound": "mfma", "achieved": achieved, "peak": PEAK["bf16_mfma_tflops"], "unit": "TFLOP/s",
+                "frac": mfma_frac,
+                "hbm_view": {"achieved": hbm_gbs, "peak": PEAK["hbm_gbs"], "unit": "GB/s", "frac": hbm_frac}}
+    span = {"avg_launch_us": span_us, "frac": (hbm_frac if hbm_frac > mfma_frac else mfma_frac) * avg_ms * 1e3 / span_us,
             "what": "first wave's start to last wave's end of the kernel (device time stamps in the replayed HIP graph; HIP "
                     "events in eager mode): its own execution, without the wait for CUs that a dispatch span includes",
             "instrumented_replay_ms_per_step": instr_ms}
@@ -647,11 +662,11 @@ def main():
                    "logits_and_loss_fused": bool(args.fused_head_loss),
                    "wgrad_on_second_stream": bool(args.wgrad_overlap),
                    "next_layer_shards_read_ahead_into_cache": bool(ring.warm_ahead())},
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK["bf16_mfma_tflops"], "unit": "TFLOP/s",
-                     "frac": achieved / PEAK["bf16_mfma_tflops"],
-                     "traffic": (MEASURED_TRAFFIC_KIB[dom_name] * 1024.0 if dom_name in MEASURED_TRAFFIC_KIB else None),
+        "roofline": dict(roof,
+                     traffic=(MEASURED_TRAFFIC_KIB[dom_name] * 1024.0 if dom_name in MEASURED_TRAFFIC_KIB else None),
+                     **{
                      "traffic_unit": "bytes per launch (counter runs, see profiles/)",
-                     "algorithmic_bytes_per_launch": dom["bytes"] / dom["launches"], "kernel": dom_name,
+                     "algorithmic_bytes_per_launch": alg_bytes, "kernel": dom_name,
                      "avg_launch_us": avg_ms * 1e3,
                      "launches_per_step": dom["launches"] // (5 if graph_stats is not None else prof_steps),
                      "flops_per_launch": dom["flops"] / dom["launches"],
@@ -660,7 +675,7 @@ def main():
                                   if graph_stats is not None else "eager launches, HIP events"),
                      "dispatch_over_execution_span": ratio,
                      "execution_span": span,
-                     "eager_ms_per_step_with_event_pairs": eager_ms},
+                     "eager_ms_per_step_with_event_pairs": eager_ms}),
         "gemm_kernels_in_graph_replay": graph_gemms,
         "measured_attainable": dict(peaks, dominant_kernel_frac_of_measured_gemm=achieved / peaks["gemm_bf16_4096_cubed_tflops"]),
         "step_mfma_frac": flops / dt / (PEAK["bf16_mfma_tflops"] * 1e12),
