@@ -9,6 +9,7 @@ import torch
 import torch.nn as nn
 
 from .. import ops
+from .. import ring as _ring
 
 
 class _DeferredParamGrads:
@@ -58,6 +59,8 @@ class _DeferredParamGrads:
 
 
 _deferred = _DeferredParamGrads()
+# reduce before the compute stream waits for the weight-gradient stream at the end of the pass, not after
+_ring.run_before_join(_deferred.flush)
 _DEFER = os.environ.get("RTP_LN_DEFER", "1") != "0"  # 0: reduce each LayerNorm's parameter gradients in its own backward
 
 

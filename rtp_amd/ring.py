@@ -136,10 +136,24 @@ def wgrad_overlap() -> bool:
     return _wgrad_overlap
 
 
+# Work of the compute stream that is due at the end of a backward pass and does not depend on the second stream (the
+# one-launch reduction of the LayerNorm parameter gradients): launched before the compute stream starts waiting for
+# the second stream, it runs beside the last weight-gradient products instead of after them.
+_before_join: List = []
+
+
+def run_before_join(fn) -> None:
+    """Register fn(device index), called at the start of every join_wgrad."""
+    if fn not in _before_join:
+        _before_join.append(fn)
+
+
 def join_wgrad(device: Optional[torch.device] = None) -> None:
     """Launch what is still deferred and make the current stream wait for the parameter-gradient work on the
     second stream."""
     idx = torch.cuda.current_device() if device is None or device.index is None else device.index
+    for fn in _before_join:
+        fn(idx)
     _flush_wgrad(idx)
     _wgrad_task.pop(idx, None)
     if _wgrad_dirty.get(idx):
