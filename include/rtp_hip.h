@@ -285,7 +285,8 @@ int rtp_ring_release(void* ring, void* main_stream, int slot);
  * memory-side cache when the products that use them start: the one-GPU form of "the next shard arrives while the
  * current one computes" (reference: the isend/irecv of the next shard that overlaps the current step's compute,
  * rtp/module/collectives.py:240-317, rtp/module/linear.py:211-220) when the shards are read from their home rows
- * and nothing is copied.  A hint: no result depends on it.  flags bit 0: non-temporal loads. */
+ * and nothing is copied.  A hint: no result depends on it.  flags bit 0: non-temporal loads (measured: those do not
+ * leave the lines in the memory-side cache, so the products that follow gain nothing; kept for such measurements). */
 int rtp_cache_warm(void* stream, const void* src, size_t bytes, int flags);
 
 /* The copy kernel on its own (16-byte vectorised, grid-stride): dst/src 16-byte aligned or any
