@@ -22,23 +22,26 @@ class _DeferredParamGrads:
 
     def __init__(self):
         self.pending = {}   # device index -> [(part, rows, cols, dgamma, dbeta, weight)]
-        self.armed = set()  # device indices with a callback queued in the running backward pass
+        self.armed = {}     # device index -> id of the backward pass that has a callback queued
         self.tables = {}    # (device index, dtype, buffer addresses and shapes) -> (table, max_cols)
 
     def add(self, device: torch.device, item) -> bool:
         idx = device.index if device.index is not None else torch.cuda.current_device()
-        if idx not in self.armed:
-            try:
-                torch.autograd.Variable._execution_engine.queue_callback(lambda: self.flush(idx))
-            except RuntimeError:
-                return False  # not inside a backward pass: the caller reduces at once
-            self.armed.add(idx)
+        task = torch._C._current_graph_task_id()
+        if task < 0:
+            return False  # not inside a backward pass: the caller reduces at once
+        if self.armed.get(idx) != task:
+            # leftovers of a pass that raised before its callback ran: its partial sums are dropped with it
+            for it in self.pending.pop(idx, []):
+                it[5]._rtp_ln_pending = False
+            torch.autograd.Variable._execution_engine.queue_callback(lambda: self.flush(idx))
+            self.armed[idx] = task
         self.pending.setdefault(idx, []).append(item)
         item[5]._rtp_ln_pending = True
         return True
 
     def flush(self, idx: int) -> None:
-        self.armed.discard(idx)
+        self.armed.pop(idx, None)
         items = self.pending.pop(idx, [])
         if not items:
             return

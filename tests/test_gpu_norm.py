@@ -99,3 +99,51 @@ def test_layer_norm_parameter_gradients_reduced_at_the_end_of_backward():
         ref(x, False).backward(g)
         for (k, p), q in zip(net.named_parameters(), ref.parameters()):
             assert_close(p.grad, q.grad, torch.float32, f"step {step} {k}")
+
+
+def test_backward_that_raises_leaves_no_partial_layer_norm_sums_behind():
+    """A backward pass that raises after a LayerNorm has left its partial sums never runs the end-of-pass reduction.
+    The next pass must queue its own reduction and must not reduce the dead pass's partial sums."""
+    import torch.nn as nn
+    from rtp_amd.module import norm as norm_mod
+    from rtp_amd.module.norm import add_layer_norm
+    from rtp_amd.optim import RotatedSGD
+
+    class Boom(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, x):
+            return x.clone()
+
+        @staticmethod
+        def backward(ctx, g):
+            raise ValueError("boom")
+
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.n1, self.n2 = nn.LayerNorm(64), nn.LayerNorm(64)
+
+        def forward(self, x, fused, boom=False):
+            f = (lambda a, b, n: add_layer_norm(a, b, n)) if fused else (lambda a, b, n: n(a + b))
+            h = f(x, x * 0.5, self.n1)
+            if boom:
+                h = Boom.apply(h)
+            return f(h, x, self.n2)
+
+    torch.manual_seed(1)
+    ref = Net()
+    net = Net().to(DEV)
+    net.load_state_dict(ref.state_dict())
+    opt = RotatedSGD(net, lr=0.0)
+    x = torch.randn(24, 64)
+    opt.zero_grad()
+    with pytest.raises(ValueError, match="boom"):
+        net(x.to(DEV), True, boom=True).sum().backward()     # n2 has left partial sums; the pass dies before n1
+    x, g = torch.randn(24, 64), torch.randn(24, 64)
+    opt.zero_grad()
+    net(x.to(DEV), True).backward(g.to(DEV))
+    ref(x, False).backward(g)
+    torch.cuda.synchronize()
+    assert not norm_mod._deferred.pending.get(0) and 0 not in norm_mod._deferred.armed
+    for (k, p), q in zip(net.named_parameters(), ref.parameters()):
+        assert_close(p.grad, q.grad, torch.float32, k)
