@@ -1164,9 +1164,15 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
 // (1/BM + 1/BN) bytes per flop: a 256 x 256 tile moves two thirds of what 256 x 128 moves.  Its 256 KiB of fp32
 // accumulators need all eight waves of the workgroup as MFMA waves (2 x 4 wave tiles of 128 x 64, 128 accumulator
 // registers each), so here the waves issue the direct-to-LDS loads themselves, each an eighth of a slab, right
-// after the barrier that frees a stage; the slab is 64 bytes of k per row (32 KiB per stage, 5 stages).  Same
-// barrier protocol as above with both roles in one wave: before barrier k+1 a wave waits for its own loads of slab
-// k+1, after it the wave refills the stage of slab k-1.  The epilogue goes through LDS in four passes of 64 rows.
+// after the barrier that frees a stage.  Both roles in one wave allow a tighter stage protocol than above: every
+// read of slab k's fragments is issued before the first read of slab k+1, and the barrier of slab k+1 sits in front
+// of that read -- so once a wave has seen its own LDS reads return (lgkmcnt 0) and has passed barrier k+1, nobody
+// reads the stage of slab k any more and slab k + NSTAGE may go there.  NSTAGE slabs are in LDS or on their way;
+// the k-step being multiplied lives in registers.  With NSTAGE = 2 this is the plain double buffer, and the two
+// stages can hold slabs of 128 bytes of k per row (2 x 64 KiB): a load instruction then fetches whole cache lines
+// of a K-contiguous operand (with 64-byte rows its operand stream alone took 1.5 x as long as that of a
+// row-contiguous operand), and a barrier comes every 4 k-steps.  The epilogue goes through LDS in four passes of
+// 64 rows.
 template <typename T, bool AKC, bool BKC, int NSTAGE, int SB, int PD>
 __global__ __launch_bounds__(512) void gemm_dma8_kernel(GemmArgs p) {
   constexpr int BM = 256, BN = 256, NL = 8;
@@ -1177,8 +1183,8 @@ __global__ __launch_bounds__(512) void gemm_dma8_kernel(GemmArgs p) {
   constexpr int WM = 128, WN = 64, MT = 4, NT = 2;
   constexpr int STAGE = DA::BYTES + DB::BYTES;
   constexpr int NI = DA::NI + DB::NI;
-  static_assert((NSTAGE - 2) * NI < 64, "vmcnt is a 6-bit counter");
-  static_assert(NSTAGE >= 3 && NSTAGE * STAGE <= 160 * 1024, "3 or more stages within 160 KiB of LDS");
+  static_assert((NSTAGE - 1) * NI < 64, "vmcnt is a 6-bit counter");
+  static_assert(NSTAGE >= 2 && NSTAGE * STAGE <= 160 * 1024, "2 or more stages within 160 KiB of LDS");
   static_assert(64 * (BN + 4) * 4 <= NSTAGE * STAGE, "an epilogue pass stages 64 rows of the fp32 tile");
   __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE];
 
@@ -1294,15 +1300,16 @@ __global__ __launch_bounds__(512) void gemm_dma8_kernel(GemmArgs p) {
     constexpr int tq = (q + PD) % KS, ds = (q + PD) / KS;
     if (steady || k + ds < nk) {
       if (ds == 1 && tq == 0) {
-        // barrier k+1: my loads of slab k+1 have landed; behind it everybody's have, and everybody has consumed
-        // the last fragments of slab k-1, whose stage takes slab k+NSTAGE-1
+        // barrier k+1: my loads of slab k+1 have landed (those of the slabs up to k+NSTAGE-1 may be on their way)
+        // and my reads of slab k have returned; behind it that holds for everybody, and the stage of slab k takes
+        // slab k+NSTAGE
         if (k + NSTAGE - 1 < nk) {
-          RTP_WAIT_VM((NSTAGE - 3) * NI);
+          RTP_WAIT_VM_LGKM0((NSTAGE - 2) * NI);
         } else {
-          RTP_WAIT_VM(0);
+          RTP_WAIT_VM_LGKM0(0);
         }
         __builtin_amdgcn_s_barrier();
-        if (k + NSTAGE - 1 < nk) issue();
+        if (k + NSTAGE < nk) issue();
         __builtin_amdgcn_sched_barrier(0);
       }
       read_step(std::integral_constant<int, (s + ds) % NSTAGE>{}, std::integral_constant<int, tq>{},
@@ -1332,11 +1339,11 @@ __global__ __launch_bounds__(512) void gemm_dma8_kernel(GemmArgs p) {
     }(std::make_integer_sequence<int, NSTAGE>{});
   };
 
-  // prologue: NSTAGE-1 slabs on their way, slab 0 landed
-  const int ahead = nk < NSTAGE - 1 ? nk : NSTAGE - 1;
+  // prologue: NSTAGE slabs on their way, slab 0 landed
+  const int ahead = nk < NSTAGE ? nk : NSTAGE;
   for (int s_ = 0; s_ < ahead; ++s_) issue();
-  if (nk >= NSTAGE - 1) {
-    RTP_WAIT_VM((NSTAGE - 2) * NI);
+  if (nk >= NSTAGE) {
+    RTP_WAIT_VM((NSTAGE - 1) * NI);
   } else {
     RTP_WAIT_VM(0);
   }
@@ -1662,8 +1669,8 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
     const char* e = getenv("RTP_GEMM_TILE");  // debugging aid: index into kShapes
     return e ? atoi(e) : -1;
   }();
-  static const double slab_ns[kNumShapes] = {966.0, 470.0, 283.0, 167.0, 800.0, 840.0};
-  static const int slab_bytes[kNumShapes] = {128, 128, 128, 128, 128, 64};
+  static const double slab_ns[kNumShapes] = {966.0, 470.0, 283.0, 167.0, 800.0, 1680.0};
+  static const int slab_bytes[kNumShapes] = {128, 128, 128, 128, 128, 128};
   int shape = 3;  // 64 x 64 unless the model finds something cheaper
   double best = 0.0;
   for (int i = 0; fast && i < kNumShapes; ++i) {
@@ -1672,7 +1679,7 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
     // layouts at 8192^3, +10 - 20 % on the expert products of the MoE layer, nothing at 4096^3, a loss where it
     // leaves CUs without a tile or K is short)
     if (i == 5 && (sizeof(T) != 2 || d->sgd_master || d->xent_mode == 1 ||
-                   ceil_div(d->m, 256) * ceil_div(d->n, 256) * nz < 256 || d->k * d->ksegs < 2048) && i != forced)
+                   ceil_div(d->m, 256) * ceil_div(d->n, 256) * nz < 256 || d->k * d->ksegs < 1024) && i != forced)
       continue;
     // never a tile that is mostly padding: a 32 x 32 problem (one attention head at seq 32) stays at 64 x 64
     if ((!akc && (kShapes[i].bm & (kShapes[i].bm - 1))) || (!bkc && (kShapes[i].bn & (kShapes[i].bn - 1)))) continue;
@@ -1779,7 +1786,7 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
     case 4:
       return launch_dma<T, 128, 192, 3, 128, 2>(s, a, akc, bkc, grid);
     case 5:
-      if constexpr (sizeof(T) == 2) return launch_dma8<T, 5, 64, 1>(s, a, akc, bkc, grid);
+      if constexpr (sizeof(T) == 2) return launch_dma8<T, 2, 128, 1>(s, a, akc, bkc, grid);
       return fail(RTP_ERR_ARG, "gemm: no 256 x 256 kernel for this dtype");
     default:
       return launch_dma<T, 64, 64, 4, 128, 3>(s, a, akc, bkc, grid);

@@ -319,6 +319,38 @@ def test_gemm_256x256_tile_path(akc, bkc):
     assert rel_err(out, ref) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("akc,bkc", [(True, True), (True, False), (False, False)])
+@pytest.mark.parametrize("k,ksegs", [(1024, 1), (1096, 1), (520, 2), (136, 8)])
+def test_gemm_256x256_tile_path_groups_segments_and_short_contractions(akc, bkc, k, ksegs):
+    """The eight-wave kernel's two-stage pipeline at its edges: a grouped launch (16 groups of 4 x 4 tiles fill the
+    256 CUs once), contraction lengths of 2 to 17 slabs with and without a ragged last slab, and a contraction cut
+    into K segments that sit apart in memory (every segment starts a new run of slabs and may end in a ragged one)."""
+    from rtp_amd import _lib
+    ops = _ops()
+    dtype = torch.bfloat16
+    gen = torch.Generator().manual_seed(91)
+    groups, m, n = 16, 1000, 1024
+    # operand of segment s, group g: a[s, g] is [m, k] (or [k, m]); the product sums over s
+    a = _rand((ksegs, groups) + ((m, k) if akc else (k, m)), dtype, gen).to(DEV)
+    b = _rand((ksegs, groups) + ((n, k) if bkc else (k, n)), dtype, gen).to(DEV)
+    A = a.float() if akc else a.float().transpose(2, 3)
+    B = b.float() if bkc else b.float().transpose(2, 3)
+    ref = torch.einsum("sgmk,sgnk->gmn", A, B)
+    out = torch.full((groups, m, n), float("nan"), dtype=dtype, device=DEV)
+    _lib.profile_enable(1)
+    try:
+        ops.gemm_raw(dtype, a=a.data_ptr(), b=b.data_ptr(), c_out=out.data_ptr(), m=m, n=n, k=k, lda=a.stride(2),
+                     ldb=b.stride(2), ldc=n, a_kcontig=akc, b_kcontig=bkc, groups=groups, a_sg=a.stride(1),
+                     b_sg=b.stride(1), c_sg=m * n, ksegs=ksegs, a_sk=a.stride(0), b_sk=b.stride(0))
+        torch.cuda.synchronize()
+        names = list(_lib.profile_collect())
+    finally:
+        _lib.profile_enable(0)
+    assert any("256x256" in nm for nm in names), names
+    assert not torch.isnan(out).any()
+    assert rel_err(out, ref) <= TOL[dtype]
+
+
 @pytest.mark.parametrize("warm_bytes", [16, 1024, 3 * 1024 + 16, 1 << 20, 80 << 20])
 def test_gemm_carries_a_warm_ahead_hint(warm_bytes):
     """rtp_gemm_warm_next: the next product reads the hinted region at its start and its result is what it is without
