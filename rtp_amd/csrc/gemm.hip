@@ -1737,6 +1737,12 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
     int pcol = 1;
     for (int c = 2; c <= 32 && c <= nbk; ++c)
       if (nbk % c == 0 && c * b_tile_bytes <= 3.0 * 1024 * 1024) pcol = c;
+    // A contraction so long that not even two B tiles fit: nothing stays in the L2 from one panel to the next, and
+    // what counts is the block of tiles that run at the same time and walk K side by side -- as square as it gets
+    // (a 16 x 1 column shares one B tile but streams 16 A tiles; 8 x 4 streams 12 tile-operands for 32 CUs).
+    if (pcol == 1)
+      for (int c = 2; c <= 4 && c <= nbk; ++c)
+        if (nbk % c == 0) pcol = c;
     int prow = 1;
     for (int r = 2; r * pcol <= 32 && r <= mbk; ++r)
       if (mbk % r == 0) prow = r;
