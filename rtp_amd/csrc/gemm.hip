@@ -1674,10 +1674,10 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   int shape = 3;  // 64 x 64 unless the model finds something cheaper
   double best = 0.0;
   for (int i = 0; fast && i < kNumShapes; ++i) {
-    // the 256 x 256 kernel is built for 16-bit operands and the plain epilogue, and pays on products with a long
-    // contraction that give every CU at least one such tile (measured: +9 % forward, +20 % on the transposed
-    // layouts at 8192^3, +10 - 20 % on the expert products of the MoE layer, nothing at 4096^3, a loss where it
-    // leaves CUs without a tile or K is short)
+    // the 256 x 256 kernel is built for 16-bit operands and the plain epilogue, and pays on products that give
+    // every CU at least one such tile and contract over 1024 or more (measured against the next best shape:
+    // +10 - 25 % at 8192^3, +10 % at 4096^3, +5 - 10 % at K = 1024 .. 1536 when the tiles fill the CUs evenly,
+    // -10 % on the MoE layer's time; a loss where it leaves CUs without a tile or K is shorter)
     if (i == 5 && (sizeof(T) != 2 || d->sgd_master || d->xent_mode == 1 ||
                    ceil_div(d->m, 256) * ceil_div(d->n, 256) * nz < 256 || d->k * d->ksegs < 1024) && i != forced)
       continue;

@@ -291,7 +291,7 @@ def test_gemm_many_rounds_tile_order(m, n, k, groups, akc, bkc):
 
 @pytest.mark.parametrize("akc,bkc", [(True, True), (True, False), (False, True)])
 def test_gemm_256x256_tile_path(akc, bkc):
-    """A product with more than 1024 tiles of 256 x 256 and a long K takes the eight-wave kernel (checked by its
+    """A product with at least 256 tiles of 256 x 256 and K >= 1024 takes the eight-wave kernel (checked by its
     name in the launch records); ragged on every edge, with bias, ReLU and an addend in the epilogue.  The yardstick
     is torch's fp32 product of the same bf16 values on the device (float64 on the CPU would take minutes)."""
     from rtp_amd import _lib
