@@ -30,16 +30,16 @@ PEAK = {"bf16_mfma_tflops": 2500.0, "fp32_mfma_tflops": 157.3, "hbm_gbs": 8000.0
 # The weight-gradient variant (128x128 rc_rc) carries the clip + SGD update: its figure includes the fp32 parameters
 # read and written and their bf16 copy written.
 MEASURED_TRAFFIC_KIB = {
-    "gemm_bf16_128x128_rc_rc": 106890.3, "gemm_bf16_128x64_kc_rc": 70132.1, "gemm_bf16_128x64_kc_kc": 46918.5,
-    "gemm_bf16_128x192_kc_kc": 74478.7, "gemm_bf16_128x128_kc_kc": 169485.9,
+    "gemm_bf16_128x128_rc_rc": 106765.4, "gemm_bf16_128x64_kc_rc": 70130.4, "gemm_bf16_128x64_kc_kc": 46902.1,
+    "gemm_bf16_128x192_kc_kc": 74492.7, "gemm_bf16_128x128_kc_kc": 169481.0,
 }
 
 
 # rocprofv3's average duration of a dispatch over the kernel's own execution span (first wave's start to last wave's
 # end, printed by this script as roofline.execution_span), both from the one rocprofv3 run of the default command
-# whose summary is profiles/lm_step_kernel_trace.txt: 47.578 us / 38.074 us for the weight-gradient product,
-# 38.341 / 31.700 for the input-gradient product.  Between runs and boxes the ratio moves by about +-3 %.
-DISPATCH_OVER_EXECUTION_SPAN = {"gemm_bf16_128x128_rc_rc": 47.578 / 38.074, "gemm_bf16_128x64_kc_rc": 38.341 / 31.700}
+# whose summary is profiles/lm_step_kernel_trace.txt: 46.744 us / 36.391 us for the weight-gradient product,
+# 35.889 / 30.888 for the input-gradient product.  Between runs and boxes the ratio moves by about +-3 %.
+DISPATCH_OVER_EXECUTION_SPAN = {"gemm_bf16_128x128_rc_rc": 46.744 / 36.391, "gemm_bf16_128x64_kc_rc": 35.889 / 30.888}
 
 
 def step_flops(c):
