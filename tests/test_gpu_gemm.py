@@ -398,3 +398,45 @@ def test_cache_warm_reads_and_changes_nothing():
         _lib.check(lib.rtp_cache_warm(torch.cuda.current_stream().cuda_stream, t.data_ptr(), nbytes, 0))
     torch.cuda.synchronize()
     assert torch.equal(t, want)
+
+
+def test_gemm_random_shapes_layouts_and_epilogues():
+    """A seeded sweep over shapes that no test picked by hand: sizes that are not multiples of anything (the guarded
+    kernel), multiples of 8 (every fast tile shape the cost model may take, the 256 x 256 kernel included), both
+    dtypes, all four operand layouts, with and without bias / addend / ReLU.  Yardstick: the fp32 product of the same
+    values on the device."""
+    import random
+    ops = _ops()
+    rng = random.Random(20240607)
+    gen = torch.Generator().manual_seed(99)
+    for case in range(72):
+        dtype = torch.bfloat16 if case % 3 else torch.float32
+        akc, bkc = bool(rng.getrandbits(1)), bool(rng.getrandbits(1))
+        if case % 4 == 0:      # ragged: not even vector-aligned
+            m, n, k = rng.randint(1, 700), rng.randint(1, 700), rng.randint(1, 900)
+        elif case % 4 == 3:    # large enough for the biggest tiles
+            m, n, k = 8 * rng.randint(200, 520), 8 * rng.randint(200, 520), 8 * rng.randint(100, 330)
+        else:
+            m, n, k = 8 * rng.randint(1, 160), 8 * rng.randint(1, 160), 8 * rng.randint(1, 300)
+        a = _rand((m, k) if akc else (k, m), dtype, gen).to(DEV)
+        b = _rand((n, k) if bkc else (k, n), dtype, gen).to(DEV)
+        use_bias, use_cin, relu = bool(rng.getrandbits(1)), bool(rng.getrandbits(1)), bool(rng.getrandbits(1))
+        bias = _rand((n,), dtype, gen).to(DEV) if use_bias else None
+        cin = _rand((m, n), dtype, gen).to(DEV) if use_cin else None
+        A = a.float() if akc else a.float().t()
+        B = b.float() if bkc else b.float().t()
+        ref = A @ B.t()
+        if use_bias:
+            ref = ref + bias.float()
+        if use_cin:
+            ref = ref + cin.float()
+        if relu:
+            ref = torch.relu(ref)
+        out = torch.full((m, n), float("nan"), dtype=dtype, device=DEV)
+        ops.gemm_raw(dtype, a=a.data_ptr(), b=b.data_ptr(), c_out=out.data_ptr(), m=m, n=n, k=k, lda=a.stride(0),
+                     ldb=b.stride(0), ldc=n, a_kcontig=akc, b_kcontig=bkc, bias=bias.data_ptr() if use_bias else None,
+                     c_in=cin.data_ptr() if use_cin else None, ld_cin=n, relu=relu)
+        torch.cuda.synchronize()
+        what = f"case {case}: {dtype} m {m} n {n} k {k} akc {akc} bkc {bkc} bias {use_bias} cin {use_cin} relu {relu}"
+        assert not torch.isnan(out).any(), what
+        assert rel_err(out, ref) <= TOL[dtype], what
