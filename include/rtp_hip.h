@@ -222,8 +222,8 @@ int rtp_gemm(void* stream, int dtype, const rtp_gemm_desc* d);
  * That launch requests them at its start, so they sit in the GPU's memory-side cache when their own products run
  * (weights are read once per pass and would otherwise come from HBM at their turn).  Up to 192 KiB per workgroup
  * of the carrying launch.  A hint: no result depends on it; it ends with that next product launch whether or not
- * the launch could carry it (other kernels than the wave-specialised one cannot), so `src` has to stay allocated
- * only until then.  bytes == 0 withdraws a pending hint. */
+ * the launch could carry it (other kernels than the wave-specialised one cannot).  The carrying kernel reads `src` when
+ * it RUNS, not when it is launched: `src` has to stay mapped until that launch has completed on its stream.  bytes == 0 withdraws a pending hint. */
 int rtp_gemm_warm_next(const void* src, size_t bytes);
 
 /* Measurement aid (no counterpart in the reference; bench.py reports it beside the published peak): TFLOP/s of a
@@ -480,7 +480,8 @@ int rtp_layernorm_bwd_finalize(void* stream, int dtype, const rtp_ln_final_item*
  *   reduce: out[0] = sum_r loss[r], divided by the number of rows with target != ignore_index when `mean`;
  *        scale[0] = 1 / that number (1 without `mean`) -- the `scale` of the backward pass of a mean loss.  One
  *        workgroup, fixed summation order; no rows at all or all ignored gives NaN, as torch does.
- * A row whose target equals ignore_index has loss 0 and gradient 0.  Any other target outside [0, cols) is the
+ * A row whose target equals ignore_index (inside the class range or not: a padding id such as 0 counts) has loss 0
+ * and gradient 0, in fwd, reduce and bwd alike.  Any other target outside [0, cols) is the
  * caller's error (torch asserts on the device): its loss is NaN, which shows in every sum over the rows, and its
  * gradient 0.  fp32 or bf16 logits, statistics in fp32.  Rows of whole 16-byte vectors (cols and both leading
  * dimensions multiples of 16 bytes, 16-byte aligned, at most 8192 vectors: 65536 bf16 or 32768 fp32 classes) are
@@ -496,8 +497,8 @@ int rtp_softmax_xent_combine(void* stream, const float* part, int64_t blocks, co
 int rtp_softmax_xent_reduce(void* stream, const float* loss, const int64_t* target, int64_t ignore_index,
                             int64_t rows, int mean, float* out, float* scale);
 int rtp_softmax_xent_bwd(void* stream, int dtype, const void* logits, int64_t ld, int64_t rows, int64_t cols,
-                         const int64_t* target, const float* stats, const float* dloss, int64_t dloss_stride,
-                         const float* scale, void* dlogits, int64_t ld_dlogits);
+                         const int64_t* target, int64_t ignore_index, const float* stats, const float* dloss,
+                         int64_t dloss_stride, const float* scale, void* dlogits, int64_t ld_dlogits);
 
 /* ---------------------------------------------------------------------------------------------
  * Top-2 routing (reference: top2gating, rtp/module/top2gate.py:43-105).
@@ -661,10 +662,9 @@ int rtp_cast(void* stream, int dtype_src, const void* src, int dtype_dst, void* 
  * its kernel-variant name with the algorithmic flops and bytes of that launch.  rtp_profile_collect
  * synchronises the device, sums the event durations per name into `out` (at most `max_out`
  * entries, *n_out receives the count) and clears the records.  rtp_profile_read does the same without
- * clearing them.  Profiling may be on while a stream is captured into a HIP graph: the events then become
- * nodes of that graph, every replay stamps them again, and rtp_profile_read after a replay returns the
- * durations of that replay -- per-kernel times of the graph-replayed schedule, all streams live.  Call
- * rtp_profile_collect only when the graph will not be replayed again (it destroys the events).
+ * clearing them.  Event timing (mode 1) is for eager launches only: timing events recorded while a stream is
+ * captured into a HIP graph read 0 after a replay, so a launch made on a capturing stream is not timed in mode 1.
+ * Launches inside a replayed graph are timed by mode 2 (below).
  * --------------------------------------------------------------------------------------------- */
 typedef struct {
   char name[64];

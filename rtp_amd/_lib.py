@@ -144,7 +144,7 @@ PROTOTYPES = {
     "rtp_layernorm_bwd": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _sz]),
     "rtp_softmax_xent_fwd": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _vp]),
     "rtp_softmax_xent_reduce": (_i, [_vp, _vp, _vp, _i64, _i64, _i, _vp, _vp]),
-    "rtp_softmax_xent_bwd": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _i64]),
+    "rtp_softmax_xent_bwd": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _i64, _vp, _vp, _i64]),
     "rtp_top2_route_workspace_bytes": (_sz, [_i64, _i64]),
     "rtp_top2_route": (_i, [_vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz]),
     "rtp_top2_route_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),

@@ -1678,8 +1678,9 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
     // every CU at least one such tile and contract over 1024 or more (measured against the next best shape:
     // +10 - 25 % at 8192^3, +10 % at 4096^3, +5 - 10 % at K = 1024 .. 1536 when the tiles fill the CUs evenly,
     // -10 % on the MoE layer's time; a loss where it leaves CUs without a tile or K is shorter)
-    if (i == 5 && (sizeof(T) != 2 || d->sgd_master || d->xent_mode == 1 ||
-                   ceil_div(d->m, 256) * ceil_div(d->n, 256) * nz < 256 || d->k * d->ksegs < 1024) && i != forced)
+    // (its epilogue is the plain one: the update and the statistics epilogue are never routed to it, forced or not)
+    if (i == 5 && (sizeof(T) != 2 || d->sgd_master || d->xent_mode == 1)) continue;
+    if (i == 5 && (ceil_div(d->m, 256) * ceil_div(d->n, 256) * nz < 256 || d->k * d->ksegs < 1024) && i != forced)
       continue;
     // never a tile that is mostly padding: a 32 x 32 problem (one attention head at seq 32) stays at 64 x 64
     if ((!akc && (kShapes[i].bm & (kShapes[i].bm - 1))) || (!bkc && (kShapes[i].bn & (kShapes[i].bn - 1)))) continue;
@@ -1772,7 +1773,17 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
   const double upd_sz = d->sgd_master ? 8.0 + (d->sgd_weights ? (double)sizeof(T) : 0.0) -
                                             ((d->flags & RTP_GEMM_SGD_SKIP_OUT) ? out_sz : 0.0)
                                       : 0.0;
-  const double bytes = ((double)d->m + (double)d->n) * kk * nz * sizeof(T) + mn * (out_sz + cin_sz + upd_sz);
+  // An operand that every group / batch entry / K segment reads from the same address (stride 0: the activations of a
+  // column layer's forward and weight-gradient products) is counted once, not once per shard.
+  const auto copies = [&](int64_t so, int64_t si, int64_t sg, int64_t sk) {
+    const double per_batch = (d->batch > 1 && (so != 0 || si != 0)) ? (double)d->batch : 1.0;
+    const double per_group = (d->groups > 1 && sg != 0) ? (double)d->groups : 1.0;
+    const double per_kseg = (d->ksegs > 1 && sk != 0) ? (double)d->ksegs : 1.0;
+    return per_batch * per_group * per_kseg;
+  };
+  const double bytes = ((double)d->m * copies(d->a_so, d->a_si, d->a_sg, d->a_sk) +
+                        (double)d->n * copies(d->b_so, d->b_si, d->b_sg, d->b_sk)) * (double)d->k * sizeof(T) +
+                       mn * (out_sz + cin_sz + upd_sz);
   ProfileScope prof(s, name, 2.0 * mn * kk, bytes);
   a.trace = fast ? prof.trace_slot() : nullptr;
   a.warm = nullptr;

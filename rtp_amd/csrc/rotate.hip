@@ -35,6 +35,10 @@ static int g_trace_next = 0;
 ProfileScope::ProfileScope(hipStream_t stream, const char* name, double flops, double bytes)
     : stream_(stream), name_(name), flops_(flops), bytes_(bytes) {
   if (g_profile_mode != 1) return;
+  // Timing events recorded while a stream is captured read 0 after a replay (observed): such launches are not timed
+  // in this mode -- device time stamps (mode 2) are for them.
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream_, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) return;
   if (hipEventCreate(&start_) != hipSuccess) {
     start_ = nullptr;
     return;
@@ -189,7 +193,7 @@ using namespace rtp;
 
 extern "C" const char* rtp_last_error(void) { return error_buffer(); }
 
-extern "C" int rtp_abi_version(void) { return 2; }
+extern "C" int rtp_abi_version(void) { return 3; }
 
 extern "C" int rtp_device_check(char* name_out, int name_len) {
   int dev = 0;
@@ -338,9 +342,9 @@ extern "C" int rtp_profile_reset_stamps(void* stream) {
   return RTP_OK;
 }
 
-// Sums the recorded launches per kernel name.  `clear`: destroy the event pairs afterwards.  Without it they stay
-// valid -- what a HIP graph needs whose capture recorded them as event nodes: every replay stamps them anew, and a
-// read after a replay returns that replay's durations.
+// Sums the recorded launches per kernel name.  `clear`: destroy the event pairs and forget the stamp slots afterwards.
+// Without it the stamp slots stay booked -- what a replayed HIP graph needs whose launches carry them: every replay
+// stamps them anew, and a read after a replay returns that replay's durations.
 static int profile_sum(rtp_kernel_stat* out, int max_out, int* n_out, bool clear) {
   RTP_REQUIRE(out && n_out && max_out > 0, "rtp_profile_collect: bad arguments");
   RTP_HIP_TRY(hipDeviceSynchronize());

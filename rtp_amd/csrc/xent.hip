@@ -105,14 +105,14 @@ __global__ __launch_bounds__(kXentThreads) void xent_fwd_any_kernel(const T* x, 
 
 template <typename T>
 __global__ __launch_bounds__(kXentThreads) void xent_bwd_any_kernel(const T* x, long ld, int cols, const long* target,
-                                                                    const float2* stats, const float* dloss,
-                                                                    long dloss_stride, const float* scale, T* dx,
-                                                                    long ld_dx) {
+                                                                    long ignore, const float2* stats,
+                                                                    const float* dloss, long dloss_stride,
+                                                                    const float* scale, T* dx, long ld_dx) {
   const long row = blockIdx.x;
   const T* xr = x + row * ld;
   T* dr = dx + row * ld_dx;
   const long t = target[row];
-  const bool live = t >= 0 && t < cols;
+  const bool live = t != ignore && t >= 0 && t < cols;
   const float2 st = stats[row];
   const float inv = 1.0f / st.y;
   const float s = live ? dloss[row * dloss_stride] * (scale ? *scale : 1.0f) : 0.0f;
@@ -165,9 +165,9 @@ __global__ __launch_bounds__(kXentThreads) void xent_reduce_kernel(const float* 
 
 template <typename T, int NV>
 __global__ __launch_bounds__(kXentThreads) void xent_bwd_kernel(const T* x, long ld, int cols, const long* target,
-                                                                const float2* stats, const float* dloss, long dloss_stride,
-                                                                const float* scale, T* dx, long ld_dx) {
-  touch_kernel_arguments<80>();
+                                                                long ignore, const float2* stats, const float* dloss,
+                                                                long dloss_stride, const float* scale, T* dx, long ld_dx) {
+  touch_kernel_arguments<88>();
   constexpr int VEC = XVec<T>::N;
   const long row = blockIdx.x;
   const T* xr = x + row * ld;
@@ -180,7 +180,7 @@ __global__ __launch_bounds__(kXentThreads) void xent_bwd_kernel(const T* x, long
     v[i].q = reinterpret_cast<const uint4*>(xr)[c < nvec ? c : 0];
   }
   const long t = target[row];
-  const bool live = t >= 0 && t < cols;
+  const bool live = t != ignore && t >= 0 && t < cols;
   const float2 st = stats[row];
   const float mx = st.x, inv = 1.0f / st.y;
   const float s = live ? dloss[row * dloss_stride] * (scale ? *scale : 1.0f) : 0.0f;
@@ -301,8 +301,8 @@ extern "C" int rtp_softmax_xent_reduce(void* stream, const float* loss, const in
 }
 
 extern "C" int rtp_softmax_xent_bwd(void* stream, int dtype, const void* logits, int64_t ld, int64_t rows, int64_t cols,
-                                    const int64_t* target, const float* stats, const float* dloss, int64_t dloss_stride,
-                                    const float* scale, void* dlogits, int64_t ld_dlogits) {
+                                    const int64_t* target, int64_t ignore_index, const float* stats, const float* dloss,
+                                    int64_t dloss_stride, const float* scale, void* dlogits, int64_t ld_dlogits) {
   RTP_REQUIRE(logits && target && stats && dloss && dlogits, "rtp_softmax_xent_bwd: null pointer");
   RTP_REQUIRE((uintptr_t)stats % 8 == 0, "rtp_softmax_xent_bwd: stats must be 8-byte aligned");
   RTP_REQUIRE(dloss_stride == 0 || dloss_stride == 1, "rtp_softmax_xent_bwd: dloss_stride must be 0 or 1");
@@ -315,11 +315,11 @@ extern "C" int rtp_softmax_xent_bwd(void* stream, int dtype, const void* logits,
   if (!xent_vectors(dtype, ld, cols, logits) || !xent_vectors(dtype, ld_dlogits, cols, dlogits)) {
     if (dtype == RTP_F32)
       hipLaunchKernelGGL(xent_bwd_any_kernel<float>, grid, block, 0, st, (const float*)logits, (long)ld, (int)cols,
-                         (const long*)target, (const float2*)stats, dloss, (long)dloss_stride, scale, (float*)dlogits,
+                         (const long*)target, (long)ignore_index, (const float2*)stats, dloss, (long)dloss_stride, scale, (float*)dlogits,
                          (long)ld_dlogits);
     else
       hipLaunchKernelGGL(xent_bwd_any_kernel<bf16_t>, grid, block, 0, st, (const bf16_t*)logits, (long)ld, (int)cols,
-                         (const long*)target, (const float2*)stats, dloss, (long)dloss_stride, scale, (bf16_t*)dlogits,
+                         (const long*)target, (long)ignore_index, (const float2*)stats, dloss, (long)dloss_stride, scale, (bf16_t*)dlogits,
                          (long)ld_dlogits);
     RTP_LAUNCH_CHECK();
     return RTP_OK;
@@ -327,10 +327,10 @@ extern "C" int rtp_softmax_xent_bwd(void* stream, int dtype, const void* logits,
   const int nv = (int)ceil_div(cols / (dtype == RTP_F32 ? 4 : 8), kXentThreads);
   if (dtype == RTP_F32)
     launch_xent_bwd<float>(nv, grid, st, (const float*)logits, (long)ld, (int)cols, (const long*)target,
-                           (const float2*)stats, dloss, (long)dloss_stride, scale, (float*)dlogits, (long)ld_dlogits);
+                           (long)ignore_index, (const float2*)stats, dloss, (long)dloss_stride, scale, (float*)dlogits, (long)ld_dlogits);
   else
     launch_xent_bwd<bf16_t>(nv, grid, st, (const bf16_t*)logits, (long)ld, (int)cols, (const long*)target,
-                            (const float2*)stats, dloss, (long)dloss_stride, scale, (bf16_t*)dlogits, (long)ld_dlogits);
+                            (long)ignore_index, (const float2*)stats, dloss, (long)dloss_stride, scale, (bf16_t*)dlogits, (long)ld_dlogits);
   RTP_LAUNCH_CHECK();
   return RTP_OK;
 }

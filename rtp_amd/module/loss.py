@@ -18,6 +18,7 @@ class _RowLossFn(torch.autograd.Function):
     def forward(ctx, logits, target, ignore_index):
         loss, stats = ops.softmax_xent_fwd(logits, target, ignore_index)
         ctx.save_for_backward(logits, target, stats)
+        ctx.ignore_index = ignore_index
         return loss
 
     @staticmethod
@@ -26,7 +27,7 @@ class _RowLossFn(torch.autograd.Function):
         dloss = dloss.float()
         if dloss.dim() == 1 and dloss.shape[0] > 1 and dloss.stride(0) not in (0, 1):
             dloss = dloss.contiguous()
-        return ops.softmax_xent_bwd(logits, target, stats, dloss), None, None
+        return ops.softmax_xent_bwd(logits, target, stats, dloss, ignore_index=ctx.ignore_index), None, None
 
 
 class _ReducedLossFn(torch.autograd.Function):
@@ -37,12 +38,14 @@ class _ReducedLossFn(torch.autograd.Function):
         rows, stats = ops.softmax_xent_fwd(logits, target, ignore_index)
         loss, scale = ops.softmax_xent_reduce(rows, target, ignore_index, mean)
         ctx.save_for_backward(logits, target, stats, scale)
+        ctx.ignore_index = ignore_index
         return loss
 
     @staticmethod
     def backward(ctx, dloss):
         logits, target, stats, scale = ctx.saved_tensors
-        return ops.softmax_xent_bwd(logits, target, stats, dloss.float().reshape(1), scale=scale), None, None, None
+        return ops.softmax_xent_bwd(logits, target, stats, dloss.float().reshape(1), scale=scale,
+                                    ignore_index=ctx.ignore_index), None, None, None
 
 
 class _LinearCrossEntropyFn(torch.autograd.Function):

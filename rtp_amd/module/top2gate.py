@@ -159,7 +159,11 @@ class Top2Gate(RotatedLayer):
         self.num_experts = num_experts
         self.world_size, self.rank, self.num_local_experts = 1, 0, num_experts
         self._init_store([nn.Linear(model_dim, num_experts, bias=False)])
-        self.wg = self.shards[0]
+        # registered once, under the reference's name: state_dict() is exactly {"wg.weight"} (top2gate.py:124)
+        wg = self.shards[0]
+        del self._modules["shards"]
+        self.shards = [wg]
+        self.wg = wg
 
     def forward(self, input: Tensor, noise: Optional[Tensor] = None) -> Tuple[Tensor, Tensor, Tensor]:
         logits = _GateProjectionFn.apply(input, self._anchor, self)

@@ -711,9 +711,11 @@ def softmax_xent_reduce(loss_rows: torch.Tensor, target: torch.Tensor, ignore_in
 
 
 def softmax_xent_bwd(logits: torch.Tensor, target: torch.Tensor, stats: torch.Tensor, dloss: torch.Tensor,
-                     out: Optional[torch.Tensor] = None, scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     out: Optional[torch.Tensor] = None, scale: Optional[torch.Tensor] = None,
+                     ignore_index: int = -100) -> torch.Tensor:
     """dlogits = (softmax(logits) - onehot(target)) * dloss[row] (* scale[0]); dloss fp32 [rows] with stride 0 or
-    1, or one element for all rows; scale: an fp32 device scalar."""
+    1, or one element for all rows; scale: an fp32 device scalar.  Rows whose target equals `ignore_index` (also one
+    inside the class range, such as a padding id) get a zero gradient."""
     _xent_check("softmax_xent_bwd", logits, target)
     rows, cols = logits.shape
     if dloss.dtype != torch.float32 or dloss.numel() not in (1, rows) or dloss.dim() > 1:
@@ -732,7 +734,8 @@ def softmax_xent_bwd(logits: torch.Tensor, target: torch.Tensor, stats: torch.Te
     _lib.require_device()
     check(_lib.load().rtp_softmax_xent_bwd(_stream(), dtype_code(logits.dtype), logits.data_ptr(),
                                            logits.stride(0) if rows > 1 else cols, rows, cols, target.data_ptr(),
-                                           stats.data_ptr(), dloss.data_ptr(), 0 if rows <= 1 else stride,
+                                           int(ignore_index), stats.data_ptr(), dloss.data_ptr(),
+                                           0 if rows <= 1 else stride,
                                            _ptr(scale), out.data_ptr(), out.stride(0) if rows > 1 else cols))
     return out
 
@@ -940,9 +943,21 @@ class FusedSgd:
     """What a weight-gradient product needs to apply clip + SGD in its own epilogue: the step's scalars, whether the
     gradient is still to be stored, and the record of what was (or could not be) updated this way."""
 
-    def __init__(self, lr: float, clip: float, keep_grads: bool = False):
-        self.lr, self.clip, self.keep_grads = float(lr), float(clip), bool(keep_grads)
+    def __init__(self, lr: float, clip: float, keep_grads: bool = False, source=None):
+        """`source`: an object whose `lr` / `clip_value` attributes are read at every launch (the optimiser), so that a
+        learning-rate schedule reaches the fused epilogues like every other update; without one the two scalars
+        given here stay fixed."""
+        self._lr, self._clip, self.keep_grads = float(lr), float(clip), bool(keep_grads)
+        self._source = source
         self.missed = False
+
+    @property
+    def lr(self) -> float:
+        return float(self._source.lr) if self._source is not None else self._lr
+
+    @property
+    def clip(self) -> float:
+        return float(self._source.clip_value) if self._source is not None else self._clip
 
 
 class ShardSum:

@@ -97,7 +97,7 @@ class RotatedSGD:
         self._rest_table = self._rest_key = None
         self._rest_params = 0
         if self.fused_backward:
-            ctx = ops.FusedSgd(self.lr, self.clip_value, keep_grads)
+            ctx = ops.FusedSgd(self.lr, self.clip_value, keep_grads, source=self)
             for st, master in zip(self.stores, self.masters):
                 st.fused_sgd = _FusedBinding(ctx, master)
         if self.overlap_backward and self.stores:

@@ -379,6 +379,8 @@ def test_lm_sgd_fused_into_weight_gradient_products_is_bit_identical(dtype, wgra
         for step in range(3):
             ids = torch.randint(0, V, (L, N), generator=gen).to(DEV)
             for lm, opt in zip(lms, opts):
+                if step == 1:     # a schedule: the fused epilogues must follow the optimiser's current scalars
+                    opt.lr, opt.clip_value = 0.02, 0.03
                 opt.zero_grad()
                 F.cross_entropy(lm(ids).float().view(-1, V), ids.view(-1)).backward()
                 opt.step()

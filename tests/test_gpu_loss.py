@@ -52,6 +52,52 @@ def test_cross_entropy_reductions_ignore_index_and_upstream_gradient(reduction):
     assert torch.count_nonzero(x.grad[::5]).item() == 0   # ignored rows get no gradient
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("reduction", ["none", "sum", "mean"])
+@pytest.mark.parametrize("cols", [512, 37])
+def test_cross_entropy_ignore_index_inside_the_class_range(dtype, reduction, cols):
+    """A padding id such as 0 is a valid class index AND the ignore index: its rows give zero loss and zero gradient
+    in the vector kernels (512 classes) and the element-wise ones (37), and the mean runs over the other rows."""
+    from rtp_amd.module.loss import cross_entropy
+    rows = 50
+    store, target = _case(rows, cols, dtype, 11 + cols)
+    target[::3] = 0
+    ref_in = store.float().clone().requires_grad_()
+    ref = F.cross_entropy(ref_in, target, reduction=reduction, ignore_index=0)
+    w = torch.linspace(0.5, 2.0, rows) if reduction == "none" else torch.tensor(0.6)
+    (ref * w).sum().backward()
+    x = store.to(DEV).requires_grad_()
+    out = cross_entropy(x, target.to(DEV), ignore_index=0, reduction=reduction)
+    (out * w.to(DEV)).sum().backward()
+    assert_close(out, ref, torch.float32, "loss")
+    assert_close(x.grad, ref_in.grad, dtype, "dlogits")
+    assert torch.count_nonzero(x.grad[::3]).item() == 0
+    assert torch.count_nonzero(x.grad[1]).item() > 0
+
+
+def test_linear_cross_entropy_ignore_index_inside_the_class_range():
+    from rtp_amd import emulate_shards
+    from rtp_amd.module.linear import ColumnParallelLinear
+    from rtp_amd.module.loss import linear_cross_entropy
+    gen = torch.Generator().manual_seed(21)
+    rows, k, vocab = 96, 64, 512
+    master = torch.nn.Linear(k, vocab)
+    with emulate_shards(4):
+        layer = ColumnParallelLinear(k, vocab, linear_layer=master, device=DEV, dtype=torch.float32)
+    x = torch.randn(rows, k, generator=gen)
+    target = torch.randint(0, vocab, (rows,), generator=gen)
+    target[::4] = 0
+    xd = x.to(DEV).requires_grad_()
+    loss = linear_cross_entropy(xd, layer, target.to(DEV), ignore_index=0)
+    loss.backward()
+    xr = x.clone().requires_grad_()
+    ref = F.cross_entropy(master(xr), target, ignore_index=0)
+    ref.backward()
+    assert abs(float(loss) - float(ref)) <= 1e-5 * abs(float(ref))
+    assert_close(xd.grad, xr.grad, torch.float32, "dx")
+    assert torch.count_nonzero(xd.grad[::4]).item() == 0
+
+
 def test_cross_entropy_extreme_logits_stay_finite():
     from rtp_amd.module.loss import cross_entropy
     x = torch.zeros(4, 64, dtype=torch.float32)

@@ -150,3 +150,56 @@ def test_wrapped_model_trains_with_a_stock_optimizer(overlap):
     m = model.module
     assert_close(torch.cat([s.weight for s in m.fc1.module_list], 0), ref.fc1.weight, torch.float32, "fc1 after 3 steps")
     assert_close(torch.cat([s.weight for s in m.emb.module_list], 1), ref.emb.weight, torch.float32, "emb after 3 steps")
+
+
+def test_leaves_wrapped_by_hand_with_the_reference_constructor():
+    """Code that cuts a leaf to a rank's share and wraps it itself (rtp/rotated_tensor_parallel.py:454-470 done by
+    hand): column shards of one Linear and row shards of the next, through the reference's import path."""
+    from rtp.rotated_tensor_parallel import FlyweightWarpper, split_tensor
+    from rtp_amd import emulate_shards
+    ws = 4
+    torch.manual_seed(1)
+    fc1, fc2 = nn.Linear(16, 24), nn.Linear(24, 6)
+    cols, rows = [], []
+    for r in range(ws):
+        leaf = nn.Linear(16, 6)
+        leaf.weight = nn.Parameter(split_tensor(fc1.weight, ws, dim=0)[r].clone())
+        leaf.bias = nn.Parameter(split_tensor(fc1.bias, ws, dim=0)[r].clone())
+        cols.append(leaf.to(DEV))
+        leaf = nn.Linear(6, 6)
+        leaf.weight = nn.Parameter(split_tensor(fc2.weight, ws, dim=-1)[r].clone())
+        leaf.bias = nn.Parameter(fc2.bias.detach() / ws)
+        rows.append(leaf.to(DEV))
+    with emulate_shards(ws):
+        w1 = FlyweightWarpper(cols, None)
+        w2 = FlyweightWarpper(rows, None, row_partition=True, input_partition_dim=-1)
+    x, g = torch.randn(9, 16), torch.randn(9, 6)
+    xd = x.to(DEV).requires_grad_()
+    out = w2(torch.relu(w1(xd)))
+    out.backward(g.to(DEV))
+    xr = x.clone().requires_grad_()
+    want = fc2(torch.relu(fc1(xr)))
+    want.backward(g)
+    assert_close(out, want, torch.float32, "output")
+    assert_close(xd.grad, xr.grad, torch.float32, "input grad")
+    assert_close(torch.cat([s.weight.grad for s in w1.module_list], 0), fc1.weight.grad, torch.float32, "fc1")
+    assert_close(torch.cat([s.weight.grad for s in w2.module_list], 1), fc2.weight.grad, torch.float32, "fc2")
+    assert_close(w2.module.bias.grad, fc2.bias.grad, torch.float32, "fc2 bias")
+
+
+def test_language_model_through_the_reference_import_path():
+    """`from rtp.models.transformer_lm_rtp import TransformerLM` with the reference's argument list builds the
+    rotated model of this library and runs a step on the device."""
+    from rtp.models.transformer_lm_rtp import TransformerLM
+    from rtp.module.collectives import zero_full_grads
+    from rtp_amd.models import transformer_lm_rtp as mine
+    assert TransformerLM is mine.TransformerLM
+    V, ws = 64, 2
+    lm = TransformerLM(V, 32, 2, 32, 0.0, 0.1, 1, ws, 0, device=DEV, dtype=torch.float32)
+    ids = torch.randint(0, V, (6, 3)).to(DEV)
+    logits = lm(ids)
+    assert logits.shape == (6, 3, V)
+    torch.nn.functional.cross_entropy(logits.view(-1, V), ids.view(-1)).backward()
+    assert all(s.weight.grad is not None for s in lm[-1].linear.linears)
+    zero_full_grads(lm)
+    assert all(s.weight.grad is None for s in lm[-1].linear.linears)

@@ -138,6 +138,19 @@ def test_moe_and_gate_shards():
             moe.WeightMOELayer(gate, nn.Linear(8, 8))
 
 
+def test_top2gate_state_dict_has_the_reference_key_set():
+    """The unsharded gate's state dict is {'wg.weight'} (rtp/module/top2gate.py:124): a plain dict of that form
+    loads strictly, the flat home row follows, and dtype moves keep the aliasing."""
+    g = top2gate.Top2Gate(8, 4)
+    assert list(g.state_dict().keys()) == ["wg.weight"]
+    assert [n for n, _ in g.named_parameters()] == ["wg.weight"]
+    w = torch.arange(32, dtype=torch.float32).view(4, 8)
+    g.load_state_dict({"wg.weight": w}, strict=True)
+    assert torch.equal(g.wg.weight, w) and torch.equal(g._store.home.view(4, 8), w)
+    g.to(torch.bfloat16)
+    assert g.wg.weight.data_ptr() == g._store.home.data_ptr() and g.shards[0] is g.wg
+
+
 def test_forward_without_gpu_fails_loudly():
     from rtp_amd._lib import RtpError
     with emulate_shards(2):
@@ -166,6 +179,111 @@ def test_forward_without_gpu_fails_loudly():
 def test_constructor_signatures_match_reference(cls, expected):
     params = [p for p in inspect.signature(cls.__init__).parameters if p != "self"]
     assert params == expected
+
+
+def test_reference_import_paths_resolve_to_the_same_objects():
+    """Every import path of the reference's hot path (rtp/rotated_tensor_parallel.py, rtp/attention.py,
+    rtp/module/*.py, rtp/models/transformer_lm_rtp.py) resolves here, to the very objects of rtp_amd."""
+    import importlib
+    pairs = {
+        "rtp.rotated_tensor_parallel": ["RotatedTensorParallel", "FlyweightWarpper", "split_tensor"],
+        "rtp.attention": ["ParallelMultiheadAttention"],
+        "rtp.module.linear": ["ColumnParallelLinear", "RowParallelLinear", "ModelParallelLinear", "ModelParallelLinear2"],
+        "rtp.module.embedding": ["ParallelEmbedding", "ModelParallelEmbedding"],
+        "rtp.module.attention": ["ParallelMultiheadAttention", "SubParallelMultiheadAttention"],
+        "rtp.module.moe": ["WeightMOELayer"],
+        "rtp.module.top2gate": ["top2gating", "Top2Gate", "WeightTop2Gate", "gumbel_rsample"],
+        "rtp.module.collectives": ["zero_full_grads"],
+        "rtp.module.conv": ["ColumnParallelConv2d", "ModelParallelConv2d"],
+        "rtp.module.utils": ["affine_weight", "affine_weight_attention", "divide_and_check_no_remainder",
+                             "ensure_divisibility", "split_tensor_along_last_dim"],
+        "rtp.models.transformer_lm_rtp": ["TransformerLM", "EmbeddingLayer", "PositionalEncodingLayer",
+                                          "FeedForwardLayer", "FeedForwardLayer_expert", "TransformerDecoderLayer",
+                                          "TransformerEncoderLayer", "LinearLayer"],
+    }
+    for path, names in pairs.items():
+        theirs = importlib.import_module(path)
+        mine = importlib.import_module(path.replace("rtp.", "rtp_amd.", 1))
+        assert theirs is mine, path
+        for n in names:
+            assert getattr(theirs, n) is getattr(mine, n), f"{path}.{n}"
+    from rtp.module.linear import ColumnParallelLinear as C1   # the `from ... import` form as well
+    assert C1 is linear.ColumnParallelLinear
+    import rtp.attention
+    import rtp.module.attention
+    assert rtp.attention.ParallelMultiheadAttention is not rtp.module.attention.ParallelMultiheadAttention
+
+
+def test_flyweight_wrapper_takes_the_reference_constructor_arguments():
+    """rtp/rotated_tensor_parallel.py:296-310, and a leaf cut to one rank's share by hand (:454-529)."""
+    from rtp_amd.rotated_tensor_parallel import FlyweightWarpper, split_tensor
+    params = [p for p in inspect.signature(FlyweightWarpper.__init__).parameters if p != "self"]
+    assert params == ["module", "group", "param_list", "flat_param_names", "partition_dim", "output_partition_dim",
+                      "row_partition", "input_partition_dim", "cat_output", "inplace"]
+    ws = 2
+    master = nn.Linear(6, 4)
+    leaves = []
+    for r in range(ws):       # what rank r of the reference does before wrapping a column shard
+        leaf = nn.Linear(6, 2)
+        leaf.weight = nn.Parameter(split_tensor(master.weight, ws, dim=0)[r].clone())
+        leaf.bias = nn.Parameter(split_tensor(master.bias, ws, dim=0)[r].clone())
+        leaves.append(leaf)
+    with emulate_shards(ws):
+        col = FlyweightWarpper(leaves, None)
+        one = FlyweightWarpper(leaves[0])                     # a single leaf: every rank starts from a copy
+        rows = []
+        for r in range(ws):   # row shards: weight columns, bias / ws
+            leaf = nn.Linear(3, 4)
+            leaf.weight = nn.Parameter(split_tensor(master.weight, ws, dim=-1)[r].clone())
+            leaf.bias = nn.Parameter(master.bias.detach() / ws)
+            rows.append(leaf)
+        row = FlyweightWarpper(rows, None, row_partition=True, input_partition_dim=-1)
+        with pytest.raises(NotImplementedError):
+            FlyweightWarpper(nn.LayerNorm(4))
+        with pytest.raises(ValueError):
+            FlyweightWarpper(leaves + leaves)
+        with pytest.raises(NotImplementedError):
+            FlyweightWarpper(nn.Conv2d(2, 4, 3))              # conv outputs concatenate on dim 1
+        convw = FlyweightWarpper(nn.Conv2d(2, 4, 3), output_partition_dim=1)
+        emb = FlyweightWarpper(nn.Embedding(10, 3))
+    assert type(col.rotated) is linear.ColumnParallelLinear and col.world_size == ws and col.rank == 0
+    assert torch.equal(torch.cat([m.weight for m in col.module_list], 0), master.weight)
+    assert torch.equal(torch.cat([m.bias for m in col.module_list], 0), master.bias)
+    assert col.flat_param.data_ptr() == col.module.weight.data_ptr() and col.partition_dim == -1
+    assert torch.equal(one.module_list[1].weight, leaves[0].weight)
+    assert type(row.rotated) is linear.RowParallelLinear and row.row_partition
+    assert torch.equal(torch.cat([m.weight for m in row.module_list], 1), master.weight)
+    assert type(convw.rotated) is conv.ColumnParallelConv2d and convw.rotated.out_channels == 8
+    assert type(emb.rotated) is embedding.ParallelEmbedding and emb.rotated.embedding_dim == 6
+
+
+def test_attention_leaf_of_the_wrapper_module():
+    """rtp/attention.py's ParallelMultiheadAttention is one rank's head group; wrapped, it is the rotated layer."""
+    from rtp_amd.attention import ParallelMultiheadAttention as Leaf
+    from rtp_amd.rotated_tensor_parallel import FlyweightWarpper
+    params = [p for p in inspect.signature(Leaf.__init__).parameters if p != "self"]
+    assert params == ["embed_dim", "num_heads", "dropout", "bias", "add_bias_kv", "add_zero_attn", "kdim", "vdim",
+                      "batch_first", "device", "dtype", "MultiheadAttention", "empty_init", "group"]
+    mha = nn.MultiheadAttention(8, 4)
+    ws = 2
+    with emulate_shards(ws):
+        leaf = Leaf(8, 4, MultiheadAttention=mha)
+        assert leaf.in_proj_weight.shape == (12, 8) and leaf.out_proj.weight.shape == (8, 4) and leaf.rank == 0
+        leaves = [leaf]
+        for r in range(1, ws):
+            other = Leaf(8, 4)
+            other.rank = r
+            other.affine_weight(mha)
+            leaves.append(other)
+        wrapped = FlyweightWarpper(leaves, None, cat_output=False)
+        with pytest.raises(NotImplementedError):
+            FlyweightWarpper(leaves, None)                    # attention outputs are summed, not concatenated
+    assert type(wrapped.rotated) is attention.ParallelMultiheadAttention
+    direct = attention.ParallelMultiheadAttention(8, 4, ws, 0, MultiheadAttention_layer=mha)
+    for a, b in zip(wrapped.rotated._store.home, direct._store.home):
+        assert torch.equal(a, b)
+    with pytest.raises(NotImplementedError):
+        leaf(torch.zeros(2, 1, 8), torch.zeros(2, 1, 8), torch.zeros(2, 1, 8))
 
 
 def test_rank_state_dicts_follow_the_reference_layout_and_round_trip():
