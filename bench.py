@@ -24,22 +24,70 @@ if ROOT not in sys.path:
 
 CFG = dict(vocab=10240, ninp=2048, nhid=2048, nhead=32, layers=10, seq=32, batch=32, shards=8)
 PEAK = {"bf16_mfma_tflops": 2500.0, "fp32_mfma_tflops": 157.3, "hbm_gbs": 8000.0}
-# Memory-side traffic per launch of the GEMM variants of this workload, KiB, averaged over the launches of a step:
-# FETCH_SIZE * 1.9999 + WRITE_SIZE * 1.0000 from two rocprofv3 --pmc runs of this script; the factors are what the same
-# counters read for the library's plain copy kernel on a copy of known size (profiles/lm_step_pmc_fetch_write.txt).
-# The weight-gradient variant (128x128 rc_rc) carries the clip + SGD update: its figure includes the fp32 parameters
-# read and written and their bf16 copy written.
-MEASURED_TRAFFIC_KIB = {
-    "gemm_bf16_128x128_rc_rc": 106765.4, "gemm_bf16_128x64_kc_rc": 70130.4, "gemm_bf16_128x64_kc_kc": 46902.1,
-    "gemm_bf16_128x192_kc_kc": 74492.7, "gemm_bf16_128x128_kc_kc": 169481.0,
-}
+PROFILES = os.path.join(ROOT, "profiles")
 
 
-# rocprofv3's average duration of a dispatch over the kernel's own execution span (first wave's start to last wave's
-# end, printed by this script as roofline.execution_span), both from the one rocprofv3 run of the default command
-# whose summary is profiles/lm_step_kernel_trace.txt: 46.744 us / 36.391 us for the weight-gradient product,
-# 35.889 / 30.888 for the input-gradient product.  Between runs and boxes the ratio moves by about +-3 %.
-DISPATCH_OVER_EXECUTION_SPAN = {"gemm_bf16_128x128_rc_rc": 46.744 / 36.391, "gemm_bf16_128x64_kc_rc": 35.889 / 30.888}
+def _variant_of(kernel: str):
+    """Library name of a product kernel (gemm_bf16_128x64_kc_rc ...) from the symbol rocprofv3 prints for
+    rtp::gemm_dma_kernel<T, BM, BN, A k-contiguous, B k-contiguous, ...>; None for anything else."""
+    import re
+    m = re.search(r"gemm_dma_kernelI(DF16b|f)Li(\d+)ELi(\d+)ELb([01])ELb([01])E", kernel)
+    if not m:
+        return None
+    return "gemm_%s_%sx%s_%s_%s" % ("bf16" if m.group(1) == "DF16b" else "f32", m.group(2), m.group(3),
+                                    "kc" if m.group(4) == "1" else "rc", "kc" if m.group(5) == "1" else "rc")
+
+
+def _table_rows(path):
+    """(header comment lines, {variant: last-column-by-name dict}) of one summary under profiles/: a '#' header, one line
+    of column names, then one row per kernel whose numeric columns are the trailing fields."""
+    head, cols, rows = [], None, {}
+    with open(path) as f:
+        for line in f:
+            if line.startswith("#"):
+                head.append(line[1:].strip())
+                continue
+            fields = line.split()
+            if cols is None:
+                cols = fields[1:]
+                continue
+            v = _variant_of(line)
+            if v is None or len(fields) < len(cols) + 1:
+                continue
+            try:
+                rows[v] = dict(zip(cols, (float(x) for x in fields[-len(cols):])))
+            except ValueError:
+                continue
+    return head, rows
+
+
+def profile_reference(variant: str) -> dict:
+    """What the committed rocprofv3 summaries of this script's LM step say about one product variant: memory-side
+    traffic per dispatch (FETCH_SIZE / WRITE_SIZE runs, already scaled by the copy-kernel factors stated in the file),
+    rocprofv3's average dispatch duration, and the kernel's own execution span that this script printed in that same
+    profiled run (the `bench_json` header line).  Missing files or rows give None entries: nothing is assumed."""
+    ref = {"traffic_bytes": None, "rocprof_avg_us": None, "execution_span_us": None, "dispatch_over_execution_span": None,
+           "source": ["profiles/lm_step_pmc_fetch_write.txt", "profiles/lm_step_kernel_trace.txt"]}
+    try:
+        _, rows = _table_rows(os.path.join(PROFILES, "lm_step_pmc_fetch_write.txt"))
+        if variant in rows and "traffic_KiB" in rows[variant]:
+            ref["traffic_bytes"] = rows[variant]["traffic_KiB"] * 1024.0
+    except OSError:
+        pass
+    try:
+        head, rows = _table_rows(os.path.join(PROFILES, "lm_step_kernel_trace.txt"))
+        if variant in rows and "avg_us" in rows[variant]:
+            ref["rocprof_avg_us"] = rows[variant]["avg_us"]
+        for line in head:
+            if line.startswith("bench_json:"):
+                span = json.loads(line[len("bench_json:"):]).get("execution_span_us", {}).get(variant)
+                if span:
+                    ref["execution_span_us"] = float(span)
+        if ref["rocprof_avg_us"] and ref["execution_span_us"]:
+            ref["dispatch_over_execution_span"] = ref["rocprof_avg_us"] / ref["execution_span_us"]
+    except (OSError, ValueError):
+        pass
+    return ref
 
 
 def step_flops(c):
@@ -70,15 +118,15 @@ def build(c, device, dtype):
 
 
 def cpu_baseline(c, steps=5, warmup=2):
-    """The oracle LM (stock nn.Embedding / nn.MultiheadAttention / nn.Linear / nn.LayerNorm, fp32) on the host
-    cores: same shapes, same step (zero grads, fwd, CE, bwd, clip, SGD).  It is the UNSHARDED stock model, which
-    does the same arithmetic as the reference's shard loop without its per-shard launches and concatenations."""
+    """The oracle LM on the host cores, evaluated the reference's way: every rotated layer a loop over its `shards`
+    shards (per-shard F.linear / F.embedding / attention, outputs concatenated or summed), fp32, same shapes, same
+    step (zero grads, fwd, CE, bwd, clip, SGD)."""
     import torch
     import torch.nn.functional as F
     from oracle import rtp_oracle as O
 
     torch.manual_seed(0)
-    ref = O.TransformerLM(c["vocab"], c["ninp"], c["nhead"], c["nhid"], c["layers"])
+    ref = O.TransformerLM(c["vocab"], c["ninp"], c["nhead"], c["nhid"], c["layers"], ws=c["shards"], shard_loop=True)
     with torch.no_grad():
         for n, p in ref.named_parameters():
             if "norm" not in n:
@@ -105,7 +153,8 @@ def cpu_baseline(c, steps=5, warmup=2):
     dt = sorted(times)[len(times) // 2]
     return {"value": c["seq"] * c["batch"] / dt, "unit": "tokens/s", "cores": torch.get_num_threads(),
             "kind": "port", "sample": f"median of {steps} full steps of the same configuration after {warmup} warm-ups, "
-            f"fp32, unsharded stock model ({dt * 1e3:.0f} ms/step, os.cpu_count()={os.cpu_count()})"}
+            f"fp32, every rotated layer looped over its {c['shards']} shards as the reference does ({dt * 1e3:.0f} ms/step, "
+            f"os.cpu_count()={os.cpu_count()})"}
 
 
 def _time_cpu(one, steps):
@@ -225,9 +274,34 @@ def gemm_workload(shape, operands, engine, steps, warmup):
                       "config": {"workload": f"one product {m}x{n}x{k}, {operands} operands, engine {engine}"}}))
 
 
-def layer_workload(name, steps, warmup, graph=True, cpu=True):
+def linear_ring_baseline():
+    """BASELINE configuration 1 the way the reference runs it: two gloo ranks on the host cores, each with half of the
+    batch rows and one home shard, the shards (and their gradients) travelling the ring.  The rank processes are
+    started by this call, which must come before this process has touched the GPU."""
+    import torch
+    from oracle import gloo_ring
+    gen = torch.Generator().manual_seed(0)
+    w = torch.rand(2048, 2048, generator=gen) * 0.2 - 0.1
+    x_cpu, g_cpu = torch.randn(1024, 2048, generator=gen), torch.randn(1024, 2048, generator=gen)
+    threads = max(1, torch.get_num_threads() // 2)
+    # gloo announces its connections on stdout, in the rank processes: for the duration of the ring, file descriptor
+    # 1 (which they inherit) is stderr, so that this script's stdout stays the one JSON line
+    sys.stdout.flush()
+    saved = os.dup(1)
+    os.dup2(2, 1)
+    try:
+        res = gloo_ring.column_linear_ring(x_cpu, w, torch.zeros(2048), g_cpu, ws=2, steps=5, warmup=2,
+                                           threads_per_rank=threads)
+    finally:
+        sys.stdout.flush()
+        os.dup2(saved, 1)
+        os.close(saved)
+    return (sorted(res["times"])[2], 2 * threads, "median of 5 fwd+bwd passes after 2 warm-ups, 2 gloo ranks on loopback")
+
+
+def layer_workload(name, steps, warmup, graph=True, cpu=True, ring_result=None):
     """The reference's other configurations (single rotated layers), fwd+bwd, timed with the same event
-    bracketing; one JSON line with the layer's own algorithmic work and the dominant kernel's roofline."""
+    bracketing; returns the JSON record with the layer's own algorithmic work and the dominant kernel's roofline."""
     import torch
     import torch.nn as nn
     from rtp_amd import _lib, emulate_shards
@@ -237,22 +311,13 @@ def layer_workload(name, steps, warmup, graph=True, cpu=True):
     def uni(*shape):
         return torch.rand(*shape, generator=gen) * 0.2 - 0.1
 
-    ring_result = None
     if name == "linear":
         master = nn.Linear(2048, 2048)
         with torch.no_grad():
             master.weight.copy_(uni(2048, 2048)), master.bias.zero_()
         x_cpu, g_cpu = torch.randn(1024, 2048, generator=gen), torch.randn(1024, 2048, generator=gen)
-        if cpu:
-            # The reference's own execution of this configuration: two gloo ranks on the host cores, each with half
-            # of the batch rows and one home shard, the shards (and their gradients) travelling the ring.  The rank
-            # processes are started here, before this process has touched the GPU.
-            from oracle import gloo_ring
-            threads = max(1, torch.get_num_threads() // 2)
-            res = gloo_ring.column_linear_ring(x_cpu, master.weight.detach(), master.bias.detach(), g_cpu, ws=2,
-                                               steps=5, warmup=2, threads_per_rank=threads)
-            ring_result = (sorted(res["times"])[2], 2 * threads,
-                           "median of 5 fwd+bwd passes after 2 warm-ups, 2 gloo ranks on loopback")
+        if cpu and ring_result is None:
+            ring_result = linear_ring_baseline()   # same seed, same draws: identical operands
 
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
@@ -438,7 +503,7 @@ def layer_workload(name, steps, warmup, graph=True, cpu=True):
         sec, cores, sample = cpu_fn()
         out["cpu_baseline"] = {"value": sec * 1e3, "unit": "ms", "cores": cores, "kind": "port",
                                "sample": f"{sample} (os.cpu_count()={os.cpu_count()})"}
-    print(json.dumps(out))
+    return out
 
 
 def main():
@@ -480,6 +545,11 @@ def main():
                     help="--workload gemm: this library's product kernel, or torch.matmul (the vendor library) as the "
                          "yardstick on the same data")
     ap.add_argument("--shape", default="4096x4096x4096", help="--workload gemm: MxNxK of y[M,N] = x[M,K] w[N,K]^T")
+    ap.add_argument("--lm-only", action="store_true",
+                    help="--workload lm: only the headline step (the default run then also times the same step under the "
+                         "staged rotation and the reference's four single-layer configurations, after the timed region); "
+                         "what the rocprofv3 summaries of the LM step are collected with, so that their per-kernel "
+                         "averages hold the step's dispatches only")
     ap.add_argument("--no-graph", dest="graph", action="store_false",
                     help="launch every kernel eagerly instead of replaying the step from a captured HIP graph")
     args = ap.parse_args()
@@ -492,8 +562,11 @@ def main():
         gemm_workload(args.shape, args.operands, args.engine, args.steps, args.warmup)
         return
     if args.workload != "lm":
-        layer_workload(args.workload, args.steps, args.warmup, args.graph, not args.no_cpu_baseline)
+        print(json.dumps(layer_workload(args.workload, args.steps, args.warmup, args.graph, not args.no_cpu_baseline)))
         return
+    whole = not args.lm_only
+    # the gloo ranks of configuration 1's CPU baseline are started before this process touches the GPU
+    ring_result = linear_ring_baseline() if whole and not args.no_cpu_baseline else None
 
     import torch
     import torch.nn.functional as F
@@ -533,35 +606,36 @@ def main():
         opt.step()
         loss_box[0] = loss.detach()  # detached: a live autograd graph would pin last step's AccumulateGrad nodes
 
-    # Warm-up on a side stream (the documented recipe for whole-step graph capture: autograd's gradient
-    # accumulators remember the stream they were created on, and it must not be the default stream).
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        for _ in range(max(args.warmup, 1)):
-            step()
-    torch.cuda.current_stream().wait_stream(side)
-    torch.cuda.synchronize()
-    ring.fence(dev)
-    first_loss = float(loss_box[0])
-
-    run = step
-    if args.graph:
-        # The whole step (both streams of the rotation included) recorded once into a HIP graph and replayed.
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
-            step()
-        ring.fence(dev)  # the ring's last fence was recorded inside the capture; re-arm it for eager use
-        run = g.replay
-        run()
+    def timed(n_warm, n_steps):
+        """(seconds per step, the replayed graph or None): warm-up on a side stream (the documented recipe for
+        whole-step graph capture: autograd's gradient accumulators remember the stream they were created on, and it
+        must not be the default stream), the whole step -- both streams of the rotation included -- recorded once into a
+        HIP graph, then n_steps replays bracketed by device synchronisations."""
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(max(n_warm, 1)):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
+        ring.fence(dev)
+        first = float(loss_box[0])
+        run, g = step, None
+        if args.graph:
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                step()
+            ring.fence(dev)  # the ring's last fence was recorded inside the capture; re-arm it for eager use
+            run = g.replay
+            run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n_steps):
+            run()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n_steps, g, first
 
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        run()
-    torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / args.steps
+    dt, g, first_loss = timed(args.warmup, args.steps)
     last_loss = float(loss_box[0])
 
     # The dominant kernel in the TIMED mode (graph replay, both streams live): the step is captured a second time
@@ -614,10 +688,11 @@ def main():
     span_us = dom["total_ms"] / dom["launches"] * 1e3
     # rocprofv3 reports a longer duration for the same dispatches than the kernel's own first-wave-to-last-wave span:
     # its clock starts when the queue reaches the dispatch, and the workgroups then still wait for the CUs that the
-    # other stream's product holds.  The ratio of the two was measured in the rocprofv3 run of this very command
-    # (profiles/lm_step_kernel_trace.txt: average duration / the span this script printed in that run); the roofline
-    # figure is quoted on the longer, rocprofv3-compatible span.
-    ratio = DISPATCH_OVER_EXECUTION_SPAN.get(dom_name, 1.0) if graph_stats is not None else 1.0
+    # other stream's product holds.  The ratio of the two is read from the committed rocprofv3 summary of this very
+    # command (profiles/lm_step_kernel_trace.txt: the kernel's average duration / the span this script printed in
+    # that run); the roofline figure is quoted on the longer, rocprofv3-compatible span.
+    prof_ref = profile_reference(dom_name)
+    ratio = (prof_ref["dispatch_over_execution_span"] or 1.0) if graph_stats is not None else 1.0
     avg_ms = span_us * ratio * 1e-3
     achieved = dom["flops"] / dom["launches"] / (avg_ms * 1e-3) / 1e12
     # Which roof bounds the kernel: the larger of its two minimum times, flops at the MFMA peak or algorithmic bytes
@@ -667,15 +742,21 @@ def main():
                    "wgrad_on_second_stream": bool(args.wgrad_overlap),
                    "next_layer_shards_read_ahead_into_cache": bool(ring.warm_ahead())},
         "roofline": dict(roof,
-                     traffic=(MEASURED_TRAFFIC_KIB[dom_name] * 1024.0 if dom_name in MEASURED_TRAFFIC_KIB else None),
+                     traffic=prof_ref["traffic_bytes"],
                      **{
-                     "traffic_unit": "bytes per launch (counter runs, see profiles/)",
-                     "algorithmic_bytes_per_launch": alg_bytes, "kernel": dom_name,
+                     "traffic_unit": "bytes per launch, read from the committed counter summary (not measured in this run)",
+                     "from_profiles": prof_ref,
+                     "algorithmic_bytes_per_launch": alg_bytes,
+                     "algorithmic_bytes_formula": "per launch: (A rows x K + B rows x K) x 2 B, an operand that all shards "
+                                                  "of the launch share counted once, + M x N x (output + addend + fused "
+                                                  "update: 4 B master read, 4 B written, 2 B weight copy) ; averaged over "
+                                                  "the launches of this variant in a step",
+                     "kernel": dom_name,
                      "avg_launch_us": avg_ms * 1e3,
                      "launches_per_step": dom["launches"] // (5 if graph_stats is not None else prof_steps),
                      "flops_per_launch": dom["flops"] / dom["launches"],
                      "timed_in": ("HIP-graph replay of the step, both streams live: device time stamps per launch, times the "
-                                  "measured ratio of rocprofv3's dispatch duration to that span"
+                                  "ratio of rocprofv3's dispatch duration to that span in the committed profile"
                                   if graph_stats is not None else "eager launches, HIP events"),
                      "dispatch_over_execution_span": ratio,
                      "execution_span": span,
@@ -697,6 +778,40 @@ def main():
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(c)
+    if whole and args.rotation == "direct":
+        # The same step under the staged rotation: every window of shards copied home -> HBM slot by the copy kernel on
+        # a side stream while the previous window's products read the other slot (the double buffer a multi-GPU ring
+        # would fill from its neighbour).  Same model, same optimiser state layout, same timing recipe.
+        ring.set_rotation_mode("staged")
+        ring.set_warm_ahead(False)
+        dt_s, g_s, _ = timed(2, args.steps)
+        _lib.profile_enable(True)
+        step()
+        torch.cuda.synchronize()
+        copy_s = _lib.profile_collect().get("shard_copy")
+        _lib.profile_enable(False)
+        staged = staging_bytes(dev)
+        out["staged_rotation"] = {
+            "ms_per_step": dt_s * 1e3, "tokens_per_s": tokens / dt_s, "staging_bytes": staged,
+            "ratio_weights_plus_staging_to_model": (rotated_weight_bytes(lm) + staged) / rotated_weight_bytes(lm),
+            "shard_copy_launches_per_step": None if copy_s is None else copy_s["launches"],
+            "shard_copy_gbs": None if copy_s is None else copy_s["bytes"] / copy_s["total_ms"] / 1e6,
+            "shard_copy_gbs_what": "bytes read + written by the copy kernel / its HIP-event time, one eager step",
+            "hip_graph": bool(args.graph)}
+        del g_s
+        ring.set_rotation_mode("direct")
+        ring.set_warm_ahead(args.warm_ahead)
+    if whole:
+        # The reference's other four configurations, one rotated layer each, fwd+bwd, same timing recipe.
+        del g, lm, opt
+        torch.cuda.empty_cache()
+        others = {}
+        for name in ("linear", "embedding", "attention", "moe"):
+            r = layer_workload(name, args.steps, args.warmup, args.graph, not args.no_cpu_baseline, ring_result)
+            others[name] = {"workload": r["config"]["workload"], "ms": r["value"], "dtype": r["dtype"],
+                            "roofline": r["roofline"], "whole_layer": r["whole_layer"],
+                            "cpu_baseline": r.get("cpu_baseline")}
+        out["other_configs"] = others
     print(json.dumps(out))
 
 

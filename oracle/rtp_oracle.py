@@ -27,7 +27,8 @@ float32 unless the caller passes float64 tensors.  How each function is pinned (
   TransformerLM (with and without MoE blocks)    == golden vectors written from the reference's own TransformerLM run on
                                                     a 2-rank gloo ring (tests/golden/lm_ws2.npz, lm_moe_ws2.npz: logits,
                                                     losses, l_aux and every home-shard gradient), plus parameter count
-                                                    and causality
+                                                    and causality; shard_loop=True (the per-shard loops of the
+                                                    functions above inside the model) == shard_loop=False
 """
 from __future__ import annotations
 
@@ -352,8 +353,9 @@ class _DecoderLayer(nn.Module):
     `experts[e]` = (linear1, linear2); the routing noise is the attribute `noise` ([S, E], zeros if unset -- with two
     experts the noise cannot change the routing) and the layer keeps `l_aux` as the reference's moe_layer does."""
 
-    def __init__(self, ninp, nhead, nhid, num_experts=0, ws=1):
+    def __init__(self, ninp, nhead, nhid, num_experts=0, ws=1, shard_loop=False):
         super().__init__()
+        self.nhead, self.shard_loop = nhead, shard_loop
         self.self_attn = nn.MultiheadAttention(ninp, nhead, dropout=0.0)
         self.norm1 = nn.LayerNorm(ninp)
         self.norm2 = nn.LayerNorm(ninp)
@@ -368,6 +370,9 @@ class _DecoderLayer(nn.Module):
 
     def _ff(self, x):
         if not self.num_experts:
+            if self.shard_loop:      # FeedForwardLayer of two ColumnParallelLinear (transformer_lm_rtp.py:82-89)
+                h = F.relu(column_parallel_linear(x, self.linear1.weight, self.linear1.bias, self.ws))
+                return column_parallel_linear(h, self.linear2.weight, self.linear2.bias, self.ws)
             return self.linear2(F.relu(self.linear1(x)))
         S = x.shape[0] * x.shape[1]
         noise = self.noise if self.noise is not None else torch.zeros(S, self.num_experts, dtype=x.dtype)
@@ -378,24 +383,38 @@ class _DecoderLayer(nn.Module):
     def forward(self, x):
         L = x.shape[0]
         mask = torch.triu(torch.full((L, L), float("-inf"), dtype=x.dtype), diagonal=1)      # :201-204
-        x = self.norm1(x + self.self_attn(x, x, x, attn_mask=mask, need_weights=False)[0])
+        if self.shard_loop:          # ParallelMultiheadAttention's loop over head groups (attention.py:240-267)
+            a = self.self_attn
+            sa = parallel_multihead_attention(x, a.in_proj_weight, a.in_proj_bias, a.out_proj.weight, a.out_proj.bias,
+                                              self.nhead, self.ws, mask=mask)[0]
+        else:
+            sa = self.self_attn(x, x, x, attn_mask=mask, need_weights=False)[0]
+        x = self.norm1(x + sa)
         return self.norm2(x + self._ff(x))
 
 
 class TransformerLM(nn.Sequential):
     """Unsharded LM with the rotated LM's structure; weights are copied in by the tests so both sides
     start from identical values.  num_experts > 0 builds the is_moe=True model (one gate + `num_experts` experts per
-    decoder layer, `ws` shards in the MoE layer's ring order)."""
+    decoder layer, `ws` shards in the MoE layer's ring order).  shard_loop=True evaluates every rotated layer the way
+    the reference does -- a loop over `ws` shards per layer with the per-shard F.linear / F.embedding / attention and the
+    concatenation or running sum of the partial results -- on the same unsharded parameters: the same function, in the
+    reference's operation count (what bench.py times as the CPU baseline)."""
 
-    def __init__(self, ntokens, ninp, nhead, nhid, ndecoder, num_experts=0, ws=1):
-        self.ninp = ninp
+    def __init__(self, ntokens, ninp, nhead, nhid, ndecoder, num_experts=0, ws=1, shard_loop=False):
+        self.ninp, self.ws, self.shard_loop = ninp, ws, shard_loop
         layers = [nn.Embedding(ntokens, ninp), _PositionalEncoding(ninp)]
-        layers += [_DecoderLayer(ninp, nhead, nhid, num_experts, ws) for _ in range(ndecoder)]
+        layers += [_DecoderLayer(ninp, nhead, nhid, num_experts, ws, shard_loop) for _ in range(ndecoder)]
         layers.append(nn.Linear(ninp, ntokens))
         super().__init__(*layers)
 
     def forward(self, ids):
-        x = self[0](ids) * math.sqrt(self.ninp)                               # :29
-        for layer in list(self)[1:]:
+        if self.shard_loop:
+            x = parallel_embedding(ids, self[0].weight, self.ws) * math.sqrt(self.ninp)
+        else:
+            x = self[0](ids) * math.sqrt(self.ninp)                           # :29
+        for layer in list(self)[1:-1]:
             x = layer(x)
-        return x
+        if self.shard_loop:                                                   # LinearLayer = ColumnParallelLinear, :223
+            return column_parallel_linear(x, self[-1].weight, self[-1].bias, self.ws)
+        return self[-1](x)

@@ -262,6 +262,23 @@ def test_transformer_lm_structure_and_param_count():
     torch.testing.assert_close(small(ids2)[:5], out[:5])
 
 
+@pytest.mark.parametrize("ws", [2, 4])
+def test_transformer_lm_shard_loop_equals_the_unsharded_model(ws):
+    """The model evaluated the reference's way (every rotated layer a loop over its shards) is the same function of
+    the same parameters: logits, loss and every gradient agree with the stock layers at fp32 defaults."""
+    torch.manual_seed(ws)
+    a = O.TransformerLM(48, 16, 4, 24, 2)
+    b = O.TransformerLM(48, 16, 4, 24, 2, ws=ws, shard_loop=True)
+    b.load_state_dict(a.state_dict())
+    ids, tgt = torch.randint(0, 48, (7, 3)), torch.randint(0, 48, (7, 3))
+    la, lb = a(ids), b(ids)
+    torch.testing.assert_close(lb, la)
+    torch.nn.functional.cross_entropy(la.view(-1, 48), tgt.view(-1)).backward()
+    torch.nn.functional.cross_entropy(lb.view(-1, 48), tgt.view(-1)).backward()
+    for (n, pa), (_, pb) in zip(a.named_parameters(), b.named_parameters()):
+        torch.testing.assert_close(pb.grad, pa.grad, msg=lambda m, n=n: f"{n}: {m}")
+
+
 @pytest.mark.parametrize("ws", [1, 2, 4])
 @pytest.mark.parametrize("stride,padding,dilation", [(1, 0, 1), (2, 1, 1), ((1, 2), (2, 0), (2, 1))])
 def test_column_conv2d_matches_unsharded_conv_and_patch_product(ws, stride, padding, dilation):
