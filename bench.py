@@ -662,9 +662,11 @@ def main():
             torch.cuda.synchronize()
             t_i += time.perf_counter() - t1
             for k, v in _lib.profile_collect(clear=False).items():
-                acc = graph_stats.setdefault(k, {"launches": 0, "total_ms": 0.0, "flops": 0.0, "bytes": 0.0})
-                for f in acc:
+                acc = graph_stats.setdefault(k, {"launches": 0, "total_ms": 0.0, "flops": 0.0, "bytes": 0.0,
+                                                 "phase_ms": [0.0] * 4})
+                for f in ("launches", "total_ms", "flops", "bytes"):
                     acc[f] += v[f]
+                acc["phase_ms"] = [a + b for a, b in zip(acc["phase_ms"], v["phase_ms"])]
         instr_ms = t_i / reps * 1e3
         _lib.profile_collect()
         del g2
@@ -722,7 +724,12 @@ def main():
                    "gbs": round(v["bytes"] / max(v["total_ms"], 1e-9) / 1e6, 1)} for k, v in sorted(stats.items())}
     graph_gemms = None if graph_stats is None else {
         k: {"launches_per_step": v["launches"] // 5, "avg_launch_us": round(v["total_ms"] / v["launches"] * 1e3, 3),
-            "tflops": round(v["flops"] / max(v["total_ms"], 1e-9) / 1e9, 2)} for k, v in sorted(graph_stats.items())}
+            "tflops": round(v["flops"] / max(v["total_ms"], 1e-9) / 1e9, 2),
+            # a workgroup's time, averaged over the workgroups of a launch and over the launches: waiting for a CU after
+            # the launch's first workgroup started, entry -> first operands in LDS, the K loop, the epilogue
+            "workgroup_phases_us": dict(zip(("wait_for_cu", "to_first_slab", "k_loop", "epilogue"),
+                                            (round(x / v["launches"] * 1e3, 2) for x in v["phase_ms"])))}
+        for k, v in sorted(graph_stats.items())}
 
     flops = step_flops(c)
     peaks = attainable_peaks(dev)

@@ -672,12 +672,17 @@ typedef struct {
   double total_ms;
   double flops; /* algorithmic, summed over launches */
   double bytes; /* algorithmic, summed over launches */
+  /* mode 2, wave-specialised product kernels only (else 0): where a workgroup's time goes, each entry the average over
+   * the launch's workgroups, summed over launches: [0] launch start -> the workgroup's own start (waiting for a CU),
+   * [1] its start -> first operands visible in LDS, [2] the K loop, [3] the epilogue */
+  double phase_ms[4];
 } rtp_kernel_stat;
 
 int rtp_profile_enable(int mode); /* 0 off, 1 HIP events around every launch, 2 device time stamps (see below) */
 /* Mode 2 is for launches recorded into a HIP graph, where timing events do not work: every rtp_gemm launch made
  * while it is on carries the address of a two-word slot in device memory, where its workgroups leave the earliest
- * start and the latest end of the device's constant-rate wall clock, at every replay.  rtp_profile_reset_stamps
+ * start and the latest end of the device's constant-rate wall clock (and the per-workgroup phase sums behind
+ * rtp_kernel_stat.phase_ms), at every replay.  rtp_profile_reset_stamps
  * (a small kernel on `stream`) clears the slots before a replay; rtp_profile_read after it returns that replay's
  * durations per kernel variant.  Other kernels are not timed in this mode. */
 int rtp_profile_reset_stamps(void* stream);

@@ -77,7 +77,7 @@ class RotatedLinearBwdArgs(C.Structure):
 
 class KernelStat(C.Structure):
     _fields_ = [("name", C.c_char * 64), ("launches", C.c_int64), ("total_ms", C.c_double),
-                ("flops", C.c_double), ("bytes", C.c_double)]
+                ("flops", C.c_double), ("bytes", C.c_double), ("phase_ms", C.c_double * 4)]
 
 
 _vp, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
@@ -231,4 +231,4 @@ def profile_collect(clear: bool = True):
     lib = load()
     check((lib.rtp_profile_collect if clear else lib.rtp_profile_read)(buf, 64, C.byref(n)))
     return {buf[i].name.decode(): {"launches": buf[i].launches, "total_ms": buf[i].total_ms, "flops": buf[i].flops,
-                                   "bytes": buf[i].bytes} for i in range(n.value)}
+                                   "bytes": buf[i].bytes, "phase_ms": list(buf[i].phase_ms)} for i in range(n.value)}

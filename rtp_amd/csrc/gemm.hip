@@ -869,8 +869,8 @@ __device__ __forceinline__ Frag<T> read_frag_dma(const char* st, int rowbase, in
   return u.f;
 }
 
-template <typename T, int BM, int BN, bool AKC, bool BKC, int NSTAGE, int SB, int PD>
-__global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
+template <typename T, int BM, int BN, bool AKC, bool BKC, int NSTAGE, int SB, int PD, int OCC = 2>
+__global__ __launch_bounds__(512, OCC) void gemm_dma_kernel(GemmArgs p) {
   constexpr int NL = 4;  // loader waves (waves 4..7); waves 0..3 compute
   using DA = DmaOperand<T, BM, AKC, NL, SB>;
   using DB = DmaOperand<T, BN, BKC, NL, SB>;
@@ -889,7 +889,11 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
 
   touch_kernel_arguments<sizeof(GemmArgs)>();
   const int tid = threadIdx.x;
-  if (p.trace != nullptr && tid == 0) atomicMin(p.trace, (unsigned long long)wall_clock64());
+  unsigned long long t_start = 0, t_ready = 0, t_loop = 0;  // phase stamps of thread 0 (an MFMA wave), mode 2 only
+  if (p.trace != nullptr && tid == 0) {
+    t_start = (unsigned long long)wall_clock64();
+    atomicMin(p.trace, t_start);
+  }
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = (wave >> 1) & 1, wn = wave & 1;
@@ -1112,6 +1116,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
       }
     }
     __builtin_amdgcn_s_barrier();  // barrier 0
+    if (p.trace != nullptr && tid == 0) t_ready = (unsigned long long)wall_clock64();
     [&]<int... Q>(std::integer_sequence<int, Q...>) {
       (read_step(std::integral_constant<int, 0>{}, std::integral_constant<int, Q>{}, std::integral_constant<int, Q>{}),
        ...);
@@ -1120,6 +1125,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
     int kt = 0;
     for (; kt + NSTAGE < nk; kt += NSTAGE) round(kt, std::true_type{});
     for (; kt < nk; kt += NSTAGE) round(kt, std::false_type{});
+    if (p.trace != nullptr && tid == 0) t_loop = (unsigned long long)wall_clock64();
   }
   const bool computes = wave < 4;
   if (computes && p.a_rowsum != nullptr && tile_n == 0 && wn == 0) {
@@ -1155,7 +1161,15 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
     finish_tile_xent_stats<T, BM, BN, 512>(p, ct, m0, n0, tid, grp);
   else
     finish_tile<T, BM, BN, 512>(p, ct, m0, n0, tid, grp, zo, zi);
-  if (p.trace != nullptr && tid == 0) atomicMax(p.trace + 1, (unsigned long long)wall_clock64());
+  if (p.trace != nullptr && tid == 0) {
+    const unsigned long long t_end = (unsigned long long)wall_clock64();
+    atomicMax(p.trace + 1, t_end);
+    atomicAdd(p.trace + 2, t_start);
+    atomicAdd(p.trace + 3, t_ready - t_start);
+    atomicAdd(p.trace + 4, t_loop - t_ready);
+    atomicAdd(p.trace + 5, t_end - t_loop);
+    atomicAdd(p.trace + 6, 1ull);
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1404,7 +1418,7 @@ static int launch_dma8(hipStream_t s, const GemmArgs& a, bool akc, bool bkc, dim
   return RTP_OK;
 }
 
-template <typename T, int BM, int BN, int NSTAGE, int SB, int PD>
+template <typename T, int BM, int BN, int NSTAGE, int SB, int PD, int OCC = 2>
 static int launch_dma(hipStream_t s, const GemmArgs& a, bool akc, bool bkc, dim3 grid) {
   const dim3 block(512);
   // A row-contiguous operand is staged as k lines of R elements, and a 1 KiB load must cover whole lines (or a
@@ -1414,20 +1428,20 @@ static int launch_dma(hipStream_t s, const GemmArgs& a, bool akc, bool bkc, dim3
     RTP_REQUIRE((akc || A_RC_OK) && (bkc || B_RC_OK), "gemm: tile %d x %d needs K-contiguous operands", BM, BN);
     if constexpr (!B_RC_OK && A_RC_OK) {
       if (akc)
-        hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, true, NSTAGE, SB, PD>), grid, block, 0, s, a);
+        hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, true, NSTAGE, SB, PD, OCC>), grid, block, 0, s, a);
       else
-        hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, true, NSTAGE, SB, PD>), grid, block, 0, s, a);
+        hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, true, NSTAGE, SB, PD, OCC>), grid, block, 0, s, a);
     }
     RTP_LAUNCH_CHECK();
     return RTP_OK;
   } else if (akc && bkc)
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, true, NSTAGE, SB, PD>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, true, NSTAGE, SB, PD, OCC>), grid, block, 0, s, a);
   else if (akc && !bkc)
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, false, NSTAGE, SB, PD>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, false, NSTAGE, SB, PD, OCC>), grid, block, 0, s, a);
   else if (!akc && bkc)
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, true, NSTAGE, SB, PD>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, true, NSTAGE, SB, PD, OCC>), grid, block, 0, s, a);
   else
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, false, NSTAGE, SB, PD>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, false, NSTAGE, SB, PD, OCC>), grid, block, 0, s, a);
   RTP_LAUNCH_CHECK();
   return RTP_OK;
 }
@@ -1512,9 +1526,9 @@ struct TileShape {
   int bm, bn;
   const char* tag;
 };
-static const TileShape kShapes[6] = {{256, 128, "256x128"}, {128, 128, "128x128"}, {128, 64, "128x64"}, {64, 64, "64x64"},
-                                     {128, 192, "128x192"}, {256, 256, "256x256"}};
-constexpr int kNumShapes = 6;
+static const TileShape kShapes[7] = {{256, 128, "256x128"}, {128, 128, "128x128"}, {128, 64, "128x64"}, {64, 64, "64x64"},
+                                     {128, 192, "128x192"}, {256, 256, "256x256"}, {128, 64, "128x64c"}};
+constexpr int kNumShapes = 7;
 
 // One wavefront per 32 x 32 block is the better kernel for one attention head at sequence length <= 64.
 static bool is_tiny(const rtp_gemm_desc* d) { return d->m <= 64 && d->n <= 64 && d->k * d->ksegs <= 256; }
@@ -1669,8 +1683,12 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
     const char* e = getenv("RTP_GEMM_TILE");  // debugging aid: index into kShapes
     return e ? atoi(e) : -1;
   }();
-  static const double slab_ns[kNumShapes] = {966.0, 470.0, 283.0, 167.0, 800.0, 1680.0};
-  static const int slab_bytes[kNumShapes] = {128, 128, 128, 128, 128, 128};
+  static const double slab_ns[kNumShapes] = {966.0, 470.0, 283.0, 167.0, 800.0, 1680.0, 283.0};
+  static const int slab_bytes[kNumShapes] = {128, 128, 128, 128, 128, 128, 128};
+  static const int co = [] {
+    const char* e = getenv("RTP_GEMM_CO");  // experiment: co-resident 128 x 64 kernel instead of 128x64 (1) / also 128x128 (2)
+    return e ? atoi(e) : 0;
+  }();
   int shape = 3;  // 64 x 64 unless the model finds something cheaper
   double best = 0.0;
   for (int i = 0; fast && i < kNumShapes; ++i) {
@@ -1680,6 +1698,7 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
     // -10 % on the MoE layer's time; a loss where it leaves CUs without a tile or K is shorter)
     // (its epilogue is the plain one: the update and the statistics epilogue are never routed to it, forced or not)
     if (i == 5 && (sizeof(T) != 2 || d->sgd_master || d->xent_mode == 1)) continue;
+    if (i == 6 && i != forced) continue;
     if (i == 5 && (ceil_div(d->m, 256) * ceil_div(d->n, 256) * nz < 256 || d->k * d->ksegs < 1024) && i != forced)
       continue;
     // never a tile that is mostly padding: a 32 x 32 problem (one attention head at seq 32) stays at 64 x 64
@@ -1694,6 +1713,7 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
       shape = i;
     }
   }
+  if (fast && sizeof(T) == 2 && ((co >= 1 && shape == 2) || (co >= 2 && shape == 1))) shape = 6;
   const TileShape& ts = kShapes[shape];
   a.tiles_m = (int)ceil_div(d->m, ts.bm);
   a.tiles_n = (int)ceil_div(d->n, ts.bn);
@@ -1805,6 +1825,8 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
       return launch_dma<T, 128, 64, 5, 128, 4>(s, a, akc, bkc, grid);
     case 4:
       return launch_dma<T, 128, 192, 3, 128, 2>(s, a, akc, bkc, grid);
+    case 6:
+      return launch_dma<T, 128, 64, 3, 128, 1, 4>(s, a, akc, bkc, grid);
     case 5:
       if constexpr (sizeof(T) == 2) return launch_dma8<T, 2, 128, 1>(s, a, akc, bkc, grid);
       return fail(RTP_ERR_ARG, "gemm: no 256 x 256 kernel for this dtype");

@@ -29,6 +29,10 @@ static std::vector<ProfileRecord> g_profile_records;
 // (atomic max).  The slot address is a kernel argument, so a launch recorded into a HIP graph stamps its slot at
 // every replay -- which HIP timing events recorded during a capture do not do.
 constexpr int kTraceSlots = 8192;
+// Words of a slot: earliest start, latest end, then sums over the launch's workgroups of the wall-clock ticks from the
+// launch's... (see ProfileScope::trace_slot): [2] workgroup start, [3] entry -> first operands in LDS, [4] the K loop,
+// [5] the epilogue, [6] the number of workgroups that reported.
+constexpr int kTraceWords = 8;
 static unsigned long long* g_trace_buf = nullptr;
 static int g_trace_next = 0;
 
@@ -64,14 +68,15 @@ unsigned long long* ProfileScope::trace_slot() {
   if (!g_trace_buf || g_trace_next >= kTraceSlots) return nullptr;
   const int slot = g_trace_next++;
   g_profile_records.push_back({nullptr, nullptr, slot, name_, flops_, bytes_});
-  return g_trace_buf + 2 * (size_t)slot;
+  return g_trace_buf + kTraceWords * (size_t)slot;
 }
 
 __global__ void trace_reset_kernel(unsigned long long* buf, int slots) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < slots) {
-    buf[2 * i] = ~0ull;
-    buf[2 * i + 1] = 0ull;
+    buf[kTraceWords * i] = ~0ull;
+#pragma unroll
+    for (int w = 1; w < kTraceWords; ++w) buf[kTraceWords * i + w] = 0ull;
   }
 }
 
@@ -193,7 +198,7 @@ using namespace rtp;
 
 extern "C" const char* rtp_last_error(void) { return error_buffer(); }
 
-extern "C" int rtp_abi_version(void) { return 3; }
+extern "C" int rtp_abi_version(void) { return 4; }
 
 extern "C" int rtp_device_check(char* name_out, int name_len) {
   int dev = 0;
@@ -324,7 +329,7 @@ extern "C" int rtp_profile_enable(int mode) {
   RTP_REQUIRE(mode >= 0 && mode <= 2, "rtp_profile_enable: mode 0 (off), 1 (events) or 2 (device time stamps)");
   std::lock_guard<std::mutex> lock(g_profile_mutex);
   if (mode == 2 && !g_trace_buf) {
-    RTP_HIP_TRY(hipMalloc((void**)&g_trace_buf, sizeof(unsigned long long) * 2 * kTraceSlots));
+    RTP_HIP_TRY(hipMalloc((void**)&g_trace_buf, sizeof(unsigned long long) * kTraceWords * kTraceSlots));
     hipLaunchKernelGGL(trace_reset_kernel, dim3((kTraceSlots + 255) / 256), dim3(256), 0, nullptr, g_trace_buf, kTraceSlots);
     RTP_LAUNCH_CHECK();
     RTP_HIP_TRY(hipDeviceSynchronize());
@@ -352,7 +357,7 @@ static int profile_sum(rtp_kernel_stat* out, int max_out, int* n_out, bool clear
   std::vector<unsigned long long> stamps;
   double ticks_per_ms = 1e5;  // the wall clock runs at 100 MHz unless the device says otherwise
   if (g_trace_buf && g_trace_next > 0) {
-    stamps.resize(2 * (size_t)g_trace_next);
+    stamps.resize((size_t)kTraceWords * g_trace_next);
     RTP_HIP_TRY(hipMemcpy(stamps.data(), g_trace_buf, stamps.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost));
     int dev = 0, khz = 0;
     if (hipGetDevice(&dev) == hipSuccess &&
@@ -362,10 +367,17 @@ static int profile_sum(rtp_kernel_stat* out, int max_out, int* n_out, bool clear
   std::map<std::string, rtp_kernel_stat> agg;
   for (const ProfileRecord& r : g_profile_records) {
     float ms = 0.0f;
+    double phase[4] = {0.0, 0.0, 0.0, 0.0};
     if (r.slot >= 0) {
-      const unsigned long long t0 = stamps[2 * (size_t)r.slot], t1 = stamps[2 * (size_t)r.slot + 1];
+      const unsigned long long* w = &stamps[(size_t)kTraceWords * r.slot];
+      const unsigned long long t0 = w[0], t1 = w[1];
       if (t1 < t0) continue;  // the launch did not run since the last reset
       ms = (float)((double)(t1 - t0) / ticks_per_ms);
+      if (w[6] > 0) {  // per-workgroup phases, averaged over the workgroups of the launch
+        const double n = (double)w[6];
+        phase[0] = ((double)w[2] / n - (double)t0) / ticks_per_ms;
+        for (int i = 1; i < 4; ++i) phase[i] = (double)w[2 + i] / n / ticks_per_ms;
+      }
     } else {
       if (hipEventElapsedTime(&ms, r.start, r.stop) != hipSuccess) ms = 0.0f;
       if (clear) {
@@ -382,6 +394,7 @@ static int profile_sum(rtp_kernel_stat* out, int max_out, int* n_out, bool clear
     st.total_ms += ms;
     st.flops += r.flops;
     st.bytes += r.bytes;
+    for (int i = 0; i < 4; ++i) st.phase_ms[i] += phase[i];
   }
   if (clear) {
     g_profile_records.clear();
