@@ -468,6 +468,36 @@ __device__ __forceinline__ void store8(T* dst, const float (&v)[8], bool stream)
   }
 }
 
+// Raw 16-byte-vector image of 8 consecutive epilogue operand values (c_in in `dtype` or fp32, bias, gate): what a thread
+// requests for all of its chunks before it consumes any of them.
+template <typename T>
+struct Raw8 {
+  uint4 q[sizeof(T) == 2 ? 1 : 2];
+  __device__ __forceinline__ void load(const T* src) {
+    q[0] = reinterpret_cast<const uint4*>(src)[0];
+    if (sizeof(T) == 4) q[sizeof(T) == 2 ? 0 : 1] = reinterpret_cast<const uint4*>(src)[1];
+  }
+  __device__ __forceinline__ void get(float (&v)[8]) const {
+    if (sizeof(T) == 2) {
+      union {
+        uint4 q;
+        T e[8];
+      } u;
+      u.q = q[0];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = to_f32(u.e[e]);
+    } else {
+      union {
+        uint4 q[2];
+        float f[8];
+      } u;
+      u.q[0] = q[0], u.q[1] = q[sizeof(T) == 2 ? 0 : 1];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = u.f[e];
+    }
+  }
+};
+
 template <typename T, int BM, int BN, int NTHR>
 __device__ __forceinline__ void finish_tile(const GemmArgs& p, const float* ct, int m0, int n0, int tid, int grp,
                                             long zo, long zi) {
@@ -488,6 +518,78 @@ __device__ __forceinline__ void finish_tile(const GemmArgs& p, const float* ct, 
   float* master = p.sgd_master ? p.sgd_master + zoff : nullptr;
   T* wcopy = p.sgd_w ? reinterpret_cast<T*>(p.sgd_w) + zoff : nullptr;
   const bool skip_out = p.flags & RTP_GEMM_SGD_SKIP_OUT;
+
+  if constexpr (CHUNKS % NTHR == 0) {
+    // The common form (vector-aligned operands, one bias vector): a thread requests the bias, the addend and the mask
+    // of ALL its chunks before it consumes the first -- one trip to memory for the whole epilogue instead of one per
+    // chunk (a store to c_out may alias a later chunk's c_in as far as the compiler knows, so left alone the loads of
+    // chunk i + 1 wait behind the store of chunk i).  When the thread count is a multiple of the chunks per row all of
+    // a thread's chunks lie in the same 8 columns and share one bias vector.
+    if (p.vec_c && nb_seg == 1 && p.xent_mode == 0 && master == nullptr) {
+      constexpr int NCH = CHUNKS / NTHR;
+      constexpr bool SAMECOL = NTHR % CPR == 0;
+      constexpr int NB = SAMECOL ? 1 : NCH;
+      Raw8<T> rb[NB], rg[NCH], rc16[NCH];
+      Raw8<float> rc32[NCH];
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) {
+        const int c = tid + i * NTHR;
+        const int row = m0 + c / CPR, col = n0 + (c % CPR) * 8;
+        const int colc = col < p.n ? col : 0;
+        const long rowc = row < p.m ? row : p.m - 1;
+        if (bias && (i == 0 || !SAMECOL)) rb[SAMECOL ? 0 : i].load(bias + colc);
+        if (cin) {
+          if (cin_f32)
+            rc32[i].load(reinterpret_cast<const float*>(cin) + rowc * p.ld_cin + colc);
+          else
+            rc16[i].load(reinterpret_cast<const T*>(cin) + rowc * p.ld_cin + colc);
+        }
+        if (gate) rg[i].load(gate + rowc * p.ld_gate + colc);
+      }
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) {
+        const int c = tid + i * NTHR;
+        const int lr = c / CPR, lc = (c % CPR) * 8;
+        const int row = m0 + lr, col = n0 + lc;
+        const bool col_ok = col < p.n;
+        float v[8], t[8];
+        const float4 lo = *reinterpret_cast<const float4*>(ct + lr * CP + lc);
+        const float4 hi = *reinterpret_cast<const float4*>(ct + lr * CP + lc + 4);
+        v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w, v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] *= p.alpha;
+        if (cin) {
+          if (cin_f32)
+            rc32[i].get(t);
+          else
+            rc16[i].get(t);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] += t[e];
+        }
+        if (bias) {
+          rb[SAMECOL ? 0 : i].get(t);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] += t[e];
+        }
+        if (relu) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] = fmaxf(v[e], 0.0f);
+        }
+        if (gate) {
+          rg[i].get(t);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] = t[e] > 0.0f ? v[e] : 0.0f;
+        }
+        if (row >= p.m || !col_ok) continue;
+        const long off = (long)row * p.ldc + col;
+        if (out_f32)
+          store8(reinterpret_cast<float*>(cbase) + off, v, stream_out);
+        else
+          store8(reinterpret_cast<T*>(cbase) + off, v, stream_out);
+      }
+      return;
+    }
+  }
 
   for (int c = tid; c < CHUNKS; c += NTHR) {
     const int lr = c / CPR, lc = (c % CPR) * 8;
