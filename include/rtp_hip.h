@@ -365,6 +365,22 @@ int rtp_embedding_scatter_add_sgd(void* stream, int dtype, const void* grad_out,
                                   int64_t groups, int64_t grad_out_sg, int64_t grad_table_sg, float grad_scale,
                                   float* master, void* weights, float lr, float clip, int store_grad);
 
+/* The backward of F.embedding in ONE launch, straight from the token ids (reference: the autograd backward of
+ * rtp/module/embedding.py:146, there a dense zeros + index_add_ per shard): the arguments and results of
+ * rtp_embedding_scatter_add_scaled / _sgd (same order of summation, bit for bit) without the sort and without a
+ * separate fill.  Every workgroup keeps the step's ids in LDS; the workgroup of token position t sums the upstream rows
+ * of all positions that name the same id, ascending, if t is the first of them, for all `groups` shards; with
+ * zero_fill the rows that no token names are cleared by further workgroups of the same launch.  master == NULL: the
+ * gradient is written (zero_fill != 0: overwriting, else added to what is there); master != NULL: the update of
+ * rtp_embedding_scatter_add_sgd (weights may be NULL; store_grad as there).  At most 4096 ids
+ * (rtp_embedding_backward_supported); longer steps take rtp_embedding_sort_ids + rtp_embedding_scatter_add_*. */
+int rtp_embedding_backward_supported(int64_t n_ids);
+int rtp_embedding_backward(void* stream, int dtype, const void* grad_out, int64_t ld_grad_out, int64_t n_ids,
+                           const int64_t* ids, void* grad_table, int64_t ld_grad_table, int grad_table_f32,
+                           int64_t row_begin, int64_t row_count, int64_t cols, int64_t padding_idx, int scale_by_freq,
+                           int zero_fill, int64_t groups, int64_t grad_out_sg, int64_t grad_table_sg, float grad_scale,
+                           float* master, void* weights, float lr, float clip, int store_grad);
+
 /* ---------------------------------------------------------------------------------------------
  * Attention softmax (reference: rtp/module/functional.py:779-792 baddbmm+softmax, :825
  * scaled_dot_product_attention with an additive float mask).

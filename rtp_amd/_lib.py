@@ -123,6 +123,9 @@ PROTOTYPES = {
                                               _i64, _i, _i, _i64, _i64, _i64, _f]),
     "rtp_embedding_scatter_add_sgd": (_i, [_vp, _i, _vp, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i, _i64,
                                            _i64, _i64, _f, _vp, _vp, _f, _f, _i]),
+    "rtp_embedding_backward_supported": (_i, [_i64]),
+    "rtp_embedding_backward": (_i, [_vp, _i, _vp, _i64, _i64, _vp, _vp, _i64, _i, _i64, _i64, _i64, _i64, _i, _i, _i64,
+                                    _i64, _i64, _f, _vp, _vp, _f, _f, _i]),
     "rtp_softmax_fwd": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _i64, _i, _f, _i64, _i64, _i64, _vp]),
     "rtp_softmax_fwd_masks": (_i, [_vp, _i, _vp, _vp, _i64, _vp, _i64, _i64, _i, _f, _i64, _i64, _i64, _vp, _vp, _vp]),
     "rtp_softmax_bwd": (_i, [_vp, _i, _vp, _vp, _vp, _f, _i64, _i64, _i64, _vp]),

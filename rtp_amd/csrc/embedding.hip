@@ -163,6 +163,171 @@ __global__ __launch_bounds__(256) void scatter_kernel(const T* grad_out, long ld
   }
 }
 
+// V consecutive elements of type X as floats and back; V > 1 means whole 16-byte vectors (the caller checked alignment).
+template <typename X, int V>
+__device__ __forceinline__ void vec_load(const X* p, float (&f)[V]) {
+  if constexpr (V == 1) {
+    f[0] = to_f32(p[0]);
+  } else {
+    constexpr int NQ = V * (int)sizeof(X) / 16;
+    union {
+      uint4 q[NQ];
+      X e[V];
+    } u;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) u.q[q] = reinterpret_cast<const uint4*>(p)[q];
+#pragma unroll
+    for (int v = 0; v < V; ++v) f[v] = to_f32(u.e[v]);
+  }
+}
+template <typename X, int V>
+__device__ __forceinline__ void vec_store(X* p, const float (&f)[V]) {
+  if constexpr (V == 1) {
+    p[0] = from_f32<X>(f[0]);
+  } else {
+    constexpr int NQ = V * (int)sizeof(X) / 16;
+    union {
+      uint4 q[NQ];
+      X e[V];
+    } u;
+#pragma unroll
+    for (int v = 0; v < V; ++v) u.e[v] = from_f32<X>(f[v]);
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) reinterpret_cast<uint4*>(p)[q] = u.q[q];
+  }
+}
+
+// The whole backward of the sharded embedding in ONE launch, for steps of up to kBwdMaxIds tokens: no sort.  Every
+// workgroup stages the step's ids in LDS.  Workgroup t < n owns token position t: if an earlier position names the
+// same id it leaves at once; otherwise it marks the later positions with that id in an LDS bitmap, lists them in
+// ascending order and sums their upstream rows front to back, starting from +0.0f with position t -- the order of a
+// sequential index_add_ into a zeroed table, for all shards (groups) of the layer.  With a zero fill requested the
+// grid has further workgroups, one per block of table rows: each finds the rows of its block that no token names
+// (bitmap over the same ids) and clears them; rows that are named are written in full by their token workgroup, so
+// nothing is written twice and no ordering between the two kinds of workgroup is needed.
+constexpr int kBwdMaxIds = 4096;
+template <typename T, typename G, int V>
+__global__ __launch_bounds__(256) void embedding_bwd_kernel(const T* grad_out, long ld_go, int n, const int64_t* ids,
+                                                            G* grad_table, long ld_gt, long row_begin, long row_count,
+                                                            long cols, long padding_idx, int scale_by_freq,
+                                                            int overwrite, int groups, long go_sg, long gt_sg,
+                                                            float grad_scale, float* master, T* weights, float lr,
+                                                            float clip, int store_grad, int zero_rows) {
+  __shared__ int s_ids[kBwdMaxIds];
+  __shared__ unsigned s_bits[kBwdMaxIds / 32];
+  __shared__ int s_count;
+  const int tid = threadIdx.x;
+  for (int i = tid; i < n; i += 256) s_ids[i] = (int)ids[i];
+  for (int i = tid; i < kBwdMaxIds / 32; i += 256) s_bits[i] = 0u;
+  __syncthreads();
+  if ((long)blockIdx.x >= n) {
+    // ---- rows that no token names: cleared ----
+    const long r0 = ((long)blockIdx.x - n) * zero_rows;
+    for (int i = tid; i < n; i += 256) {
+      const int id = s_ids[i];
+      const long r = (long)id - row_begin - r0;
+      if (id != padding_idx && r >= 0 && r < zero_rows) atomicOr(&s_bits[r >> 5], 1u << (r & 31));
+    }
+    __syncthreads();
+    const long per_row = cols / V;  // vectors of a row in one group
+    const long total = (long)zero_rows * groups * per_row;
+    for (long e = tid; e < total; e += 256) {
+      const long r = e / (groups * per_row), rem = e - r * (groups * per_row);
+      const long g = rem / per_row, c = (rem - g * per_row) * V;
+      if (r0 + r >= row_count || ((s_bits[r >> 5] >> (r & 31)) & 1u)) continue;
+      G* dst = grad_table + g * gt_sg + (r0 + r) * ld_gt + c;
+      if (V == 1) {
+        dst[0] = from_f32<G>(0.0f);
+      } else {
+        constexpr int NQ = V * (int)sizeof(G) / 16;
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) reinterpret_cast<uint4*>(dst)[q] = make_uint4(0u, 0u, 0u, 0u);
+      }
+    }
+    return;
+  }
+  // ---- token position t ----
+  const int t = blockIdx.x;
+  const int id = s_ids[t];
+  const long row = (long)id - row_begin;
+  if (id == padding_idx || row < 0 || row >= row_count) return;
+  int early = 0;
+  for (int j = tid; j < t; j += 256) early |= (s_ids[j] == id) ? 1 : 0;
+  if (__syncthreads_or(early)) return;  // an earlier position owns this id
+  for (int j = t + tid; j < n; j += 256)
+    if (s_ids[j] == id) atomicOr(&s_bits[j >> 5], 1u << (j & 31));
+  __syncthreads();
+  if (tid == 0) {
+    // the positions with this id, ascending, written over the ids (which nobody reads any more)
+    int cnt = 0;
+    for (int w = t >> 5; w < (n + 31) / 32; ++w) {
+      unsigned bits = s_bits[w];
+      while (bits) {
+        const int b = __builtin_ctz(bits);
+        bits &= bits - 1;
+        s_ids[cnt++] = w * 32 + b;
+      }
+    }
+    s_count = cnt;
+  }
+  __syncthreads();
+  const int cnt = s_count;
+  const float inv = scale_by_freq ? 1.0f / (float)cnt : 1.0f;
+  const long per_row = cols / V;
+  for (long e = tid; e < (long)groups * per_row; e += 256) {
+    const long g = e / per_row, c = (e - g * per_row) * V;
+    const T* src = grad_out + g * go_sg + c;
+    float acc[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) acc[v] = 0.0f;
+    for (int k = 0; k < cnt; ++k) {
+#pragma clang fp contract(off)
+      const T* sp = src + (long)s_ids[k] * ld_go;
+      union {
+        uint4 q;
+        T e[16 / sizeof(T)];
+      } u;
+      if (V == 1)
+        u.e[0] = sp[0];
+      else
+        u.q = *reinterpret_cast<const uint4*>(sp);
+#pragma unroll
+      for (int v = 0; v < V; ++v) {
+        // grad_scale != 1: the upstream gradient of a scaled embedding, T(grad * scale), rounded as the separate
+        // multiplication would round it before it joins the sum (no fused multiply-add)
+        const float x = grad_scale == 1.0f ? to_f32(u.e[v]) : to_f32(from_f32<T>(to_f32(u.e[v]) * grad_scale));
+        acc[v] += x;
+      }
+    }
+    const long off = g * gt_sg + row * ld_gt + c;
+    {
+#pragma clang fp contract(off)
+      if (scale_by_freq) {
+#pragma unroll
+        for (int v = 0; v < V; ++v) acc[v] *= inv;
+      }
+      if (master != nullptr) {
+        // clip + SGD where the row's gradient is produced (the caller guarantees it is the row's whole gradient)
+        float w[V];
+        vec_load<float, V>(master + off, w);
+#pragma unroll
+        for (int v = 0; v < V; ++v) w[v] = sgd_update<G>(w[v], acc[v], lr, clip);
+        vec_store<float, V>(master + off, w);
+        if (weights != nullptr) vec_store<T, V>(weights + off, w);
+        if (store_grad) vec_store<G, V>(grad_table + off, acc);
+        continue;
+      }
+      if (!overwrite) {
+        float old[V];
+        vec_load<G, V>(grad_table + off, old);
+#pragma unroll
+        for (int v = 0; v < V; ++v) acc[v] = old[v] + acc[v];
+      }
+      vec_store<G, V>(grad_table + off, acc);
+    }
+  }
+}
+
 struct SortLayout {
   size_t keys_in, vals_in, keys_out, vals_out, temp, total, temp_bytes;
 };
@@ -376,4 +541,68 @@ extern "C" int rtp_embedding_scatter_add_sgd(void* stream, int dtype, const void
   return scatter_impl(stream, dtype, grad_out, ld_grad_out, n_ids, workspace, grad_table, ld_grad_table, 0, row_begin,
                       row_count, cols, padding_idx, scale_by_freq, store_grad ? 1 : 0, groups, grad_out_sg,
                       grad_table_sg, grad_scale, master, dtype == RTP_F32 ? nullptr : weights, lr, clip, store_grad);
+}
+
+extern "C" int rtp_embedding_backward_supported(int64_t n_ids) { return n_ids >= 0 && n_ids <= kBwdMaxIds ? 1 : 0; }
+
+extern "C" int rtp_embedding_backward(void* stream, int dtype, const void* grad_out, int64_t ld_grad_out, int64_t n_ids,
+                                      const int64_t* ids, void* grad_table, int64_t ld_grad_table, int grad_table_f32,
+                                      int64_t row_begin, int64_t row_count, int64_t cols, int64_t padding_idx,
+                                      int scale_by_freq, int zero_fill, int64_t groups, int64_t grad_out_sg,
+                                      int64_t grad_table_sg, float grad_scale, float* master, void* weights, float lr,
+                                      float clip, int store_grad) {
+  RTP_REQUIRE(grad_out && grad_table && (ids || n_ids == 0), "rtp_embedding_backward: null pointer");
+  RTP_REQUIRE(rtp_embedding_backward_supported(n_ids), "rtp_embedding_backward: %lld ids, at most %d (sort + scatter beyond)",
+              (long long)n_ids, kBwdMaxIds);
+  RTP_REQUIRE(dtype == RTP_F32 || dtype == RTP_BF16, "rtp_embedding_backward: unknown dtype %d", dtype);
+  RTP_REQUIRE(groups >= 1 && groups < 65536, "rtp_embedding_backward: groups %lld not in 1..65535", (long long)groups);
+  RTP_REQUIRE(cols >= 0 && ld_grad_out >= cols && ld_grad_table >= cols && row_count >= 0 && row_count < (1ll << 31),
+              "rtp_embedding_backward: bad shape");
+  if (master != nullptr) {
+    RTP_REQUIRE(!grad_table_f32 || dtype == RTP_F32, "rtp_embedding_backward: with an update the gradient table has the table's dtype");
+    RTP_REQUIRE(dtype != RTP_F32 || weights == nullptr || weights == (void*)master,
+                "rtp_embedding_backward: fp32 tables are their own master");
+    RTP_REQUIRE(zero_fill || !store_grad, "rtp_embedding_backward: a stored gradient beside the update starts from a zero fill");
+    if (!store_grad) zero_fill = 0;  // the update replaces the dense gradient: nothing to fill
+    if (dtype == RTP_F32) weights = nullptr;
+  } else {
+    store_grad = 1;
+  }
+  if (cols == 0 || row_count == 0 || (n_ids == 0 && !zero_fill)) return RTP_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const size_t esz = dtype == RTP_F32 ? 4 : 2, gsz = (dtype == RTP_F32 || grad_table_f32) ? 4 : 2;
+  // 16-byte accesses when every row of every operand allows them
+  const int64_t vec = 16 / (int64_t)esz;
+  const bool aligned = cols % vec == 0 && (uintptr_t)grad_out % 16 == 0 && (ld_grad_out * esz) % 16 == 0 &&
+                       (grad_out_sg * esz) % 16 == 0 && (uintptr_t)grad_table % 16 == 0 &&
+                       (ld_grad_table * gsz) % 16 == 0 && (grad_table_sg * gsz) % 16 == 0 &&
+                       (master == nullptr || (uintptr_t)master % 16 == 0) &&
+                       (weights == nullptr || (uintptr_t)weights % 16 == 0);
+  // a zero-fill workgroup clears about 64 KiB: a block of rows over all groups
+  int64_t zero_rows = 0, zero_wgs = 0;
+  if (zero_fill) {
+    zero_rows = std::max<int64_t>(1, std::min<int64_t>(kBwdMaxIds, 65536 / std::max<int64_t>(1, groups * cols * (int64_t)gsz)));
+    zero_wgs = ceil_div(row_count, zero_rows);
+  }
+  RTP_REQUIRE(n_ids + zero_wgs < (1ll << 31), "rtp_embedding_backward: grid too large");
+  const dim3 grid((unsigned)(n_ids + zero_wgs));
+  // algorithmic bytes: every upstream row read once, every named row written (or read, modified and written) once;
+  // the fill of the rows nobody names is extra
+  ProfileScope prof(s, "embedding_backward", (double)groups * n_ids * cols,
+                    (double)groups * n_ids * cols * (esz + (zero_fill || master ? 1.0 : 2.0) * gsz) + 8.0 * n_ids);
+#define RTP_EMB_BWD(T, G, V)                                                                                          \
+  hipLaunchKernelGGL((embedding_bwd_kernel<T, G, V>), grid, dim3(256), 0, s, (const T*)grad_out, (long)ld_grad_out,    \
+                     (int)n_ids, ids, (G*)grad_table, (long)ld_grad_table, (long)row_begin, (long)row_count, (long)cols, \
+                     (long)padding_idx, scale_by_freq, zero_fill ? 1 : 0, (int)groups, (long)grad_out_sg,               \
+                     (long)grad_table_sg, grad_scale, master, (T*)weights, lr, clip, store_grad, (int)zero_rows)
+  if (dtype == RTP_F32) {
+    if (aligned) RTP_EMB_BWD(float, float, 4); else RTP_EMB_BWD(float, float, 1);
+  } else if (grad_table_f32) {
+    if (aligned) RTP_EMB_BWD(bf16_t, float, 8); else RTP_EMB_BWD(bf16_t, float, 1);
+  } else {
+    if (aligned) RTP_EMB_BWD(bf16_t, bf16_t, 8); else RTP_EMB_BWD(bf16_t, bf16_t, 1);
+  }
+#undef RTP_EMB_BWD
+  RTP_LAUNCH_CHECK();
+  return RTP_OK;
 }

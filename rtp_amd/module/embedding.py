@@ -72,7 +72,10 @@ class _EmbeddingFn(torch.autograd.Function):
         g2 = dout.reshape(-1, layer.embedding_dim)
         if g2.stride(1) != 1:
             g2 = g2.contiguous()
-        workspace = ops.embedding_sort_ids(flat_ids)
+        # up to a few thousand tokens: one launch per run of shards, from the raw ids; longer steps sort the ids once
+        # and scatter-add per run
+        onepass = ops.embedding_backward_supported(flat_ids.numel())
+        workspace = None if onepass else ops.embedding_sort_ids(flat_ids)
         pad = -1 if layer.padding_idx is None else layer.padding_idx
         if store.on_backward is not None:
             store.on_backward(store)
@@ -82,10 +85,13 @@ class _EmbeddingFn(torch.autograd.Function):
             # an optimiser that applies its update where gradients are produced: the rows the step's tokens name are
             # updated by the scatter-add itself, the dense [V, D/ws] gradient is neither zero-filled nor written
             kw = _fused(store, accumulate, first, cnt, store.offsets[0], store.numels[0])
-            ops.embedding_scatter_add(g2[:, first * d_s:(first + 1) * d_s], flat_ids.numel(), workspace, table,
-                                      padding_idx=pad, scale_by_freq=layer.scale_grad_by_freq,
-                                      zero_fill=not accumulate, groups=cnt, grad_out_sg=d_s,
-                                      grad_table_sg=store.grads.shape[1], grad_scale=ctx.grad_scale, **kw)
+            common = dict(padding_idx=pad, scale_by_freq=layer.scale_grad_by_freq, zero_fill=not accumulate, groups=cnt,
+                          grad_out_sg=d_s, grad_table_sg=store.grads.shape[1], grad_scale=ctx.grad_scale, **kw)
+            if onepass:
+                ops.embedding_backward(g2[:, first * d_s:(first + 1) * d_s], flat_ids, table, **common)
+            else:
+                ops.embedding_scatter_add(g2[:, first * d_s:(first + 1) * d_s], flat_ids.numel(), workspace, table,
+                                          **common)
             _fused_done(store, kw)
         store.grads_ready()
         return None, None, None, None, None

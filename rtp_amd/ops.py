@@ -364,6 +364,39 @@ def embedding_sort_ids(ids: torch.Tensor) -> torch.Tensor:
     return ws
 
 
+def embedding_backward_supported(n_ids: int) -> bool:
+    """Whether a step of n_ids tokens fits the one-launch embedding backward (its ids are staged in LDS)."""
+    return bool(_lib.load().rtp_embedding_backward_supported(int(n_ids)))
+
+
+def embedding_backward(grad_out: torch.Tensor, ids: torch.Tensor, grad_table: torch.Tensor, *, row_begin: int = 0,
+                       padding_idx: int = -1, scale_by_freq: bool = False, zero_fill: bool = True, groups: int = 1,
+                       grad_out_sg: int = 0, grad_table_sg: int = 0, grad_scale: float = 1.0,
+                       sgd: Optional["FusedSgd"] = None, sgd_master: int = 0, sgd_weights: int = 0) -> None:
+    """embedding_sort_ids + embedding_scatter_add in one launch, from the raw ids (contiguous int64, one per row of
+    grad_out): same arguments, same results bit for bit; rows no token names are cleared by the same launch when
+    zero_fill.  Only for steps embedding_backward_supported() accepts."""
+    for t in (grad_out, ids, grad_table):
+        _dev(t)
+    n, cols, ld_go = _mat(grad_out, "grad_out")
+    rows, cols_t, ld_gt = _mat(grad_table, "grad_table")
+    if ids.dtype != torch.int64 or not ids.is_contiguous() or ids.numel() != n or cols != cols_t:
+        raise ValueError("embedding_backward: ids must be contiguous int64, one per row of grad_out; tables [rows, cols]")
+    if grad_table.dtype not in (grad_out.dtype, torch.float32):
+        raise TypeError("embedding_backward: grad_table must be the grad dtype or float32")
+    if sgd is not None and (not zero_fill or grad_table.dtype != grad_out.dtype):
+        raise ValueError("embedding_backward: the fused update takes the whole gradient of the step, in the table's "
+                         "own dtype")
+    _lib.require_device()
+    check(_lib.load().rtp_embedding_backward(
+        _stream(), dtype_code(grad_out.dtype), grad_out.data_ptr(), ld_go, n, ids.data_ptr(), grad_table.data_ptr(),
+        ld_gt, int(grad_table.dtype == torch.float32), row_begin, rows, cols,
+        -1 if padding_idx is None else padding_idx, int(scale_by_freq), int(zero_fill), groups, grad_out_sg,
+        grad_table_sg, float(grad_scale), (sgd_master or None) if sgd is not None else None,
+        (sgd_weights or None) if sgd is not None else None, sgd.lr if sgd is not None else 0.0,
+        sgd.clip if sgd is not None else 0.0, int(sgd.keep_grads) if sgd is not None else 1))
+
+
 def embedding_scatter_add(grad_out: torch.Tensor, n_ids: int, workspace: torch.Tensor, grad_table: torch.Tensor,
                           *, row_begin: int = 0, padding_idx: int = -1, scale_by_freq: bool = False,
                           zero_fill: bool = True, groups: int = 1, grad_out_sg: int = 0,

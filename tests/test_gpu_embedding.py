@@ -166,3 +166,41 @@ def test_embedding_update_applied_by_the_scatter_add_is_bit_identical(dtype):
             assert torch.equal(a, b), f"step {step}"
     # the fused twin never filled or wrote its dense gradient table
     assert twins[1][0]._store.fused_sgd is not None
+
+
+@pytest.mark.parametrize("dtype,table_f32", [(torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)])
+@pytest.mark.parametrize("n,vocab,cols,groups", [(1024, 10240, 512, 4), (257, 5, 12, 2), (64, 3, 8, 1), (4096, 50, 24, 3),
+                                                 (1, 9, 7, 1), (300, 40, 33, 2)])
+def test_one_launch_backward_equals_sort_and_scatter(dtype, table_f32, n, vocab, cols, groups):
+    """rtp_embedding_backward (no sort, ids staged in LDS, zero fill in the same launch) against
+    rtp_embedding_sort_ids + rtp_embedding_scatter_add_*: bit for bit, overwriting and accumulating, with a padding
+    id, frequency scaling, a gradient scale, a shard that owns only part of the vocabulary rows, and column counts that
+    are not whole 16-byte vectors (the element-wise form)."""
+    from rtp_amd import ops
+    gen = torch.Generator().manual_seed(n + cols)
+    ids = torch.randint(0, vocab, (n,), generator=gen)
+    if n > 8:
+        ids[n // 2:n // 2 + 3] = ids[0]                                  # repeats far apart
+    g = torch.randn(n, groups * cols, generator=gen).to(dtype).to(DEV)
+    tdt = torch.float32 if table_f32 else dtype
+    row_begin, rows = (vocab // 4, vocab // 2) if vocab >= 8 else (0, vocab)  # a shard of the vocabulary rows
+    start = torch.randn(groups, rows, cols, generator=gen).to(tdt).to(DEV)
+    dev_ids = ids.to(DEV)
+    ws = ops.embedding_sort_ids(dev_ids)
+    for zero_fill, by_freq, scale, pad in ((True, False, 1.0, -1), (False, False, 1.0, int(ids[0])), (True, True, 0.25, -1),
+                                           (False, True, 3.0, int(ids[-1]))):
+        a, b = start.clone(), start.clone()
+        kw = dict(row_begin=row_begin, padding_idx=pad, scale_by_freq=by_freq, zero_fill=zero_fill, groups=groups,
+                  grad_out_sg=cols, grad_table_sg=rows * cols, grad_scale=scale)
+        ops.embedding_scatter_add(g[:, :cols], n, ws, a[0], **kw)
+        ops.embedding_backward(g[:, :cols], dev_ids, b[0], **kw)
+        torch.cuda.synchronize()
+        assert torch.equal(a, b), f"zero_fill={zero_fill} by_freq={by_freq} scale={scale} pad={pad}"
+    assert ops.embedding_backward_supported(4096) and not ops.embedding_backward_supported(4097)
+
+
+def test_long_steps_take_the_sorted_path_and_stay_bit_exact():
+    """More tokens than the one-launch backward stages in LDS: the module sorts the ids once and scatter-adds."""
+    master = nn.Embedding(97, 24)
+    ids = torch.randint(0, 97, (5000,))
+    _check(master, ids, torch.randn(5000, 24), 4)
