@@ -407,7 +407,7 @@ def layer_workload(name, steps, warmup, graph=True, cpu=True, ring_result=None):
         u = torch.rand(4096, 8, generator=gen).clamp(min=torch.finfo(torch.float32).tiny, max=1 - torch.finfo(torch.float32).eps)
         noise_cpu = -torch.log(-torch.log(u))  # Gumbel(0,1) routing noise, drawn on the host
         noise = noise_cpu.to(dev)
-        fn = lambda: (layer(x, noise=noise) * g).sum().backward()
+        fn = lambda: layer(x, noise=noise).backward(g)
 
         def cpu_fn():
             from oracle import rtp_oracle as O

@@ -525,13 +525,14 @@ int rtp_softmax_xent_bwd(void* stream, int dtype, const void* logits, int64_t ld
  *   weight[s,2] fp32 (renormalised gate probabilities, 0 if dropped), gates[S,E] fp32 (softmax),
  *   slot_token[E*C] int32 (token occupying each capacity slot, -1 if empty), l_aux fp32 scalar,
  *   counts[2*E] int32 (first-choice and second-choice totals per expert before the drop).
- * capacity C = 2*S/E; requires S % E == 0 and E <= 64.
+ * capacity C = 2*S/E; requires S % E == 0 and E <= 64.  l_aux_bf16 (may be NULL): a bf16 copy of l_aux for a layer
+ * that runs in bf16 (the reference returns l_aux in the logits' dtype, top2gate.py:105).
  * --------------------------------------------------------------------------------------------- */
 size_t rtp_top2_route_workspace_bytes(int64_t s, int64_t e);
 int rtp_top2_route(void* stream, const float* logits, const float* noise, int64_t s, int64_t e,
                    int32_t* expert, int32_t* slot, int32_t* keep, float* weight, float* gates,
                    int32_t* slot_token, float* l_aux, int32_t* counts, void* workspace,
-                   size_t workspace_bytes);
+                   size_t workspace_bytes, void* l_aux_bf16);
 
 /* Backward of the differentiable part of top2gating: d_logits[S,E] from d_weight[S,2] and the
  * scalar d_l_aux (device pointer, may be NULL for 0). */
@@ -565,7 +566,9 @@ int rtp_moe_combine_dweight(void* stream, int dtype, const void* dout, int64_t l
  * rtp/module/top2gate.py:195-207 -- an nn.Linear without bias whose expert rows are sharded -- and its autograd
  * backward).  With E <= 16 output columns these are streaming passes over the tokens, not tiled products:
  *   fwd:   logits[s][e] = sum_m x[s][m] * w[e][m]                  fp32 logits
- *   dgrad: dx[s][m]     = sum_e dlogits[s][e] * w[e][m]            fp32 dlogits, e ascending, rounded once
+ *   dgrad: dx[s][m]     = sum_e dlogits[s][e] * w[e][m]            fp32 dlogits, e ascending, rounded once; with
+ *          dx_init (may be NULL; `dtype`, may alias dx) dx = dx_init + that, the sum autograd forms where the gradients
+ *          of a tensor's two consumers meet (the MoE layer's tokens feed the gate and the dispatch, moe.py:146-148)
  *   wgrad: dw[e][m]   (+)= sum_s dlogits[s][e] * x[s][m]           partial sums of 64 token rows, then summed in order
  * x [S, M], w and dw [E, M] in `dtype` with element row pitches; rtp_gate_supported says whether (E, M) qualify
  * (E <= 16, M a multiple of 16 bytes); x, w, dx must be 16-byte aligned with pitches that keep rows so.  The rows
@@ -576,7 +579,7 @@ int rtp_gate_supported(int dtype, int64_t experts, int64_t model_dim);
 int rtp_gate_fwd(void* stream, int dtype, const void* x, int64_t ldx, const void* w, int64_t ldw, int64_t S,
                  int64_t M, int64_t E, float* logits, int64_t ld_logits);
 int rtp_gate_dgrad(void* stream, int dtype, const float* dlogits, int64_t ld_dlogits, const void* w, int64_t ldw,
-                   int64_t S, int64_t M, int64_t E, void* dx, int64_t ldx);
+                   int64_t S, int64_t M, int64_t E, void* dx, int64_t ldx, const void* dx_init, int64_t ld_dx_init);
 size_t rtp_gate_wgrad_workspace_bytes(int64_t S, int64_t M, int64_t E);
 int rtp_gate_wgrad(void* stream, int dtype, const float* dlogits, int64_t ld_dlogits, const void* x, int64_t ldx,
                    int64_t S, int64_t M, int64_t E, void* dw, int64_t ld_dw, int accumulate, void* workspace,

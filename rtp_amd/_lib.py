@@ -149,14 +149,14 @@ PROTOTYPES = {
     "rtp_softmax_xent_reduce": (_i, [_vp, _vp, _vp, _i64, _i64, _i, _vp, _vp]),
     "rtp_softmax_xent_bwd": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _i64, _vp, _vp, _i64]),
     "rtp_top2_route_workspace_bytes": (_sz, [_i64, _i64]),
-    "rtp_top2_route": (_i, [_vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz]),
+    "rtp_top2_route": (_i, [_vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "rtp_top2_route_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
     "rtp_moe_dispatch": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64]),
     "rtp_moe_combine": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _i64]),
     "rtp_moe_combine_dweight": (_i, [_vp, _i, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "rtp_gate_supported": (_i, [_i, _i64, _i64]),
     "rtp_gate_fwd": (_i, [_vp, _i, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64]),
-    "rtp_gate_dgrad": (_i, [_vp, _i, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64]),
+    "rtp_gate_dgrad": (_i, [_vp, _i, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _i64]),
     "rtp_gate_wgrad_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "rtp_gate_wgrad": (_i, [_vp, _i, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i, _vp, _sz]),
     "rtp_gate_wgrad_static": (_i, [_vp, _i, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i]),

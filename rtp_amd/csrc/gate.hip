@@ -86,7 +86,7 @@ __device__ __forceinline__ void stage_dl(const float* dl, long ldl, long s0, lon
 // row in registers and walks the token rows of its workgroup's block; dl[s][*] comes from LDS.
 template <typename T, int EB>
 __global__ __launch_bounds__(256) void gate_dgrad_kernel(const float* dl, long ldl, const T* w, long ldw, long S, int M,
-                                                         int E, T* dx, long ldx) {
+                                                         int E, T* dx, long ldx, const T* init, long ld_init) {
   constexpr int VEC = Vec16<T>::N;
   __shared__ float dls[kGateDgradRows][EB];
   const int c = blockIdx.x * 256 + threadIdx.x;
@@ -112,6 +112,14 @@ __global__ __launch_bounds__(256) void gate_dgrad_kernel(const float* dl, long l
     Vec16<T> ov;
 #pragma unroll
     for (int k = 0; k < VEC; ++k) ov.e[k] = from_f32<T>(o[k]);
+    if (init != nullptr) {
+      // the gradient that reached the same input along another path: added as autograd would add the two rounded
+      // tensors (sum of the rounded values, rounded once more)
+      Vec16<T> iv;
+      iv.q = *reinterpret_cast<const uint4*>(init + (s0 + r) * ld_init + c * VEC);
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) ov.e[k] = from_f32<T>(to_f32(iv.e[k]) + to_f32(ov.e[k]));
+    }
     *reinterpret_cast<uint4*>(dx + (s0 + r) * ldx + c * VEC) = ov.q;
   }
 }
@@ -247,7 +255,8 @@ extern "C" int rtp_gate_fwd(void* stream, int dtype, const void* x, int64_t ldx,
 }
 
 extern "C" int rtp_gate_dgrad(void* stream, int dtype, const float* dlogits, int64_t ld_dlogits, const void* w,
-                              int64_t ldw, int64_t S, int64_t M, int64_t E, void* dx, int64_t ldx) {
+                              int64_t ldw, int64_t S, int64_t M, int64_t E, void* dx, int64_t ldx, const void* dx_init,
+                              int64_t ld_dx_init) {
   if (int rc = gate_check("rtp_gate_dgrad", dtype, S, M, E)) return rc;
   const int64_t vec = dtype == RTP_F32 ? 4 : 8;
   RTP_REQUIRE(dlogits && w && dx, "rtp_gate_dgrad: null pointer");
@@ -255,16 +264,20 @@ extern "C" int rtp_gate_dgrad(void* stream, int dtype, const float* dlogits, int
                   ld_dlogits >= E,
               "rtp_gate_dgrad: dx and w must be 16-byte aligned with row pitches >= M that are multiples of %lld",
               (long long)vec);
+  RTP_REQUIRE(dx_init == nullptr || (aligned16(dx_init) && ld_dx_init % vec == 0 && ld_dx_init >= M),
+              "rtp_gate_dgrad: dx_init must be 16-byte aligned with a row pitch >= M that is a multiple of %lld",
+              (long long)vec);
   hipStream_t st = (hipStream_t)stream;
   const double esz = dtype == RTP_F32 ? 4.0 : 2.0;
-  ProfileScope prof(st, "gate_dgrad", 2.0 * S * M * E, esz * ((double)S * M + (double)E * M) + 4.0 * S * E);
+  ProfileScope prof(st, "gate_dgrad", 2.0 * S * M * E,
+                    esz * ((double)S * M * (dx_init ? 2.0 : 1.0) + (double)E * M) + 4.0 * S * E);
   const dim3 grid((unsigned)ceil_div(M / vec, 256), (unsigned)ceil_div(S, kGateDgradRows));
   if (dtype == RTP_F32)
     RTP_GATE_LAUNCH(gate_dgrad_kernel, float, E, grid, st, dlogits, (long)ld_dlogits, (const float*)w, (long)ldw, (long)S,
-                    (int)M, (int)E, (float*)dx, (long)ldx);
+                    (int)M, (int)E, (float*)dx, (long)ldx, (const float*)dx_init, (long)ld_dx_init);
   else
     RTP_GATE_LAUNCH(gate_dgrad_kernel, bf16_t, E, grid, st, dlogits, (long)ld_dlogits, (const bf16_t*)w, (long)ldw,
-                    (long)S, (int)M, (int)E, (bf16_t*)dx, (long)ldx);
+                    (long)S, (int)M, (int)E, (bf16_t*)dx, (long)ldx, (const bf16_t*)dx_init, (long)ld_dx_init);
   RTP_LAUNCH_CHECK();
   return RTP_OK;
 }

@@ -88,7 +88,8 @@ __global__ __launch_bounds__(kTok) void route_choose_kernel(const float* logits,
 // Phase 2 (one workgroup): exclusive scan of the per-workgroup totals per expert, the grand totals and
 // the auxiliary loss  l_aux = mean_e( mean_s gates[s,e] * mean_s [e1(s)==e] ).
 __global__ __launch_bounds__(kMaxExperts) void route_scan_kernel(int* blockcnt, const float* blockgate, long nblocks,
-                                                                 long S, int E, int* counts, float* l_aux) {
+                                                                 long S, int E, int* counts, float* l_aux,
+                                                                 bf16_t* l_aux_bf16) {
   __shared__ float term[kMaxExperts];
   const int e = threadIdx.x;
   if (e < E) {
@@ -112,6 +113,7 @@ __global__ __launch_bounds__(kMaxExperts) void route_scan_kernel(int* blockcnt, 
     float t = 0.0f;
     for (int i = 0; i < E; ++i) t += term[i];
     *l_aux = t / (float)E;
+    if (l_aux_bf16 != nullptr) *l_aux_bf16 = from_f32<bf16_t>(t / (float)E);
   }
 }
 
@@ -267,7 +269,7 @@ extern "C" size_t rtp_top2_route_workspace_bytes(int64_t s, int64_t e) {
 extern "C" int rtp_top2_route(void* stream, const float* logits, const float* noise, int64_t s, int64_t e,
                               int32_t* expert, int32_t* slot, int32_t* keep, float* weight, float* gates,
                               int32_t* slot_token, float* l_aux, int32_t* counts, void* workspace,
-                              size_t workspace_bytes) {
+                              size_t workspace_bytes, void* l_aux_bf16) {
   RTP_REQUIRE(logits && noise && expert && slot && keep && weight && gates && slot_token && l_aux && counts &&
                   workspace,
               "rtp_top2_route: null pointer");
@@ -291,7 +293,7 @@ extern "C" int rtp_top2_route(void* stream, const float* logits, const float* no
                      (int)e, expert, rank, gates, slot_token, blockcnt, blockgate);
   RTP_LAUNCH_CHECK();
   hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(kMaxExperts), 0, st, blockcnt, blockgate, L.nblocks, (long)s,
-                     (int)e, counts, l_aux);
+                     (int)e, counts, l_aux, (bf16_t*)l_aux_bf16);
   RTP_LAUNCH_CHECK();
   hipLaunchKernelGGL(route_finalize_kernel, dim3((unsigned)L.nblocks), dim3(kTok), 0, st, gates, expert, rank,
                      blockcnt, counts, (long)s, (int)e, C, slot, keep, weight, slot_token);

@@ -19,12 +19,39 @@ from ..ring import Rotation, ring_order
 from .collectives import RotatedLayer, resolve_world
 
 
+_JOIN_INPUT_GRADIENTS = True  # False: autograd adds the two input gradients itself (what the tests compare with)
+
+
+class _ForkFn(torch.autograd.Function):
+    """The layer's tokens feed two consumers, the gate projection and the dispatch (rtp/module/moe.py:146-148), and
+    autograd would add their two input gradients with a kernel of its own.  Here both consumers read an alias made by
+    this function and share `box`: the dispatch's backward (which autograd runs first: it was recorded later) leaves its
+    gradient in the box, the gate projection's input-gradient kernel adds it in its epilogue, and this backward passes
+    that sum on.  If the order or the shapes do not allow that, the two gradients are added here."""
+
+    @staticmethod
+    def forward(ctx, x, box):
+        ctx.box = box
+        return x.view_as(x), x.view_as(x)
+
+    @staticmethod
+    def backward(ctx, d_gate, d_dispatch):
+        box = ctx.box
+        box.pop("dx", None)
+        if d_gate is None or d_dispatch is None:
+            return (d_dispatch if d_gate is None else d_gate), None
+        if box.pop("summed", False):
+            return d_gate, None
+        return d_gate + d_dispatch, None
+
+
 class _DispatchFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, routing):
+    def forward(ctx, x, routing, box=None):
         out = torch.empty(routing.e * routing.capacity, x.shape[1], dtype=x.dtype, device=x.device)
         ops.moe_dispatch(x, routing, out)
         ctx.routing = routing
+        ctx.box = box
         return out
 
     @staticmethod
@@ -33,7 +60,9 @@ class _DispatchFn(torch.autograd.Function):
         d_out = d_out if d_out.stride(1) == 1 else d_out.contiguous()
         dx = torch.empty(r.s, d_out.shape[1], dtype=d_out.dtype, device=d_out.device)
         ops.moe_combine(d_out, r, dx, None)
-        return dx, None
+        if ctx.box is not None:
+            ctx.box["dx"] = dx
+        return dx, None, None
 
 
 class _CombineFn(torch.autograd.Function):
@@ -222,9 +251,14 @@ class WeightMOELayer(RotatedLayer):
         reshaped = x.reshape(-1, d_model)
         if reshaped.stride(1) != 1 or (reshaped.shape[0] > 1 and reshaped.stride(0) != d_model):
             reshaped = reshaped.contiguous()
-        routing, weight, l_aux = self.gate.route(reshaped, noise)
-        self.l_aux = l_aux.to(x.dtype)
-        dispatched = _DispatchFn.apply(reshaped, routing)
+        box = None
+        to_gate = to_dispatch = reshaped
+        if _JOIN_INPUT_GRADIENTS and reshaped.requires_grad and torch.is_grad_enabled():
+            box = {}
+            to_gate, to_dispatch = _ForkFn.apply(reshaped, box)
+        routing, weight, l_aux = self.gate.route(to_gate, noise, box)
+        self.l_aux = l_aux
+        dispatched = _DispatchFn.apply(to_dispatch, routing, box)
         expert_out = _ExpertsFn.apply(dispatched, self._anchor, self)
         combined = _CombineFn.apply(expert_out, weight, routing)
         return combined.reshape(x.shape)

@@ -28,28 +28,36 @@ def gumbel_rsample(shape, device: torch.device) -> Tensor:
 
 
 class _RouteFn(torch.autograd.Function):
-    """logits[S,E] (+ noise) -> (weight[S,2], l_aux); the integer routing rides on `holder`."""
+    """logits[S,E] (+ noise) -> (weight[S,2], l_aux); the integer routing rides on `holder`.  l_aux comes out in
+    `l_aux_dtype` (fp32, or bf16 written by the routing kernels themselves: no cast kernel)."""
 
     @staticmethod
-    def forward(ctx, logits, noise, holder):
-        r = ops.top2_route(logits.float().contiguous(), noise.float().contiguous())
+    def forward(ctx, logits, noise, holder, l_aux_dtype):
+        typed = l_aux_dtype if l_aux_dtype == torch.bfloat16 else None
+        r = ops.top2_route(logits.float().contiguous(), noise.float().contiguous(), typed)
         holder.append(r)
         ctx.routing = r
         ctx.in_dtype = logits.dtype
-        return r.weight, r.l_aux
+        ctx.set_materialize_grads(False)  # an unused output (l_aux outside the loss) arrives as None, not as zeros
+        l_aux = r.l_aux_typed if typed is not None else r.l_aux
+        if l_aux.dtype != l_aux_dtype:
+            l_aux = l_aux.to(l_aux_dtype)
+        return r.weight, l_aux
 
     @staticmethod
     def backward(ctx, d_weight, d_l_aux):
+        if d_weight is None and d_l_aux is None:
+            return None, None, None, None
         d_logits = ops.top2_route_bwd(ctx.routing, d_weight, d_l_aux)
-        return d_logits.to(ctx.in_dtype), None, None
+        return (d_logits if d_logits.dtype == ctx.in_dtype else d_logits.to(ctx.in_dtype)), None, None, None
 
 
-def top2_route(logits: Tensor, noise: Optional[Tensor] = None):
-    """Differentiable compact routing: returns (routing, weight[S,2], l_aux)."""
+def top2_route(logits: Tensor, noise: Optional[Tensor] = None, l_aux_dtype: Optional[torch.dtype] = None):
+    """Differentiable compact routing: returns (routing, weight[S,2], l_aux); l_aux in l_aux_dtype (default fp32)."""
     if noise is None:
         noise = gumbel_rsample(logits.shape, logits.device)
     holder = []
-    weight, l_aux = _RouteFn.apply(logits, noise, holder)
+    weight, l_aux = _RouteFn.apply(logits, noise, holder, l_aux_dtype or torch.float32)
     return holder[0], weight, l_aux
 
 
@@ -67,9 +75,9 @@ def dense_from_routing(r: ops.Routing, weight: Tensor, dtype: torch.dtype) -> Tu
 
 def top2gating(logits: Tensor, noise: Optional[Tensor] = None) -> Tuple[Tensor, Tensor, Tensor]:
     """(l_aux, combine_weights, dispatch_mask) as rtp/module/top2gate.py:43-105 returns them."""
-    r, weight, l_aux = top2_route(logits, noise)
+    r, weight, l_aux = top2_route(logits, noise, logits.dtype)
     combine, dispatch = dense_from_routing(r, weight, logits.dtype)
-    return l_aux.to(logits.dtype), combine, dispatch
+    return l_aux, combine, dispatch
 
 
 def _run_rows(flat: Tensor, e_s: int, m: int) -> Optional[Tensor]:
@@ -85,10 +93,14 @@ class _GateProjectionFn(torch.autograd.Function):
     experts take the streaming gate kernels (one pass over the tokens each way), others the tiled product."""
 
     @staticmethod
-    def forward(ctx, x, anchor, layer):
+    def forward(ctx, x, anchor, layer, box=None):
+        """`box` (a dict, optional): where another consumer of the same x leaves its input gradient under "dx" before
+        this backward runs; the input-gradient kernel here then adds it in its epilogue and sets box["summed"], so that
+        whoever joins the two paths hands this one on as their sum (see moe._ForkFn)."""
         store = layer._store
         ws, e_s = layer.world_size, layer.num_local_experts
         x2 = as_rows(x, layer.model_dim)
+        ctx.box = box
         logits = torch.empty(x2.shape[0], layer.num_experts, dtype=torch.float32, device=x2.device)
         rot = Rotation(store.home, ring_order(layer.rank, ws), group=store.stage_group)
         for j in range(rot.steps):
@@ -132,7 +144,13 @@ class _GateProjectionFn(torch.autograd.Function):
                 for flat, first, cnt in rot.acquire(j):
                     rows = _run_rows(flat, e_s, m)
                     if steps == 1 and rows is not None and ops.gate_supported(dx, rows):
-                        ops.gate_dgrad(dl32, first * e_s, rows, dx)   # the only run: dx needs no summing
+                        other = ctx.box.pop("dx", None) if ctx.box is not None else None
+                        if other is not None and (other.shape != dx.shape or other.dtype != dx.dtype or
+                                                  other.stride(1) != 1):
+                            ctx.box["dx"], other = other, None
+                        ops.gate_dgrad(dl32, first * e_s, rows, dx, init=other)   # the only run: dx needs no summing
+                        if other is not None:
+                            ctx.box["summed"] = True
                     else:
                         c_out, c_in = acc.target(i)
                         S.col_dgrad(low(), flat, 0, e_s, m, c_out, first * e_s, c_in=c_in)
@@ -145,7 +163,7 @@ class _GateProjectionFn(torch.autograd.Function):
             else:
                 S.col_wgrad(low(), x2, store.grads, first, 0, e_s, m, first * e_s, cnt, accumulate)
         store.grads_ready()
-        return dx, None, None
+        return dx, None, None, None
 
 
 class Top2Gate(RotatedLayer):
@@ -167,9 +185,9 @@ class Top2Gate(RotatedLayer):
 
     def forward(self, input: Tensor, noise: Optional[Tensor] = None) -> Tuple[Tensor, Tensor, Tensor]:
         logits = _GateProjectionFn.apply(input, self._anchor, self)
-        r, weight, l_aux = top2_route(logits, noise)
+        r, weight, l_aux = top2_route(logits, noise, input.dtype)
         combine, dispatch = dense_from_routing(r, weight, input.dtype)
-        return l_aux.to(input.dtype), combine, dispatch
+        return l_aux, combine, dispatch
 
 
 class WeightTop2Gate(RotatedLayer):
@@ -198,13 +216,14 @@ class WeightTop2Gate(RotatedLayer):
         self.wgs = list(self.shards)
         self.wg = self.wgs[self.rank]
 
-    def logits(self, input: Tensor) -> Tensor:
-        return _GateProjectionFn.apply(input, self._anchor, self)
+    def logits(self, input: Tensor, box=None) -> Tensor:
+        return _GateProjectionFn.apply(input, self._anchor, self, box)
 
-    def route(self, input: Tensor, noise: Optional[Tensor] = None):
-        return top2_route(self.logits(input), noise)
+    def route(self, input: Tensor, noise: Optional[Tensor] = None, box=None):
+        """(routing, weight[S,2], l_aux in the input's dtype)."""
+        return top2_route(self.logits(input, box), noise, input.dtype)
 
     def forward(self, input: Tensor, noise: Optional[Tensor] = None) -> Tuple[Tensor, Tensor, Tensor]:
         r, weight, l_aux = self.route(input, noise)
         combine, dispatch = dense_from_routing(r, weight, input.dtype)
-        return l_aux.to(input.dtype), combine, dispatch
+        return l_aux, combine, dispatch

@@ -809,16 +809,22 @@ def gate_fwd(x2: torch.Tensor, w_rows: torch.Tensor, logits: torch.Tensor, col0:
                                    logits.data_ptr() + 4 * col0, logits.stride(0)))
 
 
-def gate_dgrad(d_logits: torch.Tensor, col0: int, w_rows: torch.Tensor, dx: torch.Tensor) -> None:
-    """dx = d_logits[:, col0 : col0 + E] @ w_rows (d_logits fp32; dx in the weights' dtype, fully overwritten)."""
+def gate_dgrad(d_logits: torch.Tensor, col0: int, w_rows: torch.Tensor, dx: torch.Tensor,
+               init: Optional[torch.Tensor] = None) -> None:
+    """dx = (init +) d_logits[:, col0 : col0 + E] @ w_rows (d_logits fp32; dx in the weights' dtype, fully
+    overwritten; `init`: an addend of dx's shape and dtype, e.g. the gradient that reached the same input along
+    another path -- added to the rounded product and rounded again, as autograd's own sum of the two would be)."""
     _dev(dx)
+    if init is not None and (init.shape != dx.shape or init.dtype != dx.dtype or init.stride(1) != 1):
+        raise ValueError("gate_dgrad: init must match dx")
     if d_logits.dtype != torch.float32 or d_logits.stride(1) != 1 or dx.dtype != w_rows.dtype or dx.stride(1) != 1 or \
             d_logits.shape[0] != dx.shape[0] or dx.shape[1] != w_rows.shape[1]:
         raise ValueError("gate_dgrad: need fp32 d_logits [S, E] and dx [S, M] of the weights' dtype")
     _lib.require_device()
     check(_lib.load().rtp_gate_dgrad(_stream(), dtype_code(dx.dtype), d_logits.data_ptr() + 4 * col0, d_logits.stride(0),
                                      w_rows.data_ptr(), w_rows.stride(0), dx.shape[0], dx.shape[1], w_rows.shape[0],
-                                     dx.data_ptr(), dx.stride(0)))
+                                     dx.data_ptr(), dx.stride(0), _ptr(init),
+                                     init.stride(0) if init is not None else 0))
 
 
 def gate_wgrad(d_logits: torch.Tensor, col0: int, x2: torch.Tensor, dw_rows: torch.Tensor, accumulate: bool) -> None:
@@ -1019,11 +1025,13 @@ class ShardSum:
 class Routing:
     """Compact result of top-2 routing for S tokens over E experts with capacity C = 2S/E."""
 
-    __slots__ = ("s", "e", "capacity", "expert", "slot", "keep", "weight", "gates", "slot_token", "l_aux", "counts")
+    __slots__ = ("s", "e", "capacity", "expert", "slot", "keep", "weight", "gates", "slot_token", "l_aux", "counts",
+                 "l_aux_typed")
 
 
-def top2_route(logits: torch.Tensor, noise: torch.Tensor) -> Routing:
-    """Run the routing kernels on fp32 logits[S,E] and noise[S,E]."""
+def top2_route(logits: torch.Tensor, noise: torch.Tensor, l_aux_dtype: Optional[torch.dtype] = None) -> Routing:
+    """Run the routing kernels on fp32 logits[S,E] and noise[S,E].  l_aux_dtype=torch.bfloat16: the routing also
+    leaves `l_aux_typed`, the auxiliary loss in that dtype (what a bf16 layer hands on), from the same kernels."""
     _dev(logits)
     _dev(noise)
     if logits.dtype != torch.float32 or noise.dtype != torch.float32 or logits.dim() != 2 or \
@@ -1042,17 +1050,21 @@ def top2_route(logits: torch.Tensor, noise: torch.Tensor) -> Routing:
     r.slot_token = torch.empty(2 * s, dtype=torch.int32, device=dev)
     r.l_aux = torch.empty((), dtype=torch.float32, device=dev)
     r.counts = torch.empty(2 * e, dtype=torch.int32, device=dev)
+    r.l_aux_typed = torch.empty((), dtype=torch.bfloat16, device=dev) if l_aux_dtype == torch.bfloat16 else None
     _lib.require_device()
     lib = _lib.load()
     nbytes = lib.rtp_top2_route_workspace_bytes(s, e)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     check(lib.rtp_top2_route(_stream(), logits.data_ptr(), noise.data_ptr(), s, e, r.expert.data_ptr(),
                              r.slot.data_ptr(), r.keep.data_ptr(), r.weight.data_ptr(), r.gates.data_ptr(),
-                             r.slot_token.data_ptr(), r.l_aux.data_ptr(), r.counts.data_ptr(), ws.data_ptr(), nbytes))
+                             r.slot_token.data_ptr(), r.l_aux.data_ptr(), r.counts.data_ptr(), ws.data_ptr(), nbytes,
+                             _ptr(r.l_aux_typed)))
     return r
 
 
-def top2_route_bwd(r: Routing, d_weight: torch.Tensor, d_l_aux: Optional[torch.Tensor]) -> torch.Tensor:
+def top2_route_bwd(r: Routing, d_weight: Optional[torch.Tensor], d_l_aux: Optional[torch.Tensor]) -> torch.Tensor:
+    if d_weight is None:  # only the auxiliary loss was used
+        d_weight = torch.zeros(r.s, 2, dtype=torch.float32, device=r.gates.device)
     d_weight = d_weight.contiguous().float()
     d_logits = torch.empty(r.s, r.e, dtype=torch.float32, device=r.gates.device)
     if d_l_aux is not None:

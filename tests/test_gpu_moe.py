@@ -239,6 +239,13 @@ def test_gate_streaming_kernels_against_torch(dtype, S, M, E):
     dx = torch.empty(S, M, dtype=dtype, device=DEV)
     ops.gate_dgrad(dld, 1, wd, dx)
     assert_close(dx, dl[:, 1:E + 1] @ w.float(), dtype, "dx")
+    # with an addend: the sum autograd would form of the two rounded tensors, bit for bit (also in place)
+    other = torch.randn(S, M, generator=gen).to(dtype).to(DEV)
+    dx2 = torch.empty_like(dx)
+    ops.gate_dgrad(dld, 1, wd, dx2, init=other)
+    assert torch.equal(dx2, other + dx)
+    ops.gate_dgrad(dld, 1, wd, other, init=other)
+    assert torch.equal(other, dx2)
     dw = torch.zeros(E, M, dtype=dtype, device=DEV)
     ops.gate_wgrad(dld, 1, xd, dw, False)
     want = dl[:, 1:E + 1].T @ x.float()
@@ -259,3 +266,44 @@ def test_gate_streaming_kernels_limits():
     assert not ops.gate_supported(x[:, 1:9], torch.zeros(4, 8, dtype=torch.bfloat16, device=DEV))   # misaligned rows
     with pytest.raises(RtpError):
         ops.gate_fwd(x, torch.zeros(17, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(8, 17, device=DEV), 0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_moe_input_gradient_paths_meet_in_the_gate_kernel(dtype):
+    """The tokens feed the gate and the dispatch; the gate's input-gradient kernel adds the dispatch path's gradient in
+    its epilogue.  Same bits as autograd's own sum of the two (taken from two layers that share weights, one fed
+    through a leaf per path), l_aux arrives in the layer's dtype, and a loss that uses only l_aux still works."""
+    from rtp_amd import emulate_shards
+    from rtp_amd.models.transformer_lm_rtp import FeedForwardLayer_expert
+    from rtp_amd.module import moe as moe_mod
+    from rtp_amd.module.moe import WeightMOELayer
+    from rtp_amd.module.top2gate import Top2Gate, WeightTop2Gate
+    gen = torch.Generator().manual_seed(4)
+    M, Fd, E, ws = 64, 128, 4, 4
+    mg = Top2Gate(M, E)
+    masters = [FeedForwardLayer_expert(M, Fd, torch.nn.ReLU(), 0.0) for _ in range(E)]
+    with emulate_shards(ws):
+        gate = WeightTop2Gate(M, E, gate=mg, device=DEV, dtype=dtype)
+        layer = WeightMOELayer(gate, torch.nn.ModuleList([FeedForwardLayer_expert(M, Fd, torch.nn.ReLU(), 0.0)]),
+                               device=DEV, dtype=dtype, original_experts=[torch.nn.ModuleList([m]) for m in masters])
+    x = torch.randn(4, 16, M, generator=gen).to(dtype).to(DEV)
+    g = torch.randn(4, 16, M, generator=gen).to(dtype).to(DEV)
+    u = torch.rand(64, E, generator=gen).clamp(min=1e-6, max=1 - 1e-6)
+    noise = (-torch.log(-torch.log(u))).to(DEV)
+    xa = x.clone().requires_grad_()
+    out = layer(xa, noise=noise)
+    assert layer.l_aux.dtype == dtype
+    out.backward(g)
+    fused = xa.grad.clone()
+    # the same pass with the meeting point switched off: autograd adds the two paths itself
+    try:
+        moe_mod._JOIN_INPUT_GRADIENTS = False
+        xb = x.clone().requires_grad_()
+        layer(xb, noise=noise).backward(g)
+    finally:
+        moe_mod._JOIN_INPUT_GRADIENTS = True
+    assert torch.equal(fused, xb.grad)
+    xc = x.clone().requires_grad_()
+    layer(xc, noise=noise)
+    layer.l_aux.backward()                                        # only the auxiliary loss: the outputs' grads are None
+    assert xc.grad is not None and torch.isfinite(xc.grad).all() and float(xc.grad.abs().sum()) > 0
