@@ -971,8 +971,8 @@ __device__ __forceinline__ Frag<T> read_frag_dma(const char* st, int rowbase, in
   return u.f;
 }
 
-template <typename T, int BM, int BN, bool AKC, bool BKC, int NSTAGE, int SB, int PD, int OCC = 2>
-__global__ __launch_bounds__(512, OCC) void gemm_dma_kernel(GemmArgs p) {
+template <typename T, int BM, int BN, bool AKC, bool BKC, int NSTAGE, int SB, int PD>
+__global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   constexpr int NL = 4;  // loader waves (waves 4..7); waves 0..3 compute
   using DA = DmaOperand<T, BM, AKC, NL, SB>;
   using DB = DmaOperand<T, BN, BKC, NL, SB>;
@@ -1520,7 +1520,7 @@ static int launch_dma8(hipStream_t s, const GemmArgs& a, bool akc, bool bkc, dim
   return RTP_OK;
 }
 
-template <typename T, int BM, int BN, int NSTAGE, int SB, int PD, int OCC = 2>
+template <typename T, int BM, int BN, int NSTAGE, int SB, int PD>
 static int launch_dma(hipStream_t s, const GemmArgs& a, bool akc, bool bkc, dim3 grid) {
   const dim3 block(512);
   // A row-contiguous operand is staged as k lines of R elements, and a 1 KiB load must cover whole lines (or a
@@ -1530,20 +1530,20 @@ static int launch_dma(hipStream_t s, const GemmArgs& a, bool akc, bool bkc, dim3
     RTP_REQUIRE((akc || A_RC_OK) && (bkc || B_RC_OK), "gemm: tile %d x %d needs K-contiguous operands", BM, BN);
     if constexpr (!B_RC_OK && A_RC_OK) {
       if (akc)
-        hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, true, NSTAGE, SB, PD, OCC>), grid, block, 0, s, a);
+        hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, true, NSTAGE, SB, PD>), grid, block, 0, s, a);
       else
-        hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, true, NSTAGE, SB, PD, OCC>), grid, block, 0, s, a);
+        hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, true, NSTAGE, SB, PD>), grid, block, 0, s, a);
     }
     RTP_LAUNCH_CHECK();
     return RTP_OK;
   } else if (akc && bkc)
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, true, NSTAGE, SB, PD, OCC>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, true, NSTAGE, SB, PD>), grid, block, 0, s, a);
   else if (akc && !bkc)
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, false, NSTAGE, SB, PD, OCC>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, true, false, NSTAGE, SB, PD>), grid, block, 0, s, a);
   else if (!akc && bkc)
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, true, NSTAGE, SB, PD, OCC>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, true, NSTAGE, SB, PD>), grid, block, 0, s, a);
   else
-    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, false, NSTAGE, SB, PD, OCC>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_dma_kernel<T, BM, BN, false, false, NSTAGE, SB, PD>), grid, block, 0, s, a);
   RTP_LAUNCH_CHECK();
   return RTP_OK;
 }
@@ -1628,9 +1628,9 @@ struct TileShape {
   int bm, bn;
   const char* tag;
 };
-static const TileShape kShapes[7] = {{256, 128, "256x128"}, {128, 128, "128x128"}, {128, 64, "128x64"}, {64, 64, "64x64"},
-                                     {128, 192, "128x192"}, {256, 256, "256x256"}, {128, 64, "128x64c"}};
-constexpr int kNumShapes = 7;
+static const TileShape kShapes[6] = {{256, 128, "256x128"}, {128, 128, "128x128"}, {128, 64, "128x64"}, {64, 64, "64x64"},
+                                     {128, 192, "128x192"}, {256, 256, "256x256"}};
+constexpr int kNumShapes = 6;
 
 // One wavefront per 32 x 32 block is the better kernel for one attention head at sequence length <= 64.
 static bool is_tiny(const rtp_gemm_desc* d) { return d->m <= 64 && d->n <= 64 && d->k * d->ksegs <= 256; }
@@ -1785,12 +1785,8 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
     const char* e = getenv("RTP_GEMM_TILE");  // debugging aid: index into kShapes
     return e ? atoi(e) : -1;
   }();
-  static const double slab_ns[kNumShapes] = {966.0, 470.0, 283.0, 167.0, 800.0, 1680.0, 283.0};
-  static const int slab_bytes[kNumShapes] = {128, 128, 128, 128, 128, 128, 128};
-  static const int co = [] {
-    const char* e = getenv("RTP_GEMM_CO");  // experiment: co-resident 128 x 64 kernel instead of 128x64 (1) / also 128x128 (2)
-    return e ? atoi(e) : 0;
-  }();
+  static const double slab_ns[kNumShapes] = {966.0, 470.0, 283.0, 167.0, 800.0, 1680.0};
+  static const int slab_bytes[kNumShapes] = {128, 128, 128, 128, 128, 128};
   int shape = 3;  // 64 x 64 unless the model finds something cheaper
   double best = 0.0;
   for (int i = 0; fast && i < kNumShapes; ++i) {
@@ -1800,7 +1796,6 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
     // -10 % on the MoE layer's time; a loss where it leaves CUs without a tile or K is shorter)
     // (its epilogue is the plain one: the update and the statistics epilogue are never routed to it, forced or not)
     if (i == 5 && (sizeof(T) != 2 || d->sgd_master || d->xent_mode == 1)) continue;
-    if (i == 6 && i != forced) continue;
     if (i == 5 && (ceil_div(d->m, 256) * ceil_div(d->n, 256) * nz < 256 || d->k * d->ksegs < 1024) && i != forced)
       continue;
     // never a tile that is mostly padding: a 32 x 32 problem (one attention head at seq 32) stays at 64 x 64
@@ -1815,7 +1810,6 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
       shape = i;
     }
   }
-  if (fast && sizeof(T) == 2 && ((co >= 1 && shape == 2) || (co >= 2 && shape == 1))) shape = 6;
   const TileShape& ts = kShapes[shape];
   a.tiles_m = (int)ceil_div(d->m, ts.bm);
   a.tiles_n = (int)ceil_div(d->n, ts.bn);
@@ -1927,8 +1921,6 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
       return launch_dma<T, 128, 64, 5, 128, 4>(s, a, akc, bkc, grid);
     case 4:
       return launch_dma<T, 128, 192, 3, 128, 2>(s, a, akc, bkc, grid);
-    case 6:
-      return launch_dma<T, 128, 64, 3, 128, 1, 4>(s, a, akc, bkc, grid);
     case 5:
       if constexpr (sizeof(T) == 2) return launch_dma8<T, 2, 128, 1>(s, a, akc, bkc, grid);
       return fail(RTP_ERR_ARG, "gemm: no 256 x 256 kernel for this dtype");
