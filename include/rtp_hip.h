@@ -692,7 +692,7 @@ typedef struct {
   double flops; /* algorithmic, summed over launches */
   double bytes; /* algorithmic, summed over launches */
   /* mode 2, wave-specialised product kernels only (else 0): where a workgroup's time goes, each entry the average over
-   * the launch's workgroups, summed over launches: [0] launch start -> the workgroup's own start (waiting for a CU),
+   * every 16th workgroup of the launch, summed over launches: [0] launch start -> the workgroup's own start (waiting for a CU),
    * [1] its start -> first operands visible in LDS, [2] the K loop, [3] the epilogue */
   double phase_ms[4];
 } rtp_kernel_stat;
