@@ -598,14 +598,22 @@ int rtp_gate_wgrad_static(void* stream, int dtype, const float* dlogits, int64_t
 
 /* ---------------------------------------------------------------------------------------------
  * Out-channel-sharded 2-D convolution (reference: the per-shard `self.layers[index](input_)` = F.conv2d of
- * ColumnParallelConv2d, rtp/module/conv.py:108, and its autograd backward) as a column-sharded product on
- * rtp_gemm:  Y[N*Ho*Wo, Co_s] = patches[N*Ho*Wo, Ci*kh*kw] x W_s^T + b_s  (a shard's weight [Co_s, Ci, kh, kw] is,
- * as stored, that row-major operand), dW_s = dY_s^T patches, dpatches = sum_s dY_s W_s.  These two entry points
- * build the patch matrix and fold patch gradients back (zero padding, groups = 1):
- *   im2col: patches[(n*Ho+ho)*Wo+wo][(ci*kh+i)*kw+j] = x[n][ci][ho*sh-ph+i*dh][wo*sw-pw+j*dw], 0 outside; x is
- *           addressed by element strides (any memory format), columns beyond Ci*kh*kw up to ld_cols are zeroed
- *   col2im: dx[n][ci][h][w] (contiguous NCHW) = sum of the patch-gradient entries that read x[n][ci][h][w],
- *           fp32, ascending (i, j)
+ * ColumnParallelConv2d, rtp/module/conv.py:99-114, and its autograd backward) as an implicit GEMM: the patch matrix
+ *   patches[(n*Ho+ho)*Wo+wo][(ci*kh+i)*kw+j] = x[n][ci][ho*sh-ph+i*dh][wo*sw-pw+j*dw]   (0 outside: zero padding)
+ * is gathered by the product kernel as it goes and never written to memory (groups = 1).  A run of `shards`
+ * consecutive shards is described like a rotated linear layer: `w` / `grads` point at the run's first shard row,
+ * rows are `numel` elements apart, a shard's weight [n_s, Ci, kh, kw] (as stored: row-major [n_s, Ci*kh*kw]) sits at
+ * element w_off of its row and its bias [n_s] at bias_off (bias_off < 0: none); the run produces / reads output
+ * channels co_first .. co_first + shards*n_s - 1.  Activations x and dy are addressed by element strides (any memory
+ * format); y and dx are contiguous NCHW.
+ *   fwd:    y[n][co][ho][wo] = sum_k W[co][k] patches[pix][k] + b[co]; y has co_total channels in all
+ *   wgrad:  grads_s[w_off + co*K + k] (+)= sum_pix dy[n][co][ho][wo] patches[pix][k], and with bias_off >= 0
+ *           grads_s[bias_off + co] (+)= sum_pix dy[n][co][ho][wo]   (fp32 sums in a fixed order; (+) = accumulate != 0);
+ *           the sum over the pixels is dealt over several workgroups whose fp32 partial sums go through `workspace`
+ *           (rtp_conv2d_wgrad_workspace_bytes of device memory, 0 for small problems; 16-byte aligned)
+ *   dgrad:  dx[n][ci][h][w] = addend + sum over the run's (co, i, j) of W[co][ci][i][j] dy[n][co][ho][wo] for the
+ *           output pixels that read x[n][ci][h][w]; dx_f32 / addend_f32: that array is fp32 although dtype is bf16
+ *           (the sum over several runs is kept in fp32 and rounded by the last one); addend may be NULL or dx itself
  * ho / wo must equal floor((h + 2*ph - dh*(kh-1) - 1) / sh) + 1 (and likewise for w).
  * --------------------------------------------------------------------------------------------- */
 typedef struct {
@@ -616,9 +624,19 @@ typedef struct {
   int64_t dh, dw;       /* dilation */
   int64_t ho, wo;       /* output height, width */
 } rtp_conv_geom;
-int rtp_im2col(void* stream, int dtype, const void* x, int64_t sx_n, int64_t sx_c, int64_t sx_h, int64_t sx_w,
-               const rtp_conv_geom* geom, void* cols, int64_t ld_cols);
-int rtp_col2im(void* stream, int dtype, const void* dcols, int64_t ld_dcols, const rtp_conv_geom* geom, void* dx);
+int rtp_conv2d_fwd(void* stream, int dtype, const void* x, int64_t sx_n, int64_t sx_c, int64_t sx_h, int64_t sx_w,
+                   const rtp_conv_geom* geom, const void* w, int64_t numel, int64_t shards, int64_t w_off,
+                   int64_t bias_off, int64_t n_s, void* y, int64_t co_first, int64_t co_total);
+int rtp_conv2d_wgrad(void* stream, int dtype, const void* dy, int64_t sdy_n, int64_t sdy_c, int64_t sdy_h,
+                     int64_t sdy_w, const void* x, int64_t sx_n, int64_t sx_c, int64_t sx_h, int64_t sx_w,
+                     const rtp_conv_geom* geom, void* grads, int64_t numel, int64_t shards, int64_t w_off,
+                     int64_t bias_off, int64_t n_s, int64_t co_first, int accumulate, void* workspace,
+                     size_t workspace_bytes);
+size_t rtp_conv2d_wgrad_workspace_bytes(const rtp_conv_geom* geom, int64_t shards, int64_t n_s);
+int rtp_conv2d_dgrad(void* stream, int dtype, const void* dy, int64_t sdy_n, int64_t sdy_c, int64_t sdy_h,
+                     int64_t sdy_w, const rtp_conv_geom* geom, const void* w, int64_t numel, int64_t shards,
+                     int64_t w_off, int64_t n_s, int64_t co_first, void* dx, int dx_f32, const void* addend,
+                     int addend_f32);
 
 /* ---------------------------------------------------------------------------------------------
  * Optimiser step on a flat shard buffer (reference harness: clip_grad_value_ + optimizer.step,

@@ -160,8 +160,13 @@ PROTOTYPES = {
     "rtp_gate_wgrad_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "rtp_gate_wgrad": (_i, [_vp, _i, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i, _vp, _sz]),
     "rtp_gate_wgrad_static": (_i, [_vp, _i, _vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i]),
-    "rtp_im2col": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _i64, C.POINTER(ConvGeom), _vp, _i64]),
-    "rtp_col2im": (_i, [_vp, _i, _vp, _i64, C.POINTER(ConvGeom), _vp]),
+    "rtp_conv2d_fwd": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _i64, C.POINTER(ConvGeom), _vp, _i64, _i64, _i64, _i64, _i64,
+                            _vp, _i64, _i64]),
+    "rtp_conv2d_wgrad": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _i64, C.POINTER(ConvGeom), _vp,
+                              _i64, _i64, _i64, _i64, _i64, _i64, _i, _vp, _sz]),
+    "rtp_conv2d_wgrad_workspace_bytes": (_sz, [C.POINTER(ConvGeom), _i64, _i64]),
+    "rtp_conv2d_dgrad": (_i, [_vp, _i, _vp, _i64, _i64, _i64, _i64, C.POINTER(ConvGeom), _vp, _i64, _i64, _i64, _i64, _i64,
+                              _vp, _i, _vp, _i]),
     "rtp_sgd_step": (_i, [_vp, _i, _vp, _vp, _vp, _i64, _f, _f]),
     "rtp_adam_step": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i64, C.c_double, C.c_double, C.c_double, C.c_double,
                            C.c_double, _i64, _vp, C.c_double]),

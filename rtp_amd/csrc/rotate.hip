@@ -198,7 +198,7 @@ using namespace rtp;
 
 extern "C" const char* rtp_last_error(void) { return error_buffer(); }
 
-extern "C" int rtp_abi_version(void) { return 4; }
+extern "C" int rtp_abi_version(void) { return 5; }
 
 extern "C" int rtp_device_check(char* name_out, int name_len) {
   int dev = 0;

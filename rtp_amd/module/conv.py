@@ -2,15 +2,14 @@
 
 Shard s owns output channels [s*Co/ws, (s+1)*Co/ws): weight [Co/ws, Ci, kh, kw] and the bias slice (conv.py:43-47,
 affine_weight along dim 0); the shards' outputs are concatenated on the channel dimension (conv.py:114).  A shard's
-weight is, as stored in the flat buffer, the row-major [Co/ws, Ci*kh*kw] operand of a column-sharded linear layer
-over the patch matrix of the input, so the layer runs on the same grouped products as ColumnParallelLinear:
+weight is, as stored in the flat buffer, the row-major [Co/ws, Ci*kh*kw] operand of a product over the patch matrix
+of the input, and the library runs the three products of the layer as implicit GEMMs that gather the patches as they
+go -- the patch matrix never exists in memory:
 
-    patches = im2col(x)                       [N*Ho*Wo, Ci*kh*kw]   one kernel, any input memory format
-    y2d     = patches W^T + b                 [N*Ho*Wo, Co]         one grouped GEMM per rotation window
-    dW, db  = dY^T patches, colsum(dY)        the weight-gradient product carries the bias gradient
-    dx      = col2im(dY W)                    gather per input element, fixed summation order
+    y[:, shard's channels] = W_s . patches(x) + b_s       one launch per rotation window, NCHW written directly
+    dW_s, db_s             = dy_s . patches(x)^T, sums    one launch per run of gradient rows
+    dx                     = sum_s W_s^T . dy_s           one launch per rotation window (fp32 between windows)
 
-The product's natural layout is NHWC; the layer returns a contiguous NCHW tensor as the reference does (torch copy).
 groups = 1 and zero padding only.
 """
 from __future__ import annotations
@@ -22,7 +21,6 @@ import torch.nn as nn
 
 from .. import ops
 from ..ring import Rotation, ring_order, run_wgrad
-from . import shard_ops as S
 from .collectives import RotatedLayer, resolve_world
 from .utils import affine_weight, divide_and_check_no_remainder
 
@@ -65,55 +63,46 @@ class _ColumnConvFn(torch.autograd.Function):
         n_s, ws, co = layer.output_size_per_partition, layer.world_size, layer.out_channels
         geom = ops.conv_geom(x.shape, layer.kernel_size, layer.stride, layer.padding, layer.dilation)
         k = geom.c * geom.kh * geom.kw
-        rows = geom.n * geom.ho * geom.wo
-        cols = torch.empty(rows, k, dtype=x.dtype, device=x.device)
-        ops.im2col(x, geom, cols)
-        y = torch.empty(rows, co, dtype=x.dtype, device=x.device)
+        y = torch.empty(geom.n, co, geom.ho, geom.wo, dtype=x.dtype, device=x.device)
         b_off = n_s * k if layer.has_bias else None
         rot = Rotation(store.home, ring_order(layer.rank, ws), group=store.stage_group)
         for j in range(rot.steps):
             for flat, first, cnt in rot.acquire(j):
-                S.col_fwd(cols, flat, 0, n_s, k, b_off, y, first * n_s)
+                ops.conv2d_fwd(x, geom, flat, 0, b_off, n_s, y, first * n_s)
             rot.release(j)
         ctx.layer, ctx.geom = layer, geom
-        ctx.save_for_backward(cols)
-        return y.view(geom.n, geom.ho, geom.wo, co).permute(0, 3, 1, 2).contiguous()
+        ctx.save_for_backward(x)
+        return y
 
     @staticmethod
     def backward(ctx, dy):
         layer, geom = ctx.layer, ctx.geom
-        (cols,) = ctx.saved_tensors
+        (x,) = ctx.saved_tensors
         store = layer._store
-        n_s, ws, co = layer.output_size_per_partition, layer.world_size, layer.out_channels
-        k = cols.shape[1]
-        dy2 = dy.permute(0, 2, 3, 1).reshape(-1, co)
-        if not dy2.is_contiguous():
-            dy2 = dy2.contiguous()
-        need_dx = ctx.needs_input_grad[0]
+        n_s, ws = layer.output_size_per_partition, layer.world_size
+        k = geom.c * geom.kh * geom.kw
         order = ring_order(layer.rank, ws, reverse=True)
         dx = None
-        if need_dx:
-            dcols = torch.empty_like(cols)
+        if ctx.needs_input_grad[0]:
+            dx = torch.empty(geom.n, geom.c, geom.h, geom.w, dtype=dy.dtype, device=dy.device)
             rot = Rotation(store.home, order, group=store.stage_group)
-            acc = ops.ShardSum(dcols, sum(len(w) for w in rot.windows))
+            acc = ops.ShardSum(dx, sum(len(w) for w in rot.windows))
             i = 0
             for j in range(rot.steps):
                 for flat, first, cnt in rot.acquire(j):
                     c_out, c_in = acc.target(i)
-                    S.col_dgrad(dy2, flat, 0, n_s, k, c_out, first * n_s, c_in=c_in)
+                    ops.conv2d_dgrad(dy, geom, flat, 0, n_s, first * n_s, c_out, addend=c_in)
                     i += 1
                 rot.release(j)
-            dx = torch.empty(geom.n, geom.c, geom.h, geom.w, dtype=dy.dtype, device=dy.device)
-            ops.col2im(dcols, geom, dx)
         runs = store.grad_runs(order)
+        b_off = n_s * k if layer.has_bias else None
 
         def param_grads():
             for first, cnt, accumulate in runs:
-                S.col_wgrad(dy2, cols, store.grads, first, 0, n_s, k, first * n_s, cnt, accumulate,
-                            b_off=n_s * k if layer.has_bias else None, store=store)
+                ops.conv2d_wgrad(dy, x, geom, store.grads[first:first + cnt], 0, b_off, n_s, first * n_s, accumulate)
             store.grads_ready()
 
-        run_wgrad(dy2.device, param_grads, (dy2, cols))
+        run_wgrad(dy.device, param_grads, (dy, x))
         return dx, None, None
 
 

@@ -854,27 +854,74 @@ def conv_geom(x_shape, kernel_size, stride, padding, dilation) -> "_lib.ConvGeom
     return _lib.ConvGeom(n, c, h, w, kh, kw, sh, sw, ph, pw, dh, dw, ho, wo)
 
 
-def im2col(x: torch.Tensor, geom, cols: torch.Tensor) -> None:
-    """cols[N*Ho*Wo, ld] <- the patch matrix of NCHW `x` (any strides); columns beyond C*kh*kw are zeroed."""
+def _conv_run(who: str, flat: torch.Tensor, n_s: int, geom, w_off: int, bias_off: Optional[int]):
+    """(numel, shards, element size) of a run of shard rows [shards, numel] that holds a [n_s, C, kh, kw] weight at
+    w_off and, if bias_off is given, a bias [n_s]."""
+    _dev(flat)
+    if flat.dim() != 2 or flat.stride(1) != 1 or (flat.shape[0] > 1 and flat.stride(0) != flat.shape[1]):
+        raise ValueError(f"{who}: the shards of a run are the rows of a dense [shards, numel] tensor")
+    kp = geom.c * geom.kh * geom.kw
+    if w_off < 0 or w_off + n_s * kp > flat.shape[1] or (bias_off is not None and bias_off + n_s > flat.shape[1]):
+        raise ValueError(f"{who}: weight / bias offsets outside a shard row of {flat.shape[1]} elements")
+    return flat.shape[1], flat.shape[0], flat.element_size()
+
+
+def conv2d_fwd(x: torch.Tensor, geom, flat: torch.Tensor, w_off: int, bias_off: Optional[int], n_s: int,
+               y: torch.Tensor, co_first: int) -> None:
+    """y[:, co_first : co_first + shards*n_s] (contiguous NCHW `y` with all the layer's channels) = conv2d(x, W_g) + b_g
+    for the shards g of the run `flat` [shards, numel]; x in any memory format.  Implicit GEMM: no patch matrix."""
+    numel, shards, _ = _conv_run("conv2d_fwd", flat, n_s, geom, w_off, bias_off)
     _dev(x)
-    if x.dim() != 4 or cols.dim() != 2 or cols.dtype != x.dtype or cols.stride(1) != 1 or \
-            cols.shape[0] != geom.n * geom.ho * geom.wo or cols.stride(0) != cols.shape[1]:
-        raise ValueError("im2col: need a 4-D input and a dense [N*Ho*Wo, ld] patch matrix of its dtype")
+    if x.dim() != 4 or tuple(x.shape) != (geom.n, geom.c, geom.h, geom.w) or x.dtype != flat.dtype or \
+            y.dtype != flat.dtype or not y.is_contiguous() or y.dim() != 4 or \
+            (y.shape[0], y.shape[2], y.shape[3]) != (geom.n, geom.ho, geom.wo) or co_first + shards * n_s > y.shape[1]:
+        raise ValueError("conv2d_fwd: x [N,C,H,W] and a contiguous y [N,Co,Ho,Wo] of the weights' dtype")
     _lib.require_device()
-    check(_lib.load().rtp_im2col(_stream(), dtype_code(x.dtype), x.data_ptr(), *x.stride(), geom, cols.data_ptr(),
-                                 cols.shape[1]))
+    check(_lib.load().rtp_conv2d_fwd(_stream(), dtype_code(x.dtype), x.data_ptr(), *x.stride(), geom, flat.data_ptr(),
+                                     numel, shards, w_off, -1 if bias_off is None else bias_off, n_s, y.data_ptr(),
+                                     co_first, y.shape[1]))
 
 
-def col2im(dcols: torch.Tensor, geom, dx: torch.Tensor) -> None:
-    """dx (contiguous NCHW) <- patch gradients dcols[N*Ho*Wo, ld] folded back onto the input."""
-    _dev(dcols)
-    if dcols.dim() != 2 or dcols.stride(1) != 1 or dcols.stride(0) != dcols.shape[1] or dx.dtype != dcols.dtype or \
-            not dx.is_contiguous() or tuple(dx.shape) != (geom.n, geom.c, geom.h, geom.w) or \
-            dcols.shape[0] != geom.n * geom.ho * geom.wo:
-        raise ValueError("col2im: need a dense [N*Ho*Wo, ld] patch-gradient matrix and a contiguous NCHW output")
+def conv2d_wgrad(dy: torch.Tensor, x: torch.Tensor, geom, grads: torch.Tensor, w_off: int, bias_off: Optional[int],
+                 n_s: int, co_first: int, accumulate: bool) -> None:
+    """The gradient rows `grads` [shards, numel] of a run of shards: weight gradients at w_off, bias gradients at
+    bias_off (if given), from dy[:, co_first : co_first + shards*n_s] and the layer input x (both in any memory
+    format); added to what is there when `accumulate`."""
+    numel, shards, _ = _conv_run("conv2d_wgrad", grads, n_s, geom, w_off, bias_off)
+    _dev(x)
+    _dev(dy)
+    if x.dim() != 4 or tuple(x.shape) != (geom.n, geom.c, geom.h, geom.w) or dy.dim() != 4 or \
+            (dy.shape[0], dy.shape[2], dy.shape[3]) != (geom.n, geom.ho, geom.wo) or \
+            co_first + shards * n_s > dy.shape[1] or x.dtype != grads.dtype or dy.dtype != grads.dtype:
+        raise ValueError("conv2d_wgrad: x [N,C,H,W] and dy [N,Co,Ho,Wo] of the gradients' dtype")
     _lib.require_device()
-    check(_lib.load().rtp_col2im(_stream(), dtype_code(dcols.dtype), dcols.data_ptr(), dcols.shape[1], geom,
-                                 dx.data_ptr()))
+    lib = _lib.load()
+    nbytes = lib.rtp_conv2d_wgrad_workspace_bytes(geom, shards, n_s)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+    check(lib.rtp_conv2d_wgrad(_stream(), dtype_code(x.dtype), dy.data_ptr(), *dy.stride(), x.data_ptr(),
+                               *x.stride(), geom, grads.data_ptr(), numel, shards, w_off,
+                               -1 if bias_off is None else bias_off, n_s, co_first, int(accumulate), ws.data_ptr(),
+                               nbytes))
+
+
+def conv2d_dgrad(dy: torch.Tensor, geom, flat: torch.Tensor, w_off: int, n_s: int, co_first: int, dx: torch.Tensor,
+                 addend: Optional[torch.Tensor] = None) -> None:
+    """dx [N,C,H,W] (contiguous; the weights' dtype or fp32) = addend + the input gradient through the shards of the
+    run `flat`, which own dy's channels co_first .. co_first + shards*n_s - 1."""
+    numel, shards, _ = _conv_run("conv2d_dgrad", flat, n_s, geom, w_off, None)
+    _dev(dy)
+    _dev(dx)
+    ok = (torch.float32, flat.dtype)
+    if dy.dim() != 4 or (dy.shape[0], dy.shape[2], dy.shape[3]) != (geom.n, geom.ho, geom.wo) or \
+            co_first + shards * n_s > dy.shape[1] or dy.dtype != flat.dtype or not dx.is_contiguous() or \
+            tuple(dx.shape) != (geom.n, geom.c, geom.h, geom.w) or dx.dtype not in ok or \
+            (addend is not None and (addend.shape != dx.shape or not addend.is_contiguous() or addend.dtype not in ok)):
+        raise ValueError("conv2d_dgrad: dy [N,Co,Ho,Wo] of the weights' dtype, contiguous dx / addend [N,C,H,W]")
+    _lib.require_device()
+    check(_lib.load().rtp_conv2d_dgrad(_stream(), dtype_code(dy.dtype), dy.data_ptr(), *dy.stride(), geom,
+                                       flat.data_ptr(), numel, shards, w_off, n_s, co_first, dx.data_ptr(),
+                                       int(dx.dtype == torch.float32), None if addend is None else addend.data_ptr(),
+                                       int(addend is not None and addend.dtype == torch.float32)))
 
 
 def adam_step(master: torch.Tensor, grad: torch.Tensor, shadow: Optional[torch.Tensor], exp_avg: torch.Tensor,

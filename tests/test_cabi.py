@@ -40,7 +40,7 @@ def test_loader_binds_and_reports_version():
     if not os.path.exists(_lib.LIB_PATH):
         pytest.skip("librtp_hip.so not built")
     lib = _lib.load()
-    assert lib.rtp_abi_version() == 4
+    assert lib.rtp_abi_version() == 5
     assert isinstance(_lib.last_error(), str)
 
 

@@ -1,6 +1,6 @@
 """Rotated ColumnParallelConv2d and the wrapper's Conv2d rule against stock torch.nn.Conv2d on the CPU (the
 reference's own oracle for this layer: test_net.py:135-177 compares the wrapped MNIST Net with an untouched copy),
-and the patch-matrix kernels against F.unfold / F.fold."""
+and the implicit-GEMM entry points against products over the explicit patch matrix (F.unfold / F.fold)."""
 import copy
 
 import pytest
@@ -15,51 +15,89 @@ pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("rotation_window")]
 
 GEOMS = [
     # (N, Ci, H, W, Co, kernel, stride, padding, dilation)
-    (3, 1, 28, 28, 32, 3, 1, 0, 1),                   # MNIST conv1: 9-element patches (element-wise GEMM path)
-    (2, 32, 26, 26, 64, 3, 1, 0, 1),                  # MNIST conv2: 288-element patches (vector path)
+    (3, 1, 28, 28, 32, 3, 1, 0, 1),                   # MNIST conv1: 9-element patches, one input channel
+    (2, 32, 26, 26, 64, 3, 1, 0, 1),                  # MNIST conv2: 288-element patches
     (2, 8, 13, 11, 16, (3, 2), (2, 1), (1, 2), (1, 2)),
     (1, 4, 9, 9, 8, 5, 3, 2, 1),
 ]
 
 
+def _pair(v):
+    return (v, v) if isinstance(v, int) else v
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("geom", GEOMS)
-def test_patch_kernels_match_unfold_and_fold(geom, dtype):
+def test_implicit_products_match_the_patch_matrix_oracle(geom, dtype):
+    """The three entry points on a run of two shards against products over the oracle's explicit patch matrix
+    (F.unfold) and its fold back (F.fold)."""
     from rtp_amd import ops
-    n, ci, h, w, _, k, s, p, d = geom
-    pair = lambda v: (v, v) if isinstance(v, int) else v
-    k, s, p, d = pair(k), pair(s), pair(p), pair(d)
-    gen = torch.Generator().manual_seed(h * w)
+    n, ci, h, w, co, k, s, p, d = geom
+    k, s, p, d = _pair(k), _pair(s), _pair(p), _pair(d)
+    gen = torch.Generator().manual_seed(h * w + co)
     x = torch.randn(n, ci, h, w, generator=gen).to(dtype)
     g = ops.conv_geom(x.shape, k, s, p, d)
-    ref = O.conv_patches(x.float(), k, s, p, d)
-    cols = torch.empty(ref.shape, dtype=dtype, device=DEV)
-    ops.im2col(x.to(DEV), g, cols)
-    assert torch.equal(cols.float().cpu(), ref)                       # pure data movement: bit-exact
-    # a channels-last input is read through its strides
-    cols2 = torch.empty_like(cols)
-    ops.im2col(x.to(DEV).contiguous(memory_format=torch.channels_last), g, cols2)
-    assert torch.equal(cols2, cols)
-    # padded row pitch: the extra columns are zeroed
-    ld = ref.shape[1] + 5
-    wide = torch.full((ref.shape[0], ld), 7.0, dtype=dtype, device=DEV)
-    ops.im2col(x.to(DEV), g, wide)
-    assert torch.equal(wide[:, :ref.shape[1]], cols) and not wide[:, ref.shape[1]:].any()
-    dcols = torch.randn(ref.shape, generator=gen).to(dtype)
+    kp, shards, extra = ci * k[0] * k[1], 2, 3                         # `extra` unused elements in front of a row
+    n_s = co // shards
+    numel = extra + n_s * kp + n_s
+    flat = (torch.randn(shards, numel, generator=gen) * 0.2).to(dtype)
+    w2d = torch.cat([flat[i, extra:extra + n_s * kp].view(n_s, kp) for i in range(shards)], 0).float()
+    bias = torch.cat([flat[i, extra + n_s * kp:] for i in range(shards)], 0).float()
+    patches = O.conv_patches(x.float(), k, s, p, d)                    # [n*ho*wo, kp]
+    to_nchw = lambda m2d, c: m2d.view(n, g.ho, g.wo, c).permute(0, 3, 1, 2)
+    xd, fd = x.to(DEV), flat.to(DEV)
+    # forward into the middle channels of a wider output
+    y = torch.full((n, co + 2, g.ho, g.wo), 7.0, dtype=dtype, device=DEV)
+    ops.conv2d_fwd(xd, g, fd, extra, extra + n_s * kp, n_s, y, 1)
+    assert_close(y[:, 1:1 + co], to_nchw(patches @ w2d.t() + bias, co), dtype, "forward")
+    assert bool((y[:, 0] == 7).all()) and bool((y[:, -1] == 7).all())
+    y2 = torch.empty_like(y)
+    ops.conv2d_fwd(xd.contiguous(memory_format=torch.channels_last), g, fd, extra, None, n_s, y2, 1)
+    assert_close(y2[:, 1:1 + co], to_nchw(patches @ w2d.t(), co), dtype, "forward, channels-last input, no bias")
+    # weight and bias gradients, written and then accumulated
+    dy = torch.randn(n, co + 2, g.ho, g.wo, generator=gen).to(dtype)
+    dy2d = dy[:, 1:1 + co].permute(0, 2, 3, 1).reshape(-1, co).float()
+    grads = torch.full((shards, numel), 5.0, dtype=dtype, device=DEV)
+    ops.conv2d_wgrad(dy.to(DEV), xd, g, grads, extra, extra + n_s * kp, n_s, 1, False)
+    dw = torch.cat([grads[i, extra:extra + n_s * kp].view(n_s, kp) for i in range(shards)], 0)
+    db = torch.cat([grads[i, extra + n_s * kp:] for i in range(shards)], 0)
+    assert_close(dw, dy2d.t() @ patches, dtype, "weight gradient")
+    assert_close(db, dy2d.sum(0), dtype, "bias gradient")
+    assert bool((grads[:, :extra] == 5).all())
+    if dtype == torch.float32:
+        ops.conv2d_wgrad(dy.to(DEV), xd, g, grads, extra, extra + n_s * kp, n_s, 1, True)
+        dw2 = torch.cat([grads[i, extra:extra + n_s * kp].view(n_s, kp) for i in range(shards)], 0)
+        assert_close(dw2, 2 * (dy2d.t() @ patches), dtype, "accumulated weight gradient")
+    # input gradient: plain, and as the last window of a sum kept in fp32
+    want_dx = O.conv_fold(dy2d @ w2d, x.shape, k, s, p, d)
     dx = torch.empty(n, ci, h, w, dtype=dtype, device=DEV)
-    ops.col2im(dcols.to(DEV), g, dx)
-    assert_close(dx, O.conv_fold(dcols.float(), x.shape, k, s, p, d), dtype, "col2im")
+    ops.conv2d_dgrad(dy.to(DEV), g, fd, extra, n_s, 1, dx)
+    assert_close(dx, want_dx, dtype, "input gradient")
+    part = torch.randn(n, ci, h, w, generator=gen)
+    scratch = torch.empty(n, ci, h, w, device=DEV)
+    ops.conv2d_dgrad(dy.to(DEV), g, fd, extra, n_s, 1, scratch, addend=part.to(dtype).to(DEV))
+    assert_close(scratch, want_dx + part.to(dtype).float(), torch.float32 if dtype == torch.float32 else dtype,
+                 "input gradient into fp32 with an addend")
+    ops.conv2d_dgrad(dy.to(DEV), g, fd, extra, n_s, 1, dx, addend=scratch)
+    assert_close(dx, 2 * want_dx + part.to(dtype).float(), dtype, "input gradient from an fp32 addend")
 
 
-def test_patch_kernels_reject_bad_geometry():
+def test_conv_entry_points_reject_bad_geometry():
     from rtp_amd import _lib, ops
     x = torch.zeros(1, 1, 4, 4, device=DEV)
     with pytest.raises(ValueError):
         ops.conv_geom(x.shape, (5, 5), (1, 1), (0, 0), (1, 1))
     g = ops.conv_geom(x.shape, (3, 3), (1, 1), (0, 0), (1, 1))
+    flat = torch.zeros(1, 2 * 9 + 2, device=DEV)
+    y = torch.zeros(1, 2, 2, 2, device=DEV)
+    ops.conv2d_fwd(x, g, flat, 0, 18, 2, y, 0)
+    with pytest.raises(ValueError):
+        ops.conv2d_fwd(x, g, flat, 4, 18, 2, y, 0)                    # the weight does not fit the shard row
+    with pytest.raises(ValueError):
+        ops.conv2d_fwd(x, g, flat, 0, 18, 2, y, 1)                    # channels beyond the output
     g.ho = 3                                                          # inconsistent with the geometry
     with pytest.raises(_lib.RtpError):
-        ops.im2col(x, g, torch.zeros(3 * 2, 9, device=DEV))
+        ops.conv2d_fwd(x, g, flat, 0, 18, 2, torch.zeros(1, 2, 3, 2, device=DEV), 0)
 
 
 @pytest.mark.parametrize("dtype,ws", [(torch.float32, 4), (torch.float32, 1), (torch.bfloat16, 4)])
@@ -151,3 +189,34 @@ def test_wrapper_shards_the_mnist_net():
         assert_close(mine, getattr(ref, name).weight.grad, torch.float32, name)
     with emulate_shards(4), pytest.raises(ValueError):
         RotatedTensorParallel(nn.Sequential(nn.Conv2d(3, 6, 3)))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rotated_sgd_updates_conv_layers_with_and_without_fused_backward(dtype):
+    """A convolution's weight gradient does not carry the optimiser's update in its own launch: under
+    RotatedSGD(fused_backward=True) its parameters take the separate update, and two steps leave the same weights
+    as the plain optimiser, bit for bit."""
+    from rtp_amd import emulate_shards
+    from rtp_amd.module.conv import ColumnParallelConv2d
+    from rtp_amd.module.linear import ColumnParallelLinear
+    from rtp_amd.optim import RotatedSGD
+    torch.manual_seed(5)
+    ref_conv, ref_fc = nn.Conv2d(3, 8, 3, padding=1), nn.Linear(8 * 6 * 6, 16)
+    x = torch.randn(4, 3, 6, 6).to(dtype).to(DEV)
+    models = []
+    for fused in (False, True):
+        with emulate_shards(2):
+            conv = ColumnParallelConv2d(3, 8, 3, padding=1, Conv2d_layer=ref_conv, device=DEV, dtype=dtype)
+            fc = ColumnParallelLinear(8 * 6 * 6, 16, linear_layer=ref_fc, device=DEV, dtype=dtype)
+        model = nn.Sequential(conv, nn.Flatten(), fc)
+        opt = RotatedSGD(model, lr=0.05, clip_value=0.05, fused_backward=fused)
+        for _ in range(2):
+            opt.zero_grad()
+            model(x).float().square().mean().backward()
+            opt.step()
+        models.append(model)
+    torch.cuda.synchronize()
+    for a, b in zip(models[0].parameters(), models[1].parameters()):
+        assert torch.equal(a, b)
+    moved = (models[0][0].layers[0].weight.float().cpu() - ref_conv.weight[:4].to(dtype).float()).abs().max()
+    assert float(moved) > 0
