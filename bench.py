@@ -814,6 +814,20 @@ def main():
         del g_s
         ring.set_rotation_mode("direct")
         ring.set_warm_ahead(args.warm_ahead)
+    if whole and args.optimizer == "sgd":
+        # The same step with the reference harness's own optimiser (benchmarks/rtp_benchmark.py:41-42, 185-186:
+        # clip_grad_value_(0.05), then torch.optim.Adam(lr 1e-3)) instead of the SGD the headline asks for: gradients
+        # are stored, fp32 moments live beside the fp32 master, one update launch over a device chunk table.
+        for st in opt.stores:
+            st.fused_sgd = None
+        opt = RotatedAdam(lm, lr=1e-3, clip_value=0.05)
+        dt_a, g_a, _ = timed(2, args.steps)
+        out["reference_harness_optimizer"] = {
+            "optimizer": "adam", "ms_per_step": dt_a * 1e3, "tokens_per_s": tokens / dt_a,
+            "what": "clip 0.05 + Adam lr 1e-3 (torch.optim.Adam's arithmetic, fp32 moments), same model, rotation, "
+                    "graph replay and fresh batch per step as the headline line",
+            "hip_graph": bool(args.graph)}
+        del g_a
     if whole:
         # The reference's other four configurations, one rotated layer each, fwd+bwd, same timing recipe.
         del g, lm, opt
