@@ -971,8 +971,11 @@ __device__ __forceinline__ Frag<T> read_frag_dma(const char* st, int rowbase, in
   return u.f;
 }
 
+// The body of the product kernel: workgroup `id` of the `nwg` that work on the problem `p` (`bx`, `by`: its
+// coordinates in a launch that does not use XCD bricks).  `p` lives in the kernel-argument segment.
 template <typename T, int BM, int BN, bool AKC, bool BKC, int NSTAGE, int SB, int PD>
-__global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
+__device__ __forceinline__ void gemm_dma_body(const GemmArgs& p, const unsigned id, const unsigned bx, const unsigned by,
+                                              const unsigned nwg) {
   constexpr int NL = 4;  // loader waves (waves 4..7); waves 0..3 compute
   using DA = DmaOperand<T, BM, AKC, NL, SB>;
   using DB = DmaOperand<T, BN, BKC, NL, SB>;
@@ -989,7 +992,6 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   // is where the loads of warm_ahead() land.
   __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE + 1024];
 
-  touch_kernel_arguments<sizeof(GemmArgs)>();
   const int tid = threadIdx.x;
   unsigned long long t_start = 0, t_ready = 0, t_loop = 0;  // phase stamps of thread 0 (an MFMA wave), mode 2 only
   if (p.trace != nullptr && tid == 0) {
@@ -1006,7 +1008,6 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   // the operand rows one XCD touches are as few as possible; workgroup `id` works on brick id % 8.
   // Both mappings are computed and one is selected, without a branch: every kernel argument is then fetched by
   // one batch of scalar loads at entry instead of three dependent rounds (each a trip to memory on a cold cache).
-  const unsigned id = blockIdx.x + blockIdx.y * gridDim.x;
   const unsigned xcd = id & 7, slot = id >> 3;
   // The ~32 workgroups an XCD runs at a time should cover a compact block of the brick, not a row of it: they
   // share the XCD's L2, and a 4 x 8 block of tiles reads 12 tile-operands where a 1 x 32 row reads 33.  Over the
@@ -1020,11 +1021,11 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
   const int tile_n_x = (int)((xcd & ((1u << p.xn_shift) - 1)) * p.nbk + qn * p.pcol + cn);
   const int tile_m_x = (int)(((xcd >> p.xn_shift) & ((1u << p.xm_shift) - 1)) * p.mbk + qm * p.prow + cm);
   const int z_x = (int)((xcd >> (p.xn_shift + p.xm_shift)) * p.zbk + zl);
-  const int tile_m_p = (int)fast_div(blockIdx.x, p.d_tiles_n);
-  const int tile_n_p = (int)(blockIdx.x - tile_m_p * p.d_tiles_n.d);
+  const int tile_m_p = (int)fast_div(bx, p.d_tiles_n);
+  const int tile_n_p = (int)(bx - tile_m_p * p.d_tiles_n.d);
   const bool bricks = p.xg != 0;
   const int tile_m = bricks ? tile_m_x : tile_m_p, tile_n = bricks ? tile_n_x : tile_n_p;
-  const int z = bricks ? z_x : (int)blockIdx.y;
+  const int z = bricks ? z_x : (int)by;
   const int m0 = tile_m * BM;
   const int n0 = tile_n * BN;
   const int grp = (int)fast_div(z, p.d_batch), zb = z - grp * (int)p.d_batch.d;
@@ -1183,7 +1184,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
         (phase(std::integral_constant<int, S>{}, kt + S, STEADY), ...);
       }(std::make_integer_sequence<int, NSTAGE>{});
     };
-    warm_ahead(p, (unsigned)(uintptr_t)(lptr_t)lds + NSTAGE * STAGE, id, gridDim.x * gridDim.y, wave, lane);
+    warm_ahead(p, (unsigned)(uintptr_t)(lptr_t)lds + NSTAGE * STAGE, id, nwg, wave, lane);
     if (p.bias != nullptr && wave == 0) {
       // the epilogue's bias values (one vector per K segment of a row-parallel layer, each in another home row) are
       // requested now and sit in the L2 when the epilogue asks for them
@@ -1274,6 +1275,13 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
     atomicAdd(p.trace + 5, t_end - t_loop);
     atomicAdd(p.trace + 6, 1ull);
   }
+}
+
+template <typename T, int BM, int BN, bool AKC, bool BKC, int NSTAGE, int SB, int PD>
+__global__ __launch_bounds__(512) void gemm_dma_kernel(GemmArgs p) {
+  touch_kernel_arguments<sizeof(GemmArgs)>();
+  gemm_dma_body<T, BM, BN, AKC, BKC, NSTAGE, SB, PD>(p, blockIdx.x + blockIdx.y * gridDim.x, blockIdx.x, blockIdx.y,
+                                                     gridDim.x * gridDim.y);
 }
 
 // ---------------------------------------------------------------------------------------------
