@@ -981,7 +981,11 @@ __device__ __forceinline__ void gemm_dma_body(const GemmArgs& p, const unsigned 
   using DB = DmaOperand<T, BN, BKC, NL, SB>;
   constexpr int BK = SB / sizeof(T);
   constexpr int KS = SB / 32;  // MFMA k-steps per slab
-  constexpr int WM = BM / 2, WN = BN / 2, MT = WM / 32, NT = WN / 32;
+  // the four MFMA waves form a 2 x 2 grid of wave tiles, or 4 x 1 where half the tile's columns are no whole number
+  // of 32-column MFMA blocks (BN = 160)
+  constexpr int WGM = (BN / 2) % 32 == 0 ? 2 : 4, WGN = 4 / WGM;
+  constexpr int WM = BM / WGM, WN = BN / WGN, MT = WM / 32, NT = WN / 32;
+  static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tiles are whole 32 x 32 MFMA blocks");
   constexpr int STAGE = DA::BYTES + DB::BYTES;
   constexpr int NI = DA::NI + DB::NI;  // loads per loader wave and slab
   static_assert((NSTAGE - 2) * NI < 64, "vmcnt is a 6-bit counter");
@@ -1000,7 +1004,7 @@ __device__ __forceinline__ void gemm_dma_body(const GemmArgs& p, const unsigned 
   }
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = (wave >> 1) & 1, wn = wave & 1;
+  const int wm = WGM == 2 ? (wave >> 1) & 1 : wave & 3, wn = WGM == 2 ? wave & 1 : 0;
   const int li = lane & 31, g = lane >> 5;
 
   // Workgroups are handed to the 8 XCDs round-robin in launch order, and every XCD has its own L2.  The
@@ -1260,9 +1264,10 @@ __device__ __forceinline__ void gemm_dma_body(const GemmArgs& p, const unsigned 
   __syncthreads();
   if (p.sgd_master != nullptr && p.vec_c)
     finish_tile_sgd<T, BM, BN, 512>(p, ct, m0, n0, tid, grp, zo, zi);
-  else if (p.xent_mode == 1)
-    finish_tile_xent_stats<T, BM, BN, 512>(p, ct, m0, n0, tid, grp);
-  else
+  else if (p.xent_mode == 1) {
+    // (tiles whose width is no multiple of the 64-column statistics blocks are never chosen for this epilogue)
+    if constexpr (BN % 64 == 0) finish_tile_xent_stats<T, BM, BN, 512>(p, ct, m0, n0, tid, grp);
+  } else
     finish_tile<T, BM, BN, 512>(p, ct, m0, n0, tid, grp, zo, zi);
   if (p.trace != nullptr && tid == 0) {
     const unsigned long long t_end = (unsigned long long)wall_clock64();
@@ -1638,9 +1643,9 @@ struct TileShape {
   int bm, bn;
   const char* tag;
 };
-static const TileShape kShapes[6] = {{256, 128, "256x128"}, {128, 128, "128x128"}, {128, 64, "128x64"}, {64, 64, "64x64"},
-                                     {128, 192, "128x192"}, {256, 256, "256x256"}};
-constexpr int kNumShapes = 6;
+static const TileShape kShapes[7] = {{256, 128, "256x128"}, {128, 128, "128x128"}, {128, 64, "128x64"}, {64, 64, "64x64"},
+                                     {128, 192, "128x192"}, {256, 256, "256x256"}, {128, 160, "128x160"}};
+constexpr int kNumShapes = 7;
 
 // One wavefront per 32 x 32 block is the better kernel for one attention head at sequence length <= 64.
 static bool is_tiny(const rtp_gemm_desc* d) { return d->m <= 64 && d->n <= 64 && d->k * d->ksegs <= 256; }
@@ -1795,8 +1800,8 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
     const char* e = getenv("RTP_GEMM_TILE");  // debugging aid: index into kShapes
     return e ? atoi(e) : -1;
   }();
-  static const double slab_ns[kNumShapes] = {966.0, 470.0, 283.0, 167.0, 800.0, 1680.0};
-  static const int slab_bytes[kNumShapes] = {128, 128, 128, 128, 128, 128};
+  static const double slab_ns[kNumShapes] = {966.0, 470.0, 283.0, 167.0, 800.0, 1680.0, 545.0};
+  static const int slab_bytes[kNumShapes] = {128, 128, 128, 128, 128, 128, 128};
   int shape = 3;  // 64 x 64 unless the model finds something cheaper
   double best = 0.0;
   for (int i = 0; fast && i < kNumShapes; ++i) {
@@ -1806,6 +1811,10 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
     // -10 % on the MoE layer's time; a loss where it leaves CUs without a tile or K is shorter)
     // (its epilogue is the plain one: the update and the statistics epilogue are never routed to it, forced or not)
     if (i == 5 && (sizeof(T) != 2 || d->sgd_master || d->xent_mode == 1)) continue;
+    if (i == 6 && d->xent_mode == 1) continue;  // 160 columns are no whole number of 64-column statistics blocks
+    // 128 x 160 is priced at the rate measured where it is meant for -- products of at most two rounds of tiles, such
+    // as the LM's logits layer (shards of 1280 columns); larger products keep the shapes measured on large products
+    if (i == 6 && ceil_div(d->m, 128) * ceil_div(d->n, 160) * nz > 512 && i != forced) continue;
     if (i == 5 && (ceil_div(d->m, 256) * ceil_div(d->n, 256) * nz < 256 || d->k * d->ksegs < 1024) && i != forced)
       continue;
     // never a tile that is mostly padding: a 32 x 32 problem (one attention head at seq 32) stays at 64 x 64
@@ -1931,6 +1940,10 @@ static int launch_gemm(hipStream_t s, const rtp_gemm_desc* d) {
       return launch_dma<T, 128, 64, 5, 128, 4>(s, a, akc, bkc, grid);
     case 4:
       return launch_dma<T, 128, 192, 3, 128, 2>(s, a, akc, bkc, grid);
+    case 6:
+      // 4 x 1 wave tiles of 32 x 160: a layer whose shards are 1280 columns wide (the LM's logits) is 8 tiles per
+      // shard and fills the CUs in two even rounds where 128 x 128 tiles need two and a half
+      return launch_dma<T, 128, 160, 4, 128, 1>(s, a, akc, bkc, grid);
     case 5:
       if constexpr (sizeof(T) == 2) return launch_dma8<T, 2, 128, 1>(s, a, akc, bkc, grid);
       return fail(RTP_ERR_ARG, "gemm: no 256 x 256 kernel for this dtype");

@@ -440,3 +440,36 @@ def test_gemm_random_shapes_layouts_and_epilogues():
         what = f"case {case}: {dtype} m {m} n {n} k {k} akc {akc} bkc {bkc} bias {use_bias} cin {use_cin} relu {relu}"
         assert not torch.isnan(out).any(), what
         assert rel_err(out, ref) <= TOL[dtype], what
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("akc", [True, False])
+@pytest.mark.parametrize("m,k,ksegs", [(1024, 2048, 1), (1000, 520, 1), (1024, 264, 2)])
+def test_gemm_128x160_tile_path(akc, dtype, m, k, ksegs):
+    """Shards 1280 columns wide (the LM's logits layer) take 128 x 160 tiles -- 4 x 1 wave tiles of 32 x 160 -- for a
+    K-contiguous second operand: 8 groups of 8 x 8 tiles fill the CUs in two even rounds (checked by the kernel's name
+    in the launch records).  Grouped, with bias, ReLU and an addend, ragged rows, a ragged last slab and K segments."""
+    from rtp_amd import _lib
+    ops = _ops()
+    gen = torch.Generator().manual_seed(m + k)
+    groups, n_s = 8, 1280
+    n = groups * n_s
+    a = _rand((m, k * ksegs) if akc else (k * ksegs, m), dtype, gen).to(DEV)
+    b = _rand((n, k * ksegs), dtype, gen).to(DEV)
+    bias, cin = _rand((n,), dtype, gen).to(DEV), _rand((m, n), dtype, gen).to(DEV)
+    A = a.float() if akc else a.float().t()
+    ref = torch.relu(A @ b.float().t() + bias.float() + cin.float())
+    out = torch.full((m, n), float("nan"), dtype=dtype, device=DEV)
+    es = a.element_size()
+    _lib.profile_enable(1)
+    try:
+        ops.gemm_raw(dtype, a=a.data_ptr(), b=b.data_ptr(), c_out=out.data_ptr(), m=m, n=n_s, k=k, lda=a.stride(0),
+                     ldb=b.stride(0), ldc=n, a_kcontig=akc, b_kcontig=True, bias=bias.data_ptr(), c_in=cin.data_ptr(),
+                     ld_cin=n, relu=True, groups=groups, b_sg=n_s * k * ksegs, c_sg=n_s, cin_sg=n_s, bias_sg=n_s,
+                     ksegs=ksegs, a_sk=k if akc else k * m, b_sk=k)
+        torch.cuda.synchronize()
+        names = list(_lib.profile_collect())
+    finally:
+        _lib.profile_enable(0)
+    assert any("128x160" in nm for nm in names), names
+    assert rel_err(out, ref) <= TOL[dtype]
