@@ -509,7 +509,7 @@ def layer_workload(name, steps, warmup, graph=True, cpu=True, ring_result=None):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--workload", default="lm", choices=["lm", "linear", "embedding", "attention", "moe", "gemm"],
